@@ -1,0 +1,190 @@
+"""Pins the CPU oracle against what the reference's own tests hold for this path and against what
+the mathematics fixes, without running the reference.
+
+- REF_HASHES (src/ggml.rs:1547-1577): FNV-1a-64 of gguf-py's dequantization of the seeded fixtures.
+- f16 / bf16 conversions: exhaustive against numpy / torch.
+- e4m3: all 256 bytes against torch.float8_e4m3fn and the closed form (src/ggml.rs:1505-1523).
+- quantize_act: the scalar definition of src/quant.rs:633-658 including its special cases.
+- decode_i8: the invariant of src/ggml.rs:1663-1681.
+"""
+import numpy as np
+import pytest
+import torch
+
+# (type id, hash) copied from the reference's golden table, src/ggml.rs:1547-1577
+REF_HASHES = {
+    "BF16": (30, 0x767e77c423088e31),
+    "F16": (1, 0xd03c69ee7934955f),
+    "F32": (0, 0x8c4157552256808b),
+    "Q2_K": (10, 0x44b0a081c4b9c71c),
+    "Q4_0": (2, 0xc2ac60f0d9d22bc8),
+    "Q4_1": (3, 0x8a49b60459c03fa2),
+    "Q4_K": (12, 0xde4da39c1d9096b2),
+    "Q5_0": (6, 0x46640e791feaf19f),
+    "Q5_1": (7, 0xb0fd98e61b74d61d),
+    "Q5_K": (13, 0x4be2f59b66cc7042),
+    "Q6_K": (14, 0x20a51cc0feaae638),
+    "Q8_0": (8, 0x3199be3deddf5c1a),
+}
+FIXTURE_ELEMS = 1024
+
+
+def fixture_blocks(oxref, kind):
+    raw, _ = oxref.random_blocks(kind, FIXTURE_ELEMS // oxref.block_size(kind), 1000 + kind)
+    return raw
+
+
+@pytest.mark.parametrize("name", sorted(REF_HASHES))
+def test_dequantization_matches_ggml_hashes(oxref, name):
+    kind, want = REF_HASHES[name]
+    y = oxref.dequantize_row(kind, fixture_blocks(oxref, kind), FIXTURE_ELEMS)
+    assert oxref.fnv1a_f32(y) == want, f"{name}: dequantized fixture differs from ggml"
+
+
+def test_fnv_known_answer(oxref):
+    # FNV-1a-64 of the empty input is the offset basis; of one zero byte quadruple a fixed value.
+    assert oxref.fnv1a_f32(np.zeros(0, np.float32)) == 0xcbf29ce484222325
+    h = 0xcbf29ce484222325
+    for b in np.float32(1.5).tobytes():
+        h = ((h ^ b) * 0x100000001b3) % (1 << 64)
+    assert oxref.fnv1a_f32(np.array([1.5], np.float32)) == h
+
+
+def test_lcg_known_answers(oxref):
+    s, out = 7, []
+    for _ in range(4):
+        s = (s * 6364136223846793005 + 1442695040888963407) % (1 << 64)
+        out.append(s >> 33)
+    got, end = oxref.lcg_stream(7, 4)
+    assert list(got) == out and end == s
+
+
+def test_f16_to_f32_exhaustive(oxref):
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([oxref.lib.oxref_f16_to_f32(int(v)) for v in h], np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+
+
+def test_f32_to_f16_rne(oxref):
+    rng = np.random.default_rng(1)
+    # every f16 value, the midpoints between neighbours, values just off them, and random bits
+    h = np.arange(0x7C00, dtype=np.uint16).view(np.float16).astype(np.float64)
+    mids = (h[:-1] + h[1:]) / 2
+    vals = np.concatenate([h, mids, np.nextafter(mids.astype(np.float32), np.float32(np.inf)).astype(np.float64),
+                           np.nextafter(mids.astype(np.float32), np.float32(-np.inf)).astype(np.float64),
+                           [65504.0, 65519.9, 65520.0, 1e9, 2.0 ** -25, 2.0 ** -24, 1.0000001 * 2.0 ** -25, 0.0]])
+    vals = np.concatenate([vals, -vals]).astype(np.float32)
+    rnd = rng.integers(0, 1 << 32, 200000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    rnd = rnd[np.isfinite(rnd)]
+    for x in (vals, rnd):
+        with np.errstate(over="ignore"):
+            want = x.astype(np.float16).view(np.uint16)
+        got = np.array([oxref.lib.oxref_f32_to_f16(float(v)) for v in x], np.uint16)
+        assert np.array_equal(got, want)
+
+
+def test_f32_to_bf16_rne(oxref):
+    rng = np.random.default_rng(2)
+    x = rng.integers(0, 1 << 32, 200000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    x = x[np.isfinite(x)]
+    x = np.concatenate([x, np.array([1.0, 1.00390625, 1.005859375, 1.001953125, 3.3895314e38, -0.0], np.float32)])
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = np.array([oxref.lib.oxref_f32_to_bf16(float(v)) for v in x], np.uint16)
+    assert np.array_equal(got, want)
+    back = np.array([oxref.lib.oxref_bf16_to_f32(int(v)) for v in got[:1000]], np.float32)
+    assert np.array_equal(back.view(np.uint32), (got[:1000].astype(np.uint32) << 16))
+
+
+def test_e4m3_all_bytes(oxref):
+    b = np.arange(256, dtype=np.uint8)
+    want = torch.from_numpy(b).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    got = np.array([oxref.e4m3_to_f32(v) for v in b], np.float32)
+    nan = np.isnan(want)
+    assert list(np.nonzero(nan)[0]) == [0x7F, 0xFF]
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+    assert got[0x7E] == 448.0 and got[0x01] == 2.0 ** -9 and got[0x08] == 2.0 ** -6
+
+
+def test_e4m3_scaled_matches_the_table(oxref):
+    # src/ggml.rs:1505-1523: the bit-built conversion times s equals the table value times s
+    bytes_ = np.concatenate([np.arange(256), np.arange(255, -1, -1)]).astype(np.uint8)
+    table = np.array([oxref.e4m3_to_f32(v) for v in range(256)], np.float32)
+    for s in (1.0, 0.003741, -2.5):
+        for n in (0, 1, 7, 16, 33, 128, 300, 512):
+            got = oxref.e4m3_scaled(bytes_[:n], s)
+            want = table[bytes_[:n]] * np.float32(s)
+            nan = np.isnan(want)
+            assert np.array_equal(np.isnan(got), nan)
+            assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+
+
+def test_fp8_block_scale_indexing(oxref):
+    # scale of weight (r, c) is s[(r / rows) * ceil(n_in / cols) + c / cols] (src/ggml.rs:250-256)
+    n_out, n_in = 256, 320  # 3 column blocks, the last partial
+    data = np.full((n_out, n_in), 0x38, np.uint8)  # 1.0
+    scales = np.arange(1, 2 * 3 + 1, dtype=np.float32)
+    w = oxref.fp8_dequant_rows(data, scales, n_out, n_in)
+    for r, c in [(0, 0), (127, 127), (127, 128), (128, 0), (255, 319), (130, 256)]:
+        assert w[r, c] == scales[(r // 128) * 3 + c // 128]
+
+
+def test_activation_quantization_matches_scalar(oxref):
+    # src/quant.rs:633-658
+    t, n = 5, 4 * 32
+    s, xs = 7, []
+    for _ in range(t * n):
+        s = (s * 6364136223846793005 + 1442695040888963407) % (1 << 64)
+        xs.append(np.float32((s >> 33) % 20001) / np.float32(1000.0) - np.float32(10.0))
+    x = np.array(xs, np.float32)
+    x[32:64] = 0.0
+    x[2 * 32 + 3] = 1e-30
+    for tt in (1, t):
+        q, scales, sums, fsums, hsums = oxref.quantize_act(x[: tt * n], tt, n)
+        q, scales, sums, fsums, hsums = (a.reshape(-1) for a in (q, scales, sums, fsums, hsums))
+        for bi in range(tt * n // 32):
+            blk = x[bi * 32:(bi + 1) * 32]
+            amax = np.float32(0)
+            for v in blk:
+                amax = max(amax, np.float32(abs(v)))
+            inv = np.float32(127.0) / amax if amax > 0 else np.float32(0)
+            p = blk * inv
+            qq = (np.sign(p) * np.floor(np.abs(p) + np.float32(0.5))).astype(np.int8)  # half away from zero
+            assert np.array_equal(q[bi * 32:(bi + 1) * 32], qq), bi
+            assert scales[bi].view(np.uint32) == (amax / np.float32(127.0)).view(np.uint32)
+            assert sums[bi] == int(qq.astype(np.int32).sum())
+            acc = np.float32(0)
+            for v in blk:
+                acc = np.float32(acc + v)
+            assert fsums[bi].view(np.uint32) == acc.view(np.uint32)
+            acc = np.float32(0)
+            for v in blk[16:]:
+                acc = np.float32(acc + v)
+            assert hsums[2 * bi + 1].view(np.uint32) == acc.view(np.uint32)
+        assert np.all(q[32:64] == 0) and scales[1] == 0.0
+
+
+@pytest.mark.parametrize("name", [k for k in sorted(REF_HASHES) if k not in ("F32", "F16", "BF16")])
+def test_int8_decoding_matches_dequantization(oxref, name):
+    # src/ggml.rs:1663-1681
+    kind, _ = REF_HASHES[name]
+    raw = fixture_blocks(oxref, kind)
+    want = oxref.dequantize_row(kind, raw, FIXTURE_ELEMS)
+    bs, ts = oxref.block_size(kind), oxref.type_size(kind)
+    for bi in range(FIXTURE_ELEMS // bs):
+        q, s, m, has_min = oxref.decode_i8(kind, raw[bi * ts:(bi + 1) * ts])
+        if not has_min:
+            m[:] = 0
+        v = np.repeat(s, 16) * q.astype(np.float32) + np.repeat(m, 16)
+        w = want[bi * bs:(bi + 1) * bs]
+        assert np.all(np.abs(v - w) <= 1e-6 * np.maximum(np.abs(w), 1e-3)), (name, bi)
+
+
+def test_type_geometry(oxref):
+    # src/ggml.rs:1683-1690 and the row sizes of the benchmark shapes
+    assert oxref.row_bytes(12, 5120) == 20 * 144
+    assert oxref.row_bytes(8, 4096) == 4352 and oxref.row_bytes(12, 4096) == 2304 and oxref.row_bytes(14, 4096) == 3360
+    assert oxref.block_size(15) == 0  # Q8_K is not a weight format
