@@ -1,0 +1,129 @@
+/* liboxinfer_hip: MI355X (gfx950) quantized-weight matmuls behind oxinfer's accelerator surface.
+ *
+ * A C ABI (plain pointers and sizes) that an `impl Backend for HipBackend` on the Rust side binds at
+ * run time with dlsym, the way src/cuda.rs:31-86 binds libcuda. Each entry point names the
+ * reference interface it stands behind (paths relative to the oxinfer tree).
+ *
+ * Conventions (those of `trait Backend`, src/gpu.rs:151-294):
+ *   - functions returning int: 1 = done, 0 = declined and NOTHING was written; the caller then runs
+ *     its CPU path (src/gpu.rs:158-160, src/model.rs:877-882). Handle-returning calls give NULL.
+ *   - oxhip_last_error() holds the reason of the calling thread's last decline.
+ *   - every call may come from any thread, concurrently (src/cuda.rs:2047-2077, :2410-2438).
+ *   - matrices are [n_out, n_in] row-major, outputs y[t][n_out] f32 (src/kernels.rs:54-57).
+ *
+ * Two layers:
+ *   1. the Backend surface: host pointers in, host pointers out (the library owns staging);
+ *   2. device-pointer entry points (oxhip_dev_*): the same kernels on buffers already in HBM, on a
+ *      caller-chosen stream, for callers that keep activations resident and for measurement.
+ */
+#ifndef OXHIP_H
+#define OXHIP_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct oxhip_ctx oxhip_ctx;       /* one per device: `HipBackend` (cf. CudaBackend, src/cuda.rs:404-446) */
+typedef struct oxhip_weight oxhip_weight; /* `DeviceWeight` of one matrix (src/gpu.rs:57) */
+typedef struct oxhip_moe oxhip_moe;       /* `DeviceWeight` of one MoE layer's experts (src/gpu.rs:206-216) */
+
+/* `WeightRef` (src/gpu.rs:15-21) plus the MLX triplet before `from_mlx_q4` (src/quant.rs:518). */
+enum {
+    OXHIP_W_BF16 = 0,   /* data: u16 bf16 [n_out, n_in] */
+    OXHIP_W_Q8 = 1,     /* QMatrix: data i8 [n_out, n_in], scales f32 [n_out, n_in/32] (src/quant.rs) */
+    OXHIP_W_Q4 = 2,     /* Q4Matrix: data nibbles [n_out, n_in/2], scales f16 [n_out, n_in/32],
+                           offsets bf16 [n_out, n_in/group] or NULL (src/quant.rs:427-440) */
+    OXHIP_W_GGUF = 3,   /* GgufMatrix: raw blocks of ggml_type; F8E4M3 with block_scales (src/ggml.rs:240-256) */
+    OXHIP_W_MLX_Q4 = 4  /* MLX affine 4-bit: data u32 [n_out, n_in/8], scales / offsets(=biases) bf16
+                           [n_out, n_in/group]; repacked on the device exactly as from_mlx_q4 does */
+};
+
+/* GGUF type ids handled (src/ggml.rs:42-93). */
+enum { OXHIP_GGML_Q8_0 = 8, OXHIP_GGML_Q4_K = 12, OXHIP_GGML_Q6_K = 14, OXHIP_GGML_F8E4M3 = 0x1000 };
+
+typedef struct {
+    uint32_t kind;            /* OXHIP_W_* */
+    uint32_t ggml_type;       /* OXHIP_GGML_* when kind == OXHIP_W_GGUF */
+    size_t n_out, n_in;
+    const void* data;
+    const void* scales;
+    const void* offsets;
+    uint32_t group;           /* elements per offset (Q4) / per scale and bias (MLX) */
+    const float* block_scales;/* FP8: [ceil(n_out/bs_rows), ceil(n_in/bs_cols)] */
+    uint32_t bs_rows, bs_cols;
+} oxhip_weight_desc;
+
+/* `Job` (src/gpu.rs:60-65). */
+typedef struct {
+    const oxhip_weight* w;
+    size_t n_out;
+    float* y; /* host, [t, n_out] */
+} oxhip_job;
+
+/* `RowsJob` (src/gpu.rs:69-75): y = W x, or with `up`: y = silu(W x) * (U x). */
+typedef struct {
+    const oxhip_weight* w;
+    const oxhip_weight* up; /* NULL for a plain product */
+    size_t n_out;
+    float* y;
+} oxhip_rows_job;
+
+/* `MoeAct` (src/gpu.rs:35-54); the CPU-only kinds are declined like the reference's backends do. */
+enum { OXHIP_ACT_SILU = 0, OXHIP_ACT_GELU_TANH = 1, OXHIP_ACT_SILU_CLAMP = 2 };
+
+/* ---- life cycle -------------------------------------------------------------------------- */
+/* CudaBackend::new (src/cuda.rs:448-570). 1 on success; 0 when the device cannot start. */
+int oxhip_open(int device, oxhip_ctx** out);
+void oxhip_close(oxhip_ctx* ctx);
+/* Backend::name (src/gpu.rs:152), e.g. "hip (gfx950)". */
+const char* oxhip_name(const oxhip_ctx* ctx);
+const char* oxhip_last_error(void);
+/* Backend::stats (src/gpu.rs:291): cumulative copy-in / gpu / copy-out ms; returns bytes written. */
+size_t oxhip_stats(oxhip_ctx* ctx, char* buf, size_t len);
+
+/* ---- Backend surface (host pointers) ------------------------------------------------------ */
+/* Backend::wants (src/gpu.rs:155; CUDA's policy src/cuda.rs:1134-1136). */
+int oxhip_wants(const oxhip_ctx* ctx, size_t n_out, size_t n_in, size_t t);
+/* Backend::upload (src/gpu.rs:157; src/cuda.rs:640-699). NULL when declined (unsupported format
+ * or shape, memory short under a 512 MiB reserve). */
+oxhip_weight* oxhip_upload(oxhip_ctx* ctx, const oxhip_weight_desc* desc);
+/* Dropping a DeviceWeight. */
+void oxhip_free_weight(oxhip_ctx* ctx, oxhip_weight* w);
+/* Bytes the weight occupies in HBM. */
+size_t oxhip_weight_bytes(const oxhip_weight* w);
+/* Backend::matmul (src/gpu.rs:160; src/cuda.rs:1428-1493): all jobs share x [t, n_in] (host f32);
+ * computes every job or none. t <= 16 runs the int8 decode kernels (the CPU's decode semantics,
+ * src/kernels.rs:1908-1928); more tokens run the MFMA GEMM. */
+int oxhip_matmul(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_job* jobs, size_t n_jobs);
+/* ---- device-pointer entry points ---------------------------------------------------------- */
+/* `QAct` (src/quant.rs:222-238) in HBM, plus sums16: the integer sum of each 16 int8 values (what
+ * the centred nibble formats fold their offset through; the CPU derives it from `sums`). */
+typedef struct {
+    int8_t* q;        /* [t, n_in] */
+    float* scales;    /* [t, n_in/32] */
+    int32_t* sums;    /* [t, n_in/32] */
+    float* fsums;     /* [t, n_in/32] */
+    float* hsums;     /* [t, n_in/16] */
+    int32_t* sums16;  /* [t, n_in/16] */
+    size_t t, n_in;
+} oxhip_qact;
+
+/* quant::quantize_act (src/quant.rs:294-343) on device rows x [t, n_in] f32. */
+int oxhip_dev_quantize_act(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, const oxhip_qact* out, void* stream);
+/* QMat::dequantize_rows (src/kernels.rs:1336, src/ggml.rs:409-459): rows r0..r1 as f32 [r1-r0, n_in]. */
+int oxhip_dev_dequantize(oxhip_ctx* ctx, const oxhip_weight* w, size_t r0, size_t r1, float* out, void* stream);
+/* The decode kernels (QMat::rows_t1 / rows_tc, src/kernels.rs:1339-1369, src/ggml.rs:1319-1354):
+ * y [t, n_out] f32 from quantized activations, t <= 16. FP8 / bf16 weights are float-stored
+ * (`dense`, src/ggml.rs:1370): they take f32 rows `x` instead and `xa` may be NULL. */
+int oxhip_dev_decode(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa, const float* x, size_t t, float* y,
+                     void* stream);
+/* The exact integer accumulators of the decode kernels: per block of 32 for Q4
+ * ([t, n_out, n_in/32]), per 16 for GGUF ([t, n_out, n_in/16]). For parity checks. */
+int oxhip_dev_isums(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa, int32_t* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

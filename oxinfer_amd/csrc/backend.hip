@@ -1,0 +1,521 @@
+// The C ABI: the device context, uploads, and the `Backend` surface (src/gpu.rs:151-294 of the
+// reference) over the kernels of this library.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "internal.hpp"
+
+namespace oxhip {
+
+static thread_local std::string g_err;
+void set_error(const std::string& m) { g_err = m; }
+
+#define HIP_TRY(expr, what)                                                              \
+    do {                                                                                 \
+        hipError_t e__ = (expr);                                                         \
+        if (e__ != hipSuccess) {                                                         \
+            set_error(std::string(what) + ": " + hipGetErrorString(e__));                \
+            return 0;                                                                    \
+        }                                                                                \
+    } while (0)
+
+constexpr size_t VRAM_RESERVE = 512ull << 20;  // kept free for activations (src/cuda.rs:573-588)
+
+struct DevBuf {
+    void* p = nullptr;
+    size_t cap = 0;
+    bool grow(size_t need) {
+        if (cap >= need && p) return true;
+        if (p) (void)hipFree(p);
+        p = nullptr;
+        cap = 0;
+        size_t want = (need < 256 ? 256 : need) * 2;
+        if (hipMalloc(&p, want) != hipSuccess) {
+            p = nullptr;
+            return false;
+        }
+        cap = want;
+        return true;
+    }
+    void release() {
+        if (p) (void)hipFree(p);
+        p = nullptr;
+        cap = 0;
+    }
+};
+
+}  // namespace oxhip
+
+using namespace oxhip;
+
+struct oxhip_weight {
+    WeightView v{};
+    void* base = nullptr;
+    size_t bytes = 0;
+};
+
+struct oxhip_ctx {
+    int device = 0;
+    std::string name;
+    hipStream_t stream = nullptr;
+    std::mutex mu;  // serializes the host-pointer surface (staging is shared), as Mutex<Staging> does
+    DevBuf x, xq, y;
+    double ms_in = 0, ms_gpu = 0, ms_out = 0;
+    size_t calls = 0;
+};
+
+namespace {
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct Planes {
+    size_t off[4] = {0, 0, 0, 0};
+    size_t total = 0;
+    void add(int i, size_t bytes) {
+        off[i] = total;
+        total = align_up(total + bytes, 256);
+    }
+};
+
+bool have_memory(size_t bytes) {
+    size_t free_b = 0, total_b = 0;
+    if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) return false;
+    return free_b >= bytes + VRAM_RESERVE;
+}
+
+void bind(oxhip_weight* w, const Planes& pl, int nplanes) {
+    const uint8_t* b = static_cast<const uint8_t*>(w->base);
+    const uint8_t** dst[4] = {&w->v.p0, &w->v.p1, &w->v.p2, &w->v.p3};
+    for (int i = 0; i < nplanes; i++) *dst[i] = b + pl.off[i];
+}
+
+// Uploads host bytes into a temporary device buffer.
+struct Temp {
+    void* p = nullptr;
+    ~Temp() {
+        if (p) (void)hipFree(p);
+    }
+    bool put(const void* src, size_t bytes, hipStream_t s) {
+        if (hipMalloc(&p, bytes ? bytes : 1) != hipSuccess) return false;
+        return hipMemcpyAsync(p, src, bytes, hipMemcpyHostToDevice, s) == hipSuccess;
+    }
+};
+
+QActView view_of(const oxhip_qact& a) { return QActView{a.q, a.scales, a.sums, a.fsums, a.hsums, a.sums16}; }
+
+// Carves a QAct for t rows of n_in out of one buffer.
+size_t qact_bytes(size_t t, size_t n_in) {
+    size_t b32 = t * n_in / 32, b16 = t * n_in / 16;
+    return align_up(t * n_in, 256) + 3 * align_up(b32 * 4, 256) + 2 * align_up(b16 * 4, 256);
+}
+oxhip_qact carve_qact(void* base, size_t t, size_t n_in) {
+    uint8_t* p = static_cast<uint8_t*>(base);
+    size_t b32 = t * n_in / 32, b16 = t * n_in / 16;
+    oxhip_qact a{};
+    a.q = reinterpret_cast<int8_t*>(p);
+    p += align_up(t * n_in, 256);
+    a.scales = reinterpret_cast<float*>(p);
+    p += align_up(b32 * 4, 256);
+    a.sums = reinterpret_cast<int32_t*>(p);
+    p += align_up(b32 * 4, 256);
+    a.fsums = reinterpret_cast<float*>(p);
+    p += align_up(b32 * 4, 256);
+    a.hsums = reinterpret_cast<float*>(p);
+    p += align_up(b16 * 4, 256);
+    a.sums16 = reinterpret_cast<int32_t*>(p);
+    a.t = t;
+    a.n_in = n_in;
+    return a;
+}
+
+bool is_dense(const oxhip_weight* w) { return w->v.fmt == FMT_FP8 || w->v.fmt == FMT_BF16; }
+
+}  // namespace
+
+extern "C" {
+
+const char* oxhip_last_error(void) { return g_err.c_str(); }
+
+int oxhip_open(int device, oxhip_ctx** out) {
+    if (!out) return 0;
+    *out = nullptr;
+    int n = 0;
+    HIP_TRY(hipGetDeviceCount(&n), "hipGetDeviceCount");
+    if (device < 0 || device >= n) {
+        set_error("device " + std::to_string(device) + ": not available (" + std::to_string(n) + " HIP devices)");
+        return 0;
+    }
+    HIP_TRY(hipSetDevice(device), "hipSetDevice");
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties");
+    std::string arch = prop.gcnArchName;
+    arch = arch.substr(0, arch.find(':'));
+    if (arch != "gfx950") {
+        set_error("device " + std::to_string(device) + " is " + arch + ": this library holds gfx950 code only");
+        return 0;
+    }
+    auto* c = new oxhip_ctx();
+    c->device = device;
+    c->name = "hip (" + arch + ")";
+    if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
+        set_error("hipStreamCreate failed");
+        delete c;
+        return 0;
+    }
+    *out = c;
+    return 1;
+}
+
+void oxhip_close(oxhip_ctx* c) {
+    if (!c) return;
+    (void)hipSetDevice(c->device);
+    (void)hipStreamSynchronize(c->stream);
+    c->x.release();
+    c->xq.release();
+    c->y.release();
+    (void)hipStreamDestroy(c->stream);
+    delete c;
+}
+
+const char* oxhip_name(const oxhip_ctx* c) { return c ? c->name.c_str() : ""; }
+
+size_t oxhip_stats(oxhip_ctx* c, char* buf, size_t len) {
+    if (!c || !buf || !len) return 0;
+    std::lock_guard<std::mutex> g(c->mu);
+    int n = snprintf(buf, len, "hip: %zu calls, copy-in %.2f ms, gpu %.2f ms, copy-out %.2f ms", c->calls, c->ms_in, c->ms_gpu,
+                     c->ms_out);
+    return n < 0 ? 0 : ((size_t)n < len ? (size_t)n : len - 1);
+}
+
+// The device reads weights at several TB/s and a launch costs a few microseconds, so unlike the
+// reference's PCIe-attached policy (t >= 32, 1 GFLOP) any whole-block shape is worth taking; the
+// activations still cross the host link on this surface, which is what bounds small calls.
+int oxhip_wants(const oxhip_ctx* c, size_t n_out, size_t n_in, size_t t) {
+    if (!c || !t || !n_out) return 0;
+    return n_in % 32 == 0 && n_in >= 32;
+}
+
+size_t oxhip_weight_bytes(const oxhip_weight* w) { return w ? w->bytes : 0; }
+
+void oxhip_free_weight(oxhip_ctx* c, oxhip_weight* w) {
+    if (!w) return;
+    if (c) (void)hipSetDevice(c->device);
+    if (w->base) (void)hipFree(w->base);
+    delete w;
+}
+
+oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) {
+    if (!c || !d || !d->data) {
+        set_error("upload: null argument");
+        return nullptr;
+    }
+    const size_t n_out = d->n_out, n_in = d->n_in;
+    if (!n_out || !n_in || n_out > 0x7FFFFFFFu || n_in > 0x7FFFFFFFu) {
+        set_error("upload: bad shape");
+        return nullptr;
+    }
+    if (hipSetDevice(c->device) != hipSuccess) {
+        set_error("hipSetDevice failed");
+        return nullptr;
+    }
+    auto w = new oxhip_weight();
+    w->v.n_out = (uint32_t)n_out;
+    w->v.n_in = (uint32_t)n_in;
+    auto fail = [&](const std::string& why) -> oxhip_weight* {
+        set_error("upload: " + why);
+        if (w->base) (void)hipFree(w->base);
+        delete w;
+        return nullptr;
+    };
+    auto alloc = [&](const Planes& pl, int nplanes) -> bool {
+        if (!have_memory(pl.total)) return false;
+        if (hipMalloc(&w->base, pl.total) != hipSuccess) {
+            w->base = nullptr;
+            return false;
+        }
+        w->bytes = pl.total;
+        bind(w, pl, nplanes);
+        return true;
+    };
+    hipStream_t s = c->stream;
+    Planes pl;
+    switch (d->kind) {
+        case OXHIP_W_BF16: {
+            if (n_in % 8) return fail("bf16 rows must be a multiple of 8");
+            w->v.fmt = FMT_BF16;
+            pl.add(0, n_out * n_in * 2);
+            if (!alloc(pl, 1)) return fail("device memory short");
+            if (hipMemcpyAsync(w->base, d->data, n_out * n_in * 2, hipMemcpyHostToDevice, s) != hipSuccess) return fail("copy failed");
+            break;
+        }
+        case OXHIP_W_Q4: {
+            if (n_in % 32 || !d->scales) return fail("Q4 needs n_in % 32 == 0 and scales");
+            size_t group = d->offsets ? d->group : 0;
+            if (d->offsets && (group == 0 || group % 32 || n_in % group)) return fail("Q4 offset group must be a multiple of 32 dividing n_in");
+            w->v.fmt = FMT_Q4;
+            w->v.group = (uint32_t)group;
+            // one scale per offset group when the blocks of a group agree (MLX), else per 32
+            size_t sgroup = group ? group : 32;
+            for (int attempt = 0; attempt < 2; attempt++) {
+                pl = Planes();
+                pl.add(0, n_out * n_in / 2);
+                pl.add(1, n_out * (n_in / sgroup) * 2);
+                if (group) pl.add(2, n_out * (n_in / group) * 2);
+                if (!alloc(pl, group ? 3 : 2)) return fail("device memory short");
+                w->v.sgroup = (uint32_t)sgroup;
+                uint8_t* b = static_cast<uint8_t*>(w->base);
+                if (hipMemcpyAsync(b + pl.off[0], d->data, n_out * n_in / 2, hipMemcpyHostToDevice, s) != hipSuccess) return fail("copy failed");
+                if (group && hipMemcpyAsync(b + pl.off[2], d->offsets, n_out * (n_in / group) * 2, hipMemcpyHostToDevice, s) != hipSuccess)
+                    return fail("copy failed");
+                if (sgroup == 32) {
+                    if (hipMemcpyAsync(b + pl.off[1], d->scales, n_out * (n_in / 32) * 2, hipMemcpyHostToDevice, s) != hipSuccess)
+                        return fail("copy failed");
+                    break;
+                }
+                Temp t32, flag;
+                int zero = 0, mismatch = 0;
+                if (!t32.put(d->scales, n_out * (n_in / 32) * 2, s) || !flag.put(&zero, sizeof zero, s)) return fail("device memory short");
+                if (launch_q4_scale_groups(static_cast<const uint16_t*>(t32.p), n_out, n_in, sgroup, reinterpret_cast<uint16_t*>(b + pl.off[1]),
+                                           static_cast<int*>(flag.p), s) != hipSuccess)
+                    return fail("scale repack launch failed");
+                if (hipMemcpyAsync(&mismatch, flag.p, sizeof mismatch, hipMemcpyDeviceToHost, s) != hipSuccess ||
+                    hipStreamSynchronize(s) != hipSuccess)
+                    return fail("scale repack failed");
+                if (!mismatch) break;
+                (void)hipFree(w->base);  // scales differ inside a group: keep one per block
+                w->base = nullptr;
+                sgroup = 32;
+            }
+            break;
+        }
+        case OXHIP_W_MLX_Q4: {
+            size_t group = d->group;
+            if (!d->scales || !d->offsets || group == 0 || group % 32 || n_in % group) return fail("MLX 4-bit needs scales, biases and a group that is a multiple of 32 dividing n_in");
+            w->v.fmt = FMT_Q4;
+            w->v.group = w->v.sgroup = (uint32_t)group;
+            pl.add(0, n_out * n_in / 2);
+            pl.add(1, n_out * (n_in / group) * 2);
+            pl.add(2, n_out * (n_in / group) * 2);
+            if (!alloc(pl, 3)) return fail("device memory short");
+            Temp tw, ts, tb;
+            if (!tw.put(d->data, n_out * n_in / 2, s) || !ts.put(d->scales, n_out * (n_in / group) * 2, s) ||
+                !tb.put(d->offsets, n_out * (n_in / group) * 2, s))
+                return fail("device memory short");
+            if (launch_repack_mlx_q4(static_cast<const uint32_t*>(tw.p), static_cast<const uint16_t*>(ts.p), static_cast<const uint16_t*>(tb.p),
+                                     n_out, n_in, group, w->v, s) != hipSuccess)
+                return fail("repack launch failed");
+            if (hipStreamSynchronize(s) != hipSuccess) return fail("repack failed");
+            break;
+        }
+        case OXHIP_W_GGUF: {
+            if (d->ggml_type == OXHIP_GGML_F8E4M3) {
+                if (!d->block_scales || !d->bs_rows || !d->bs_cols) return fail("FP8 needs block scales");
+                if (n_in % 16 || d->bs_cols % 16) return fail("FP8 rows and scale blocks must be multiples of 16 columns");
+                w->v.fmt = FMT_FP8;
+                w->v.br = d->bs_rows;
+                w->v.bc = d->bs_cols;
+                size_t ns = ((n_out + d->bs_rows - 1) / d->bs_rows) * ((n_in + d->bs_cols - 1) / d->bs_cols);
+                pl.add(0, n_out * n_in);
+                pl.add(1, ns * 4);
+                if (!alloc(pl, 2)) return fail("device memory short");
+                uint8_t* b = static_cast<uint8_t*>(w->base);
+                if (hipMemcpyAsync(b + pl.off[0], d->data, n_out * n_in, hipMemcpyHostToDevice, s) != hipSuccess ||
+                    hipMemcpyAsync(b + pl.off[1], d->block_scales, ns * 4, hipMemcpyHostToDevice, s) != hipSuccess)
+                    return fail("copy failed");
+                break;
+            }
+            size_t raw_bytes;
+            int np;
+            if (d->ggml_type == OXHIP_GGML_Q8_0) {
+                if (n_in % 32) return fail("Q8_0 rows must be whole blocks of 32");
+                w->v.fmt = FMT_Q8_0;
+                pl.add(0, n_out * n_in);
+                pl.add(1, n_out * (n_in / 32) * 2);
+                raw_bytes = n_out * (n_in / 32) * 34;
+                np = 2;
+            } else if (d->ggml_type == OXHIP_GGML_Q4_K) {
+                if (n_in % 256) return fail("Q4_K rows must be whole blocks of 256");
+                w->v.fmt = FMT_Q4_K;
+                pl.add(0, n_out * (n_in / 256) * 128);
+                pl.add(1, n_out * (n_in / 256) * 16);
+                raw_bytes = n_out * (n_in / 256) * 144;
+                np = 2;
+            } else if (d->ggml_type == OXHIP_GGML_Q6_K) {
+                if (n_in % 256) return fail("Q6_K rows must be whole blocks of 256");
+                w->v.fmt = FMT_Q6_K;
+                size_t nb = n_out * (n_in / 256);
+                pl.add(0, nb * 128);
+                pl.add(1, nb * 64);
+                pl.add(2, nb * 16);
+                pl.add(3, nb * 2);
+                raw_bytes = nb * 210;
+                np = 4;
+            } else {
+                return fail("GGUF type " + std::to_string(d->ggml_type) + " has no device kernels");
+            }
+            if (!alloc(pl, np)) return fail("device memory short");
+            Temp raw;
+            if (!have_memory(raw_bytes) || !raw.put(d->data, raw_bytes, s)) return fail("device memory short");
+            if (launch_repack_gguf(w->v.fmt, static_cast<const uint8_t*>(raw.p), n_out, n_in, w->v, s) != hipSuccess)
+                return fail("repack launch failed");
+            if (hipStreamSynchronize(s) != hipSuccess) return fail("repack failed");
+            break;
+        }
+        default: return fail("weight kind " + std::to_string(d->kind) + " has no device kernels");
+    }
+    if (hipStreamSynchronize(s) != hipSuccess) return fail("upload failed");
+    return w;
+}
+
+// ---- device-pointer entry points ---------------------------------------------------------------
+int oxhip_dev_quantize_act(oxhip_ctx* c, const float* x, size_t t, size_t n_in, const oxhip_qact* out, void* stream) {
+    if (!c || !x || !out || n_in % 32) {
+        set_error("quantize_act: bad arguments (n_in must be a multiple of 32)");
+        return 0;
+    }
+    HIP_TRY(launch_quantize_act(x, t, n_in, *out, static_cast<hipStream_t>(stream)), "quantize_act launch");
+    return 1;
+}
+
+int oxhip_dev_dequantize(oxhip_ctx* c, const oxhip_weight* w, size_t r0, size_t r1, float* out, void* stream) {
+    if (!c || !w || !out || r0 > r1 || r1 > w->v.n_out) {
+        set_error("dequantize: bad arguments");
+        return 0;
+    }
+    HIP_TRY(launch_dequantize(w->v, r0, r1, out, static_cast<hipStream_t>(stream)), "dequantize launch");
+    return 1;
+}
+
+int oxhip_dev_decode(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa, const float* x, size_t t, float* y, void* stream) {
+    if (!c || !w || !y || t == 0 || t > 16) {
+        set_error("decode: bad arguments (1 <= t <= 16)");
+        return 0;
+    }
+    QActView v{};
+    if (is_dense(w)) {
+        if (!x) {
+            set_error("decode: float-stored weights take f32 rows");
+            return 0;
+        }
+    } else {
+        if (!xa || xa->n_in != w->v.n_in || xa->t < t) {
+            set_error("decode: quantized activations missing or of another shape");
+            return 0;
+        }
+        v = view_of(*xa);
+    }
+    HIP_TRY(launch_decode(w->v, v, x, t, y, static_cast<hipStream_t>(stream)), "decode launch");
+    return 1;
+}
+
+int oxhip_dev_isums(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa, int32_t* out, void* stream) {
+    if (!c || !w || !xa || !out || is_dense(w) || xa->n_in != w->v.n_in) {
+        set_error("isums: bad arguments");
+        return 0;
+    }
+    HIP_TRY(launch_isums(w->v, view_of(*xa), xa->t, out, static_cast<hipStream_t>(stream)), "isums launch");
+    return 1;
+}
+
+// ---- Backend surface ---------------------------------------------------------------------------
+int oxhip_matmul(oxhip_ctx* c, const float* x, size_t t, size_t n_in, oxhip_job* jobs, size_t n_jobs) {
+    if (!c || !x || !jobs || !t || !n_jobs || n_in % 32) {
+        set_error("matmul: bad arguments");
+        return 0;
+    }
+    if (t > 16) {
+        set_error("matmul: more than 16 tokens take the prefill GEMM, which this build does not route here yet");
+        return 0;
+    }
+    size_t y_total = 0;
+    bool any_q = false;
+    for (size_t j = 0; j < n_jobs; j++) {
+        const oxhip_weight* w = jobs[j].w;
+        if (!w || !jobs[j].y || w->v.n_in != n_in || w->v.n_out != jobs[j].n_out) {
+            set_error("matmul: job " + std::to_string(j) + " does not match its weight");
+            return 0;
+        }
+        y_total += t * w->v.n_out;
+        any_q |= !is_dense(w);
+    }
+    std::lock_guard<std::mutex> g(c->mu);
+    HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
+    hipStream_t s = c->stream;
+    if (!c->x.grow(t * n_in * 4) || !c->y.grow(y_total * 4) || (any_q && !c->xq.grow(qact_bytes(t, n_in)))) {
+        set_error("matmul: device memory short");
+        return 0;
+    }
+    hipEvent_t e0, e1, e2, e3;
+    HIP_TRY(hipEventCreate(&e0), "event");
+    HIP_TRY(hipEventCreate(&e1), "event");
+    HIP_TRY(hipEventCreate(&e2), "event");
+    HIP_TRY(hipEventCreate(&e3), "event");
+    auto done = [&](int rc) {
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        (void)hipEventDestroy(e2);
+        (void)hipEventDestroy(e3);
+        return rc;
+    };
+    // Everything is computed into device staging first; y is written only once all jobs ran.
+    (void)hipEventRecord(e0, s);
+    if (hipMemcpyAsync(c->x.p, x, t * n_in * 4, hipMemcpyHostToDevice, s) != hipSuccess) {
+        set_error("matmul: copy-in failed");
+        return done(0);
+    }
+    (void)hipEventRecord(e1, s);
+    oxhip_qact xa{};
+    if (any_q) {
+        xa = carve_qact(c->xq.p, t, n_in);
+        if (launch_quantize_act(static_cast<const float*>(c->x.p), t, n_in, xa, s) != hipSuccess) {
+            set_error("matmul: quantize_act launch failed");
+            return done(0);
+        }
+    }
+    float* yd = static_cast<float*>(c->y.p);
+    size_t off = 0;
+    for (size_t j = 0; j < n_jobs; j++) {
+        const oxhip_weight* w = jobs[j].w;
+        if (launch_decode(w->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off, s) != hipSuccess) {
+            set_error("matmul: decode launch failed");
+            (void)hipStreamSynchronize(s);
+            return done(0);
+        }
+        off += t * w->v.n_out;
+    }
+    (void)hipEventRecord(e2, s);
+    if (hipStreamSynchronize(s) != hipSuccess) {
+        set_error("matmul: kernels failed");
+        return done(0);
+    }
+    off = 0;
+    std::vector<float> host(y_total);
+    if (hipMemcpyAsync(host.data(), yd, y_total * 4, hipMemcpyDeviceToHost, s) != hipSuccess) {
+        set_error("matmul: copy-out failed");
+        return done(0);
+    }
+    (void)hipEventRecord(e3, s);
+    if (hipStreamSynchronize(s) != hipSuccess) {
+        set_error("matmul: copy-out failed");
+        return done(0);
+    }
+    for (size_t j = 0; j < n_jobs; j++) {
+        size_t n = t * jobs[j].w->v.n_out;
+        std::memcpy(jobs[j].y, host.data() + off, n * 4);
+        off += n;
+    }
+    float a = 0, b = 0, d = 0;
+    (void)hipEventElapsedTime(&a, e0, e1);
+    (void)hipEventElapsedTime(&b, e1, e2);
+    (void)hipEventElapsedTime(&d, e2, e3);
+    c->ms_in += a;
+    c->ms_gpu += b;
+    c->ms_out += d;
+    c->calls++;
+    return done(1);
+}
+
+}  // extern "C"

@@ -1,0 +1,129 @@
+// Shared declarations of liboxinfer_hip: device layouts, launchers, small device helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include <mutex>
+#include <string>
+
+#include "../../include/oxhip.h"
+
+namespace oxhip {
+
+// ------------------------------------------------------------------------------------------------
+// Device layouts. Uploads repack every format into planes whose rows start on 16-byte boundaries,
+// so each lane of a wavefront reads one aligned 16-byte chunk and consecutive lanes read
+// consecutive chunks. The bytes are those of the source format, only rearranged.
+//
+//   Q4    q   [n_out][n_in/2]      byte j of a 32-block: element j (low nibble), j+16 (high)
+//         sc  [n_out][n_in/sgroup] f16 scale; sgroup = 32, or the offset group when every block of
+//                                  a group carries the same scale (MLX checkpoints)
+//         off [n_out][n_in/group]  bf16 offsets, optional
+//   Q8_0  q   [n_out][n_in]        int8
+//         d   [n_out][n_in/32]     f16
+//   Q4_K  qs  [n_out][nb][128]     nibbles as in the block
+//         mt  [n_out][nb][16]      d, dmin (f16) and the 12 packed scale bytes
+//   Q6_K  ql  [n_out][nb][128], qh [n_out][nb][64], sc [n_out][nb][16] int8, d [n_out][nb] f16
+//   FP8   q   [n_out][n_in]        e4m3 bytes; bs f32 [ceil(n_out/br)][ceil(n_in/bc)]
+//   BF16  q   [n_out][n_in]        bf16
+// ------------------------------------------------------------------------------------------------
+enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5 };
+
+struct WeightView {
+    int fmt;
+    uint32_t n_out, n_in;
+    const uint8_t* p0;
+    const uint8_t* p1;
+    const uint8_t* p2;
+    const uint8_t* p3;
+    uint32_t sgroup;  // Q4: elements per scale
+    uint32_t group;   // Q4: elements per offset (0: none)
+    uint32_t br, bc;  // FP8 block scale geometry
+};
+
+struct QActView {
+    const int8_t* q;
+    const float* scales;
+    const int32_t* sums;
+    const float* fsums;
+    const float* hsums;
+    const int32_t* sums16;
+};
+
+// Launchers (each returns hipSuccess or the launch error).
+hipError_t launch_quantize_act(const float* x, size_t t, size_t n_in, const oxhip_qact& out, hipStream_t s);
+hipError_t launch_dequantize(const WeightView& w, size_t r0, size_t r1, float* out, hipStream_t s);
+hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s);
+hipError_t launch_isums(const WeightView& w, const QActView& xa, size_t t, int32_t* out, hipStream_t s);
+hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t n_in, const WeightView& dst, hipStream_t s);
+hipError_t launch_repack_mlx_q4(const uint32_t* w, const uint16_t* scales, const uint16_t* biases, size_t n_out,
+                                size_t n_in, size_t group, const WeightView& dst, hipStream_t s);
+hipError_t launch_q4_scale_groups(const uint16_t* sc32, size_t n_out, size_t n_in, size_t sgroup, uint16_t* dst,
+                                  int* mismatch, hipStream_t s);
+
+void set_error(const std::string& msg);
+
+// ------------------------------------------------------------------------------------------------
+// Device helpers
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+    return (float)__builtin_bit_cast(_Float16, h);  // exact
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+// IEEE round-to-nearest-even f32 -> bf16 bits (NaN quieted), as half::bf16::from_f32.
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
+    uint32_t b = __float_as_uint(x);
+    if ((b & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((b >> 16) | 0x0040);
+    return (uint16_t)((b + 0x7FFFu + ((b >> 16) & 1)) >> 16);
+}
+// IEEE round-to-nearest-even f32 -> f16 bits (the hardware conversion is RNE, denormals kept).
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float x) {
+    _Float16 h = (_Float16)x;
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+// OCP e4m3 (float8_e4m3fn) byte -> f32 from the bits: (1 + m/8) 2^(e-7), subnormals m 2^-9,
+// 0x7f / 0xff NaN.
+__device__ __forceinline__ float e4m3_to_f32(uint32_t b) {
+    uint32_t e = (b >> 3) & 0xF, m = b & 7;
+    uint32_t normal = ((e + 120) << 23) | (m << 20);
+    uint32_t sub = __float_as_uint((float)(int)m * (1.0f / 512.0f));
+    uint32_t mag = e == 0 ? sub : normal;
+    mag = (b & 0x7F) == 0x7F ? 0x7FC00000u : mag;
+    return __uint_as_float(mag | ((b & 0x80) << 24));
+}
+
+// Scale and min `i` (0..8) of a Q4_K block from its 12 packed bytes held as three dwords.
+__device__ __forceinline__ void scale_min_k4(uint32_t i, uint32_t d0, uint32_t d1, uint32_t d2, uint32_t& sc, uint32_t& mn) {
+    uint32_t sh = 8 * (i & 3);
+    uint32_t a = (d0 >> sh) & 0xFF, b = (d1 >> sh) & 0xFF, c = (d2 >> sh) & 0xFF;
+    if (i < 4) {
+        sc = a & 63;
+        mn = b & 63;
+    } else {
+        sc = (c & 15) | ((a >> 6) << 4);
+        mn = (c >> 4) | ((b >> 6) << 4);
+    }
+}
+
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
+
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, true));
+}
+// Sum over the 64 lanes of a wavefront, result in every lane: DPP inside rows of 16, then the
+// cross-row exchanges.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141>(v);  // row_half_mirror
+    v += dpp_f32<0x140>(v);  // row_mirror
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+
+}  // namespace oxhip

@@ -1,0 +1,237 @@
+"""ctypes binding of liboxinfer_hip.so and `HipBackend`, the mirror of `trait Backend`
+(src/gpu.rs:151-294 of the reference): name / wants / upload / matmul / stats with the reference's
+conventions (False / None = declined, nothing written), plus the device-pointer entry points.
+
+Device buffers are torch tensors (torch is plumbing for memory and streams only).
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "liboxinfer_hip.so")
+
+W_BF16, W_Q8, W_Q4, W_GGUF, W_MLX_Q4 = 0, 1, 2, 3, 4
+GGML_Q8_0, GGML_Q4_K, GGML_Q6_K, GGML_F8E4M3 = 8, 12, 14, 0x1000
+GGML_BLOCK = {GGML_Q8_0: (32, 34), GGML_Q4_K: (256, 144), GGML_Q6_K: (256, 210)}
+
+
+class WeightDesc(C.Structure):
+    _fields_ = [("kind", C.c_uint32), ("ggml_type", C.c_uint32), ("n_out", C.c_size_t), ("n_in", C.c_size_t),
+                ("data", C.c_void_p), ("scales", C.c_void_p), ("offsets", C.c_void_p), ("group", C.c_uint32),
+                ("block_scales", C.c_void_p), ("bs_rows", C.c_uint32), ("bs_cols", C.c_uint32)]
+
+
+class Job(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("n_out", C.c_size_t), ("y", C.c_void_p)]
+
+
+class QActC(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("scales", C.c_void_p), ("sums", C.c_void_p), ("fsums", C.c_void_p),
+                ("hsums", C.c_void_p), ("sums16", C.c_void_p), ("t", C.c_size_t), ("n_in", C.c_size_t)]
+
+
+_lib = None
+
+
+def library_path():
+    return _SO
+
+
+def load_library():
+    """Loads liboxinfer_hip.so (built in-tree by `python -m oxinfer_amd.build`). Raises if it is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_SO):
+        raise RuntimeError(f"{_SO} is not built: run `python -m oxinfer_amd.build` (hipcc, gfx950). "
+                           "There is no CPU fallback in this package.")
+    try:
+        import torch  # noqa: F401  (its bundled HIP runtime must be the one this process uses)
+    except ImportError:
+        pass
+    lib = C.CDLL(_SO)
+    vp, sz = C.c_void_p, C.c_size_t
+    sig = {
+        "oxhip_open": (C.c_int, [C.c_int, C.POINTER(vp)]),
+        "oxhip_close": (None, [vp]),
+        "oxhip_name": (C.c_char_p, [vp]),
+        "oxhip_last_error": (C.c_char_p, []),
+        "oxhip_stats": (sz, [vp, C.c_char_p, sz]),
+        "oxhip_wants": (C.c_int, [vp, sz, sz, sz]),
+        "oxhip_upload": (vp, [vp, C.POINTER(WeightDesc)]),
+        "oxhip_free_weight": (None, [vp, vp]),
+        "oxhip_weight_bytes": (sz, [vp]),
+        "oxhip_matmul": (C.c_int, [vp, vp, sz, sz, C.POINTER(Job), sz]),
+        "oxhip_dev_quantize_act": (C.c_int, [vp, vp, sz, sz, C.POINTER(QActC), vp]),
+        "oxhip_dev_dequantize": (C.c_int, [vp, vp, sz, sz, vp, vp]),
+        "oxhip_dev_decode": (C.c_int, [vp, vp, C.POINTER(QActC), vp, sz, vp, vp]),
+        "oxhip_dev_isums": (C.c_int, [vp, vp, C.POINTER(QActC), vp, vp]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = res, args
+    _lib = lib
+    return lib
+
+
+def _np_ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+class DeviceWeight:
+    """`gpu::DeviceWeight` of one matrix (src/gpu.rs:57): freed when dropped."""
+
+    def __init__(self, be, handle, n_out, n_in):
+        self.be, self.handle, self.n_out, self.n_in = be, handle, n_out, n_in
+
+    @property
+    def bytes(self):
+        return load_library().oxhip_weight_bytes(self.handle)
+
+    def __del__(self):
+        if getattr(self, "handle", None) and self.be.ctx:
+            load_library().oxhip_free_weight(self.be.ctx, self.handle)
+            self.handle = None
+
+
+class QAct:
+    """`quant::QAct` (src/quant.rs:222-238) in device memory (torch tensors)."""
+
+    def __init__(self, t, n_in, device):
+        import torch
+        self.t, self.n_in = t, n_in
+        self.q = torch.empty((t, n_in), dtype=torch.int8, device=device)
+        self.scales = torch.empty((t, n_in // 32), dtype=torch.float32, device=device)
+        self.sums = torch.empty((t, n_in // 32), dtype=torch.int32, device=device)
+        self.fsums = torch.empty((t, n_in // 32), dtype=torch.float32, device=device)
+        self.hsums = torch.empty((t, n_in // 16), dtype=torch.float32, device=device)
+        self.sums16 = torch.empty((t, n_in // 16), dtype=torch.int32, device=device)
+        self.c = QActC(self.q.data_ptr(), self.scales.data_ptr(), self.sums.data_ptr(), self.fsums.data_ptr(),
+                       self.hsums.data_ptr(), self.sums16.data_ptr(), t, n_in)
+
+
+class HipBackend:
+    """Mirror of `impl Backend for CudaBackend` (src/cuda.rs) over the HIP library."""
+
+    def __init__(self, device=0):
+        self.lib = load_library()
+        ctx = C.c_void_p()
+        if not self.lib.oxhip_open(device, C.byref(ctx)):
+            raise RuntimeError("device hip: " + self.last_error())
+        self.ctx = ctx
+        self.device = device
+
+    def close(self):
+        if self.ctx:
+            self.lib.oxhip_close(self.ctx)
+            self.ctx = None
+
+    def last_error(self):
+        return (self.lib.oxhip_last_error() or b"").decode()
+
+    # ---- Backend surface -------------------------------------------------------------------
+    def name(self):
+        return self.lib.oxhip_name(self.ctx).decode()
+
+    def wants(self, n_out, n_in, t):
+        return bool(self.lib.oxhip_wants(self.ctx, n_out, n_in, t))
+
+    def stats(self):
+        buf = C.create_string_buffer(256)
+        self.lib.oxhip_stats(self.ctx, buf, 256)
+        return buf.value.decode()
+
+    def _upload(self, desc, keep):
+        h = self.lib.oxhip_upload(self.ctx, C.byref(desc))
+        del keep
+        return DeviceWeight(self, h, desc.n_out, desc.n_in) if h else None
+
+    def upload_gguf(self, ggml_type, data, n_out, n_in):
+        """WeightRef::Gguf: raw blocks, rows of `row_bytes` (src/ggml.rs:240-248)."""
+        data = np.ascontiguousarray(data, np.uint8)
+        bs, ts = GGML_BLOCK.get(ggml_type, (1, 0))
+        if ts and data.size != n_out * (n_in // bs) * ts:
+            raise ValueError("GGUF byte count does not match the shape")
+        d = WeightDesc(kind=W_GGUF, ggml_type=ggml_type, n_out=n_out, n_in=n_in, data=_np_ptr(data))
+        return self._upload(d, data)
+
+    def upload_fp8(self, data, block_scales, n_out, n_in, block=(128, 128)):
+        """GgufMatrix::fp8 (src/ggml.rs:325-341)."""
+        data = np.ascontiguousarray(data, np.uint8)
+        bs = np.ascontiguousarray(block_scales, np.float32)
+        d = WeightDesc(kind=W_GGUF, ggml_type=GGML_F8E4M3, n_out=n_out, n_in=n_in, data=_np_ptr(data),
+                       block_scales=_np_ptr(bs), bs_rows=block[0], bs_cols=block[1])
+        return self._upload(d, (data, bs))
+
+    def upload_q4(self, q, scales, offsets, group, n_out, n_in):
+        """WeightRef::Q4 (src/quant.rs:427-440): nibbles, f16 scales per 32, optional bf16 offsets."""
+        q, scales = np.ascontiguousarray(q, np.uint8), np.ascontiguousarray(scales, np.uint16)
+        offsets = None if offsets is None else np.ascontiguousarray(offsets, np.uint16)
+        d = WeightDesc(kind=W_Q4, n_out=n_out, n_in=n_in, data=_np_ptr(q), scales=_np_ptr(scales),
+                       offsets=_np_ptr(offsets), group=group if offsets is not None else 0)
+        return self._upload(d, (q, scales, offsets))
+
+    def upload_mlx_q4(self, w, scales, biases, group, n_out, n_in):
+        """The MLX triplet; the device does what from_mlx_q4 does (src/quant.rs:518-563)."""
+        w = np.ascontiguousarray(w, np.uint32)
+        scales, biases = np.ascontiguousarray(scales, np.uint16), np.ascontiguousarray(biases, np.uint16)
+        d = WeightDesc(kind=W_MLX_Q4, n_out=n_out, n_in=n_in, data=_np_ptr(w), scales=_np_ptr(scales),
+                       offsets=_np_ptr(biases), group=group)
+        return self._upload(d, (w, scales, biases))
+
+    def upload_bf16(self, w, n_out, n_in):
+        w = np.ascontiguousarray(w, np.uint16)
+        d = WeightDesc(kind=W_BF16, n_out=n_out, n_in=n_in, data=_np_ptr(w))
+        return self._upload(d, w)
+
+    def matmul(self, x, t, n_in, jobs):
+        """Backend::matmul: jobs = [(DeviceWeight, y ndarray [t, n_out] f32)]; True if every y was written."""
+        x = np.ascontiguousarray(x, np.float32)
+        arr = (Job * len(jobs))()
+        for i, (w, y) in enumerate(jobs):
+            assert y.dtype == np.float32 and y.flags.c_contiguous
+            arr[i] = Job(w.handle, w.n_out, y.ctypes.data)
+        return bool(self.lib.oxhip_matmul(self.ctx, _np_ptr(x), t, n_in, arr, len(jobs)))
+
+    # ---- device-pointer entry points -------------------------------------------------------
+    @staticmethod
+    def _stream():
+        import torch
+        return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def quantize_act(self, x, out=None):
+        """x: torch f32 [t, n_in] on the device -> QAct (device)."""
+        t, n_in = x.shape
+        out = out or QAct(t, n_in, x.device)
+        if not self.lib.oxhip_dev_quantize_act(self.ctx, x.data_ptr(), t, n_in, C.byref(out.c), self._stream()):
+            raise RuntimeError(self.last_error())
+        return out
+
+    def dequantize(self, w, r0=0, r1=None):
+        import torch
+        r1 = w.n_out if r1 is None else r1
+        out = torch.empty((r1 - r0, w.n_in), dtype=torch.float32, device=f"cuda:{self.device}")
+        if not self.lib.oxhip_dev_dequantize(self.ctx, w.handle, r0, r1, out.data_ptr(), self._stream()):
+            raise RuntimeError(self.last_error())
+        return out
+
+    def decode(self, w, xa=None, x=None, t=None, y=None):
+        """The decode kernels on device buffers: xa (QAct) for quantized weights, x (f32) for float-stored ones."""
+        import torch
+        t = t or (xa.t if xa is not None else x.shape[0])
+        if y is None:
+            y = torch.empty((t, w.n_out), dtype=torch.float32, device=f"cuda:{self.device}")
+        ok = self.lib.oxhip_dev_decode(self.ctx, w.handle, C.byref(xa.c) if xa is not None else None,
+                                       x.data_ptr() if x is not None else None, t, y.data_ptr(), self._stream())
+        if not ok:
+            raise RuntimeError(self.last_error())
+        return y
+
+    def isums(self, w, xa, per):
+        import torch
+        out = torch.empty((xa.t, w.n_out, w.n_in // per), dtype=torch.int32, device=f"cuda:{self.device}")
+        if not self.lib.oxhip_dev_isums(self.ctx, w.handle, C.byref(xa.c), out.data_ptr(), self._stream()):
+            raise RuntimeError(self.last_error())
+        return out

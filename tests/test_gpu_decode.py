@@ -1,0 +1,273 @@
+"""GPU parity of the decode path against the CPU oracle, through the C ABI.
+
+Bars: activation quantization, dequantized weights and the int32 accumulators bit-exact; matmul
+outputs within 1e-3 of the oracle's (f32 accumulation), measured like the reference's `row_err`
+(src/cuda.rs:1583-1592): worst error of a token row over that row's largest reference value.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def be():
+    import torch
+    assert torch.cuda.is_available(), "the gpu tests need a device"
+    from oxinfer_amd import HipBackend
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def row_err(y, ref):
+    m = np.maximum(np.abs(ref).max(axis=1), 1e-30)
+    return float((np.abs(y - ref).max(axis=1) / m).max())
+
+
+def lcg_input(t, n, seed, oxref):
+    """Token rows of very different magnitudes (src/cuda.rs:1579-1581), values from the reference's LCG."""
+    v, _ = oxref.lcg_stream(seed, t * n)
+    x = ((v >> 7).astype(np.float64) / float(1 << 24) - 0.5).astype(np.float32).reshape(t, n)
+    mags = np.array([1e-3, 1.0, 300.0, 2e5], np.float32)
+    return x * mags[np.arange(t) % 4][:, None]
+
+
+def test_name_and_wants(be):
+    assert be.name() == "hip (gfx950)"
+    assert be.wants(4096, 4096, 1) and not be.wants(64, 40, 1) and not be.wants(64, 64, 0)
+
+
+def test_quantize_act_bit_exact(be, oxref):
+    t, n = 7, 4 * 256 + 96
+    x = lcg_input(t, n, 7, oxref)
+    x[0, 32:64] = 0.0          # an all-zero block
+    x[0, 64 + 3] = 1e-30
+    x[1, :32] = -0.0           # an all -0.0 block: the sums stay -0.0
+    x[2, 5] = 3.0e38
+    x[3, 96:128] = np.float32(0.5)  # ties: every product is 127.0 or rounds half away
+    x[3, 97] = np.float32(0.5 * 64.5 / 127.0)
+    xa = be.quantize_act(dev(x))
+    q, scales, sums, fsums, hsums = oxref.quantize_act(x, t, n)
+    assert np.array_equal(xa.q.cpu().numpy(), q)
+    assert np.array_equal(xa.scales.cpu().numpy().view(np.uint32), scales.view(np.uint32))
+    assert np.array_equal(xa.sums.cpu().numpy(), sums)
+    assert np.array_equal(xa.fsums.cpu().numpy().view(np.uint32), fsums.view(np.uint32))
+    assert np.array_equal(xa.hsums.cpu().numpy().view(np.uint32), hsums.view(np.uint32))
+    s16 = q.astype(np.int32).reshape(t, n // 16, 16).sum(axis=2)
+    assert np.array_equal(xa.sums16.cpu().numpy(), s16)
+
+
+REF_HASHES = {Q8_0: 0x3199be3deddf5c1a, Q4_K: 0xde4da39c1d9096b2, Q6_K: 0x20a51cc0feaae638}
+
+
+@pytest.mark.parametrize("kind", [Q8_0, Q4_K, Q6_K])
+def test_gguf_dequant_matches_ggml_hash_on_device(be, oxref, kind):
+    """The device dequantizer reproduces the reference's golden hashes (src/ggml.rs:1547-1577)."""
+    raw, _ = oxref.random_blocks(kind, 1024 // oxref.block_size(kind), 1000 + kind)
+    w = be.upload_gguf(kind, raw, 1, 1024)
+    assert w is not None, be.last_error()
+    y = be.dequantize(w).cpu().numpy()
+    assert oxref.fnv1a_f32(y) == REF_HASHES[kind]
+
+
+@pytest.mark.parametrize("kind", [Q8_0, Q4_K, Q6_K])
+def test_gguf_dequant_and_isums_bit_exact(be, oxref, kind):
+    n_out, n_in, t = 37, 3 * 256, 5
+    raw, seed = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 13 + kind)
+    w = be.upload_gguf(kind, raw, n_out, n_in)
+    assert w is not None, be.last_error()
+    want = oxref.dequantize_rows(kind, raw, n_out, n_in)
+    got = be.dequantize(w).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    part = be.dequantize(w, 5, 9).cpu().numpy()
+    assert np.array_equal(part.view(np.uint32), want[5:9].view(np.uint32))
+    x = lcg_input(t, n_in, seed, oxref)
+    xa = be.quantize_act(dev(x))
+    _, isums = oxref.gguf_decode(kind, raw, n_out, n_in, x, t, want_isums=True)
+    got = be.isums(w, xa, 16).cpu().numpy()
+    assert np.array_equal(got, isums)
+
+
+@pytest.mark.parametrize("kind", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [1, 2, 3, 5, 8, 11, 16])
+def test_gguf_decode_matches_oracle(be, oxref, kind, t):
+    # rows not a multiple of the wave's row group; Q8_0 with a block count that is not a multiple of 4
+    n_out = 21
+    n_in = 3 * 256 + 96 if kind == Q8_0 else 3 * 256
+    raw, seed = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 77 + kind)
+    w = be.upload_gguf(kind, raw, n_out, n_in)
+    v, _ = oxref.lcg_stream(seed, t * n_in)
+    x = ((v % 2001).astype(np.float32) / np.float32(1000.0) - np.float32(1.0)).reshape(t, n_in)  # src/ggml.rs:1887
+    ref = oxref.gguf_decode(kind, raw, n_out, n_in, x, t)
+    y = be.decode(w, xa=be.quantize_act(dev(x))).cpu().numpy()
+    assert row_err(y, ref) < TOL
+    # batch invariance (src/ggml.rs:1829-1848): every token's row equals a one-token pass, bit for bit
+    for c in range(t):
+        y1 = be.decode(w, xa=be.quantize_act(dev(x[c:c + 1]))).cpu().numpy()
+        assert np.array_equal(y1[0].view(np.uint32), y[c].view(np.uint32)), c
+
+
+@pytest.mark.parametrize("kind", [Q8_0, Q4_K, Q6_K])
+def test_gguf_decode_row_magnitudes(be, oxref, kind):
+    n_out, n_in, t = 64, 4096, 4
+    raw, seed = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 5 + kind)
+    w = be.upload_gguf(kind, raw, n_out, n_in)
+    x = lcg_input(t, n_in, seed, oxref)
+    ref = oxref.gguf_decode(kind, raw, n_out, n_in, x, t)
+    y = be.decode(w, xa=be.quantize_act(dev(x))).cpu().numpy()
+    assert row_err(y, ref) < TOL
+
+
+def test_mlx_q4_repack_dequant_isums_decode(be, oxref):
+    from oxinfer_amd import synth
+    n_out, n_in, group = 37, 4160, 64  # src/kernels.rs:2458-2502 uses n_in = 4160
+    wq, sc, bi = synth.mlx_q4(n_out, n_in, 3, group)
+    # scales 0.002..0.012 and biases -8 s + 0.01 u as the reference's test draws them, plus scales in the
+    # f16 subnormal range and ones f16 cannot hold exactly
+    rng = np.random.default_rng(4)
+    sc = synth.bf16_bits((0.002 + 0.01 * np.abs(rng.uniform(-1, 1, sc.shape))).astype(np.float32))
+    sc[0, :4] = synth.bf16_bits(np.array([3e-6, 6.1e-5, 1e-7, 2.0 ** -17], np.float32))
+    sf = (sc.astype(np.uint32) << 16).view(np.float32)
+    bi = synth.bf16_bits((np.float32(-8.0) * sf + 0.01 * rng.uniform(-1, 1, sc.shape)).astype(np.float32))
+    q, s16, off = oxref.from_mlx_q4(wq, sc, bi, n_out, n_in, group)
+    want = oxref.dequant_rows_q4(q, s16, off, group, n_out, n_in)
+    for w in (be.upload_mlx_q4(wq, sc, bi, group, n_out, n_in), be.upload_q4(q, s16, off, group, n_out, n_in)):
+        assert w is not None, be.last_error()
+        got = be.dequantize(w).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        # invariant of the repack (src/kernels.rs:2484-2488)
+        assert np.abs(got - oxref.mlx_dequant_rows(wq, sc, bi, n_out, n_in)).max() < 2e-4
+        for t in (1, 2, 3, 5, 9):
+            x = lcg_input(t, n_in, 100 + t, oxref)
+            ref, isums = oxref.q4_decode(q, s16, off, group, n_out, n_in, x, t, want_isums=True)
+            xa = be.quantize_act(dev(x))
+            assert np.array_equal(be.isums(w, xa, 32).cpu().numpy(), isums)
+            y = be.decode(w, xa=xa).cpu().numpy()
+            assert row_err(y, ref) < TOL
+
+
+def test_q4_without_offsets_and_mixed_scales(be, oxref):
+    """A plain Q4_0-layout matrix (no offsets; src/quant.rs:457-513) keeps one scale per block of 32."""
+    n_out, n_in = 10, 512
+    rng = np.random.default_rng(9)
+    q = rng.integers(0, 256, (n_out, n_in // 2), dtype=np.uint8)
+    sc = np.abs(rng.normal(0, 0.01, (n_out, n_in // 32))).astype(np.float16).view(np.uint16)
+    x = lcg_input(3, n_in, 1, oxref)
+    for off, group in ((None, 0), (synth_offsets(n_out, n_in, 64), 64)):
+        w = be.upload_q4(q, sc, off, group, n_out, n_in)
+        assert w is not None, be.last_error()
+        want = oxref.dequant_rows_q4(q, sc, off, group or 32, n_out, n_in)
+        assert np.array_equal(be.dequantize(w).cpu().numpy().view(np.uint32), want.view(np.uint32))
+        ref = oxref.q4_decode(q, sc, off, group or 32, n_out, n_in, x, 3)
+        y = be.decode(w, xa=be.quantize_act(dev(x))).cpu().numpy()
+        assert row_err(y, ref) < TOL
+
+
+def synth_offsets(n_out, n_in, group):
+    from oxinfer_amd import synth
+    rng = np.random.default_rng(10)
+    return synth.bf16_bits(rng.normal(0, 0.05, (n_out, n_in // group)).astype(np.float32))
+
+
+def test_q4_integer_extremes(be, oxref):
+    """Nibbles 0 / 8 / 15 against +-127 activations with power-of-two scales: every f32 operation is exact,
+    so the outputs compare bit for bit (src/kernels_x86.rs:880-906)."""
+    n_out, n_in = 4, 96
+    for nib, xv in ((15, 127), (15, -127), (0, 127), (0, -127), (8, 127)):
+        q = np.full((n_out, n_in // 2), nib | (nib << 4), np.uint8)
+        sc = np.array([[0.5, 1.0, 2.0]] * n_out, np.float16).view(np.uint16)
+        x = np.full((1, n_in), np.float32(xv))
+        ref, isums = oxref.q4_decode(q, sc, None, 32, n_out, n_in, x, 1, want_isums=True)
+        w = be.upload_q4(q, sc, None, 0, n_out, n_in)
+        xa = be.quantize_act(dev(x))
+        assert np.array_equal(be.isums(w, xa, 32).cpu().numpy(), isums)
+        assert isums[0, 0, 0] == (nib - 8) * 127 * 32 * (1 if xv > 0 else -1)
+        y = be.decode(w, xa=xa).cpu().numpy()
+        assert np.array_equal(y.view(np.uint32), ref.view(np.uint32))
+
+
+def test_fp8_dequant_and_decode(be, oxref):
+    from oxinfer_amd import synth
+    n_out, n_in = 200, 512
+    data, scales = synth.fp8_e4m3(n_out, n_in, 11)
+    data[0, :256] = np.arange(256, dtype=np.uint8)  # every byte value, NaNs included
+    w = be.upload_fp8(data, scales, n_out, n_in)
+    assert w is not None, be.last_error()
+    want = oxref.fp8_dequant_rows(data, scales, n_out, n_in)
+    got = be.dequantize(w).cpu().numpy()
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan) and nan.sum() == 2
+    assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+    for t in (1, 3, 4, 7):
+        x = synth.activations(t, n_in, 12 + t, bf16=True)
+        ref = oxref.gemm_quant(oxref.F8E4M3, data, scales, None, n_out, n_in, x, t)
+        # float-stored rows take the f32 path for every t (src/kernels.rs:1802)
+        y = be.decode(w, x=dev(x)).cpu().numpy()
+        assert np.isnan(y[:, 0]).all() and np.isnan(ref[:, 0]).all()  # row 0 holds the NaN bytes
+        assert row_err(y[:, 1:], ref[:, 1:]) < TOL
+
+
+def test_fp8_rows_scale_blocks(oxref, be):
+    """Scale rows change every 128 weight rows; the row-1 dequant check above would miss a wrong row index."""
+    from oxinfer_amd import synth
+    n_out, n_in = 260, 256
+    data, scales = synth.fp8_e4m3(n_out, n_in, 21)
+    w = be.upload_fp8(data, scales, n_out, n_in)
+    x = synth.activations(2, n_in, 22, bf16=True)
+    ref = oxref.gemm_quant(oxref.F8E4M3, data, scales, None, n_out, n_in, x, 2)
+    assert row_err(be.decode(w, x=dev(x)).cpu().numpy(), ref) < TOL
+
+
+def test_host_matmul_matches_device_path_and_declines(be, oxref):
+    n_in = 512
+    raws = [(k, n, oxref.random_blocks(k, n * n_in // oxref.block_size(k), 31 + k)[0]) for k, n in ((Q4_K, 24), (Q6_K, 8), (Q8_0, 40))]
+    ws = [be.upload_gguf(k, raw, n, n_in) for k, n, raw in raws]
+    for t in (1, 3, 9):
+        x = lcg_input(t, n_in, 40 + t, oxref)
+        ys = [np.full((t, n), np.nan, np.float32) for _, n, _ in raws]
+        assert be.matmul(x, t, n_in, list(zip(ws, ys))), be.last_error()
+        for (k, n, raw), y in zip(raws, ys):
+            assert row_err(y, oxref.gguf_decode(k, raw, n, n_in, x, t)) < TOL
+    # a job whose weight has another n_in: declined, and nothing is written
+    other = be.upload_gguf(Q8_0, oxref.random_blocks(Q8_0, 8 * 64 // 32, 1)[0], 8, 64)
+    y0, y1 = np.full((1, 24), np.nan, np.float32), np.full((1, 8), np.nan, np.float32)
+    assert not be.matmul(lcg_input(1, n_in, 1, oxref), 1, n_in, [(ws[0], y0), (other, y1)])
+    assert np.isnan(y0).all() and np.isnan(y1).all() and "job 1" in be.last_error()
+    assert "calls" in be.stats()
+
+
+def test_upload_declines(be):
+    assert be.upload_gguf(2, np.zeros(18 * 4, np.uint8), 1, 128) is None  # Q4_0: no device kernels
+    assert "no device kernels" in be.last_error()
+    assert be.upload_gguf(Q4_K, np.zeros(144, np.uint8), 1, 256) is not None
+
+
+@pytest.mark.parametrize("kind,n_out,n_in", [(Q8_0, 14336, 4096), (Q4_K, 14336, 4096), (Q4_K, 4096, 14336), (Q6_K, 4096, 14336)])
+def test_full_size_rows_against_oracle(be, oxref, kind, n_out, n_in):
+    """The benchmark shapes: a sample of rows of the full-size product against the oracle, plus properties
+    that hold at any size: the all-ones-activation row sums and batch invariance."""
+    from oxinfer_amd import synth
+    gen = {Q8_0: synth.gguf_q8_0, Q4_K: synth.gguf_q4_k, Q6_K: synth.gguf_q6_k}[kind]
+    raw = gen(n_out, n_in, 1000 + kind)
+    w = be.upload_gguf(kind, raw, n_out, n_in)
+    assert w is not None, be.last_error()
+    rb = oxref.row_bytes(kind, n_in)
+    t = 8
+    x = synth.activations(t, n_in, 2000 + kind)
+    y = be.decode(w, xa=be.quantize_act(dev(x))).cpu().numpy()
+    rows = np.r_[0:8, n_out // 2 - 3:n_out // 2 + 3, n_out - 8:n_out, np.random.default_rng(1).integers(0, n_out, 44)]
+    sub = np.concatenate([raw[r * rb:(r + 1) * rb] for r in rows])
+    ref = oxref.gguf_decode(kind, sub, len(rows), n_in, x, t)
+    m = np.maximum(np.abs(y).max(axis=1), 1e-30)
+    assert float((np.abs(y[:, rows] - ref).max(axis=1) / m).max()) < TOL
+    y1 = be.decode(w, xa=be.quantize_act(dev(x[3:4]))).cpu().numpy()
+    assert np.array_equal(y1[0].view(np.uint32), y[3].view(np.uint32))
