@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-weight matmul path on one MI355X.
+
+Default workload = BASELINE.json configs[1]: GGUF GEMV at batch 1 and 8 over Llama-8B MLP shapes
+(4096->14336 and 14336->4096) in Q8_0 and Q4_K. One step = the eight matmuls of that set, each on
+the next of a rotating pool of distinct weight copies (>= 1.5 GB per format and shape) so the 256 MB
+Infinity Cache cannot serve them; activations are quantized on the device before the timed region
+(the kernels measured are the dequant-fused GEMVs). value = algorithmic bytes of a step / time.
+
+Prints ONE JSON line (see README / DESIGN.md for the fields). `--workload` selects other
+configurations for profiling runs; the default is what the driver records.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "quant GEMV GB/s (% of 8 TB/s); quant GEMM TFLOPS (% MFMA peak); vs CPU"
+HBM_PEAK_GBS = 8000.0
+POOL_BYTES = 1.5e9
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+ROW_BYTES = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
+FMT_NAME = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
+KERNEL_FMT = {Q8_0: 1, Q4_K: 2, Q6_K: 3}  # template argument in the kernel symbol
+
+
+def weight_bytes(kind, n_out, n_in):
+    bs, ts = ROW_BYTES[kind]
+    return n_out * (n_in // bs) * ts
+
+
+def algorithmic_bytes(kind, n_out, n_in, t):
+    """Format-native weight bytes + the quantized activations read (int8 + f32 scale per 32, + f32 half sums
+    and int32 sums per 16 where the format uses them) + the f32 outputs written, each counted once."""
+    act = t * (n_in + n_in // 32 * 4)
+    if kind == Q4_K:
+        act += t * (n_in // 16) * 8
+    elif kind == Q6_K:
+        act += t * (n_in // 16) * 4
+    return weight_bytes(kind, n_out, n_in) + act + t * n_out * 4
+
+
+def gemv_cases(kinds):
+    cases = []
+    for kind in kinds:
+        for n_in, n_out in ((4096, 14336), (14336, 4096)):
+            for t in (1, 8):
+                cases.append(dict(kind=kind, n_out=n_out, n_in=n_in, t=t,
+                                  name=f"{FMT_NAME[kind]}_{n_in}x{n_out}_t{t}",
+                                  bytes=algorithmic_bytes(kind, n_out, n_in, t)))
+    return cases
+
+
+def cpu_baseline(cases, gens, seconds=20.0):
+    """The oracle's AVX2 restatement of the reference's x86 decode kernels, scheduled like
+    matmul_quant_multi_at over all host cores, on the same eight matmuls: best of 5 per case over rotating
+    weight copies (so the caches do not help). Tokens up to 8 take the int-dot kernels, as with
+    set_decode_max_tokens(8) in the reference's kernel_bench."""
+    from oracle import oxref
+    from oxinfer_amd import synth
+    threads = oxref.hw_threads()
+    total_bytes, total_s, per = 0, 0.0, {}
+    t_start = time.time()
+    host = {}
+    for c in cases:
+        key = (c["kind"], c["n_out"], c["n_in"])
+        if key not in host:
+            raw = gens[c["kind"]](c["n_out"], c["n_in"], 1)
+            ncopies = max(2, int(np.ceil(4.0e8 / raw.size)))  # 0.4 GB per shape: well past the host caches
+            host[key] = [raw] + [raw.copy() for _ in range(ncopies - 1)]
+        x = synth.activations(c["t"], c["n_in"], 5)
+        best = float("inf")
+        copies = host[key]
+        reps = 0
+        while reps < 5 or (reps < 50 and time.time() - t_start < seconds * 0.1):
+            raw = copies[reps % len(copies)]
+            t0 = time.perf_counter()
+            oxref.gguf_decode(c["kind"], raw, c["n_out"], c["n_in"], x, c["t"], avx2=True, threads=threads)
+            best = min(best, time.perf_counter() - t0)
+            reps += 1
+        per[c["name"]] = round(weight_bytes(c["kind"], c["n_out"], c["n_in"]) / best / 1e9, 2)
+        total_bytes += c["bytes"]
+        total_s += best
+    return {"value": round(total_bytes / total_s / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "the 8 matmuls of one step, best of >=5 runs each over rotating weight copies; C++ AVX2 "
+                      "restatement of kernels_ggml_x86 (int8 dot path, decode_max_tokens >= 8), activation "
+                      "quantization included",
+            "per_case_weight_GBs": per}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="gguf_gemv", choices=["gguf_gemv", "gguf_gemv_q6k"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--pool-gb", type=float, default=POOL_BYTES / 1e9)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus must be 1 (nothing here uses a second device)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from oxinfer_amd import HipBackend, synth
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    be = HipBackend(0)
+    gens = {Q8_0: synth.gguf_q8_0, Q4_K: synth.gguf_q4_k, Q6_K: synth.gguf_q6_k}
+    kinds = [Q8_0, Q4_K] if args.workload == "gguf_gemv" else [Q6_K]
+    cases = gemv_cases(kinds)
+
+    # rotating pools of distinct device copies per (format, shape)
+    pools = {}
+    for c in cases:
+        key = (c["kind"], c["n_out"], c["n_in"])
+        if key in pools:
+            continue
+        raw = gens[c["kind"]](c["n_out"], c["n_in"], 1)
+        n = max(2, int(np.ceil(args.pool_gb * 1e9 / raw.size)))
+        pools[key] = []
+        for _ in range(n):
+            w = be.upload_gguf(c["kind"], raw, c["n_out"], c["n_in"])
+            if w is None:
+                raise RuntimeError(be.last_error())
+            pools[key].append(w)
+    for c in cases:
+        x = torch.from_numpy(synth.activations(c["t"], c["n_in"], 5)).cuda()
+        c["xa"] = be.quantize_act(x)
+        c["y"] = torch.empty((c["t"], c["n_out"]), dtype=torch.float32, device="cuda")
+        c["pool"] = pools[(c["kind"], c["n_out"], c["n_in"])]
+    torch.cuda.synchronize()
+
+    # the dominant kernel: the largest algorithmic bytes at the larger batch (same symbol for both shapes)
+    dom_kind = kinds[0]
+    for c in cases:
+        c["dom"] = c["kind"] == dom_kind and c["t"] == 8
+    dom = [c for c in cases if c["dom"]]
+    dom_symbol = f"decode_kernel<{KERNEL_FMT[dom_kind]}, 8, 4>"
+
+    # One call per step: the job arrays (one per rotation phase) are built once; the dominant launches carry
+    # HIP events recorded on the launch stream.
+    n_ev = args.steps * len(dom)
+    ev = [(be.event(), be.event()) for _ in range(min(n_ev, 4096))]
+
+    def jobs_for(i, timed_slot=None):
+        jobs, k = [], 0
+        for c in cases:
+            w = c["pool"][(2 * i + (c["t"] > 1)) % len(c["pool"])]
+            e0 = e1 = None
+            if timed_slot is not None and c["dom"]:
+                e0, e1 = ev[(timed_slot * len(dom) + k) % len(ev)]
+                k += 1
+            jobs.append((w, c["xa"], None, c["t"], c["y"], e0, e1))
+        return be.decode_jobs(jobs)
+
+    warm = [jobs_for(i) for i in range(args.warmup)]
+    timed = [jobs_for(args.warmup + i, i) for i in range(args.steps)]
+    for arr in warm:
+        be.decode_batch(arr)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for arr in timed:
+        be.decode_batch(arr)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    used = min(n_ev, len(ev))
+    dom_ms = [be.elapsed_ms(a, b) for a, b in ev[:used]]
+
+    step_bytes = sum(c["bytes"] for c in cases)
+    value = step_bytes * args.steps / elapsed / 1e9
+    dom_avg_s = float(np.mean(dom_ms)) / 1e3
+    dom_bytes = float(np.mean([c["bytes"] for c in dom]))
+    achieved = dom_bytes / dom_avg_s / 1e9
+
+    # per-case detail (untimed pass, one event pair per launch)
+    detail = {}
+    for c in cases:
+        ms = []
+        for i in range(30):
+            w = c["pool"][i % len(c["pool"])]
+            arr = be.decode_jobs([(w, c["xa"], None, c["t"], c["y"], ev[0][0], ev[0][1])])
+            be.decode_batch(arr)
+            ms.append(be.elapsed_ms(ev[0][0], ev[0][1]))
+        us = float(np.median(ms)) * 1e3
+        detail[c["name"]] = {"us": round(us, 2), "GBs": round(c["bytes"] / us / 1e3, 1),
+                             "frac_hbm": round(c["bytes"] / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+    out = {
+        "metric": METRIC, "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(elapsed / args.steps * 1e3, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "configs[1]: GGUF GEMV batch 1 and 8, Llama-8B MLP shapes 4096->14336 and 14336->4096, "
+                               + " + ".join(FMT_NAME[k] for k in kinds),
+                   "launches_per_step": len(cases), "bytes_per_step": step_bytes,
+                   "weight_pool_GB_per_shape": args.pool_gb, "activations": "int8 per 32 (quantize_act), resident in HBM"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom_symbol,
+                     "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_avg_s * 1e6, 2)},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "detail": detail,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(cases, gens)
+    print(json.dumps(out))
+    be.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -119,8 +119,27 @@ int oxhip_dev_dequantize(oxhip_ctx* ctx, const oxhip_weight* w, size_t r0, size_
  * (`dense`, src/ggml.rs:1370): they take f32 rows `x` instead and `xa` may be NULL. */
 int oxhip_dev_decode(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa, const float* x, size_t t, float* y,
                      void* stream);
-/* The exact integer accumulators of the decode kernels: per block of 32 for Q4
- * ([t, n_out, n_in/32]), per 16 for GGUF ([t, n_out, n_in/16]). For parity checks. */
+/* Several decode launches in one call (a decode step issues many small matmuls; what
+ * matmul_quant_batch does for the CPU, src/kernels.rs:1937-1994). Jobs run in order on `stream`;
+ * ev_start / ev_stop (from oxhip_event_create, or NULL) are recorded around that job's launches. */
+typedef struct {
+    const oxhip_weight* w;
+    const oxhip_qact* xa; /* quantized weights */
+    const float* x;       /* float-stored weights */
+    size_t t;
+    float* y;
+    void* ev_start;
+    void* ev_stop;
+} oxhip_decode_job;
+int oxhip_dev_decode_batch(oxhip_ctx* ctx, const oxhip_decode_job* jobs, size_t n_jobs, void* stream);
+/* HIP events for timing launches on a stream (Backend::stats-style measurement without a profiler). */
+void* oxhip_event_create(void);
+void oxhip_event_destroy(void* ev);
+/* Milliseconds between two recorded events; waits for `stop`. Negative on error. */
+float oxhip_event_elapsed_ms(void* start, void* stop);
+/* The exact integer accumulators of the decode kernels, written by the kernels themselves: per
+ * block of 32 ([t, n_out, n_in/32]) for Q4, Q8_0 and Q4_K, per 16 ([t, n_out, n_in/16]) for Q6_K.
+ * For parity checks (the CPU's per-16 sums add up to the per-32 ones exactly). */
 int oxhip_dev_isums(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa, int32_t* out, void* stream);
 
 #ifdef __cplusplus

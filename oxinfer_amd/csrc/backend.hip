@@ -7,6 +7,7 @@
 #include <vector>
 
 #include "internal.hpp"
+#include "layout.hpp"
 
 namespace oxhip {
 
@@ -332,17 +333,15 @@ oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) {
             if (d->ggml_type == OXHIP_GGML_Q8_0) {
                 if (n_in % 32) return fail("Q8_0 rows must be whole blocks of 32");
                 w->v.fmt = FMT_Q8_0;
-                pl.add(0, n_out * n_in);
-                pl.add(1, n_out * (n_in / 32) * 2);
+                pl.add(0, t8_bytes((uint32_t)n_out, (uint32_t)n_in));
                 raw_bytes = n_out * (n_in / 32) * 34;
-                np = 2;
+                np = 1;
             } else if (d->ggml_type == OXHIP_GGML_Q4_K) {
                 if (n_in % 256) return fail("Q4_K rows must be whole blocks of 256");
                 w->v.fmt = FMT_Q4_K;
-                pl.add(0, n_out * (n_in / 256) * 128);
-                pl.add(1, n_out * (n_in / 256) * 16);
+                pl.add(0, tk4_bytes((uint32_t)n_out, (uint32_t)n_in));
                 raw_bytes = n_out * (n_in / 256) * 144;
-                np = 2;
+                np = 1;
             } else if (d->ggml_type == OXHIP_GGML_Q6_K) {
                 if (n_in % 256) return fail("Q6_K rows must be whole blocks of 256");
                 w->v.fmt = FMT_Q6_K;
@@ -367,6 +366,25 @@ oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) {
         default: return fail("weight kind " + std::to_string(d->kind) + " has no device kernels");
     }
     if (hipStreamSynchronize(s) != hipSuccess) return fail("upload failed");
+    if (w->v.fmt == FMT_Q4 && w->v.group == 64 && w->v.sgroup == 64) {
+        // one scale and one offset per 64 (MLX checkpoints): tile-packed for the matrix cores
+        const size_t bytes = t4m_bytes((uint32_t)n_out, (uint32_t)n_in);
+        void* packed = nullptr;
+        if (have_memory(bytes) && hipMalloc(&packed, bytes) == hipSuccess) {
+            if (launch_pack_q4m(w->v.p0, reinterpret_cast<const uint16_t*>(w->v.p1), reinterpret_cast<const uint16_t*>(w->v.p2), n_out,
+                                n_in, static_cast<uint8_t*>(packed), s) != hipSuccess ||
+                hipStreamSynchronize(s) != hipSuccess) {
+                (void)hipFree(packed);
+                return fail("tile packing failed");
+            }
+            (void)hipFree(w->base);
+            w->base = packed;
+            w->bytes = bytes;
+            w->v.fmt = FMT_Q4M;
+            w->v.p0 = static_cast<const uint8_t*>(packed);
+            w->v.p1 = w->v.p2 = nullptr;
+        }
+    }
     return w;
 }
 
@@ -409,6 +427,42 @@ int oxhip_dev_decode(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa, 
     }
     HIP_TRY(launch_decode(w->v, v, x, t, y, static_cast<hipStream_t>(stream)), "decode launch");
     return 1;
+}
+
+int oxhip_dev_decode_batch(oxhip_ctx* c, const oxhip_decode_job* jobs, size_t n_jobs, void* stream) {
+    if (!c || (!jobs && n_jobs)) {
+        set_error("decode_batch: bad arguments");
+        return 0;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    for (size_t j = 0; j < n_jobs; j++) {
+        const oxhip_decode_job& jb = jobs[j];
+        if (jb.ev_start) HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jb.ev_start), s), "event record");
+        if (!oxhip_dev_decode(c, jb.w, jb.xa, jb.x, jb.t, jb.y, stream)) return 0;
+        if (jb.ev_stop) HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jb.ev_stop), s), "event record");
+    }
+    return 1;
+}
+
+void* oxhip_event_create(void) {
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) {
+        set_error("hipEventCreate failed");
+        return nullptr;
+    }
+    return e;
+}
+
+void oxhip_event_destroy(void* ev) {
+    if (ev) (void)hipEventDestroy(static_cast<hipEvent_t>(ev));
+}
+
+float oxhip_event_elapsed_ms(void* a, void* b) {
+    float ms = -1.0f;
+    if (!a || !b) return ms;
+    if (hipEventSynchronize(static_cast<hipEvent_t>(b)) != hipSuccess) return -1.0f;
+    if (hipEventElapsedTime(&ms, static_cast<hipEvent_t>(a), static_cast<hipEvent_t>(b)) != hipSuccess) return -1.0f;
+    return ms;
 }
 
 int oxhip_dev_isums(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa, int32_t* out, void* stream) {

@@ -1,5 +1,6 @@
-// Decode kernels: dequant-fused GEMV / skinny GEMM over int8 activations, one wavefront per
-// group of R weight rows.
+// Decode kernels on the vector ALUs (v_dot4_i32_i8) for the formats stored in planes (Q6_K, Q4
+// with per-32 scales) and for float-stored weights: dequant-fused GEMV / skinny GEMM, one wavefront
+// per group of R weight rows. Q8_0, Q4_K and MLX Q4 run on the matrix cores (decode_mfma.hip).
 //
 // What they compute is what the reference's CPU decode kernels compute (QMat::rows_t1 / rows_tc,
 // src/kernels.rs:1339-1369; dot_row_generic, src/ggml.rs:1288-1315; q4_dot_rows_tc_scalar,
@@ -76,74 +77,6 @@ struct F<FMT_Q4> {
         int i;
         isums(w, a, &i);
         return ((float)i * w.d) * a[0].xs;
-    }
-};
-
-// ---- Q8_0: unit = half a block (16 int8) ----------------------------------------------------------
-template <>
-struct F<FMT_Q8_0> {
-    static constexpr int NG = 1;
-    static constexpr bool MIN = false, S16 = false;
-    static constexpr int ISUMS_PER_UNIT = 1;
-    struct W {
-        uint4 q;
-        float d;
-    };
-    __device__ static uint32_t units(const WeightView& w) { return w.n_in / 16; }
-    __device__ static uint32_t group(uint32_t u, int) { return u; }
-    __device__ static void load(const WeightView& w, uint32_t r, uint32_t u, W& o) {
-        o.q = *reinterpret_cast<const uint4*>(w.p0 + (size_t)r * w.n_in + (size_t)u * 16);
-        o.d = f16_bits_to_f32(reinterpret_cast<const uint16_t*>(w.p1)[(size_t)r * (w.n_in / 32) + u / 2]);
-    }
-    __device__ static void isums(const W& w, const ActG* a, int* out) { out[0] = dot16(w.q, a[0].xq); }
-    __device__ static float dot(const W& w, const ActG* a) {
-        int i;
-        isums(w, a, &i);
-        return (w.d * a[0].xs) * (float)i;
-    }
-};
-
-// ---- Q4_K: unit = 16 bytes of qs: 16 low nibbles of sub-block 2j, 16 high nibbles of 2j+1 ---------
-template <>
-struct F<FMT_Q4_K> {
-    static constexpr int NG = 2;
-    static constexpr bool MIN = true, S16 = true;
-    static constexpr int ISUMS_PER_UNIT = 2;
-    struct W {
-        uint4 lo, hi;
-        float s_lo, s_hi, m_lo, m_hi;
-    };
-    __device__ static uint32_t units(const WeightView& w) { return w.n_in / 32; }
-    // unit u = 8 sb + 2 j + half covers elements 64 j + 16 half .. (low) and 64 j + 32 + 16 half .. (high)
-    __device__ static uint32_t group(uint32_t u, int g) { return 2 * u - (u & 1) + 2 * g; }
-    __device__ static void load(const WeightView& w, uint32_t r, uint32_t u, W& o) {
-        size_t nb = w.n_in / 256;
-        uint32_t sb = u >> 3, j = (u >> 1) & 3;
-        uint4 v = *reinterpret_cast<const uint4*>(w.p0 + ((size_t)r * nb * 8 + u) * 16);
-        uint4 mt = *reinterpret_cast<const uint4*>(w.p1 + ((size_t)r * nb + sb) * 16);
-        o.lo = lo_nibbles(v);
-        o.hi = hi_nibbles(v);
-        float d = f16_bits_to_f32((uint16_t)(mt.x & 0xFFFF)), dmin = f16_bits_to_f32((uint16_t)(mt.x >> 16));
-        uint32_t sc0, mn0, sc1, mn1;
-        scale_min_k4(2 * j, mt.y, mt.z, mt.w, sc0, mn0);
-        scale_min_k4(2 * j + 1, mt.y, mt.z, mt.w, sc1, mn1);
-        o.s_lo = d * (float)sc0;
-        o.s_hi = d * (float)sc1;
-        o.m_lo = 8.0f * o.s_lo - dmin * (float)mn0;
-        o.m_hi = 8.0f * o.s_hi - dmin * (float)mn1;
-    }
-    __device__ static void isums(const W& w, const ActG* a, int* out) {
-        out[0] = dot16(w.lo, a[0].xq) - 8 * a[0].s16;
-        out[1] = dot16(w.hi, a[1].xq) - 8 * a[1].s16;
-    }
-    __device__ static float dot(const W& w, const ActG* a) {
-        int i[2];
-        isums(w, a, i);
-        float sum = (w.s_lo * a[0].xs) * (float)i[0];
-        sum += (w.s_hi * a[1].xs) * (float)i[1];
-        sum += w.m_lo * a[0].hs;
-        sum += w.m_hi * a[1].hs;
-        return sum;
     }
 };
 
@@ -401,9 +334,10 @@ hipError_t decode_dense_t(const WeightView& w, const float* x, size_t t, float* 
 
 hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s) {
     switch (w.fmt) {
+        case FMT_Q8_0:
+        case FMT_Q4_K:
+        case FMT_Q4M: return launch_decode_mfma(w, xa, t, y, s);
         case FMT_Q4: return decode_t<FMT_Q4, 4>(w, xa, t, y, s);
-        case FMT_Q8_0: return decode_t<FMT_Q8_0, 4>(w, xa, t, y, s);
-        case FMT_Q4_K: return decode_t<FMT_Q4_K, 4>(w, xa, t, y, s);
         case FMT_Q6_K: return decode_t<FMT_Q6_K, 4>(w, xa, t, y, s);
         case FMT_FP8: return decode_dense_t<FMT_FP8, 4>(w, x, t, y, s);
         case FMT_BF16: return decode_dense_t<FMT_BF16, 4>(w, x, t, y, s);
@@ -412,13 +346,12 @@ hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x
 }
 
 hipError_t launch_isums(const WeightView& w, const QActView& xa, size_t t, int32_t* out, hipStream_t s) {
-    size_t units = w.fmt == FMT_Q8_0 ? w.n_in / 16 : w.n_in / 32;
+    if (w.fmt == FMT_Q8_0 || w.fmt == FMT_Q4_K || w.fmt == FMT_Q4M) return launch_isums_mfma(w, xa, t, nullptr, out, s);
+    size_t units = w.n_in / 32;
     size_t total = t * w.n_out * units;
     unsigned grid = (unsigned)((total + 255) / 256);
     switch (w.fmt) {
         case FMT_Q4: isums_kernel<FMT_Q4><<<grid, 256, 0, s>>>(w, xa, (uint32_t)t, out); break;
-        case FMT_Q8_0: isums_kernel<FMT_Q8_0><<<grid, 256, 0, s>>>(w, xa, (uint32_t)t, out); break;
-        case FMT_Q4_K: isums_kernel<FMT_Q4_K><<<grid, 256, 0, s>>>(w, xa, (uint32_t)t, out); break;
         case FMT_Q6_K: isums_kernel<FMT_Q6_K><<<grid, 256, 0, s>>>(w, xa, (uint32_t)t, out); break;
         default: return hipErrorInvalidValue;
     }

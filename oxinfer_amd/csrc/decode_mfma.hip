@@ -1,0 +1,360 @@
+// Decode (1..8 tokens) on the matrix cores: a dequant-fused skinny GEMM over int8 activations.
+//
+// The arithmetic is the CPU decode kernels' (QMat::rows_t1 / rows_tc, src/kernels.rs:1339-1369;
+// dot_row_generic, src/ggml.rs:1288-1315 of the reference): exact int32 sums of int8 weight codes
+// times int8 activations per block of 32, scaled in f32 by weight scale x activation scale, plus
+// the min / offset terms over the exact f32 activation sums. Each (token, row) result depends on
+// that token alone and is summed in a fixed order, so a token's row is bit-identical whatever
+// the batch (the reference's batch invariance, src/ggml.rs:1829-1848).
+//
+// Mapping onto v_mfma_i32_16x16x64_i8 (D[m][n] += sum_k A[m][k] B[k][n], lane l = 16 kq + idx
+// supplies 16 K-bytes of row idx of A and of column idx of B, and receives D[4 kq + i][idx]):
+//   B = weights: column n is row n of a 16-row tile; a lane's bytes 0-7 are 8 codes of one block of
+//       32 and bytes 8-15 the 8 codes of the next block at the same positions;
+//   A = activations: row m = 8 half + token carries token's int8 values of block `half` of the pair
+//       in the matching byte half and zeros in the other, so that D[8 half + token][n] is the
+//       integer dot product of one whole block: one instruction yields 2 blocks x 8 tokens x 16
+//       rows of exact block sums, and every output lane is useful at 8 tokens.
+// Weights stream from HBM through a register ring (several 1 KiB records in flight per wave, see
+// layout.hpp); the activations' int8 values come from L2 / L1 (they are shared by every wave),
+// their per-block scales and sums are staged once per workgroup into LDS, transposed so that a
+// lane reads the four tokens it owns with one ds_read_b128.
+//
+// A workgroup owns `rt` row tiles and splits K over `kw` waves per tile; the partial sums meet in
+// LDS in a fixed order. No atomics, no second launch.
+#include "internal.hpp"
+#include "layout.hpp"
+
+namespace oxhip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int PF = 4;  // records in flight per wave beyond the one being consumed
+
+struct Meta4 {
+    float xs[4];
+    int su[4];
+    float fs[4];
+};
+
+// LDS: xs | su | fs, each [nblk][TPAD] (su, fs only for the formats that use them)
+template <int TPAD, bool SUMS>
+__device__ __forceinline__ void stage_meta(const QActView& xa, uint32_t t, uint32_t nblk, float* lds) {
+    float* xs = lds;
+    int* su = reinterpret_cast<int*>(lds + (size_t)nblk * TPAD);
+    float* fs = lds + (size_t)2 * nblk * TPAD;
+    for (uint32_t i = threadIdx.x; i < nblk * TPAD; i += blockDim.x) {
+        uint32_t tok = i / nblk, b = i % nblk;  // consecutive threads read consecutive blocks of one token
+        bool live = tok < t;
+        size_t src = (size_t)tok * nblk + b;
+        xs[b * TPAD + tok] = live ? xa.scales[src] : 0.0f;
+        if (SUMS) {
+            su[b * TPAD + tok] = live ? xa.sums[src] : 0;
+            fs[b * TPAD + tok] = live ? xa.fsums[src] : 0.0f;
+        }
+    }
+}
+
+template <int TPAD, bool SUMS>
+__device__ __forceinline__ void load_meta(const float* lds, uint32_t nblk, uint32_t b, uint32_t tok0, Meta4& m) {
+    const float4 x = *reinterpret_cast<const float4*>(lds + (size_t)b * TPAD + tok0);
+    m.xs[0] = x.x; m.xs[1] = x.y; m.xs[2] = x.z; m.xs[3] = x.w;
+    if (SUMS) {
+        const int4 s = *reinterpret_cast<const int4*>(lds + (size_t)nblk * TPAD + (size_t)b * TPAD + tok0);
+        const float4 f = *reinterpret_cast<const float4*>(lds + (size_t)2 * nblk * TPAD + (size_t)b * TPAD + tok0);
+        m.su[0] = s.x; m.su[1] = s.y; m.su[2] = s.z; m.su[3] = s.w;
+        m.fs[0] = f.x; m.fs[1] = f.y; m.fs[2] = f.z; m.fs[3] = f.w;
+    }
+}
+
+}  // namespace
+
+// FMT: FMT_Q8_0 / FMT_Q4_K / FMT_Q4M. NT: tokens handled (1, 2, 4 or 8). DUMP: also write the exact
+// integer block sums to `dump` ([t][n_out][n_in/32]) for parity checks.
+template <int FMT, int NT, bool DUMP>
+__global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw,
+                                                           float* __restrict__ y, int32_t* __restrict__ dump) {
+    constexpr int TPAD = NT <= 4 ? 4 : 8;
+    constexpr int NI = NT < 4 ? NT : 4;          // accumulator registers that hold live tokens
+    constexpr bool SUMS = FMT != FMT_Q8_0;
+    extern __shared__ float lds[];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t n = lane & 15, kq = lane >> 4;  // B / D role: row n of the tile; A role: slot n
+    const uint32_t nblk = w.n_in / 32;
+    const uint32_t r = wave / kw, ks = wave % kw;
+    const uint32_t tile = blockIdx.x * rt + r;
+    const uint32_t ntiles = row_tiles(w.n_out);
+
+    stage_meta<TPAD, SUMS>(xa, t, nblk, lds);
+    __syncthreads();
+    float* red = lds + (size_t)(SUMS ? 3 : 1) * nblk * TPAD;  // [rt * kw][TPAD][16]
+
+    // A role: slot n of this lane = (half, token); tokens past t read token t - 1 (their sums are dropped)
+    const uint32_t a_half = n >> 3, a_tok = min(n & 7u, t - 1);
+    const int8_t* xrow = xa.q + (size_t)a_tok * w.n_in;
+    const uint32_t amask0 = a_half ? 0u : 0xFFFFFFFFu, amask1 = ~amask0;
+    // D role: this lane's registers are tokens 4 (kq & 1) + i of block parity kq >> 1
+    const uint32_t d_half = kq >> 1, d_tok0 = 4 * (kq & 1);
+
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bool live_tile = tile < ntiles;
+
+    // One MFMA over a pair of blocks (b0 for half 0, b1 for half 1) with weight codes `bw`
+    auto block_pair = [&](v4i bw, uint32_t b0, uint32_t b1, uint32_t apos0, uint32_t apos1, bool split) -> v4i {
+        const uint32_t ab = min(a_half ? b1 : b0, nblk - 1);
+        uint32_t d0, d1;
+        if (split) {  // Q4M: positions 4 kq.. and 16 + 4 kq..
+            d0 = *reinterpret_cast<const uint32_t*>(xrow + ab * 32 + apos0);
+            d1 = *reinterpret_cast<const uint32_t*>(xrow + ab * 32 + apos1);
+        } else {
+            const uint2 v = *reinterpret_cast<const uint2*>(xrow + ab * 32 + apos0);
+            d0 = v.x;
+            d1 = v.y;
+        }
+        v4i a = {(int)(d0 & amask0), (int)(d1 & amask0), (int)(d0 & amask1), (int)(d1 & amask1)};
+        v4i c = {0, 0, 0, 0};
+        return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bw, c, 0, 0, 0);
+    };
+    auto dump_block = [&](uint32_t b, const int* isum) {
+        if (!DUMP) return;
+        const uint32_t row = tile * 16 + n;
+        if (b >= nblk || row >= w.n_out) return;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (d_tok0 + i < t) dump[((size_t)(d_tok0 + i) * w.n_out + row) * nblk + b] = isum[i];
+    };
+
+    if (live_tile) {
+        if (FMT == FMT_Q8_0) {
+            const uint32_t nsteps = t8_steps(w.n_in);
+            const uint32_t per = (nsteps + kw - 1) / kw;
+            const uint32_t s0 = ks * per, s1 = min(nsteps, s0 + per);
+            const uint8_t* base = w.p0 + (size_t)tile * nsteps * T8_REC;
+            uint4 ring[PF];
+#pragma unroll
+            for (int p = 0; p < PF; p++)
+                if (s0 + p < s1) ring[p] = *reinterpret_cast<const uint4*>(base + (size_t)(s0 + p) * T8_REC + 16 * lane);
+            for (uint32_t sb = s0; sb < s1; sb += PF) {
+                uint4 next[PF];
+#pragma unroll
+                for (int p = 0; p < PF; p++)
+                    if (sb + PF + p < s1) next[p] = *reinterpret_cast<const uint4*>(base + (size_t)(sb + PF + p) * T8_REC + 16 * lane);
+#pragma unroll
+                for (int p = 0; p < PF; p++) {
+                    const uint32_t s = sb + p;
+                    if (s >= s1) break;
+                    const uint4 c = ring[p];
+                    const uint32_t dd = *reinterpret_cast<const uint32_t*>(base + (size_t)s * T8_REC + 1024 + 4 * n);
+                    const float d = f16_bits_to_f32((uint16_t)(d_half ? dd >> 16 : dd & 0xFFFF));
+                    v4i bw = {(int)c.x, (int)c.y, (int)c.z, (int)c.w};
+                    v4i D = block_pair(bw, 2 * s, 2 * s + 1, 8 * kq, 0, false);
+                    const uint32_t b = 2 * s + d_half;
+                    Meta4 m;
+                    load_meta<TPAD, SUMS>(lds, nblk, min(b, nblk - 1), d_tok0, m);
+                    int isum[4] = {D.x, D.y, D.z, D.w};
+#pragma unroll
+                    for (int i = 0; i < NI; i++) acc[i] += (d * m.xs[i]) * (float)isum[i];
+                    dump_block(b, isum);
+                }
+#pragma unroll
+                for (int p = 0; p < PF; p++) ring[p] = next[p];
+            }
+        } else if (FMT == FMT_Q4_K) {
+            const uint32_t nsb = tk4_sbs(w.n_in);
+            const uint32_t nsteps = 2 * nsb;
+            const uint32_t per = (nsteps + kw - 1) / kw;
+            const uint32_t s0 = ks * per, s1 = min(nsteps, s0 + per);
+            const uint8_t* base = w.p0 + (size_t)tile * nsb * TK4_REC;
+            auto rec = [&](uint32_t s) { return base + (size_t)(s >> 1) * TK4_REC + (s & 1) * 1024; };
+            uint4 ring[PF];
+#pragma unroll
+            for (int p = 0; p < PF; p++)
+                if (s0 + p < s1) ring[p] = *reinterpret_cast<const uint4*>(rec(s0 + p) + 16 * lane);
+            for (uint32_t sb = s0; sb < s1; sb += PF) {
+                uint4 next[PF];
+#pragma unroll
+                for (int p = 0; p < PF; p++)
+                    if (sb + PF + p < s1) next[p] = *reinterpret_cast<const uint4*>(rec(sb + PF + p) + 16 * lane);
+#pragma unroll
+                for (int p = 0; p < PF; p++) {
+                    const uint32_t s = sb + p;
+                    if (s >= s1) break;
+                    const uint4 c = ring[p];
+                    const uint8_t* mt = base + (size_t)(s >> 1) * TK4_REC + 2048;
+                    // this step's four sub-blocks are 4 (s & 1) .. + 3 of the super-block
+                    const uint32_t sc4 = *reinterpret_cast<const uint32_t*>(mt + 16 * n + 4 * (s & 1));
+                    const uint32_t mn4 = *reinterpret_cast<const uint32_t*>(mt + 16 * n + 8 + 4 * (s & 1));
+                    const uint32_t dd = *reinterpret_cast<const uint32_t*>(mt + 256 + 4 * n);
+                    const float d = f16_bits_to_f32((uint16_t)(dd & 0xFFFF)), dmin = f16_bits_to_f32((uint16_t)(dd >> 16));
+#pragma unroll
+                    for (int pr = 0; pr < 2; pr++) {  // the two byte pairs of the lane's chunk
+                        const uint32_t lo = pr ? c.z : c.x, hi = pr ? c.w : c.y;
+                        v4i bw = {(int)(lo & 0x0F0F0F0Fu), (int)(hi & 0x0F0F0F0Fu), (int)((lo >> 4) & 0x0F0F0F0Fu),
+                                  (int)((hi >> 4) & 0x0F0F0F0Fu)};
+                        const uint32_t b0 = 4 * s + 2 * pr;  // global block (sub-block) index of half 0
+                        v4i D = block_pair(bw, b0, b0 + 1, 8 * kq, 0, false);
+                        const uint32_t q = 2 * pr + d_half;
+                        const float sc = (float)((sc4 >> (8 * q)) & 0xFF), mn = (float)((mn4 >> (8 * q)) & 0xFF);
+                        const float sv = d * sc;
+                        const float mv = 8.0f * sv - dmin * mn;
+                        Meta4 m;
+                        load_meta<TPAD, SUMS>(lds, nblk, b0 + d_half, d_tok0, m);
+                        int isum[4] = {D.x - 8 * m.su[0], D.y - 8 * m.su[1], D.z - 8 * m.su[2], D.w - 8 * m.su[3]};
+#pragma unroll
+                        for (int i = 0; i < NI; i++) {
+                            acc[i] += (sv * m.xs[i]) * (float)isum[i];
+                            acc[i] += mv * m.fs[i];
+                        }
+                        dump_block(b0 + d_half, isum);
+                    }
+                }
+#pragma unroll
+                for (int p = 0; p < PF; p++) ring[p] = next[p];
+            }
+        } else {  // FMT_Q4M
+            const uint32_t nsteps = t4m_steps(w.n_in);
+            const uint32_t per = (nsteps + kw - 1) / kw;
+            const uint32_t s0 = ks * per, s1 = min(nsteps, s0 + per);
+            const uint8_t* base = w.p0 + (size_t)tile * nsteps * T4M_REC;
+            uint4 ring[PF];
+#pragma unroll
+            for (int p = 0; p < PF; p++)
+                if (s0 + p < s1) ring[p] = *reinterpret_cast<const uint4*>(base + (size_t)(s0 + p) * T4M_REC + 16 * lane);
+            for (uint32_t sb = s0; sb < s1; sb += PF) {
+                uint4 next[PF];
+#pragma unroll
+                for (int p = 0; p < PF; p++)
+                    if (sb + PF + p < s1) next[p] = *reinterpret_cast<const uint4*>(base + (size_t)(sb + PF + p) * T4M_REC + 16 * lane);
+#pragma unroll
+                for (int p = 0; p < PF; p++) {
+                    const uint32_t s = sb + p;
+                    if (s >= s1) break;
+                    const uint4 c = ring[p];
+                    const uint8_t* rc = base + (size_t)s * T4M_REC;
+                    const uint32_t dd = *reinterpret_cast<const uint32_t*>(rc + 1024 + 4 * n);
+                    const uint32_t oo = *reinterpret_cast<const uint32_t*>(rc + 1088 + 4 * n);
+#pragma unroll
+                    for (int g = 0; g < 2; g++) {  // the two groups of 64 of the step
+                        const uint32_t w0 = g ? c.z : c.x, w1 = g ? c.w : c.y;  // blocks 2 g, 2 g + 1
+                        v4i bw = {(int)(w0 & 0x0F0F0F0Fu), (int)((w0 >> 4) & 0x0F0F0F0Fu), (int)(w1 & 0x0F0F0F0Fu),
+                                  (int)((w1 >> 4) & 0x0F0F0F0Fu)};
+                        const uint32_t b0 = 4 * s + 2 * g;
+                        v4i D = block_pair(bw, b0, b0 + 1, 4 * kq, 16 + 4 * kq, true);
+                        const float d = f16_bits_to_f32((uint16_t)(g ? dd >> 16 : dd & 0xFFFF));
+                        const float off = bf16_bits_to_f32((uint16_t)(g ? oo >> 16 : oo & 0xFFFF));
+                        Meta4 m;
+                        load_meta<TPAD, SUMS>(lds, nblk, min(b0 + d_half, nblk - 1), d_tok0, m);
+                        int isum[4] = {D.x - 8 * m.su[0], D.y - 8 * m.su[1], D.z - 8 * m.su[2], D.w - 8 * m.su[3]};
+                        const bool real = b0 + d_half < nblk;  // padding blocks hold zero codes but the -8 still applies
+#pragma unroll
+                        for (int i = 0; i < NI; i++) {
+                            if (real) {
+                                acc[i] += ((float)isum[i] * d) * m.xs[i];
+                                acc[i] += off * m.fs[i];
+                            }
+                        }
+                        dump_block(b0 + d_half, isum);
+                    }
+                }
+#pragma unroll
+                for (int p = 0; p < PF; p++) ring[p] = next[p];
+            }
+        }
+    }
+    // the two block parities of a token meet across lane groups kq and kq ^ 2
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i] += __shfl_xor(acc[i], 32);
+    if (kq < 2) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (d_tok0 + i < (uint32_t)TPAD) red[((size_t)wave * TPAD + d_tok0 + i) * 16 + n] = acc[i];
+    }
+    __syncthreads();
+    // K-slices in order
+    for (uint32_t idx = threadIdx.x; idx < rt * TPAD * 16; idx += blockDim.x) {
+        const uint32_t rr = idx / (TPAD * 16), tok = (idx / 16) % TPAD, nn = idx % 16;
+        const uint32_t row = (blockIdx.x * rt + rr) * 16 + nn;
+        if (tok >= t || row >= w.n_out || !y) continue;
+        float sum = 0.0f;
+        for (uint32_t k = 0; k < kw; k++) sum += red[((size_t)(rr * kw + k) * TPAD + tok) * 16 + nn];
+        y[(size_t)tok * w.n_out + row] = sum;
+    }
+}
+
+namespace {
+
+struct Shape {
+    uint32_t rt, kw;
+};
+
+// Waves per workgroup and how they split: enough workgroups to cover the CUs, and K split so that
+// about 4096-8192 waves exist while each keeps a few records to stream.
+Shape shape_for(uint32_t ntiles, uint32_t nsteps) {
+    uint32_t kw = 1;
+    while (kw < 16 && (size_t)ntiles * kw < 4096 && nsteps / (kw * 2) >= 4) kw *= 2;
+    if (kw < 4 && nsteps / 4 >= 2) kw = 4;
+    return Shape{1, kw};
+}
+
+template <int FMT, bool DUMP>
+hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* dump, hipStream_t s) {
+    const uint32_t ntiles = row_tiles(w.n_out);
+    const uint32_t nsteps = FMT == FMT_Q8_0 ? t8_steps(w.n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in) : t4m_steps(w.n_in));
+    const Shape sh = shape_for(ntiles, nsteps);
+    const uint32_t nblk = w.n_in / 32;
+    dim3 grid((ntiles + sh.rt - 1) / sh.rt), block(64 * sh.rt * sh.kw);
+    size_t c0 = 0;
+    while (c0 < t) {
+        const size_t tc = t - c0 < 8 ? t - c0 : 8;
+        QActView v = xa;
+        v.q += c0 * w.n_in;
+        v.scales += c0 * nblk;
+        v.sums += c0 * nblk;
+        v.fsums += c0 * nblk;
+        float* yo = y ? y + c0 * w.n_out : nullptr;  // no output rows when only the block sums are wanted
+        int32_t* du = dump ? dump + c0 * (size_t)w.n_out * nblk : nullptr;
+        const int tpad = tc <= 4 ? 4 : 8;
+        const size_t lds = ((size_t)(FMT == FMT_Q8_0 ? 1 : 3) * nblk * tpad + (size_t)sh.rt * sh.kw * tpad * 16) * 4;
+        if (lds > 160 * 1024) return hipErrorInvalidValue;  // rows too long for the staged activation scales
+        const uint32_t tt = (uint32_t)tc;
+        hipError_t e = hipSuccess;
+        auto go = [&](auto kern) {
+            if (lds > 48 * 1024) e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, v, tt, sh.rt, sh.kw, yo, du);
+        };
+        if (tc == 1) go(decode_mfma_kernel<FMT, 1, DUMP>);
+        else if (tc == 2) go(decode_mfma_kernel<FMT, 2, DUMP>);
+        else if (tc <= 4) go(decode_mfma_kernel<FMT, 4, DUMP>);
+        else go(decode_mfma_kernel<FMT, 8, DUMP>);
+        if (e != hipSuccess) return e;
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        c0 += tc;
+    }
+    return hipSuccess;
+}
+
+}  // namespace
+
+hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, hipStream_t s) {
+    switch (w.fmt) {
+        case FMT_Q8_0: return run<FMT_Q8_0, false>(w, xa, t, y, nullptr, s);
+        case FMT_Q4_K: return run<FMT_Q4_K, false>(w, xa, t, y, nullptr, s);
+        case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+// The integer block sums the kernel forms ([t][n_out][n_in/32]); y is scratch of [t][n_out].
+hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* out, hipStream_t s) {
+    switch (w.fmt) {
+        case FMT_Q8_0: return run<FMT_Q8_0, true>(w, xa, t, y, out, s);
+        case FMT_Q4_K: return run<FMT_Q4_K, true>(w, xa, t, y, out, s);
+        case FMT_Q4M: return run<FMT_Q4M, true>(w, xa, t, y, out, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace oxhip

@@ -10,6 +10,7 @@
 //   FP8   e4m3(byte) * block scale                        src/ggml.rs:282-293, :433-444
 //   MLX 4-bit -> Q4 + offsets                             src/quant.rs:518-563
 #include "internal.hpp"
+#include "layout.hpp"
 
 namespace oxhip {
 
@@ -31,21 +32,33 @@ __global__ __launch_bounds__(256) void dequantize_kernel(WeightView w, uint32_t 
             break;
         }
         case FMT_Q8_0: {
-            float d = f16_bits_to_f32(reinterpret_cast<const uint16_t*>(w.p1)[r * (n / 32) + c / 32]);
-            v = (float)reinterpret_cast<const int8_t*>(w.p0)[r * n + c] * d;
+            uint32_t tile = r >> 4, nn = r & 15, b = c >> 5, st = b >> 1, h = b & 1, e = c & 31, kq = e >> 3, j = e & 7;
+            const uint8_t* rec = w.p0 + ((size_t)tile * t8_steps(n) + st) * T8_REC;
+            float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(rec + 1024 + 4 * nn + 2 * h));
+            v = (float)(int8_t)rec[16 * (kq * 16 + nn) + 8 * h + j] * d;
             break;
         }
         case FMT_Q4_K: {
-            size_t nb = n / 256;
-            uint32_t sb = c / 256, e = c % 256, j = e / 64, h = (e % 64) / 32, l = e % 32;
-            uint8_t byte = w.p0[(r * nb + sb) * 128 + 32 * j + l];
-            uint32_t q = (byte >> (4 * h)) & 0xF;
-            uint4 mt = *reinterpret_cast<const uint4*>(w.p1 + (r * nb + sb) * 16);
-            float d = f16_bits_to_f32((uint16_t)(mt.x & 0xFFFF)), dmin = f16_bits_to_f32((uint16_t)(mt.x >> 16));
-            uint32_t sc, mn;
-            scale_min_k4(2 * j + h, mt.y, mt.z, mt.w, sc, mn);
+            uint32_t tile = r >> 4, nn = r & 15, sb = c / 256, e = c % 256, pair = e / 64, hi = (e % 64) / 32, l = e % 32;
+            uint32_t st = pair >> 1, jj = pair & 1, kq = l >> 3;
+            const uint8_t* rec = w.p0 + ((size_t)tile * tk4_sbs(n) + sb) * TK4_REC;
+            uint8_t byte = rec[st * 1024 + 16 * (kq * 16 + nn) + 8 * jj + (l & 7)];
+            uint32_t q = hi ? (byte >> 4) : (byte & 0xF);
+            uint32_t sc = rec[2048 + 16 * nn + 2 * pair + hi], mn = rec[2048 + 16 * nn + 8 + 2 * pair + hi];
+            float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(rec + 2304 + 4 * nn));
+            float dmin = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(rec + 2304 + 4 * nn + 2));
             float d1 = d * (float)sc, m1 = dmin * (float)mn;
             v = d1 * (float)q - m1;
+            break;
+        }
+        case FMT_Q4M: {
+            uint32_t tile = r >> 4, nn = r & 15, b = c >> 5, st = b >> 2, bi = b & 3, e = c & 31, hi = e >> 4, pp = e & 15, kq = pp >> 2;
+            const uint8_t* rec = w.p0 + ((size_t)tile * t4m_steps(n) + st) * T4M_REC;
+            uint8_t byte = rec[16 * (kq * 16 + nn) + 4 * bi + (pp & 3)];
+            int nib = hi ? (byte >> 4) : (byte & 0xF);
+            float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(rec + 1024 + 4 * nn + 2 * (bi >> 1)));
+            float m = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(rec + 1088 + 4 * nn + 2 * (bi >> 1)));
+            v = (float)(nib - 8) * d + m;
             break;
         }
         case FMT_Q6_K: {
@@ -80,37 +93,139 @@ hipError_t launch_dequantize(const WeightView& w, size_t r0, size_t r1, float* o
 }
 
 // ---- upload-time repacking ---------------------------------------------------------------------
-// One thread per source block; runs once per matrix.
-__global__ __launch_bounds__(256) void repack_gguf_kernel(int fmt, const uint8_t* __restrict__ raw, size_t nblocks, uint8_t* p0,
-                                                          uint8_t* p1, uint8_t* p2, uint8_t* p3) {
-    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (b >= nblocks) return;
-    if (fmt == FMT_Q8_0) {
-        const uint8_t* s = raw + b * 34;
-        p1[2 * b] = s[0];
-        p1[2 * b + 1] = s[1];
-        for (int i = 0; i < 32; i++) p0[b * 32 + i] = s[2 + i];
-    } else if (fmt == FMT_Q4_K) {
-        const uint8_t* s = raw + b * 144;
-        for (int i = 0; i < 16; i++) p1[b * 16 + i] = s[i];
-        for (int i = 0; i < 128; i++) p0[b * 128 + i] = s[16 + i];
-    } else if (fmt == FMT_Q6_K) {
-        const uint8_t* s = raw + b * 210;
-        for (int i = 0; i < 128; i++) p0[b * 128 + i] = s[i];
-        for (int i = 0; i < 64; i++) p1[b * 64 + i] = s[128 + i];
-        for (int i = 0; i < 16; i++) p2[b * 16 + i] = s[192 + i];
-        p3[2 * b] = s[208];
-        p3[2 * b + 1] = s[209];
+// Tile-packing of raw GGUF blocks (layout.hpp). One thread per 16-byte chunk of the destination;
+// the threads of lane group kq = 0 also write the record's scales. Runs once per matrix.
+__global__ __launch_bounds__(256) void pack_t8_kernel(const uint8_t* __restrict__ raw, uint32_t n_out, uint32_t n_in, uint8_t* __restrict__ dst) {
+    const uint32_t nsteps = t8_steps(n_in), nblk = n_in / 32;
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t total = (size_t)row_tiles(n_out) * nsteps * 64;
+    if (idx >= total) return;
+    uint32_t l = idx & 63, nn = l & 15, kq = l >> 4;
+    size_t ts = idx >> 6;
+    uint32_t st = ts % nsteps;
+    size_t tile = ts / nsteps;
+    size_t row = tile * 16 + nn;
+    uint8_t* rec = dst + ts * T8_REC;
+    uint32_t out[4] = {0, 0, 0, 0};
+    uint16_t d[2] = {0, 0};
+    for (uint32_t h = 0; h < 2; h++) {
+        uint32_t b = 2 * st + h;
+        if (row < n_out && b < nblk) {
+            const uint8_t* src = raw + (row * nblk + b) * 34;
+            d[h] = (uint16_t)(src[0] | (src[1] << 8));
+            for (int j = 0; j < 8; j++) out[2 * h + j / 4] |= (uint32_t)src[2 + 8 * kq + j] << (8 * (j & 3));
+        }
+    }
+    *reinterpret_cast<uint4*>(rec + 16 * l) = make_uint4(out[0], out[1], out[2], out[3]);
+    if (kq == 0) *reinterpret_cast<uint32_t*>(rec + 1024 + 4 * nn) = d[0] | ((uint32_t)d[1] << 16);
+}
+
+__global__ __launch_bounds__(256) void pack_tk4_kernel(const uint8_t* __restrict__ raw, uint32_t n_out, uint32_t n_in, uint8_t* __restrict__ dst) {
+    const uint32_t nsb = tk4_sbs(n_in);
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t total = (size_t)row_tiles(n_out) * nsb * 128;  // two steps of 64 chunks per super-block
+    if (idx >= total) return;
+    uint32_t l = idx & 63, nn = l & 15, kq = l >> 4, st = (idx >> 6) & 1;
+    size_t tsb = idx >> 7;
+    uint32_t sb = tsb % nsb;
+    size_t tile = tsb / nsb;
+    size_t row = tile * 16 + nn;
+    uint8_t* rec = dst + tsb * TK4_REC;
+    const uint8_t* src = raw + (row * nsb + sb) * 144;
+    uint32_t out[4] = {0, 0, 0, 0};
+    if (row < n_out)
+        for (uint32_t jj = 0; jj < 2; jj++)
+            for (int j = 0; j < 8; j++) out[2 * jj + j / 4] |= (uint32_t)src[16 + 32 * (2 * st + jj) + 8 * kq + j] << (8 * (j & 3));
+    *reinterpret_cast<uint4*>(rec + st * 1024 + 16 * l) = make_uint4(out[0], out[1], out[2], out[3]);
+    if (kq == 0 && st == 0) {
+        uint32_t sc[2] = {0, 0}, mn[2] = {0, 0}, dd = 0;
+        if (row < n_out) {
+            uint32_t d0 = src[4] | (src[5] << 8) | (src[6] << 16) | ((uint32_t)src[7] << 24);
+            uint32_t d1 = src[8] | (src[9] << 8) | (src[10] << 16) | ((uint32_t)src[11] << 24);
+            uint32_t d2 = src[12] | (src[13] << 8) | (src[14] << 16) | ((uint32_t)src[15] << 24);
+            for (uint32_t i = 0; i < 8; i++) {
+                uint32_t s, m;
+                scale_min_k4(i, d0, d1, d2, s, m);
+                sc[i >> 2] |= s << (8 * (i & 3));
+                mn[i >> 2] |= m << (8 * (i & 3));
+            }
+            dd = src[0] | (src[1] << 8) | (src[2] << 16) | ((uint32_t)src[3] << 24);
+        }
+        *reinterpret_cast<uint4*>(rec + 2048 + 16 * nn) = make_uint4(sc[0], sc[1], mn[0], mn[1]);
+        *reinterpret_cast<uint32_t*>(rec + 2304 + 4 * nn) = dd;
     }
 }
 
+// Planar Q4 with one scale and one offset per 64 -> tile-packed (layout.hpp).
+__global__ __launch_bounds__(256) void pack_q4m_kernel(const uint8_t* __restrict__ q, const uint16_t* __restrict__ sc,
+                                                       const uint16_t* __restrict__ off, uint32_t n_out, uint32_t n_in,
+                                                       uint8_t* __restrict__ dst) {
+    const uint32_t nsteps = t4m_steps(n_in), nblk = n_in / 32;
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t total = (size_t)row_tiles(n_out) * nsteps * 64;
+    if (idx >= total) return;
+    uint32_t l = idx & 63, nn = l & 15, kq = l >> 4;
+    size_t ts = idx >> 6;
+    uint32_t st = ts % nsteps;
+    size_t tile = ts / nsteps;
+    size_t row = tile * 16 + nn;
+    uint8_t* rec = dst + ts * T4M_REC;
+    uint32_t out[4] = {0, 0, 0, 0};
+    for (uint32_t b = 0; b < 4; b++) {
+        uint32_t blk = 4 * st + b;
+        if (row < n_out && blk < nblk) out[b] = *reinterpret_cast<const uint32_t*>(q + row * (n_in / 2) + blk * 16 + 4 * kq);
+    }
+    *reinterpret_cast<uint4*>(rec + 16 * l) = make_uint4(out[0], out[1], out[2], out[3]);
+    if (kq == 0) {
+        uint32_t d = 0, o = 0;
+        for (uint32_t g = 0; g < 2; g++) {
+            uint32_t grp = 2 * st + g;
+            if (row < n_out && grp < n_in / 64) {
+                d |= (uint32_t)sc[row * (n_in / 64) + grp] << (16 * g);
+                o |= (uint32_t)off[row * (n_in / 64) + grp] << (16 * g);
+            }
+        }
+        *reinterpret_cast<uint32_t*>(rec + 1024 + 4 * nn) = d;
+        *reinterpret_cast<uint32_t*>(rec + 1088 + 4 * nn) = o;
+    }
+}
+
+hipError_t launch_pack_q4m(const uint8_t* q, const uint16_t* sc, const uint16_t* off, size_t n_out, size_t n_in, uint8_t* dst,
+                           hipStream_t s) {
+    size_t total = (size_t)row_tiles((uint32_t)n_out) * t4m_steps((uint32_t)n_in) * 64;
+    pack_q4m_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(q, sc, off, (uint32_t)n_out, (uint32_t)n_in, dst);
+    return hipGetLastError();
+}
+
+// Q6_K: planes, one thread per source block.
+__global__ __launch_bounds__(256) void repack_q6k_kernel(const uint8_t* __restrict__ raw, size_t nblocks, uint8_t* p0, uint8_t* p1,
+                                                         uint8_t* p2, uint8_t* p3) {
+    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    const uint8_t* s = raw + b * 210;
+    for (int i = 0; i < 128; i++) p0[b * 128 + i] = s[i];
+    for (int i = 0; i < 64; i++) p1[b * 64 + i] = s[128 + i];
+    for (int i = 0; i < 16; i++) p2[b * 16 + i] = s[192 + i];
+    p3[2 * b] = s[208];
+    p3[2 * b + 1] = s[209];
+}
+
 hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t n_in, const WeightView& d, hipStream_t s) {
-    size_t bs = fmt == FMT_Q8_0 ? 32 : 256;
-    size_t nblocks = n_out * (n_in / bs);
-    if (!nblocks) return hipSuccess;
-    repack_gguf_kernel<<<(unsigned)((nblocks + 255) / 256), 256, 0, s>>>(fmt, raw, nblocks, const_cast<uint8_t*>(d.p0),
-                                                                        const_cast<uint8_t*>(d.p1), const_cast<uint8_t*>(d.p2),
-                                                                        const_cast<uint8_t*>(d.p3));
+    uint8_t* p0 = const_cast<uint8_t*>(d.p0);
+    if (fmt == FMT_Q8_0) {
+        size_t total = (size_t)row_tiles((uint32_t)n_out) * t8_steps((uint32_t)n_in) * 64;
+        pack_t8_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
+    } else if (fmt == FMT_Q4_K) {
+        size_t total = (size_t)row_tiles((uint32_t)n_out) * tk4_sbs((uint32_t)n_in) * 128;
+        pack_tk4_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
+    } else if (fmt == FMT_Q6_K) {
+        size_t nblocks = n_out * (n_in / 256);
+        if (!nblocks) return hipSuccess;
+        repack_q6k_kernel<<<(unsigned)((nblocks + 255) / 256), 256, 0, s>>>(raw, nblocks, p0, const_cast<uint8_t*>(d.p1),
+                                                                           const_cast<uint8_t*>(d.p2), const_cast<uint8_t*>(d.p3));
+    } else {
+        return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

@@ -12,23 +12,20 @@
 namespace oxhip {
 
 // ------------------------------------------------------------------------------------------------
-// Device layouts. Uploads repack every format into planes whose rows start on 16-byte boundaries,
-// so each lane of a wavefront reads one aligned 16-byte chunk and consecutive lanes read
-// consecutive chunks. The bytes are those of the source format, only rearranged.
+// Device layouts. Uploads repack every format so that each lane of a wavefront reads one aligned
+// 16-byte chunk and consecutive lanes read consecutive chunks. The bytes are those of the source
+// format, only rearranged. Q8_0, Q4_K and Q4 with one scale and offset per 64 (MLX) are stored
+// tile-packed for the matrix cores (layout.hpp: all in p0); the others in planes:
 //
-//   Q4    q   [n_out][n_in/2]      byte j of a 32-block: element j (low nibble), j+16 (high)
-//         sc  [n_out][n_in/sgroup] f16 scale; sgroup = 32, or the offset group when every block of
-//                                  a group carries the same scale (MLX checkpoints)
-//         off [n_out][n_in/group]  bf16 offsets, optional
-//   Q8_0  q   [n_out][n_in]        int8
-//         d   [n_out][n_in/32]     f16
-//   Q4_K  qs  [n_out][nb][128]     nibbles as in the block
-//         mt  [n_out][nb][16]      d, dmin (f16) and the 12 packed scale bytes
-//   Q6_K  ql  [n_out][nb][128], qh [n_out][nb][64], sc [n_out][nb][16] int8, d [n_out][nb] f16
-//   FP8   q   [n_out][n_in]        e4m3 bytes; bs f32 [ceil(n_out/br)][ceil(n_in/bc)]
-//   BF16  q   [n_out][n_in]        bf16
+//   Q4    p0 q   [n_out][n_in/2]      byte j of a 32-block: element j (low nibble), j+16 (high)
+//         p1 sc  [n_out][n_in/sgroup] f16 scale; sgroup = 32, or the offset group when every block
+//                                     of a group carries the same scale
+//         p2 off [n_out][n_in/group]  bf16 offsets, optional
+//   Q6_K  p0 ql  [n_out][nb][128], p1 qh [n_out][nb][64], p2 sc [n_out][nb][16] int8, p3 d [n_out][nb] f16
+//   FP8   p0 q   [n_out][n_in]        e4m3 bytes; p1 bs f32 [ceil(n_out/br)][ceil(n_in/bc)]
+//   BF16  p0 q   [n_out][n_in]        bf16
 // ------------------------------------------------------------------------------------------------
-enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5 };
+enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6 };
 
 struct WeightView {
     int fmt;
@@ -56,7 +53,11 @@ hipError_t launch_quantize_act(const float* x, size_t t, size_t n_in, const oxhi
 hipError_t launch_dequantize(const WeightView& w, size_t r0, size_t r1, float* out, hipStream_t s);
 hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s);
 hipError_t launch_isums(const WeightView& w, const QActView& xa, size_t t, int32_t* out, hipStream_t s);
+hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, hipStream_t s);
+hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* out, hipStream_t s);
 hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t n_in, const WeightView& dst, hipStream_t s);
+hipError_t launch_pack_q4m(const uint8_t* q, const uint16_t* sc, const uint16_t* off, size_t n_out, size_t n_in, uint8_t* dst,
+                           hipStream_t s);
 hipError_t launch_repack_mlx_q4(const uint32_t* w, const uint16_t* scales, const uint16_t* biases, size_t n_out,
                                 size_t n_in, size_t group, const WeightView& dst, hipStream_t s);
 hipError_t launch_q4_scale_groups(const uint16_t* sc32, size_t n_out, size_t n_in, size_t sgroup, uint16_t* dst,

@@ -1,0 +1,44 @@
+// Tile-packed device layouts of the quantized formats, shared by the upload repackers, the
+// dequantizers and the MFMA kernels.
+//
+// A matrix is cut into row tiles of 16 rows; a tile is a sequence of K-steps, and each K-step is
+// stored as one record so that a wavefront reads it with one fully coalesced 16-byte-per-lane
+// load: lane l = 16 * kq + n holds bytes [16 l, 16 l + 16) of the record, which are the codes of
+// row n of the tile at the K positions MFMA lane group kq consumes. Scales (and mins / offsets) of
+// the 16 rows follow the codes in the same record. Rows past n_out and blocks past n_in are zero.
+// The bytes are those of the source format (Q4_K: its 12 packed scale bytes are stored unpacked as
+// 16 bytes, 2.8 % more), only rearranged.
+//
+//   Q8_0 (T8)   step = 2 blocks of 32 (64 K), record 1088 B:
+//               codes[16 l + 8 h + j] = q[row n][block 2 s + h][8 kq + j]          1024 B
+//               d[n][h] f16                                                          64 B
+//   Q4_K (TK4)  super-block record 2368 B = 2 steps of 128 K + metadata:
+//               codes[1024 t + 16 l + 8 jj + j] = qs[32 (2 t + jj) + 8 kq + j]     2048 B
+//                  (low nibble: sub-block 2 (2 t + jj), high nibble: the next one)
+//               sc[n][8], mn[n][8] bytes (the 6-bit scales and mins, unpacked)       256 B
+//               d[n], dmin[n] f16                                                     64 B
+//   Q4 with one scale and one offset per 64 (MLX; T4M)  step = 4 blocks (128 K), record 1152 B:
+//               codes[16 l + 4 b + j] = q[row n][block 4 s + b][4 kq + j]           1024 B
+//                  (low nibble: element 4 kq + j, high nibble: element 16 + 4 kq + j)
+//               d[n][2] f16 (blocks 0-1, blocks 2-3)                                  64 B
+//               off[n][2] bf16                                                        64 B
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+namespace oxhip {
+
+constexpr uint32_t T8_REC = 1088;
+constexpr uint32_t TK4_REC = 2368;
+constexpr uint32_t T4M_REC = 1152;
+
+__host__ __device__ inline uint32_t t8_steps(uint32_t n_in) { return (n_in / 32 + 1) / 2; }
+__host__ __device__ inline uint32_t tk4_sbs(uint32_t n_in) { return n_in / 256; }
+__host__ __device__ inline uint32_t t4m_steps(uint32_t n_in) { return (n_in / 32 + 3) / 4; }
+__host__ __device__ inline uint32_t row_tiles(uint32_t n_out) { return (n_out + 15) / 16; }
+
+__host__ __device__ inline size_t t8_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t8_steps(n_in) * T8_REC; }
+__host__ __device__ inline size_t tk4_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * tk4_sbs(n_in) * TK4_REC; }
+__host__ __device__ inline size_t t4m_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t4m_steps(n_in) * T4M_REC; }
+
+}  // namespace oxhip

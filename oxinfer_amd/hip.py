@@ -27,6 +27,11 @@ class Job(C.Structure):
     _fields_ = [("w", C.c_void_p), ("n_out", C.c_size_t), ("y", C.c_void_p)]
 
 
+class DecodeJob(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("xa", C.c_void_p), ("x", C.c_void_p), ("t", C.c_size_t), ("y", C.c_void_p),
+                ("ev_start", C.c_void_p), ("ev_stop", C.c_void_p)]
+
+
 class QActC(C.Structure):
     _fields_ = [("q", C.c_void_p), ("scales", C.c_void_p), ("sums", C.c_void_p), ("fsums", C.c_void_p),
                 ("hsums", C.c_void_p), ("sums16", C.c_void_p), ("t", C.c_size_t), ("n_in", C.c_size_t)]
@@ -68,6 +73,10 @@ def load_library():
         "oxhip_dev_dequantize": (C.c_int, [vp, vp, sz, sz, vp, vp]),
         "oxhip_dev_decode": (C.c_int, [vp, vp, C.POINTER(QActC), vp, sz, vp, vp]),
         "oxhip_dev_isums": (C.c_int, [vp, vp, C.POINTER(QActC), vp, vp]),
+        "oxhip_dev_decode_batch": (C.c_int, [vp, C.POINTER(DecodeJob), sz, vp]),
+        "oxhip_event_create": (vp, []),
+        "oxhip_event_destroy": (None, [vp]),
+        "oxhip_event_elapsed_ms": (C.c_float, [vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -228,6 +237,27 @@ class HipBackend:
         if not ok:
             raise RuntimeError(self.last_error())
         return y
+
+    def decode_jobs(self, jobs):
+        """Builds a reusable job array for decode_batch: jobs = [(DeviceWeight, QAct | None, x | None, t, y, ev0, ev1)]."""
+        arr = (DecodeJob * len(jobs))()
+        for i, (w, xa, x, t, y, e0, e1) in enumerate(jobs):
+            arr[i] = DecodeJob(w.handle, C.addressof(xa.c) if xa is not None else None,
+                               x.data_ptr() if x is not None else None, t, y.data_ptr(), e0, e1)
+        return arr
+
+    def decode_batch(self, arr):
+        if not self.lib.oxhip_dev_decode_batch(self.ctx, arr, len(arr), self._stream()):
+            raise RuntimeError(self.last_error())
+
+    def event(self):
+        e = self.lib.oxhip_event_create()
+        if not e:
+            raise RuntimeError(self.last_error())
+        return e
+
+    def elapsed_ms(self, a, b):
+        return self.lib.oxhip_event_elapsed_ms(a, b)
 
     def isums(self, w, xa, per):
         import torch
