@@ -146,7 +146,8 @@ def main():
     for c in cases:
         c["dom"] = c["kind"] == dom_kind and c["t"] == 8
     dom = [c for c in cases if c["dom"]]
-    dom_symbol = f"decode_kernel<{KERNEL_FMT[dom_kind]}, 8, 4>"
+    dom_symbol = (f"decode_mfma_kernel<{KERNEL_FMT[dom_kind]}, 8, false>" if dom_kind != Q6_K
+                  else f"decode_kernel<{KERNEL_FMT[dom_kind]}, 8, 4>")
 
     # One call per step: the job arrays (one per rotation phase) are built once; the dominant launches carry
     # HIP events recorded on the launch stream.

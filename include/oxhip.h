@@ -97,6 +97,21 @@ size_t oxhip_weight_bytes(const oxhip_weight* w);
  * computes every job or none. t <= 16 runs the int8 decode kernels (the CPU's decode semantics,
  * src/kernels.rs:1908-1928); more tokens run the MFMA GEMM. */
 int oxhip_matmul(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_job* jobs, size_t n_jobs);
+/* Backend::matvec_rows (src/gpu.rs:165): t in 1..=4. */
+int oxhip_matvec_rows(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_rows_job* jobs, size_t n_jobs);
+
+/* Backend::upload_moe / upload_moe_transient (src/gpu.rs:206-231): expert e has gate_up[e]
+ * ([2*inter, h] fused, or [inter, h] when `up` is given) and down[e] ([h, inter]). */
+oxhip_moe* oxhip_upload_moe(oxhip_ctx* ctx, const oxhip_weight_desc* gate_up, const oxhip_weight_desc* up,
+                            const oxhip_weight_desc* down, size_t n_experts, size_t h, size_t inter,
+                            uint32_t act_kind, float act_param);
+void oxhip_free_moe(oxhip_ctx* ctx, oxhip_moe* m);
+/* Backend::moe (src/gpu.rs:237-248) with `routes` flattened as CUDA's moe_run does
+ * (src/cuda.rs:802-838): token i goes through experts route_idx[i*k .. i*k+k] with weights
+ * route_w[...]; y[i] += sum_j w_j * down(act(gate x) * up x), in route order. */
+int oxhip_moe_forward(oxhip_ctx* ctx, const float* x, size_t t, size_t h, size_t inter, const uint32_t* route_idx,
+                      const float* route_w, size_t k, oxhip_moe* m, float* y);
+
 /* ---- device-pointer entry points ---------------------------------------------------------- */
 /* `QAct` (src/quant.rs:222-238) in HBM, plus sums16: the integer sum of each 16 int8 values (what
  * the centred nibble formats fold their offset through; the CPU derives it from `sums`). */
@@ -137,6 +152,16 @@ void* oxhip_event_create(void);
 void oxhip_event_destroy(void* ev);
 /* Milliseconds between two recorded events; waits for `stop`. Negative on error. */
 float oxhip_event_elapsed_ms(void* start, void* stop);
+/* moe::route_top_k (src/moe.rs:180-193) for t rows of n_experts logits (n_experts <= 1024, k <= 32):
+ * idx / w [t, k], sorted by descending logit, ties to the lower index, w = softmax over the k. */
+int oxhip_dev_route_top_k(oxhip_ctx* ctx, const float* logits, size_t t, size_t n_experts, size_t k, uint32_t* idx, float* w,
+                          void* stream);
+/* Backend::moe on device buffers: x [t, h] f32, route_idx / route_w [t, k], y [t, h] f32 (added to).
+ * One grouped launch per projection over the routed token lists. The scratch it needs lives in
+ * `m` and grows on first use (a call with a larger t * k than any before synchronizes and
+ * reallocates); calls on one oxhip_moe must not overlap. */
+int oxhip_dev_moe(oxhip_ctx* ctx, oxhip_moe* m, const float* x, size_t t, const uint32_t* route_idx, const float* route_w,
+                  size_t k, float* y, void* stream);
 /* The exact integer accumulators of the decode kernels, written by the kernels themselves: per
  * block of 32 ([t, n_out, n_in/32]) for Q4, Q8_0 and Q4_K, per 16 ([t, n_out, n_in/16]) for Q6_K.
  * For parity checks (the CPU's per-16 sums add up to the per-32 ones exactly). */

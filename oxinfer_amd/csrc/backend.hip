@@ -1,76 +1,17 @@
 // The C ABI: the device context, uploads, and the `Backend` surface (src/gpu.rs:151-294 of the
 // reference) over the kernels of this library.
-#include <cmath>
-#include <cstdio>
-#include <cstring>
-#include <string>
-#include <vector>
-
-#include "internal.hpp"
-#include "layout.hpp"
+#include "backend.hpp"
 
 namespace oxhip {
 
 static thread_local std::string g_err;
 void set_error(const std::string& m) { g_err = m; }
 
-#define HIP_TRY(expr, what)                                                              \
-    do {                                                                                 \
-        hipError_t e__ = (expr);                                                         \
-        if (e__ != hipSuccess) {                                                         \
-            set_error(std::string(what) + ": " + hipGetErrorString(e__));                \
-            return 0;                                                                    \
-        }                                                                                \
-    } while (0)
-
-constexpr size_t VRAM_RESERVE = 512ull << 20;  // kept free for activations (src/cuda.rs:573-588)
-
-struct DevBuf {
-    void* p = nullptr;
-    size_t cap = 0;
-    bool grow(size_t need) {
-        if (cap >= need && p) return true;
-        if (p) (void)hipFree(p);
-        p = nullptr;
-        cap = 0;
-        size_t want = (need < 256 ? 256 : need) * 2;
-        if (hipMalloc(&p, want) != hipSuccess) {
-            p = nullptr;
-            return false;
-        }
-        cap = want;
-        return true;
-    }
-    void release() {
-        if (p) (void)hipFree(p);
-        p = nullptr;
-        cap = 0;
-    }
-};
-
 }  // namespace oxhip
 
 using namespace oxhip;
 
-struct oxhip_weight {
-    WeightView v{};
-    void* base = nullptr;
-    size_t bytes = 0;
-};
-
-struct oxhip_ctx {
-    int device = 0;
-    std::string name;
-    hipStream_t stream = nullptr;
-    std::mutex mu;  // serializes the host-pointer surface (staging is shared), as Mutex<Staging> does
-    DevBuf x, xq, y;
-    double ms_in = 0, ms_gpu = 0, ms_out = 0;
-    size_t calls = 0;
-};
-
 namespace {
-
-size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct Planes {
     size_t off[4] = {0, 0, 0, 0};
@@ -104,35 +45,6 @@ struct Temp {
         return hipMemcpyAsync(p, src, bytes, hipMemcpyHostToDevice, s) == hipSuccess;
     }
 };
-
-QActView view_of(const oxhip_qact& a) { return QActView{a.q, a.scales, a.sums, a.fsums, a.hsums, a.sums16}; }
-
-// Carves a QAct for t rows of n_in out of one buffer.
-size_t qact_bytes(size_t t, size_t n_in) {
-    size_t b32 = t * n_in / 32, b16 = t * n_in / 16;
-    return align_up(t * n_in, 256) + 3 * align_up(b32 * 4, 256) + 2 * align_up(b16 * 4, 256);
-}
-oxhip_qact carve_qact(void* base, size_t t, size_t n_in) {
-    uint8_t* p = static_cast<uint8_t*>(base);
-    size_t b32 = t * n_in / 32, b16 = t * n_in / 16;
-    oxhip_qact a{};
-    a.q = reinterpret_cast<int8_t*>(p);
-    p += align_up(t * n_in, 256);
-    a.scales = reinterpret_cast<float*>(p);
-    p += align_up(b32 * 4, 256);
-    a.sums = reinterpret_cast<int32_t*>(p);
-    p += align_up(b32 * 4, 256);
-    a.fsums = reinterpret_cast<float*>(p);
-    p += align_up(b32 * 4, 256);
-    a.hsums = reinterpret_cast<float*>(p);
-    p += align_up(b16 * 4, 256);
-    a.sums16 = reinterpret_cast<int32_t*>(p);
-    a.t = t;
-    a.n_in = n_in;
-    return a;
-}
-
-bool is_dense(const oxhip_weight* w) { return w->v.fmt == FMT_FP8 || w->v.fmt == FMT_BF16; }
 
 }  // namespace
 

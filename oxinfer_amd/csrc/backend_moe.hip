@@ -1,0 +1,300 @@
+// Backend::upload_moe / moe / matvec_rows (src/gpu.rs:165, :206-248 of the reference) over the grouped
+// decode kernel, plus their device-pointer forms.
+#include <cstring>
+#include <vector>
+
+#include "backend.hpp"
+
+using namespace oxhip;
+
+struct oxhip_moe {
+    std::vector<oxhip_weight*> gate_up, up, down;  // up empty when gate/up are fused
+    size_t n_exp = 0, h = 0, inter = 0;
+    uint32_t act_kind = 0;
+    float act_param = 0;
+    const uint8_t** bases_gu = nullptr;  // device arrays of tile-packed bases
+    const uint8_t** bases_up = nullptr;
+    const uint8_t** bases_dn = nullptr;
+    DevBuf ws;                           // scratch of one pass
+    size_t ws_pairs = 0, ws_t = 0;
+};
+
+namespace {
+
+bool mfma_format(const oxhip_weight* w) { return w->v.fmt == FMT_Q8_0 || w->v.fmt == FMT_Q4_K || w->v.fmt == FMT_Q4M; }
+
+size_t up256(size_t v) { return (v + 255) / 256 * 256; }
+
+// The scratch of one pass, carved from one allocation.
+struct Scratch {
+    int* row_of;
+    int* src;
+    int4* chunks;
+    int* nchunks;
+    oxhip_qact xa;  // x quantized, [t][h]
+    float* gu;      // [pairs][2 inter] (fused) or g [pairs][inter] then u [pairs][inter]
+    float* a;       // [pairs][inter]
+    oxhip_qact aq;  // a quantized
+    float* o;       // [pairs][h]
+    uint32_t max_chunks;
+    size_t bytes;
+};
+
+Scratch carve(uint8_t* base, size_t t, size_t pairs, size_t n_exp, size_t h, size_t inter) {
+    Scratch s{};
+    s.max_chunks = (uint32_t)((pairs < n_exp ? pairs : n_exp) + pairs / 8 + 1);
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        uint8_t* p = base ? base + off : nullptr;
+        off += up256(bytes);
+        return p;
+    };
+    s.row_of = reinterpret_cast<int*>(take(pairs * 4));
+    s.src = reinterpret_cast<int*>(take(pairs * 4));
+    s.chunks = reinterpret_cast<int4*>(take((size_t)s.max_chunks * 16));
+    s.nchunks = reinterpret_cast<int*>(take(4));
+    s.xa = carve_qact(take(qact_bytes(t, h)), t, h);
+    s.gu = reinterpret_cast<float*>(take(pairs * 2 * inter * 4));
+    s.a = reinterpret_cast<float*>(take(pairs * inter * 4));
+    s.aq = carve_qact(take(qact_bytes(pairs, inter)), pairs, inter);
+    s.o = reinterpret_cast<float*>(take(pairs * h * 4));
+    s.bytes = off;
+    return s;
+}
+
+int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t* route_idx, const float* route_w, size_t k,
+            float* y, hipStream_t s) {
+    const size_t pairs = t * k, h = m->h, inter = m->inter;
+    if (!pairs) return 1;
+    if (pairs > m->ws_pairs || t > m->ws_t) {
+        (void)hipStreamSynchronize(s);  // an earlier pass may still read the old scratch
+        const size_t np = pairs > m->ws_pairs ? pairs : m->ws_pairs, nt = t > m->ws_t ? t : m->ws_t;
+        Scratch probe = carve(nullptr, nt, np, m->n_exp, h, inter);
+        if (!m->ws.grow(probe.bytes)) {
+            m->ws_pairs = m->ws_t = 0;
+            set_error("moe: device memory short");
+            return 0;
+        }
+        m->ws_pairs = np;
+        m->ws_t = nt;
+    }
+    Scratch sc = carve(static_cast<uint8_t*>(m->ws.p), t, pairs, m->n_exp, h, inter);
+    const uint32_t max_rows = (uint32_t)(t < 8 ? t : 8);
+    HIP_TRY(launch_moe_plan(route_idx, pairs, k, m->n_exp, sc.row_of, sc.src, sc.chunks, sc.nchunks, s), "moe plan launch");
+    HIP_TRY(launch_quantize_act(x, t, h, sc.xa, s), "moe quantize launch");
+    GroupView g{};
+    g.chunks = sc.chunks;
+    g.nchunks = sc.nchunks;
+    // gate / up over the routed rows of x (row i of the gathered order is token src[i])
+    g.rowmap = sc.src;
+    g.bases = m->bases_gu;
+    const bool fused = m->up.empty();
+    HIP_TRY(launch_decode_mfma_grouped(m->gate_up[0]->v, view_of(sc.xa), g, sc.max_chunks, max_rows, sc.gu, s), "moe gate launch");
+    const float* up_out = sc.gu + inter;
+    size_t stride = 2 * inter;
+    if (!fused) {
+        g.bases = m->bases_up;
+        float* u = sc.gu + pairs * inter;
+        HIP_TRY(launch_decode_mfma_grouped(m->up[0]->v, view_of(sc.xa), g, sc.max_chunks, max_rows, u, s), "moe up launch");
+        up_out = u;
+        stride = inter;
+    }
+    HIP_TRY(launch_moe_act(sc.gu, up_out, stride, pairs, inter, m->act_kind, m->act_param, sc.a, s), "moe act launch");
+    HIP_TRY(launch_quantize_act(sc.a, pairs, inter, sc.aq, s), "moe quantize launch");
+    g.rowmap = nullptr;
+    g.bases = m->bases_dn;
+    HIP_TRY(launch_decode_mfma_grouped(m->down[0]->v, view_of(sc.aq), g, sc.max_chunks, max_rows, sc.o, s), "moe down launch");
+    HIP_TRY(launch_moe_combine(sc.o, sc.row_of, route_w, t, k, h, y, s), "moe combine launch");
+    return 1;
+}
+
+}  // namespace
+
+extern "C" {
+
+void oxhip_free_moe(oxhip_ctx* c, oxhip_moe* m) {
+    if (!m) return;
+    if (c) {
+        (void)hipSetDevice(c->device);
+        (void)hipDeviceSynchronize();
+    }
+    for (auto* w : m->gate_up) oxhip_free_weight(c, w);
+    for (auto* w : m->up) oxhip_free_weight(c, w);
+    for (auto* w : m->down) oxhip_free_weight(c, w);
+    if (m->bases_gu) (void)hipFree(m->bases_gu);
+    if (m->bases_up) (void)hipFree(m->bases_up);
+    if (m->bases_dn) (void)hipFree(m->bases_dn);
+    m->ws.release();
+    delete m;
+}
+
+oxhip_moe* oxhip_upload_moe(oxhip_ctx* c, const oxhip_weight_desc* gate_up, const oxhip_weight_desc* up, const oxhip_weight_desc* down,
+                            size_t n_experts, size_t h, size_t inter, uint32_t act_kind, float act_param) {
+    if (!c || !gate_up || !down || !n_experts || !h || !inter) {
+        set_error("upload_moe: null argument");
+        return nullptr;
+    }
+    if (act_kind > OXHIP_ACT_SILU_CLAMP) {
+        set_error("upload_moe: this activation runs on the CPU only");
+        return nullptr;
+    }
+    if (h % 32 || inter % 32) {
+        set_error("upload_moe: h and inter must be multiples of 32");
+        return nullptr;
+    }
+    auto* m = new oxhip_moe();
+    m->n_exp = n_experts;
+    m->h = h;
+    m->inter = inter;
+    m->act_kind = act_kind;
+    m->act_param = act_param;
+    auto fail = [&](const std::string& why) -> oxhip_moe* {
+        const std::string msg = "upload_moe: " + why;
+        oxhip_free_moe(c, m);
+        set_error(msg);
+        return nullptr;
+    };
+    const size_t gu_rows = up ? inter : 2 * inter;
+    for (size_t e = 0; e < n_experts; e++) {
+        if (gate_up[e].n_out != gu_rows || gate_up[e].n_in != h || down[e].n_out != h || down[e].n_in != inter ||
+            (up && (up[e].n_out != inter || up[e].n_in != h)))
+            return fail("expert " + std::to_string(e) + " has another shape");
+        oxhip_weight* w = oxhip_upload(c, &gate_up[e]);
+        if (!w) return fail(oxhip_last_error());
+        m->gate_up.push_back(w);
+        if (up) {
+            w = oxhip_upload(c, &up[e]);
+            if (!w) return fail(oxhip_last_error());
+            m->up.push_back(w);
+        }
+        w = oxhip_upload(c, &down[e]);
+        if (!w) return fail(oxhip_last_error());
+        m->down.push_back(w);
+    }
+    auto same = [&](const std::vector<oxhip_weight*>& v) {
+        for (auto* w : v)
+            if (w->v.fmt != v[0]->v.fmt || !mfma_format(w)) return false;
+        return true;
+    };
+    if (!same(m->gate_up) || !same(m->down) || (up && !same(m->up))) return fail("experts must share one of the formats the grouped kernel runs (Q8_0, Q4_K, MLX Q4)");
+    auto table = [&](const std::vector<oxhip_weight*>& v, const uint8_t*** out) {
+        std::vector<const uint8_t*> host(v.size());
+        for (size_t i = 0; i < v.size(); i++) host[i] = v[i]->v.p0;
+        if (hipMalloc(reinterpret_cast<void**>(out), host.size() * sizeof(void*)) != hipSuccess) return false;
+        return hipMemcpy(*out, host.data(), host.size() * sizeof(void*), hipMemcpyHostToDevice) == hipSuccess;
+    };
+    if (!table(m->gate_up, &m->bases_gu) || !table(m->down, &m->bases_dn) || (up && !table(m->up, &m->bases_up)))
+        return fail("device memory short");
+    return m;
+}
+
+int oxhip_dev_route_top_k(oxhip_ctx* c, const float* logits, size_t t, size_t n_experts, size_t k, uint32_t* idx, float* w, void* stream) {
+    if (!c || !logits || !idx || !w || !k || k > 32 || k > n_experts || n_experts > 1024) {
+        set_error("route_top_k: bad arguments (k <= 32, k <= n_experts <= 1024)");
+        return 0;
+    }
+    HIP_TRY(launch_route_top_k(logits, t, n_experts, k, idx, w, static_cast<hipStream_t>(stream)), "route_top_k launch");
+    return 1;
+}
+
+int oxhip_dev_moe(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t* route_idx, const float* route_w, size_t k,
+                  float* y, void* stream) {
+    if (!c || !m || !x || !route_idx || !route_w || !y || !k) {
+        set_error("moe: null argument");
+        return 0;
+    }
+    return moe_run(c, m, x, t, route_idx, route_w, k, y, static_cast<hipStream_t>(stream));
+}
+
+int oxhip_moe_forward(oxhip_ctx* c, const float* x, size_t t, size_t h, size_t inter, const uint32_t* route_idx, const float* route_w,
+                      size_t k, oxhip_moe* m, float* y) {
+    if (!c || !m || !x || !route_idx || !route_w || !y || !t || !k || h != m->h || inter != m->inter) {
+        set_error("moe: bad arguments");
+        return 0;
+    }
+    for (size_t i = 0; i < t * k; i++)
+        if (route_idx[i] >= m->n_exp) {  // bad routes decline (src/cuda.rs:803-813)
+            set_error("moe: route to expert " + std::to_string(route_idx[i]) + " of " + std::to_string(m->n_exp));
+            return 0;
+        }
+    std::lock_guard<std::mutex> g(c->mu);
+    HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
+    hipStream_t s = c->stream;
+    const size_t xb = t * h * 4, rb = t * k * 4;
+    if (!c->x.grow(xb + 2 * up256(rb)) || !c->y.grow(xb)) {
+        set_error("moe: device memory short");
+        return 0;
+    }
+    uint8_t* xd = static_cast<uint8_t*>(c->x.p);
+    uint32_t* ri = reinterpret_cast<uint32_t*>(xd + up256(xb));
+    float* rw = reinterpret_cast<float*>(xd + up256(xb) + up256(rb));
+    HIP_TRY(hipMemcpyAsync(xd, x, xb, hipMemcpyHostToDevice, s), "moe copy-in");
+    HIP_TRY(hipMemcpyAsync(ri, route_idx, rb, hipMemcpyHostToDevice, s), "moe copy-in");
+    HIP_TRY(hipMemcpyAsync(rw, route_w, rb, hipMemcpyHostToDevice, s), "moe copy-in");
+    HIP_TRY(hipMemcpyAsync(c->y.p, y, xb, hipMemcpyHostToDevice, s), "moe copy-in");  // y is added to
+    if (!moe_run(c, m, reinterpret_cast<const float*>(xd), t, ri, rw, k, static_cast<float*>(c->y.p), s)) {
+        (void)hipStreamSynchronize(s);
+        return 0;
+    }
+    std::vector<float> host(t * h);
+    HIP_TRY(hipMemcpyAsync(host.data(), c->y.p, xb, hipMemcpyDeviceToHost, s), "moe copy-out");
+    HIP_TRY(hipStreamSynchronize(s), "moe");
+    std::memcpy(y, host.data(), xb);
+    c->calls++;
+    return 1;
+}
+
+// Backend::matvec_rows: y = W x, or y = silu(W x) * (U x) (silu_mul's fast_exp form), 1 <= t <= 4.
+int oxhip_matvec_rows(oxhip_ctx* c, const float* x, size_t t, size_t n_in, oxhip_rows_job* jobs, size_t n_jobs) {
+    if (!c || !x || !jobs || !n_jobs || t < 1 || t > 4 || n_in % 32) {
+        set_error("matvec_rows: bad arguments (1 <= t <= 4)");
+        return 0;
+    }
+    size_t y_total = 0;
+    bool any_q = false;
+    for (size_t j = 0; j < n_jobs; j++) {
+        const oxhip_rows_job& jb = jobs[j];
+        if (!jb.w || !jb.y || jb.w->v.n_in != n_in || jb.w->v.n_out != jb.n_out ||
+            (jb.up && (jb.up->v.n_in != n_in || jb.up->v.n_out != jb.n_out))) {
+            set_error("matvec_rows: job " + std::to_string(j) + " does not match its weights");
+            return 0;
+        }
+        y_total += t * jb.n_out * (jb.up ? 2 : 1);
+        any_q |= !is_dense(jb.w) || (jb.up && !is_dense(jb.up));
+    }
+    std::lock_guard<std::mutex> g(c->mu);
+    HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
+    hipStream_t s = c->stream;
+    if (!c->x.grow(t * n_in * 4) || !c->y.grow(y_total * 4) || (any_q && !c->xq.grow(qact_bytes(t, n_in)))) {
+        set_error("matvec_rows: device memory short");
+        return 0;
+    }
+    HIP_TRY(hipMemcpyAsync(c->x.p, x, t * n_in * 4, hipMemcpyHostToDevice, s), "matvec_rows copy-in");
+    oxhip_qact xa{};
+    if (any_q) {
+        xa = carve_qact(c->xq.p, t, n_in);
+        HIP_TRY(launch_quantize_act(static_cast<const float*>(c->x.p), t, n_in, xa, s), "quantize_act launch");
+    }
+    float* yd = static_cast<float*>(c->y.p);
+    size_t off = 0;
+    std::vector<size_t> at(n_jobs);
+    for (size_t j = 0; j < n_jobs; j++) {
+        const oxhip_rows_job& jb = jobs[j];
+        const size_t n = t * jb.n_out;
+        at[j] = off;
+        HIP_TRY(launch_decode(jb.w->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off, s), "decode launch");
+        if (jb.up) {
+            HIP_TRY(launch_decode(jb.up->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off + n, s), "decode launch");
+            HIP_TRY(launch_moe_act(yd + off, yd + off + n, jb.n_out, t, jb.n_out, OXHIP_ACT_SILU, 0.0f, yd + off, s), "act launch");
+        }
+        off += n * (jb.up ? 2 : 1);
+    }
+    std::vector<float> host(y_total);
+    HIP_TRY(hipMemcpyAsync(host.data(), yd, y_total * 4, hipMemcpyDeviceToHost, s), "matvec_rows copy-out");
+    HIP_TRY(hipStreamSynchronize(s), "matvec_rows");
+    for (size_t j = 0; j < n_jobs; j++) std::memcpy(jobs[j].y, host.data() + at[j], t * jobs[j].n_out * 4);
+    c->calls++;
+    return 1;
+}
+
+}  // extern "C"

@@ -22,6 +22,8 @@
 //
 // A workgroup owns `rt` row tiles and splits K over `kw` waves per tile; the partial sums meet in
 // LDS in a fixed order. No atomics, no second launch.
+#include <cstdlib>
+
 #include "internal.hpp"
 #include "layout.hpp"
 
@@ -40,15 +42,15 @@ struct Meta4 {
 };
 
 // LDS: xs | su | fs, each [nblk][TPAD] (su, fs only for the formats that use them)
-template <int TPAD, bool SUMS>
-__device__ __forceinline__ void stage_meta(const QActView& xa, uint32_t t, uint32_t nblk, float* lds) {
+template <int TPAD, bool SUMS, class RowOf>
+__device__ __forceinline__ void stage_meta(const QActView& xa, uint32_t t, uint32_t nblk, float* lds, RowOf row_of) {
     float* xs = lds;
     int* su = reinterpret_cast<int*>(lds + (size_t)nblk * TPAD);
     float* fs = lds + (size_t)2 * nblk * TPAD;
     for (uint32_t i = threadIdx.x; i < nblk * TPAD; i += blockDim.x) {
         uint32_t tok = i / nblk, b = i % nblk;  // consecutive threads read consecutive blocks of one token
         bool live = tok < t;
-        size_t src = (size_t)tok * nblk + b;
+        size_t src = (live ? row_of(tok) : 0) * nblk + b;
         xs[b * TPAD + tok] = live ? xa.scales[src] : 0.0f;
         if (SUMS) {
             su[b * TPAD + tok] = live ? xa.sums[src] : 0;
@@ -71,11 +73,38 @@ __device__ __forceinline__ void load_meta(const float* lds, uint32_t nblk, uint3
 
 }  // namespace
 
+// Everything one K-step needs from global memory, loaded a ring-length ahead of its use: the
+// record's 16 bytes of codes for this lane, the scales of its row, and the int8 activations this
+// lane feeds to the A operand (two dwords per MFMA).
+template <int FMT>
+struct Step;
+template <>
+struct Step<FMT_Q8_0> {
+    uint4 w;
+    uint32_t dd;
+    uint32_t a[2];
+};
+template <>
+struct Step<FMT_Q4_K> {
+    uint4 w;
+    uint32_t sc4, mn4, dd;
+    uint32_t a[4];
+};
+template <>
+struct Step<FMT_Q4M> {
+    uint4 w;
+    uint32_t dd, oo;
+    uint32_t a[4];
+};
+
 // FMT: FMT_Q8_0 / FMT_Q4_K / FMT_Q4M. NT: tokens handled (1, 2, 4 or 8). DUMP: also write the exact
 // integer block sums to `dump` ([t][n_out][n_in/32]) for parity checks.
-template <int FMT, int NT, bool DUMP>
-__global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw,
-                                                           float* __restrict__ y, int32_t* __restrict__ dump) {
+// GROUPED: blockIdx.y walks the chunks of a grouped launch (MoE experts over their routed tokens): chunk c is
+// {expert, first row, rows (<= 8)}; the weights are expert's, activation row i of the chunk is row
+// rowmap[first + i] of xa (or first + i without a map), and its output is row first + i of y.
+template <int FMT, int NT, bool DUMP, bool GROUPED>
+__global__ __launch_bounds__(512) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw,
+                                                           float* __restrict__ y, int32_t* __restrict__ dump, GroupView grp) {
     constexpr int TPAD = NT <= 4 ? 4 : 8;
     constexpr int NI = NT < 4 ? NT : 4;          // accumulator registers that hold live tokens
     constexpr bool SUMS = FMT != FMT_Q8_0;
@@ -86,33 +115,69 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
     const uint32_t r = wave / kw, ks = wave % kw;
     const uint32_t tile = blockIdx.x * rt + r;
     const uint32_t ntiles = row_tiles(w.n_out);
-
-    stage_meta<TPAD, SUMS>(xa, t, nblk, lds);
-    __syncthreads();
     float* red = lds + (size_t)(SUMS ? 3 : 1) * nblk * TPAD;  // [rt * kw][TPAD][16]
+    uint32_t row0 = 0;  // first activation / output row of this launch unit
+    if (GROUPED) {
+        if (blockIdx.y >= (uint32_t)*grp.nchunks) return;  // uniform over the workgroup
+        const int4 ch = grp.chunks[blockIdx.y];
+        w.p0 = grp.bases[ch.x];
+        row0 = (uint32_t)ch.y;
+        t = (uint32_t)ch.z;
+        y += (size_t)row0 * w.n_out;
+    }
+    auto src_row = [&](uint32_t i) -> size_t { return GROUPED && grp.rowmap ? (size_t)grp.rowmap[row0 + i] : (size_t)row0 + i; };
 
     // A role: slot n of this lane = (half, token); tokens past t read token t - 1 (their sums are dropped)
     const uint32_t a_half = n >> 3, a_tok = min(n & 7u, t - 1);
-    const int8_t* xrow = xa.q + (size_t)a_tok * w.n_in;
+    const int8_t* xrow = xa.q + src_row(a_tok) * w.n_in;
     const uint32_t amask0 = a_half ? 0u : 0xFFFFFFFFu, amask1 = ~amask0;
     // D role: this lane's registers are tokens 4 (kq & 1) + i of block parity kq >> 1
     const uint32_t d_half = kq >> 1, d_tok0 = 4 * (kq & 1);
 
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    const bool live_tile = tile < ntiles;
+    const uint32_t nsteps = FMT == FMT_Q8_0 ? t8_steps(w.n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in) : t4m_steps(w.n_in));
+    const uint32_t per = (nsteps + kw - 1) / kw;
+    const uint32_t s0 = ks * per;
+    const uint32_t s1 = tile < ntiles ? min(nsteps, s0 + per) : 0;  // a tile past the matrix streams nothing
+    const uint8_t* base = w.p0 + (size_t)min(tile, ntiles - 1) * (FMT == FMT_Q8_0   ? (size_t)nsteps * T8_REC
+                                                                  : FMT == FMT_Q4_K ? (size_t)(nsteps / 2) * TK4_REC
+                                                                                    : (size_t)nsteps * T4M_REC);
 
-    // One MFMA over a pair of blocks (b0 for half 0, b1 for half 1) with weight codes `bw`
-    auto block_pair = [&](v4i bw, uint32_t b0, uint32_t b1, uint32_t apos0, uint32_t apos1, bool split) -> v4i {
-        const uint32_t ab = min(a_half ? b1 : b0, nblk - 1);
-        uint32_t d0, d1;
-        if (split) {  // Q4M: positions 4 kq.. and 16 + 4 kq..
-            d0 = *reinterpret_cast<const uint32_t*>(xrow + ab * 32 + apos0);
-            d1 = *reinterpret_cast<const uint32_t*>(xrow + ab * 32 + apos1);
+    auto act2 = [&](uint32_t b, uint32_t pos, uint32_t* out) {  // 8 consecutive activations of block b
+        const uint2 v = *reinterpret_cast<const uint2*>(xrow + min(b, nblk - 1) * 32 + pos);
+        out[0] = v.x;
+        out[1] = v.y;
+    };
+    auto load_step = [&](Step<FMT>& st, uint32_t s) {
+        if constexpr (FMT == FMT_Q8_0) {
+            const uint8_t* rec = base + (size_t)s * T8_REC;
+            st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+            st.dd = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
+            act2(2 * s + a_half, 8 * kq, st.a);
+        } else if constexpr (FMT == FMT_Q4_K) {
+            const uint8_t* rec = base + (size_t)(s >> 1) * TK4_REC;
+            st.w = *reinterpret_cast<const uint4*>(rec + (s & 1) * 1024 + 16 * lane);
+            // this step's four sub-blocks are 4 (s & 1) .. + 3 of the super-block
+            st.sc4 = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 4 * (s & 1));
+            st.mn4 = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
+            st.dd = *reinterpret_cast<const uint32_t*>(rec + 2304 + 4 * n);
+            act2(4 * s + a_half, 8 * kq, st.a);
+            act2(4 * s + 2 + a_half, 8 * kq, st.a + 2);
         } else {
-            const uint2 v = *reinterpret_cast<const uint2*>(xrow + ab * 32 + apos0);
-            d0 = v.x;
-            d1 = v.y;
+            const uint8_t* rec = base + (size_t)s * T4M_REC;
+            st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+            st.dd = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
+            st.oo = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
+#pragma unroll
+            for (int g = 0; g < 2; g++) {  // positions 4 kq.. and 16 + 4 kq.. of block 4 s + 2 g + half
+                const int8_t* xb = xrow + min(4 * s + 2 * g + a_half, nblk - 1) * 32;
+                st.a[2 * g] = *reinterpret_cast<const uint32_t*>(xb + 4 * kq);
+                st.a[2 * g + 1] = *reinterpret_cast<const uint32_t*>(xb + 16 + 4 * kq);
+            }
         }
+    };
+
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto mfma = [&](v4i bw, uint32_t d0, uint32_t d1) -> v4i {
         v4i a = {(int)(d0 & amask0), (int)(d1 & amask0), (int)(d0 & amask1), (int)(d1 & amask1)};
         v4i c = {0, 0, 0, 0};
         return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bw, c, 0, 0, 0);
@@ -125,143 +190,85 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
         for (int i = 0; i < 4; i++)
             if (d_tok0 + i < t) dump[((size_t)(d_tok0 + i) * w.n_out + row) * nblk + b] = isum[i];
     };
-
-    if (live_tile) {
-        if (FMT == FMT_Q8_0) {
-            const uint32_t nsteps = t8_steps(w.n_in);
-            const uint32_t per = (nsteps + kw - 1) / kw;
-            const uint32_t s0 = ks * per, s1 = min(nsteps, s0 + per);
-            const uint8_t* base = w.p0 + (size_t)tile * nsteps * T8_REC;
-            uint4 ring[PF];
+    auto compute_step = [&](const Step<FMT>& st, uint32_t s) {
+        const uint4 c = st.w;
+        if constexpr (FMT == FMT_Q8_0) {
+            const float d = f16_bits_to_f32((uint16_t)(d_half ? st.dd >> 16 : st.dd & 0xFFFF));
+            v4i bw = {(int)c.x, (int)c.y, (int)c.z, (int)c.w};
+            v4i D = mfma(bw, st.a[0], st.a[1]);
+            const uint32_t b = 2 * s + d_half;
+            Meta4 m;
+            load_meta<TPAD, SUMS>(lds, nblk, min(b, nblk - 1), d_tok0, m);
+            int isum[4] = {D.x, D.y, D.z, D.w};
 #pragma unroll
-            for (int p = 0; p < PF; p++)
-                if (s0 + p < s1) ring[p] = *reinterpret_cast<const uint4*>(base + (size_t)(s0 + p) * T8_REC + 16 * lane);
-            for (uint32_t sb = s0; sb < s1; sb += PF) {
-                uint4 next[PF];
+            for (int i = 0; i < NI; i++) acc[i] += (d * m.xs[i]) * (float)isum[i];
+            dump_block(b, isum);
+        } else if constexpr (FMT == FMT_Q4_K) {
+            const float d = f16_bits_to_f32((uint16_t)(st.dd & 0xFFFF)), dmin = f16_bits_to_f32((uint16_t)(st.dd >> 16));
 #pragma unroll
-                for (int p = 0; p < PF; p++)
-                    if (sb + PF + p < s1) next[p] = *reinterpret_cast<const uint4*>(base + (size_t)(sb + PF + p) * T8_REC + 16 * lane);
+            for (int pr = 0; pr < 2; pr++) {  // the two byte pairs of the lane's chunk
+                const uint32_t lo = pr ? c.z : c.x, hi = pr ? c.w : c.y;
+                v4i bw = {(int)(lo & 0x0F0F0F0Fu), (int)(hi & 0x0F0F0F0Fu), (int)((lo >> 4) & 0x0F0F0F0Fu),
+                          (int)((hi >> 4) & 0x0F0F0F0Fu)};
+                v4i D = mfma(bw, st.a[2 * pr], st.a[2 * pr + 1]);
+                const uint32_t b = 4 * s + 2 * pr + d_half;  // global index of this lane's block of 32
+                const uint32_t q = 2 * pr + d_half;
+                const float sc = (float)((st.sc4 >> (8 * q)) & 0xFF), mn = (float)((st.mn4 >> (8 * q)) & 0xFF);
+                const float sv = d * sc;
+                const float mv = 8.0f * sv - dmin * mn;
+                Meta4 m;
+                load_meta<TPAD, SUMS>(lds, nblk, b, d_tok0, m);
+                int isum[4] = {D.x - 8 * m.su[0], D.y - 8 * m.su[1], D.z - 8 * m.su[2], D.w - 8 * m.su[3]};
 #pragma unroll
-                for (int p = 0; p < PF; p++) {
-                    const uint32_t s = sb + p;
-                    if (s >= s1) break;
-                    const uint4 c = ring[p];
-                    const uint32_t dd = *reinterpret_cast<const uint32_t*>(base + (size_t)s * T8_REC + 1024 + 4 * n);
-                    const float d = f16_bits_to_f32((uint16_t)(d_half ? dd >> 16 : dd & 0xFFFF));
-                    v4i bw = {(int)c.x, (int)c.y, (int)c.z, (int)c.w};
-                    v4i D = block_pair(bw, 2 * s, 2 * s + 1, 8 * kq, 0, false);
-                    const uint32_t b = 2 * s + d_half;
-                    Meta4 m;
-                    load_meta<TPAD, SUMS>(lds, nblk, min(b, nblk - 1), d_tok0, m);
-                    int isum[4] = {D.x, D.y, D.z, D.w};
-#pragma unroll
-                    for (int i = 0; i < NI; i++) acc[i] += (d * m.xs[i]) * (float)isum[i];
-                    dump_block(b, isum);
+                for (int i = 0; i < NI; i++) {
+                    acc[i] += (sv * m.xs[i]) * (float)isum[i];
+                    acc[i] += mv * m.fs[i];
                 }
-#pragma unroll
-                for (int p = 0; p < PF; p++) ring[p] = next[p];
+                dump_block(b, isum);
             }
-        } else if (FMT == FMT_Q4_K) {
-            const uint32_t nsb = tk4_sbs(w.n_in);
-            const uint32_t nsteps = 2 * nsb;
-            const uint32_t per = (nsteps + kw - 1) / kw;
-            const uint32_t s0 = ks * per, s1 = min(nsteps, s0 + per);
-            const uint8_t* base = w.p0 + (size_t)tile * nsb * TK4_REC;
-            auto rec = [&](uint32_t s) { return base + (size_t)(s >> 1) * TK4_REC + (s & 1) * 1024; };
-            uint4 ring[PF];
+        } else {
 #pragma unroll
-            for (int p = 0; p < PF; p++)
-                if (s0 + p < s1) ring[p] = *reinterpret_cast<const uint4*>(rec(s0 + p) + 16 * lane);
-            for (uint32_t sb = s0; sb < s1; sb += PF) {
-                uint4 next[PF];
+            for (int g = 0; g < 2; g++) {  // the two groups of 64 of the step
+                const uint32_t w0 = g ? c.z : c.x, w1 = g ? c.w : c.y;  // blocks 2 g, 2 g + 1
+                v4i bw = {(int)(w0 & 0x0F0F0F0Fu), (int)((w0 >> 4) & 0x0F0F0F0Fu), (int)(w1 & 0x0F0F0F0Fu),
+                          (int)((w1 >> 4) & 0x0F0F0F0Fu)};
+                v4i D = mfma(bw, st.a[2 * g], st.a[2 * g + 1]);
+                const uint32_t b = 4 * s + 2 * g + d_half;
+                const float d = f16_bits_to_f32((uint16_t)(g ? st.dd >> 16 : st.dd & 0xFFFF));
+                const float off = bf16_bits_to_f32((uint16_t)(g ? st.oo >> 16 : st.oo & 0xFFFF));
+                Meta4 m;
+                load_meta<TPAD, SUMS>(lds, nblk, min(b, nblk - 1), d_tok0, m);
+                int isum[4] = {D.x - 8 * m.su[0], D.y - 8 * m.su[1], D.z - 8 * m.su[2], D.w - 8 * m.su[3]};
+                if (b < nblk) {  // padding blocks hold zero codes, but the -8 would still count
 #pragma unroll
-                for (int p = 0; p < PF; p++)
-                    if (sb + PF + p < s1) next[p] = *reinterpret_cast<const uint4*>(rec(sb + PF + p) + 16 * lane);
-#pragma unroll
-                for (int p = 0; p < PF; p++) {
-                    const uint32_t s = sb + p;
-                    if (s >= s1) break;
-                    const uint4 c = ring[p];
-                    const uint8_t* mt = base + (size_t)(s >> 1) * TK4_REC + 2048;
-                    // this step's four sub-blocks are 4 (s & 1) .. + 3 of the super-block
-                    const uint32_t sc4 = *reinterpret_cast<const uint32_t*>(mt + 16 * n + 4 * (s & 1));
-                    const uint32_t mn4 = *reinterpret_cast<const uint32_t*>(mt + 16 * n + 8 + 4 * (s & 1));
-                    const uint32_t dd = *reinterpret_cast<const uint32_t*>(mt + 256 + 4 * n);
-                    const float d = f16_bits_to_f32((uint16_t)(dd & 0xFFFF)), dmin = f16_bits_to_f32((uint16_t)(dd >> 16));
-#pragma unroll
-                    for (int pr = 0; pr < 2; pr++) {  // the two byte pairs of the lane's chunk
-                        const uint32_t lo = pr ? c.z : c.x, hi = pr ? c.w : c.y;
-                        v4i bw = {(int)(lo & 0x0F0F0F0Fu), (int)(hi & 0x0F0F0F0Fu), (int)((lo >> 4) & 0x0F0F0F0Fu),
-                                  (int)((hi >> 4) & 0x0F0F0F0Fu)};
-                        const uint32_t b0 = 4 * s + 2 * pr;  // global block (sub-block) index of half 0
-                        v4i D = block_pair(bw, b0, b0 + 1, 8 * kq, 0, false);
-                        const uint32_t q = 2 * pr + d_half;
-                        const float sc = (float)((sc4 >> (8 * q)) & 0xFF), mn = (float)((mn4 >> (8 * q)) & 0xFF);
-                        const float sv = d * sc;
-                        const float mv = 8.0f * sv - dmin * mn;
-                        Meta4 m;
-                        load_meta<TPAD, SUMS>(lds, nblk, b0 + d_half, d_tok0, m);
-                        int isum[4] = {D.x - 8 * m.su[0], D.y - 8 * m.su[1], D.z - 8 * m.su[2], D.w - 8 * m.su[3]};
-#pragma unroll
-                        for (int i = 0; i < NI; i++) {
-                            acc[i] += (sv * m.xs[i]) * (float)isum[i];
-                            acc[i] += mv * m.fs[i];
-                        }
-                        dump_block(b0 + d_half, isum);
+                    for (int i = 0; i < NI; i++) {
+                        acc[i] += ((float)isum[i] * d) * m.xs[i];
+                        acc[i] += off * m.fs[i];
                     }
                 }
-#pragma unroll
-                for (int p = 0; p < PF; p++) ring[p] = next[p];
-            }
-        } else {  // FMT_Q4M
-            const uint32_t nsteps = t4m_steps(w.n_in);
-            const uint32_t per = (nsteps + kw - 1) / kw;
-            const uint32_t s0 = ks * per, s1 = min(nsteps, s0 + per);
-            const uint8_t* base = w.p0 + (size_t)tile * nsteps * T4M_REC;
-            uint4 ring[PF];
-#pragma unroll
-            for (int p = 0; p < PF; p++)
-                if (s0 + p < s1) ring[p] = *reinterpret_cast<const uint4*>(base + (size_t)(s0 + p) * T4M_REC + 16 * lane);
-            for (uint32_t sb = s0; sb < s1; sb += PF) {
-                uint4 next[PF];
-#pragma unroll
-                for (int p = 0; p < PF; p++)
-                    if (sb + PF + p < s1) next[p] = *reinterpret_cast<const uint4*>(base + (size_t)(sb + PF + p) * T4M_REC + 16 * lane);
-#pragma unroll
-                for (int p = 0; p < PF; p++) {
-                    const uint32_t s = sb + p;
-                    if (s >= s1) break;
-                    const uint4 c = ring[p];
-                    const uint8_t* rc = base + (size_t)s * T4M_REC;
-                    const uint32_t dd = *reinterpret_cast<const uint32_t*>(rc + 1024 + 4 * n);
-                    const uint32_t oo = *reinterpret_cast<const uint32_t*>(rc + 1088 + 4 * n);
-#pragma unroll
-                    for (int g = 0; g < 2; g++) {  // the two groups of 64 of the step
-                        const uint32_t w0 = g ? c.z : c.x, w1 = g ? c.w : c.y;  // blocks 2 g, 2 g + 1
-                        v4i bw = {(int)(w0 & 0x0F0F0F0Fu), (int)((w0 >> 4) & 0x0F0F0F0Fu), (int)(w1 & 0x0F0F0F0Fu),
-                                  (int)((w1 >> 4) & 0x0F0F0F0Fu)};
-                        const uint32_t b0 = 4 * s + 2 * g;
-                        v4i D = block_pair(bw, b0, b0 + 1, 4 * kq, 16 + 4 * kq, true);
-                        const float d = f16_bits_to_f32((uint16_t)(g ? dd >> 16 : dd & 0xFFFF));
-                        const float off = bf16_bits_to_f32((uint16_t)(g ? oo >> 16 : oo & 0xFFFF));
-                        Meta4 m;
-                        load_meta<TPAD, SUMS>(lds, nblk, min(b0 + d_half, nblk - 1), d_tok0, m);
-                        int isum[4] = {D.x - 8 * m.su[0], D.y - 8 * m.su[1], D.z - 8 * m.su[2], D.w - 8 * m.su[3]};
-                        const bool real = b0 + d_half < nblk;  // padding blocks hold zero codes but the -8 still applies
-#pragma unroll
-                        for (int i = 0; i < NI; i++) {
-                            if (real) {
-                                acc[i] += ((float)isum[i] * d) * m.xs[i];
-                                acc[i] += off * m.fs[i];
-                            }
-                        }
-                        dump_block(b0 + d_half, isum);
-                    }
-                }
-#pragma unroll
-                for (int p = 0; p < PF; p++) ring[p] = next[p];
+                dump_block(b, isum);
             }
         }
+    };
+
+    // The first ring of records is requested before anything else, so that HBM latency overlaps the
+    // staging of the activation scales.
+    Step<FMT> ring[PF];
+#pragma unroll
+    for (int p = 0; p < PF; p++)
+        if (s0 + p < s1) load_step(ring[p], s0 + p);
+    stage_meta<TPAD, SUMS>(xa, t, nblk, lds, src_row);
+    __syncthreads();
+    for (uint32_t sb = s0; sb < s1; sb += PF) {
+        Step<FMT> next[PF];
+#pragma unroll
+        for (int p = 0; p < PF; p++)
+            if (sb + PF + p < s1) load_step(next[p], sb + PF + p);
+#pragma unroll
+        for (int p = 0; p < PF; p++)
+            if (sb + p < s1) compute_step(ring[p], sb + p);
+#pragma unroll
+        for (int p = 0; p < PF; p++) ring[p] = next[p];
     }
     // the two block parities of a token meet across lane groups kq and kq ^ 2
 #pragma unroll
@@ -293,8 +300,12 @@ struct Shape {
 // about 4096-8192 waves exist while each keeps a few records to stream.
 Shape shape_for(uint32_t ntiles, uint32_t nsteps) {
     uint32_t kw = 1;
-    while (kw < 16 && (size_t)ntiles * kw < 4096 && nsteps / (kw * 2) >= 4) kw *= 2;
+    while (kw < 8 && (size_t)ntiles * kw < 4096 && nsteps / (kw * 2) >= 4) kw *= 2;
     if (kw < 4 && nsteps / 4 >= 2) kw = 4;
+    if (const char* e = getenv("OXHIP_DECODE_KW")) {  // developer override for tuning runs
+        uint32_t v = (uint32_t)atoi(e);
+        if (v >= 1 && v <= 8) kw = v;
+    }
     return Shape{1, kw};
 }
 
@@ -322,12 +333,12 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
         hipError_t e = hipSuccess;
         auto go = [&](auto kern) {
             if (lds > 48 * 1024) e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, v, tt, sh.rt, sh.kw, yo, du);
+            if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, v, tt, sh.rt, sh.kw, yo, du, GroupView{});
         };
-        if (tc == 1) go(decode_mfma_kernel<FMT, 1, DUMP>);
-        else if (tc == 2) go(decode_mfma_kernel<FMT, 2, DUMP>);
-        else if (tc <= 4) go(decode_mfma_kernel<FMT, 4, DUMP>);
-        else go(decode_mfma_kernel<FMT, 8, DUMP>);
+        if (tc == 1) go(decode_mfma_kernel<FMT, 1, DUMP, false>);
+        else if (tc == 2) go(decode_mfma_kernel<FMT, 2, DUMP, false>);
+        else if (tc <= 4) go(decode_mfma_kernel<FMT, 4, DUMP, false>);
+        else go(decode_mfma_kernel<FMT, 8, DUMP, false>);
         if (e != hipSuccess) return e;
         e = hipGetLastError();
         if (e != hipSuccess) return e;
@@ -336,7 +347,43 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
     return hipSuccess;
 }
 
+template <int FMT>
+hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks, uint32_t max_rows,
+                       float* y, hipStream_t s) {
+    const uint32_t ntiles = row_tiles(w.n_out);
+    const uint32_t nsteps = FMT == FMT_Q8_0 ? t8_steps(w.n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in) : t4m_steps(w.n_in));
+    // the same K split as a plain launch on this matrix, so that a row's sum is associated the same way
+    // (and is bit-identical) whether its expert runs alone or in a group
+    Shape sh = shape_for(ntiles, nsteps);
+    const uint32_t nblk = w.n_in / 32;
+    dim3 grid((ntiles + sh.rt - 1) / sh.rt, max_chunks), block(64 * sh.rt * sh.kw);
+    const int tpad = max_rows <= 4 ? 4 : 8;
+    const size_t lds = ((size_t)(FMT == FMT_Q8_0 ? 1 : 3) * nblk * tpad + (size_t)sh.rt * sh.kw * tpad * 16) * 4;
+    if (lds > 160 * 1024) return hipErrorInvalidValue;
+    hipError_t e = hipSuccess;
+    auto go = [&](auto kern) {
+        if (lds > 48 * 1024) e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, xa, 0u, sh.rt, sh.kw, y, nullptr, g);
+    };
+    if (max_rows == 1) go(decode_mfma_kernel<FMT, 1, false, true>);
+    else if (max_rows <= 4) go(decode_mfma_kernel<FMT, 4, false, true>);
+    else go(decode_mfma_kernel<FMT, 8, false, true>);
+    if (e != hipSuccess) return e;
+    return hipGetLastError();
+}
+
 }  // namespace
+
+hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks,
+                                      uint32_t max_rows_per_chunk, float* y, hipStream_t s) {
+    if (!max_chunks) return hipSuccess;
+    switch (w.fmt) {
+        case FMT_Q8_0: return run_grouped<FMT_Q8_0>(w, xa, g, max_chunks, max_rows_per_chunk, y, s);
+        case FMT_Q4_K: return run_grouped<FMT_Q4_K>(w, xa, g, max_chunks, max_rows_per_chunk, y, s);
+        case FMT_Q4M: return run_grouped<FMT_Q4M>(w, xa, g, max_chunks, max_rows_per_chunk, y, s);
+        default: return hipErrorInvalidValue;
+    }
+}
 
 hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, hipStream_t s) {
     switch (w.fmt) {

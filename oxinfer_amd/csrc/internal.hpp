@@ -48,12 +48,22 @@ struct QActView {
     const int32_t* sums16;
 };
 
+// A grouped launch (MoE): chunk c = {expert, first row, rows (<= 8), 0}; see decode_mfma.hip.
+struct GroupView {
+    const uint8_t* const* bases;  // per expert: tile-packed weights
+    const int4* chunks;
+    const int* nchunks;           // device scalar: chunks in use (the grid covers the worst case)
+    const int* rowmap;            // optional: activation row of each gathered row
+};
+
 // Launchers (each returns hipSuccess or the launch error).
 hipError_t launch_quantize_act(const float* x, size_t t, size_t n_in, const oxhip_qact& out, hipStream_t s);
 hipError_t launch_dequantize(const WeightView& w, size_t r0, size_t r1, float* out, hipStream_t s);
 hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s);
 hipError_t launch_isums(const WeightView& w, const QActView& xa, size_t t, int32_t* out, hipStream_t s);
 hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, hipStream_t s);
+hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks,
+                                      uint32_t max_rows_per_chunk, float* y, hipStream_t s);
 hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* out, hipStream_t s);
 hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t n_in, const WeightView& dst, hipStream_t s);
 hipError_t launch_pack_q4m(const uint8_t* q, const uint16_t* sc, const uint16_t* off, size_t n_out, size_t n_in, uint8_t* dst,
@@ -62,6 +72,14 @@ hipError_t launch_repack_mlx_q4(const uint32_t* w, const uint16_t* scales, const
                                 size_t n_in, size_t group, const WeightView& dst, hipStream_t s);
 hipError_t launch_q4_scale_groups(const uint16_t* sc32, size_t n_out, size_t n_in, size_t sgroup, uint16_t* dst,
                                   int* mismatch, hipStream_t s);
+
+hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, hipStream_t s);
+hipError_t launch_moe_plan(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, int* row_of, int* src, int4* chunks,
+                           int* nchunks, hipStream_t s);
+hipError_t launch_moe_act(const float* g, const float* u, size_t stride, size_t rows, size_t inter, uint32_t kind, float param,
+                          float* a, hipStream_t s);
+hipError_t launch_moe_combine(const float* o, const int* row_of, const float* route_w, size_t t, size_t k, size_t h, float* y,
+                              hipStream_t s);
 
 void set_error(const std::string& msg);
 

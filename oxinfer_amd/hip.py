@@ -32,6 +32,10 @@ class DecodeJob(C.Structure):
                 ("ev_start", C.c_void_p), ("ev_stop", C.c_void_p)]
 
 
+class RowsJob(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("up", C.c_void_p), ("n_out", C.c_size_t), ("y", C.c_void_p)]
+
+
 class QActC(C.Structure):
     _fields_ = [("q", C.c_void_p), ("scales", C.c_void_p), ("sums", C.c_void_p), ("fsums", C.c_void_p),
                 ("hsums", C.c_void_p), ("sums16", C.c_void_p), ("t", C.c_size_t), ("n_in", C.c_size_t)]
@@ -74,6 +78,12 @@ def load_library():
         "oxhip_dev_decode": (C.c_int, [vp, vp, C.POINTER(QActC), vp, sz, vp, vp]),
         "oxhip_dev_isums": (C.c_int, [vp, vp, C.POINTER(QActC), vp, vp]),
         "oxhip_dev_decode_batch": (C.c_int, [vp, C.POINTER(DecodeJob), sz, vp]),
+        "oxhip_matvec_rows": (C.c_int, [vp, vp, sz, sz, C.POINTER(RowsJob), sz]),
+        "oxhip_upload_moe": (vp, [vp, C.POINTER(WeightDesc), C.POINTER(WeightDesc), C.POINTER(WeightDesc), sz, sz, sz, C.c_uint32, C.c_float]),
+        "oxhip_free_moe": (None, [vp, vp]),
+        "oxhip_moe_forward": (C.c_int, [vp, vp, sz, sz, sz, vp, vp, sz, vp, vp]),
+        "oxhip_dev_route_top_k": (C.c_int, [vp, vp, sz, sz, sz, vp, vp, vp]),
+        "oxhip_dev_moe": (C.c_int, [vp, vp, vp, sz, vp, vp, sz, vp, vp]),
         "oxhip_event_create": (vp, []),
         "oxhip_event_destroy": (None, [vp]),
         "oxhip_event_elapsed_ms": (C.c_float, [vp, vp]),
@@ -103,6 +113,21 @@ class DeviceWeight:
         if getattr(self, "handle", None) and self.be.ctx:
             load_library().oxhip_free_weight(self.be.ctx, self.handle)
             self.handle = None
+
+
+class DeviceMoe:
+    """`DeviceWeight` of the routed experts of one MoE layer (Backend::upload_moe, src/gpu.rs:206-216)."""
+
+    def __init__(self, be, handle, n_exp, h, inter):
+        self.be, self.handle, self.n_exp, self.h, self.inter = be, handle, n_exp, h, inter
+
+    def __del__(self):
+        if getattr(self, "handle", None) and self.be.ctx:
+            load_library().oxhip_free_moe(self.be.ctx, self.handle)
+            self.handle = None
+
+
+ACT_SILU, ACT_GELU_TANH, ACT_SILU_CLAMP = 0, 1, 2
 
 
 class QAct:
@@ -156,6 +181,63 @@ class HipBackend:
         h = self.lib.oxhip_upload(self.ctx, C.byref(desc))
         del keep
         return DeviceWeight(self, h, desc.n_out, desc.n_in) if h else None
+
+    @staticmethod
+    def desc_gguf(ggml_type, data, n_out, n_in):
+        data = np.ascontiguousarray(data, np.uint8)
+        return WeightDesc(kind=W_GGUF, ggml_type=ggml_type, n_out=n_out, n_in=n_in, data=_np_ptr(data)), (data,)
+
+    @staticmethod
+    def desc_mlx_q4(w, scales, biases, group, n_out, n_in):
+        w = np.ascontiguousarray(w, np.uint32)
+        scales, biases = np.ascontiguousarray(scales, np.uint16), np.ascontiguousarray(biases, np.uint16)
+        return (WeightDesc(kind=W_MLX_Q4, n_out=n_out, n_in=n_in, data=_np_ptr(w), scales=_np_ptr(scales), offsets=_np_ptr(biases),
+                           group=group), (w, scales, biases))
+
+    def upload_moe(self, gate_up, down, h, inter, up=None, act=ACT_SILU, act_param=0.0):
+        """Backend::upload_moe: gate_up / down (/ up) are lists of (WeightDesc, keepalive) per expert."""
+        n = len(gate_up)
+
+        def arr(ds):
+            a = (WeightDesc * n)()
+            for i, (d, _) in enumerate(ds):
+                a[i] = d
+            return a
+        hnd = self.lib.oxhip_upload_moe(self.ctx, arr(gate_up), arr(up) if up else None, arr(down), n, h, inter, act, act_param)
+        return DeviceMoe(self, hnd, n, h, inter) if hnd else None
+
+    def moe(self, x, t, h, inter, route_idx, route_w, k, dev, y):
+        """Backend::moe: adds the routed experts' output into y ([t, h] f32, host). False = declined, y untouched."""
+        x = np.ascontiguousarray(x, np.float32)
+        ri, rw = np.ascontiguousarray(route_idx, np.uint32), np.ascontiguousarray(route_w, np.float32)
+        assert y.dtype == np.float32 and y.flags.c_contiguous
+        return bool(self.lib.oxhip_moe_forward(self.ctx, _np_ptr(x), t, h, inter, _np_ptr(ri), _np_ptr(rw), k, dev.handle, _np_ptr(y)))
+
+    def dev_moe(self, dev, x, route_idx, route_w, y):
+        """The same on device tensors: x [t, h] f32, route_idx [t, k] int32 (values as u32), route_w [t, k] f32, y += ."""
+        t, k = route_idx.shape
+        if not self.lib.oxhip_dev_moe(self.ctx, dev.handle, x.data_ptr(), t, route_idx.data_ptr(), route_w.data_ptr(), k,
+                                      y.data_ptr(), self._stream()):
+            raise RuntimeError(self.last_error())
+        return y
+
+    def route_top_k(self, logits, k):
+        """moe::route_top_k on device logits [t, n_experts] -> (idx int32 [t, k], w f32 [t, k])."""
+        import torch
+        t, n = logits.shape
+        idx = torch.empty((t, k), dtype=torch.int32, device=logits.device)
+        w = torch.empty((t, k), dtype=torch.float32, device=logits.device)
+        if not self.lib.oxhip_dev_route_top_k(self.ctx, logits.data_ptr(), t, n, k, idx.data_ptr(), w.data_ptr(), self._stream()):
+            raise RuntimeError(self.last_error())
+        return idx, w
+
+    def matvec_rows(self, x, t, n_in, jobs):
+        """Backend::matvec_rows: jobs = [(w, up or None, y ndarray [t, n_out])], 1 <= t <= 4."""
+        x = np.ascontiguousarray(x, np.float32)
+        arr = (RowsJob * len(jobs))()
+        for i, (w, up, y) in enumerate(jobs):
+            arr[i] = RowsJob(w.handle, up.handle if up is not None else None, w.n_out, y.ctypes.data)
+        return bool(self.lib.oxhip_matvec_rows(self.ctx, _np_ptr(x), t, n_in, arr, len(jobs)))
 
     def upload_gguf(self, ggml_type, data, n_out, n_in):
         """WeightRef::Gguf: raw blocks, rows of `row_bytes` (src/ggml.rs:240-248)."""

@@ -1,0 +1,174 @@
+"""GPU parity of the MoE expert path (routing, grouped expert matmuls, activation, combination) against
+the CPU oracle, through the C ABI. Shapes follow the reference's tests (src/moe.rs:1135-1219: 6 experts,
+top-3; src/cuda.rs:2145-2179) with widths that are whole MLX groups."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+Q8_0, Q4_K = 8, 12
+
+
+@pytest.fixture(scope="module")
+def be():
+    from oxinfer_amd import HipBackend
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+def row_err(y, ref):
+    m = np.maximum(np.abs(ref).max(axis=1), 1e-30)
+    return float((np.abs(y - ref).max(axis=1) / m).max())
+
+
+def make_routes(oxref, t, ne, k, seed):
+    from oxinfer_amd import synth
+    logits = synth.router_logits(t, ne, seed)
+    idx = np.zeros((t, k), np.uint32)
+    w = np.zeros((t, k), np.float32)
+    for i in range(t):
+        idx[i], w[i] = oxref.route_top_k(logits[i], k)
+    return logits, idx, w
+
+
+def test_route_top_k_matches_oracle_and_definition(be, oxref):
+    import torch
+    from oxinfer_amd import synth
+    t, ne, k = 33, 128, 8
+    logits = synth.router_logits(t, ne, 5)
+    logits[0, 7] = logits[0, 90] = logits[0].max() + 1.0   # a tie at the top: the lower index first
+    logits[1, :] = 0.25                                      # all equal: indices 0..k-1
+    logits[2, 3] = -0.0
+    logits[2, 4] = 0.0                                       # total order: +0.0 above -0.0
+    idx, w = be.route_top_k(torch.from_numpy(logits).cuda(), k)
+    idx, w = idx.cpu().numpy().astype(np.uint32), w.cpu().numpy()
+    for i in range(t):
+        ri, rw = oxref.route_top_k(logits[i], k)
+        assert np.array_equal(idx[i], ri), i
+        assert np.allclose(w[i], rw, rtol=1e-6, atol=0)
+        # the definition: softmax over all experts, the k largest, renormalized
+        p = np.exp(logits[i].astype(np.float64) - logits[i].max())
+        p /= p.sum()
+        top = p[ri] / p[ri].sum()
+        assert np.allclose(rw, top, rtol=1e-5)
+    assert list(idx[0, :2]) == [7, 90] and list(idx[1]) == list(range(k))
+
+
+def moe_reference(oxref, kind, gate_up, down, h, inter, x, idx, w, y0):
+    """Each (token, route) pair on the oracle's decode kernels, combined in route order (what
+    forward_batched computes row by row, src/moe.rs:438-617)."""
+    y = y0.copy()
+    t, k = idx.shape
+    for i in range(t):
+        for j in range(k):
+            e = int(idx[i, j])
+            if kind == "mlx":
+                gu = oxref.q4_decode(*gate_up[e], 64, 2 * inter, h, x[i], 1)[0]
+            else:
+                gu = oxref.gguf_decode(kind, gate_up[e], 2 * inter, h, x[i], 1)[0]
+            a = oxref.silu_mul(gu[:inter], gu[inter:])
+            if kind == "mlx":
+                o = oxref.q4_decode(*down[e], 64, h, inter, a, 1)[0]
+            else:
+                o = oxref.gguf_decode(kind, down[e], h, inter, a, 1)[0]
+            y[i] = y[i] + w[i, j] * o
+    return y
+
+
+@pytest.fixture(scope="module")
+def mlx_experts(oxref):
+    from oxinfer_amd import synth
+    ne, h, inter = 6, 256, 128
+    raw_gu = [synth.mlx_q4(2 * inter, h, 100 + e) for e in range(ne)]
+    raw_dn = [synth.mlx_q4(h, inter, 200 + e) for e in range(ne)]
+    q_gu = [oxref.from_mlx_q4(*r, 2 * inter, h, 64) for r in raw_gu]
+    q_dn = [oxref.from_mlx_q4(*r, h, inter, 64) for r in raw_dn]
+    return ne, h, inter, raw_gu, raw_dn, q_gu, q_dn
+
+
+def test_moe_mlx_matches_oracle(be, oxref, mlx_experts):
+    from oxinfer_amd import synth
+    ne, h, inter, raw_gu, raw_dn, q_gu, q_dn = mlx_experts
+    k = 3
+    dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)
+    assert dev is not None, be.last_error()
+    for t in (1, 2, 5, 7, 8, 19, 40):
+        x = synth.activations(t, h, 300 + t)
+        _, idx, w = make_routes(oxref, t, ne, k, 400 + t)
+        y0 = synth.activations(t, h, 500 + t)  # the call adds into y
+        y = y0.copy()
+        assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
+        ref = moe_reference(oxref, "mlx", q_gu, q_dn, h, inter, x, idx, w, y0)
+        assert row_err(y - y0, ref - y0) < 1e-3, t
+        # the oracle's own MoE driver agrees with the composition above (decode path)
+        ref2 = oxref.moe_q4(q_gu, q_dn, 64, h, inter, x, t, idx, w, y0, decode_path=True)
+        assert np.array_equal(ref2.view(np.uint32), ref.view(np.uint32))
+        if t >= 8:
+            # from 8 tokens on the CPU takes its grouped f32 path (exact activations, libm exp): the int8
+            # activations of the decode kernels stay within the reference's own bound for them against the
+            # exact product (3e-2, src/ggml.rs:1904)
+            ref3 = oxref.moe_q4(q_gu, q_dn, 64, h, inter, x, t, idx, w, y0, decode_path=False)
+            assert row_err(y - y0, ref3 - y0) < 3e-2, t
+
+
+def test_moe_batched_equals_one_at_a_time(be, oxref, mlx_experts):
+    """src/moe.rs:1135-1219: every token's row is bit-identical whether it runs alone or in a batch."""
+    from oxinfer_amd import synth
+    ne, h, inter, raw_gu, raw_dn, _, _ = mlx_experts
+    k, t = 3, 7
+    dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)
+    x = synth.activations(t, h, 1)
+    _, idx, w = make_routes(oxref, t, ne, k, 2)
+    y = np.zeros((t, h), np.float32)
+    assert be.moe(x, t, h, inter, idx, w, k, dev, y)
+    for i in range(t):
+        y1 = np.zeros((1, h), np.float32)
+        assert be.moe(x[i:i + 1], 1, h, inter, idx[i:i + 1], w[i:i + 1], k, dev, y1)
+        assert np.array_equal(y1[0].view(np.uint32), y[i].view(np.uint32)), i
+
+
+@pytest.mark.parametrize("kind", [Q8_0, Q4_K])
+def test_moe_gguf_experts(be, oxref, kind):
+    from oxinfer_amd import synth
+    ne, h, inter, k = 4, 256, 256, 2
+    gu = [oxref.random_blocks(kind, 2 * inter * h // oxref.block_size(kind), 10 + e)[0] for e in range(ne)]
+    dn = [oxref.random_blocks(kind, h * inter // oxref.block_size(kind), 20 + e)[0] for e in range(ne)]
+    dev = be.upload_moe([be.desc_gguf(kind, g, 2 * inter, h) for g in gu], [be.desc_gguf(kind, d, h, inter) for d in dn], h, inter)
+    assert dev is not None, be.last_error()
+    for t in (1, 3, 11):
+        x = synth.activations(t, h, 30 + t)
+        _, idx, w = make_routes(oxref, t, ne, k, 40 + t)
+        y = np.zeros((t, h), np.float32)
+        assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
+        ref = moe_reference(oxref, kind, gu, dn, h, inter, x, idx, w, np.zeros((t, h), np.float32))
+        assert row_err(y, ref) < 1e-3, t
+
+
+def test_moe_declines(be, oxref, mlx_experts):
+    ne, h, inter, raw_gu, raw_dn, _, _ = mlx_experts
+    dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)
+    y = np.full((1, h), np.nan, np.float32)
+    bad = np.array([[0, 1, ne]], np.uint32)  # a route past the experts (src/cuda.rs:803-813)
+    assert not be.moe(np.zeros((1, h), np.float32), 1, h, inter, bad, np.ones((1, 3), np.float32), 3, dev, y)
+    assert np.isnan(y).all() and "route" in be.last_error()
+    # a CPU-only activation kind is declined at upload
+    assert be.upload_moe([be.desc_mlx_q4(*raw_gu[0], 64, 2 * inter, h)], [be.desc_mlx_q4(*raw_dn[0], 64, h, inter)], h, inter, act=3) is None
+
+
+def test_matvec_rows(be, oxref):
+    """Backend::matvec_rows (src/gpu.rs:165): plain and silu(W x) * (U x) products, t in 1..=4."""
+    n_out, n_in = 96, 512
+    wk, _ = oxref.random_blocks(Q4_K, n_out * n_in // 256, 3)
+    uk, _ = oxref.random_blocks(Q4_K, n_out * n_in // 256, 4)
+    w, u = be.upload_gguf(Q4_K, wk, n_out, n_in), be.upload_gguf(Q4_K, uk, n_out, n_in)
+    from oxinfer_amd import synth
+    for t in (1, 4):
+        x = synth.activations(t, n_in, 50 + t)
+        y0, y1 = np.zeros((t, n_out), np.float32), np.zeros((t, n_out), np.float32)
+        assert be.matvec_rows(x, t, n_in, [(w, None, y0), (w, u, y1)]), be.last_error()
+        g = oxref.gguf_decode(Q4_K, wk, n_out, n_in, x, t)
+        assert row_err(y0, g) < 1e-3
+        ref = oxref.silu_mul(g, oxref.gguf_decode(Q4_K, uk, n_out, n_in, x, t))
+        assert row_err(y1, ref) < 1e-3
+    assert not be.matvec_rows(np.zeros((5, n_in), np.float32), 5, n_in, [(w, None, np.zeros((5, n_out), np.float32))])
