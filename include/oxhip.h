@@ -152,6 +152,15 @@ void* oxhip_event_create(void);
 void oxhip_event_destroy(void* ev);
 /* Milliseconds between two recorded events; waits for `stop`. Negative on error. */
 float oxhip_event_elapsed_ms(void* start, void* stop);
+/* Prefill: y [t, n_out] = x [t, n_in] W^T on the matrix cores (what matmul_quant_multi's GEMM paths compute,
+ * src/kernels.rs:1774-1847). x_dtype / y_dtype: OXHIP_F32 or OXHIP_BF16. variant:
+ *   OXHIP_GEMM_BF16  weights dequantized to bf16 (through LDS), bf16 MFMA, f32 accumulation (the x86 CPU's
+ *                    f32 GEMM rounded to bf16 operands);
+ * Packed activations live in scratch owned by ctx (grown on first use; calls on one ctx must not overlap). */
+enum { OXHIP_F32 = 0, OXHIP_BF16 = 1 };
+enum { OXHIP_GEMM_BF16 = 0 };
+int oxhip_dev_gemm(oxhip_ctx* ctx, const oxhip_weight* w, const void* x, int x_dtype, size_t t, void* y, int y_dtype, int variant,
+                   void* stream);
 /* moe::route_top_k (src/moe.rs:180-193) for t rows of n_experts logits (n_experts <= 1024, k <= 32):
  * idx / w [t, k], sorted by descending logit, ties to the lower index, w = softmax over the k. */
 int oxhip_dev_route_top_k(oxhip_ctx* ctx, const float* logits, size_t t, size_t n_experts, size_t k, uint32_t* idx, float* w,

@@ -1,0 +1,217 @@
+// Prefill GEMM, variant (a): weights dequantized to bf16 on the way to the matrix cores, bf16 MFMA with f32
+// accumulation. y[t][n_out] = x[t][n_in] * W^T for the tile-packed MLX 4-bit format.
+//
+// The CPU computes this product from the f32-dequantized rows with one fused multiply-add chain per output
+// (matmul_quant_block_prefill + gemm_8x8, src/kernels.rs:1998-2038, src/kernels_x86.rs:296-324 of the reference);
+// here weights and activations are rounded to bf16 first, so results agree to bf16 precision, not bit for bit.
+//
+// Work split: a workgroup of 4 waves owns 256 tokens x 128 weight rows; wave v owns tokens 64 v .. 64 v + 63 and
+// all 128 rows (4 x 8 MFMA tiles of 16 x 16, 128 accumulator registers).
+//   B (weights): each K-step of 128 the four waves dequantize the step's 8 row tiles (two each) from the packed
+//     records into bf16 MFMA fragments in LDS (double-buffered, one barrier per step); every wave then reads all
+//     8 x 4 fragments with ds_read_b128. A weight is dequantized once per workgroup: (code - 8) * d + offset in
+//     f32 as one fma(code, d, offset - 8 d), rounded to bf16.
+//   A (activations): packed beforehand (pack_a_kernel) into MFMA fragments, one 1 KiB record per (16 tokens,
+//     block of 32) in the K order the weight fragments use, so a wave fetches its fragment with one coalesced
+//     16-byte-per-lane load straight from global memory / L2, a block ahead of its use.
+#include "internal.hpp"
+#include "layout.hpp"
+
+namespace oxhip {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Activations [t][n_in] (f32 or bf16) -> fragments [mtile][block][lane][8 bf16]; lane = 16 kq + m holds token
+// 16 mtile + m at K positions 32 b + 4 kq + {0..3} then 32 b + 16 + 4 kq + {0..3} (SPLIT, the order of the
+// nibble pairs of Q4 bytes) or 32 b + 8 kq + {0..7}. Tokens past t and columns past n_in are zero.
+template <bool SPLIT, bool SRC_BF16>
+__global__ __launch_bounds__(256) void pack_a_kernel(const void* __restrict__ x, uint32_t t, uint32_t n_in, uint32_t mtiles,
+                                                     uint32_t kblocks, uint4* __restrict__ out) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)mtiles * kblocks * 64) return;
+    const uint32_t lane = idx & 63, m = lane & 15, kq = lane >> 4;
+    const uint32_t b = (idx >> 6) % kblocks, mt = (idx >> 6) / kblocks;
+    const uint32_t tok = mt * 16 + m;
+    uint32_t pk[4] = {0, 0, 0, 0};
+    if (tok < t) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t k = SPLIT ? 32 * b + (j < 4 ? 4 * kq + j : 16 + 4 * kq + (j - 4)) : 32 * b + 8 * kq + j;
+            uint16_t h = 0;
+            if (k < n_in) {
+                if (SRC_BF16) h = reinterpret_cast<const uint16_t*>(x)[(size_t)tok * n_in + k];
+                else h = f32_to_bf16_bits(reinterpret_cast<const float*>(x)[(size_t)tok * n_in + k]);
+            }
+            pk[j >> 1] |= (uint32_t)h << (16 * (j & 1));
+        }
+    }
+    out[idx] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+}
+
+hipError_t launch_pack_a(const void* x, bool src_bf16, bool split, size_t t, size_t n_in, size_t mtiles, size_t kblocks, void* out,
+                         hipStream_t s) {
+    size_t total = mtiles * kblocks * 64;
+    if (!total) return hipSuccess;
+    unsigned grid = (unsigned)((total + 255) / 256);
+    uint4* o = static_cast<uint4*>(out);
+    if (split) {
+        if (src_bf16) pack_a_kernel<true, true><<<grid, 256, 0, s>>>(x, (uint32_t)t, (uint32_t)n_in, (uint32_t)mtiles, (uint32_t)kblocks, o);
+        else pack_a_kernel<true, false><<<grid, 256, 0, s>>>(x, (uint32_t)t, (uint32_t)n_in, (uint32_t)mtiles, (uint32_t)kblocks, o);
+    } else {
+        if (src_bf16) pack_a_kernel<false, true><<<grid, 256, 0, s>>>(x, (uint32_t)t, (uint32_t)n_in, (uint32_t)mtiles, (uint32_t)kblocks, o);
+        else pack_a_kernel<false, false><<<grid, 256, 0, s>>>(x, (uint32_t)t, (uint32_t)n_in, (uint32_t)mtiles, (uint32_t)kblocks, o);
+    }
+    return hipGetLastError();
+}
+
+namespace {
+
+constexpr int WG_MT = 16;  // token tiles per workgroup (256 tokens), 4 per wave
+constexpr int WG_NT = 8;   // row tiles per workgroup (128 rows)
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+}
+
+// One dword of a T4M chunk (4 bytes of one block: low nibbles = elements 4 kq + i, high = 16 + 4 kq + i) -> the
+// lane's 8 bf16 of that block.
+__device__ __forceinline__ uint4 dequant_q4m(uint32_t w, float d, float c) {
+    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+    float f[8];
+    f[0] = __builtin_fmaf((float)(lo & 0xFF), d, c);
+    f[1] = __builtin_fmaf((float)((lo >> 8) & 0xFF), d, c);
+    f[2] = __builtin_fmaf((float)((lo >> 16) & 0xFF), d, c);
+    f[3] = __builtin_fmaf((float)(lo >> 24), d, c);
+    f[4] = __builtin_fmaf((float)(hi & 0xFF), d, c);
+    f[5] = __builtin_fmaf((float)((hi >> 8) & 0xFF), d, c);
+    f[6] = __builtin_fmaf((float)((hi >> 16) & 0xFF), d, c);
+    f[7] = __builtin_fmaf((float)(hi >> 24), d, c);
+    return make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
+}
+
+}  // namespace
+
+// grid: (row groups of 128, token groups of 256). apk: packed activations [mtiles][kblocks][64][16 B] with
+// kblocks = 4 * steps. OUT_BF16: y is bf16 [t][n_out], else f32.
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256) void gemm_q4m_bf16_kernel(WeightView w, const uint4* __restrict__ apk, uint32_t t, uint32_t mtiles,
+                                                            void* __restrict__ yv) {
+    extern __shared__ uint4 bfrag[];  // [2][4 blocks][8 row tiles][64 lanes]
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t n = lane & 15;
+    const uint32_t nsteps = t4m_steps(w.n_in), kblocks = 4 * nsteps;
+    const uint32_t ntiles = row_tiles(w.n_out);
+    const uint32_t nt0 = blockIdx.x * WG_NT;               // first row tile of the workgroup
+    const uint32_t mt0 = blockIdx.y * WG_MT + wave * 4;    // first token tile of the wave
+
+    // the two row tiles this wave dequantizes
+    const uint8_t* wbase[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) wbase[i] = w.p0 + (size_t)min(nt0 + 2 * wave + i, ntiles - 1) * nsteps * T4M_REC;
+    // A fragments of the wave's 4 token tiles (tiles past the end repeat the last one; their rows are not stored)
+    const uint4* abase[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) abase[i] = apk + ((size_t)min(mt0 + i, mtiles - 1) * kblocks) * 64 + lane;
+
+    f32x4 acc[4][WG_NT];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < WG_NT; j++) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    struct Raw {
+        uint4 c;
+        uint32_t dd, oo;
+    };
+    auto load_raw = [&](Raw* r, uint32_t s) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint8_t* rec = wbase[i] + (size_t)s * T4M_REC;
+            r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+            r[i].dd = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
+            r[i].oo = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
+        }
+    };
+    auto dequant_to_lds = [&](const Raw* r, uint32_t buf) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint32_t cw[4] = {r[i].c.x, r[i].c.y, r[i].c.z, r[i].c.w};
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const int g = b >> 1;
+                const float d = f16_bits_to_f32((uint16_t)(g ? r[i].dd >> 16 : r[i].dd & 0xFFFF));
+                const float off = bf16_bits_to_f32((uint16_t)(g ? r[i].oo >> 16 : r[i].oo & 0xFFFF));
+                bfrag[((buf * 4 + b) * WG_NT + 2 * wave + i) * 64 + lane] = dequant_q4m(cw[b], d, off - 8.0f * d);
+            }
+        }
+    };
+
+    Raw raw[2];
+    load_raw(raw, 0);
+    dequant_to_lds(raw, 0);
+    uint4 a_cur[4], a_nxt[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) a_cur[i] = abase[i][0];
+    __syncthreads();
+    for (uint32_t s = 0; s < nsteps; s++) {
+        const uint32_t buf = s & 1;
+        if (s + 1 < nsteps) load_raw(raw, s + 1);
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const uint32_t kb = 4 * s + b;
+            if (kb + 1 < kblocks) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) a_nxt[i] = abase[i][(size_t)(kb + 1) * 64];
+            }
+#pragma unroll
+            for (int j = 0; j < WG_NT; j++) {
+                const uint4 bv = bfrag[((buf * 4 + b) * WG_NT + j) * 64 + lane];
+                const bf16x8 bb = __builtin_bit_cast(bf16x8, bv);
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_cur[i]), bb, acc[i][j], 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) a_cur[i] = a_nxt[i];
+        }
+        if (s + 1 < nsteps) dequant_to_lds(raw, buf ^ 1);
+        __syncthreads();
+    }
+    // D[token 4 kq + r][row n] per tile
+    const uint32_t kq = lane >> 4;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int j = 0; j < WG_NT; j++) {
+            const uint32_t row = (nt0 + j) * 16 + n;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const uint32_t tok = (mt0 + i) * 16 + 4 * kq + r;
+                if (tok < t && row < w.n_out && mt0 + i < mtiles) {
+                    if (OUT_BF16) reinterpret_cast<uint16_t*>(yv)[(size_t)tok * w.n_out + row] = f32_to_bf16_bits(acc[i][j][r]);
+                    else reinterpret_cast<float*>(yv)[(size_t)tok * w.n_out + row] = acc[i][j][r];
+                }
+            }
+        }
+    }
+}
+
+hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, hipStream_t s) {
+    if (w.fmt != FMT_Q4M) return hipErrorInvalidValue;
+    dim3 grid((row_tiles(w.n_out) + WG_NT - 1) / WG_NT, (unsigned)((mtiles + WG_MT - 1) / WG_MT));
+    const size_t lds = 2 * 4 * WG_NT * 64 * 16;  // 64 KiB
+    hipError_t e;
+    if (out_bf16) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4m_bf16_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        gemm_q4m_bf16_kernel<true><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, y);
+    } else {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4m_bf16_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        gemm_q4m_bf16_kernel<false><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, y);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace oxhip
