@@ -14,6 +14,8 @@
 //   A (activations): packed beforehand (pack_a_kernel) into MFMA fragments, one 1 KiB record per (16 tokens,
 //     block of 32) in the K order the weight fragments use, so a wave fetches its fragment with one coalesced
 //     16-byte-per-lane load straight from global memory / L2, a block ahead of its use.
+#include <type_traits>
+
 #include "internal.hpp"
 #include "layout.hpp"
 
@@ -70,8 +72,11 @@ namespace {
 constexpr int WG_MT = 16;  // token tiles per workgroup (256 tokens), 4 per wave
 constexpr int WG_NT = 8;   // row tiles per workgroup (128 rows)
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+// Two f32 -> packed bf16 (round to nearest even) with the hardware conversion, one instruction, no branches.
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
 }
 
 // One dword of a T4M chunk (4 bytes of one block: low nibbles = elements 4 kq + i, high = 16 + 4 kq + i) -> the
@@ -133,51 +138,90 @@ __global__ __launch_bounds__(256) void gemm_q4m_bf16_kernel(WeightView w, const 
             r[i].oo = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
         }
     };
-    auto dequant_to_lds = [&](const Raw* r, uint32_t buf) {
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const uint32_t cw[4] = {r[i].c.x, r[i].c.y, r[i].c.z, r[i].c.w};
-#pragma unroll
-            for (int b = 0; b < 4; b++) {
-                const int g = b >> 1;
-                const float d = f16_bits_to_f32((uint16_t)(g ? r[i].dd >> 16 : r[i].dd & 0xFFFF));
-                const float off = bf16_bits_to_f32((uint16_t)(g ? r[i].oo >> 16 : r[i].oo & 0xFFFF));
-                bfrag[((buf * 4 + b) * WG_NT + 2 * wave + i) * 64 + lane] = dequant_q4m(cw[b], d, off - 8.0f * d);
-            }
-        }
-    };
-
-    Raw raw[2];
-    load_raw(raw, 0);
-    dequant_to_lds(raw, 0);
-    uint4 a_cur[4], a_nxt[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) a_cur[i] = abase[i][0];
-    __syncthreads();
-    for (uint32_t s = 0; s < nsteps; s++) {
-        const uint32_t buf = s & 1;
-        if (s + 1 < nsteps) load_raw(raw, s + 1);
+    auto dequant_tile = [&](const Raw& r, int i, uint32_t buf) {  // one of the wave's two row tiles, 4 blocks
+        const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
         for (int b = 0; b < 4; b++) {
-            const uint32_t kb = 4 * s + b;
-            if (kb + 1 < kblocks) {
+            const int g = b >> 1;
+            const float d = f16_bits_to_f32((uint16_t)(g ? r.dd >> 16 : r.dd & 0xFFFF));
+            const float off = bf16_bits_to_f32((uint16_t)(g ? r.oo >> 16 : r.oo & 0xFFFF));
+            bfrag[((buf * 4 + b) * WG_NT + 2 * wave + i) * 64 + lane] = dequant_q4m(cw[b], d, off - 8.0f * d);
+        }
+    };
+    auto read_b = [&](uint4* dst, uint32_t buf, uint32_t b) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) a_nxt[i] = abase[i][(size_t)(kb + 1) * 64];
+        for (int j = 0; j < WG_NT; j++) dst[j] = bfrag[((buf * 4 + b) * WG_NT + j) * 64 + lane];
+    };
+    auto read_a_step = [&](uint4 (*dst)[4], uint32_t st) {  // the A fragments of the 4 blocks of a step
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[b][i] = abase[i][(size_t)(4 * st + b) * 64];
+    };
+    // LDS traffic only: outstanding global loads (the prefetches) stay in flight across the barrier
+    auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    // B fragments are read from LDS one block ahead of the MFMAs that consume them; A fragments come from global
+    // memory a whole K-step (four blocks, ~2000 MFMA cycles) ahead, the packed records of the next step two blocks
+    // before they are dequantized into the other LDS buffer.
+    Raw raw[2];
+    load_raw(raw, 0);
+    uint4 a_cur[4][4], a_nxt[4][4], b_cur[WG_NT], b_nxt[WG_NT];
+    read_a_step(a_cur, 0);
+    dequant_tile(raw[0], 0, 0);
+    dequant_tile(raw[1], 1, 0);
+    if (nsteps > 1) load_raw(raw, 1);
+    lds_barrier();
+    read_b(b_cur, 0, 0);
+    // One K-step. MORE: another step follows (its records are dequantized during blocks 0 and 1, and block 3
+    // prefetches from the other LDS buffer after the barrier). LOAD2: the records of step s + 2 exist.
+    // The steady-state instance has no branches, so the whole step is scheduled as one region and the dequantizing
+    // VALU work is interleaved with the MFMAs instead of stalling the matrix pipe.
+    auto step = [&](uint32_t s, auto more_c, auto load2_c) {
+        constexpr bool MORE = decltype(more_c)::value, LOAD2 = decltype(load2_c)::value;
+        const uint32_t buf = s & 1;
+        if (MORE) read_a_step(a_nxt, s + 1);
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            if (b < 3) {
+                read_b(b_nxt, buf, b + 1);
+            } else if (MORE) {
+                lds_barrier();  // the other buffer is complete, and nobody still reads this one
+                read_b(b_nxt, buf ^ 1, 0);
             }
 #pragma unroll
             for (int j = 0; j < WG_NT; j++) {
-                const uint4 bv = bfrag[((buf * 4 + b) * WG_NT + j) * 64 + lane];
-                const bf16x8 bb = __builtin_bit_cast(bf16x8, bv);
+                const bf16x8 bb = __builtin_bit_cast(bf16x8, b_cur[j]);
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_cur[i]), bb, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_cur[b][i]), bb, acc[i][j], 0, 0, 0);
+            }
+            if (MORE && b == 0) dequant_tile(raw[0], 0, buf ^ 1);
+            if (MORE && b == 1) dequant_tile(raw[1], 1, buf ^ 1);
+            if (LOAD2 && b == 2) load_raw(raw, s + 2);
+            if (MORE && b < 2) {
+#pragma unroll
+                for (int k = 0; k < 32; k++) {  // one MFMA, then a few of the dequantizing VALU ops in its shadow
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+                }
             }
 #pragma unroll
-            for (int i = 0; i < 4; i++) a_cur[i] = a_nxt[i];
+            for (int j = 0; j < WG_NT; j++) b_cur[j] = b_nxt[j];
         }
-        if (s + 1 < nsteps) dequant_to_lds(raw, buf ^ 1);
-        __syncthreads();
-    }
+        if (MORE) {
+#pragma unroll
+            for (int b = 0; b < 4; b++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) a_cur[b][i] = a_nxt[b][i];
+        }
+    };
+    using T_ = std::integral_constant<bool, true>;
+    using F_ = std::integral_constant<bool, false>;
+    uint32_t s = 0;
+    for (; s + 2 < nsteps; s++) step(s, T_{}, T_{});
+    if (nsteps >= 2) step(s++, T_{}, F_{});
+    step(s, F_{}, F_{});
     // D[token 4 kq + r][row n] per tile
     const uint32_t kq = lane >> 4;
 #pragma unroll
