@@ -12,7 +12,9 @@ int gemm_bf16_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf1
         return 0;
     }
     const size_t mtiles = (t + 15) / 16, kblocks = 4 * (size_t)t4m_steps(w->v.n_in);
-    const size_t bytes = mtiles * kblocks * 64 * 16;
+    const size_t pack_bytes = align_up(mtiles * kblocks * 64 * 16, 256);
+    const uint32_t slices = gemm_k_slices(w->v, mtiles);
+    const size_t bytes = pack_bytes + (slices > 1 ? (size_t)slices * t * w->v.n_out * 4 : 0);
     if (c->gemm_ws.cap < bytes) {
         (void)hipStreamSynchronize(s);  // an earlier GEMM may still read the old scratch
         if (!c->gemm_ws.grow(bytes)) {
@@ -21,7 +23,8 @@ int gemm_bf16_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf1
         }
     }
     HIP_TRY(launch_pack_a(x, x_bf16, true, t, w->v.n_in, mtiles, kblocks, c->gemm_ws.p, s), "gemm pack launch");
-    HIP_TRY(launch_gemm_bf16(w->v, c->gemm_ws.p, t, mtiles, y, y_bf16, s), "gemm launch");
+    float* partial = reinterpret_cast<float*>(static_cast<uint8_t*>(c->gemm_ws.p) + pack_bytes);
+    HIP_TRY(launch_gemm_bf16(w->v, c->gemm_ws.p, t, mtiles, y, y_bf16, partial, s), "gemm launch");
     return 1;
 }
 

@@ -99,13 +99,18 @@ __device__ __forceinline__ uint4 dequant_q4m(uint32_t w, float d, float c) {
 
 // grid: (row groups of 128, token groups of 256). apk: packed activations [mtiles][kblocks][64][16 B] with
 // kblocks = 4 * steps. OUT_BF16: y is bf16 [t][n_out], else f32.
+// With gridDim.z > 1 the K-steps are split over z and each slice writes its partial sums as f32 to
+// yv + z * t * n_out (a second kernel adds the slices in order).
 template <bool OUT_BF16>
 __global__ __launch_bounds__(256) void gemm_q4m_bf16_kernel(WeightView w, const uint4* __restrict__ apk, uint32_t t, uint32_t mtiles,
                                                             void* __restrict__ yv) {
     extern __shared__ uint4 bfrag[];  // [2][4 blocks][8 row tiles][64 lanes]
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t n = lane & 15;
-    const uint32_t nsteps = t4m_steps(w.n_in), kblocks = 4 * nsteps;
+    const uint32_t all_steps = t4m_steps(w.n_in), kblocks = 4 * all_steps;
+    const uint32_t per_z = (all_steps + gridDim.z - 1) / gridDim.z;
+    const uint32_t step0 = blockIdx.z * per_z;              // this slice's K-steps: step0 .. step0 + nsteps
+    const uint32_t nsteps = min(all_steps, step0 + per_z) - step0;
     const uint32_t ntiles = row_tiles(w.n_out);
     const uint32_t nt0 = blockIdx.x * WG_NT;               // first row tile of the workgroup
     const uint32_t mt0 = blockIdx.y * WG_MT + wave * 4;    // first token tile of the wave
@@ -113,11 +118,11 @@ __global__ __launch_bounds__(256) void gemm_q4m_bf16_kernel(WeightView w, const 
     // the two row tiles this wave dequantizes
     const uint8_t* wbase[2];
 #pragma unroll
-    for (int i = 0; i < 2; i++) wbase[i] = w.p0 + (size_t)min(nt0 + 2 * wave + i, ntiles - 1) * nsteps * T4M_REC;
+    for (int i = 0; i < 2; i++) wbase[i] = w.p0 + ((size_t)min(nt0 + 2 * wave + i, ntiles - 1) * all_steps + step0) * T4M_REC;
     // A fragments of the wave's 4 token tiles (tiles past the end repeat the last one; their rows are not stored)
     const uint4* abase[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) abase[i] = apk + ((size_t)min(mt0 + i, mtiles - 1) * kblocks) * 64 + lane;
+    for (int i = 0; i < 4; i++) abase[i] = apk + ((size_t)min(mt0 + i, mtiles - 1) * kblocks + 4 * step0) * 64 + lane;
 
     f32x4 acc[4][WG_NT];
 #pragma unroll
@@ -224,6 +229,7 @@ __global__ __launch_bounds__(256) void gemm_q4m_bf16_kernel(WeightView w, const 
     step(s, F_{}, F_{});
     // D[token 4 kq + r][row n] per tile
     const uint32_t kq = lane >> 4;
+    if (gridDim.z > 1) yv = reinterpret_cast<float*>(yv) + (size_t)blockIdx.z * t * w.n_out;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
 #pragma unroll
@@ -241,20 +247,50 @@ __global__ __launch_bounds__(256) void gemm_q4m_bf16_kernel(WeightView w, const 
     }
 }
 
-hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, hipStream_t s) {
+// Adds the K slices in order: y = p[0] + p[1] + ... (f32 or bf16 out).
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restrict__ p, size_t n, uint32_t slices, void* __restrict__ yv) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = p[i];
+    for (uint32_t z = 1; z < slices; z++) v += p[(size_t)z * n + i];
+    if (OUT_BF16) reinterpret_cast<uint16_t*>(yv)[i] = f32_to_bf16_bits(v);
+    else reinterpret_cast<float*>(yv)[i] = v;
+}
+
+// K slices for a launch: enough workgroups to cover the CUs while each keeps at least 8 steps.
+uint32_t gemm_k_slices(const WeightView& w, size_t mtiles) {
+    const uint32_t wgs = ((row_tiles(w.n_out) + WG_NT - 1) / WG_NT) * (uint32_t)((mtiles + WG_MT - 1) / WG_MT);
+    const uint32_t steps = t4m_steps(w.n_in);
+    uint32_t z = 1;
+    while (z < 8 && wgs * z * 2 <= 256 && steps / (z * 2) >= 8) z *= 2;
+    return z;
+}
+
+// `partial`: scratch of slices * t * n_out floats when gemm_k_slices() > 1.
+hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
+                            hipStream_t s) {
     if (w.fmt != FMT_Q4M) return hipErrorInvalidValue;
-    dim3 grid((row_tiles(w.n_out) + WG_NT - 1) / WG_NT, (unsigned)((mtiles + WG_MT - 1) / WG_MT));
+    const uint32_t slices = gemm_k_slices(w, mtiles);
+    dim3 grid((row_tiles(w.n_out) + WG_NT - 1) / WG_NT, (unsigned)((mtiles + WG_MT - 1) / WG_MT), slices);
     const size_t lds = 2 * 4 * WG_NT * 64 * 16;  // 64 KiB
+    const bool direct_bf16 = out_bf16 && slices == 1;
+    void* dst = slices > 1 ? static_cast<void*>(partial) : y;
     hipError_t e;
-    if (out_bf16) {
+    if (direct_bf16) {
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4m_bf16_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        gemm_q4m_bf16_kernel<true><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, y);
+        gemm_q4m_bf16_kernel<true><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
     } else {
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4m_bf16_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        gemm_q4m_bf16_kernel<false><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, y);
+        gemm_q4m_bf16_kernel<false><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
     }
+    e = hipGetLastError();
+    if (e != hipSuccess || slices == 1) return e;
+    const size_t n = t * (size_t)w.n_out;
+    if (out_bf16) gemm_reduce_kernel<true><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
+    else gemm_reduce_kernel<false><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
     return hipGetLastError();
 }
 
