@@ -155,10 +155,13 @@ float oxhip_event_elapsed_ms(void* start, void* stop);
 /* Prefill: y [t, n_out] = x [t, n_in] W^T on the matrix cores (what matmul_quant_multi's GEMM paths compute,
  * src/kernels.rs:1774-1847). x_dtype / y_dtype: OXHIP_F32 or OXHIP_BF16. variant:
  *   OXHIP_GEMM_BF16  weights dequantized to bf16 (through LDS), bf16 MFMA, f32 accumulation (the x86 CPU's
- *                    f32 GEMM rounded to bf16 operands);
+ *                    f32 GEMM rounded to bf16 operands); MLX 4-bit weights;
+ *   OXHIP_GEMM_FP8   FP8 weights with 128 x 128 block scales: activations quantized on the device to e4m3 per token
+ *                    and 128 columns (scale amax / 448), fp8 MFMA, the two scales applied to each block's f32
+ *                    partial sum (the reference has no activation-FP8 path: parity is against its f32 product);
  * Packed activations live in scratch owned by ctx (grown on first use; calls on one ctx must not overlap). */
 enum { OXHIP_F32 = 0, OXHIP_BF16 = 1 };
-enum { OXHIP_GEMM_BF16 = 0 };
+enum { OXHIP_GEMM_BF16 = 0, OXHIP_GEMM_I8 = 1, OXHIP_GEMM_FP8 = 2 };
 int oxhip_dev_gemm(oxhip_ctx* ctx, const oxhip_weight* w, const void* x, int x_dtype, size_t t, void* y, int y_dtype, int variant,
                    void* stream);
 /* moe::route_top_k (src/moe.rs:180-193) for t rows of n_experts logits (n_experts <= 1024, k <= 32):

@@ -7,11 +7,12 @@ namespace oxhip {
 
 // Packs x and runs the bf16 GEMM; the packed activations live in ctx scratch.
 int gemm_bf16_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf16, size_t t, void* y, bool y_bf16, hipStream_t s) {
-    if (w->v.fmt != FMT_Q4M) {
-        set_error("gemm: the bf16 variant runs MLX 4-bit weights");
+    const bool fp8 = w->v.fmt == FMT_FP8 && w->v.br % 16 == 0 && w->v.bc % 128 == 0 && w->v.n_in % 128 == 0;
+    if (w->v.fmt != FMT_Q4M && !fp8) {
+        set_error("gemm: the bf16 variant runs MLX 4-bit weights and FP8 weights whose rows are multiples of 128");
         return 0;
     }
-    const size_t mtiles = (t + 15) / 16, kblocks = 4 * (size_t)t4m_steps(w->v.n_in);
+    const size_t mtiles = (t + 15) / 16, kblocks = 4 * (size_t)((w->v.n_in + 127) / 128);
     const size_t pack_bytes = align_up(mtiles * kblocks * 64 * 16, 256);
     const uint32_t slices = gemm_k_slices(w->v, mtiles);
     const size_t bytes = pack_bytes + (slices > 1 ? (size_t)slices * t * w->v.n_out * 4 : 0);
@@ -22,9 +23,34 @@ int gemm_bf16_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf1
             return 0;
         }
     }
-    HIP_TRY(launch_pack_a(x, x_bf16, true, t, w->v.n_in, mtiles, kblocks, c->gemm_ws.p, s), "gemm pack launch");
+    HIP_TRY(launch_pack_a(x, x_bf16, fp8 ? 2 : 1, t, w->v.n_in, mtiles, kblocks, c->gemm_ws.p, s), "gemm pack launch");
     float* partial = reinterpret_cast<float*>(static_cast<uint8_t*>(c->gemm_ws.p) + pack_bytes);
     HIP_TRY(launch_gemm_bf16(w->v, c->gemm_ws.p, t, mtiles, y, y_bf16, partial, s), "gemm launch");
+    return 1;
+}
+
+// FP8 block-scaled weights: activations quantized to e4m3 per 1 x 128 tile, fp8 MFMA.
+int gemm_fp8_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf16, size_t t, void* y, bool y_bf16, hipStream_t s) {
+    if (w->v.fmt != FMT_FP8 || w->v.br != 128 || w->v.bc != 128 || w->v.n_in % 128) {
+        set_error("gemm: the fp8 variant runs FP8 weights with 128 x 128 block scales and rows that are multiples of 128");
+        return 0;
+    }
+    const size_t mtiles = (t + 15) / 16, kblocks = w->v.n_in / 128;
+    const size_t pack_bytes = align_up(mtiles * kblocks * 64 * 32, 256), sx_bytes = align_up(kblocks * mtiles * 16 * 4, 256);
+    const uint32_t slices = gemm_fp8_k_slices(w->v, mtiles);
+    const size_t bytes = pack_bytes + sx_bytes + (slices > 1 ? (size_t)slices * t * w->v.n_out * 4 : 0);
+    if (c->gemm_ws.cap < bytes) {
+        (void)hipStreamSynchronize(s);
+        if (!c->gemm_ws.grow(bytes)) {
+            set_error("gemm: device memory short");
+            return 0;
+        }
+    }
+    uint8_t* base = static_cast<uint8_t*>(c->gemm_ws.p);
+    float* sx = reinterpret_cast<float*>(base + pack_bytes);
+    float* partial = reinterpret_cast<float*>(base + pack_bytes + sx_bytes);
+    HIP_TRY(launch_quantize_act_fp8(x, x_bf16, t, w->v.n_in, mtiles, kblocks, base, sx, s), "fp8 activation quantization launch");
+    HIP_TRY(launch_gemm_fp8(w->v, base, sx, t, mtiles, y, y_bf16, partial, s), "fp8 gemm launch");
     return 1;
 }
 
@@ -41,6 +67,7 @@ int oxhip_dev_gemm(oxhip_ctx* c, const oxhip_weight* w, const void* x, int x_dty
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (variant) {
         case OXHIP_GEMM_BF16: return gemm_bf16_run(c, w, x, x_dtype == OXHIP_BF16, t, y, y_dtype == OXHIP_BF16, s);
+        case OXHIP_GEMM_FP8: return gemm_fp8_run(c, w, x, x_dtype == OXHIP_BF16, t, y, y_dtype == OXHIP_BF16, s);
         default: set_error("gemm: unknown variant"); return 0;
     }
 }

@@ -27,7 +27,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // Activations [t][n_in] (f32 or bf16) -> fragments [mtile][block][lane][8 bf16]; lane = 16 kq + m holds token
 // 16 mtile + m at K positions 32 b + 4 kq + {0..3} then 32 b + 16 + 4 kq + {0..3} (SPLIT, the order of the
 // nibble pairs of Q4 bytes) or 32 b + 8 kq + {0..7}. Tokens past t and columns past n_in are zero.
-template <bool SPLIT, bool SRC_BF16>
+// MODE 2 (FP8 weights read 32 row bytes per lane): block kb = 4 s + b of step s holds columns 128 s + 32 kq + 8 b + j.
+template <int MODE, bool SRC_BF16>
 __global__ __launch_bounds__(256) void pack_a_kernel(const void* __restrict__ x, uint32_t t, uint32_t n_in, uint32_t mtiles,
                                                      uint32_t kblocks, uint4* __restrict__ out) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -39,7 +40,9 @@ __global__ __launch_bounds__(256) void pack_a_kernel(const void* __restrict__ x,
     if (tok < t) {
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const uint32_t k = SPLIT ? 32 * b + (j < 4 ? 4 * kq + j : 16 + 4 * kq + (j - 4)) : 32 * b + 8 * kq + j;
+            const uint32_t k = MODE == 1   ? 32 * b + (j < 4 ? 4 * kq + j : 16 + 4 * kq + (j - 4))
+                               : MODE == 2 ? 128 * (b >> 2) + 32 * kq + 8 * (b & 3) + j
+                                           : 32 * b + 8 * kq + j;
             uint16_t h = 0;
             if (k < n_in) {
                 if (SRC_BF16) h = reinterpret_cast<const uint16_t*>(x)[(size_t)tok * n_in + k];
@@ -51,18 +54,22 @@ __global__ __launch_bounds__(256) void pack_a_kernel(const void* __restrict__ x,
     out[idx] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
 }
 
-hipError_t launch_pack_a(const void* x, bool src_bf16, bool split, size_t t, size_t n_in, size_t mtiles, size_t kblocks, void* out,
+hipError_t launch_pack_a(const void* x, bool src_bf16, int mode, size_t t, size_t n_in, size_t mtiles, size_t kblocks, void* out,
                          hipStream_t s) {
     size_t total = mtiles * kblocks * 64;
     if (!total) return hipSuccess;
     unsigned grid = (unsigned)((total + 255) / 256);
     uint4* o = static_cast<uint4*>(out);
-    if (split) {
-        if (src_bf16) pack_a_kernel<true, true><<<grid, 256, 0, s>>>(x, (uint32_t)t, (uint32_t)n_in, (uint32_t)mtiles, (uint32_t)kblocks, o);
-        else pack_a_kernel<true, false><<<grid, 256, 0, s>>>(x, (uint32_t)t, (uint32_t)n_in, (uint32_t)mtiles, (uint32_t)kblocks, o);
+    const uint32_t tt = (uint32_t)t, kk = (uint32_t)n_in, mt = (uint32_t)mtiles, kb = (uint32_t)kblocks;
+    if (mode == 1) {
+        if (src_bf16) pack_a_kernel<1, true><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
+        else pack_a_kernel<1, false><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
+    } else if (mode == 2) {
+        if (src_bf16) pack_a_kernel<2, true><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
+        else pack_a_kernel<2, false><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
     } else {
-        if (src_bf16) pack_a_kernel<false, true><<<grid, 256, 0, s>>>(x, (uint32_t)t, (uint32_t)n_in, (uint32_t)mtiles, (uint32_t)kblocks, o);
-        else pack_a_kernel<false, false><<<grid, 256, 0, s>>>(x, (uint32_t)t, (uint32_t)n_in, (uint32_t)mtiles, (uint32_t)kblocks, o);
+        if (src_bf16) pack_a_kernel<0, true><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
+        else pack_a_kernel<0, false><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
     }
     return hipGetLastError();
 }
@@ -101,13 +108,16 @@ __device__ __forceinline__ uint4 dequant_q4m(uint32_t w, float d, float c) {
 // kblocks = 4 * steps. OUT_BF16: y is bf16 [t][n_out], else f32.
 // With gridDim.z > 1 the K-steps are split over z and each slice writes its partial sums as f32 to
 // yv + z * t * n_out (a second kernel adds the slices in order).
-template <bool OUT_BF16>
-__global__ __launch_bounds__(256) void gemm_q4m_bf16_kernel(WeightView w, const uint4* __restrict__ apk, uint32_t t, uint32_t mtiles,
-                                                            void* __restrict__ yv) {
+// FMT: FMT_Q4M (tile-packed MLX 4-bit) or FMT_FP8 (row-major e4m3 bytes with 128 x 128 block scales: the bytes are
+// exact in bf16, the block scale multiplies in f32 before the rounding, and a lane takes 32 consecutive row bytes
+// per step, which pack_a's mode 2 mirrors on the activation side).
+template <int FMT, bool OUT_BF16>
+__global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint4* __restrict__ apk, uint32_t t, uint32_t mtiles,
+                                                        void* __restrict__ yv) {
     extern __shared__ uint4 bfrag[];  // [2][4 blocks][8 row tiles][64 lanes]
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t n = lane & 15;
-    const uint32_t all_steps = t4m_steps(w.n_in), kblocks = 4 * all_steps;
+    const uint32_t all_steps = (w.n_in + 127) / 128, kblocks = 4 * all_steps;  // == t4m_steps(n_in)
     const uint32_t per_z = (all_steps + gridDim.z - 1) / gridDim.z;
     const uint32_t step0 = blockIdx.z * per_z;              // this slice's K-steps: step0 .. step0 + nsteps
     const uint32_t nsteps = min(all_steps, step0 + per_z) - step0;
@@ -117,8 +127,18 @@ __global__ __launch_bounds__(256) void gemm_q4m_bf16_kernel(WeightView w, const 
 
     // the two row tiles this wave dequantizes
     const uint8_t* wbase[2];
+    const float* sbase[2] = {nullptr, nullptr};  // FP8: the block scales of the tile's rows
 #pragma unroll
-    for (int i = 0; i < 2; i++) wbase[i] = w.p0 + ((size_t)min(nt0 + 2 * wave + i, ntiles - 1) * all_steps + step0) * T4M_REC;
+    for (int i = 0; i < 2; i++) {
+        const uint32_t tile = min(nt0 + 2 * wave + i, ntiles - 1);
+        if (FMT == FMT_Q4M) {
+            wbase[i] = w.p0 + ((size_t)tile * all_steps + step0) * T4M_REC;
+        } else {
+            const uint32_t row = min(tile * 16 + n, w.n_out - 1);
+            wbase[i] = w.p0 + (size_t)row * w.n_in + 128 * (size_t)step0 + 32 * (lane >> 4);
+            sbase[i] = reinterpret_cast<const float*>(w.p1) + (size_t)(tile * 16 / w.br) * ((w.n_in + w.bc - 1) / w.bc) + step0;
+        }
+    }
     // A fragments of the wave's 4 token tiles (tiles past the end repeat the last one; their rows are not stored)
     const uint4* abase[4];
 #pragma unroll
@@ -131,26 +151,48 @@ __global__ __launch_bounds__(256) void gemm_q4m_bf16_kernel(WeightView w, const 
         for (int j = 0; j < WG_NT; j++) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
     struct Raw {
-        uint4 c;
-        uint32_t dd, oo;
+        uint4 c, c2;      // Q4M: one chunk; FP8: 32 row bytes
+        uint32_t dd, oo;  // Q4M: scales, offsets; FP8: dd = the block scale's bits
     };
     auto load_raw = [&](Raw* r, uint32_t s) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            const uint8_t* rec = wbase[i] + (size_t)s * T4M_REC;
-            r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
-            r[i].dd = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
-            r[i].oo = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
+            if (FMT == FMT_Q4M) {
+                const uint8_t* rec = wbase[i] + (size_t)s * T4M_REC;
+                r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+                r[i].dd = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
+                r[i].oo = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
+            } else {
+                const uint8_t* p = wbase[i] + 128 * (size_t)s;
+                r[i].c = *reinterpret_cast<const uint4*>(p);
+                r[i].c2 = *reinterpret_cast<const uint4*>(p + 16);
+                r[i].dd = __float_as_uint(sbase[i][(128 * s) / w.bc]);
+            }
         }
     };
     auto dequant_tile = [&](const Raw& r, int i, uint32_t buf) {  // one of the wave's two row tiles, 4 blocks
-        const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
+        if (FMT == FMT_Q4M) {
+            const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            const int g = b >> 1;
-            const float d = f16_bits_to_f32((uint16_t)(g ? r.dd >> 16 : r.dd & 0xFFFF));
-            const float off = bf16_bits_to_f32((uint16_t)(g ? r.oo >> 16 : r.oo & 0xFFFF));
-            bfrag[((buf * 4 + b) * WG_NT + 2 * wave + i) * 64 + lane] = dequant_q4m(cw[b], d, off - 8.0f * d);
+            for (int b = 0; b < 4; b++) {
+                const int g = b >> 1;
+                const float d = f16_bits_to_f32((uint16_t)(g ? r.dd >> 16 : r.dd & 0xFFFF));
+                const float off = bf16_bits_to_f32((uint16_t)(g ? r.oo >> 16 : r.oo & 0xFFFF));
+                bfrag[((buf * 4 + b) * WG_NT + 2 * wave + i) * 64 + lane] = dequant_q4m(cw[b], d, off - 8.0f * d);
+            }
+        } else {
+            const uint32_t cw[8] = {r.c.x, r.c.y, r.c.z, r.c.w, r.c2.x, r.c2.y, r.c2.z, r.c2.w};
+            const float sc = __uint_as_float(r.dd);
+#pragma unroll
+            for (int b = 0; b < 4; b++) {  // bytes 8 b .. 8 b + 7 of the lane's 32
+                const f32x2 v0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)cw[2 * b], false);
+                const f32x2 v1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)cw[2 * b], true);
+                const f32x2 v2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)cw[2 * b + 1], false);
+                const f32x2 v3 = __builtin_amdgcn_cvt_pk_f32_fp8((int)cw[2 * b + 1], true);
+                const uint32_t o[4] = {pack_bf16(v0.x * sc, v0.y * sc), pack_bf16(v1.x * sc, v1.y * sc),
+                                       pack_bf16(v2.x * sc, v2.y * sc), pack_bf16(v3.x * sc, v3.y * sc)};
+                bfrag[((buf * 4 + b) * WG_NT + 2 * wave + i) * 64 + lane] = make_uint4(o[0], o[1], o[2], o[3]);
+            }
         }
     };
     auto read_b = [&](uint4* dst, uint32_t buf, uint32_t b) {
@@ -261,16 +303,16 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restric
 // K slices for a launch: enough workgroups to cover the CUs while each keeps at least 8 steps.
 uint32_t gemm_k_slices(const WeightView& w, size_t mtiles) {
     const uint32_t wgs = ((row_tiles(w.n_out) + WG_NT - 1) / WG_NT) * (uint32_t)((mtiles + WG_MT - 1) / WG_MT);
-    const uint32_t steps = t4m_steps(w.n_in);
+    const uint32_t steps = (w.n_in + 127) / 128;
     uint32_t z = 1;
     while (z < 8 && wgs * z * 2 <= 256 && steps / (z * 2) >= 8) z *= 2;
     return z;
 }
 
-// `partial`: scratch of slices * t * n_out floats when gemm_k_slices() > 1.
-hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
-                            hipStream_t s) {
-    if (w.fmt != FMT_Q4M) return hipErrorInvalidValue;
+namespace {
+template <int FMT>
+hipError_t run_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
+                         hipStream_t s) {
     const uint32_t slices = gemm_k_slices(w, mtiles);
     dim3 grid((row_tiles(w.n_out) + WG_NT - 1) / WG_NT, (unsigned)((mtiles + WG_MT - 1) / WG_MT), slices);
     const size_t lds = 2 * 4 * WG_NT * 64 * 16;  // 64 KiB
@@ -278,13 +320,13 @@ hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size
     void* dst = slices > 1 ? static_cast<void*>(partial) : y;
     hipError_t e;
     if (direct_bf16) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4m_bf16_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        gemm_q4m_bf16_kernel<true><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
+        gemm_bf16_kernel<FMT, true><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
     } else {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4m_bf16_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        gemm_q4m_bf16_kernel<false><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
+        gemm_bf16_kernel<FMT, false><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
     }
     e = hipGetLastError();
     if (e != hipSuccess || slices == 1) return e;
@@ -292,6 +334,16 @@ hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size
     if (out_bf16) gemm_reduce_kernel<true><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
     else gemm_reduce_kernel<false><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
     return hipGetLastError();
+}
+}  // namespace
+
+// `partial`: scratch of slices * t * n_out floats when gemm_k_slices() > 1.
+hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
+                            hipStream_t s) {
+    if (w.fmt == FMT_Q4M) return run_gemm_bf16<FMT_Q4M>(w, apk, t, mtiles, y, out_bf16, partial, s);
+    if (w.fmt == FMT_FP8 && w.br % 16 == 0 && w.bc % 128 == 0 && w.n_in % 128 == 0)
+        return run_gemm_bf16<FMT_FP8>(w, apk, t, mtiles, y, out_bf16, partial, s);
+    return hipErrorInvalidValue;
 }
 
 }  // namespace oxhip

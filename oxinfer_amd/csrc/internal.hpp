@@ -73,11 +73,16 @@ hipError_t launch_repack_mlx_q4(const uint32_t* w, const uint16_t* scales, const
 hipError_t launch_q4_scale_groups(const uint16_t* sc32, size_t n_out, size_t n_in, size_t sgroup, uint16_t* dst,
                                   int* mismatch, hipStream_t s);
 
-hipError_t launch_pack_a(const void* x, bool src_bf16, bool split, size_t t, size_t n_in, size_t mtiles, size_t kblocks, void* out,
+hipError_t launch_pack_a(const void* x, bool src_bf16, int mode, size_t t, size_t n_in, size_t mtiles, size_t kblocks, void* out,
                          hipStream_t s);
 uint32_t gemm_k_slices(const WeightView& w, size_t mtiles);
 hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                             hipStream_t s);
+hipError_t launch_quantize_act_fp8(const void* x, bool src_bf16, size_t t, size_t n_in, size_t mtiles, size_t kblocks, void* out,
+                                   float* sx, hipStream_t s);
+uint32_t gemm_fp8_k_slices(const WeightView& w, size_t mtiles);
+hipError_t launch_gemm_fp8(const WeightView& w, const void* apk, const float* sx, size_t t, size_t mtiles, void* y, bool out_bf16,
+                           float* partial, hipStream_t s);
 hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, hipStream_t s);
 hipError_t launch_moe_plan(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, int* row_of, int* src, int4* chunks,
                            int* nchunks, hipStream_t s);
