@@ -30,6 +30,10 @@ Q8_0, Q4_K, Q6_K = 8, 12, 14
 ROW_BYTES = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
 FMT_NAME = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
 KERNEL_FMT = {Q8_0: 1, Q4_K: 2, Q6_K: 3}  # template argument in the kernel symbol
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
+# benchmark (KiB per dispatch, FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000: what a 256 MiB device copy
+# reads on the same counters); profiles/decode_mfma_gguf_gemv.md holds the summary.
+TRAFFIC_BYTES = {"decode_mfma_kernel<1, 8, false>": 63415984}
 
 
 def weight_bytes(kind, n_out, n_in):
@@ -101,7 +105,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gguf_gemv", choices=["gguf_gemv", "gguf_gemv_q6k"])
+    ap.add_argument("--workload", default="gguf_gemv", choices=["gguf_gemv", "gguf_gemv_q6k", "copy"],
+                    help="copy = a plain 256 MiB device copy, the known-size kernel that scales the HBM traffic counters")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pool-gb", type=float, default=POOL_BYTES / 1e9)
     args = ap.parse_args()
@@ -115,6 +120,15 @@ def main():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if args.workload == "copy":
+        n = 256 << 20
+        src = torch.full((n,), 3, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup + args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"workload": "copy", "bytes_read": n, "bytes_written": n, "launches": args.warmup + args.steps}))
+        return
     be = HipBackend(0)
     gens = {Q8_0: synth.gguf_q8_0, Q4_K: synth.gguf_q4_k, Q6_K: synth.gguf_q6_k}
     kinds = [Q8_0, Q4_K] if args.workload == "gguf_gemv" else [Q6_K]
@@ -206,7 +220,7 @@ def main():
                    "launches_per_step": len(cases), "bytes_per_step": step_bytes,
                    "weight_pool_GB_per_shape": args.pool_gb, "activations": "int8 per 32 (quantize_act), resident in HBM"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom_symbol,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES.get(dom_symbol), "kernel": dom_symbol,
                      "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_avg_s * 1e6, 2)},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "detail": detail,
