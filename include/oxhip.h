@@ -156,6 +156,11 @@ float oxhip_event_elapsed_ms(void* start, void* stop);
  * src/kernels.rs:1774-1847). x_dtype / y_dtype: OXHIP_F32 or OXHIP_BF16. variant:
  *   OXHIP_GEMM_BF16  weights dequantized to bf16 (through LDS), bf16 MFMA, f32 accumulation (the x86 CPU's
  *                    f32 GEMM rounded to bf16 operands); MLX 4-bit weights;
+ *                    also FP8 weights whose rows are multiples of 128 (e4m3 x block scale rounded to bf16);
+ *   OXHIP_GEMM_I8    MLX 4-bit weights on the int8 matrix cores: activations quantized per token and block of 32
+ *                    as quantize_act does, exact int32 block sums, f32 rescale by the block and activation scales,
+ *                    offsets times the exact activation sums (the reference's int8 GEMM, one activation plane,
+ *                    src/kernels_i8gemm.rs:160-315);
  *   OXHIP_GEMM_FP8   FP8 weights with 128 x 128 block scales: activations quantized on the device to e4m3 per token
  *                    and 128 columns (scale amax / 448), fp8 MFMA, the two scales applied to each block's f32
  *                    partial sum (the reference has no activation-FP8 path: parity is against its f32 product);
@@ -164,6 +169,9 @@ enum { OXHIP_F32 = 0, OXHIP_BF16 = 1 };
 enum { OXHIP_GEMM_BF16 = 0, OXHIP_GEMM_I8 = 1, OXHIP_GEMM_FP8 = 2 };
 int oxhip_dev_gemm(oxhip_ctx* ctx, const oxhip_weight* w, const void* x, int x_dtype, size_t t, void* y, int y_dtype, int variant,
                    void* stream);
+/* The exact int32 block sums of the OXHIP_GEMM_I8 variant, [t, n_out, n_in/32], written by the GEMM kernel itself
+ * (kernels_i8gemm's `block` accumulators, src/kernels_i8gemm.rs:249-334). For parity checks. */
+int oxhip_dev_gemm_isums(oxhip_ctx* ctx, const oxhip_weight* w, const void* x, int x_dtype, size_t t, int32_t* out, void* stream);
 /* moe::route_top_k (src/moe.rs:180-193) for t rows of n_experts logits (n_experts <= 1024, k <= 32):
  * idx / w [t, k], sorted by descending logit, ties to the lower index, w = softmax over the k. */
 int oxhip_dev_route_top_k(oxhip_ctx* ctx, const float* logits, size_t t, size_t n_experts, size_t k, uint32_t* idx, float* w,

@@ -54,9 +54,48 @@ int gemm_fp8_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf16
     return 1;
 }
 
+// MLX 4-bit weights on the int8 matrix cores: activations quantized per token and block of 32, exact int32 block
+// sums, f32 rescale (the reference's int8 GEMM, src/kernels_i8gemm.rs:160-315). `dump` (optional) receives the sums.
+int gemm_i8_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf16, size_t t, void* y, bool y_bf16, int32_t* dump,
+                hipStream_t s) {
+    if (w->v.fmt != FMT_Q4M) {
+        set_error("gemm: the int8 variant runs MLX 4-bit weights (group 64)");
+        return 0;
+    }
+    size_t slots, ngrp;
+    gemm_i8_geometry(w->v, t, &slots, &ngrp);
+    const size_t frag_bytes = align_up(slots / 16 * ngrp * 64 * 16, 256), xs_bytes = align_up(slots * ngrp * 8, 256),
+                 fs_bytes = align_up(slots * ngrp * 4, 256);
+    const uint32_t slices = gemm_i8_k_slices(w->v, t);
+    const bool direct = slices == 1 && !y_bf16 && y;
+    const size_t bytes = frag_bytes + xs_bytes + fs_bytes + (direct ? 0 : (size_t)slices * t * w->v.n_out * 4);
+    if (c->gemm_ws.cap < bytes) {
+        (void)hipStreamSynchronize(s);
+        if (!c->gemm_ws.grow(bytes)) {
+            set_error("gemm: device memory short");
+            return 0;
+        }
+    }
+    uint8_t* base = static_cast<uint8_t*>(c->gemm_ws.p);
+    void *frag = base, *xs = base + frag_bytes, *fs = base + frag_bytes + xs_bytes;
+    float* partial = reinterpret_cast<float*>(base + frag_bytes + xs_bytes + fs_bytes);
+    HIP_TRY(launch_quantize_pack_i8(x, x_bf16, t, w->v, frag, xs, fs, s), "int8 activation quantization launch");
+    HIP_TRY(launch_gemm_i8(w->v, frag, xs, fs, t, direct ? static_cast<float*>(y) : partial, dump, s), "int8 gemm launch");
+    if (!direct && y) HIP_TRY(launch_gemm_reduce(partial, t * (size_t)w->v.n_out, slices, y, y_bf16, s), "gemm reduce launch");
+    return 1;
+}
+
 }  // namespace oxhip
 
 extern "C" {
+
+int oxhip_dev_gemm_isums(oxhip_ctx* c, const oxhip_weight* w, const void* x, int x_dtype, size_t t, int32_t* out, void* stream) {
+    if (!c || !w || !x || !out || !t || x_dtype < 0 || x_dtype > 1) {
+        set_error("gemm_isums: bad arguments");
+        return 0;
+    }
+    return gemm_i8_run(c, w, x, x_dtype == OXHIP_BF16, t, nullptr, false, out, static_cast<hipStream_t>(stream));
+}
 
 int oxhip_dev_gemm(oxhip_ctx* c, const oxhip_weight* w, const void* x, int x_dtype, size_t t, void* y, int y_dtype, int variant,
                    void* stream) {
@@ -67,6 +106,7 @@ int oxhip_dev_gemm(oxhip_ctx* c, const oxhip_weight* w, const void* x, int x_dty
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (variant) {
         case OXHIP_GEMM_BF16: return gemm_bf16_run(c, w, x, x_dtype == OXHIP_BF16, t, y, y_dtype == OXHIP_BF16, s);
+        case OXHIP_GEMM_I8: return gemm_i8_run(c, w, x, x_dtype == OXHIP_BF16, t, y, y_dtype == OXHIP_BF16, nullptr, s);
         case OXHIP_GEMM_FP8: return gemm_fp8_run(c, w, x, x_dtype == OXHIP_BF16, t, y, y_dtype == OXHIP_BF16, s);
         default: set_error("gemm: unknown variant"); return 0;
     }

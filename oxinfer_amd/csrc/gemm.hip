@@ -337,6 +337,13 @@ hipError_t run_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t 
 }
 }  // namespace
 
+hipError_t launch_gemm_reduce(const float* partial, size_t n, uint32_t slices, void* y, bool out_bf16, hipStream_t s) {
+    if (!n) return hipSuccess;
+    if (out_bf16) gemm_reduce_kernel<true><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
+    else gemm_reduce_kernel<false><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
+    return hipGetLastError();
+}
+
 // `partial`: scratch of slices * t * n_out floats when gemm_k_slices() > 1.
 hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                             hipStream_t s) {

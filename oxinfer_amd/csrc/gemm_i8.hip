@@ -1,0 +1,300 @@
+// Prefill GEMM on the int8 matrix cores over tile-packed MLX 4-bit weights: the semantics of the reference's int8
+// GEMM (src/kernels_i8gemm.rs:160-315, one activation plane). Activations are quantized per token and block of 32
+// exactly as quantize_act does (src/quant.rs:267-292: q = round_half_away(x * 127 / amax), scale = amax / 127,
+// f = sum of x); per weight row, token and block the int32 sum I = sum (nib - 8) * q is exact, and
+//     y[t][r] = sum_b I_b * (d_b * xs_b) + sum_g off_g * F_g          (F_g = f of the group's two blocks)
+// in f32. One v_mfma_i32_16x16x32_i8 yields a block's sums for 16 rows x 16 tokens; the weights are the A operand,
+// so a lane's four results are rows 4 kq + i of the tile for token n: its row scales come from one 16-byte load of
+// the record and its token's activation scales are its own.
+#include "internal.hpp"
+#include "layout.hpp"
+
+namespace oxhip {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+// Four nibbles (one per byte, 0..15) -> four int8 codes nib - 8: flip bit 3, then extend it into bits 4..7.
+__device__ __forceinline__ uint32_t center4(uint32_t nib) {
+    const uint32_t s = nib ^ 0x08080808u;
+    return s | ((s & 0x08080808u) * 0x1Eu);
+}
+
+__device__ __forceinline__ long pack64(uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); }
+
+// One thread per (token slot, group of 64 columns). Writes, for token tile tt = slot / 16 and group g:
+//   frag[(tt * ngrp + g) * 64 + 16 kq + slot % 16] = {blk0 cols 4kq.., blk0 cols 16+4kq.., blk1 cols 4kq.., blk1 cols 16+4kq..}
+//   xs[(tt * ngrp + g) * 16 + slot % 16] = the two block scales;  fs[...] = f_0 + f_1
+// Slots past t and groups past n_in / 64 hold zeros.
+template <bool SRC_BF16>
+__global__ __launch_bounds__(256) void quantize_pack_i8_kernel(const void* __restrict__ xv, uint32_t t, uint32_t n_in, uint32_t slots,
+                                                               uint32_t ngrp, uint4* __restrict__ frag, float2* __restrict__ xs,
+                                                               float* __restrict__ fs) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)slots * ngrp) return;
+    const uint32_t g = (uint32_t)(idx % ngrp), slot = (uint32_t)(idx / ngrp);
+    const uint32_t tt = slot >> 4, n = slot & 15;
+    uint32_t word[2][8];
+    float scale[2] = {0.0f, 0.0f}, fsum[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) word[h][i] = 0;
+    if (slot < t && g < n_in / 64) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            float v[32];
+            const size_t at = (size_t)slot * n_in + 64 * (size_t)g + 32 * h;
+            if (SRC_BF16) {
+                const uint4* src = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(xv) + at);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint4 u = src[i];
+                    const uint32_t d[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        v[8 * i + 2 * k] = __uint_as_float(d[k] << 16);
+                        v[8 * i + 2 * k + 1] = __uint_as_float(d[k] & 0xFFFF0000u);
+                    }
+                }
+            } else {
+                const float4* src = reinterpret_cast<const float4*>(static_cast<const float*>(xv) + at);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float4 f = src[i];
+                    v[4 * i] = f.x; v[4 * i + 1] = f.y; v[4 * i + 2] = f.z; v[4 * i + 3] = f.w;
+                }
+            }
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 32; i++) amax = fmaxf(amax, fabsf(v[i]));
+            const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+            float f = -0.0f;
+#pragma unroll
+            for (int i = 0; i < 32; i++) f += v[i];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                uint32_t wv = 0;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const float r = roundf(v[4 * i + k] * inv);
+                    const int iv = r != r ? 0 : (int)fminf(fmaxf(r, -128.0f), 127.0f);
+                    wv |= ((uint32_t)iv & 0xFF) << (8 * k);
+                }
+                word[h][i] = wv;
+            }
+            scale[h] = amax / 127.0f;
+            fsum[h] = f;
+        }
+    }
+    const size_t base = (size_t)tt * ngrp + g;
+#pragma unroll
+    for (int kq = 0; kq < 4; kq++) frag[base * 64 + 16 * kq + n] = make_uint4(word[0][kq], word[0][4 + kq], word[1][kq], word[1][4 + kq]);
+    xs[base * 16 + n] = make_float2(scale[0], scale[1]);
+    fs[base * 16 + n] = fsum[0] + fsum[1];
+}
+
+// Workgroup: 4 waves, each two row tiles (32 rows) x TT token tiles (16 TT tokens) over one K slice; no LDS and no
+// barrier: every operand a lane needs is its own (weights, row scales) or its token's (activation fragments, scales).
+// DUMP also stores the exact block sums to dump[(token * n_out + row) * (n_in / 32) + block].
+template <int TT, bool DUMP>
+__global__ __launch_bounds__(256) void gemm_i8_q4m_kernel(WeightView w, const uint4* __restrict__ afrag, const float2* __restrict__ axs,
+                                                          const float* __restrict__ afs, uint32_t t, uint32_t ngrp,
+                                                          float* __restrict__ y, int32_t* __restrict__ dump) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t n = lane & 15, kq = lane >> 4;
+    const uint32_t ntiles = row_tiles(w.n_out), all_steps = t4m_steps(w.n_in), nblk = w.n_in / 32;
+    const uint32_t rt0 = blockIdx.x * 8 + 2 * wave;
+    if (rt0 >= ntiles) return;
+    const uint32_t tt0 = blockIdx.y * TT;
+    const uint32_t per = (all_steps + gridDim.z - 1) / gridDim.z;
+    const uint32_t s0 = blockIdx.z * per, s1 = min(all_steps, s0 + per);
+    y += (size_t)blockIdx.z * t * w.n_out;
+
+    const uint8_t* wbase[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) wbase[i] = w.p0 + (size_t)min(rt0 + i, ntiles - 1) * all_steps * T4M_REC;
+    float acc[2][TT][4];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[i][tt][e] = 0.0f;
+
+    constexpr int TH = TT / 2;  // token tiles per phase: a group of 64 columns is worked in two halves
+    struct Rec {
+        uint4 c, dd, oo;
+    };
+    struct Act {
+        uint4 f[TH];
+        float2 xs[TH];
+        float fs[TH];
+    };
+    auto load_rec = [&](Rec* r, uint32_t s) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint8_t* rec = wbase[i] + (size_t)s * T4M_REC;
+            r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+            r[i].dd = *reinterpret_cast<const uint4*>(rec + 1024 + 16 * kq);
+            r[i].oo = *reinterpret_cast<const uint4*>(rec + 1088 + 16 * kq);
+        }
+    };
+    // phase p = 2 * group + half
+    const uint4* fb = afrag + (size_t)tt0 * ngrp * 64 + lane;
+    const float2* xb = axs + (size_t)tt0 * ngrp * 16 + n;
+    const float* sb = afs + (size_t)tt0 * ngrp * 16 + n;
+    auto load_act = [&](Act& a, uint32_t p) {
+        const uint32_t grp = p >> 1, h = p & 1;
+#pragma unroll
+        for (int tt = 0; tt < TH; tt++) {
+            const size_t at = (size_t)(h * TH + tt) * ngrp + grp;
+            a.f[tt] = fb[at * 64];
+            a.xs[tt] = xb[at * 16];
+            a.fs[tt] = sb[at * 16];
+        }
+    };
+    auto compute = [&](const Rec* r, const Act& a, uint32_t grp, int g, int h) {
+        long wa[2][2];
+        float ds[2][4], off[2][4];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint32_t w0 = g ? r[i].c.z : r[i].c.x, w1 = g ? r[i].c.w : r[i].c.y;
+            wa[i][0] = pack64(center4(w0 & 0x0F0F0F0Fu), center4((w0 >> 4) & 0x0F0F0F0Fu));
+            wa[i][1] = pack64(center4(w1 & 0x0F0F0F0Fu), center4((w1 >> 4) & 0x0F0F0F0Fu));
+            const uint32_t dd[4] = {r[i].dd.x, r[i].dd.y, r[i].dd.z, r[i].dd.w};
+            const uint32_t oo[4] = {r[i].oo.x, r[i].oo.y, r[i].oo.z, r[i].oo.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                ds[i][e] = f16_bits_to_f32((uint16_t)(g ? dd[e] >> 16 : dd[e] & 0xFFFF));
+                off[i][e] = bf16_bits_to_f32((uint16_t)(g ? oo[e] >> 16 : oo[e] & 0xFFFF));
+            }
+        }
+#pragma unroll
+        for (int tt = 0; tt < TH; tt++) {
+            const long b0 = pack64(a.f[tt].x, a.f[tt].y), b1 = pack64(a.f[tt].z, a.f[tt].w);
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const v4i z = {0, 0, 0, 0};
+                const v4i d0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wa[i][0], b0, z, 0, 0, 0);
+                const v4i d1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wa[i][1], b1, z, 0, 0, 0);
+                float* ac = acc[i][h * TH + tt];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float u = (float)d0[e] * a.xs[tt].x;
+                    u = fmaf((float)d1[e], a.xs[tt].y, u);
+                    ac[e] = fmaf(u, ds[i][e], ac[e]);
+                    ac[e] = fmaf(off[i][e], a.fs[tt], ac[e]);
+                }
+                if (DUMP) {
+                    const uint32_t tok = 16 * (tt0 + h * TH + tt) + n;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const uint32_t row = 16 * (rt0 + i) + 4 * kq + e;
+                        if (tok < t && row < w.n_out) {
+                            if (2 * grp < nblk) dump[((size_t)tok * w.n_out + row) * nblk + 2 * grp] = d0[e];
+                            if (2 * grp + 1 < nblk) dump[((size_t)tok * w.n_out + row) * nblk + 2 * grp + 1] = d1[e];
+                        }
+                    }
+                }
+            }
+        }
+    };
+
+    if (s0 < s1) {
+        // Each phase's activation operands are requested one phase ahead, the next step's record a step ahead;
+        // past the end the requests repeat the last valid address and are dropped.
+        const uint32_t plast = 4 * s1 - 1;
+        Rec rec[2], rnext[2];
+        Act cur, nxt;
+        load_rec(rec, s0);
+        load_act(cur, 4 * s0);
+        for (uint32_t s = s0; s < s1; s++) {
+            load_rec(rnext, min(s + 1, s1 - 1));
+#pragma unroll
+            for (int ph = 0; ph < 4; ph++) {
+                load_act(nxt, min(4 * s + ph + 1, plast));
+                compute(rec, cur, 2 * s + (ph >> 1), ph >> 1, ph & 1);
+                cur = nxt;
+            }
+            rec[0] = rnext[0];
+            rec[1] = rnext[1];
+        }
+    }
+
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        if (rt0 + i >= ntiles) continue;
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++) {
+            const uint32_t tok = 16 * (tt0 + tt) + n;
+            if (tok >= t) continue;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const uint32_t row = 16 * (rt0 + i) + 4 * kq + e;
+                if (row < w.n_out) y[(size_t)tok * w.n_out + row] = acc[i][tt][e];
+            }
+        }
+    }
+}
+
+constexpr uint32_t tt_for(size_t t) { return t <= 64 ? 4u : 8u; }
+
+}  // namespace
+
+// Token slots (a multiple of the kernel's token tile count x 16) and column groups the packed activations hold.
+void gemm_i8_geometry(const WeightView& w, size_t t, size_t* slots, size_t* ngrp) {
+    const size_t tt = tt_for(t), ttiles = ((t + 15) / 16 + tt - 1) / tt * tt;
+    *slots = ttiles * 16;
+    *ngrp = 2 * (size_t)t4m_steps(w.n_in);
+}
+
+uint32_t gemm_i8_k_slices(const WeightView& w, size_t t) {
+    size_t slots, ngrp;
+    gemm_i8_geometry(w, t, &slots, &ngrp);
+    const size_t waves = (size_t)((row_tiles(w.n_out) + 7) / 8) * 4 * (slots / 16 / tt_for(t));
+    const uint32_t steps = t4m_steps(w.n_in);
+    uint32_t z = 1;
+    while (z < 8 && waves * z < 2048 && steps / (z * 2) >= 4) z *= 2;
+    return z;
+}
+
+hipError_t launch_quantize_pack_i8(const void* x, bool src_bf16, size_t t, const WeightView& w, void* frag, void* xs, void* fs,
+                                   hipStream_t s) {
+    size_t slots, ngrp;
+    gemm_i8_geometry(w, t, &slots, &ngrp);
+    const size_t total = slots * ngrp;
+    const unsigned grid = (unsigned)((total + 255) / 256);
+    if (src_bf16)
+        quantize_pack_i8_kernel<true><<<grid, 256, 0, s>>>(x, (uint32_t)t, w.n_in, (uint32_t)slots, (uint32_t)ngrp, static_cast<uint4*>(frag),
+                                                           static_cast<float2*>(xs), static_cast<float*>(fs));
+    else
+        quantize_pack_i8_kernel<false><<<grid, 256, 0, s>>>(x, (uint32_t)t, w.n_in, (uint32_t)slots, (uint32_t)ngrp, static_cast<uint4*>(frag),
+                                                            static_cast<float2*>(xs), static_cast<float*>(fs));
+    return hipGetLastError();
+}
+
+// `y` receives gemm_i8_k_slices() partial results of t * n_out floats each (one when there is one slice);
+// `dump` (optional) the exact block sums.
+hipError_t launch_gemm_i8(const WeightView& w, const void* frag, const void* xs, const void* fs, size_t t, float* y, int32_t* dump,
+                          hipStream_t s) {
+    if (w.fmt != FMT_Q4M) return hipErrorInvalidValue;
+    size_t slots, ngrp;
+    gemm_i8_geometry(w, t, &slots, &ngrp);
+    const uint32_t tt = tt_for(t);
+    dim3 grid((row_tiles(w.n_out) + 7) / 8, (unsigned)(slots / 16 / tt), gemm_i8_k_slices(w, t));
+    const uint4* f = static_cast<const uint4*>(frag);
+    const float2* x2 = static_cast<const float2*>(xs);
+    const float* f1 = static_cast<const float*>(fs);
+    if (tt == 4) {
+        if (dump) gemm_i8_q4m_kernel<4, true><<<grid, 256, 0, s>>>(w, f, x2, f1, (uint32_t)t, (uint32_t)ngrp, y, dump);
+        else gemm_i8_q4m_kernel<4, false><<<grid, 256, 0, s>>>(w, f, x2, f1, (uint32_t)t, (uint32_t)ngrp, y, dump);
+    } else {
+        if (dump) gemm_i8_q4m_kernel<8, true><<<grid, 256, 0, s>>>(w, f, x2, f1, (uint32_t)t, (uint32_t)ngrp, y, dump);
+        else gemm_i8_q4m_kernel<8, false><<<grid, 256, 0, s>>>(w, f, x2, f1, (uint32_t)t, (uint32_t)ngrp, y, dump);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace oxhip

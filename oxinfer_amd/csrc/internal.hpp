@@ -76,6 +76,11 @@ hipError_t launch_q4_scale_groups(const uint16_t* sc32, size_t n_out, size_t n_i
 hipError_t launch_pack_a(const void* x, bool src_bf16, int mode, size_t t, size_t n_in, size_t mtiles, size_t kblocks, void* out,
                          hipStream_t s);
 uint32_t gemm_k_slices(const WeightView& w, size_t mtiles);
+hipError_t launch_gemm_reduce(const float* partial, size_t n, uint32_t slices, void* y, bool out_bf16, hipStream_t s);
+void gemm_i8_geometry(const WeightView& w, size_t t, size_t* slots, size_t* ngrp);
+uint32_t gemm_i8_k_slices(const WeightView& w, size_t t);
+hipError_t launch_quantize_pack_i8(const void* x, bool src_bf16, size_t t, const WeightView& w, void* frag, void* xs, void* fs, hipStream_t s);
+hipError_t launch_gemm_i8(const WeightView& w, const void* frag, const void* xs, const void* fs, size_t t, float* y, int32_t* dump, hipStream_t s);
 hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                             hipStream_t s);
 hipError_t launch_quantize_act_fp8(const void* x, bool src_bf16, size_t t, size_t n_in, size_t mtiles, size_t kblocks, void* out,

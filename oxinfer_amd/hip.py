@@ -79,6 +79,7 @@ def load_library():
         "oxhip_dev_isums": (C.c_int, [vp, vp, C.POINTER(QActC), vp, vp]),
         "oxhip_dev_decode_batch": (C.c_int, [vp, C.POINTER(DecodeJob), sz, vp]),
         "oxhip_dev_gemm": (C.c_int, [vp, vp, vp, C.c_int, sz, vp, C.c_int, C.c_int, vp]),
+        "oxhip_dev_gemm_isums": (C.c_int, [vp, vp, vp, C.c_int, sz, vp, vp]),
         "oxhip_matvec_rows": (C.c_int, [vp, vp, sz, sz, C.POINTER(RowsJob), sz]),
         "oxhip_upload_moe": (vp, [vp, C.POINTER(WeightDesc), C.POINTER(WeightDesc), C.POINTER(WeightDesc), sz, sz, sz, C.c_uint32, C.c_float]),
         "oxhip_free_moe": (None, [vp, vp]),
@@ -352,6 +353,17 @@ class HipBackend:
         if not self.lib.oxhip_dev_gemm(self.ctx, w.handle, x.data_ptr(), xd, t, y.data_ptr(), int(out_bf16), variant, self._stream()):
             raise RuntimeError(self.last_error())
         return y
+
+    def gemm_isums(self, w, x):
+        """The int8 GEMM's exact block sums [t, n_out, n_in/32] (int32)."""
+        import torch
+        t = x.shape[0]
+        out = torch.zeros((t, w.n_out, w.n_in // 32), dtype=torch.int32, device=x.device)
+        xd = 1 if x.dtype == torch.bfloat16 else 0
+        assert x.dtype in (torch.bfloat16, torch.float32) and x.is_contiguous()
+        if not self.lib.oxhip_dev_gemm_isums(self.ctx, w.handle, x.data_ptr(), xd, t, out.data_ptr(), self._stream()):
+            raise RuntimeError(self.last_error())
+        return out
 
     def isums(self, w, xa, per):
         import torch

@@ -167,3 +167,63 @@ def test_gemm_fp8_full_size_sampled_rows(be, oxref):
     assert e8 < 8e-2
     y1 = be.decode(w, x=torch.from_numpy(x[:1]).cuda()).cpu().numpy()
     assert float(np.abs(y1[0, rows] - ref[0]).max() / np.abs(y1).max()) < 1e-3
+
+
+@pytest.mark.parametrize("n_out,n_in", [(37, 4160), (256, 512), (200, 64)])
+def test_gemm_i8_block_sums_bit_exact_and_outputs(be, oxref, n_out, n_in):
+    """Variant (b): the int32 block sums equal the CPU's bit for bit (src/kernels_i8gemm.rs:249-334); outputs within
+    1e-3 of the oracle's restatement (same integer sums, f32 rescale in another order) and within the int8 bound
+    of the exact product."""
+    import torch
+    from oxinfer_amd import synth
+    raw, (q, s16, off) = mlx_case(oxref, n_out, n_in, 17)
+    w = be.upload_mlx_q4(*raw, 64, n_out, n_in)
+    assert w is not None, be.last_error()
+    for t in (1, 16, 37, 64, 65, 150, 300):
+        x = synth.activations(t, n_in, 200 + t, bf16=True)
+        ref, isums = oxref.i8gemm_q4(q, s16, off, 64, n_out, n_in, x, t, want_isums=True)
+        for xd in (torch.from_numpy(x).cuda(), torch.from_numpy(x).cuda().to(torch.bfloat16)):
+            got = be.gemm_isums(w, xd).cpu().numpy()
+            assert np.array_equal(got, isums), (t, xd.dtype)
+            y = be.gemm(w, xd, variant=1).cpu().numpy()
+            assert row_err(y, ref) < 1e-3, (t, xd.dtype)
+        yb = be.gemm(w, torch.from_numpy(x).cuda(), variant=1, out_bf16=True).float().cpu().numpy()
+        assert row_err(yb, ref) < 1e-2
+        exact = oxref.gemm_quant(-1, q, s16, off, n_out, n_in, x, t)
+        if n_in >= 512:
+            assert row_err(y, exact) < 3e-2
+
+
+def test_gemm_i8_extremes_bit_exact(be, oxref):
+    """Nibbles 0, 8 and 15 against activations at the block maximum (src/kernels_x86.rs:829, :893)."""
+    import torch
+    from oxinfer_amd import synth
+    n_out, n_in, t = 32, 256, 20
+    rng = np.random.default_rng(5)
+    wq = rng.choice(np.array([0x00000000, 0x88888888, 0xFFFFFFFF, 0xF0F0F0F0, 0x0F8F0F8F], np.uint32), (n_out, n_in // 8))
+    sc = synth.bf16_bits(np.full((n_out, n_in // 64), 2.0 ** -6, np.float32))
+    bi = synth.bf16_bits(np.full((n_out, n_in // 64), -8 * 2.0 ** -6, np.float32))
+    q, s16, off = oxref.from_mlx_q4(wq, sc, bi, n_out, n_in, 64)
+    w = be.upload_mlx_q4(wq, sc, bi, 64, n_out, n_in)
+    x = rng.choice(np.array([-4.0, 4.0], np.float32), (t, n_in))
+    ref, isums = oxref.i8gemm_q4(q, s16, off, 64, n_out, n_in, x, t, want_isums=True)
+    assert np.array_equal(be.gemm_isums(w, torch.from_numpy(x).cuda()).cpu().numpy(), isums)
+    assert row_err(be.gemm(w, torch.from_numpy(x).cuda(), variant=1).cpu().numpy(), ref) < 1e-5
+
+
+def test_gemm_i8_full_size_sampled_rows(be, oxref):
+    import torch
+    from oxinfer_amd import synth
+    n_out, n_in, t = 4096, 14336, 512
+    wq, sc, bi = synth.mlx_q4(n_out, n_in, 21)
+    w = be.upload_mlx_q4(wq, sc, bi, 64, n_out, n_in)
+    assert w is not None, be.last_error()
+    x = synth.activations(t, n_in, 22, bf16=True)
+    y = be.gemm(w, torch.from_numpy(x).cuda().to(torch.bfloat16), variant=1).cpu().numpy()
+    rows = np.r_[0:4, 2046:2050, n_out - 4:n_out, np.random.default_rng(1).integers(0, n_out, 12)]
+    q, s16, off = oxref.from_mlx_q4(wq[rows], sc[rows], bi[rows], len(rows), n_in, 64)
+    ref = oxref.i8gemm_q4(q, s16, off, 64, len(rows), n_in, x, t)
+    m = np.maximum(np.abs(y).max(axis=1), 1e-30)
+    assert float((np.abs(y[:, rows] - ref).max(axis=1) / m).max()) < 1e-3
+    exact = oxref.gemm_quant(-1, q, s16, off, len(rows), n_in, x, t)
+    assert float((np.abs(y[:, rows] - exact).max(axis=1) / m).max()) < 2e-2
