@@ -16,9 +16,11 @@
 //       integer dot product of one whole block: one instruction yields 2 blocks x 8 tokens x 16
 //       rows of exact block sums, and every output lane is useful at 8 tokens.
 // Weights stream from HBM through a register ring (several 1 KiB records in flight per wave, see
-// layout.hpp); the activations' int8 values come from L2 / L1 (they are shared by every wave),
-// their per-block scales and sums are staged once per workgroup into LDS, transposed so that a
-// lane reads the four tokens it owns with one ds_read_b128.
+// layout.hpp). The activations are staged once per workgroup into LDS: the int8 values in A-operand
+// order (one conflict-free ds_read_b64 per instruction; reading them from global memory per record
+// instead costs three times the weights' L2 requests and doubles the kernel's time), the per-block
+// scales and sums transposed so that a lane reads the four tokens it owns with one ds_read_b128.
+// Rows too long for LDS fall back to reading the int8 values from L2.
 //
 // A workgroup owns `rt` row tiles and splits K over `kw` waves per tile; the partial sums meet in
 // LDS in a fixed order. No atomics, no second launch.
@@ -33,41 +35,60 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int PF = 4;  // records in flight per wave beyond the one being consumed
+// Records a wave keeps in flight. HBM delivers about 8 TB/s at about 2 us of loaded latency, so some 16 MB must be
+// on request across the chip at any moment: about 4000 resident waves x PF KiB.
+template <int FMT, int NT>
+constexpr int pf_for() { return FMT == FMT_Q4_K ? 6 : 8; }
 
 struct Meta4 {
     float xs[4];
-    int su[4];
+    float c[4];
     float fs[4];
+    int su[4];
 };
 
-// LDS: xs | su | fs, each [nblk][TPAD] (su, fs only for the formats that use them)
-template <int TPAD, bool SUMS, class RowOf>
+// The kernels evaluate a block's contribution with the fewest f32 operations per (row, token):
+//   Q8_0:  d * (xs * I)
+//   Q4_K:  d * sc * (xs * U + c) - dmin * mn * fs,   c = 8 * (fs - xs * su)      [U = sum of unsigned nibbles * q]
+//   MLX:   d * (xs * U + c) + off * fs,              c = -8 * xs * su
+// which equal the reference's (s * xs) * (U - 8 su) + m * fs (src/ggml.rs:1288-1315, src/kernels.rs:1287-1297)
+// up to f32 rounding; the integer sums U - 8 su themselves are exact (and are what the DUMP variant writes).
+// LDS: xs | c | fs | su, each [nblk][TPAD] (c, fs only for the formats with sums; su only for DUMP)
+template <int FMT, int TPAD, bool SUMS, bool DUMP, class RowOf>
 __device__ __forceinline__ void stage_meta(const QActView& xa, uint32_t t, uint32_t nblk, float* lds, RowOf row_of) {
     float* xs = lds;
-    int* su = reinterpret_cast<int*>(lds + (size_t)nblk * TPAD);
+    float* cc = lds + (size_t)nblk * TPAD;
     float* fs = lds + (size_t)2 * nblk * TPAD;
+    int* su = reinterpret_cast<int*>(lds + (size_t)3 * nblk * TPAD);
     for (uint32_t i = threadIdx.x; i < nblk * TPAD; i += blockDim.x) {
         uint32_t tok = i / nblk, b = i % nblk;  // consecutive threads read consecutive blocks of one token
         bool live = tok < t;
         size_t src = (live ? row_of(tok) : 0) * nblk + b;
-        xs[b * TPAD + tok] = live ? xa.scales[src] : 0.0f;
+        const float x = live ? xa.scales[src] : 0.0f;
+        xs[b * TPAD + tok] = x;
         if (SUMS) {
-            su[b * TPAD + tok] = live ? xa.sums[src] : 0;
-            fs[b * TPAD + tok] = live ? xa.fsums[src] : 0.0f;
+            const int sq = live ? xa.sums[src] : 0;
+            const float f = live ? xa.fsums[src] : 0.0f;
+            cc[b * TPAD + tok] = FMT == FMT_Q4_K ? 8.0f * (f - x * (float)sq) : -8.0f * (x * (float)sq);
+            fs[b * TPAD + tok] = f;
+            if (DUMP) su[b * TPAD + tok] = sq;
         }
     }
 }
 
-template <int TPAD, bool SUMS>
+template <int TPAD, bool SUMS, bool DUMP>
 __device__ __forceinline__ void load_meta(const float* lds, uint32_t nblk, uint32_t b, uint32_t tok0, Meta4& m) {
     const float4 x = *reinterpret_cast<const float4*>(lds + (size_t)b * TPAD + tok0);
     m.xs[0] = x.x; m.xs[1] = x.y; m.xs[2] = x.z; m.xs[3] = x.w;
     if (SUMS) {
-        const int4 s = *reinterpret_cast<const int4*>(lds + (size_t)nblk * TPAD + (size_t)b * TPAD + tok0);
+        const float4 c = *reinterpret_cast<const float4*>(lds + (size_t)nblk * TPAD + (size_t)b * TPAD + tok0);
         const float4 f = *reinterpret_cast<const float4*>(lds + (size_t)2 * nblk * TPAD + (size_t)b * TPAD + tok0);
-        m.su[0] = s.x; m.su[1] = s.y; m.su[2] = s.z; m.su[3] = s.w;
+        m.c[0] = c.x; m.c[1] = c.y; m.c[2] = c.z; m.c[3] = c.w;
         m.fs[0] = f.x; m.fs[1] = f.y; m.fs[2] = f.z; m.fs[3] = f.w;
+        if (DUMP) {
+            const int4 q = *reinterpret_cast<const int4*>(lds + (size_t)3 * nblk * TPAD + (size_t)b * TPAD + tok0);
+            m.su[0] = q.x; m.su[1] = q.y; m.su[2] = q.z; m.su[3] = q.w;
+        }
     }
 }
 
@@ -102,20 +123,26 @@ struct Step<FMT_Q4M> {
 // GROUPED: blockIdx.y walks the chunks of a grouped launch (MoE experts over their routed tokens): chunk c is
 // {expert, first row, rows (<= 8)}; the weights are expert's, activation row i of the chunk is row
 // rowmap[first + i] of xa (or first + i without a map), and its output is row first + i of y.
-template <int FMT, int NT, bool DUMP, bool GROUPED>
-__global__ __launch_bounds__(512) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw,
+// ALDS: the int8 activations are staged into LDS in operand order (the launcher checks that they fit).
+template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS>
+__global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw,
                                                            float* __restrict__ y, int32_t* __restrict__ dump, GroupView grp) {
     constexpr int TPAD = NT <= 4 ? 4 : 8;
     constexpr int NI = NT < 4 ? NT : 4;          // accumulator registers that hold live tokens
     constexpr bool SUMS = FMT != FMT_Q8_0;
-    extern __shared__ float lds[];
+    extern __shared__ float lds_all[];
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t n = lane & 15, kq = lane >> 4;  // B / D role: row n of the tile; A role: slot n
     const uint32_t nblk = w.n_in / 32;
     const uint32_t r = wave / kw, ks = wave % kw;
     const uint32_t tile = blockIdx.x * rt + r;
     const uint32_t ntiles = row_tiles(w.n_out);
-    float* red = lds + (size_t)(SUMS ? 3 : 1) * nblk * TPAD;  // [rt * kw][TPAD][16]
+    // LDS: [operand-order activations: 512 B per pair of blocks] [scales, sums] [partial sums]; with ALDS the
+    // partial sums reuse the activations' space once every wave is done with them
+    const uint32_t nmf = (nblk + 1) / 2;
+    uint2* afr = reinterpret_cast<uint2*>(lds_all);
+    float* lds = lds_all + (ALDS ? (size_t)nmf * 128 : 0);
+    float* red = ALDS ? lds_all : lds + (size_t)(SUMS ? (DUMP ? 4 : 3) : 1) * nblk * TPAD;  // [rt * kw][TPAD][16]
     uint32_t row0 = 0;  // first activation / output row of this launch unit
     if (GROUPED) {
         if (blockIdx.y >= (uint32_t)*grp.nchunks) return;  // uniform over the workgroup
@@ -152,7 +179,7 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(WeightView w, QActView
             const uint8_t* rec = base + (size_t)s * T8_REC;
             st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
             st.dd = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
-            act2(2 * s + a_half, 8 * kq, st.a);
+            if (!ALDS) act2(2 * s + a_half, 8 * kq, st.a);
         } else if constexpr (FMT == FMT_Q4_K) {
             const uint8_t* rec = base + (size_t)(s >> 1) * TK4_REC;
             st.w = *reinterpret_cast<const uint4*>(rec + (s & 1) * 1024 + 16 * lane);
@@ -160,24 +187,34 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(WeightView w, QActView
             st.sc4 = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 4 * (s & 1));
             st.mn4 = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
             st.dd = *reinterpret_cast<const uint32_t*>(rec + 2304 + 4 * n);
-            act2(4 * s + a_half, 8 * kq, st.a);
-            act2(4 * s + 2 + a_half, 8 * kq, st.a + 2);
+            if (!ALDS) {
+                act2(4 * s + a_half, 8 * kq, st.a);
+                act2(4 * s + 2 + a_half, 8 * kq, st.a + 2);
+            }
         } else {
             const uint8_t* rec = base + (size_t)s * T4M_REC;
             st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
             st.dd = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
             st.oo = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
+            if (!ALDS) {
 #pragma unroll
-            for (int g = 0; g < 2; g++) {  // positions 4 kq.. and 16 + 4 kq.. of block 4 s + 2 g + half
-                const int8_t* xb = xrow + min(4 * s + 2 * g + a_half, nblk - 1) * 32;
-                st.a[2 * g] = *reinterpret_cast<const uint32_t*>(xb + 4 * kq);
-                st.a[2 * g + 1] = *reinterpret_cast<const uint32_t*>(xb + 16 + 4 * kq);
+                for (int g = 0; g < 2; g++) {  // positions 4 kq.. and 16 + 4 kq.. of block 4 s + 2 g + half
+                    const int8_t* xb = xrow + min(4 * s + 2 * g + a_half, nblk - 1) * 32;
+                    st.a[2 * g] = *reinterpret_cast<const uint32_t*>(xb + 4 * kq);
+                    st.a[2 * g + 1] = *reinterpret_cast<const uint32_t*>(xb + 16 + 4 * kq);
+                }
             }
         }
     };
 
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    auto mfma = [&](v4i bw, uint32_t d0, uint32_t d1) -> v4i {
+    // `m`: index of the instruction along K (pair of blocks 2 m, 2 m + 1); with ALDS its operand comes from LDS
+    auto mfma = [&](v4i bw, uint32_t m, uint32_t d0, uint32_t d1) -> v4i {
+        if (ALDS) {
+            const uint2 av = afr[(size_t)m * 64 + lane];
+            d0 = av.x;
+            d1 = av.y;
+        }
         v4i a = {(int)(d0 & amask0), (int)(d1 & amask0), (int)(d0 & amask1), (int)(d1 & amask1)};
         v4i c = {0, 0, 0, 0};
         return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bw, c, 0, 0, 0);
@@ -195,84 +232,113 @@ __global__ __launch_bounds__(512) void decode_mfma_kernel(WeightView w, QActView
         if constexpr (FMT == FMT_Q8_0) {
             const float d = f16_bits_to_f32((uint16_t)(d_half ? st.dd >> 16 : st.dd & 0xFFFF));
             v4i bw = {(int)c.x, (int)c.y, (int)c.z, (int)c.w};
-            v4i D = mfma(bw, st.a[0], st.a[1]);
+            v4i D = mfma(bw, s, st.a[0], st.a[1]);
             const uint32_t b = 2 * s + d_half;
             Meta4 m;
-            load_meta<TPAD, SUMS>(lds, nblk, min(b, nblk - 1), d_tok0, m);
+            load_meta<TPAD, SUMS, DUMP>(lds, nblk, min(b, nblk - 1), d_tok0, m);
             int isum[4] = {D.x, D.y, D.z, D.w};
 #pragma unroll
-            for (int i = 0; i < NI; i++) acc[i] += (d * m.xs[i]) * (float)isum[i];
+            for (int i = 0; i < NI; i++) acc[i] = fmaf(d, m.xs[i] * (float)isum[i], acc[i]);
             dump_block(b, isum);
         } else if constexpr (FMT == FMT_Q4_K) {
-            const float d = f16_bits_to_f32((uint16_t)(st.dd & 0xFFFF)), dmin = f16_bits_to_f32((uint16_t)(st.dd >> 16));
+            const float d = f16_bits_to_f32((uint16_t)(st.dd & 0xFFFF)), ndmin = -f16_bits_to_f32((uint16_t)(st.dd >> 16));
+            float P[4] = {0.0f, 0.0f, 0.0f, 0.0f}, Q[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int pr = 0; pr < 2; pr++) {  // the two byte pairs of the lane's chunk
                 const uint32_t lo = pr ? c.z : c.x, hi = pr ? c.w : c.y;
                 v4i bw = {(int)(lo & 0x0F0F0F0Fu), (int)(hi & 0x0F0F0F0Fu), (int)((lo >> 4) & 0x0F0F0F0Fu),
                           (int)((hi >> 4) & 0x0F0F0F0Fu)};
-                v4i D = mfma(bw, st.a[2 * pr], st.a[2 * pr + 1]);
+                v4i D = mfma(bw, 2 * s + pr, st.a[2 * pr], st.a[2 * pr + 1]);
                 const uint32_t b = 4 * s + 2 * pr + d_half;  // global index of this lane's block of 32
                 const uint32_t q = 2 * pr + d_half;
                 const float sc = (float)((st.sc4 >> (8 * q)) & 0xFF), mn = (float)((st.mn4 >> (8 * q)) & 0xFF);
-                const float sv = d * sc;
-                const float mv = 8.0f * sv - dmin * mn;
                 Meta4 m;
-                load_meta<TPAD, SUMS>(lds, nblk, b, d_tok0, m);
-                int isum[4] = {D.x - 8 * m.su[0], D.y - 8 * m.su[1], D.z - 8 * m.su[2], D.w - 8 * m.su[3]};
+                load_meta<TPAD, SUMS, DUMP>(lds, nblk, b, d_tok0, m);
+                const int U[4] = {D.x, D.y, D.z, D.w};
 #pragma unroll
                 for (int i = 0; i < NI; i++) {
-                    acc[i] += (sv * m.xs[i]) * (float)isum[i];
-                    acc[i] += mv * m.fs[i];
+                    P[i] = fmaf(sc, fmaf(m.xs[i], (float)U[i], m.c[i]), P[i]);
+                    Q[i] = fmaf(mn, m.fs[i], Q[i]);
                 }
-                dump_block(b, isum);
+                if (DUMP) {
+                    int isum[4] = {U[0] - 8 * m.su[0], U[1] - 8 * m.su[1], U[2] - 8 * m.su[2], U[3] - 8 * m.su[3]};
+                    dump_block(b, isum);
+                }
             }
+#pragma unroll
+            for (int i = 0; i < NI; i++) acc[i] = fmaf(ndmin, Q[i], fmaf(d, P[i], acc[i]));
         } else {
 #pragma unroll
             for (int g = 0; g < 2; g++) {  // the two groups of 64 of the step
                 const uint32_t w0 = g ? c.z : c.x, w1 = g ? c.w : c.y;  // blocks 2 g, 2 g + 1
                 v4i bw = {(int)(w0 & 0x0F0F0F0Fu), (int)((w0 >> 4) & 0x0F0F0F0Fu), (int)(w1 & 0x0F0F0F0Fu),
                           (int)((w1 >> 4) & 0x0F0F0F0Fu)};
-                v4i D = mfma(bw, st.a[2 * g], st.a[2 * g + 1]);
+                v4i D = mfma(bw, 2 * s + g, st.a[2 * g], st.a[2 * g + 1]);
                 const uint32_t b = 4 * s + 2 * g + d_half;
                 const float d = f16_bits_to_f32((uint16_t)(g ? st.dd >> 16 : st.dd & 0xFFFF));
                 const float off = bf16_bits_to_f32((uint16_t)(g ? st.oo >> 16 : st.oo & 0xFFFF));
                 Meta4 m;
-                load_meta<TPAD, SUMS>(lds, nblk, min(b, nblk - 1), d_tok0, m);
-                int isum[4] = {D.x - 8 * m.su[0], D.y - 8 * m.su[1], D.z - 8 * m.su[2], D.w - 8 * m.su[3]};
-                if (b < nblk) {  // padding blocks hold zero codes, but the -8 would still count
+                load_meta<TPAD, SUMS, DUMP>(lds, nblk, min(b, nblk - 1), d_tok0, m);
+                const int U[4] = {D.x, D.y, D.z, D.w};
+                if (b < nblk) {  // padding blocks hold zero codes and zero scales, but their staged sums are a real block's
 #pragma unroll
-                    for (int i = 0; i < NI; i++) {
-                        acc[i] += ((float)isum[i] * d) * m.xs[i];
-                        acc[i] += off * m.fs[i];
-                    }
+                    for (int i = 0; i < NI; i++) acc[i] = fmaf(off, m.fs[i], fmaf(d, fmaf(m.xs[i], (float)U[i], m.c[i]), acc[i]));
                 }
-                dump_block(b, isum);
+                if (DUMP) {
+                    int isum[4] = {U[0] - 8 * m.su[0], U[1] - 8 * m.su[1], U[2] - 8 * m.su[2], U[3] - 8 * m.su[3]};
+                    dump_block(b, isum);
+                }
             }
         }
     };
 
     // The first ring of records is requested before anything else, so that HBM latency overlaps the
     // staging of the activation scales.
+    constexpr int PF = pf_for<FMT, NT>();
     Step<FMT> ring[PF];
 #pragma unroll
     for (int p = 0; p < PF; p++)
         if (s0 + p < s1) load_step(ring[p], s0 + p);
-    stage_meta<TPAD, SUMS>(xa, t, nblk, lds, src_row);
+    stage_meta<FMT, TPAD, SUMS, DUMP>(xa, t, nblk, lds, src_row);
+    if (ALDS) {
+        // slot (m, lane) of the operand array: lane = 16 kq + 8 half + token holds the 8 values of block 2 m + half
+        // that the weights' lane group kq pairs with (Q4: positions 4 kq.. and 16 + 4 kq..; else 8 kq..). A thread
+        // moves 16 (Q4: 32) consecutive bytes of one token's row, so the global reads are whole lines. Absent tokens
+        // and a padding block keep whatever LDS holds: those products meet zero weights or are dropped.
+        if (FMT == FMT_Q4M) {
+            for (uint32_t i = threadIdx.x; i < t * nblk; i += blockDim.x) {
+                const uint32_t tok = i / nblk, b = i % nblk;
+                const uint4* xb = reinterpret_cast<const uint4*>(xa.q + src_row(tok) * w.n_in + (size_t)b * 32);
+                const uint4 lo = xb[0], hi = xb[1];
+                uint2* dst = afr + (size_t)(b >> 1) * 64 + 8 * (b & 1) + tok;
+                dst[0] = make_uint2(lo.x, hi.x);
+                dst[16] = make_uint2(lo.y, hi.y);
+                dst[32] = make_uint2(lo.z, hi.z);
+                dst[48] = make_uint2(lo.w, hi.w);
+            }
+        } else {
+            for (uint32_t i = threadIdx.x; i < t * 2 * nblk; i += blockDim.x) {
+                const uint32_t tok = i / (2 * nblk), c = i % (2 * nblk), b = c >> 1;
+                const uint4 v = *reinterpret_cast<const uint4*>(xa.q + src_row(tok) * w.n_in + (size_t)c * 16);
+                uint2* dst = afr + (size_t)(b >> 1) * 64 + 32 * (c & 1) + 8 * (b & 1) + tok;
+                dst[0] = make_uint2(v.x, v.y);
+                dst[16] = make_uint2(v.z, v.w);
+            }
+        }
+    }
     __syncthreads();
+    // each slot is refilled as soon as its record has been consumed, so PF - 1 records stay on request
     for (uint32_t sb = s0; sb < s1; sb += PF) {
-        Step<FMT> next[PF];
 #pragma unroll
-        for (int p = 0; p < PF; p++)
-            if (sb + PF + p < s1) load_step(next[p], sb + PF + p);
-#pragma unroll
-        for (int p = 0; p < PF; p++)
+        for (int p = 0; p < PF; p++) {
             if (sb + p < s1) compute_step(ring[p], sb + p);
-#pragma unroll
-        for (int p = 0; p < PF; p++) ring[p] = next[p];
+            if (sb + PF + p < s1) load_step(ring[p], sb + PF + p);
+        }
     }
     // the two block parities of a token meet across lane groups kq and kq ^ 2
 #pragma unroll
     for (int i = 0; i < 4; i++) acc[i] += __shfl_xor(acc[i], 32);
+    if (ALDS) __syncthreads();  // the partial sums overwrite the staged activations
     if (kq < 2) {
 #pragma unroll
         for (int i = 0; i < 4; i++)
@@ -296,17 +362,51 @@ struct Shape {
     uint32_t rt, kw;
 };
 
-// Waves per workgroup and how they split: enough workgroups to cover the CUs, and K split so that
-// about 4096-8192 waves exist while each keeps a few records to stream.
+// Waves per workgroup (rt row tiles x kw K slices, 16 waves when the matrix allows) and how they split. A function
+// of the weight's shape only, so a row's sum is associated the same way whatever the batch or launch kind.
+// K is split as far as each wave keeps about four records; then row tiles are added per workgroup until the
+// workgroups fit the chip at once (256 CUs, one 16-wave workgroup each), so that the whole matrix is on request
+// from the first microsecond instead of in successive generations of workgroups.
 Shape shape_for(uint32_t ntiles, uint32_t nsteps) {
     uint32_t kw = 1;
-    while (kw < 8 && (size_t)ntiles * kw < 4096 && nsteps / (kw * 2) >= 4) kw *= 2;
-    if (kw < 4 && nsteps / 4 >= 2) kw = 4;
+    while (kw < 16 && nsteps / (kw * 2) >= 4) kw *= 2;
+    uint32_t rt = 16 / kw;
+    while (kw > 1 && (ntiles + rt - 1) / rt > 256) {
+        kw /= 2;
+        rt *= 2;
+    }
     if (const char* e = getenv("OXHIP_DECODE_KW")) {  // developer override for tuning runs
         uint32_t v = (uint32_t)atoi(e);
-        if (v >= 1 && v <= 8) kw = v;
+        if (v == 1 || v == 2 || v == 4 || v == 8 || v == 16) {
+            kw = v;
+            rt = 16 / kw;
+        }
     }
-    return Shape{1, kw};
+    return Shape{rt, kw};
+}
+
+constexpr size_t LDS_MAX = 160 * 1024;
+
+// Dynamic LDS of a launch; `alds` comes back false when the operand-order activations do not fit.
+size_t lds_bytes(bool sums, bool dump, uint32_t nblk, int tpad, const Shape& sh, bool* alds) {
+    const size_t meta = (size_t)(sums ? (dump ? 4 : 3) : 1) * nblk * tpad * 4, red = (size_t)sh.rt * sh.kw * tpad * 16 * 4;
+    const size_t act = (size_t)((nblk + 1) / 2) * 512;
+    const size_t with = act + meta > red ? act + meta : red;  // the partial sums reuse the activations' space
+    *alds = with <= LDS_MAX && act >= red;
+    return *alds ? with : meta + red;
+}
+
+template <int FMT, int NT, bool DUMP, bool GROUPED>
+hipError_t launch_one(bool alds, dim3 grid, dim3 block, size_t lds, hipStream_t s, const WeightView& w, const QActView& v, uint32_t t,
+                      const Shape& sh, float* y, int32_t* dump, const GroupView& g) {
+    hipError_t e = hipSuccess;
+    auto go = [&](auto kern) {
+        if (lds > 48 * 1024) e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, v, t, sh.rt, sh.kw, y, dump, g);
+    };
+    if (alds) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, true>);
+    else go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, false>);
+    return e != hipSuccess ? e : hipGetLastError();
 }
 
 template <int FMT, bool DUMP>
@@ -327,20 +427,15 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
         float* yo = y ? y + c0 * w.n_out : nullptr;  // no output rows when only the block sums are wanted
         int32_t* du = dump ? dump + c0 * (size_t)w.n_out * nblk : nullptr;
         const int tpad = tc <= 4 ? 4 : 8;
-        const size_t lds = ((size_t)(FMT == FMT_Q8_0 ? 1 : 3) * nblk * tpad + (size_t)sh.rt * sh.kw * tpad * 16) * 4;
-        if (lds > 160 * 1024) return hipErrorInvalidValue;  // rows too long for the staged activation scales
+        bool alds;
+        const size_t lds = lds_bytes(FMT != FMT_Q8_0, DUMP, nblk, tpad, sh, &alds);
+        if (lds > LDS_MAX) return hipErrorInvalidValue;  // rows too long for the staged activation scales
         const uint32_t tt = (uint32_t)tc;
-        hipError_t e = hipSuccess;
-        auto go = [&](auto kern) {
-            if (lds > 48 * 1024) e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, v, tt, sh.rt, sh.kw, yo, du, GroupView{});
-        };
-        if (tc == 1) go(decode_mfma_kernel<FMT, 1, DUMP, false>);
-        else if (tc == 2) go(decode_mfma_kernel<FMT, 2, DUMP, false>);
-        else if (tc <= 4) go(decode_mfma_kernel<FMT, 4, DUMP, false>);
-        else go(decode_mfma_kernel<FMT, 8, DUMP, false>);
-        if (e != hipSuccess) return e;
-        e = hipGetLastError();
+        hipError_t e;
+        if (tc == 1) e = launch_one<FMT, 1, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{});
+        else if (tc == 2) e = launch_one<FMT, 2, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{});
+        else if (tc <= 4) e = launch_one<FMT, 4, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{});
+        else e = launch_one<FMT, 8, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{});
         if (e != hipSuccess) return e;
         c0 += tc;
     }
@@ -354,22 +449,16 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
     const uint32_t nsteps = FMT == FMT_Q8_0 ? t8_steps(w.n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in) : t4m_steps(w.n_in));
     // the same K split as a plain launch on this matrix, so that a row's sum is associated the same way
     // (and is bit-identical) whether its expert runs alone or in a group
-    Shape sh = shape_for(ntiles, nsteps);
+    const Shape sh = shape_for(ntiles, nsteps);
     const uint32_t nblk = w.n_in / 32;
     dim3 grid((ntiles + sh.rt - 1) / sh.rt, max_chunks), block(64 * sh.rt * sh.kw);
     const int tpad = max_rows <= 4 ? 4 : 8;
-    const size_t lds = ((size_t)(FMT == FMT_Q8_0 ? 1 : 3) * nblk * tpad + (size_t)sh.rt * sh.kw * tpad * 16) * 4;
-    if (lds > 160 * 1024) return hipErrorInvalidValue;
-    hipError_t e = hipSuccess;
-    auto go = [&](auto kern) {
-        if (lds > 48 * 1024) e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, xa, 0u, sh.rt, sh.kw, y, nullptr, g);
-    };
-    if (max_rows == 1) go(decode_mfma_kernel<FMT, 1, false, true>);
-    else if (max_rows <= 4) go(decode_mfma_kernel<FMT, 4, false, true>);
-    else go(decode_mfma_kernel<FMT, 8, false, true>);
-    if (e != hipSuccess) return e;
-    return hipGetLastError();
+    bool alds;
+    const size_t lds = lds_bytes(FMT != FMT_Q8_0, false, nblk, tpad, sh, &alds);
+    if (lds > LDS_MAX) return hipErrorInvalidValue;
+    if (max_rows == 1) return launch_one<FMT, 1, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g);
+    if (max_rows <= 4) return launch_one<FMT, 4, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g);
+    return launch_one<FMT, 8, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g);
 }
 
 }  // namespace

@@ -9,6 +9,8 @@
 #include "internal.hpp"
 #include "layout.hpp"
 
+#include <cstdlib>
+
 namespace oxhip {
 
 namespace {
@@ -95,58 +97,60 @@ __global__ __launch_bounds__(256) void quantize_pack_i8_kernel(const void* __res
     fs[base * 16 + n] = fsum[0] + fsum[1];
 }
 
-// Workgroup: 4 waves, each two row tiles (32 rows) x TT token tiles (16 TT tokens) over one K slice; no LDS and no
+// Workgroup: 4 waves, each RT row tiles (16 RT rows) x TT token tiles (16 TT tokens) over one K slice; no LDS and no
 // barrier: every operand a lane needs is its own (weights, row scales) or its token's (activation fragments, scales).
+// A group of 64 columns is worked in PH phases of TT / PH token tiles, each phase's activation operands requested one
+// phase ahead. Two waves per SIMD keep the matrix-core results in ordinary registers.
 // DUMP also stores the exact block sums to dump[(token * n_out + row) * (n_in / 32) + block].
-template <int TT, bool DUMP>
-__global__ __launch_bounds__(256) void gemm_i8_q4m_kernel(WeightView w, const uint4* __restrict__ afrag, const float2* __restrict__ axs,
-                                                          const float* __restrict__ afs, uint32_t t, uint32_t ngrp,
-                                                          float* __restrict__ y, int32_t* __restrict__ dump) {
+template <int RT, int TT, int PH, bool DUMP>
+__global__ __launch_bounds__(256, 2) void gemm_i8_q4m_kernel(WeightView w, const uint4* __restrict__ afrag, const float2* __restrict__ axs,
+                                                             const float* __restrict__ afs, uint32_t t, uint32_t ngrp,
+                                                             float* __restrict__ y, int32_t* __restrict__ dump) {
+    constexpr int TH = TT / PH;
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t n = lane & 15, kq = lane >> 4;
     const uint32_t ntiles = row_tiles(w.n_out), all_steps = t4m_steps(w.n_in), nblk = w.n_in / 32;
-    const uint32_t rt0 = blockIdx.x * 8 + 2 * wave;
+    const uint32_t rt0 = (blockIdx.x * 4 + wave) * RT;
     if (rt0 >= ntiles) return;
     const uint32_t tt0 = blockIdx.y * TT;
     const uint32_t per = (all_steps + gridDim.z - 1) / gridDim.z;
     const uint32_t s0 = blockIdx.z * per, s1 = min(all_steps, s0 + per);
     y += (size_t)blockIdx.z * t * w.n_out;
 
-    const uint8_t* wbase[2];
+    const uint8_t* wbase[RT];
 #pragma unroll
-    for (int i = 0; i < 2; i++) wbase[i] = w.p0 + (size_t)min(rt0 + i, ntiles - 1) * all_steps * T4M_REC;
-    float acc[2][TT][4];
+    for (int i = 0; i < RT; i++) wbase[i] = w.p0 + (size_t)min(rt0 + i, ntiles - 1) * all_steps * T4M_REC;
+    float acc[RT][TT][4];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < RT; i++)
 #pragma unroll
         for (int tt = 0; tt < TT; tt++)
 #pragma unroll
             for (int e = 0; e < 4; e++) acc[i][tt][e] = 0.0f;
 
-    constexpr int TH = TT / 2;  // token tiles per phase: a group of 64 columns is worked in two halves
-    struct Rec {
-        uint4 c, dd, oo;
-    };
     struct Act {
         uint4 f[TH];
         float2 xs[TH];
         float fs[TH];
     };
-    auto load_rec = [&](Rec* r, uint32_t s) {
+    auto load_codes = [&](uint4* c, uint32_t s) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < RT; i++) c[i] = *reinterpret_cast<const uint4*>(wbase[i] + (size_t)s * T4M_REC + 16 * lane);
+    };
+    auto load_scales = [&](uint4* dd, uint4* oo, uint32_t s) {
+#pragma unroll
+        for (int i = 0; i < RT; i++) {
             const uint8_t* rec = wbase[i] + (size_t)s * T4M_REC;
-            r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
-            r[i].dd = *reinterpret_cast<const uint4*>(rec + 1024 + 16 * kq);
-            r[i].oo = *reinterpret_cast<const uint4*>(rec + 1088 + 16 * kq);
+            dd[i] = *reinterpret_cast<const uint4*>(rec + 1024 + 16 * kq);
+            oo[i] = *reinterpret_cast<const uint4*>(rec + 1088 + 16 * kq);
         }
     };
-    // phase p = 2 * group + half
+    // phase p = PH * group + part
     const uint4* fb = afrag + (size_t)tt0 * ngrp * 64 + lane;
     const float2* xb = axs + (size_t)tt0 * ngrp * 16 + n;
     const float* sb = afs + (size_t)tt0 * ngrp * 16 + n;
     auto load_act = [&](Act& a, uint32_t p) {
-        const uint32_t grp = p >> 1, h = p & 1;
+        const uint32_t grp = p / PH, h = p % PH;
 #pragma unroll
         for (int tt = 0; tt < TH; tt++) {
             const size_t at = (size_t)(h * TH + tt) * ngrp + grp;
@@ -155,16 +159,16 @@ __global__ __launch_bounds__(256) void gemm_i8_q4m_kernel(WeightView w, const ui
             a.fs[tt] = sb[at * 16];
         }
     };
-    auto compute = [&](const Rec* r, const Act& a, uint32_t grp, int g, int h) {
-        long wa[2][2];
-        float ds[2][4], off[2][4];
+    auto compute = [&](const uint4* c, const uint4* dv, const uint4* ov, const Act& a, uint32_t grp, int g, int h) {
+        long wa[RT][2];
+        float ds[RT][4], off[RT][4];
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const uint32_t w0 = g ? r[i].c.z : r[i].c.x, w1 = g ? r[i].c.w : r[i].c.y;
+        for (int i = 0; i < RT; i++) {
+            const uint32_t w0 = g ? c[i].z : c[i].x, w1 = g ? c[i].w : c[i].y;
             wa[i][0] = pack64(center4(w0 & 0x0F0F0F0Fu), center4((w0 >> 4) & 0x0F0F0F0Fu));
             wa[i][1] = pack64(center4(w1 & 0x0F0F0F0Fu), center4((w1 >> 4) & 0x0F0F0F0Fu));
-            const uint32_t dd[4] = {r[i].dd.x, r[i].dd.y, r[i].dd.z, r[i].dd.w};
-            const uint32_t oo[4] = {r[i].oo.x, r[i].oo.y, r[i].oo.z, r[i].oo.w};
+            const uint32_t dd[4] = {dv[i].x, dv[i].y, dv[i].z, dv[i].w};
+            const uint32_t oo[4] = {ov[i].x, ov[i].y, ov[i].z, ov[i].w};
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 ds[i][e] = f16_bits_to_f32((uint16_t)(g ? dd[e] >> 16 : dd[e] & 0xFFFF));
@@ -175,7 +179,7 @@ __global__ __launch_bounds__(256) void gemm_i8_q4m_kernel(WeightView w, const ui
         for (int tt = 0; tt < TH; tt++) {
             const long b0 = pack64(a.f[tt].x, a.f[tt].y), b1 = pack64(a.f[tt].z, a.f[tt].w);
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
+            for (int i = 0; i < RT; i++) {
                 const v4i z = {0, 0, 0, 0};
                 const v4i d0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wa[i][0], b0, z, 0, 0, 0);
                 const v4i d1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wa[i][1], b1, z, 0, 0, 0);
@@ -203,28 +207,34 @@ __global__ __launch_bounds__(256) void gemm_i8_q4m_kernel(WeightView w, const ui
     };
 
     if (s0 < s1) {
-        // Each phase's activation operands are requested one phase ahead, the next step's record a step ahead;
-        // past the end the requests repeat the last valid address and are dropped.
-        const uint32_t plast = 4 * s1 - 1;
-        Rec rec[2], rnext[2];
+        // The next step's record is requested a step ahead and each phase's activation operands a phase ahead; past
+        // the end the requests repeat the last valid address and are dropped.
+        const uint32_t plast = 2 * PH * s1 - 1;
+        uint4 c[RT], cnext[RT], dd[RT], oo[RT], dnext[RT], onext[RT];
         Act cur, nxt;
-        load_rec(rec, s0);
-        load_act(cur, 4 * s0);
+        load_codes(c, s0);
+        load_scales(dd, oo, s0);
+        load_act(cur, 2 * PH * s0);
         for (uint32_t s = s0; s < s1; s++) {
-            load_rec(rnext, min(s + 1, s1 - 1));
+            load_codes(cnext, min(s + 1, s1 - 1));
+            load_scales(dnext, onext, min(s + 1, s1 - 1));
 #pragma unroll
-            for (int ph = 0; ph < 4; ph++) {
-                load_act(nxt, min(4 * s + ph + 1, plast));
-                compute(rec, cur, 2 * s + (ph >> 1), ph >> 1, ph & 1);
+            for (int ph = 0; ph < 2 * PH; ph++) {
+                load_act(nxt, min(2 * PH * s + ph + 1, plast));
+                compute(c, dd, oo, cur, 2 * s + ph / PH, ph / PH, ph % PH);
                 cur = nxt;
             }
-            rec[0] = rnext[0];
-            rec[1] = rnext[1];
+#pragma unroll
+            for (int i = 0; i < RT; i++) {
+                c[i] = cnext[i];
+                dd[i] = dnext[i];
+                oo[i] = onext[i];
+            }
         }
     }
 
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
+    for (int i = 0; i < RT; i++) {
         if (rt0 + i >= ntiles) continue;
 #pragma unroll
         for (int tt = 0; tt < TT; tt++) {
@@ -239,24 +249,58 @@ __global__ __launch_bounds__(256) void gemm_i8_q4m_kernel(WeightView w, const ui
     }
 }
 
-constexpr uint32_t tt_for(size_t t) { return t <= 64 ? 4u : 8u; }
+// Wave tiles on offer: {row tiles, token tiles, phases}. The pick spreads the (row tile, token tile) pairs evenly
+// over the 1024 SIMDs at two waves each: time goes as the pairs the busiest SIMD works through; larger tiles win ties
+// (fewer loads). Four row tiles per wave measured 1.6 to 2.5 times slower than two and are not offered.
+struct Tile {
+    uint32_t rt, tt, ph;
+};
+constexpr Tile TILES[] = {{2, 8, 2}, {2, 4, 1}, {2, 2, 1}};
+constexpr int NTILES = sizeof(TILES) / sizeof(TILES[0]);
+
+int pick_tile(uint32_t ntiles, uint32_t ttiles) {
+    if (const char* e = getenv("OXHIP_I8_TILE")) {  // developer override for tuning runs
+        const int v = atoi(e);
+        if (v >= 0 && v < NTILES) return v;
+    }
+    int best = 0;
+    uint64_t best_cost = ~0ull;
+    for (int i = 0; i < NTILES; i++) {
+        const Tile& c = TILES[i];
+        const uint64_t waves = (uint64_t)((ntiles + c.rt - 1) / c.rt) * ((ttiles + c.tt - 1) / c.tt);
+        const uint64_t cost = ((waves + 2047) / 2048) * c.rt * c.tt;
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = i;
+        }
+    }
+    return best;
+}
+
+template <int RT, int TT, int PH>
+void launch_tile(dim3 grid, hipStream_t s, const WeightView& w, const uint4* f, const float2* x2, const float* f1, uint32_t t, uint32_t ngrp,
+                 float* y, int32_t* dump) {
+    if (dump) gemm_i8_q4m_kernel<RT, TT, PH, true><<<grid, 256, 0, s>>>(w, f, x2, f1, t, ngrp, y, dump);
+    else gemm_i8_q4m_kernel<RT, TT, PH, false><<<grid, 256, 0, s>>>(w, f, x2, f1, t, ngrp, y, dump);
+}
 
 }  // namespace
 
-// Token slots (a multiple of the kernel's token tile count x 16) and column groups the packed activations hold.
+// Token slots (a multiple of the picked tile's tokens) and column groups the packed activations hold.
 void gemm_i8_geometry(const WeightView& w, size_t t, size_t* slots, size_t* ngrp) {
-    const size_t tt = tt_for(t), ttiles = ((t + 15) / 16 + tt - 1) / tt * tt;
-    *slots = ttiles * 16;
+    const uint32_t ttiles = (uint32_t)((t + 15) / 16);
+    const Tile& c = TILES[pick_tile(row_tiles(w.n_out), ttiles)];
+    *slots = (size_t)((ttiles + c.tt - 1) / c.tt) * c.tt * 16;
     *ngrp = 2 * (size_t)t4m_steps(w.n_in);
 }
 
 uint32_t gemm_i8_k_slices(const WeightView& w, size_t t) {
-    size_t slots, ngrp;
-    gemm_i8_geometry(w, t, &slots, &ngrp);
-    const size_t waves = (size_t)((row_tiles(w.n_out) + 7) / 8) * 4 * (slots / 16 / tt_for(t));
+    const uint32_t ttiles = (uint32_t)((t + 15) / 16);
+    const Tile& c = TILES[pick_tile(row_tiles(w.n_out), ttiles)];
+    const size_t waves = (size_t)((row_tiles(w.n_out) + c.rt - 1) / c.rt) * ((ttiles + c.tt - 1) / c.tt);
     const uint32_t steps = t4m_steps(w.n_in);
     uint32_t z = 1;
-    while (z < 8 && waves * z < 2048 && steps / (z * 2) >= 4) z *= 2;
+    while (z < 8 && waves * z < 1024 && steps / (z * 2) >= 4) z *= 2;
     return z;
 }
 
@@ -282,17 +326,19 @@ hipError_t launch_gemm_i8(const WeightView& w, const void* frag, const void* xs,
     if (w.fmt != FMT_Q4M) return hipErrorInvalidValue;
     size_t slots, ngrp;
     gemm_i8_geometry(w, t, &slots, &ngrp);
-    const uint32_t tt = tt_for(t);
-    dim3 grid((row_tiles(w.n_out) + 7) / 8, (unsigned)(slots / 16 / tt), gemm_i8_k_slices(w, t));
+    const uint32_t ttiles = (uint32_t)((t + 15) / 16);
+    const int pick = pick_tile(row_tiles(w.n_out), ttiles);
+    const Tile& c = TILES[pick];
+    const uint32_t wrt = (row_tiles(w.n_out) + c.rt - 1) / c.rt;
+    dim3 grid((wrt + 3) / 4, (unsigned)(slots / 16 / c.tt), gemm_i8_k_slices(w, t));
     const uint4* f = static_cast<const uint4*>(frag);
     const float2* x2 = static_cast<const float2*>(xs);
     const float* f1 = static_cast<const float*>(fs);
-    if (tt == 4) {
-        if (dump) gemm_i8_q4m_kernel<4, true><<<grid, 256, 0, s>>>(w, f, x2, f1, (uint32_t)t, (uint32_t)ngrp, y, dump);
-        else gemm_i8_q4m_kernel<4, false><<<grid, 256, 0, s>>>(w, f, x2, f1, (uint32_t)t, (uint32_t)ngrp, y, dump);
-    } else {
-        if (dump) gemm_i8_q4m_kernel<8, true><<<grid, 256, 0, s>>>(w, f, x2, f1, (uint32_t)t, (uint32_t)ngrp, y, dump);
-        else gemm_i8_q4m_kernel<8, false><<<grid, 256, 0, s>>>(w, f, x2, f1, (uint32_t)t, (uint32_t)ngrp, y, dump);
+    const uint32_t tt = (uint32_t)t, ng = (uint32_t)ngrp;
+    switch (pick) {
+        case 0: launch_tile<2, 8, 2>(grid, s, w, f, x2, f1, tt, ng, y, dump); break;
+        case 1: launch_tile<2, 4, 1>(grid, s, w, f, x2, f1, tt, ng, y, dump); break;
+        default: launch_tile<2, 2, 1>(grid, s, w, f, x2, f1, tt, ng, y, dump); break;
     }
     return hipGetLastError();
 }
