@@ -73,8 +73,22 @@ int oxhip_open(int device, oxhip_ctx** out) {
     auto* c = new oxhip_ctx();
     c->device = device;
     c->name = "hip (" + arch + ")";
+    // 16 MiB of partial rows (32 slices x 8 tokens x 16384 outputs) and 16384 counters, zero between launches
+    c->dec.partial_floats = (size_t)4 << 20;
+    c->dec.ncounters = 16384;
+    if (hipMalloc(reinterpret_cast<void**>(&c->dec.partial), c->dec.partial_floats * 4) != hipSuccess ||
+        hipMalloc(reinterpret_cast<void**>(&c->dec.counters), c->dec.ncounters * 4) != hipSuccess ||
+        hipMemset(c->dec.counters, 0, c->dec.ncounters * 4) != hipSuccess) {
+        set_error("decode scratch allocation failed");
+        if (c->dec.partial) (void)hipFree(c->dec.partial);
+        if (c->dec.counters) (void)hipFree(c->dec.counters);
+        delete c;
+        return 0;
+    }
     if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess) {
         set_error("hipStreamCreate failed");
+        (void)hipFree(c->dec.partial);
+        (void)hipFree(c->dec.counters);
         delete c;
         return 0;
     }
@@ -89,6 +103,9 @@ void oxhip_close(oxhip_ctx* c) {
     c->x.release();
     c->xq.release();
     c->y.release();
+    c->gemm_ws.release();
+    (void)hipFree(c->dec.partial);
+    (void)hipFree(c->dec.counters);
     (void)hipStreamDestroy(c->stream);
     delete c;
 }
@@ -337,7 +354,7 @@ int oxhip_dev_decode(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa, 
         }
         v = view_of(*xa);
     }
-    HIP_TRY(launch_decode(w->v, v, x, t, y, static_cast<hipStream_t>(stream)), "decode launch");
+    HIP_TRY(launch_decode(w->v, v, x, t, y, static_cast<hipStream_t>(stream), c->dec), "decode launch");
     return 1;
 }
 
@@ -445,7 +462,7 @@ int oxhip_matmul(oxhip_ctx* c, const float* x, size_t t, size_t n_in, oxhip_job*
     size_t off = 0;
     for (size_t j = 0; j < n_jobs; j++) {
         const oxhip_weight* w = jobs[j].w;
-        if (launch_decode(w->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off, s) != hipSuccess) {
+        if (launch_decode(w->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off, s, c->dec) != hipSuccess) {
             set_error("matmul: decode launch failed");
             (void)hipStreamSynchronize(s);
             return done(0);

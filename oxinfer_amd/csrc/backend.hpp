@@ -60,6 +60,7 @@ struct oxhip_ctx {
     std::mutex mu;  // serializes the host-pointer surface (staging is shared), as Mutex<Staging> does
     oxhip::DevBuf x, xq, y;
     oxhip::DevBuf gemm_ws;  // packed activations of the prefill GEMMs
+    oxhip::DecodeScratch dec;  // partial rows and counters of the decode kernels that split K across workgroups
     double ms_in = 0, ms_gpu = 0, ms_out = 0;
     size_t calls = 0;
 };

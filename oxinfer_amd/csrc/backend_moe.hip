@@ -282,9 +282,9 @@ int oxhip_matvec_rows(oxhip_ctx* c, const float* x, size_t t, size_t n_in, oxhip
         const oxhip_rows_job& jb = jobs[j];
         const size_t n = t * jb.n_out;
         at[j] = off;
-        HIP_TRY(launch_decode(jb.w->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off, s), "decode launch");
+        HIP_TRY(launch_decode(jb.w->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off, s, c->dec), "decode launch");
         if (jb.up) {
-            HIP_TRY(launch_decode(jb.up->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off + n, s), "decode launch");
+            HIP_TRY(launch_decode(jb.up->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off + n, s, c->dec), "decode launch");
             HIP_TRY(launch_moe_act(yd + off, yd + off + n, jb.n_out, t, jb.n_out, OXHIP_ACT_SILU, 0.0f, yd + off, s), "act launch");
         }
         off += n * (jb.up ? 2 : 1);

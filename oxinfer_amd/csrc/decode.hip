@@ -332,11 +332,12 @@ hipError_t decode_dense_t(const WeightView& w, const float* x, size_t t, float* 
 
 }  // namespace
 
-hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s) {
+hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s,
+                         const DecodeScratch& sc) {
     switch (w.fmt) {
         case FMT_Q8_0:
         case FMT_Q4_K:
-        case FMT_Q4M: return launch_decode_mfma(w, xa, t, y, s);
+        case FMT_Q4M: return launch_decode_mfma(w, xa, t, y, sc, s);
         case FMT_Q4: return decode_t<FMT_Q4, 4>(w, xa, t, y, s);
         case FMT_Q6_K: return decode_t<FMT_Q6_K, 4>(w, xa, t, y, s);
         case FMT_FP8: return decode_dense_t<FMT_FP8, 4>(w, x, t, y, s);

@@ -22,9 +22,16 @@
 // scales and sums transposed so that a lane reads the four tokens it owns with one ds_read_b128.
 // Rows too long for LDS fall back to reading the int8 values from L2.
 //
-// A workgroup owns `rt` row tiles and splits K over `kw` waves per tile; the partial sums meet in
-// LDS in a fixed order. No atomics, no second launch.
+// A workgroup owns `rt` row tiles over one of `ksplit` slices of K (grid y) and splits its slice over `kw` waves
+// per tile; the waves' partial sums meet in LDS in a fixed order. With more than one slice each workgroup leaves
+// its partial rows in global scratch and the last one to arrive (a counter per row group) adds the slices in slice
+// order: the association of a row's sum depends on the weight's shape only, never on arrival order, and there is
+// no second launch. A workgroup stages only its slice of the activations.
+#include <atomic>
+#include <cstdio>
 #include <cstdlib>
+#include <map>
+#include <mutex>
 
 #include "internal.hpp"
 #include "layout.hpp"
@@ -38,7 +45,7 @@ namespace {
 // Records a wave keeps in flight. HBM delivers about 8 TB/s at about 2 us of loaded latency, so some 16 MB must be
 // on request across the chip at any moment: about 4000 resident waves x PF KiB.
 template <int FMT, int NT>
-constexpr int pf_for() { return FMT == FMT_Q4_K ? 6 : 8; }
+constexpr int pf_for() { return 8; }
 
 struct Meta4 {
     float xs[4];
@@ -53,29 +60,8 @@ struct Meta4 {
 //   MLX:   d * (xs * U + c) + off * fs,              c = -8 * xs * su
 // which equal the reference's (s * xs) * (U - 8 su) + m * fs (src/ggml.rs:1288-1315, src/kernels.rs:1287-1297)
 // up to f32 rounding; the integer sums U - 8 su themselves are exact (and are what the DUMP variant writes).
-// LDS: xs | c | fs | su, each [nblk][TPAD] (c, fs only for the formats with sums; su only for DUMP)
-template <int FMT, int TPAD, bool SUMS, bool DUMP, class RowOf>
-__device__ __forceinline__ void stage_meta(const QActView& xa, uint32_t t, uint32_t nblk, float* lds, RowOf row_of) {
-    float* xs = lds;
-    float* cc = lds + (size_t)nblk * TPAD;
-    float* fs = lds + (size_t)2 * nblk * TPAD;
-    int* su = reinterpret_cast<int*>(lds + (size_t)3 * nblk * TPAD);
-    for (uint32_t i = threadIdx.x; i < nblk * TPAD; i += blockDim.x) {
-        uint32_t tok = i / nblk, b = i % nblk;  // consecutive threads read consecutive blocks of one token
-        bool live = tok < t;
-        size_t src = (live ? row_of(tok) : 0) * nblk + b;
-        const float x = live ? xa.scales[src] : 0.0f;
-        xs[b * TPAD + tok] = x;
-        if (SUMS) {
-            const int sq = live ? xa.sums[src] : 0;
-            const float f = live ? xa.fsums[src] : 0.0f;
-            cc[b * TPAD + tok] = FMT == FMT_Q4_K ? 8.0f * (f - x * (float)sq) : -8.0f * (x * (float)sq);
-            fs[b * TPAD + tok] = f;
-            if (DUMP) su[b * TPAD + tok] = sq;
-        }
-    }
-}
-
+// LDS: xs | c | fs | su, each [nbl][TPAD] over the workgroup's nbl blocks from b0 (c, fs only for the formats with
+// sums; su only for DUMP)
 template <int TPAD, bool SUMS, bool DUMP>
 __device__ __forceinline__ void load_meta(const float* lds, uint32_t nblk, uint32_t b, uint32_t tok0, Meta4& m) {
     const float4 x = *reinterpret_cast<const float4*>(lds + (size_t)b * TPAD + tok0);
@@ -126,23 +112,35 @@ struct Step<FMT_Q4M> {
 // ALDS: the int8 activations are staged into LDS in operand order (the launcher checks that they fit).
 template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS>
 __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw,
-                                                           float* __restrict__ y, int32_t* __restrict__ dump, GroupView grp) {
+                                                           float* __restrict__ y, int32_t* __restrict__ dump, GroupView grp,
+                                                           uint32_t ksplit, float* __restrict__ partial,
+                                                           uint32_t* __restrict__ counters) {
     constexpr int TPAD = NT <= 4 ? 4 : 8;
     constexpr int NI = NT < 4 ? NT : 4;          // accumulator registers that hold live tokens
     constexpr bool SUMS = FMT != FMT_Q8_0;
-    extern __shared__ float lds_all[];
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // 16-byte aligned whatever static LDS the kernel also holds: the 8- and 16-byte LDS reads below are split into
+    // dwords (and the kernel runs two to three times longer) when this array starts at an odd dword
+    extern __shared__ __align__(16) float lds_all[];
+    // the wave index and everything derived from it (tile, K range) live in scalar registers: branches on them are
+    // scalar, and the load counters the compiler keeps stay exact across them
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t n = lane & 15, kq = lane >> 4;  // B / D role: row n of the tile; A role: slot n
     const uint32_t nblk = w.n_in / 32;
     const uint32_t r = wave / kw, ks = wave % kw;
     const uint32_t tile = blockIdx.x * rt + r;
     const uint32_t ntiles = row_tiles(w.n_out);
+    // this workgroup's slice of K: steps [S0, S1), blocks [B0, B0 + nbl) (a multiple of 4 blocks)
+    constexpr uint32_t BPS = FMT == FMT_Q8_0 ? 2 : 4;  // blocks of 32 per step
+    const uint32_t nsteps = FMT == FMT_Q8_0 ? t8_steps(w.n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in) : t4m_steps(w.n_in));
+    const uint32_t slice = GROUPED ? 0 : blockIdx.y;
+    const uint32_t sl = (nsteps + ksplit - 1) / ksplit;
+    const uint32_t S0 = min(nsteps, slice * sl), S1 = min(nsteps, S0 + sl);
+    const uint32_t B0 = BPS * S0, nbl = BPS * sl, M0 = B0 / 2;
     // LDS: [operand-order activations: 512 B per pair of blocks] [scales, sums] [partial sums]; with ALDS the
     // partial sums reuse the activations' space once every wave is done with them
-    const uint32_t nmf = (nblk + 1) / 2;
     uint2* afr = reinterpret_cast<uint2*>(lds_all);
-    float* lds = lds_all + (ALDS ? (size_t)nmf * 128 : 0);
-    float* red = ALDS ? lds_all : lds + (size_t)(SUMS ? (DUMP ? 4 : 3) : 1) * nblk * TPAD;  // [rt * kw][TPAD][16]
+    float* lds = lds_all + (ALDS ? (size_t)(nbl / 2) * 128 : 0);
+    float* red = ALDS ? lds_all : lds + (size_t)(SUMS ? (DUMP ? 4 : 3) : 1) * nbl * TPAD;  // [rt * kw][TPAD][16]
     uint32_t row0 = 0;  // first activation / output row of this launch unit
     if (GROUPED) {
         if (blockIdx.y >= (uint32_t)*grp.nchunks) return;  // uniform over the workgroup
@@ -161,10 +159,9 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
     // D role: this lane's registers are tokens 4 (kq & 1) + i of block parity kq >> 1
     const uint32_t d_half = kq >> 1, d_tok0 = 4 * (kq & 1);
 
-    const uint32_t nsteps = FMT == FMT_Q8_0 ? t8_steps(w.n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in) : t4m_steps(w.n_in));
-    const uint32_t per = (nsteps + kw - 1) / kw;
-    const uint32_t s0 = ks * per;
-    const uint32_t s1 = tile < ntiles ? min(nsteps, s0 + per) : 0;  // a tile past the matrix streams nothing
+    const uint32_t per = (S1 - S0 + kw - 1) / kw;
+    const uint32_t s0 = S0 + ks * per;
+    const uint32_t s1 = tile < ntiles ? min(S1, s0 + per) : 0;  // a tile past the matrix streams nothing
     const uint8_t* base = w.p0 + (size_t)min(tile, ntiles - 1) * (FMT == FMT_Q8_0   ? (size_t)nsteps * T8_REC
                                                                   : FMT == FMT_Q4_K ? (size_t)(nsteps / 2) * TK4_REC
                                                                                     : (size_t)nsteps * T4M_REC);
@@ -211,7 +208,7 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
     // `m`: index of the instruction along K (pair of blocks 2 m, 2 m + 1); with ALDS its operand comes from LDS
     auto mfma = [&](v4i bw, uint32_t m, uint32_t d0, uint32_t d1) -> v4i {
         if (ALDS) {
-            const uint2 av = afr[(size_t)m * 64 + lane];
+            const uint2 av = afr[(size_t)(m - M0) * 64 + lane];
             d0 = av.x;
             d1 = av.y;
         }
@@ -235,7 +232,7 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
             v4i D = mfma(bw, s, st.a[0], st.a[1]);
             const uint32_t b = 2 * s + d_half;
             Meta4 m;
-            load_meta<TPAD, SUMS, DUMP>(lds, nblk, min(b, nblk - 1), d_tok0, m);
+            load_meta<TPAD, SUMS, DUMP>(lds, nbl, min(b, nblk - 1) - B0, d_tok0, m);
             int isum[4] = {D.x, D.y, D.z, D.w};
 #pragma unroll
             for (int i = 0; i < NI; i++) acc[i] = fmaf(d, m.xs[i] * (float)isum[i], acc[i]);
@@ -253,7 +250,7 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
                 const uint32_t q = 2 * pr + d_half;
                 const float sc = (float)((st.sc4 >> (8 * q)) & 0xFF), mn = (float)((st.mn4 >> (8 * q)) & 0xFF);
                 Meta4 m;
-                load_meta<TPAD, SUMS, DUMP>(lds, nblk, b, d_tok0, m);
+                load_meta<TPAD, SUMS, DUMP>(lds, nbl, b - B0, d_tok0, m);
                 const int U[4] = {D.x, D.y, D.z, D.w};
 #pragma unroll
                 for (int i = 0; i < NI; i++) {
@@ -278,7 +275,7 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
                 const float d = f16_bits_to_f32((uint16_t)(g ? st.dd >> 16 : st.dd & 0xFFFF));
                 const float off = bf16_bits_to_f32((uint16_t)(g ? st.oo >> 16 : st.oo & 0xFFFF));
                 Meta4 m;
-                load_meta<TPAD, SUMS, DUMP>(lds, nblk, min(b, nblk - 1), d_tok0, m);
+                load_meta<TPAD, SUMS, DUMP>(lds, nbl, min(b, nblk - 1) - B0, d_tok0, m);
                 const int U[4] = {D.x, D.y, D.z, D.w};
                 if (b < nblk) {  // padding blocks hold zero codes and zero scales, but their staged sums are a real block's
 #pragma unroll
@@ -292,39 +289,102 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
         }
     };
 
-    // The first ring of records is requested before anything else, so that HBM latency overlaps the
-    // staging of the activation scales.
+    // Order of the requests: a wave's loads return in order, so the activations and their scales (L2 hits, needed by
+    // every step) are requested first, into registers; then the first ring of weight records (HBM); then the staged
+    // values go to LDS while the weights are still on their way. Requested after the weights, the activations would
+    // only arrive behind them and no step could start before the whole ring had landed.
     constexpr int PF = pf_for<FMT, NT>();
-    Step<FMT> ring[PF];
-#pragma unroll
-    for (int p = 0; p < PF; p++)
-        if (s0 + p < s1) load_step(ring[p], s0 + p);
-    stage_meta<FMT, TPAD, SUMS, DUMP>(xa, t, nblk, lds, src_row);
-    if (ALDS) {
-        // slot (m, lane) of the operand array: lane = 16 kq + 8 half + token holds the 8 values of block 2 m + half
-        // that the weights' lane group kq pairs with (Q4: positions 4 kq.. and 16 + 4 kq..; else 8 kq..). A thread
-        // moves 16 (Q4: 32) consecutive bytes of one token's row, so the global reads are whole lines. Absent tokens
-        // and a padding block keep whatever LDS holds: those products meet zero weights or are dropped.
+    constexpr int SA = 8, SM = 4;  // 16-byte activation chunks / scale entries a thread holds in registers; more go later
+    const uint32_t nb = min(nblk, B0 + nbl) - min(nblk, B0);  // real blocks of the slice
+    // slot (m, lane) of the operand array: lane = 16 kq + 8 half + token holds the 8 values of block 2 m + half that
+    // the weights' lane group kq pairs with (Q4: positions 4 kq.. and 16 + 4 kq..; else 8 kq..). A thread moves 16
+    // (Q4: 32) consecutive bytes of one token's row, so the global reads are whole lines. Absent tokens and a padding
+    // block keep whatever LDS holds: those products meet zero weights or are dropped.
+    constexpr int AU = FMT == FMT_Q4M ? 2 : 1;  // 16-byte loads per unit of staging work
+    const uint32_t na = ALDS ? t * nb * (FMT == FMT_Q4M ? 1 : 2) : 0;
+    auto act_load = [&](uint32_t i, uint4* v) {
         if (FMT == FMT_Q4M) {
-            for (uint32_t i = threadIdx.x; i < t * nblk; i += blockDim.x) {
-                const uint32_t tok = i / nblk, b = i % nblk;
-                const uint4* xb = reinterpret_cast<const uint4*>(xa.q + src_row(tok) * w.n_in + (size_t)b * 32);
-                const uint4 lo = xb[0], hi = xb[1];
-                uint2* dst = afr + (size_t)(b >> 1) * 64 + 8 * (b & 1) + tok;
-                dst[0] = make_uint2(lo.x, hi.x);
-                dst[16] = make_uint2(lo.y, hi.y);
-                dst[32] = make_uint2(lo.z, hi.z);
-                dst[48] = make_uint2(lo.w, hi.w);
-            }
+            const uint32_t tok = i / nb, b = i % nb;  // b: block within the slice
+            const uint4* xb = reinterpret_cast<const uint4*>(xa.q + src_row(tok) * w.n_in + (size_t)(B0 + b) * 32);
+            v[0] = xb[0];
+            v[1] = xb[1];
         } else {
-            for (uint32_t i = threadIdx.x; i < t * 2 * nblk; i += blockDim.x) {
-                const uint32_t tok = i / (2 * nblk), c = i % (2 * nblk), b = c >> 1;
-                const uint4 v = *reinterpret_cast<const uint4*>(xa.q + src_row(tok) * w.n_in + (size_t)c * 16);
-                uint2* dst = afr + (size_t)(b >> 1) * 64 + 32 * (c & 1) + 8 * (b & 1) + tok;
-                dst[0] = make_uint2(v.x, v.y);
-                dst[16] = make_uint2(v.z, v.w);
-            }
+            const uint32_t tok = i / (2 * nb), c = i % (2 * nb);
+            v[0] = *reinterpret_cast<const uint4*>(xa.q + src_row(tok) * w.n_in + (size_t)B0 * 32 + (size_t)c * 16);
         }
+    };
+    auto act_store = [&](uint32_t i, const uint4* v) {
+        if (FMT == FMT_Q4M) {
+            const uint32_t tok = i / nb, b = i % nb;
+            uint2* dst = afr + (size_t)(b >> 1) * 64 + 8 * (b & 1) + tok;
+            dst[0] = make_uint2(v[0].x, v[1].x);
+            dst[16] = make_uint2(v[0].y, v[1].y);
+            dst[32] = make_uint2(v[0].z, v[1].z);
+            dst[48] = make_uint2(v[0].w, v[1].w);
+        } else {
+            const uint32_t tok = i / (2 * nb), c = i % (2 * nb), b = c >> 1;
+            uint2* dst = afr + (size_t)(b >> 1) * 64 + 32 * (c & 1) + 8 * (b & 1) + tok;
+            dst[0] = make_uint2(v[0].x, v[0].y);
+            dst[16] = make_uint2(v[0].z, v[0].w);
+        }
+    };
+    // scales and sums: entry i = (token i / nbl, block i % nbl of the slice), see stage_meta's layout
+    struct MetaReg {
+        float x, f;
+        int sq;
+    };
+    const uint32_t nm = nbl * TPAD;
+    auto meta_load = [&](uint32_t i, MetaReg& r) {
+        const uint32_t tok = i / nbl, b = i % nbl;  // consecutive threads read consecutive blocks of one token
+        const bool live = tok < t && B0 + b < nblk;
+        const size_t src = (live ? src_row(tok) : 0) * nblk + B0 + (live ? b : 0);
+        r.x = live ? xa.scales[src] : 0.0f;
+        r.sq = SUMS && live ? xa.sums[src] : 0;
+        r.f = SUMS && live ? xa.fsums[src] : 0.0f;
+    };
+    auto meta_store = [&](uint32_t i, const MetaReg& r) {
+        const uint32_t tok = i / nbl, b = i % nbl;
+        lds[b * TPAD + tok] = r.x;
+        if (SUMS) {
+            lds[(size_t)nm + b * TPAD + tok] = FMT == FMT_Q4_K ? 8.0f * (r.f - r.x * (float)r.sq) : -8.0f * (r.x * (float)r.sq);
+            lds[(size_t)2 * nm + b * TPAD + tok] = r.f;
+            if (DUMP) reinterpret_cast<int*>(lds)[(size_t)3 * nm + b * TPAD + tok] = r.sq;
+        }
+    };
+    uint4 sa[SA];
+    MetaReg smr[SM];
+    // (every request below is issued by every lane, with its index clamped into range, so that the waits can be
+    // counted exactly; the extra requests hit lines that are being fetched anyway)
+    if (ALDS) {
+#pragma unroll
+        for (int j = 0; j < SA / AU; j++) act_load(min(threadIdx.x + j * blockDim.x, na - 1), sa + AU * j);
+    }
+#pragma unroll
+    for (int j = 0; j < SM; j++) meta_load(min(threadIdx.x + j * blockDim.x, nm - 1), smr[j]);
+    Step<FMT> ring[PF];
+    const uint32_t slast = max(s1, 1u) - 1;
+#pragma unroll
+    for (int p = 0; p < PF; p++) load_step(ring[p], min(s0 + p, slast));
+#pragma unroll
+    for (int j = 0; j < SA / AU; j++) {
+        const uint32_t i = threadIdx.x + j * blockDim.x;
+        if (i < na) act_store(i, sa + AU * j);
+    }
+#pragma unroll
+    for (int j = 0; j < SM; j++) {
+        const uint32_t i = threadIdx.x + j * blockDim.x;
+        if (i < nm) meta_store(i, smr[j]);
+    }
+    // what did not fit the registers (long rows, small workgroups) follows behind the weights
+    for (uint32_t i = threadIdx.x + (SA / AU) * blockDim.x; i < na; i += blockDim.x) {
+        uint4 v[AU];
+        act_load(i, v);
+        act_store(i, v);
+    }
+    for (uint32_t i = threadIdx.x + SM * blockDim.x; i < nm; i += blockDim.x) {
+        MetaReg r;
+        meta_load(i, r);
+        meta_store(i, r);
     }
     __syncthreads();
     // each slot is refilled as soon as its record has been consumed, so PF - 1 records stay on request
@@ -345,13 +405,39 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
             if (d_tok0 + i < (uint32_t)TPAD) red[((size_t)wave * TPAD + d_tok0 + i) * 16 + n] = acc[i];
     }
     __syncthreads();
-    // K-slices in order
+    // the waves of a tile in order; with one slice that is the result, else this slice's partial rows
+    float* out = ksplit > 1 ? partial + (size_t)slice * t * w.n_out : y;
     for (uint32_t idx = threadIdx.x; idx < rt * TPAD * 16; idx += blockDim.x) {
         const uint32_t rr = idx / (TPAD * 16), tok = (idx / 16) % TPAD, nn = idx % 16;
         const uint32_t row = (blockIdx.x * rt + rr) * 16 + nn;
         if (tok >= t || row >= w.n_out || !y) continue;
         float sum = 0.0f;
         for (uint32_t k = 0; k < kw; k++) sum += red[((size_t)(rr * kw + k) * TPAD + tok) * 16 + nn];
+        // partial rows go out as device-scope stores (written through to memory, where the other XCDs' L2s see them)
+        if (ksplit > 1) __hip_atomic_store(out + (size_t)tok * w.n_out + row, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else out[(size_t)tok * w.n_out + row] = sum;
+    }
+    if (GROUPED || ksplit == 1 || !y) return;  // uniform over the workgroup
+    // The last workgroup of this row group to get here adds the slices in slice order; the counter returns to zero
+    // for the next launch. Every access to the partial rows and the counter is a device-scope atomic access, and each
+    // thread waits for its stores to complete before the workgroup's arrival is counted, so no cache-wide write-back
+    // or invalidation is needed (a device-scope fence here costs tens of microseconds per launch).
+    __shared__ uint32_t is_last;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t seen = __hip_atomic_fetch_add(&counters[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = seen == ksplit - 1;
+        if (seen == ksplit - 1) __hip_atomic_store(&counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!is_last) return;
+    for (uint32_t idx = threadIdx.x; idx < rt * 16 * t; idx += blockDim.x) {
+        const uint32_t tok = idx / (rt * 16), row = blockIdx.x * rt * 16 + idx % (rt * 16);
+        if (row >= w.n_out) continue;
+        const float* p = partial + (size_t)tok * w.n_out + row;
+        float sum = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (uint32_t z = 1; z < ksplit; z++) sum += __hip_atomic_load(p + (size_t)z * t * w.n_out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         y[(size_t)tok * w.n_out + row] = sum;
     }
 }
@@ -359,63 +445,107 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
 namespace {
 
 struct Shape {
-    uint32_t rt, kw;
+    uint32_t rt, kw, ks;
 };
 
-// Waves per workgroup (rt row tiles x kw K slices, 16 waves when the matrix allows) and how they split. A function
-// of the weight's shape only, so a row's sum is associated the same way whatever the batch or launch kind.
-// K is split as far as each wave keeps about four records; then row tiles are added per workgroup until the
-// workgroups fit the chip at once (256 CUs, one 16-wave workgroup each), so that the whole matrix is on request
-// from the first microsecond instead of in successive generations of workgroups.
-Shape shape_for(uint32_t ntiles, uint32_t nsteps) {
-    uint32_t kw = 1;
-    while (kw < 16 && nsteps / (kw * 2) >= 4) kw *= 2;
-    uint32_t rt = 16 / kw;
-    while (kw > 1 && (ntiles + rt - 1) / rt > 256) {
-        kw /= 2;
-        rt *= 2;
+constexpr uint32_t NCU = 256;
+
+// Workgroup shape (rt row tiles x kw waves per tile, at most 16 waves) and the number of K slices across workgroups:
+// a function of the weight's shape only, so a row's sum is associated the same way whatever the batch. The pick
+// minimizes the work of the busiest CU when the workgroups are dealt out one per CU per generation (the whole matrix
+// should be on request from the first microsecond), then prefers enough waves to cover HBM latency, a few records
+// per wave, and few slices. 896 row tiles, for one, run as 128 groups of 7 tiles x 2 slices = 256 workgroups.
+Shape search_shape(uint32_t ntiles, uint32_t nsteps, bool allow_slices) {
+    Shape best{1, 1, 1};
+    double best_cost = 1e300;
+    for (uint32_t kw = 1; kw <= 16; kw *= 2)
+        for (uint32_t rt = 1; rt * kw <= 16; rt++)
+            for (uint32_t ks = 1; ks <= (allow_slices ? 32u : 1u); ks *= 2) {
+                if (ks > 1 && (nsteps + ks - 1) / ks * (ks - 1) >= nsteps) continue;  // an empty slice
+                const uint32_t sl = (nsteps + ks - 1) / ks, per = (sl + kw - 1) / kw;
+                const uint64_t wgs = (uint64_t)((ntiles + rt - 1) / rt) * ks;
+                const uint64_t gens = (wgs + NCU - 1) / NCU;
+                double cost = (double)gens * rt * per * kw;  // records through the busiest CU
+                const uint32_t waves = rt * kw;
+                if (waves < 8) cost *= 1.0 + 0.08 * (8 - waves);
+                if (per < 4) cost *= 1.0 + 0.10 * (4 - per);
+                if (ks > 1) cost *= 1.15 + 0.01 * ks;  // the last-arrival pass costs about 1.5 us of dependent round trips
+                cost *= 1.0 + 0.002 * kw;
+                if (cost < best_cost) {
+                    best_cost = cost;
+                    best = Shape{rt, kw, ks};
+                }
+            }
+    if (const char* e = getenv("OXHIP_DECODE_SHAPE")) {  // developer override for tuning runs: "rt,kw,ks"
+        unsigned a = 0, b = 0, c = 0;
+        if (sscanf(e, "%u,%u,%u", &a, &b, &c) == 3 && a >= 1 && b >= 1 && c >= 1 && a * b <= 16 && (allow_slices || c == 1))
+            best = Shape{a, b, c};
     }
-    if (const char* e = getenv("OXHIP_DECODE_KW")) {  // developer override for tuning runs
-        uint32_t v = (uint32_t)atoi(e);
-        if (v == 1 || v == 2 || v == 4 || v == 8 || v == 16) {
-            kw = v;
-            rt = 16 / kw;
-        }
-    }
-    return Shape{rt, kw};
+    return best;
 }
 
-constexpr size_t LDS_MAX = 160 * 1024;
+// The search runs once per (shape, kind of launch): a decode launch is a few microseconds of GPU time and must not
+// spend as long on the host.
+Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices) {
+    static std::mutex mu;
+    static std::map<uint64_t, Shape> cache;
+    const uint64_t key = ((uint64_t)ntiles << 33) | ((uint64_t)nsteps << 1) | (allow_slices ? 1u : 0u);
+    std::lock_guard<std::mutex> g(mu);
+    auto it = cache.find(key);
+    if (it != cache.end()) return it->second;
+    const Shape sh = search_shape(ntiles, nsteps, allow_slices);
+    cache.emplace(key, sh);
+    return sh;
+}
+
+constexpr size_t LDS_MAX = 160 * 1024 - 256;  // dynamic LDS on offer (the kernel also holds a static word)
 
 // Dynamic LDS of a launch; `alds` comes back false when the operand-order activations do not fit.
-size_t lds_bytes(bool sums, bool dump, uint32_t nblk, int tpad, const Shape& sh, bool* alds) {
-    const size_t meta = (size_t)(sums ? (dump ? 4 : 3) : 1) * nblk * tpad * 4, red = (size_t)sh.rt * sh.kw * tpad * 16 * 4;
-    const size_t act = (size_t)((nblk + 1) / 2) * 512;
+size_t lds_bytes(bool sums, bool dump, uint32_t bps, uint32_t nsteps, int tpad, const Shape& sh, bool* alds) {
+    const uint32_t nbl = bps * ((nsteps + sh.ks - 1) / sh.ks);  // blocks of a slice
+    const size_t meta = (size_t)(sums ? (dump ? 4 : 3) : 1) * nbl * tpad * 4, red = (size_t)sh.rt * sh.kw * tpad * 16 * 4;
+    const size_t act = (size_t)(nbl / 2) * 512;
     const size_t with = act + meta > red ? act + meta : red;  // the partial sums reuse the activations' space
-    *alds = with <= LDS_MAX && act >= red;
+    *alds = with <= LDS_MAX;
     return *alds ? with : meta + red;
 }
 
 template <int FMT, int NT, bool DUMP, bool GROUPED>
 hipError_t launch_one(bool alds, dim3 grid, dim3 block, size_t lds, hipStream_t s, const WeightView& w, const QActView& v, uint32_t t,
-                      const Shape& sh, float* y, int32_t* dump, const GroupView& g) {
+                      const Shape& sh, float* y, int32_t* dump, const GroupView& g, const DecodeScratch& sc) {
     hipError_t e = hipSuccess;
     auto go = [&](auto kern) {
-        if (lds > 48 * 1024) e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, v, t, sh.rt, sh.kw, y, dump, g);
+        // once per kernel and device: allow the whole LDS
+        static std::atomic<uint64_t> allowed[4];  // one bit per device
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        const uint64_t bit = 1ull << (dev & 63);
+        if (lds > 48 * 1024 && !(allowed[(dev >> 6) & 3].load(std::memory_order_acquire) & bit)) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
+            if (e == hipSuccess) allowed[(dev >> 6) & 3].fetch_or(bit, std::memory_order_release);
+        }
+        if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, v, t, sh.rt, sh.kw, y, dump, g, sh.ks, sc.partial, sc.counters);
     };
     if (alds) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, true>);
     else go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, false>);
     return e != hipSuccess ? e : hipGetLastError();
 }
 
+template <int FMT>
+constexpr uint32_t steps_of(uint32_t n_in) {
+    return FMT == FMT_Q8_0 ? t8_steps(n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(n_in) : t4m_steps(n_in));
+}
+
 template <int FMT, bool DUMP>
-hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* dump, hipStream_t s) {
-    const uint32_t ntiles = row_tiles(w.n_out);
-    const uint32_t nsteps = FMT == FMT_Q8_0 ? t8_steps(w.n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in) : t4m_steps(w.n_in));
-    const Shape sh = shape_for(ntiles, nsteps);
+hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* dump, const DecodeScratch& sc, hipStream_t s) {
+    const uint32_t ntiles = row_tiles(w.n_out), nsteps = steps_of<FMT>(w.n_in);
+    Shape sh = shape_for(ntiles, nsteps, true);
+    const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
+    // slices need scratch: 8 token rows per slice and a counter per row group
+    if (sh.ks > 1 && (!sc.partial || !sc.counters || sc.partial_floats < (size_t)sh.ks * 8 * w.n_out || sc.ncounters < groups))
+        sh = shape_for(ntiles, nsteps, false);
     const uint32_t nblk = w.n_in / 32;
-    dim3 grid((ntiles + sh.rt - 1) / sh.rt), block(64 * sh.rt * sh.kw);
+    dim3 grid((ntiles + sh.rt - 1) / sh.rt, sh.ks), block(64 * sh.rt * sh.kw);
     size_t c0 = 0;
     while (c0 < t) {
         const size_t tc = t - c0 < 8 ? t - c0 : 8;
@@ -428,14 +558,14 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
         int32_t* du = dump ? dump + c0 * (size_t)w.n_out * nblk : nullptr;
         const int tpad = tc <= 4 ? 4 : 8;
         bool alds;
-        const size_t lds = lds_bytes(FMT != FMT_Q8_0, DUMP, nblk, tpad, sh, &alds);
+        const size_t lds = lds_bytes(FMT != FMT_Q8_0, DUMP, FMT == FMT_Q8_0 ? 2 : 4, nsteps, tpad, sh, &alds);
         if (lds > LDS_MAX) return hipErrorInvalidValue;  // rows too long for the staged activation scales
         const uint32_t tt = (uint32_t)tc;
         hipError_t e;
-        if (tc == 1) e = launch_one<FMT, 1, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{});
-        else if (tc == 2) e = launch_one<FMT, 2, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{});
-        else if (tc <= 4) e = launch_one<FMT, 4, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{});
-        else e = launch_one<FMT, 8, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{});
+        if (tc == 1) e = launch_one<FMT, 1, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
+        else if (tc == 2) e = launch_one<FMT, 2, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
+        else if (tc <= 4) e = launch_one<FMT, 4, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
+        else e = launch_one<FMT, 8, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
         if (e != hipSuccess) return e;
         c0 += tc;
     }
@@ -445,20 +575,19 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
 template <int FMT>
 hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks, uint32_t max_rows,
                        float* y, hipStream_t s) {
-    const uint32_t ntiles = row_tiles(w.n_out);
-    const uint32_t nsteps = FMT == FMT_Q8_0 ? t8_steps(w.n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in) : t4m_steps(w.n_in));
-    // the same K split as a plain launch on this matrix, so that a row's sum is associated the same way
-    // (and is bit-identical) whether its expert runs alone or in a group
-    const Shape sh = shape_for(ntiles, nsteps);
-    const uint32_t nblk = w.n_in / 32;
+    const uint32_t ntiles = row_tiles(w.n_out), nsteps = steps_of<FMT>(w.n_in);
+    // grid y walks the chunks: no K slices across workgroups here (the shape still depends on the weight alone, so a
+    // token's row is bit-identical whatever else is in the group)
+    const Shape sh = shape_for(ntiles, nsteps, false);
     dim3 grid((ntiles + sh.rt - 1) / sh.rt, max_chunks), block(64 * sh.rt * sh.kw);
     const int tpad = max_rows <= 4 ? 4 : 8;
     bool alds;
-    const size_t lds = lds_bytes(FMT != FMT_Q8_0, false, nblk, tpad, sh, &alds);
+    const size_t lds = lds_bytes(FMT != FMT_Q8_0, false, FMT == FMT_Q8_0 ? 2 : 4, nsteps, tpad, sh, &alds);
     if (lds > LDS_MAX) return hipErrorInvalidValue;
-    if (max_rows == 1) return launch_one<FMT, 1, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g);
-    if (max_rows <= 4) return launch_one<FMT, 4, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g);
-    return launch_one<FMT, 8, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g);
+    const DecodeScratch none{};
+    if (max_rows == 1) return launch_one<FMT, 1, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
+    if (max_rows <= 4) return launch_one<FMT, 4, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
+    return launch_one<FMT, 8, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
 }
 
 }  // namespace
@@ -474,11 +603,11 @@ hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, c
     }
 }
 
-hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, hipStream_t s) {
+hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, const DecodeScratch& sc, hipStream_t s) {
     switch (w.fmt) {
-        case FMT_Q8_0: return run<FMT_Q8_0, false>(w, xa, t, y, nullptr, s);
-        case FMT_Q4_K: return run<FMT_Q4_K, false>(w, xa, t, y, nullptr, s);
-        case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, s);
+        case FMT_Q8_0: return run<FMT_Q8_0, false>(w, xa, t, y, nullptr, sc, s);
+        case FMT_Q4_K: return run<FMT_Q4_K, false>(w, xa, t, y, nullptr, sc, s);
+        case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, sc, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -486,9 +615,9 @@ hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t,
 // The integer block sums the kernel forms ([t][n_out][n_in/32]); y is scratch of [t][n_out].
 hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* out, hipStream_t s) {
     switch (w.fmt) {
-        case FMT_Q8_0: return run<FMT_Q8_0, true>(w, xa, t, y, out, s);
-        case FMT_Q4_K: return run<FMT_Q4_K, true>(w, xa, t, y, out, s);
-        case FMT_Q4M: return run<FMT_Q4M, true>(w, xa, t, y, out, s);
+        case FMT_Q8_0: return run<FMT_Q8_0, true>(w, xa, t, y, out, DecodeScratch{}, s);
+        case FMT_Q4_K: return run<FMT_Q4_K, true>(w, xa, t, y, out, DecodeScratch{}, s);
+        case FMT_Q4M: return run<FMT_Q4M, true>(w, xa, t, y, out, DecodeScratch{}, s);
         default: return hipErrorInvalidValue;
     }
 }

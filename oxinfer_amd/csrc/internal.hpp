@@ -59,9 +59,18 @@ struct GroupView {
 // Launchers (each returns hipSuccess or the launch error).
 hipError_t launch_quantize_act(const float* x, size_t t, size_t n_in, const oxhip_qact& out, hipStream_t s);
 hipError_t launch_dequantize(const WeightView& w, size_t r0, size_t r1, float* out, hipStream_t s);
-hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s);
+// Global scratch of the decode kernels that split K across workgroups: `partial` holds slices x 8 token rows of
+// n_out floats, `counters` (zero between launches) one entry per group of row tiles. Launches that share a scratch
+// must be ordered on one stream. Without scratch the kernels keep K inside a workgroup.
+struct DecodeScratch {
+    float* partial = nullptr;
+    uint32_t* counters = nullptr;
+    size_t partial_floats = 0, ncounters = 0;
+};
+hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s,
+                         const DecodeScratch& sc = DecodeScratch{});
 hipError_t launch_isums(const WeightView& w, const QActView& xa, size_t t, int32_t* out, hipStream_t s);
-hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, hipStream_t s);
+hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, const DecodeScratch& sc, hipStream_t s);
 hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks,
                                       uint32_t max_rows_per_chunk, float* y, hipStream_t s);
 hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* out, hipStream_t s);
