@@ -33,7 +33,7 @@ KERNEL_FMT = {Q8_0: 1, Q4_K: 2, Q6_K: 3}  # template argument in the kernel symb
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # benchmark (KiB per dispatch, FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000: what a 256 MiB device copy
 # reads on the same counters); profiles/decode_mfma_gguf_gemv.md holds the summary.
-TRAFFIC_BYTES = {"decode_mfma_kernel<1, 8, false>": 63415984}
+TRAFFIC_BYTES = {}
 
 
 def weight_bytes(kind, n_out, n_in):
@@ -155,26 +155,33 @@ def main():
         c["pool"] = pools[(c["kind"], c["n_out"], c["n_in"])]
     torch.cuda.synchronize()
 
-    # the dominant kernel: the largest algorithmic bytes at the larger batch (same symbol for both shapes)
+    # The dominant kernel. Q8_0 / Q4_K jobs of one call share one launch (decode_batch_kernel): that launch is the
+    # step, and its events bracket it. Q6_K jobs launch one by one: there the largest matmul at the larger batch is
+    # timed (same symbol for both shapes).
+    shared = all(k in (Q8_0, Q4_K) for k in kinds)
     dom_kind = kinds[0]
     for c in cases:
-        c["dom"] = c["kind"] == dom_kind and c["t"] == 8
+        c["dom"] = shared or (c["kind"] == dom_kind and c["t"] == 8)
     dom = [c for c in cases if c["dom"]]
-    dom_symbol = (f"decode_mfma_kernel<{KERNEL_FMT[dom_kind]}, 8, false>" if dom_kind != Q6_K
-                  else f"decode_kernel<{KERNEL_FMT[dom_kind]}, 8, 4>")
+    per_step = 1 if shared else len(dom)
+    dom_symbol = "decode_batch_kernel" if shared else f"decode_kernel<{KERNEL_FMT[dom_kind]}, 8, 4>"
 
     # One call per step: the job arrays (one per rotation phase) are built once; the dominant launches carry
-    # HIP events recorded on the launch stream.
-    n_ev = args.steps * len(dom)
+    # HIP events recorded by the library on the launch stream.
+    n_ev = args.steps * per_step
     ev = [(be.event(), be.event()) for _ in range(min(n_ev, 4096))]
 
     def jobs_for(i, timed_slot=None):
         jobs, k = [], 0
-        for c in cases:
+        for n, c in enumerate(cases):
             w = c["pool"][(2 * i + (c["t"] > 1)) % len(c["pool"])]
             e0 = e1 = None
-            if timed_slot is not None and c["dom"]:
-                e0, e1 = ev[(timed_slot * len(dom) + k) % len(ev)]
+            if timed_slot is not None and shared:
+                pair = ev[timed_slot % len(ev)]
+                e0 = pair[0] if n == 0 else None
+                e1 = pair[1] if n == len(cases) - 1 else None
+            elif timed_slot is not None and c["dom"]:
+                e0, e1 = ev[(timed_slot * per_step + k) % len(ev)]
                 k += 1
             jobs.append((w, c["xa"], None, c["t"], c["y"], e0, e1))
         return be.decode_jobs(jobs)
@@ -195,7 +202,7 @@ def main():
     step_bytes = sum(c["bytes"] for c in cases)
     value = step_bytes * args.steps / elapsed / 1e9
     dom_avg_s = float(np.mean(dom_ms)) / 1e3
-    dom_bytes = float(np.mean([c["bytes"] for c in dom]))
+    dom_bytes = float(step_bytes) if shared else float(np.mean([c["bytes"] for c in dom]))
     achieved = dom_bytes / dom_avg_s / 1e9
 
     # per-case detail (untimed pass, one event pair per launch)
@@ -217,7 +224,7 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": "configs[1]: GGUF GEMV batch 1 and 8, Llama-8B MLP shapes 4096->14336 and 14336->4096, "
                                + " + ".join(FMT_NAME[k] for k in kinds),
-                   "launches_per_step": len(cases), "bytes_per_step": step_bytes,
+                   "matmuls_per_step": len(cases), "launches_per_step": 1 if shared else len(cases), "bytes_per_step": step_bytes,
                    "weight_pool_GB_per_shape": args.pool_gb, "activations": "int8 per 32 (quantize_act), resident in HBM"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES.get(dom_symbol), "kernel": dom_symbol,

@@ -2,6 +2,8 @@
 // reference) over the kernels of this library.
 #include "backend.hpp"
 
+#include <vector>
+
 namespace oxhip {
 
 static thread_local std::string g_err;
@@ -364,11 +366,38 @@ int oxhip_dev_decode_batch(oxhip_ctx* c, const oxhip_decode_job* jobs, size_t n_
         return 0;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    for (size_t j = 0; j < n_jobs; j++) {
+    // Runs of jobs that the matrix-core decode kernel takes share one launch; the others go out one by one.
+    auto fusable = [&](const oxhip_decode_job& jb) {
+        return jb.w && jb.xa && jb.y && !is_dense(jb.w) && jb.xa->n_in == jb.w->v.n_in && jb.xa->t >= jb.t && decode_batchable(jb.w->v, jb.t);
+    };
+    size_t j = 0;
+    std::vector<DecodeBatchItem> items;
+    while (j < n_jobs) {
+        size_t e = j;
+        while (e < n_jobs && fusable(jobs[e])) e++;
+        if (e - j >= 2) {
+            items.clear();
+            for (size_t k = j; k < e; k++) {
+                if (jobs[k].ev_start) HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jobs[k].ev_start), s), "event record");
+                items.push_back(DecodeBatchItem{jobs[k].w->v, view_of(*jobs[k].xa), jobs[k].y, (uint32_t)jobs[k].t});
+            }
+            const hipError_t err = launch_decode_mfma_batch(items.data(), items.size(), c->dec, s);
+            if (err == hipErrorOutOfMemory) {  // the scratch does not hold these jobs together: one launch each
+                for (size_t k = j; k < e; k++)
+                    if (!oxhip_dev_decode(c, jobs[k].w, jobs[k].xa, jobs[k].x, jobs[k].t, jobs[k].y, stream)) return 0;
+            } else {
+                HIP_TRY(err, "decode batch launch");
+            }
+            for (size_t k = j; k < e; k++)
+                if (jobs[k].ev_stop) HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jobs[k].ev_stop), s), "event record");
+            j = e;
+            continue;
+        }
         const oxhip_decode_job& jb = jobs[j];
         if (jb.ev_start) HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jb.ev_start), s), "event record");
         if (!oxhip_dev_decode(c, jb.w, jb.xa, jb.x, jb.t, jb.y, stream)) return 0;
         if (jb.ev_stop) HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jb.ev_stop), s), "event record");
+        j++;
     }
     return 1;
 }

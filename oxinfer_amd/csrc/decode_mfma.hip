@@ -32,6 +32,7 @@
 #include <cstdlib>
 #include <map>
 #include <mutex>
+#include <vector>
 
 #include "internal.hpp"
 #include "layout.hpp"
@@ -110,29 +111,28 @@ struct Step<FMT_Q4M> {
 // {expert, first row, rows (<= 8)}; the weights are expert's, activation row i of the chunk is row
 // rowmap[first + i] of xa (or first + i without a map), and its output is row first + i of y.
 // ALDS: the int8 activations are staged into LDS in operand order (the launcher checks that they fit).
+// `bx`, `by`: the workgroup's place in its launch unit (row group; K slice or chunk); `nthr` = 64 rt kw threads take
+// part (a launch may hold more: those waves have left before the first barrier); `lds_all`: the dynamic LDS.
 template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS>
-__global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw,
-                                                           float* __restrict__ y, int32_t* __restrict__ dump, GroupView grp,
-                                                           uint32_t ksplit, float* __restrict__ partial,
-                                                           uint32_t* __restrict__ counters) {
+__device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw, float* __restrict__ y,
+                                            int32_t* __restrict__ dump, GroupView grp, uint32_t ksplit, float* __restrict__ partial,
+                                            uint32_t* __restrict__ counters, uint32_t bx, uint32_t by, uint32_t nthr,
+                                            float* __restrict__ lds_all) {
     constexpr int TPAD = NT <= 4 ? 4 : 8;
     constexpr int NI = NT < 4 ? NT : 4;          // accumulator registers that hold live tokens
     constexpr bool SUMS = FMT != FMT_Q8_0;
-    // 16-byte aligned whatever static LDS the kernel also holds: the 8- and 16-byte LDS reads below are split into
-    // dwords (and the kernel runs two to three times longer) when this array starts at an odd dword
-    extern __shared__ __align__(16) float lds_all[];
     // the wave index and everything derived from it (tile, K range) live in scalar registers: branches on them are
     // scalar, and the load counters the compiler keeps stay exact across them
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t n = lane & 15, kq = lane >> 4;  // B / D role: row n of the tile; A role: slot n
     const uint32_t nblk = w.n_in / 32;
     const uint32_t r = wave / kw, ks = wave % kw;
-    const uint32_t tile = blockIdx.x * rt + r;
+    const uint32_t tile = bx * rt + r;
     const uint32_t ntiles = row_tiles(w.n_out);
     // this workgroup's slice of K: steps [S0, S1), blocks [B0, B0 + nbl) (a multiple of 4 blocks)
     constexpr uint32_t BPS = FMT == FMT_Q8_0 ? 2 : 4;  // blocks of 32 per step
     const uint32_t nsteps = FMT == FMT_Q8_0 ? t8_steps(w.n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in) : t4m_steps(w.n_in));
-    const uint32_t slice = GROUPED ? 0 : blockIdx.y;
+    const uint32_t slice = GROUPED ? 0 : by;
     const uint32_t sl = (nsteps + ksplit - 1) / ksplit;
     const uint32_t S0 = min(nsteps, slice * sl), S1 = min(nsteps, S0 + sl);
     const uint32_t B0 = BPS * S0, nbl = BPS * sl, M0 = B0 / 2;
@@ -143,8 +143,8 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
     float* red = ALDS ? lds_all : lds + (size_t)(SUMS ? (DUMP ? 4 : 3) : 1) * nbl * TPAD;  // [rt * kw][TPAD][16]
     uint32_t row0 = 0;  // first activation / output row of this launch unit
     if (GROUPED) {
-        if (blockIdx.y >= (uint32_t)*grp.nchunks) return;  // uniform over the workgroup
-        const int4 ch = grp.chunks[blockIdx.y];
+        if (by >= (uint32_t)*grp.nchunks) return;  // uniform over the workgroup
+        const int4 ch = grp.chunks[by];
         w.p0 = grp.bases[ch.x];
         row0 = (uint32_t)ch.y;
         t = (uint32_t)ch.z;
@@ -357,31 +357,31 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
     // counted exactly; the extra requests hit lines that are being fetched anyway)
     if (ALDS) {
 #pragma unroll
-        for (int j = 0; j < SA / AU; j++) act_load(min(threadIdx.x + j * blockDim.x, na - 1), sa + AU * j);
+        for (int j = 0; j < SA / AU; j++) act_load(min(threadIdx.x + j * nthr, na - 1), sa + AU * j);
     }
 #pragma unroll
-    for (int j = 0; j < SM; j++) meta_load(min(threadIdx.x + j * blockDim.x, nm - 1), smr[j]);
+    for (int j = 0; j < SM; j++) meta_load(min(threadIdx.x + j * nthr, nm - 1), smr[j]);
     Step<FMT> ring[PF];
     const uint32_t slast = max(s1, 1u) - 1;
 #pragma unroll
     for (int p = 0; p < PF; p++) load_step(ring[p], min(s0 + p, slast));
 #pragma unroll
     for (int j = 0; j < SA / AU; j++) {
-        const uint32_t i = threadIdx.x + j * blockDim.x;
+        const uint32_t i = threadIdx.x + j * nthr;
         if (i < na) act_store(i, sa + AU * j);
     }
 #pragma unroll
     for (int j = 0; j < SM; j++) {
-        const uint32_t i = threadIdx.x + j * blockDim.x;
+        const uint32_t i = threadIdx.x + j * nthr;
         if (i < nm) meta_store(i, smr[j]);
     }
     // what did not fit the registers (long rows, small workgroups) follows behind the weights
-    for (uint32_t i = threadIdx.x + (SA / AU) * blockDim.x; i < na; i += blockDim.x) {
+    for (uint32_t i = threadIdx.x + (SA / AU) * nthr; i < na; i += nthr) {
         uint4 v[AU];
         act_load(i, v);
         act_store(i, v);
     }
-    for (uint32_t i = threadIdx.x + SM * blockDim.x; i < nm; i += blockDim.x) {
+    for (uint32_t i = threadIdx.x + SM * nthr; i < nm; i += nthr) {
         MetaReg r;
         meta_load(i, r);
         meta_store(i, r);
@@ -407,9 +407,9 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
     __syncthreads();
     // the waves of a tile in order; with one slice that is the result, else this slice's partial rows
     float* out = ksplit > 1 ? partial + (size_t)slice * t * w.n_out : y;
-    for (uint32_t idx = threadIdx.x; idx < rt * TPAD * 16; idx += blockDim.x) {
+    for (uint32_t idx = threadIdx.x; idx < rt * TPAD * 16; idx += nthr) {
         const uint32_t rr = idx / (TPAD * 16), tok = (idx / 16) % TPAD, nn = idx % 16;
-        const uint32_t row = (blockIdx.x * rt + rr) * 16 + nn;
+        const uint32_t row = (bx * rt + rr) * 16 + nn;
         if (tok >= t || row >= w.n_out || !y) continue;
         float sum = 0.0f;
         for (uint32_t k = 0; k < kw; k++) sum += red[((size_t)(rr * kw + k) * TPAD + tok) * 16 + nn];
@@ -426,19 +426,78 @@ __global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActVie
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
-        const uint32_t seen = __hip_atomic_fetch_add(&counters[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t seen = __hip_atomic_fetch_add(&counters[bx], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         is_last = seen == ksplit - 1;
-        if (seen == ksplit - 1) __hip_atomic_store(&counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (seen == ksplit - 1) __hip_atomic_store(&counters[bx], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!is_last) return;
-    for (uint32_t idx = threadIdx.x; idx < rt * 16 * t; idx += blockDim.x) {
-        const uint32_t tok = idx / (rt * 16), row = blockIdx.x * rt * 16 + idx % (rt * 16);
+    for (uint32_t idx = threadIdx.x; idx < rt * 16 * t; idx += nthr) {
+        const uint32_t tok = idx / (rt * 16), row = bx * rt * 16 + idx % (rt * 16);
         if (row >= w.n_out) continue;
         const float* p = partial + (size_t)tok * w.n_out + row;
         float sum = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         for (uint32_t z = 1; z < ksplit; z++) sum += __hip_atomic_load(p + (size_t)z * t * w.n_out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         y[(size_t)tok * w.n_out + row] = sum;
+    }
+}
+
+
+// Dynamic LDS is declared 16-byte aligned whatever static LDS a kernel also holds: the 8- and 16-byte LDS reads are split
+// into dwords (and the kernel runs two to three times longer) when the array starts at an odd dword.
+template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS>
+__global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw,
+                                                           float* __restrict__ y, int32_t* __restrict__ dump, GroupView grp,
+                                                           uint32_t ksplit, float* __restrict__ partial,
+                                                           uint32_t* __restrict__ counters) {
+    extern __shared__ __align__(16) float lds_dyn[];
+    decode_body<FMT, NT, DUMP, GROUPED, ALDS>(w, xa, t, rt, kw, y, dump, grp, ksplit, partial, counters, blockIdx.x, blockIdx.y,
+                                              blockDim.x, lds_dyn);
+}
+
+// Several independent matmuls in one launch (the jobs of one Backend::matmul call, src/gpu.rs:160: Q/K/V, gate/up ...):
+// job j owns workgroups [wg0_j, wg0_{j+1}); each workgroup runs its job exactly as a launch of that job alone would
+// (same shape, same order of sums), so the results are bit-identical to separate launches. What the single launch
+// buys is time: a decode matmul is a chain of dependent latencies (stage activations, stream weights, reduce, store:
+// about 6 us before the first byte of bandwidth counts), and here the chains of neighbouring jobs overlap instead of
+// queueing behind kernel boundaries.
+constexpr int BATCH_MAX = 16;
+struct BatchJob {
+    WeightView w;
+    QActView xa;
+    float* y;
+    float* partial;      // this job's share of the scratch (K slices across workgroups)
+    uint32_t* counters;
+    uint32_t t, rt, kw, ks, wg0;
+};
+struct BatchArgs {
+    uint32_t njobs, nwg;
+    BatchJob j[BATCH_MAX];
+};
+
+template <int FMT>
+__device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid, float* lds) {
+    const uint32_t nthr = 64 * jb.rt * jb.kw;
+    if (threadIdx.x >= nthr) return;  // whole waves (nthr is a multiple of 64), before any barrier
+    const GroupView none{};
+    const uint32_t bx = bid / jb.ks, by = bid % jb.ks;  // the slices of a row group are neighbours in launch order
+    if (jb.t == 1) decode_body<FMT, 1, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
+    else if (jb.t == 2) decode_body<FMT, 2, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
+    else if (jb.t <= 4) decode_body<FMT, 4, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
+    else decode_body<FMT, 8, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
+}
+
+__global__ __launch_bounds__(1024) void decode_batch_kernel(BatchArgs a) {
+    extern __shared__ __align__(16) float lds_dyn[];
+    uint32_t j = 0;
+    while (j + 1 < a.njobs && blockIdx.x >= a.j[j + 1].wg0) j++;  // uniform
+    const BatchJob& jb = a.j[j];
+    const uint32_t bx = blockIdx.x - jb.wg0;
+    switch (jb.w.fmt) {
+        case FMT_Q8_0: batch_dispatch<FMT_Q8_0>(jb, bx, lds_dyn); break;
+        case FMT_Q4_K: batch_dispatch<FMT_Q4_K>(jb, bx, lds_dyn); break;
+        case FMT_Q4M: batch_dispatch<FMT_Q4M>(jb, bx, lds_dyn); break;
+        default: break;
     }
 }
 
@@ -450,50 +509,53 @@ struct Shape {
 
 constexpr uint32_t NCU = 256;
 
-// Workgroup shape (rt row tiles x kw waves per tile, at most 16 waves) and the number of K slices across workgroups:
-// a function of the weight's shape only, so a row's sum is associated the same way whatever the batch. The pick
-// minimizes the work of the busiest CU when the workgroups are dealt out one per CU per generation (the whole matrix
-// should be on request from the first microsecond), then prefers enough waves to cover HBM latency, a few records
-// per wave, and few slices. 896 row tiles, for one, run as 128 groups of 7 tiles x 2 slices = 256 workgroups.
-Shape search_shape(uint32_t ntiles, uint32_t nsteps, bool allow_slices) {
-    Shape best{1, 1, 1};
+// Workgroup shape (rt row tiles x kw waves per tile) and the number of K slices across workgroups (ks): a function of
+// the weight's shape only, so a row's sum is associated the same way whatever the batch or the kind of launch.
+//  * A matmul at these sizes is a chain of dependent latencies (stage activations, stream weights, reduce, store)
+//    and only overlaps them when a CU holds several workgroups in different phases: workgroups have at most 8 waves,
+//    and K is sliced until a workgroup's staged activations (11 bytes per column at 8 tokens) leave room for three
+//    workgroups in a CU's 160 KiB.
+//  * Among the (rt, kw) left, the pick minimizes the records that pass through the busiest CU when workgroups are
+//    dealt round-robin, and prefers a few records per wave, four or more waves, and little restaging.
+Shape search_shape(uint32_t ntiles, uint32_t nsteps, uint32_t cols_per_step) {
+    uint32_t ks = 1;
+    while (ks < 32 && (size_t)nsteps * cols_per_step * 11 / ks > 48 * 1024 && nsteps / (ks * 2) >= 4) ks *= 2;
+    while (ks > 1 && (nsteps + ks - 1) / ks * (ks - 1) >= nsteps) ks /= 2;  // no empty slice
+    const uint32_t sl = (nsteps + ks - 1) / ks;
+    Shape best{1, 1, ks};
     double best_cost = 1e300;
-    for (uint32_t kw = 1; kw <= 16; kw *= 2)
-        for (uint32_t rt = 1; rt * kw <= 16; rt++)
-            for (uint32_t ks = 1; ks <= (allow_slices ? 32u : 1u); ks *= 2) {
-                if (ks > 1 && (nsteps + ks - 1) / ks * (ks - 1) >= nsteps) continue;  // an empty slice
-                const uint32_t sl = (nsteps + ks - 1) / ks, per = (sl + kw - 1) / kw;
-                const uint64_t wgs = (uint64_t)((ntiles + rt - 1) / rt) * ks;
-                const uint64_t gens = (wgs + NCU - 1) / NCU;
-                double cost = (double)gens * rt * per * kw;  // records through the busiest CU
-                const uint32_t waves = rt * kw;
-                if (waves < 8) cost *= 1.0 + 0.08 * (8 - waves);
-                if (per < 4) cost *= 1.0 + 0.10 * (4 - per);
-                if (ks > 1) cost *= 1.15 + 0.01 * ks;  // the last-arrival pass costs about 1.5 us of dependent round trips
-                cost *= 1.0 + 0.002 * kw;
-                if (cost < best_cost) {
-                    best_cost = cost;
-                    best = Shape{rt, kw, ks};
-                }
+    for (uint32_t kw = 1; kw <= 8; kw *= 2)
+        for (uint32_t rt = 1; rt * kw <= 8; rt++) {
+            const uint32_t per = (sl + kw - 1) / kw;
+            const uint64_t wgs = (uint64_t)((ntiles + rt - 1) / rt) * ks;
+            double cost = (double)((wgs + NCU - 1) / NCU) * rt * per * kw;  // records through the busiest CU
+            if (rt * kw < 4) cost *= 1.0 + 0.10 * (4 - rt * kw);
+            if (per < 8) cost *= 1.0 + 0.03 * (8 - per);    // short streams: the latency chain dominates
+            if (per > 16) cost *= 1.0 + 0.02 * (per - 16);  // long streams: too few waves keep HBM busy
+            cost *= 1.0 + 0.05 / rt + 0.002 * kw;  // every workgroup stages its slice again: larger groups restage less
+            if (cost < best_cost) {
+                best_cost = cost;
+                best = Shape{rt, kw, ks};
             }
+        }
     if (const char* e = getenv("OXHIP_DECODE_SHAPE")) {  // developer override for tuning runs: "rt,kw,ks"
         unsigned a = 0, b = 0, c = 0;
-        if (sscanf(e, "%u,%u,%u", &a, &b, &c) == 3 && a >= 1 && b >= 1 && c >= 1 && a * b <= 16 && (allow_slices || c == 1))
-            best = Shape{a, b, c};
+        if (sscanf(e, "%u,%u,%u", &a, &b, &c) == 3 && a >= 1 && b >= 1 && c >= 1 && a * b <= 16) best = Shape{a, b, c};
     }
     return best;
 }
 
-// The search runs once per (shape, kind of launch): a decode launch is a few microseconds of GPU time and must not
-// spend as long on the host.
-Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices) {
+// The search runs once per shape: a decode launch is a few microseconds of GPU time and must not spend as long on
+// the host. Without scratch for the slices (allow_slices false) K stays inside a workgroup.
+Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices, uint32_t cols_per_step = 128) {
     static std::mutex mu;
     static std::map<uint64_t, Shape> cache;
-    const uint64_t key = ((uint64_t)ntiles << 33) | ((uint64_t)nsteps << 1) | (allow_slices ? 1u : 0u);
+    const uint64_t key = ((uint64_t)ntiles << 34) | ((uint64_t)nsteps << 2) | (cols_per_step == 64 ? 2u : 0u) | (allow_slices ? 1u : 0u);
     std::lock_guard<std::mutex> g(mu);
     auto it = cache.find(key);
     if (it != cache.end()) return it->second;
-    const Shape sh = search_shape(ntiles, nsteps, allow_slices);
+    Shape sh = search_shape(ntiles, nsteps, cols_per_step);
+    if (!allow_slices) sh.ks = 1;
     cache.emplace(key, sh);
     return sh;
 }
@@ -539,11 +601,11 @@ constexpr uint32_t steps_of(uint32_t n_in) {
 template <int FMT, bool DUMP>
 hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* dump, const DecodeScratch& sc, hipStream_t s) {
     const uint32_t ntiles = row_tiles(w.n_out), nsteps = steps_of<FMT>(w.n_in);
-    Shape sh = shape_for(ntiles, nsteps, true);
+    Shape sh = shape_for(ntiles, nsteps, true, FMT == FMT_Q8_0 ? 64 : 128);
     const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
     // slices need scratch: 8 token rows per slice and a counter per row group
     if (sh.ks > 1 && (!sc.partial || !sc.counters || sc.partial_floats < (size_t)sh.ks * 8 * w.n_out || sc.ncounters < groups))
-        sh = shape_for(ntiles, nsteps, false);
+        sh = shape_for(ntiles, nsteps, false, FMT == FMT_Q8_0 ? 64 : 128);
     const uint32_t nblk = w.n_in / 32;
     dim3 grid((ntiles + sh.rt - 1) / sh.rt, sh.ks), block(64 * sh.rt * sh.kw);
     size_t c0 = 0;
@@ -578,7 +640,7 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
     const uint32_t ntiles = row_tiles(w.n_out), nsteps = steps_of<FMT>(w.n_in);
     // grid y walks the chunks: no K slices across workgroups here (the shape still depends on the weight alone, so a
     // token's row is bit-identical whatever else is in the group)
-    const Shape sh = shape_for(ntiles, nsteps, false);
+    const Shape sh = shape_for(ntiles, nsteps, false, FMT == FMT_Q8_0 ? 64 : 128);
     dim3 grid((ntiles + sh.rt - 1) / sh.rt, max_chunks), block(64 * sh.rt * sh.kw);
     const int tpad = max_rows <= 4 ? 4 : 8;
     bool alds;
@@ -591,6 +653,80 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
 }
 
 }  // namespace
+
+namespace {
+uint32_t steps_rt(const WeightView& w) {
+    return w.fmt == FMT_Q8_0 ? steps_of<FMT_Q8_0>(w.n_in) : (w.fmt == FMT_Q4_K ? steps_of<FMT_Q4_K>(w.n_in) : steps_of<FMT_Q4M>(w.n_in));
+}
+}  // namespace
+
+bool decode_batchable(const WeightView& w, size_t t) {
+    if (w.fmt != FMT_Q8_0 && w.fmt != FMT_Q4_K && w.fmt != FMT_Q4M) return false;
+    if (t < 1 || t > 8) return false;
+    const Shape sh = shape_for(row_tiles(w.n_out), steps_rt(w), true, w.fmt == FMT_Q8_0 ? 64 : 128);  // as a launch of its own: same bits
+    bool alds;
+    const size_t lds = lds_bytes(w.fmt != FMT_Q8_0, false, w.fmt == FMT_Q8_0 ? 2 : 4, steps_rt(w), t <= 4 ? 4 : 8, sh, &alds);
+    return alds && lds <= LDS_MAX;
+}
+
+// Every item must be decode_batchable. Items go out in launches of up to BATCH_MAX jobs; jobs whose shape slices K
+// across workgroups take their partial rows and counters from `sc` (hipErrorOutOfMemory when it is too small:
+// nothing has been launched then and the caller launches the jobs one by one).
+hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s) {
+    static std::atomic<uint64_t> allowed[4];  // whole LDS allowed, one bit per device
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(allowed[(dev >> 6) & 3].load(std::memory_order_acquire) & bit)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_batch_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)LDS_MAX);
+        if (e != hipSuccess) return e;
+        allowed[(dev >> 6) & 3].fetch_or(bit, std::memory_order_release);
+    }
+    std::vector<BatchArgs> launches;
+    std::vector<size_t> ldss;
+    std::vector<uint32_t> threadss;
+    for (size_t i0 = 0; i0 < n; i0 += BATCH_MAX) {
+        BatchArgs a{};
+        a.njobs = (uint32_t)(n - i0 < (size_t)BATCH_MAX ? n - i0 : (size_t)BATCH_MAX);
+        size_t lds = 0, pf = 0, nc = 0;  // scratch is shared by the jobs of one launch, reused by the next launch
+        uint32_t wg = 0, threads = 64;
+        for (uint32_t j = 0; j < a.njobs; j++) {
+            const DecodeBatchItem& it = items[i0 + j];
+            const uint32_t ntiles = row_tiles(it.w.n_out), nsteps = steps_rt(it.w);
+            const Shape sh = shape_for(ntiles, nsteps, true, it.w.fmt == FMT_Q8_0 ? 64 : 128);
+            bool alds;
+            const size_t l = lds_bytes(it.w.fmt != FMT_Q8_0, false, it.w.fmt == FMT_Q8_0 ? 2 : 4, nsteps, it.t <= 4 ? 4 : 8, sh, &alds);
+            if (!alds || l > LDS_MAX || it.t < 1 || it.t > 8) return hipErrorInvalidValue;
+            const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
+            float* partial = nullptr;
+            uint32_t* counters = nullptr;
+            if (sh.ks > 1) {
+                const size_t need = (size_t)sh.ks * it.t * it.w.n_out;
+                if (!sc.partial || !sc.counters || pf + need > sc.partial_floats || nc + groups > sc.ncounters) return hipErrorOutOfMemory;
+                partial = sc.partial + pf;
+                counters = sc.counters + nc;
+                pf += (need + 63) / 64 * 64;
+                nc += groups;
+            }
+            lds = l > lds ? l : lds;
+            threads = 64 * sh.rt * sh.kw > threads ? 64 * sh.rt * sh.kw : threads;
+            a.j[j] = BatchJob{it.w, it.xa, it.y, partial, counters, it.t, sh.rt, sh.kw, sh.ks, wg};
+            wg += groups * sh.ks;
+        }
+        a.nwg = wg;
+        launches.push_back(a);
+        ldss.push_back(lds);
+        threadss.push_back(threads);
+    }
+    for (size_t i = 0; i < launches.size(); i++) {
+        if (!launches[i].nwg) continue;
+        decode_batch_kernel<<<launches[i].nwg, threadss[i], ldss[i], s>>>(launches[i]);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
 
 hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks,
                                       uint32_t max_rows_per_chunk, float* y, hipStream_t s) {

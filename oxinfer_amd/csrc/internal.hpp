@@ -70,6 +70,15 @@ struct DecodeScratch {
 hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s,
                          const DecodeScratch& sc = DecodeScratch{});
 hipError_t launch_isums(const WeightView& w, const QActView& xa, size_t t, int32_t* out, hipStream_t s);
+// Independent matmuls that may share one launch (decode_mfma.hip): each 1..8 tokens over a tile-packed weight.
+struct DecodeBatchItem {
+    WeightView w;
+    QActView xa;
+    float* y;
+    uint32_t t;
+};
+bool decode_batchable(const WeightView& w, size_t t);  // the kernel takes it and its activations fit LDS
+hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s);
 hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, const DecodeScratch& sc, hipStream_t s);
 hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks,
                                       uint32_t max_rows_per_chunk, float* y, hipStream_t s);

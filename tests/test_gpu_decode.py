@@ -273,3 +273,32 @@ def test_full_size_rows_against_oracle(be, oxref, kind, n_out, n_in):
     assert float((np.abs(y[:, rows] - ref).max(axis=1) / m).max()) < TOL
     y1 = be.decode(w, xa=be.quantize_act(dev(x[3:4]))).cpu().numpy()
     assert np.array_equal(y1[0].view(np.uint32), y[3].view(np.uint32))
+
+
+def test_decode_batch_shares_a_launch_and_keeps_the_bits(be, oxref):
+    """Independent matmuls handed over as one batch (the jobs of one Backend::matmul call, src/gpu.rs:160) run in one
+    launch; every job's rows are bit-identical to its own launch, whatever its neighbours, formats and batch sizes."""
+    import torch
+    from oxinfer_amd import synth
+    cases = [(Q8_0, 208, 512, 1), (Q4_K, 96, 1024, 8), (Q8_0, 64, 2048, 3), (Q4_K, 176, 512, 2), ("mlx", 80, 640, 5),
+             (Q6_K, 48, 512, 2), (Q4_K, 33, 256, 4), ("mlx", 128, 128, 8)]
+    jobs, alone = [], []
+    for i, (kind, n_out, n_in, t) in enumerate(cases):
+        if kind == "mlx":
+            w = be.upload_mlx_q4(*synth.mlx_q4(n_out, n_in, 70 + i), 64, n_out, n_in)
+        else:
+            raw, _ = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 80 + i)
+            w = be.upload_gguf(kind, raw, n_out, n_in)
+        assert w is not None, be.last_error()
+        xa = be.quantize_act(torch.from_numpy(synth.activations(t, n_in, 90 + i)).cuda())
+        alone.append(be.decode(w, xa=xa).cpu().numpy())
+        y = torch.full((t, n_out), float("nan"), dtype=torch.float32, device="cuda")
+        jobs.append((w, xa, None, t, y, None, None))
+    for order in (list(range(len(cases))), list(reversed(range(len(cases)))), [1, 3, 6], [4]):
+        for i in order:
+            jobs[i][4].fill_(float("nan"))
+        be.decode_batch(be.decode_jobs([jobs[i] for i in order]))
+        torch.cuda.synchronize()
+        for i in order:
+            got = jobs[i][4].cpu().numpy()
+            assert np.array_equal(got.view(np.uint32), alone[i].view(np.uint32)), (order, i, cases[i])
