@@ -100,15 +100,142 @@ def cpu_baseline(cases, gens, seconds=20.0):
             "per_case_weight_GBs": per}
 
 
+MFMA_PEAK = {"bf16": 2500.0, "i8": 5000.0, "fp8": 5000.0}
+
+
+def timed_steps(torch, step, steps, warmup):
+    """W untimed steps, then K steps between synchronizations: (wall seconds, mean milliseconds between the CUDA/HIP
+    events recorded around each step on the launch stream)."""
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        ev[i][0].record()
+        step(warmup + i)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, float(np.mean([a.elapsed_time(b) for a, b in ev]))
+
+
+def other_workload(args, be, torch, synth):
+    """The other configurations of BASELINE.json, one JSON line each (profiling and per-config numbers; the default
+    workload is what the driver records). Weights rotate over >= pool-gb of distinct copies where HBM bounds."""
+    base = {"metric": METRIC, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "data": "synthetic"}
+
+    def pool(make, nbytes):
+        return [make() for _ in range(max(2, int(np.ceil(args.pool_gb * 1e9 / nbytes))))]
+
+    if args.workload == "mlx_gemv":                      # configs[0]: N = K = 4096, T = 1
+        n = k = 4096
+        wq, sc, bi = synth.mlx_q4(n, k, 1)
+        ws = pool(lambda: be.upload_mlx_q4(wq, sc, bi, 64, n, k), n * k * 0.5625)
+        xa = be.quantize_act(torch.from_numpy(synth.activations(1, k, 2)).cuda())
+        y = torch.empty((1, n), dtype=torch.float32, device="cuda")
+        nbytes = int(n * k * 0.5625) + k * (1 + 4 / 32 + 8 / 32) + n * 4
+        wall, ms = timed_steps(torch, lambda i: be.decode(ws[i % len(ws)], xa=xa, y=y), args.steps, args.warmup)
+        ach = nbytes / (ms * 1e-3) / 1e9
+        return dict(base, value=round(nbytes * args.steps / wall / 1e9, 2), unit="GB/s", ms_per_step=round(wall / args.steps * 1e3, 5),
+                    dtype="int8", config={"workload": "configs[0]: MLX 4-bit g64 GEMV 4096 -> 4096, T = 1", "bytes_per_step": nbytes},
+                    roofline={"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "decode_mfma_kernel<6, 1, ...>",
+                              "bytes_per_launch": nbytes, "avg_launch_us": round(ms * 1e3, 2)})
+
+    if args.workload == "mlx_gemm":                      # configs[2]: M = 512, both shapes, variant (a) or (b)
+        variant = {"bf16": 0, "i8": 1}[args.variant]
+        shapes = [(14336, 4096), (4096, 14336)]
+        ws, xs = [], []
+        for n, k in shapes:
+            wq, sc, bi = synth.mlx_q4(n, k, 3)
+            ws.append([be.upload_mlx_q4(wq, sc, bi, 64, n, k) for _ in range(4)])
+            xs.append(torch.from_numpy(synth.activations(512, k, 4, bf16=True)).cuda().to(torch.bfloat16))
+        flops = sum(2 * 512 * n * k for n, k in shapes)
+
+        def step(i):
+            for j in range(2):
+                be.gemm(ws[j][i % 4], xs[j], variant=variant)
+        wall, ms = timed_steps(torch, step, args.steps, args.warmup)
+        ach = flops / (ms * 1e-3) / 1e12
+        peak = MFMA_PEAK[args.variant]
+        return dict(base, value=round(flops * args.steps / wall / 1e12, 2), unit="TFLOP/s", ms_per_step=round(wall / args.steps * 1e3, 5),
+                    dtype="bf16" if variant == 0 else "int8",
+                    config={"workload": f"configs[2]: MLX 4-bit g64 prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096, variant {args.variant}",
+                            "flops_per_step": flops, "events": "around the two calls of a step (activation packing + GEMM (+ K-slice sum))"},
+                    roofline={"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4),
+                              "traffic": None, "kernel": "gemm_bf16_kernel<6, false>" if variant == 0 else "gemm_i8_q4m_kernel",
+                              "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3 / 2, 2)})
+
+    if args.workload == "moe":                           # configs[3]: 128 experts, top-8, h = 2048, inter = 768
+        ne, k, h, inter = 128, 8, 2048, 768
+        t = args.tokens or 1
+        gu = [synth.mlx_q4(2 * inter, h, 100 + e) for e in range(ne)]
+        dn = [synth.mlx_q4(h, inter, 300 + e) for e in range(ne)]
+        expert_bytes = int((2 * inter * h + h * inter) * 0.5625)
+        devs = pool(lambda: be.upload_moe([be.desc_mlx_q4(*g, 64, 2 * inter, h) for g in gu],
+                                          [be.desc_mlx_q4(*d, 64, h, inter) for d in dn], h, inter), ne * expert_bytes)
+        x = torch.from_numpy(synth.activations(t, h, 5, bf16=True)).cuda()
+        logits = torch.from_numpy(synth.router_logits(t, ne, 6)).cuda()
+        idx, w = be.route_top_k(logits, k)
+        touched = len(set(idx.cpu().numpy().reshape(-1).tolist()))
+        y = torch.zeros((t, h), dtype=torch.float32, device="cuda")
+        nbytes = touched * expert_bytes
+        flops = 2 * t * k * (2 * inter * h + h * inter)
+
+        def step(i):
+            be.route_top_k(logits, k)
+            be.dev_moe(devs[i % len(devs)], x, idx, w, y)
+        wall, ms = timed_steps(torch, step, args.steps, args.warmup)
+        ach = nbytes / (ms * 1e-3) / 1e9
+        return dict(base, value=round(nbytes * args.steps / wall / 1e9, 2), unit="GB/s", ms_per_step=round(wall / args.steps * 1e3, 5),
+                    dtype="int8", config={"workload": f"configs[3]: MoE 128 experts top-8, h 2048, inter 768, MLX 4-bit g64, T = {t}",
+                                          "experts_touched": touched, "bytes_per_step": nbytes, "flops_per_step": flops,
+                                          "events": "around routing + the MoE call (plan, quantize, grouped gate_up, activation, quantize, grouped down, combine)"},
+                    roofline={"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                              "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "decode_mfma_kernel<6, *, false, true, true> (grouped)",
+                              "bytes_per_launch": nbytes, "avg_launch_us": round(ms * 1e3, 2)},
+                    tflops=round(flops / (ms * 1e-3) / 1e12, 2))
+
+    # configs[4]: FP8 E4M3 [7168, 18432] with 128 x 128 block scales, bf16 activations, bf16 out
+    n, k = 7168, 18432
+    m = args.tokens or 1024
+    data, scales = synth.fp8_e4m3(n, k, 7)
+    ws = pool(lambda: be.upload_fp8(data, scales, n, k), n * k)
+    x32 = torch.from_numpy(synth.activations(m, k, 8, bf16=True)).cuda()
+    xb = x32.to(torch.bfloat16)
+    variant = {"bf16": 0, "fp8": 2}.get(args.variant, 0)
+    if m <= 16:
+        step = lambda i: be.decode(ws[i % len(ws)], x=x32)
+        kern = "decode_dense_kernel<4, *>"
+    else:
+        step = lambda i: be.gemm(ws[i % len(ws)], xb, variant=variant, out_bf16=True)
+        kern = "gemm_bf16_kernel<4, true>" if variant == 0 else "gemm_fp8_kernel<true>"
+    wall, ms = timed_steps(torch, step, args.steps, args.warmup)
+    flops, nbytes = 2 * m * n * k, n * k + scales.size * 4 + m * k * 2 + m * n * 2
+    hbm = m <= 64
+    ach = nbytes / (ms * 1e-3) / 1e9 if hbm else flops / (ms * 1e-3) / 1e12
+    peak = HBM_PEAK_GBS if hbm else MFMA_PEAK["bf16" if variant == 0 else "fp8"]
+    return dict(base, value=round((nbytes / 1e9 if hbm else flops / 1e12) * args.steps / wall, 2), unit="GB/s" if hbm else "TFLOP/s",
+                ms_per_step=round(wall / args.steps * 1e3, 5), dtype="fp8 weights, " + ("f32" if m <= 16 else ("bf16" if variant == 0 else "fp8")) + " activations",
+                config={"workload": f"configs[4]: FP8 E4M3 block-scaled GEMM [7168, 18432], M = {m}, variant {args.variant if m > 16 else 'decode'}",
+                        "bytes_per_step": nbytes, "flops_per_step": flops},
+                roofline={"bound": "hbm" if hbm else "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "GB/s" if hbm else "TFLOP/s",
+                          "frac": round(ach / peak, 4), "traffic": None, "kernel": kern, "avg_launch_us": round(ms * 1e3, 2)})
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gguf_gemv", choices=["gguf_gemv", "gguf_gemv_q6k", "copy"],
+    ap.add_argument("--workload", default="gguf_gemv", choices=["gguf_gemv", "gguf_gemv_q6k", "mlx_gemv", "mlx_gemm", "moe", "fp8", "copy"],
                     help="copy = a plain 256 MiB device copy, the known-size kernel that scales the HBM traffic counters")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pool-gb", type=float, default=POOL_BYTES / 1e9)
+    ap.add_argument("--variant", default="bf16", choices=["bf16", "i8", "fp8"], help="GEMM variant of mlx_gemm / fp8")
+    ap.add_argument("--tokens", type=int, default=0, help="tokens of the moe (1 or 256) and fp8 (1, 32, 1024) workloads")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1 (nothing here uses a second device)", file=sys.stderr)
@@ -130,6 +257,10 @@ def main():
         print(json.dumps({"workload": "copy", "bytes_read": n, "bytes_written": n, "launches": args.warmup + args.steps}))
         return
     be = HipBackend(0)
+    if args.workload in ("mlx_gemv", "mlx_gemm", "moe", "fp8"):
+        print(json.dumps(other_workload(args, be, torch, synth)))
+        be.close()
+        return
     gens = {Q8_0: synth.gguf_q8_0, Q4_K: synth.gguf_q4_k, Q6_K: synth.gguf_q6_k}
     kinds = [Q8_0, Q4_K] if args.workload == "gguf_gemv" else [Q6_K]
     cases = gemv_cases(kinds)

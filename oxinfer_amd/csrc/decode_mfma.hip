@@ -30,6 +30,7 @@
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <vector>
@@ -538,9 +539,15 @@ Shape search_shape(uint32_t ntiles, uint32_t nsteps, uint32_t cols_per_step) {
                 best = Shape{rt, kw, ks};
             }
         }
-    if (const char* e = getenv("OXHIP_DECODE_SHAPE")) {  // developer override for tuning runs: "rt,kw,ks"
-        unsigned a = 0, b = 0, c = 0;
-        if (sscanf(e, "%u,%u,%u", &a, &b, &c) == 3 && a >= 1 && b >= 1 && c >= 1 && a * b <= 16) best = Shape{a, b, c};
+    if (const char* e = getenv("OXHIP_DECODE_SHAPE")) {  // developer override for tuning runs: "tiles:steps=rt,kw,ks;..."
+        for (const char* p = e; p && *p;) {
+            unsigned nt = 0, ns = 0, a = 0, b = 0, c = 0;
+            if (sscanf(p, "%u:%u=%u,%u,%u", &nt, &ns, &a, &b, &c) == 5 && nt == ntiles && ns == nsteps && a >= 1 && b >= 1 && c >= 1 &&
+                a * b <= 16)
+                best = Shape{a, b, c};
+            p = strchr(p, ';');
+            if (p) p++;
+        }
     }
     return best;
 }
