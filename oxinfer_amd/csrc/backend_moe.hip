@@ -1,5 +1,6 @@
 // Backend::upload_moe / moe / matvec_rows (src/gpu.rs:165, :206-248 of the reference) over the grouped
 // decode kernel, plus their device-pointer forms.
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -40,6 +41,7 @@ struct Scratch {
     size_t bytes;
 };
 
+// (sized for chunks of 8 rows, the most there can be)
 Scratch carve(uint8_t* base, size_t t, size_t pairs, size_t n_exp, size_t h, size_t inter) {
     Scratch s{};
     s.max_chunks = (uint32_t)((pairs < n_exp ? pairs : n_exp) + pairs / 8 + 1);
@@ -79,8 +81,17 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
         m->ws_t = nt;
     }
     Scratch sc = carve(static_cast<uint8_t*>(m->ws.p), t, pairs, m->n_exp, h, inter);
-    const uint32_t max_rows = (uint32_t)(t < 8 ? t : 8);
-    HIP_TRY(launch_moe_plan(route_idx, pairs, k, m->n_exp, sc.row_of, sc.src, sc.chunks, sc.nchunks, s), "moe plan launch");
+    // Rows per chunk: one pass over an expert's weights serves a whole chunk, so chunks grow with the rows an expert
+    // gets on average (8 rows per matrix-core instruction, up to 4 instructions per weight record).
+    uint32_t max_rows = (uint32_t)(t < 8 ? t : 8);
+    const size_t avg = pairs / m->n_exp;
+    if (avg >= 6 && mfma_format(m->gate_up[0])) max_rows = avg >= 20 ? 32 : 16;
+    if (const char* e = getenv("OXHIP_MOE_CHUNK")) {  // developer override for tuning runs
+        const int v = atoi(e);
+        if ((v == 8 || v == 16 || v == 32) && t >= 8) max_rows = (uint32_t)v;
+    }
+    const uint32_t grid_chunks = (uint32_t)((pairs < m->n_exp ? pairs : m->n_exp) + pairs / max_rows + 1);
+    HIP_TRY(launch_moe_plan(route_idx, pairs, k, m->n_exp, max_rows, sc.row_of, sc.src, sc.chunks, sc.nchunks, s), "moe plan launch");
     HIP_TRY(launch_quantize_act(x, t, h, sc.xa, s), "moe quantize launch");
     GroupView g{};
     g.chunks = sc.chunks;
@@ -89,21 +100,25 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
     g.rowmap = sc.src;
     g.bases = m->bases_gu;
     const bool fused = m->up.empty();
-    HIP_TRY(launch_decode_mfma_grouped(m->gate_up[0]->v, view_of(sc.xa), g, sc.max_chunks, max_rows, sc.gu, s), "moe gate launch");
+    HIP_TRY(launch_decode_mfma_grouped(m->gate_up[0]->v, view_of(sc.xa), g, grid_chunks, max_rows, sc.gu, s), "moe gate launch");
     const float* up_out = sc.gu + inter;
     size_t stride = 2 * inter;
     if (!fused) {
         g.bases = m->bases_up;
         float* u = sc.gu + pairs * inter;
-        HIP_TRY(launch_decode_mfma_grouped(m->up[0]->v, view_of(sc.xa), g, sc.max_chunks, max_rows, u, s), "moe up launch");
+        HIP_TRY(launch_decode_mfma_grouped(m->up[0]->v, view_of(sc.xa), g, grid_chunks, max_rows, u, s), "moe up launch");
         up_out = u;
         stride = inter;
     }
-    HIP_TRY(launch_moe_act(sc.gu, up_out, stride, pairs, inter, m->act_kind, m->act_param, sc.a, s), "moe act launch");
-    HIP_TRY(launch_quantize_act(sc.a, pairs, inter, sc.aq, s), "moe quantize launch");
+    if (inter % 32 == 0 && stride % 4 == 0) {
+        HIP_TRY(launch_moe_act_quantize(sc.gu, up_out, stride, pairs, inter, m->act_kind, m->act_param, sc.aq, s), "moe act launch");
+    } else {
+        HIP_TRY(launch_moe_act(sc.gu, up_out, stride, pairs, inter, m->act_kind, m->act_param, sc.a, s), "moe act launch");
+        HIP_TRY(launch_quantize_act(sc.a, pairs, inter, sc.aq, s), "moe quantize launch");
+    }
     g.rowmap = nullptr;
     g.bases = m->bases_dn;
-    HIP_TRY(launch_decode_mfma_grouped(m->down[0]->v, view_of(sc.aq), g, sc.max_chunks, max_rows, sc.o, s), "moe down launch");
+    HIP_TRY(launch_decode_mfma_grouped(m->down[0]->v, view_of(sc.aq), g, grid_chunks, max_rows, sc.o, s), "moe down launch");
     HIP_TRY(launch_moe_combine(sc.o, sc.row_of, route_w, t, k, h, y, s), "moe combine launch");
     return 1;
 }

@@ -64,17 +64,18 @@ struct Meta4 {
 // up to f32 rounding; the integer sums U - 8 su themselves are exact (and are what the DUMP variant writes).
 // LDS: xs | c | fs | su, each [nbl][TPAD] over the workgroup's nbl blocks from b0 (c, fs only for the formats with
 // sums; su only for DUMP)
-template <int TPAD, bool SUMS, bool DUMP>
-__device__ __forceinline__ void load_meta(const float* lds, uint32_t nblk, uint32_t b, uint32_t tok0, Meta4& m) {
-    const float4 x = *reinterpret_cast<const float4*>(lds + (size_t)b * TPAD + tok0);
+// `as`: floats per array (xs, c, fs, su in turn); `at`: index of the lane's first token in its block's row
+template <bool SUMS, bool DUMP>
+__device__ __forceinline__ void load_meta(const float* lds, uint32_t as, uint32_t at, Meta4& m) {
+    const float4 x = *reinterpret_cast<const float4*>(lds + at);
     m.xs[0] = x.x; m.xs[1] = x.y; m.xs[2] = x.z; m.xs[3] = x.w;
     if (SUMS) {
-        const float4 c = *reinterpret_cast<const float4*>(lds + (size_t)nblk * TPAD + (size_t)b * TPAD + tok0);
-        const float4 f = *reinterpret_cast<const float4*>(lds + (size_t)2 * nblk * TPAD + (size_t)b * TPAD + tok0);
+        const float4 c = *reinterpret_cast<const float4*>(lds + (size_t)as + at);
+        const float4 f = *reinterpret_cast<const float4*>(lds + (size_t)2 * as + at);
         m.c[0] = c.x; m.c[1] = c.y; m.c[2] = c.z; m.c[3] = c.w;
         m.fs[0] = f.x; m.fs[1] = f.y; m.fs[2] = f.z; m.fs[3] = f.w;
         if (DUMP) {
-            const int4 q = *reinterpret_cast<const int4*>(lds + (size_t)3 * nblk * TPAD + (size_t)b * TPAD + tok0);
+            const int4 q = *reinterpret_cast<const int4*>(lds + (size_t)3 * as + at);
             m.su[0] = q.x; m.su[1] = q.y; m.su[2] = q.z; m.su[3] = q.w;
         }
     }
@@ -109,16 +110,19 @@ struct Step<FMT_Q4M> {
 // FMT: FMT_Q8_0 / FMT_Q4_K / FMT_Q4M. NT: tokens handled (1, 2, 4 or 8). DUMP: also write the exact
 // integer block sums to `dump` ([t][n_out][n_in/32]) for parity checks.
 // GROUPED: blockIdx.y walks the chunks of a grouped launch (MoE experts over their routed tokens): chunk c is
-// {expert, first row, rows (<= 8)}; the weights are expert's, activation row i of the chunk is row
+// {expert, first row, rows (<= 8 NG)}; the weights are expert's, activation row i of the chunk is row
 // rowmap[first + i] of xa (or first + i without a map), and its output is row first + i of y.
 // ALDS: the int8 activations are staged into LDS in operand order (the launcher checks that they fit).
 // `bx`, `by`: the workgroup's place in its launch unit (row group; K slice or chunk); `nthr` = 64 rt kw threads take
 // part (a launch may hold more: those waves have left before the first barrier); `lds_all`: the dynamic LDS.
-template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS>
+// NG (grouped launches of 8 tokens per group): a chunk holds up to 8 NG rows; every weight record is used for NG
+// instructions, one per group of 8 tokens, before the next is touched.
+template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS, int NG = 1>
 __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw, float* __restrict__ y,
                                             int32_t* __restrict__ dump, GroupView grp, uint32_t ksplit, float* __restrict__ partial,
                                             uint32_t* __restrict__ counters, uint32_t bx, uint32_t by, uint32_t nthr,
                                             float* __restrict__ lds_all) {
+    static_assert(NG == 1 || (GROUPED && ALDS && !DUMP && NT == 8), "token groups are for grouped launches");
     constexpr int TPAD = NT <= 4 ? 4 : 8;
     constexpr int NI = NT < 4 ? NT : 4;          // accumulator registers that hold live tokens
     constexpr bool SUMS = FMT != FMT_Q8_0;
@@ -139,9 +143,10 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     const uint32_t B0 = BPS * S0, nbl = BPS * sl, M0 = B0 / 2;
     // LDS: [operand-order activations: 512 B per pair of blocks] [scales, sums] [partial sums]; with ALDS the
     // partial sums reuse the activations' space once every wave is done with them
-    uint2* afr = reinterpret_cast<uint2*>(lds_all);
-    float* lds = lds_all + (ALDS ? (size_t)(nbl / 2) * 128 : 0);
-    float* red = ALDS ? lds_all : lds + (size_t)(SUMS ? (DUMP ? 4 : 3) : 1) * nbl * TPAD;  // [rt * kw][TPAD][16]
+    uint2* afr = reinterpret_cast<uint2*>(lds_all);  // [NG][nbl / 2][64]
+    float* lds = lds_all + (ALDS ? (size_t)NG * (nbl / 2) * 128 : 0);
+    const uint32_t nm = nbl * TPAD, as = NG * nm;  // scale entries of a token group; floats per array
+    float* red = ALDS ? lds_all : lds + (size_t)(SUMS ? (DUMP ? 4 : 3) : 1) * as;  // [rt * kw][NG][TPAD][16]
     uint32_t row0 = 0;  // first activation / output row of this launch unit
     if (GROUPED) {
         if (by >= (uint32_t)*grp.nchunks) return;  // uniform over the workgroup
@@ -205,11 +210,15 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         }
     };
 
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float acc[NG][4];
+#pragma unroll
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[g][i] = 0.0f;
     // `m`: index of the instruction along K (pair of blocks 2 m, 2 m + 1); with ALDS its operand comes from LDS
-    auto mfma = [&](v4i bw, uint32_t m, uint32_t d0, uint32_t d1) -> v4i {
+    auto mfma = [&](v4i bw, uint32_t m, int tg, uint32_t d0, uint32_t d1) -> v4i {
         if (ALDS) {
-            const uint2 av = afr[(size_t)(m - M0) * 64 + lane];
+            const uint2 av = afr[((size_t)tg * (nbl / 2) + (m - M0)) * 64 + lane];
             d0 = av.x;
             d1 = av.y;
         }
@@ -230,61 +239,77 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         if constexpr (FMT == FMT_Q8_0) {
             const float d = f16_bits_to_f32((uint16_t)(d_half ? st.dd >> 16 : st.dd & 0xFFFF));
             v4i bw = {(int)c.x, (int)c.y, (int)c.z, (int)c.w};
-            v4i D = mfma(bw, s, st.a[0], st.a[1]);
             const uint32_t b = 2 * s + d_half;
-            Meta4 m;
-            load_meta<TPAD, SUMS, DUMP>(lds, nbl, min(b, nblk - 1) - B0, d_tok0, m);
-            int isum[4] = {D.x, D.y, D.z, D.w};
 #pragma unroll
-            for (int i = 0; i < NI; i++) acc[i] = fmaf(d, m.xs[i] * (float)isum[i], acc[i]);
-            dump_block(b, isum);
+            for (int tg = 0; tg < NG; tg++) {
+                v4i D = mfma(bw, s, tg, st.a[0], st.a[1]);
+                Meta4 m;
+                load_meta<SUMS, DUMP>(lds, as, tg * nm + (min(b, nblk - 1) - B0) * TPAD + d_tok0, m);
+                int isum[4] = {D.x, D.y, D.z, D.w};
+#pragma unroll
+                for (int i = 0; i < NI; i++) acc[tg][i] = fmaf(d, m.xs[i] * (float)isum[i], acc[tg][i]);
+                dump_block(b, isum);
+            }
         } else if constexpr (FMT == FMT_Q4_K) {
             const float d = f16_bits_to_f32((uint16_t)(st.dd & 0xFFFF)), ndmin = -f16_bits_to_f32((uint16_t)(st.dd >> 16));
-            float P[4] = {0.0f, 0.0f, 0.0f, 0.0f}, Q[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            float P[NG][4], Q[NG][4];
+#pragma unroll
+            for (int tg = 0; tg < NG; tg++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) P[tg][i] = Q[tg][i] = 0.0f;
 #pragma unroll
             for (int pr = 0; pr < 2; pr++) {  // the two byte pairs of the lane's chunk
                 const uint32_t lo = pr ? c.z : c.x, hi = pr ? c.w : c.y;
                 v4i bw = {(int)(lo & 0x0F0F0F0Fu), (int)(hi & 0x0F0F0F0Fu), (int)((lo >> 4) & 0x0F0F0F0Fu),
                           (int)((hi >> 4) & 0x0F0F0F0Fu)};
-                v4i D = mfma(bw, 2 * s + pr, st.a[2 * pr], st.a[2 * pr + 1]);
                 const uint32_t b = 4 * s + 2 * pr + d_half;  // global index of this lane's block of 32
                 const uint32_t q = 2 * pr + d_half;
                 const float sc = (float)((st.sc4 >> (8 * q)) & 0xFF), mn = (float)((st.mn4 >> (8 * q)) & 0xFF);
-                Meta4 m;
-                load_meta<TPAD, SUMS, DUMP>(lds, nbl, b - B0, d_tok0, m);
-                const int U[4] = {D.x, D.y, D.z, D.w};
 #pragma unroll
-                for (int i = 0; i < NI; i++) {
-                    P[i] = fmaf(sc, fmaf(m.xs[i], (float)U[i], m.c[i]), P[i]);
-                    Q[i] = fmaf(mn, m.fs[i], Q[i]);
-                }
-                if (DUMP) {
-                    int isum[4] = {U[0] - 8 * m.su[0], U[1] - 8 * m.su[1], U[2] - 8 * m.su[2], U[3] - 8 * m.su[3]};
-                    dump_block(b, isum);
+                for (int tg = 0; tg < NG; tg++) {
+                    v4i D = mfma(bw, 2 * s + pr, tg, st.a[2 * pr], st.a[2 * pr + 1]);
+                    Meta4 m;
+                    load_meta<SUMS, DUMP>(lds, as, tg * nm + (b - B0) * TPAD + d_tok0, m);
+                    const int U[4] = {D.x, D.y, D.z, D.w};
+#pragma unroll
+                    for (int i = 0; i < NI; i++) {
+                        P[tg][i] = fmaf(sc, fmaf(m.xs[i], (float)U[i], m.c[i]), P[tg][i]);
+                        Q[tg][i] = fmaf(mn, m.fs[i], Q[tg][i]);
+                    }
+                    if (DUMP) {
+                        int isum[4] = {U[0] - 8 * m.su[0], U[1] - 8 * m.su[1], U[2] - 8 * m.su[2], U[3] - 8 * m.su[3]};
+                        dump_block(b, isum);
+                    }
                 }
             }
 #pragma unroll
-            for (int i = 0; i < NI; i++) acc[i] = fmaf(ndmin, Q[i], fmaf(d, P[i], acc[i]));
+            for (int tg = 0; tg < NG; tg++)
+#pragma unroll
+                for (int i = 0; i < NI; i++) acc[tg][i] = fmaf(ndmin, Q[tg][i], fmaf(d, P[tg][i], acc[tg][i]));
         } else {
 #pragma unroll
             for (int g = 0; g < 2; g++) {  // the two groups of 64 of the step
                 const uint32_t w0 = g ? c.z : c.x, w1 = g ? c.w : c.y;  // blocks 2 g, 2 g + 1
                 v4i bw = {(int)(w0 & 0x0F0F0F0Fu), (int)((w0 >> 4) & 0x0F0F0F0Fu), (int)(w1 & 0x0F0F0F0Fu),
                           (int)((w1 >> 4) & 0x0F0F0F0Fu)};
-                v4i D = mfma(bw, 2 * s + g, st.a[2 * g], st.a[2 * g + 1]);
                 const uint32_t b = 4 * s + 2 * g + d_half;
                 const float d = f16_bits_to_f32((uint16_t)(g ? st.dd >> 16 : st.dd & 0xFFFF));
                 const float off = bf16_bits_to_f32((uint16_t)(g ? st.oo >> 16 : st.oo & 0xFFFF));
-                Meta4 m;
-                load_meta<TPAD, SUMS, DUMP>(lds, nbl, min(b, nblk - 1) - B0, d_tok0, m);
-                const int U[4] = {D.x, D.y, D.z, D.w};
-                if (b < nblk) {  // padding blocks hold zero codes and zero scales, but their staged sums are a real block's
 #pragma unroll
-                    for (int i = 0; i < NI; i++) acc[i] = fmaf(off, m.fs[i], fmaf(d, fmaf(m.xs[i], (float)U[i], m.c[i]), acc[i]));
-                }
-                if (DUMP) {
-                    int isum[4] = {U[0] - 8 * m.su[0], U[1] - 8 * m.su[1], U[2] - 8 * m.su[2], U[3] - 8 * m.su[3]};
-                    dump_block(b, isum);
+                for (int tg = 0; tg < NG; tg++) {
+                    v4i D = mfma(bw, 2 * s + g, tg, st.a[2 * g], st.a[2 * g + 1]);
+                    Meta4 m;
+                    load_meta<SUMS, DUMP>(lds, as, tg * nm + (min(b, nblk - 1) - B0) * TPAD + d_tok0, m);
+                    const int U[4] = {D.x, D.y, D.z, D.w};
+                    if (b < nblk) {  // padding blocks hold zero codes and zero scales, but their staged sums are a real block's
+#pragma unroll
+                        for (int i = 0; i < NI; i++)
+                            acc[tg][i] = fmaf(off, m.fs[i], fmaf(d, fmaf(m.xs[i], (float)U[i], m.c[i]), acc[tg][i]));
+                    }
+                    if (DUMP) {
+                        int isum[4] = {U[0] - 8 * m.su[0], U[1] - 8 * m.su[1], U[2] - 8 * m.su[2], U[3] - 8 * m.su[3]};
+                        dump_block(b, isum);
+                    }
                 }
             }
         }
@@ -317,14 +342,14 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     auto act_store = [&](uint32_t i, const uint4* v) {
         if (FMT == FMT_Q4M) {
             const uint32_t tok = i / nb, b = i % nb;
-            uint2* dst = afr + (size_t)(b >> 1) * 64 + 8 * (b & 1) + tok;
+            uint2* dst = afr + ((size_t)(tok >> 3) * (nbl / 2) + (b >> 1)) * 64 + 8 * (b & 1) + (tok & 7);
             dst[0] = make_uint2(v[0].x, v[1].x);
             dst[16] = make_uint2(v[0].y, v[1].y);
             dst[32] = make_uint2(v[0].z, v[1].z);
             dst[48] = make_uint2(v[0].w, v[1].w);
         } else {
             const uint32_t tok = i / (2 * nb), c = i % (2 * nb), b = c >> 1;
-            uint2* dst = afr + (size_t)(b >> 1) * 64 + 32 * (c & 1) + 8 * (b & 1) + tok;
+            uint2* dst = afr + ((size_t)(tok >> 3) * (nbl / 2) + (b >> 1)) * 64 + 32 * (c & 1) + 8 * (b & 1) + (tok & 7);
             dst[0] = make_uint2(v[0].x, v[0].y);
             dst[16] = make_uint2(v[0].z, v[0].w);
         }
@@ -334,9 +359,9 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         float x, f;
         int sq;
     };
-    const uint32_t nm = nbl * TPAD;
+    const uint32_t nma = as;  // entries in all: entry i = (group i / nm, token (i % nm) / nbl of it, block i % nbl)
     auto meta_load = [&](uint32_t i, MetaReg& r) {
-        const uint32_t tok = i / nbl, b = i % nbl;  // consecutive threads read consecutive blocks of one token
+        const uint32_t tok = 8 * (i / nm) + (i % nm) / nbl, b = i % nbl;  // consecutive threads: consecutive blocks of a token
         const bool live = tok < t && B0 + b < nblk;
         const size_t src = (live ? src_row(tok) : 0) * nblk + B0 + (live ? b : 0);
         r.x = live ? xa.scales[src] : 0.0f;
@@ -344,12 +369,12 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         r.f = SUMS && live ? xa.fsums[src] : 0.0f;
     };
     auto meta_store = [&](uint32_t i, const MetaReg& r) {
-        const uint32_t tok = i / nbl, b = i % nbl;
-        lds[b * TPAD + tok] = r.x;
+        const uint32_t at = (i / nm) * nm + (i % nbl) * TPAD + (i % nm) / nbl;
+        lds[at] = r.x;
         if (SUMS) {
-            lds[(size_t)nm + b * TPAD + tok] = FMT == FMT_Q4_K ? 8.0f * (r.f - r.x * (float)r.sq) : -8.0f * (r.x * (float)r.sq);
-            lds[(size_t)2 * nm + b * TPAD + tok] = r.f;
-            if (DUMP) reinterpret_cast<int*>(lds)[(size_t)3 * nm + b * TPAD + tok] = r.sq;
+            lds[(size_t)as + at] = FMT == FMT_Q4_K ? 8.0f * (r.f - r.x * (float)r.sq) : -8.0f * (r.x * (float)r.sq);
+            lds[(size_t)2 * as + at] = r.f;
+            if (DUMP) reinterpret_cast<int*>(lds)[(size_t)3 * as + at] = r.sq;
         }
     };
     uint4 sa[SA];
@@ -361,7 +386,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         for (int j = 0; j < SA / AU; j++) act_load(min(threadIdx.x + j * nthr, na - 1), sa + AU * j);
     }
 #pragma unroll
-    for (int j = 0; j < SM; j++) meta_load(min(threadIdx.x + j * nthr, nm - 1), smr[j]);
+    for (int j = 0; j < SM; j++) meta_load(min(threadIdx.x + j * nthr, nma - 1), smr[j]);
     Step<FMT> ring[PF];
     const uint32_t slast = max(s1, 1u) - 1;
 #pragma unroll
@@ -374,7 +399,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
 #pragma unroll
     for (int j = 0; j < SM; j++) {
         const uint32_t i = threadIdx.x + j * nthr;
-        if (i < nm) meta_store(i, smr[j]);
+        if (i < nma) meta_store(i, smr[j]);
     }
     // what did not fit the registers (long rows, small workgroups) follows behind the weights
     for (uint32_t i = threadIdx.x + (SA / AU) * nthr; i < na; i += nthr) {
@@ -382,7 +407,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         act_load(i, v);
         act_store(i, v);
     }
-    for (uint32_t i = threadIdx.x + SM * nthr; i < nm; i += nthr) {
+    for (uint32_t i = threadIdx.x + SM * nthr; i < nma; i += nthr) {
         MetaReg r;
         meta_load(i, r);
         meta_store(i, r);
@@ -398,22 +423,26 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     }
     // the two block parities of a token meet across lane groups kq and kq ^ 2
 #pragma unroll
-    for (int i = 0; i < 4; i++) acc[i] += __shfl_xor(acc[i], 32);
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[g][i] += __shfl_xor(acc[g][i], 32);
     if (ALDS) __syncthreads();  // the partial sums overwrite the staged activations
     if (kq < 2) {
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            if (d_tok0 + i < (uint32_t)TPAD) red[((size_t)wave * TPAD + d_tok0 + i) * 16 + n] = acc[i];
+        for (int g = 0; g < NG; g++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (d_tok0 + i < (uint32_t)TPAD) red[(((size_t)wave * NG + g) * TPAD + d_tok0 + i) * 16 + n] = acc[g][i];
     }
     __syncthreads();
     // the waves of a tile in order; with one slice that is the result, else this slice's partial rows
     float* out = ksplit > 1 ? partial + (size_t)slice * t * w.n_out : y;
-    for (uint32_t idx = threadIdx.x; idx < rt * TPAD * 16; idx += nthr) {
-        const uint32_t rr = idx / (TPAD * 16), tok = (idx / 16) % TPAD, nn = idx % 16;
+    for (uint32_t idx = threadIdx.x; idx < rt * NG * TPAD * 16; idx += nthr) {
+        const uint32_t rr = idx / (NG * TPAD * 16), g = (idx / (TPAD * 16)) % NG, tok = 8 * g + (idx / 16) % TPAD, nn = idx % 16;
         const uint32_t row = (bx * rt + rr) * 16 + nn;
         if (tok >= t || row >= w.n_out || !y) continue;
         float sum = 0.0f;
-        for (uint32_t k = 0; k < kw; k++) sum += red[((size_t)(rr * kw + k) * TPAD + tok) * 16 + nn];
+        for (uint32_t k = 0; k < kw; k++) sum += red[((((size_t)rr * kw + k) * NG + g) * TPAD + (idx / 16) % TPAD) * 16 + nn];
         // partial rows go out as device-scope stores (written through to memory, where the other XCDs' L2s see them)
         if (ksplit > 1) __hip_atomic_store(out + (size_t)tok * w.n_out + row, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else out[(size_t)tok * w.n_out + row] = sum;
@@ -446,14 +475,16 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
 
 // Dynamic LDS is declared 16-byte aligned whatever static LDS a kernel also holds: the 8- and 16-byte LDS reads are split
 // into dwords (and the kernel runs two to three times longer) when the array starts at an odd dword.
-template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS>
-__global__ __launch_bounds__(1024) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw,
-                                                           float* __restrict__ y, int32_t* __restrict__ dump, GroupView grp,
-                                                           uint32_t ksplit, float* __restrict__ partial,
-                                                           uint32_t* __restrict__ counters) {
+// (Grouped launches keep to 8 waves, which leaves them 256 registers for the accumulators of their token groups.)
+template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS, int NG>
+__global__ __launch_bounds__(GROUPED ? 512 : 1024) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt,
+                                                                           uint32_t kw, float* __restrict__ y,
+                                                                           int32_t* __restrict__ dump, GroupView grp, uint32_t ksplit,
+                                                                           float* __restrict__ partial,
+                                                                           uint32_t* __restrict__ counters) {
     extern __shared__ __align__(16) float lds_dyn[];
-    decode_body<FMT, NT, DUMP, GROUPED, ALDS>(w, xa, t, rt, kw, y, dump, grp, ksplit, partial, counters, blockIdx.x, blockIdx.y,
-                                              blockDim.x, lds_dyn);
+    decode_body<FMT, NT, DUMP, GROUPED, ALDS, NG>(w, xa, t, rt, kw, y, dump, grp, ksplit, partial, counters, blockIdx.x, blockIdx.y,
+                                                  blockDim.x, lds_dyn);
 }
 
 // Several independent matmuls in one launch (the jobs of one Backend::matmul call, src/gpu.rs:160: Q/K/V, gate/up ...):
@@ -570,16 +601,16 @@ Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices, uint32_t co
 constexpr size_t LDS_MAX = 160 * 1024 - 256;  // dynamic LDS on offer (the kernel also holds a static word)
 
 // Dynamic LDS of a launch; `alds` comes back false when the operand-order activations do not fit.
-size_t lds_bytes(bool sums, bool dump, uint32_t bps, uint32_t nsteps, int tpad, const Shape& sh, bool* alds) {
+size_t lds_bytes(bool sums, bool dump, uint32_t bps, uint32_t nsteps, int tpad, const Shape& sh, bool* alds, uint32_t ng = 1) {
     const uint32_t nbl = bps * ((nsteps + sh.ks - 1) / sh.ks);  // blocks of a slice
-    const size_t meta = (size_t)(sums ? (dump ? 4 : 3) : 1) * nbl * tpad * 4, red = (size_t)sh.rt * sh.kw * tpad * 16 * 4;
-    const size_t act = (size_t)(nbl / 2) * 512;
+    const size_t meta = (size_t)(sums ? (dump ? 4 : 3) : 1) * ng * nbl * tpad * 4, red = (size_t)sh.rt * sh.kw * ng * tpad * 16 * 4;
+    const size_t act = (size_t)ng * (nbl / 2) * 512;
     const size_t with = act + meta > red ? act + meta : red;  // the partial sums reuse the activations' space
     *alds = with <= LDS_MAX;
     return *alds ? with : meta + red;
 }
 
-template <int FMT, int NT, bool DUMP, bool GROUPED>
+template <int FMT, int NT, bool DUMP, bool GROUPED, int NG = 1>
 hipError_t launch_one(bool alds, dim3 grid, dim3 block, size_t lds, hipStream_t s, const WeightView& w, const QActView& v, uint32_t t,
                       const Shape& sh, float* y, int32_t* dump, const GroupView& g, const DecodeScratch& sc) {
     hipError_t e = hipSuccess;
@@ -595,8 +626,9 @@ hipError_t launch_one(bool alds, dim3 grid, dim3 block, size_t lds, hipStream_t 
         }
         if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, v, t, sh.rt, sh.kw, y, dump, g, sh.ks, sc.partial, sc.counters);
     };
-    if (alds) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, true>);
-    else go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, false>);
+    if (alds) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, true, NG>);
+    else if constexpr (NG == 1) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, false, 1>);
+    else e = hipErrorInvalidValue;  // token groups need the staged activations
     return e != hipSuccess ? e : hipGetLastError();
 }
 
@@ -645,18 +677,29 @@ template <int FMT>
 hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks, uint32_t max_rows,
                        float* y, hipStream_t s) {
     const uint32_t ntiles = row_tiles(w.n_out), nsteps = steps_of<FMT>(w.n_in);
-    // grid y walks the chunks: no K slices across workgroups here (the shape still depends on the weight alone, so a
-    // token's row is bit-identical whatever else is in the group)
-    const Shape sh = shape_for(ntiles, nsteps, false, FMT == FMT_Q8_0 ? 64 : 128);
+    // grid y walks the chunks (no K slices across workgroups). Every workgroup stages its chunk's activations, so it
+    // takes as many row tiles as 8 waves allow, each wave keeping 16 records or more where K is long enough. The shape depends on the
+    // weight alone, so a token's row is bit-identical whatever else is in the group.
+    uint32_t gkw = 1;
+    while (gkw < 8 && nsteps / (gkw * 2) >= 16) gkw *= 2;
+    Shape sh{8 / gkw, gkw, 1};
+    if (const char* e = getenv("OXHIP_GROUPED_SHAPE")) {  // developer override for tuning runs: "rt,kw"
+        unsigned a = 0, b = 0;
+        if (sscanf(e, "%u,%u", &a, &b) == 2 && a >= 1 && b >= 1 && a * b <= 16) sh = Shape{a, b, 1};
+    }
     dim3 grid((ntiles + sh.rt - 1) / sh.rt, max_chunks), block(64 * sh.rt * sh.kw);
     const int tpad = max_rows <= 4 ? 4 : 8;
+    const uint32_t ng = max_rows <= 8 ? 1 : (max_rows <= 16 ? 2 : 4);
+    if (max_rows > 32) return hipErrorInvalidValue;
     bool alds;
-    const size_t lds = lds_bytes(FMT != FMT_Q8_0, false, FMT == FMT_Q8_0 ? 2 : 4, nsteps, tpad, sh, &alds);
-    if (lds > LDS_MAX) return hipErrorInvalidValue;
+    const size_t lds = lds_bytes(FMT != FMT_Q8_0, false, FMT == FMT_Q8_0 ? 2 : 4, nsteps, tpad, sh, &alds, ng);
+    if (lds > LDS_MAX || (ng > 1 && !alds)) return hipErrorInvalidValue;
     const DecodeScratch none{};
     if (max_rows == 1) return launch_one<FMT, 1, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
     if (max_rows <= 4) return launch_one<FMT, 4, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
-    return launch_one<FMT, 8, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
+    if (ng == 1) return launch_one<FMT, 8, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
+    if (ng == 2) return launch_one<FMT, 8, false, true, 2>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
+    return launch_one<FMT, 8, false, true, 4>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
 }
 
 }  // namespace

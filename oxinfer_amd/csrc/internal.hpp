@@ -107,10 +107,12 @@ uint32_t gemm_fp8_k_slices(const WeightView& w, size_t mtiles);
 hipError_t launch_gemm_fp8(const WeightView& w, const void* apk, const float* sx, size_t t, size_t mtiles, void* y, bool out_bf16,
                            float* partial, hipStream_t s);
 hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, hipStream_t s);
-hipError_t launch_moe_plan(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, int* row_of, int* src, int4* chunks,
-                           int* nchunks, hipStream_t s);
+hipError_t launch_moe_plan(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, uint32_t chunk_rows, int* row_of, int* src,
+                           int4* chunks, int* nchunks, hipStream_t s);
 hipError_t launch_moe_act(const float* g, const float* u, size_t stride, size_t rows, size_t inter, uint32_t kind, float param,
                           float* a, hipStream_t s);
+hipError_t launch_moe_act_quantize(const float* g, const float* u, size_t stride, size_t rows, size_t inter, uint32_t kind, float param,
+                                   const oxhip_qact& o, hipStream_t s);
 hipError_t launch_moe_combine(const float* o, const int* row_of, const float* route_w, size_t t, size_t k, size_t h, float* y,
                               hipStream_t s);
 

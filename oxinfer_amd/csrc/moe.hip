@@ -43,7 +43,7 @@ __global__ __launch_bounds__(64) void route_top_k_kernel(const float* __restrict
             }
         }
         seli[r] = bj;
-        sel[r] = l[bj];
+        sel[r] = __int_as_float(bk ^ (int)(((uint32_t)(bk >> 31)) >> 1));  // the key's transform is its own inverse
 #pragma unroll
         for (int i = 0; i < PER; i++)
             if (lane + 64 * i == bj) live[i] = false;
@@ -70,52 +70,78 @@ hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k,
 }
 
 // The plan of one pass: pairs (token i, slot j) -> gathered row, grouped by expert in (token, slot)
-// order, cut into chunks of at most 8 rows. One workgroup; thread e owns expert e.
+// order, cut into chunks of at most `cr` rows (8, 16 or 32). One workgroup: counts per expert, prefix sums, then each
+// pair takes the next free row of its expert (LDS counters; the route list is staged in LDS when it fits).
 //   row_of[i * k + j]  gathered row of the pair
 //   src[row]           token of a gathered row
 //   chunks[c]          {expert, first row, rows, 0}; *nchunks
+constexpr uint32_t PLAN_LDS_PAIRS = 24 * 1024;  // route entries kept in LDS (96 KiB); longer lists are read from L2
 __global__ __launch_bounds__(1024) void moe_plan_kernel(const uint32_t* __restrict__ route_idx, uint32_t pairs, uint32_t k,
-                                                        uint32_t n_exp, int* __restrict__ row_of, int* __restrict__ src,
+                                                        uint32_t n_exp, int cr, int* __restrict__ row_of, int* __restrict__ src,
                                                         int4* __restrict__ chunks, int* __restrict__ nchunks) {
     extern __shared__ int sh[];
-    int* cnt = sh;               // [n_exp]
-    int* start = sh + n_exp;     // [n_exp]
+    int* cnt = sh;                 // [n_exp]
+    int* start = sh + n_exp;       // [n_exp]
     int* cstart = sh + 2 * n_exp;  // [n_exp]
-    for (uint32_t e = threadIdx.x; e < n_exp; e += blockDim.x) cnt[e] = 0;
+    int* fill = sh + 3 * n_exp;    // [n_exp]
+    uint32_t* routes = reinterpret_cast<uint32_t*>(sh + 4 * n_exp);
+    const bool staged = pairs <= PLAN_LDS_PAIRS;
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (uint32_t e = threadIdx.x; e < n_exp; e += blockDim.x) cnt[e] = fill[e] = 0;
     __syncthreads();
-    for (uint32_t i = threadIdx.x; i < pairs; i += blockDim.x) atomicAdd(&cnt[route_idx[i]], 1);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int r = 0, c = 0;
-        for (uint32_t e = 0; e < n_exp; e++) {
-            start[e] = r;
-            cstart[e] = c;
-            r += cnt[e];
-            c += (cnt[e] + 7) / 8;
-        }
-        *nchunks = c;
+    for (uint32_t i = threadIdx.x; i < pairs; i += blockDim.x) {
+        const uint32_t e = route_idx[i];
+        if (staged) routes[i] = e;
+        atomicAdd(&cnt[e], 1);
     }
     __syncthreads();
-    for (uint32_t e = threadIdx.x; e < n_exp; e += blockDim.x) {
-        const int n = cnt[e];
-        if (!n) continue;
-        int pos = start[e];
-        for (uint32_t i = 0; i < pairs && pos < start[e] + n; i++) {
-            if (route_idx[i] == e) {
-                row_of[i] = pos;
-                src[pos] = (int)(i / k);
-                pos++;
+    if (wave == 0) {  // exclusive prefix sums over the experts: each lane owns a run of experts, the runs meet by a wave scan
+        const uint32_t per = (n_exp + 63) / 64, e0 = lane * per, e1 = min(n_exp, e0 + per);
+        int r = 0, c = 0;
+        for (uint32_t e = e0; e < e1; e++) {
+            r += cnt[e];
+            c += (cnt[e] + cr - 1) / cr;
+        }
+        int rs = r, cs = c;  // inclusive scan over lanes
+        for (int d = 1; d < 64; d <<= 1) {
+            const int ro = __shfl_up(rs, d), co = __shfl_up(cs, d);
+            if ((int)lane >= d) {
+                rs += ro;
+                cs += co;
             }
         }
-        for (int c = 0; c < (n + 7) / 8; c++) chunks[cstart[e] + c] = make_int4((int)e, start[e] + 8 * c, min(8, n - 8 * c), 0);
+        int rb = rs - r, cb = cs - c;
+        for (uint32_t e = e0; e < e1; e++) {
+            start[e] = rb;
+            cstart[e] = cb;
+            rb += cnt[e];
+            cb += (cnt[e] + cr - 1) / cr;
+        }
+        if (lane == 63) *nchunks = cs;
+    }
+    __syncthreads();
+    // a pair's place inside its expert's run is the order of arrival: which rows share a chunk varies from run to run,
+    // but a row's result does not depend on its chunk (every (token, row) sum is formed on its own, in a fixed order)
+    for (uint32_t i = threadIdx.x; i < pairs; i += blockDim.x) {
+        const uint32_t e = staged ? routes[i] : route_idx[i];
+        const int r = start[e] + atomicAdd(&fill[e], 1);
+        row_of[i] = r;
+        src[r] = (int)(i / k);
+    }
+    for (uint32_t e = threadIdx.x; e < n_exp; e += blockDim.x) {
+        const int n = cnt[e];
+        for (int c = 0; c < (n + cr - 1) / cr; c++) chunks[cstart[e] + c] = make_int4((int)e, start[e] + cr * c, min(cr, n - cr * c), 0);
     }
 }
 
-hipError_t launch_moe_plan(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, int* row_of, int* src, int4* chunks,
-                           int* nchunks, hipStream_t s) {
-    unsigned threads = (unsigned)(n_exp < 64 ? 64 : (n_exp > 1024 ? 1024 : (n_exp + 63) / 64 * 64));
-    moe_plan_kernel<<<1, threads, 3 * n_exp * sizeof(int), s>>>(route_idx, (uint32_t)pairs, (uint32_t)k, (uint32_t)n_exp, row_of, src,
-                                                               chunks, nchunks);
+hipError_t launch_moe_plan(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, uint32_t chunk_rows, int* row_of, int* src,
+                           int4* chunks, int* nchunks, hipStream_t s) {
+    const size_t lds = 4 * n_exp * sizeof(int) + (pairs <= PLAN_LDS_PAIRS ? pairs * sizeof(uint32_t) : 0);
+    if (lds > 48 * 1024) {  // once per pass: not worth caching per device
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(moe_plan_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+        if (e != hipSuccess) return e;
+    }
+    moe_plan_kernel<<<1, 1024, lds, s>>>(route_idx, (uint32_t)pairs, (uint32_t)k, (uint32_t)n_exp, (int)chunk_rows, row_of, src, chunks, nchunks);
     return hipGetLastError();
 }
 
@@ -158,6 +184,86 @@ hipError_t launch_moe_act(const float* g, const float* u, size_t stride, size_t 
     size_t total = rows * inter;
     if (!total) return hipSuccess;
     moe_act_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(g, u, stride, rows, (uint32_t)inter, kind, param, a);
+    return hipGetLastError();
+}
+
+// The same, followed by quantize_act on the result (src/quant.rs:267-292) without the round trip through memory: one
+// lane per block of 32 of a; bit-identical to moe_act_kernel + quantize_act_kernel. `a` (optional) also keeps the
+// f32 values.
+__global__ __launch_bounds__(64) void moe_act_quantize_kernel(const float* __restrict__ gp, const float* __restrict__ up, size_t stride,
+                                                             size_t rows, uint32_t inter, uint32_t kind, float param,
+                                                             int8_t* __restrict__ q, float* __restrict__ scales, int32_t* __restrict__ sums,
+                                                             float* __restrict__ fsums, float* __restrict__ hsums,
+                                                             int32_t* __restrict__ sums16) {
+    const size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x, bpr = inter / 32;
+    if (b >= rows * bpr) return;
+    const size_t r = b / bpr, j0 = (b % bpr) * 32;
+    const float4* g4 = reinterpret_cast<const float4*>(gp + r * stride + j0);
+    const float4* u4 = reinterpret_cast<const float4*>(up + r * stride + j0);
+    float v[32];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const float4 gg = g4[i], uu = u4[i];
+        const float gs[4] = {gg.x, gg.y, gg.z, gg.w}, us[4] = {uu.x, uu.y, uu.z, uu.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float g = gs[e], u = us[e];
+            if (kind == 1) {
+                const float K2 = 2.0f * 0.7978846f;
+                const float t = K2 * (g + 0.044715f * g * g * g);
+                v[4 * i + e] = g / (1.0f + fast_exp(-t)) * u;
+            } else {
+                if (kind == 2) {
+                    g = fminf(g, param);
+                    u = fminf(fmaxf(u, -param), param);
+                }
+                v[4 * i + e] = g / (1.0f + fast_exp(-g)) * u;
+            }
+        }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) amax = fmaxf(amax, fabsf(v[i]));
+    const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+    float h0 = -0.0f, h1 = -0.0f, f = -0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) h0 += v[i];
+#pragma unroll
+    for (int i = 16; i < 32; i++) h1 += v[i];
+#pragma unroll
+    for (int i = 0; i < 32; i++) f += v[i];
+    int s0 = 0, s1 = 0;
+    uint32_t packed[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        uint32_t wv = 0;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float rr = roundf(v[4 * i + e] * inv);
+            const int iv = rr != rr ? 0 : (int)fminf(fmaxf(rr, -128.0f), 127.0f);
+            if (i < 4) s0 += iv; else s1 += iv;
+            wv |= ((uint32_t)iv & 0xFF) << (8 * e);
+        }
+        packed[i] = wv;
+    }
+    uint4* dst = reinterpret_cast<uint4*>(q + b * 32);
+    dst[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    dst[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
+    scales[b] = amax / 127.0f;
+    sums[b] = s0 + s1;
+    fsums[b] = f;
+    hsums[2 * b] = h0;
+    hsums[2 * b + 1] = h1;
+    sums16[2 * b] = s0;
+    sums16[2 * b + 1] = s1;
+}
+
+hipError_t launch_moe_act_quantize(const float* g, const float* u, size_t stride, size_t rows, size_t inter, uint32_t kind, float param,
+                                   const oxhip_qact& o, hipStream_t s) {
+    const size_t blocks = rows * (inter / 32);
+    if (!blocks) return hipSuccess;
+    moe_act_quantize_kernel<<<(unsigned)((blocks + 63) / 64), 64, 0, s>>>(g, u, stride, rows, (uint32_t)inter, kind, param, o.q, o.scales, o.sums,
+                                                                        o.fsums, o.hsums, o.sums16);
     return hipGetLastError();
 }
 
