@@ -213,7 +213,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     // before they are dequantized into the other LDS buffer.
     Raw raw[2];
     load_raw(raw, 0);
-    uint4 a_cur[4][4], a_nxt[4][4], b_cur[WG_NT], b_nxt[WG_NT];
+    // Each fragment has one home: a_cur[b] is refilled with block b of the next step as soon as this step's block b has
+    // been issued (a whole K-step ahead of its use), b_cur[j] with the next block's row tile j right after the four
+    // MFMAs that read it.
+    uint4 a_cur[4][4], b_cur[WG_NT];
     read_a_step(a_cur, 0);
     dequant_tile(raw[0], 0, 0);
     dequant_tile(raw[1], 1, 0);
@@ -221,46 +224,29 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     lds_barrier();
     read_b(b_cur, 0, 0);
     // One K-step. MORE: another step follows (its records are dequantized during blocks 0 and 1, and block 3
-    // prefetches from the other LDS buffer after the barrier). LOAD2: the records of step s + 2 exist.
-    // The steady-state instance has no branches, so the whole step is scheduled as one region and the dequantizing
-    // VALU work is interleaved with the MFMAs instead of stalling the matrix pipe.
+    // refills from the other LDS buffer after the barrier). LOAD2: the records of step s + 2 exist.
     auto step = [&](uint32_t s, auto more_c, auto load2_c) {
         constexpr bool MORE = decltype(more_c)::value, LOAD2 = decltype(load2_c)::value;
         const uint32_t buf = s & 1;
-        if (MORE) read_a_step(a_nxt, s + 1);
 #pragma unroll
         for (int b = 0; b < 4; b++) {
-            if (b < 3) {
-                read_b(b_nxt, buf, b + 1);
-            } else if (MORE) {
-                lds_barrier();  // the other buffer is complete, and nobody still reads this one
-                read_b(b_nxt, buf ^ 1, 0);
-            }
+            if (b == 3 && MORE) lds_barrier();  // the other buffer is complete, and nobody still reads this one
 #pragma unroll
             for (int j = 0; j < WG_NT; j++) {
                 const bf16x8 bb = __builtin_bit_cast(bf16x8, b_cur[j]);
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_cur[b][i]), bb, acc[i][j], 0, 0, 0);
+                if (b < 3) b_cur[j] = bfrag[((buf * 4 + b + 1) * WG_NT + j) * 64 + lane];
+                else if (MORE) b_cur[j] = bfrag[(((buf ^ 1) * 4) * WG_NT + j) * 64 + lane];
+            }
+            if (MORE) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) a_cur[b][i] = abase[i][(size_t)(4 * (s + 1) + b) * 64];
             }
             if (MORE && b == 0) dequant_tile(raw[0], 0, buf ^ 1);
             if (MORE && b == 1) dequant_tile(raw[1], 1, buf ^ 1);
             if (LOAD2 && b == 2) load_raw(raw, s + 2);
-            if (MORE && b < 2) {
-#pragma unroll
-                for (int k = 0; k < 32; k++) {  // one MFMA, then a few of the dequantizing VALU ops in its shadow
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < WG_NT; j++) b_cur[j] = b_nxt[j];
-        }
-        if (MORE) {
-#pragma unroll
-            for (int b = 0; b < 4; b++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) a_cur[b][i] = a_nxt[b][i];
         }
     };
     using T_ = std::integral_constant<bool, true>;
