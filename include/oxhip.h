@@ -94,8 +94,10 @@ void oxhip_free_weight(oxhip_ctx* ctx, oxhip_weight* w);
 /* Bytes the weight occupies in HBM. */
 size_t oxhip_weight_bytes(const oxhip_weight* w);
 /* Backend::matmul (src/gpu.rs:160; src/cuda.rs:1428-1493): all jobs share x [t, n_in] (host f32);
- * computes every job or none. t <= 16 runs the int8 decode kernels (the CPU's decode semantics,
- * src/kernels.rs:1908-1928); more tokens run the MFMA GEMM. */
+ * computes every job or none. Routing as matmul_quant_multi_at's (src/kernels.rs:1731-1879): up to 8 tokens the
+ * Q8_0 / Q4_K / MLX 4-bit jobs share one launch of the int8 decode kernel (the CPU's decode semantics,
+ * src/kernels.rs:1908-1928); more than 16 tokens over MLX 4-bit or FP8 (128-column blocks) weights run the bf16
+ * matrix-core GEMM; everything else runs the decode kernels over 16 tokens at a time. */
 int oxhip_matmul(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_job* jobs, size_t n_jobs);
 /* Backend::matvec_rows (src/gpu.rs:165): t in 1..=4. */
 int oxhip_matvec_rows(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_rows_job* jobs, size_t n_jobs);
@@ -134,9 +136,14 @@ int oxhip_dev_dequantize(oxhip_ctx* ctx, const oxhip_weight* w, size_t r0, size_
  * (`dense`, src/ggml.rs:1370): they take f32 rows `x` instead and `xa` may be NULL. */
 int oxhip_dev_decode(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa, const float* x, size_t t, float* y,
                      void* stream);
-/* Several decode launches in one call (a decode step issues many small matmuls; what
- * matmul_quant_batch does for the CPU, src/kernels.rs:1937-1994). Jobs run in order on `stream`;
- * ev_start / ev_stop (from oxhip_event_create, or NULL) are recorded around that job's launches. */
+/* Several independent decode matmuls in one call (a decode step issues many small matmuls; what
+ * matmul_quant_batch does for the CPU, src/kernels.rs:1937-1994). The jobs must not depend on one another: runs of
+ * consecutive jobs of at most 8 tokens over Q8_0 / Q4_K / MLX 4-bit weights share ONE launch (their latency chains
+ * overlap; every job's rows are bit-identical to a launch of its own), the others launch one by one, in order, on
+ * `stream`. ev_start / ev_stop (from oxhip_event_create, or NULL) are recorded before / after the launch that
+ * holds the job: for jobs that share a launch they bracket the whole shared launch.
+ * The decode entry points use scratch owned by ctx (partial rows of K slices): launches on one ctx must be ordered
+ * (one stream, or the caller's own synchronization). */
 typedef struct {
     const oxhip_weight* w;
     const oxhip_qact* xa; /* quantized weights */

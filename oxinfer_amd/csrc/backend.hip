@@ -438,10 +438,6 @@ int oxhip_matmul(oxhip_ctx* c, const float* x, size_t t, size_t n_in, oxhip_job*
         set_error("matmul: bad arguments");
         return 0;
     }
-    if (t > 16) {
-        set_error("matmul: more than 16 tokens take the prefill GEMM, which this build does not route here yet");
-        return 0;
-    }
     size_t y_total = 0;
     bool any_q = false;
     for (size_t j = 0; j < n_jobs; j++) {
@@ -488,15 +484,61 @@ int oxhip_matmul(oxhip_ctx* c, const float* x, size_t t, size_t n_in, oxhip_job*
         }
     }
     float* yd = static_cast<float*>(c->y.p);
+    // Routing, as matmul_quant_multi_at does (src/kernels.rs:1731-1879): up to 8 tokens the jobs that the matrix-core
+    // decode kernel takes share one launch; more than 16 tokens go to the prefill GEMM where the format has one (MLX
+    // 4-bit, FP8 with 128-column blocks: bf16 matrix cores, f32 accumulation); everything else runs the decode
+    // kernels over 16 tokens at a time.
+    std::vector<DecodeBatchItem> fused;
+    std::vector<size_t> offs(n_jobs);
     size_t off = 0;
     for (size_t j = 0; j < n_jobs; j++) {
+        offs[j] = off;
+        off += t * jobs[j].w->v.n_out;
+    }
+    auto fail = [&](const char* what) {
+        set_error(std::string("matmul: ") + what);
+        (void)hipStreamSynchronize(s);
+        return done(0);
+    };
+    for (size_t j = 0; j < n_jobs; j++) {
         const oxhip_weight* w = jobs[j].w;
-        if (launch_decode(w->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off, s, c->dec) != hipSuccess) {
-            set_error("matmul: decode launch failed");
-            (void)hipStreamSynchronize(s);
-            return done(0);
+        if (t <= 8 && !is_dense(w) && decode_batchable(w->v, t)) {
+            fused.push_back(DecodeBatchItem{w->v, view_of(xa), yd + offs[j], (uint32_t)t});
+            continue;
         }
-        off += t * w->v.n_out;
+        const bool gemm = t > 16 && (w->v.fmt == FMT_Q4M || (w->v.fmt == FMT_FP8 && w->v.br % 16 == 0 && w->v.bc % 128 == 0 && n_in % 128 == 0));
+        if (gemm) {
+            if (!gemm_bf16_run(c, w, c->x.p, false, t, yd + offs[j], false, s)) {
+                (void)hipStreamSynchronize(s);
+                return done(0);
+            }
+            continue;
+        }
+        for (size_t c0 = 0; c0 < t; c0 += 16) {
+            const size_t tc = t - c0 < 16 ? t - c0 : 16;
+            QActView v = view_of(xa);
+            if (!is_dense(w)) {
+                v.q += c0 * n_in;
+                v.scales += c0 * (n_in / 32);
+                v.sums += c0 * (n_in / 32);
+                v.fsums += c0 * (n_in / 32);
+                v.hsums += c0 * (n_in / 16);
+                v.sums16 += c0 * (n_in / 16);
+            }
+            if (launch_decode(w->v, v, static_cast<const float*>(c->x.p) + c0 * n_in, tc, yd + offs[j] + c0 * w->v.n_out, s, c->dec) != hipSuccess)
+                return fail("decode launch failed");
+        }
+    }
+    if (fused.size() == 1) {
+        if (launch_decode(fused[0].w, fused[0].xa, nullptr, t, fused[0].y, s, c->dec) != hipSuccess) return fail("decode launch failed");
+    } else if (!fused.empty()) {
+        hipError_t e = launch_decode_mfma_batch(fused.data(), fused.size(), c->dec, s);
+        if (e == hipErrorOutOfMemory) {
+            for (auto& it : fused)
+                if (launch_decode(it.w, it.xa, nullptr, t, it.y, s, c->dec) != hipSuccess) return fail("decode launch failed");
+        } else if (e != hipSuccess) {
+            return fail("decode batch launch failed");
+        }
     }
     (void)hipEventRecord(e2, s);
     if (hipStreamSynchronize(s) != hipSuccess) {

@@ -67,6 +67,9 @@ struct oxhip_ctx {
 
 namespace oxhip {
 
+// backend_gemm.hip: packs x and runs the bf16-matrix-core GEMM (1 = done, 0 = declined with the error set)
+int gemm_bf16_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf16, size_t t, void* y, bool y_bf16, hipStream_t s);
+
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 inline QActView view_of(const oxhip_qact& a) { return QActView{a.q, a.scales, a.sums, a.fsums, a.hsums, a.sums16}; }

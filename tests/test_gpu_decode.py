@@ -233,12 +233,24 @@ def test_host_matmul_matches_device_path_and_declines(be, oxref):
     n_in = 512
     raws = [(k, n, oxref.random_blocks(k, n * n_in // oxref.block_size(k), 31 + k)[0]) for k, n in ((Q4_K, 24), (Q6_K, 8), (Q8_0, 40))]
     ws = [be.upload_gguf(k, raw, n, n_in) for k, n, raw in raws]
-    for t in (1, 3, 9):
+    for t in (1, 3, 9, 16, 17, 40):   # up to 8 tokens the Q4_K and Q8_0 jobs share a launch; past 16 the rows go in slices
         x = lcg_input(t, n_in, 40 + t, oxref)
         ys = [np.full((t, n), np.nan, np.float32) for _, n, _ in raws]
         assert be.matmul(x, t, n_in, list(zip(ws, ys))), be.last_error()
         for (k, n, raw), y in zip(raws, ys):
             assert row_err(y, oxref.gguf_decode(k, raw, n, n_in, x, t)) < TOL
+    # more than 16 tokens over MLX 4-bit and FP8 weights take the prefill GEMM (bf16 matrix cores: 2e-2 of the f32 product)
+    from oxinfer_amd import synth
+    t, n_out = 40, 48
+    wq, sc, bi = synth.mlx_q4(n_out, n_in, 3)
+    q, s16, off = oxref.from_mlx_q4(wq, sc, bi, n_out, n_in, 64)
+    data, scales = synth.fp8_e4m3(n_out, n_in, 4)
+    wm, wf = be.upload_mlx_q4(wq, sc, bi, 64, n_out, n_in), be.upload_fp8(data, scales, n_out, n_in)
+    x = synth.activations(t, n_in, 5)
+    ym, yf = np.full((t, n_out), np.nan, np.float32), np.full((t, n_out), np.nan, np.float32)
+    assert be.matmul(x, t, n_in, [(wm, ym), (wf, yf)]), be.last_error()
+    assert row_err(ym, oxref.gemm_quant(-1, q, s16, off, n_out, n_in, x, t)) < 2e-2
+    assert row_err(yf, oxref.gemm_quant(oxref.F8E4M3, data, scales, None, n_out, n_in, x, t)) < 2e-2
     # a job whose weight has another n_in: declined, and nothing is written
     other = be.upload_gguf(Q8_0, oxref.random_blocks(Q8_0, 8 * 64 // 32, 1)[0], 8, 64)
     y0, y1 = np.full((1, 24), np.nan, np.float32), np.full((1, 8), np.nan, np.float32)
