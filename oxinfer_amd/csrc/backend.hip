@@ -250,13 +250,22 @@ oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) {
                 w->v.br = d->bs_rows;
                 w->v.bc = d->bs_cols;
                 size_t ns = ((n_out + d->bs_rows - 1) / d->bs_rows) * ((n_in + d->bs_cols - 1) / d->bs_cols);
-                pl.add(0, n_out * n_in);
+                const bool tiled = fp8_tileable(n_in, d->bs_rows, d->bs_cols);
+                w->v.group = tiled ? 1 : 0;
+                pl.add(0, tiled ? (size_t)row_tiles((uint32_t)n_out) * (n_in / 128) * 2048 : n_out * n_in);
                 pl.add(1, ns * 4);
                 if (!alloc(pl, 2)) return fail("device memory short");
                 uint8_t* b = static_cast<uint8_t*>(w->base);
-                if (hipMemcpyAsync(b + pl.off[0], d->data, n_out * n_in, hipMemcpyHostToDevice, s) != hipSuccess ||
-                    hipMemcpyAsync(b + pl.off[1], d->block_scales, ns * 4, hipMemcpyHostToDevice, s) != hipSuccess)
+                if (hipMemcpyAsync(b + pl.off[1], d->block_scales, ns * 4, hipMemcpyHostToDevice, s) != hipSuccess) return fail("copy failed");
+                if (tiled) {
+                    Temp raw;
+                    if (!raw.put(d->data, n_out * n_in, s)) return fail("device memory short");
+                    if (launch_pack_fp8(static_cast<const uint8_t*>(raw.p), n_out, n_in, b + pl.off[0], s) != hipSuccess)
+                        return fail("pack launch failed");
+                    if (hipStreamSynchronize(s) != hipSuccess) return fail("pack failed");
+                } else if (hipMemcpyAsync(b + pl.off[0], d->data, n_out * n_in, hipMemcpyHostToDevice, s) != hipSuccess) {
                     return fail("copy failed");
+                }
                 break;
             }
             size_t raw_bytes;

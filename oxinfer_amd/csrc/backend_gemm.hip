@@ -12,6 +12,18 @@ int gemm_bf16_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf1
         set_error("gemm: the bf16 variant runs MLX 4-bit weights and FP8 weights whose rows are multiples of 128");
         return 0;
     }
+    if (fp8 && skinny_fp8_ok(w->v, t)) {  // up to 32 tokens: bandwidth-bound, one pass over the weights
+        const size_t need = skinny_fp8_pack_bytes(w->v, t, 1);
+        if (c->gemm_ws.cap < need) {
+            (void)hipStreamSynchronize(s);
+            if (!c->gemm_ws.grow(need)) {
+                set_error("gemm: device memory short");
+                return 0;
+            }
+        }
+        HIP_TRY(launch_skinny_fp8(w->v, x, x_bf16, false, t, y, y_bf16, c->gemm_ws.p, s), "fp8 skinny launch");
+        return 1;
+    }
     const size_t mtiles = (t + 15) / 16, kblocks = 4 * (size_t)((w->v.n_in + 127) / 128);
     const size_t pack_bytes = align_up(mtiles * kblocks * 64 * 16, 256);
     const uint32_t slices = gemm_k_slices(w->v, mtiles);

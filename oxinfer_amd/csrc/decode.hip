@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void decode_dense_kernel(WeightView w, const f
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 uint32_t row = min(r0 + r, w.n_out - 1);
-                uint4 v = *reinterpret_cast<const uint4*>(w.p0 + ((size_t)row * units + u) * 16);
+                uint4 v = *reinterpret_cast<const uint4*>(w.p0 + (FMT == FMT_FP8 ? fp8_offset(w, row, (size_t)u * 16) : ((size_t)row * units + u) * 16));
                 uint32_t d[4] = {v.x, v.y, v.z, v.w};
                 if (FMT == FMT_FP8) {
 #pragma unroll
@@ -340,7 +340,11 @@ hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x
         case FMT_Q4M: return launch_decode_mfma(w, xa, t, y, sc, s);
         case FMT_Q4: return decode_t<FMT_Q4, 4>(w, xa, t, y, s);
         case FMT_Q6_K: return decode_t<FMT_Q6_K, 4>(w, xa, t, y, s);
-        case FMT_FP8: return decode_dense_t<FMT_FP8, 4>(w, x, t, y, s);
+        case FMT_FP8:
+            // the matrix-core kernel when the block scales allow it and the caller's scratch holds the packed activations
+            if (skinny_fp8_ok(w, t) && sc.partial && skinny_fp8_pack_bytes(w, t, 2) <= sc.partial_floats * 4)
+                return launch_skinny_fp8(w, x, false, true, t, y, false, sc.partial, s);
+            return decode_dense_t<FMT_FP8, 4>(w, x, t, y, s);
         case FMT_BF16: return decode_dense_t<FMT_BF16, 4>(w, x, t, y, s);
         default: return hipErrorInvalidValue;
     }

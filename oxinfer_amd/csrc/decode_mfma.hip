@@ -91,19 +91,16 @@ struct Step;
 template <>
 struct Step<FMT_Q8_0> {
     uint4 w;
-    uint32_t dd;
     uint32_t a[2];
 };
 template <>
 struct Step<FMT_Q4_K> {
     uint4 w;
-    uint32_t sc4, mn4, dd;
     uint32_t a[4];
 };
 template <>
 struct Step<FMT_Q4M> {
     uint4 w;
-    uint32_t dd, oo;
     uint32_t a[4];
 };
 
@@ -181,15 +178,10 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         if constexpr (FMT == FMT_Q8_0) {
             const uint8_t* rec = base + (size_t)s * T8_REC;
             st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
-            st.dd = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
             if (!ALDS) act2(2 * s + a_half, 8 * kq, st.a);
         } else if constexpr (FMT == FMT_Q4_K) {
             const uint8_t* rec = base + (size_t)(s >> 1) * TK4_REC;
             st.w = *reinterpret_cast<const uint4*>(rec + (s & 1) * 1024 + 16 * lane);
-            // this step's four sub-blocks are 4 (s & 1) .. + 3 of the super-block
-            st.sc4 = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 4 * (s & 1));
-            st.mn4 = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
-            st.dd = *reinterpret_cast<const uint32_t*>(rec + 2304 + 4 * n);
             if (!ALDS) {
                 act2(4 * s + a_half, 8 * kq, st.a);
                 act2(4 * s + 2 + a_half, 8 * kq, st.a + 2);
@@ -197,8 +189,6 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         } else {
             const uint8_t* rec = base + (size_t)s * T4M_REC;
             st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
-            st.dd = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
-            st.oo = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
             if (!ALDS) {
 #pragma unroll
                 for (int g = 0; g < 2; g++) {  // positions 4 kq.. and 16 + 4 kq.. of block 4 s + 2 g + half
@@ -208,6 +198,34 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                 }
             }
         }
+    };
+
+    // The records' scales: a request costs the memory pipeline the same for 64 bytes as for 1 KiB, and one per step
+    // and scale word (1 to 3) would cost more than the weights themselves. So one request serves four steps: lane group
+    // kq asks for the words of step `first + kq` (row n of it), and at step first + q every lane takes them from lane
+    // 16 q + n. Q8_0: {d of the two blocks}; Q4_K: {four sub-block scales, four mins, (d, dmin)}: this step's four
+    // sub-blocks are 4 (s & 1) .. + 3 of the super-block; MLX: {d of the two groups, offsets of the two groups}.
+    constexpr int NM = FMT == FMT_Q8_0 ? 1 : FMT == FMT_Q4_K ? 3 : 2;
+    const uint32_t slast = max(s1, 1u) - 1;
+    auto load_scales = [&](uint32_t* m, uint32_t first) {
+        const uint32_t s = min(first + kq, slast);
+        if constexpr (FMT == FMT_Q8_0) {
+            m[0] = *reinterpret_cast<const uint32_t*>(base + (size_t)s * T8_REC + 1024 + 4 * n);
+        } else if constexpr (FMT == FMT_Q4_K) {
+            const uint8_t* rec = base + (size_t)(s >> 1) * TK4_REC;
+            m[0] = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 4 * (s & 1));
+            m[1] = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
+            m[2] = *reinterpret_cast<const uint32_t*>(rec + 2304 + 4 * n);
+        } else {
+            const uint8_t* rec = base + (size_t)s * T4M_REC;
+            m[0] = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
+            m[1] = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
+        }
+    };
+    const int take0 = (int)(4 * n);  // byte index of lane n for the lane-to-lane read; + 64 q: lane 16 q + n
+    auto scales_of = [&](const uint32_t* grp, int q, uint32_t* m) {
+#pragma unroll
+        for (int j = 0; j < NM; j++) m[j] = (uint32_t)__builtin_amdgcn_ds_bpermute(take0 + 64 * q, (int)grp[j]);
     };
 
     float acc[NG][4];
@@ -234,10 +252,10 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         for (int i = 0; i < 4; i++)
             if (d_tok0 + i < t) dump[((size_t)(d_tok0 + i) * w.n_out + row) * nblk + b] = isum[i];
     };
-    auto compute_step = [&](const Step<FMT>& st, uint32_t s) {
+    auto compute_step = [&](const Step<FMT>& st, const uint32_t* sw, uint32_t s) {
         const uint4 c = st.w;
         if constexpr (FMT == FMT_Q8_0) {
-            const float d = f16_bits_to_f32((uint16_t)(d_half ? st.dd >> 16 : st.dd & 0xFFFF));
+            const float d = f16_bits_to_f32((uint16_t)(d_half ? sw[0] >> 16 : sw[0] & 0xFFFF));
             v4i bw = {(int)c.x, (int)c.y, (int)c.z, (int)c.w};
             const uint32_t b = 2 * s + d_half;
 #pragma unroll
@@ -251,7 +269,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                 dump_block(b, isum);
             }
         } else if constexpr (FMT == FMT_Q4_K) {
-            const float d = f16_bits_to_f32((uint16_t)(st.dd & 0xFFFF)), ndmin = -f16_bits_to_f32((uint16_t)(st.dd >> 16));
+            const float d = f16_bits_to_f32((uint16_t)(sw[2] & 0xFFFF)), ndmin = -f16_bits_to_f32((uint16_t)(sw[2] >> 16));
             float P[NG][4], Q[NG][4];
 #pragma unroll
             for (int tg = 0; tg < NG; tg++)
@@ -264,7 +282,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                           (int)((hi >> 4) & 0x0F0F0F0Fu)};
                 const uint32_t b = 4 * s + 2 * pr + d_half;  // global index of this lane's block of 32
                 const uint32_t q = 2 * pr + d_half;
-                const float sc = (float)((st.sc4 >> (8 * q)) & 0xFF), mn = (float)((st.mn4 >> (8 * q)) & 0xFF);
+                const float sc = (float)((sw[0] >> (8 * q)) & 0xFF), mn = (float)((sw[1] >> (8 * q)) & 0xFF);
 #pragma unroll
                 for (int tg = 0; tg < NG; tg++) {
                     v4i D = mfma(bw, 2 * s + pr, tg, st.a[2 * pr], st.a[2 * pr + 1]);
@@ -293,19 +311,20 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                 v4i bw = {(int)(w0 & 0x0F0F0F0Fu), (int)((w0 >> 4) & 0x0F0F0F0Fu), (int)(w1 & 0x0F0F0F0Fu),
                           (int)((w1 >> 4) & 0x0F0F0F0Fu)};
                 const uint32_t b = 4 * s + 2 * g + d_half;
-                const float d = f16_bits_to_f32((uint16_t)(g ? st.dd >> 16 : st.dd & 0xFFFF));
-                const float off = bf16_bits_to_f32((uint16_t)(g ? st.oo >> 16 : st.oo & 0xFFFF));
+                const float d = f16_bits_to_f32((uint16_t)(g ? sw[0] >> 16 : sw[0] & 0xFFFF));
+                const float off = bf16_bits_to_f32((uint16_t)(g ? sw[1] >> 16 : sw[1] & 0xFFFF));
+                const float dz = b < nblk ? d : 0.0f, offz = b < nblk ? off : 0.0f;
 #pragma unroll
                 for (int tg = 0; tg < NG; tg++) {
                     v4i D = mfma(bw, 2 * s + g, tg, st.a[2 * g], st.a[2 * g + 1]);
                     Meta4 m;
                     load_meta<SUMS, DUMP>(lds, as, tg * nm + (min(b, nblk - 1) - B0) * TPAD + d_tok0, m);
                     const int U[4] = {D.x, D.y, D.z, D.w};
-                    if (b < nblk) {  // padding blocks hold zero codes and zero scales, but their staged sums are a real block's
+                    // padding blocks hold zero codes and zero scales, but their staged sums are a real block's: they add
+                    // zeros (as a select, not a branch: a divergent branch here makes every step wait for all requests)
 #pragma unroll
-                        for (int i = 0; i < NI; i++)
-                            acc[tg][i] = fmaf(off, m.fs[i], fmaf(d, fmaf(m.xs[i], (float)U[i], m.c[i]), acc[tg][i]));
-                    }
+                    for (int i = 0; i < NI; i++)
+                        acc[tg][i] = fmaf(offz, m.fs[i], fmaf(dz, fmaf(m.xs[i], (float)U[i], m.c[i]), acc[tg][i]));
                     if (DUMP) {
                         int isum[4] = {U[0] - 8 * m.su[0], U[1] - 8 * m.su[1], U[2] - 8 * m.su[2], U[3] - 8 * m.su[3]};
                         dump_block(b, isum);
@@ -387,10 +406,20 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     }
 #pragma unroll
     for (int j = 0; j < SM; j++) meta_load(min(threadIdx.x + j * nthr, nma - 1), smr[j]);
+    // the ring's requests go out in the order in which the loop below renews them (the barriers keep the compiler from
+    // regrouping them): its waits are counted against that order
+    static_assert(PF % 4 == 0, "a request for scales serves four steps");
     Step<FMT> ring[PF];
-    const uint32_t slast = max(s1, 1u) - 1;
+    uint32_t snext[PF / 4][NM], scur[NM];
 #pragma unroll
-    for (int p = 0; p < PF; p++) load_step(ring[p], min(s0 + p, slast));
+    for (int p = 0; p < PF; p++) {
+        if (p % 4 == 0) {
+            load_scales(snext[p / 4], s0 + p);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        load_step(ring[p], min(s0 + p, slast));
+        __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int j = 0; j < SA / AU; j++) {
         const uint32_t i = threadIdx.x + j * nthr;
@@ -413,12 +442,35 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         meta_store(i, r);
     }
     __syncthreads();
-    // each slot is refilled as soon as its record has been consumed, so PF - 1 records stay on request
-    for (uint32_t sb = s0; sb < s1; sb += PF) {
+    // Each slot is refilled as soon as its record has been consumed, so PF - 1 records stay on request. No request sits
+    // under a condition: the compiler counts the requests in flight to place its waits, and where a path may or may not
+    // have issued one it waits for (nearly) all of them, which empties the ring at every step. So a generation that has
+    // a successor refills every slot (past the wave's last step: with that step again, a hit), and the last one none.
+    uint32_t sb = s0;
+    for (; sb + PF < s1; sb += PF) {
 #pragma unroll
         for (int p = 0; p < PF; p++) {
-            if (sb + p < s1) compute_step(ring[p], sb + p);
-            if (sb + PF + p < s1) load_step(ring[p], sb + PF + p);
+            if (p % 4 == 0) {
+#pragma unroll
+                for (int j = 0; j < NM; j++) scur[j] = snext[p / 4][j];
+                load_scales(snext[p / 4], sb + PF + p);
+            }
+            uint32_t sw[NM];
+            scales_of(scur, p % 4, sw);
+            compute_step(ring[p], sw, sb + p);
+            load_step(ring[p], min(sb + PF + p, slast));
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < PF; p++) {
+        if (p % 4 == 0) {
+#pragma unroll
+            for (int j = 0; j < NM; j++) scur[j] = snext[p / 4][j];
+        }
+        if (sb + p < s1) {
+            uint32_t sw[NM];
+            scales_of(scur, p % 4, sw);
+            compute_step(ring[p], sw, sb + p);
         }
     }
     // the two block parities of a token meet across lane groups kq and kq ^ 2

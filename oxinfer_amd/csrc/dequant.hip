@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(WeightView w, uint32_t 
         case FMT_FP8: {
             uint32_t ncb = (n + w.bc - 1) / w.bc;
             float s = reinterpret_cast<const float*>(w.p1)[(r / w.br) * ncb + c / w.bc];
-            v = e4m3_to_f32(w.p0[r * n + c]) * s;
+            v = e4m3_to_f32(w.p0[fp8_offset(w, r, c)]) * s;
             break;
         }
         case FMT_BF16: v = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(w.p0)[r * n + c]); break;
@@ -194,6 +194,31 @@ hipError_t launch_pack_q4m(const uint8_t* q, const uint16_t* sc, const uint16_t*
                            hipStream_t s) {
     size_t total = (size_t)row_tiles((uint32_t)n_out) * t4m_steps((uint32_t)n_in) * 64;
     pack_q4m_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(q, sc, off, (uint32_t)n_out, (uint32_t)n_in, dst);
+    return hipGetLastError();
+}
+
+// FP8 row-major -> tile-packed records (internal.hpp): one thread per lane slot of a record, 32 bytes.
+__global__ __launch_bounds__(256) void pack_fp8_kernel(const uint8_t* __restrict__ raw, uint32_t n_out, uint32_t n_in, uint8_t* __restrict__ dst) {
+    const uint32_t nsteps = n_in / 128;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x, total = (size_t)row_tiles(n_out) * nsteps * 64;
+    if (idx >= total) return;
+    const uint32_t l = idx & 63, n = l & 15, kq = l >> 4;
+    const size_t rec = idx >> 6, tile = rec / nsteps, st = rec % nsteps, row = tile * 16 + n;
+    uint4 a = make_uint4(0u, 0u, 0u, 0u), b = a;
+    if (row < n_out) {
+        const uint4* src = reinterpret_cast<const uint4*>(raw + row * n_in + 128 * st + 32 * kq);
+        a = src[0];
+        b = src[1];
+    }
+    uint4* out = reinterpret_cast<uint4*>(dst + rec * 2048 + 32 * l);
+    out[0] = a;
+    out[1] = b;
+}
+
+hipError_t launch_pack_fp8(const uint8_t* raw, size_t n_out, size_t n_in, uint8_t* dst, hipStream_t s) {
+    const size_t total = (size_t)row_tiles((uint32_t)n_out) * (n_in / 128) * 64;
+    if (!total) return hipSuccess;
+    pack_fp8_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, dst);
     return hipGetLastError();
 }
 

@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
             wbase[i] = w.p0 + ((size_t)tile * all_steps + step0) * T4M_REC;
         } else {
             const uint32_t row = min(tile * 16 + n, w.n_out - 1);
-            wbase[i] = w.p0 + (size_t)row * w.n_in + 128 * (size_t)step0 + 32 * (lane >> 4);
+            wbase[i] = w.p0 + fp8_offset(w, row, 128 * (size_t)step0 + 32 * (lane >> 4));
             sbase[i] = reinterpret_cast<const float*>(w.p1) + (size_t)(tile * 16 / w.br) * ((w.n_in + w.bc - 1) / w.bc) + step0;
         }
     }
@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
                 r[i].dd = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
                 r[i].oo = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
             } else {
-                const uint8_t* p = wbase[i] + 128 * (size_t)s;
+                const uint8_t* p = wbase[i] + (w.group == 1 ? 2048 : 128) * (size_t)s;
                 r[i].c = *reinterpret_cast<const uint4*>(p);
                 r[i].c2 = *reinterpret_cast<const uint4*>(p + 16);
                 r[i].dd = __float_as_uint(sbase[i][(128 * s) / w.bc]);

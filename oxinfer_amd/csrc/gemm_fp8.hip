@@ -96,7 +96,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
     // the two row tiles whose bytes this wave copies: row pointers of this lane (rows past the end repeat the last)
     const uint8_t* wrow[2];
 #pragma unroll
-    for (int i = 0; i < 2; i++) wrow[i] = w.p0 + (size_t)min((nt0 + 2 * wave + i) * 16 + n, w.n_out - 1) * w.n_in + 32 * kq;
+    for (int i = 0; i < 2; i++) wrow[i] = w.p0 + fp8_offset(w, min((nt0 + 2 * wave + i) * 16 + n, w.n_out - 1), 32 * kq);
+    const uint32_t wstep = w.group == 1 ? 2048 : 128;  // bytes between a lane's chunks of consecutive 128-column steps
     const uint4* abase[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) abase[i] = apk + ((size_t)min(mt0 + i, mtiles - 1) * all_kb * 64 + lane) * 2;
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
         for (int j = 0; j < F8_NT; j++) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
     auto load_w = [&](uint4 (*r)[2], uint32_t kb) {
-        const uint32_t col = 128 * kb;
+        const size_t col = (size_t)wstep * kb;
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             r[i][0] = *reinterpret_cast<const uint4*>(wrow[i] + col);

@@ -22,7 +22,8 @@ namespace oxhip {
 //                                     of a group carries the same scale
 //         p2 off [n_out][n_in/group]  bf16 offsets, optional
 //   Q6_K  p0 ql  [n_out][nb][128], p1 qh [n_out][nb][64], p2 sc [n_out][nb][16] int8, p3 d [n_out][nb] f16
-//   FP8   p0 q   [n_out][n_in]        e4m3 bytes; p1 bs f32 [ceil(n_out/br)][ceil(n_in/bc)]
+//   FP8   p0 q   [n_out][n_in]        e4m3 bytes (row-major, or tile-packed when group == 1: fp8_offset below);
+//         p1 bs f32 [ceil(n_out/br)][ceil(n_in/bc)]
 //   BF16  p0 q   [n_out][n_in]        bf16
 // ------------------------------------------------------------------------------------------------
 enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6 };
@@ -59,6 +60,18 @@ struct GroupView {
 // Launchers (each returns hipSuccess or the launch error).
 hipError_t launch_quantize_act(const float* x, size_t t, size_t n_in, const oxhip_qact& out, hipStream_t s);
 hipError_t launch_dequantize(const WeightView& w, size_t r0, size_t r1, float* out, hipStream_t s);
+// FP8 weights are tile-packed (WeightView::group == 1) when their rows are whole 128-column steps and the scale blocks
+// are multiples of 16 rows x 128 columns: record (tile of 16 rows, step of 128 columns) is 2048 contiguous bytes, lane
+// 16 kq + n of a wave owning the 32 bytes of row n at columns 32 kq .. 32 kq + 31 of the step, so a wave streams whole
+// records instead of 16 separate rows. Otherwise the bytes stay row-major. Byte offset of (row, col) either way:
+__host__ __device__ inline size_t fp8_offset(const WeightView& w, size_t row, size_t col) {
+    if (w.group != 1) return row * w.n_in + col;
+    const size_t nsteps = w.n_in / 128;
+    return ((row / 16) * nsteps + col / 128) * 2048 + 32 * (((col % 128) / 32) * 16 + row % 16) + col % 32;
+}
+inline bool fp8_tileable(size_t n_in, uint32_t br, uint32_t bc) { return n_in % 128 == 0 && bc % 128 == 0 && br % 16 == 0; }
+hipError_t launch_pack_fp8(const uint8_t* raw, size_t n_out, size_t n_in, uint8_t* dst, hipStream_t s);
+
 // Global scratch of the decode kernels that split K across workgroups: `partial` holds slices x 8 token rows of
 // n_out floats, `counters` (zero between launches) one entry per group of row tiles. Launches that share a scratch
 // must be ordered on one stream. Without scratch the kernels keep K inside a workgroup.
@@ -94,6 +107,11 @@ hipError_t launch_q4_scale_groups(const uint16_t* sc32, size_t n_out, size_t n_i
 hipError_t launch_pack_a(const void* x, bool src_bf16, int mode, size_t t, size_t n_in, size_t mtiles, size_t kblocks, void* out,
                          hipStream_t s);
 uint32_t gemm_k_slices(const WeightView& w, size_t mtiles);
+// decode_fp8.hip: FP8 weights at up to 32 tokens on the bf16 matrix cores
+bool skinny_fp8_ok(const WeightView& w, size_t t);
+size_t skinny_fp8_pack_bytes(const WeightView& w, size_t t, int planes);
+hipError_t launch_skinny_fp8(const WeightView& w, const void* x, bool x_bf16, bool exact_f32, size_t t, void* y, bool y_bf16, void* pack,
+                             hipStream_t s);
 hipError_t launch_gemm_reduce(const float* partial, size_t n, uint32_t slices, void* y, bool out_bf16, hipStream_t s);
 void gemm_i8_geometry(const WeightView& w, size_t t, size_t* slots, size_t* ngrp);
 uint32_t gemm_i8_k_slices(const WeightView& w, size_t t);
