@@ -128,14 +128,17 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t n = lane & 15, kq = lane >> 4;  // B / D role: row n of the tile; A role: slot n
     const uint32_t nblk = w.n_in / 32;
-    const uint32_t r = wave / kw, ks = wave % kw;
+    // kw and the number of K slices are powers of two (the launchers see to it): shifts, where a division by a value only
+    // known at run time costs some twenty instructions even when it is the same for the whole wave
+    const uint32_t kwsh = (uint32_t)__builtin_ctz(kw), kssh = (uint32_t)__builtin_ctz(ksplit);
+    const uint32_t r = wave >> kwsh, ks = wave & (kw - 1);
     const uint32_t tile = bx * rt + r;
     const uint32_t ntiles = row_tiles(w.n_out);
     // this workgroup's slice of K: steps [S0, S1), blocks [B0, B0 + nbl) (a multiple of 4 blocks)
     constexpr uint32_t BPS = FMT == FMT_Q8_0 ? 2 : 4;  // blocks of 32 per step
     const uint32_t nsteps = FMT == FMT_Q8_0 ? t8_steps(w.n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in) : t4m_steps(w.n_in));
     const uint32_t slice = GROUPED ? 0 : by;
-    const uint32_t sl = (nsteps + ksplit - 1) / ksplit;
+    const uint32_t sl = (nsteps + ksplit - 1) >> kssh;
     const uint32_t S0 = min(nsteps, slice * sl), S1 = min(nsteps, S0 + sl);
     const uint32_t B0 = BPS * S0, nbl = BPS * sl, M0 = B0 / 2;
     // LDS: [operand-order activations: 512 B per pair of blocks] [scales, sums] [partial sums]; with ALDS the
@@ -162,7 +165,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // D role: this lane's registers are tokens 4 (kq & 1) + i of block parity kq >> 1
     const uint32_t d_half = kq >> 1, d_tok0 = 4 * (kq & 1);
 
-    const uint32_t per = (S1 - S0 + kw - 1) / kw;
+    const uint32_t per = (S1 - S0 + kw - 1) >> kwsh;
     const uint32_t s0 = S0 + ks * per;
     const uint32_t s1 = tile < ntiles ? min(S1, s0 + per) : 0;  // a tile past the matrix streams nothing
     const uint8_t* base = w.p0 + (size_t)min(tile, ntiles - 1) * (FMT == FMT_Q8_0   ? (size_t)nsteps * T8_REC
@@ -339,56 +342,68 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // values go to LDS while the weights are still on their way. Requested after the weights, the activations would
     // only arrive behind them and no step could start before the whole ring had landed.
     constexpr int PF = pf_for<FMT, NT>();
-    constexpr int SA = 8, SM = 4;  // 16-byte activation chunks / scale entries a thread holds in registers; more go later
+    // 16-byte activation chunks / scale entries a thread holds in registers (more go later): every one is a request of
+    // every wave whether or not it has a unit to fetch, so few tokens get few
+    constexpr int SA = NG > 1 ? 8 : NT == 1 ? 2 : NT <= 4 ? 4 : 8, SM = NT <= 4 && NG == 1 ? 2 : 4;
     const uint32_t nb = min(nblk, B0 + nbl) - min(nblk, B0);  // real blocks of the slice
     // slot (m, lane) of the operand array: lane = 16 kq + 8 half + token holds the 8 values of block 2 m + half that
     // the weights' lane group kq pairs with (Q4: positions 4 kq.. and 16 + 4 kq..; else 8 kq..). A thread moves 16
     // (Q4: 32) consecutive bytes of one token's row, so the global reads are whole lines. Absent tokens and a padding
     // block keep whatever LDS holds: those products meet zero weights or are dropped.
     constexpr int AU = FMT == FMT_Q4M ? 2 : 1;  // 16-byte loads per unit of staging work
-    const uint32_t na = ALDS ? t * nb * (FMT == FMT_Q4M ? 1 : 2) : 0;
-    auto act_load = [&](uint32_t i, uint4* v) {
+    // Unit i of the staging work is (token i / adiv, chunk i % adiv); a thread takes units tid, tid + nthr, ...: one
+    // division for its first unit, then carries (a division per unit would be most of the instructions of a wave that
+    // only streams some fifteen records).
+    const uint32_t adiv = max(FMT == FMT_Q4M ? nb : 2 * nb, 1u);
+    auto advance = [](uint32_t& q, uint32_t& r, uint32_t dq, uint32_t dr, uint32_t dv) {
+        r += dr;
+        q += dq;
+        if (r >= dv) {
+            r -= dv;
+            q++;
+        }
+    };
+    const uint32_t a_dq = nthr / adiv, a_dr = nthr - a_dq * adiv;
+    auto act_load = [&](uint32_t tok, uint32_t c, uint4* v) {  // tok < t; c: chunk (Q4M: block) within the slice
         if (FMT == FMT_Q4M) {
-            const uint32_t tok = i / nb, b = i % nb;  // b: block within the slice
-            const uint4* xb = reinterpret_cast<const uint4*>(xa.q + src_row(tok) * w.n_in + (size_t)(B0 + b) * 32);
+            const uint4* xb = reinterpret_cast<const uint4*>(xa.q + src_row(tok) * w.n_in + (size_t)(B0 + c) * 32);
             v[0] = xb[0];
             v[1] = xb[1];
         } else {
-            const uint32_t tok = i / (2 * nb), c = i % (2 * nb);
             v[0] = *reinterpret_cast<const uint4*>(xa.q + src_row(tok) * w.n_in + (size_t)B0 * 32 + (size_t)c * 16);
         }
     };
-    auto act_store = [&](uint32_t i, const uint4* v) {
+    auto act_store = [&](uint32_t tok, uint32_t c, const uint4* v) {
         if (FMT == FMT_Q4M) {
-            const uint32_t tok = i / nb, b = i % nb;
+            const uint32_t b = c;
             uint2* dst = afr + ((size_t)(tok >> 3) * (nbl / 2) + (b >> 1)) * 64 + 8 * (b & 1) + (tok & 7);
             dst[0] = make_uint2(v[0].x, v[1].x);
             dst[16] = make_uint2(v[0].y, v[1].y);
             dst[32] = make_uint2(v[0].z, v[1].z);
             dst[48] = make_uint2(v[0].w, v[1].w);
         } else {
-            const uint32_t tok = i / (2 * nb), c = i % (2 * nb), b = c >> 1;
+            const uint32_t b = c >> 1;
             uint2* dst = afr + ((size_t)(tok >> 3) * (nbl / 2) + (b >> 1)) * 64 + 32 * (c & 1) + 8 * (b & 1) + (tok & 7);
             dst[0] = make_uint2(v[0].x, v[0].y);
             dst[16] = make_uint2(v[0].z, v[0].w);
         }
     };
-    // scales and sums: entry i = (token i / nbl, block i % nbl of the slice), see stage_meta's layout
+    // scales and sums: unit i = (q = i / nbl, block i % nbl of the slice) with q = TPAD group + token of the group
     struct MetaReg {
         float x, f;
         int sq;
     };
-    const uint32_t nma = as;  // entries in all: entry i = (group i / nm, token (i % nm) / nbl of it, block i % nbl)
-    auto meta_load = [&](uint32_t i, MetaReg& r) {
-        const uint32_t tok = 8 * (i / nm) + (i % nm) / nbl, b = i % nbl;  // consecutive threads: consecutive blocks of a token
+    const uint32_t m_dq = nthr / nbl, m_dr = nthr - m_dq * nbl;
+    auto meta_load = [&](uint32_t q, uint32_t b, MetaReg& r) {
+        const uint32_t tok = 8 * (q / TPAD) + q % TPAD;
         const bool live = tok < t && B0 + b < nblk;
         const size_t src = (live ? src_row(tok) : 0) * nblk + B0 + (live ? b : 0);
         r.x = live ? xa.scales[src] : 0.0f;
         r.sq = SUMS && live ? xa.sums[src] : 0;
         r.f = SUMS && live ? xa.fsums[src] : 0.0f;
     };
-    auto meta_store = [&](uint32_t i, const MetaReg& r) {
-        const uint32_t at = (i / nm) * nm + (i % nbl) * TPAD + (i % nm) / nbl;
+    auto meta_store = [&](uint32_t q, uint32_t b, const MetaReg& r) {
+        const uint32_t at = (q / TPAD) * nm + b * TPAD + q % TPAD;
         lds[at] = r.x;
         if (SUMS) {
             lds[(size_t)as + at] = FMT == FMT_Q4_K ? 8.0f * (r.f - r.x * (float)r.sq) : -8.0f * (r.x * (float)r.sq);
@@ -398,14 +413,23 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     };
     uint4 sa[SA];
     MetaReg smr[SM];
-    // (every request below is issued by every lane, with its index clamped into range, so that the waits can be
+    // (every request below is issued by every lane, with its unit clamped into range, so that the waits can be
     // counted exactly; the extra requests hit lines that are being fetched anyway)
+    const uint32_t aq0 = threadIdx.x / adiv, ar0 = threadIdx.x - aq0 * adiv;
+    const uint32_t mq0 = threadIdx.x / nbl, mr0 = threadIdx.x - mq0 * nbl;
+    uint32_t aq = aq0, ar = ar0, mq = mq0, mr = mr0;
     if (ALDS) {
 #pragma unroll
-        for (int j = 0; j < SA / AU; j++) act_load(min(threadIdx.x + j * nthr, na - 1), sa + AU * j);
+        for (int j = 0; j < SA / AU; j++) {
+            act_load(min(aq, t - 1), ar, sa + AU * j);
+            advance(aq, ar, a_dq, a_dr, adiv);
+        }
     }
 #pragma unroll
-    for (int j = 0; j < SM; j++) meta_load(min(threadIdx.x + j * nthr, nma - 1), smr[j]);
+    for (int j = 0; j < SM; j++) {
+        meta_load(mq, mr, smr[j]);
+        advance(mq, mr, m_dq, m_dr, nbl);
+    }
     // the ring's requests go out in the order in which the loop below renews them (the barriers keep the compiler from
     // regrouping them): its waits are counted against that order
     static_assert(PF % 4 == 0, "a request for scales serves four steps");
@@ -420,26 +444,31 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         load_step(ring[p], min(s0 + p, slast));
         __builtin_amdgcn_sched_barrier(0);
     }
+    aq = aq0, ar = ar0, mq = mq0, mr = mr0;
+    if (ALDS) {
 #pragma unroll
-    for (int j = 0; j < SA / AU; j++) {
-        const uint32_t i = threadIdx.x + j * nthr;
-        if (i < na) act_store(i, sa + AU * j);
+        for (int j = 0; j < SA / AU; j++) {
+            if (aq < t) act_store(aq, ar, sa + AU * j);
+            advance(aq, ar, a_dq, a_dr, adiv);
+        }
     }
 #pragma unroll
     for (int j = 0; j < SM; j++) {
-        const uint32_t i = threadIdx.x + j * nthr;
-        if (i < nma) meta_store(i, smr[j]);
+        if (mq < NG * TPAD) meta_store(mq, mr, smr[j]);
+        advance(mq, mr, m_dq, m_dr, nbl);
     }
     // what did not fit the registers (long rows, small workgroups) follows behind the weights
-    for (uint32_t i = threadIdx.x + (SA / AU) * nthr; i < na; i += nthr) {
-        uint4 v[AU];
-        act_load(i, v);
-        act_store(i, v);
+    if (ALDS) {
+        for (; aq < t; advance(aq, ar, a_dq, a_dr, adiv)) {
+            uint4 v[AU];
+            act_load(aq, ar, v);
+            act_store(aq, ar, v);
+        }
     }
-    for (uint32_t i = threadIdx.x + SM * nthr; i < nma; i += nthr) {
+    for (; mq < NG * TPAD; advance(mq, mr, m_dq, m_dr, nbl)) {
         MetaReg r;
-        meta_load(i, r);
-        meta_store(i, r);
+        meta_load(mq, mr, r);
+        meta_store(mq, mr, r);
     }
     __syncthreads();
     // Each slot is refilled as soon as its record has been consumed, so PF - 1 records stay on request. No request sits
@@ -564,7 +593,7 @@ __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid,
     const uint32_t nthr = 64 * jb.rt * jb.kw;
     if (threadIdx.x >= nthr) return;  // whole waves (nthr is a multiple of 64), before any barrier
     const GroupView none{};
-    const uint32_t bx = bid / jb.ks, by = bid % jb.ks;  // the slices of a row group are neighbours in launch order
+    const uint32_t bx = bid >> __builtin_ctz(jb.ks), by = bid & (jb.ks - 1);  // the slices of a row group are neighbours in launch order (ks: a power of two)
     if (jb.t == 1) decode_body<FMT, 1, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
     else if (jb.t == 2) decode_body<FMT, 2, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
     else if (jb.t <= 4) decode_body<FMT, 4, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
@@ -626,7 +655,7 @@ Shape search_shape(uint32_t ntiles, uint32_t nsteps, uint32_t cols_per_step) {
         for (const char* p = e; p && *p;) {
             unsigned nt = 0, ns = 0, a = 0, b = 0, c = 0;
             if (sscanf(p, "%u:%u=%u,%u,%u", &nt, &ns, &a, &b, &c) == 5 && nt == ntiles && ns == nsteps && a >= 1 && b >= 1 && c >= 1 &&
-                a * b <= 16)
+                (b & (b - 1)) == 0 && (c & (c - 1)) == 0 && a * b <= 16)  // kw and ks: powers of two
                 best = Shape{a, b, c};
             p = strchr(p, ';');
             if (p) p++;
@@ -737,7 +766,7 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
     Shape sh{8 / gkw, gkw, 1};
     if (const char* e = getenv("OXHIP_GROUPED_SHAPE")) {  // developer override for tuning runs: "rt,kw"
         unsigned a = 0, b = 0;
-        if (sscanf(e, "%u,%u", &a, &b) == 2 && a >= 1 && b >= 1 && a * b <= 16) sh = Shape{a, b, 1};
+        if (sscanf(e, "%u,%u", &a, &b) == 2 && a >= 1 && b >= 1 && (b & (b - 1)) == 0 && a * b <= 16) sh = Shape{a, b, 1};
     }
     dim3 grid((ntiles + sh.rt - 1) / sh.rt, max_chunks), block(64 * sh.rt * sh.kw);
     const int tpad = max_rows <= 4 ? 4 : 8;
