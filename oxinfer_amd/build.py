@@ -18,6 +18,15 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function",
 ]
 
+# Per-file extras. The prefill GEMMs keep 128 accumulator registers per wave; in the compiler's default form for a
+# kernel with one wave per SIMD the matrix instructions take them from the accumulation registers and are never
+# allocated in place (each accumulator moves to a new register at every instruction and is copied back around the
+# loop: more copies than useful VALU work). With the VGPR form they accumulate in place.
+EXTRA = {
+    "gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "gemm_fp8.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+
 
 def hipcc():
     for p in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
@@ -32,7 +41,7 @@ def build(verbose=False):
 
     def one(src):
         obj = os.path.join(OBJ, src.replace(".hip", ".o"))
-        cmd = [cc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [cc, *FLAGS, *EXTRA.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         # the host pass does not know the device-only target feature; that warning is harmless
         err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)

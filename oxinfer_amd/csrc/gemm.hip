@@ -78,6 +78,7 @@ namespace {
 
 constexpr int WG_MT = 16;  // token tiles per workgroup (256 tokens), 4 per wave
 constexpr int WG_NT = 8;   // row tiles per workgroup (128 rows)
+constexpr int AR = 4;      // blocks of A fragments held ahead (a whole K-step: two starve the FP8 shapes, whose activations do not stay in L2)
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -199,62 +200,52 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
 #pragma unroll
         for (int j = 0; j < WG_NT; j++) dst[j] = bfrag[((buf * 4 + b) * WG_NT + j) * 64 + lane];
     };
-    auto read_a_step = [&](uint4 (*dst)[4], uint32_t st) {  // the A fragments of the 4 blocks of a step
+    auto read_a = [&](uint4* dst, uint32_t blk) {  // the A fragments of block `blk` of this slice
 #pragma unroll
-        for (int b = 0; b < 4; b++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) dst[b][i] = abase[i][(size_t)(4 * st + b) * 64];
+        for (int i = 0; i < 4; i++) dst[i] = abase[i][(size_t)blk * 64];
     };
     // LDS traffic only: outstanding global loads (the prefetches) stay in flight across the barrier
     auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
     // B fragments are read from LDS one block ahead of the MFMAs that consume them; A fragments come from global
-    // memory a whole K-step (four blocks, ~2000 MFMA cycles) ahead, the packed records of the next step two blocks
-    // before they are dequantized into the other LDS buffer.
+    // memory a whole K-step (four blocks, ~2000 MFMA cycles) ahead; the packed records of the next step two blocks
+    // before they are dequantized into the other LDS buffer. Each fragment has one home, refilled in place right after
+    // its last use.
     Raw raw[2];
     load_raw(raw, 0);
-    // Each fragment has one home: a_cur[b] is refilled with block b of the next step as soon as this step's block b has
-    // been issued (a whole K-step ahead of its use), b_cur[j] with the next block's row tile j right after the four
-    // MFMAs that read it.
-    uint4 a_cur[4][4], b_cur[WG_NT];
-    read_a_step(a_cur, 0);
+    uint4 a_cur[AR][4], b_cur[WG_NT];
+    const uint32_t last = nsteps - 1, last_blk = 4 * nsteps - 1;
+#pragma unroll
+    for (int b = 0; b < AR; b++) read_a(a_cur[b], min((uint32_t)b, last_blk));
     dequant_tile(raw[0], 0, 0);
     dequant_tile(raw[1], 1, 0);
-    if (nsteps > 1) load_raw(raw, 1);
+    load_raw(raw, min(1u, last));
     lds_barrier();
     read_b(b_cur, 0, 0);
-    // One K-step. MORE: another step follows (its records are dequantized during blocks 0 and 1, and block 3
-    // refills from the other LDS buffer after the barrier). LOAD2: the records of step s + 2 exist.
-    auto step = [&](uint32_t s, auto more_c, auto load2_c) {
-        constexpr bool MORE = decltype(more_c)::value, LOAD2 = decltype(load2_c)::value;
+    // One K-step; every step does the same work, so that the loop is one body whose accumulators stay in place: the
+    // records of the next step are dequantized into the other LDS buffer during blocks 0 and 1, block 3 refills from
+    // that buffer after the barrier, and the step after next is requested during block 2. Past the end the indices
+    // repeat the last step: a little work that nobody reads, instead of separate loop tails.
+    for (uint32_t s = 0; s < nsteps; s++) {
         const uint32_t buf = s & 1;
 #pragma unroll
         for (int b = 0; b < 4; b++) {
-            if (b == 3 && MORE) lds_barrier();  // the other buffer is complete, and nobody still reads this one
+            if (b == 3) lds_barrier();  // the other buffer is complete, and nobody still reads this one
 #pragma unroll
             for (int j = 0; j < WG_NT; j++) {
                 const bf16x8 bb = __builtin_bit_cast(bf16x8, b_cur[j]);
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_cur[b][i]), bb, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_cur[b % AR][i]), bb, acc[i][j], 0, 0, 0);
                 if (b < 3) b_cur[j] = bfrag[((buf * 4 + b + 1) * WG_NT + j) * 64 + lane];
-                else if (MORE) b_cur[j] = bfrag[(((buf ^ 1) * 4) * WG_NT + j) * 64 + lane];
+                else b_cur[j] = bfrag[(((buf ^ 1) * 4) * WG_NT + j) * 64 + lane];
             }
-            if (MORE) {
-#pragma unroll
-                for (int i = 0; i < 4; i++) a_cur[b][i] = abase[i][(size_t)(4 * (s + 1) + b) * 64];
-            }
-            if (MORE && b == 0) dequant_tile(raw[0], 0, buf ^ 1);
-            if (MORE && b == 1) dequant_tile(raw[1], 1, buf ^ 1);
-            if (LOAD2 && b == 2) load_raw(raw, s + 2);
+            read_a(a_cur[b % AR], min(4 * s + b + AR, last_blk));
+            if (b == 0) dequant_tile(raw[0], 0, buf ^ 1);
+            if (b == 1) dequant_tile(raw[1], 1, buf ^ 1);
+            if (b == 2) load_raw(raw, min(s + 2, last));
         }
-    };
-    using T_ = std::integral_constant<bool, true>;
-    using F_ = std::integral_constant<bool, false>;
-    uint32_t s = 0;
-    for (; s + 2 < nsteps; s++) step(s, T_{}, T_{});
-    if (nsteps >= 2) step(s++, T_{}, F_{});
-    step(s, F_{}, F_{});
+    }
     // D[token 4 kq + r][row n] per tile
     const uint32_t kq = lane >> 4;
     if (gridDim.z > 1) yv = reinterpret_cast<float*>(yv) + (size_t)blockIdx.z * t * w.n_out;
