@@ -74,21 +74,24 @@ __device__ inline uint4 row_take(const uint4& v) {
                       (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v.w, ctrl, 0xf, 0xf, true));
 }
 
-// grid x: groups of RT row tiles; the workgroup's `kw` waves split K and meet in LDS in wave order.
+// grid x: groups of RT row tiles; grid y: K slices; the workgroup's `kw` waves split the slice's steps and meet in LDS in
+// wave order; with more than one slice the sums go out as f32 partial rows [slice][t][n_out] that a second kernel adds.
 // PF: 128-column steps a wave keeps on request. A step's activation fragments (L2 hits) are requested together with its
 // weights: loads complete in issue order, so fragments asked for any later would make the wave wait for every weight
 // request issued before them and cut the depth of the ring.
 template <int RT, int NTT, int NP, int TS, bool OUT_BF16>
 __global__ __launch_bounds__(512) void skinny_fp8_kernel(WeightView w, const uint4* __restrict__ apk, uint32_t t, uint32_t kw,
-                                                         void* __restrict__ yv) {
+                                                         void* __restrict__ yv, float* __restrict__ partial) {
     constexpr int CNT = TS / 4, PER = 16 / TS;  // requests per step and plane; blocks b in a request
     constexpr int PF = 2 * RT + NTT * NP * CNT > 12 ? 2 : 4;
     extern __shared__ __align__(16) float red[];  // [kw][RT][NTT][64][4]
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t n = lane & 15, kq = lane >> 4;
     const uint32_t nsteps = w.n_in / 128, ntiles = (w.n_out + 15) / 16;
-    // wave v takes steps v, v + kw, ...: at any moment the workgroup reads one contiguous window of its rows' records
-    const uint32_t cnt = (nsteps - wave + kw - 1) / kw, ilast = cnt - 1;  // kw <= nsteps
+    // wave v of slice z takes steps z kw + v, + kw slices, ...: at any moment the workgroups of a row group read one
+    // contiguous window of its records
+    const uint32_t gw = blockIdx.y * kw + wave, stride = kw * gridDim.y;  // kw * slices <= nsteps
+    const uint32_t cnt = (nsteps - gw + stride - 1) / stride, ilast = cnt - 1;
     const uint8_t* wp[RT];
     const float* sp[RT];
     const uint32_t scols = (w.n_in + w.bc - 1) / w.bc;
@@ -128,7 +131,7 @@ __global__ __launch_bounds__(512) void skinny_fp8_kernel(WeightView w, const uin
 
     St ring[PF];
 #pragma unroll
-    for (int p = 0; p < PF; p++) load(ring[p], wave + kw * min((uint32_t)p, ilast));
+    for (int p = 0; p < PF; p++) load(ring[p], gw + stride * min((uint32_t)p, ilast));
     auto frag = [&](const St& st, int tt, int pl, int b) -> uint4 {
         const uint4& v = st.a[tt][pl][b / PER];
         switch (TS * (b % PER)) {
@@ -170,7 +173,7 @@ __global__ __launch_bounds__(512) void skinny_fp8_kernel(WeightView w, const uin
 #pragma unroll
         for (int p = 0; p < PF; p++) {
             if (ib + p < cnt) compute(ring[p]);
-            load(ring[p], wave + kw * min(ib + PF + p, ilast));
+            load(ring[p], gw + stride * min(ib + PF + p, ilast));
         }
     }
 #pragma unroll
@@ -194,7 +197,8 @@ __global__ __launch_bounds__(512) void skinny_fp8_kernel(WeightView w, const uin
         for (int i = 0; i < 4; i++) {
             const uint32_t tok = 16 * tt + 4 * (l >> 4) + i;
             if (tok >= t) continue;
-            if (OUT_BF16) reinterpret_cast<uint16_t*>(yv)[(size_t)tok * w.n_out + row] = f32_to_bf16_bits(sum[i]);
+            if (gridDim.y > 1) partial[((size_t)blockIdx.y * t + tok) * w.n_out + row] = sum[i];
+            else if (OUT_BF16) reinterpret_cast<uint16_t*>(yv)[(size_t)tok * w.n_out + row] = f32_to_bf16_bits(sum[i]);
             else reinterpret_cast<float*>(yv)[(size_t)tok * w.n_out + row] = sum[i];
         }
     }
@@ -206,9 +210,16 @@ bool skinny_fp8_ok(const WeightView& w, size_t t) {
     return w.fmt == FMT_FP8 && t >= 1 && t <= 32 && w.n_in % 128 == 0 && w.bc % 128 == 0 && w.br % 16 == 0;
 }
 
-// Bytes of packed activations for t tokens at most (`planes`: 2 for f32 sources kept exact, else 1).
+// More than 16 tokens: four row tiles per wave (a step's 8 fragment requests then serve 4 records, not 2), and K in two
+// slices so that the 112 row groups of a 7168-row matrix still cover the chip.
+constexpr uint32_t WIDE_RT = 4, WIDE_SLICES = 2;
+
+static size_t frag_bytes(const WeightView& w, size_t t, int planes) { return (size_t)((t + 15) / 16) * planes * (w.n_in / 32) * 64 * 16; }
+
+// Scratch for t tokens at most (`planes`: 2 for f32 sources kept exact, else 1): the packed fragments, then the partial
+// rows of the K slices.
 size_t skinny_fp8_pack_bytes(const WeightView& w, size_t t, int planes) {
-    return (size_t)((t + 15) / 16) * planes * (w.n_in / 32) * 64 * 16;
+    return frag_bytes(w, t, planes) + (t > 16 ? (size_t)WIDE_SLICES * t * w.n_out * 4 : 0);
 }
 
 // y [t][n_out] (f32 or bf16) = x W^T; `pack` holds skinny_fp8_pack_bytes(). exact_f32: f32 sources go in as two bf16
@@ -225,31 +236,38 @@ hipError_t launch_skinny_fp8(const WeightView& w, const void* x, bool x_bf16, bo
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const uint32_t ntiles = (w.n_out + 15) / 16;
-    uint32_t kw = 8;
-    while (kw > 1 && nsteps / kw < 4) kw /= 2;
     const uint4* a = static_cast<const uint4*>(pack);
+    float* partial = reinterpret_cast<float*>(static_cast<uint8_t*>(pack) + frag_bytes(w, t, (int)planes));
+    uint32_t slices = 1;
     auto go = [&](auto kern, uint32_t rt, uint32_t ntt) {
+        uint32_t kw = 8;
+        while (kw > 1 && nsteps / (kw * slices) < 4) kw /= 2;
         const size_t lds = (size_t)kw * rt * ntt * 64 * 16;
-        kern<<<(ntiles + rt - 1) / rt, 64 * kw, lds, s>>>(w, a, (uint32_t)t, kw, y);
+        if (lds > 48 * 1024) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return;
+        }
+        kern<<<dim3((ntiles + rt - 1) / rt, slices), 64 * kw, lds, s>>>(w, a, (uint32_t)t, kw, y, partial);
     };
-    auto one_tile = [&](auto np, auto out) {
+    using one = std::integral_constant<int, 1>;
+    using two = std::integral_constant<int, 2>;
+    auto pick = [&](auto np, auto out) {
         constexpr int NP = decltype(np)::value;
         constexpr bool OB = decltype(out)::value;
         if (ts == 4) go(skinny_fp8_kernel<1, 1, NP, 4, OB>, 1, 1);
         else if (ts == 8) go(skinny_fp8_kernel<1, 1, NP, 8, OB>, 1, 1);
-        else go(skinny_fp8_kernel<1, 1, NP, 16, OB>, 1, 1);
+        else if (ttiles == 1) go(skinny_fp8_kernel<2, 1, NP, 16, OB>, 2, 1);
+        else {
+            slices = nsteps >= 8 * WIDE_SLICES ? WIDE_SLICES : 1;
+            go(skinny_fp8_kernel<WIDE_RT, 2, NP, 16, OB>, WIDE_RT, 2);
+        }
     };
-    using one = std::integral_constant<int, 1>;
-    using two = std::integral_constant<int, 2>;
-    if (ttiles == 1) {
-        if (planes == 2) y_bf16 ? one_tile(two{}, std::true_type{}) : one_tile(two{}, std::false_type{});
-        else y_bf16 ? one_tile(one{}, std::true_type{}) : one_tile(one{}, std::false_type{});
-    } else if (planes == 2) {
-        y_bf16 ? go(skinny_fp8_kernel<2, 2, 2, 16, true>, 2, 2) : go(skinny_fp8_kernel<2, 2, 2, 16, false>, 2, 2);
-    } else {
-        y_bf16 ? go(skinny_fp8_kernel<2, 2, 1, 16, true>, 2, 2) : go(skinny_fp8_kernel<2, 2, 1, 16, false>, 2, 2);
-    }
-    return hipGetLastError();
+    if (planes == 2) y_bf16 ? pick(two{}, std::true_type{}) : pick(two{}, std::false_type{});
+    else y_bf16 ? pick(one{}, std::true_type{}) : pick(one{}, std::false_type{});
+    if (e != hipSuccess) return e;
+    e = hipGetLastError();
+    if (e != hipSuccess || slices == 1) return e;
+    return launch_gemm_reduce(partial, t * (size_t)w.n_out, slices, y, y_bf16, s);
 }
 
 }  // namespace oxhip
