@@ -33,7 +33,7 @@ KERNEL_FMT = {Q8_0: 1, Q4_K: 2, Q6_K: 3}  # template argument in the kernel symb
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # benchmark (KiB per dispatch, FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000: what a 256 MiB device copy
 # reads on the same counters); profiles/decode_batch_kernel_gguf_gemv.md holds the summary.
-TRAFFIC_BYTES = {"decode_batch_kernel": 392087422}
+TRAFFIC_BYTES = {"decode_batch_kernel": 391953180}
 
 
 def weight_bytes(kind, n_out, n_in):
@@ -208,10 +208,10 @@ def other_workload(args, be, torch, synth):
     variant = {"bf16": 0, "fp8": 2}.get(args.variant, 0)
     if m <= 16:
         step = lambda i: be.decode(ws[i % len(ws)], x=x32)
-        kern = "decode_dense_kernel<4, *>"
+        kern = "skinny_fp8_kernel<*, 1, 2, *, false> (+ pack_skinny_kernel)"
     else:
         step = lambda i: be.gemm(ws[i % len(ws)], xb, variant=variant, out_bf16=True)
-        kern = "gemm_bf16_kernel<4, true>" if variant == 0 else "gemm_fp8_kernel<true>"
+        kern = ("skinny_fp8_kernel<4, 2, 1, 16, true> (+ pack_skinny_kernel, gemm_reduce_kernel)" if m <= 32 else "gemm_bf16_kernel<4, true>") if variant == 0 else "gemm_fp8_kernel<true>"
     wall, ms = timed_steps(torch, step, args.steps, args.warmup)
     flops, nbytes = 2 * m * n * k, n * k + scales.size * 4 + m * k * 2 + m * n * 2
     hbm = m <= 64
