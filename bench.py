@@ -286,16 +286,16 @@ def main():
         c["pool"] = pools[(c["kind"], c["n_out"], c["n_in"])]
     torch.cuda.synchronize()
 
-    # The dominant kernel. Q8_0 / Q4_K jobs of one call share one launch (decode_batch_kernel): that launch is the
-    # step, and its events bracket it. Q6_K jobs launch one by one: there the largest matmul at the larger batch is
-    # timed (same symbol for both shapes).
-    shared = all(k in (Q8_0, Q4_K) for k in kinds)
+    # The dominant kernel. The jobs of one call share one launch (decode_batch_kernel): that launch is the step, and
+    # its events bracket it. (Formats the shared launch does not take would launch one by one: then the largest
+    # matmul at the larger batch is timed.)
+    shared = all(k in (Q8_0, Q4_K, Q6_K) for k in kinds)
     dom_kind = kinds[0]
     for c in cases:
         c["dom"] = shared or (c["kind"] == dom_kind and c["t"] == 8)
     dom = [c for c in cases if c["dom"]]
     per_step = 1 if shared else len(dom)
-    dom_symbol = "decode_batch_kernel" if shared else f"decode_kernel<{KERNEL_FMT[dom_kind]}, 8, 4>"
+    dom_symbol = "decode_batch_kernel"
 
     # One call per step: the job arrays (one per rotation phase) are built once; the dominant launches carry
     # HIP events recorded by the library on the launch stream.
@@ -358,7 +358,7 @@ def main():
                    "matmuls_per_step": len(cases), "launches_per_step": 1 if shared else len(cases), "bytes_per_step": step_bytes,
                    "weight_pool_GB_per_shape": args.pool_gb, "activations": "int8 per 32 (quantize_act), resident in HBM"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES.get(dom_symbol), "kernel": dom_symbol,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES.get(dom_symbol) if all(k in (Q8_0, Q4_K) for k in kinds) else None, "kernel": dom_symbol,
                      "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_avg_s * 1e6, 2)},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "detail": detail,

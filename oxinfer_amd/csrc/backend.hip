@@ -285,13 +285,9 @@ oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) {
             } else if (d->ggml_type == OXHIP_GGML_Q6_K) {
                 if (n_in % 256) return fail("Q6_K rows must be whole blocks of 256");
                 w->v.fmt = FMT_Q6_K;
-                size_t nb = n_out * (n_in / 256);
-                pl.add(0, nb * 128);
-                pl.add(1, nb * 64);
-                pl.add(2, nb * 16);
-                pl.add(3, nb * 2);
-                raw_bytes = nb * 210;
-                np = 4;
+                pl.add(0, t6k_bytes((uint32_t)n_out, (uint32_t)n_in));
+                raw_bytes = n_out * (n_in / 256) * 210;
+                np = 1;
             } else {
                 return fail("GGUF type " + std::to_string(d->ggml_type) + " has no device kernels");
             }

@@ -1,11 +1,11 @@
-// Decode kernels on the vector ALUs (v_dot4_i32_i8) for the formats stored in planes (Q6_K, Q4
-// with per-32 scales) and for float-stored weights: dequant-fused GEMV / skinny GEMM, one wavefront
-// per group of R weight rows. Q8_0, Q4_K and MLX Q4 run on the matrix cores (decode_mfma.hip).
+// Decode kernels on the vector ALUs (v_dot4_i32_i8) for the planar Q4 format (per-32 scales, any offset
+// group) and for float-stored weights: dequant-fused GEMV / skinny GEMM, one wavefront per group of R
+// weight rows. Q8_0, Q4_K, Q6_K and MLX Q4 run on the matrix cores (decode_mfma.hip).
 //
 // What they compute is what the reference's CPU decode kernels compute (QMat::rows_t1 / rows_tc,
 // src/kernels.rs:1339-1369; dot_row_generic, src/ggml.rs:1288-1315; q4_dot_rows_tc_scalar,
 // src/kernels_x86.rs:447-474): exact int32 dot products of the unpacked int8 weights with the int8
-// activations per 16 (GGUF) or 32 (Q4) elements, scaled in f32 by weight scale x activation scale,
+// activations per 32 elements, scaled in f32 by weight scale x activation scale,
 // plus offset terms over the exact f32 activation sums. Only the order of the f32 additions
 // differs (lanes, then a DPP tree).
 //
@@ -13,7 +13,7 @@
 // takes units l, l+64, ... of a row, so a wave-wide load reads 1 KiB of consecutive bytes. The
 // activations of a unit are loaded once per token and reused for the R rows of the wave; packed
 // nibbles are split in registers and multiplied with v_dot4_i32_i8; the bias of the unsigned
-// nibble / 6-bit codes is folded through the per-16 integer sums of the activations, so no
+// nibble codes is folded through the per-16 integer sums of the activations, so no
 // per-element subtraction is needed.
 #include "internal.hpp"
 
@@ -77,47 +77,6 @@ struct F<FMT_Q4> {
         int i;
         isums(w, a, &i);
         return ((float)i * w.d) * a[0].xs;
-    }
-};
-
-// ---- Q6_K: unit = 16 bytes of ql with the matching 16 bytes of qh ---------------------------------
-template <>
-struct F<FMT_Q6_K> {
-    static constexpr int NG = 2;
-    static constexpr bool MIN = false, S16 = true;
-    static constexpr int ISUMS_PER_UNIT = 2;
-    struct W {
-        uint4 lo, hi;
-        float s_lo, s_hi;
-    };
-    __device__ static uint32_t units(const WeightView& w) { return w.n_in / 32; }
-    // unit u = 8 sb + 4 n + c: low nibbles are group 16 sb + 8 n + c, high nibbles that + 4
-    __device__ static uint32_t group(uint32_t u, int g) { return 16 * (u >> 3) + 8 * ((u >> 2) & 1) + (u & 3) + 4 * g; }
-    __device__ static void load(const WeightView& w, uint32_t r, uint32_t u, W& o) {
-        size_t nb = w.n_in / 256;
-        uint32_t sb = u >> 3, n = (u >> 2) & 1, c = u & 3;
-        uint4 ql = *reinterpret_cast<const uint4*>(w.p0 + ((size_t)r * nb * 8 + u) * 16);
-        uint4 qh = *reinterpret_cast<const uint4*>(w.p1 + ((size_t)r * nb + sb) * 64 + 32 * n + 16 * (c & 1));
-        uint32_t sl = c >= 2 ? 2 : 0, sh = sl + 4;
-        auto mix = [](uint32_t nib, uint32_t h, uint32_t s) { return nib | (((h >> s) & 0x03030303u) << 4); };
-        uint4 l = lo_nibbles(ql), h = hi_nibbles(ql);
-        o.lo = make_uint4(mix(l.x, qh.x, sl), mix(l.y, qh.y, sl), mix(l.z, qh.z, sl), mix(l.w, qh.w, sl));
-        o.hi = make_uint4(mix(h.x, qh.x, sh), mix(h.y, qh.y, sh), mix(h.z, qh.z, sh), mix(h.w, qh.w, sh));
-        const int8_t* sc = reinterpret_cast<const int8_t*>(w.p2) + ((size_t)r * nb + sb) * 16 + 8 * n + c;
-        float d = f16_bits_to_f32(reinterpret_cast<const uint16_t*>(w.p3)[(size_t)r * nb + sb]);
-        o.s_lo = d * (float)sc[0];
-        o.s_hi = d * (float)sc[4];
-    }
-    __device__ static void isums(const W& w, const ActG* a, int* out) {
-        out[0] = dot16(w.lo, a[0].xq) - 32 * a[0].s16;
-        out[1] = dot16(w.hi, a[1].xq) - 32 * a[1].s16;
-    }
-    __device__ static float dot(const W& w, const ActG* a) {
-        int i[2];
-        isums(w, a, i);
-        float sum = (w.s_lo * a[0].xs) * (float)i[0];
-        sum += (w.s_hi * a[1].xs) * (float)i[1];
-        return sum;
     }
 };
 
@@ -337,9 +296,9 @@ hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x
     switch (w.fmt) {
         case FMT_Q8_0:
         case FMT_Q4_K:
+        case FMT_Q6_K:
         case FMT_Q4M: return launch_decode_mfma(w, xa, t, y, sc, s);
         case FMT_Q4: return decode_t<FMT_Q4, 4>(w, xa, t, y, s);
-        case FMT_Q6_K: return decode_t<FMT_Q6_K, 4>(w, xa, t, y, s);
         case FMT_FP8:
             // the matrix-core kernel when the block scales allow it and the caller's scratch holds the packed activations
             if (skinny_fp8_ok(w, t) && sc.partial && skinny_fp8_pack_bytes(w, t, 2) <= sc.partial_floats * 4)
@@ -351,13 +310,12 @@ hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x
 }
 
 hipError_t launch_isums(const WeightView& w, const QActView& xa, size_t t, int32_t* out, hipStream_t s) {
-    if (w.fmt == FMT_Q8_0 || w.fmt == FMT_Q4_K || w.fmt == FMT_Q4M) return launch_isums_mfma(w, xa, t, nullptr, out, s);
+    if (w.fmt == FMT_Q8_0 || w.fmt == FMT_Q4_K || w.fmt == FMT_Q6_K || w.fmt == FMT_Q4M) return launch_isums_mfma(w, xa, t, nullptr, out, s);
     size_t units = w.n_in / 32;
     size_t total = t * w.n_out * units;
     unsigned grid = (unsigned)((total + 255) / 256);
     switch (w.fmt) {
         case FMT_Q4: isums_kernel<FMT_Q4><<<grid, 256, 0, s>>>(w, xa, (uint32_t)t, out); break;
-        case FMT_Q6_K: isums_kernel<FMT_Q6_K><<<grid, 256, 0, s>>>(w, xa, (uint32_t)t, out); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -47,7 +47,7 @@ namespace {
 // Records a wave keeps in flight. HBM delivers about 8 TB/s at about 2 us of loaded latency, so some 16 MB must be
 // on request across the chip at any moment: about 4000 resident waves x PF KiB.
 template <int FMT, int NT>
-constexpr int pf_for() { return 8; }
+constexpr int pf_for() { return FMT == FMT_Q6_K ? 4 : 8; }  // Q6_K records are 1.7 KiB and its step needs the registers
 
 struct Meta4 {
     float xs[4];
@@ -103,6 +103,12 @@ struct Step<FMT_Q4M> {
     uint4 w;
     uint32_t a[4];
 };
+template <>
+struct Step<FMT_Q6_K> {
+    uint4 w;   // low nibbles
+    uint2 h;   // high bit pairs
+    uint32_t a[1];
+};
 
 // FMT: FMT_Q8_0 / FMT_Q4_K / FMT_Q4M. NT: tokens handled (1, 2, 4 or 8). DUMP: also write the exact
 // integer block sums to `dump` ([t][n_out][n_in/32]) for parity checks.
@@ -136,7 +142,10 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     const uint32_t ntiles = row_tiles(w.n_out);
     // this workgroup's slice of K: steps [S0, S1), blocks [B0, B0 + nbl) (a multiple of 4 blocks)
     constexpr uint32_t BPS = FMT == FMT_Q8_0 ? 2 : 4;  // blocks of 32 per step
-    const uint32_t nsteps = FMT == FMT_Q8_0 ? t8_steps(w.n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in) : t4m_steps(w.n_in));
+    const uint32_t nsteps = FMT == FMT_Q8_0   ? t8_steps(w.n_in)
+                            : FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in)
+                            : FMT == FMT_Q6_K ? t6k_steps(w.n_in)
+                                              : t4m_steps(w.n_in);
     const uint32_t slice = GROUPED ? 0 : by;
     const uint32_t sl = (nsteps + ksplit - 1) >> kssh;
     const uint32_t S0 = min(nsteps, slice * sl), S1 = min(nsteps, S0 + sl);
@@ -170,6 +179,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     const uint32_t s1 = tile < ntiles ? min(S1, s0 + per) : 0;  // a tile past the matrix streams nothing
     const uint8_t* base = w.p0 + (size_t)min(tile, ntiles - 1) * (FMT == FMT_Q8_0   ? (size_t)nsteps * T8_REC
                                                                   : FMT == FMT_Q4_K ? (size_t)(nsteps / 2) * TK4_REC
+                                                                  : FMT == FMT_Q6_K ? (size_t)nsteps * T6K_REC
                                                                                     : (size_t)nsteps * T4M_REC);
 
     auto act2 = [&](uint32_t b, uint32_t pos, uint32_t* out) {  // 8 consecutive activations of block b
@@ -189,6 +199,11 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                 act2(4 * s + a_half, 8 * kq, st.a);
                 act2(4 * s + 2 + a_half, 8 * kq, st.a + 2);
             }
+        } else if constexpr (FMT == FMT_Q6_K) {
+            static_assert(FMT != FMT_Q6_K || ALDS, "Q6_K takes its activations from LDS");
+            const uint8_t* rec = base + (size_t)s * T6K_REC;
+            st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+            st.h = *reinterpret_cast<const uint2*>(rec + 1024 + 8 * lane);
         } else {
             const uint8_t* rec = base + (size_t)s * T4M_REC;
             st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
@@ -208,7 +223,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // kq asks for the words of step `first + kq` (row n of it), and at step first + q every lane takes them from lane
     // 16 q + n. Q8_0: {d of the two blocks}; Q4_K: {four sub-block scales, four mins, (d, dmin)}: this step's four
     // sub-blocks are 4 (s & 1) .. + 3 of the super-block; MLX: {d of the two groups, offsets of the two groups}.
-    constexpr int NM = FMT == FMT_Q8_0 ? 1 : FMT == FMT_Q4_K ? 3 : 2;
+    constexpr int NM = FMT == FMT_Q8_0 ? 1 : (FMT == FMT_Q4_K || FMT == FMT_Q6_K) ? 3 : 2;
     const uint32_t slast = max(s1, 1u) - 1;
     auto load_scales = [&](uint32_t* m, uint32_t first) {
         const uint32_t s = min(first + kq, slast);
@@ -219,6 +234,11 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             m[0] = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 4 * (s & 1));
             m[1] = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
             m[2] = *reinterpret_cast<const uint32_t*>(rec + 2304 + 4 * n);
+        } else if constexpr (FMT == FMT_Q6_K) {  // {scales of sub-blocks 0..3, of 4..7, d}
+            const uint8_t* rec = base + (size_t)s * T6K_REC;
+            m[0] = *reinterpret_cast<const uint32_t*>(rec + 1536 + 8 * n);
+            m[1] = *reinterpret_cast<const uint32_t*>(rec + 1540 + 8 * n);
+            m[2] = *reinterpret_cast<const uint16_t*>(rec + 1664 + 2 * n);
         } else {
             const uint8_t* rec = base + (size_t)s * T4M_REC;
             m[0] = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
@@ -236,6 +256,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     for (int g = 0; g < NG; g++)
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[g][i] = 0.0f;
+    // Q6_K: every lane group sums its own 16-column sub-block for tokens 4 tg + i
+    float acc6a[4] = {0.0f, 0.0f, 0.0f, 0.0f}, acc6b[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // tg = 0, 1
     // `m`: index of the instruction along K (pair of blocks 2 m, 2 m + 1); with ALDS its operand comes from LDS
     auto mfma = [&](v4i bw, uint32_t m, int tg, uint32_t d0, uint32_t d1) -> v4i {
         if (ALDS) {
@@ -307,6 +329,51 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             for (int tg = 0; tg < NG; tg++)
 #pragma unroll
                 for (int i = 0; i < NI; i++) acc[tg][i] = fmaf(ndmin, Q[tg][i], fmaf(d, P[tg][i], acc[tg][i]));
+        } else if constexpr (FMT == FMT_Q6_K) {
+            // Scales go per 16 columns, so an instruction's 16 operand slots are (sub-block sb, token t4): lane group kq
+            // supplies sub-block kq's 16 activations of token t4 in the slots with sb = kq and zeros elsewhere, and lane
+            // (kq, n) receives sub-block kq's exact sums for tokens 4 tg + i of row n. Eight tokens take two instructions.
+            const float d = f16_bits_to_f32((uint16_t)(sw[2] & 0xFFFF));
+            const uint32_t hq[2] = {st.h.x, st.h.y};
+            const bool on = (n >> 2) == kq;
+            const uint4* afr6 = reinterpret_cast<const uint4*>(afr);  // [64-column group][8 tokens][kq]
+#pragma unroll
+            for (int h = 0; h < 2; h++) {  // the step's two groups of 64 columns
+                const uint32_t lo = h ? c.z : c.x, hi = h ? c.w : c.y, hh = hq[h];
+                const v4i bw = {(int)((lo & 0x0F0F0F0Fu) | ((hh & 0x03030303u) << 4)), (int)(((lo >> 4) & 0x0F0F0F0Fu) | (((hh >> 2) & 0x03030303u) << 4)),
+                                (int)((hi & 0x0F0F0F0Fu) | (((hh >> 4) & 0x03030303u) << 4)), (int)(((hi >> 4) & 0x0F0F0F0Fu) | (((hh >> 6) & 0x03030303u) << 4))};
+                const float dsc = d * (float)(int)(int8_t)((sw[h] >> (8 * kq)) & 0xFF);
+                const uint32_t m64 = 2 * s + h, b = 2 * m64 + (kq >> 1);  // the lane's 32-block (its scale's) and its half
+                const uint32_t at = (min(b, nblk - 1) - B0) * TPAD;
+#pragma unroll
+                for (int tg = 0; tg < (NT > 4 ? 2 : 1); tg++) {
+                    const uint4 av = afr6[((size_t)(m64 - M0) * 8 + 4 * tg + (n & 3)) * 4 + kq];
+                    const v4i a = {on ? (int)av.x : 0, on ? (int)av.y : 0, on ? (int)av.z : 0, on ? (int)av.w : 0};
+                    const v4i z = {0, 0, 0, 0};
+                    const v4i D = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bw, z, 0, 0, 0);
+                    const float4 xs = *reinterpret_cast<const float4*>(lds + at + 4 * tg);
+                    const float4 cc = *reinterpret_cast<const float4*>(lds + (size_t)(1 + (kq & 1)) * as + at + 4 * tg);
+                    const float xv[4] = {xs.x, xs.y, xs.z, xs.w}, cv[4] = {cc.x, cc.y, cc.z, cc.w};
+                    const int U[4] = {D.x, D.y, D.z, D.w};
+#pragma unroll
+                    for (int i = 0; i < NI; i++) {
+                        const float v = fmaf(xv[i], (float)U[i], cv[i]);
+                        if (tg == 0) acc6a[i] = fmaf(dsc, v, acc6a[i]);
+                        else acc6b[i] = fmaf(dsc, v, acc6b[i]);
+                    }
+                    if (DUMP) {
+                        const int4 sp = *reinterpret_cast<const int4*>(lds + (size_t)3 * as + at + 4 * tg);
+                        const int su[4] = {sp.x, sp.y, sp.z, sp.w};
+                        const uint32_t row = tile * 16 + n;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const int s16 = (kq & 1) ? (su[i] >> 16) : (int)(int16_t)(su[i] & 0xFFFF);
+                            if (4 * tg + i < (int)t && row < w.n_out && b < nblk)
+                                dump[((size_t)(4 * tg + i) * w.n_out + row) * (w.n_in / 16) + 4 * m64 + kq] = U[i] - 32 * s16;
+                        }
+                    }
+                }
+            }
         } else {
 #pragma unroll
             for (int g = 0; g < 2; g++) {  // the two groups of 64 of the step
@@ -381,6 +448,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             dst[16] = make_uint2(v[0].y, v[1].y);
             dst[32] = make_uint2(v[0].z, v[1].z);
             dst[48] = make_uint2(v[0].w, v[1].w);
+        } else if (FMT == FMT_Q6_K) {  // chunk c = columns 16 c ..: sub-block c % 4 of 64-column group c / 4
+            reinterpret_cast<uint4*>(afr)[((size_t)(c >> 2) * 8 + (tok & 7)) * 4 + (c & 3)] = make_uint4(v[0].x, v[0].y, v[0].z, v[0].w);
         } else {
             const uint32_t b = c >> 1;
             uint2* dst = afr + ((size_t)(tok >> 3) * (nbl / 2) + (b >> 1)) * 64 + 32 * (c & 1) + 8 * (b & 1) + (tok & 7);
@@ -391,7 +460,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // scales and sums: unit i = (q = i / nbl, block i % nbl of the slice) with q = TPAD group + token of the group
     struct MetaReg {
         float x, f;
-        int sq;
+        int sq, sq2;  // Q6_K: the sums of the block's two halves
     };
     const uint32_t m_dq = nthr / nbl, m_dr = nthr - m_dq * nbl;
     auto meta_load = [&](uint32_t q, uint32_t b, MetaReg& r) {
@@ -399,13 +468,24 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         const bool live = tok < t && B0 + b < nblk;
         const size_t src = (live ? src_row(tok) : 0) * nblk + B0 + (live ? b : 0);
         r.x = live ? xa.scales[src] : 0.0f;
-        r.sq = SUMS && live ? xa.sums[src] : 0;
-        r.f = SUMS && live ? xa.fsums[src] : 0.0f;
+        if (FMT == FMT_Q6_K) {
+            r.sq = live ? xa.sums16[2 * src] : 0;
+            r.sq2 = live ? xa.sums16[2 * src + 1] : 0;
+            r.f = 0.0f;
+        } else {
+            r.sq = SUMS && live ? xa.sums[src] : 0;
+            r.sq2 = 0;
+            r.f = SUMS && live ? xa.fsums[src] : 0.0f;
+        }
     };
     auto meta_store = [&](uint32_t q, uint32_t b, const MetaReg& r) {
         const uint32_t at = (q / TPAD) * nm + b * TPAD + q % TPAD;
         lds[at] = r.x;
-        if (SUMS) {
+        if (FMT == FMT_Q6_K) {  // the codes are unsigned (0..63): -32 x the half's activation sum, scaled like the dot
+            lds[(size_t)as + at] = -32.0f * (r.x * (float)r.sq);
+            lds[(size_t)2 * as + at] = -32.0f * (r.x * (float)r.sq2);
+            if (DUMP) reinterpret_cast<int*>(lds)[(size_t)3 * as + at] = (r.sq & 0xFFFF) | (r.sq2 << 16);
+        } else if (SUMS) {
             lds[(size_t)as + at] = FMT == FMT_Q4_K ? 8.0f * (r.f - r.x * (float)r.sq) : -8.0f * (r.x * (float)r.sq);
             lds[(size_t)2 * as + at] = r.f;
             if (DUMP) reinterpret_cast<int*>(lds)[(size_t)3 * as + at] = r.sq;
@@ -502,11 +582,24 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             compute_step(ring[p], sw, sb + p);
         }
     }
-    // the two block parities of a token meet across lane groups kq and kq ^ 2
+    if constexpr (FMT == FMT_Q6_K) {
+        // the four sub-blocks of a token meet across the lane groups; group 0 then holds tokens 0..3, group 1 tokens 4..7
 #pragma unroll
-    for (int g = 0; g < NG; g++)
+        for (int i = 0; i < 4; i++) {
+            float a = acc6a[i], b = acc6b[i];
+            a += __shfl_xor(a, 16);
+            a += __shfl_xor(a, 32);
+            b += __shfl_xor(b, 16);
+            b += __shfl_xor(b, 32);
+            acc[0][i] = (kq & 1) ? b : a;
+        }
+    } else {
+        // the two block parities of a token meet across lane groups kq and kq ^ 2
 #pragma unroll
-        for (int i = 0; i < 4; i++) acc[g][i] += __shfl_xor(acc[g][i], 32);
+        for (int g = 0; g < NG; g++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[g][i] += __shfl_xor(acc[g][i], 32);
+    }
     if (ALDS) __syncthreads();  // the partial sums overwrite the staged activations
     if (kq < 2) {
 #pragma unroll
@@ -595,7 +688,8 @@ __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid,
     const GroupView none{};
     const uint32_t bx = bid >> __builtin_ctz(jb.ks), by = bid & (jb.ks - 1);  // the slices of a row group are neighbours in launch order (ks: a power of two)
     if (jb.t == 1) decode_body<FMT, 1, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
-    else if (jb.t == 2) decode_body<FMT, 2, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
+    else if (jb.t == 2 && FMT != FMT_Q4M) decode_body<FMT, 2, false, false, true>(  // (MLX at 2 tokens: the 4-token body, which fits the registers)
+        jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
     else if (jb.t <= 4) decode_body<FMT, 4, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
     else decode_body<FMT, 8, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
 }
@@ -609,6 +703,7 @@ __global__ __launch_bounds__(1024) void decode_batch_kernel(BatchArgs a) {
     switch (jb.w.fmt) {
         case FMT_Q8_0: batch_dispatch<FMT_Q8_0>(jb, bx, lds_dyn); break;
         case FMT_Q4_K: batch_dispatch<FMT_Q4_K>(jb, bx, lds_dyn); break;
+        case FMT_Q6_K: batch_dispatch<FMT_Q6_K>(jb, bx, lds_dyn); break;
         case FMT_Q4M: batch_dispatch<FMT_Q4M>(jb, bx, lds_dyn); break;
         default: break;
     }
@@ -708,14 +803,14 @@ hipError_t launch_one(bool alds, dim3 grid, dim3 block, size_t lds, hipStream_t 
         if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, v, t, sh.rt, sh.kw, y, dump, g, sh.ks, sc.partial, sc.counters);
     };
     if (alds) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, true, NG>);
-    else if constexpr (NG == 1) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, false, 1>);
-    else e = hipErrorInvalidValue;  // token groups need the staged activations
+    else if constexpr (NG == 1 && FMT != FMT_Q6_K) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, false, 1>);
+    else e = hipErrorInvalidValue;  // token groups and Q6_K need the staged activations
     return e != hipSuccess ? e : hipGetLastError();
 }
 
 template <int FMT>
 constexpr uint32_t steps_of(uint32_t n_in) {
-    return FMT == FMT_Q8_0 ? t8_steps(n_in) : (FMT == FMT_Q4_K ? 2 * tk4_sbs(n_in) : t4m_steps(n_in));
+    return FMT == FMT_Q8_0 ? t8_steps(n_in) : FMT == FMT_Q4_K ? 2 * tk4_sbs(n_in) : FMT == FMT_Q6_K ? t6k_steps(n_in) : t4m_steps(n_in);
 }
 
 template <int FMT, bool DUMP>
@@ -736,8 +831,10 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
         v.scales += c0 * nblk;
         v.sums += c0 * nblk;
         v.fsums += c0 * nblk;
+        if (v.hsums) v.hsums += c0 * 2 * nblk;
+        if (v.sums16) v.sums16 += c0 * 2 * nblk;
         float* yo = y ? y + c0 * w.n_out : nullptr;  // no output rows when only the block sums are wanted
-        int32_t* du = dump ? dump + c0 * (size_t)w.n_out * nblk : nullptr;
+        int32_t* du = dump ? dump + c0 * (size_t)w.n_out * nblk * (FMT == FMT_Q6_K ? 2 : 1) : nullptr;
         const int tpad = tc <= 4 ? 4 : 8;
         bool alds;
         const size_t lds = lds_bytes(FMT != FMT_Q8_0, DUMP, FMT == FMT_Q8_0 ? 2 : 4, nsteps, tpad, sh, &alds);
@@ -745,7 +842,7 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
         const uint32_t tt = (uint32_t)tc;
         hipError_t e;
         if (tc == 1) e = launch_one<FMT, 1, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
-        else if (tc == 2) e = launch_one<FMT, 2, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
+        else if (tc == 2 && FMT != FMT_Q4M) e = launch_one<FMT, 2, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
         else if (tc <= 4) e = launch_one<FMT, 4, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
         else e = launch_one<FMT, 8, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
         if (e != hipSuccess) return e;
@@ -787,12 +884,15 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
 
 namespace {
 uint32_t steps_rt(const WeightView& w) {
-    return w.fmt == FMT_Q8_0 ? steps_of<FMT_Q8_0>(w.n_in) : (w.fmt == FMT_Q4_K ? steps_of<FMT_Q4_K>(w.n_in) : steps_of<FMT_Q4M>(w.n_in));
+    return w.fmt == FMT_Q8_0   ? steps_of<FMT_Q8_0>(w.n_in)
+           : w.fmt == FMT_Q4_K ? steps_of<FMT_Q4_K>(w.n_in)
+           : w.fmt == FMT_Q6_K ? steps_of<FMT_Q6_K>(w.n_in)
+                               : steps_of<FMT_Q4M>(w.n_in);
 }
 }  // namespace
 
 bool decode_batchable(const WeightView& w, size_t t) {
-    if (w.fmt != FMT_Q8_0 && w.fmt != FMT_Q4_K && w.fmt != FMT_Q4M) return false;
+    if (w.fmt != FMT_Q8_0 && w.fmt != FMT_Q4_K && w.fmt != FMT_Q6_K && w.fmt != FMT_Q4M) return false;
     if (t < 1 || t > 8) return false;
     const Shape sh = shape_for(row_tiles(w.n_out), steps_rt(w), true, w.fmt == FMT_Q8_0 ? 64 : 128);  // as a launch of its own: same bits
     bool alds;
@@ -874,16 +974,18 @@ hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t,
     switch (w.fmt) {
         case FMT_Q8_0: return run<FMT_Q8_0, false>(w, xa, t, y, nullptr, sc, s);
         case FMT_Q4_K: return run<FMT_Q4_K, false>(w, xa, t, y, nullptr, sc, s);
+        case FMT_Q6_K: return run<FMT_Q6_K, false>(w, xa, t, y, nullptr, sc, s);
         case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, sc, s);
         default: return hipErrorInvalidValue;
     }
 }
 
-// The integer block sums the kernel forms ([t][n_out][n_in/32]); y is scratch of [t][n_out].
+// The integer block sums the kernel forms ([t][n_out][n_in/32]; Q6_K: per 16, [t][n_out][n_in/16]); y is scratch of [t][n_out].
 hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* out, hipStream_t s) {
     switch (w.fmt) {
         case FMT_Q8_0: return run<FMT_Q8_0, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q4_K: return run<FMT_Q4_K, true>(w, xa, t, y, out, DecodeScratch{}, s);
+        case FMT_Q6_K: return run<FMT_Q6_K, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q4M: return run<FMT_Q4M, true>(w, xa, t, y, out, DecodeScratch{}, s);
         default: return hipErrorInvalidValue;
     }

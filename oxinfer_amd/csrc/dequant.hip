@@ -62,14 +62,15 @@ __global__ __launch_bounds__(256) void dequantize_kernel(WeightView w, uint32_t 
             break;
         }
         case FMT_Q6_K: {
-            size_t nb = n / 256;
-            uint32_t sb = c / 256, e = c % 256, nn = e / 128, k = (e % 128) / 32, l = e % 32, is = l / 16;
-            const uint8_t* ql = w.p0 + (r * nb + sb) * 128 + 64 * nn;
-            uint8_t qh = w.p1[(r * nb + sb) * 64 + 32 * nn + l];
-            uint8_t lo = ql[l + 32 * (k & 1)];
-            int q = (int)((k < 2 ? (lo & 0xF) : (lo >> 4)) | (((qh >> (2 * k)) & 3) << 4)) - 32;
-            float sc = (float)reinterpret_cast<const int8_t*>(w.p2)[(r * nb + sb) * 16 + 8 * nn + is + 2 * k];
-            float d = f16_bits_to_f32(reinterpret_cast<const uint16_t*>(w.p3)[r * nb + sb]);
+            const uint32_t tile = r >> 4, nn = r & 15, st = c >> 7, wi = c & 127, h = wi >> 6, kq = (wi & 63) >> 4, j = wi & 15;
+            const uint8_t* rec = w.p0 + ((size_t)tile * t6k_steps(n) + st) * T6K_REC;
+            const uint32_t ln = 16 * kq + nn, bb = j & 3;
+            const uint32_t dw = *reinterpret_cast<const uint32_t*>(rec + 16 * ln + 4 * (2 * h + (j >> 3)));
+            const uint32_t hh = *reinterpret_cast<const uint32_t*>(rec + 1024 + 8 * ln + 4 * h);
+            const uint32_t lo4 = (dw >> (8 * bb + 4 * ((j & 7) >> 2))) & 0xF, hi2 = (hh >> (8 * bb + 2 * (j >> 2))) & 3;
+            int q = (int)(lo4 | (hi2 << 4)) - 32;
+            float sc = (float)reinterpret_cast<const int8_t*>(rec + 1536 + 8 * nn)[4 * h + kq];
+            float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(rec + 1664 + 2 * nn));
             v = d * sc * (float)q;
             break;
         }
@@ -222,17 +223,47 @@ hipError_t launch_pack_fp8(const uint8_t* raw, size_t n_out, size_t n_in, uint8_
     return hipGetLastError();
 }
 
-// Q6_K: planes, one thread per source block.
-__global__ __launch_bounds__(256) void repack_q6k_kernel(const uint8_t* __restrict__ raw, size_t nblocks, uint8_t* p0, uint8_t* p1,
-                                                         uint8_t* p2, uint8_t* p3) {
-    size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (b >= nblocks) return;
-    const uint8_t* s = raw + b * 210;
-    for (int i = 0; i < 128; i++) p0[b * 128 + i] = s[i];
-    for (int i = 0; i < 64; i++) p1[b * 64 + i] = s[128 + i];
-    for (int i = 0; i < 16; i++) p2[b * 16 + i] = s[192 + i];
-    p3[2 * b] = s[208];
-    p3[2 * b + 1] = s[209];
+// Q6_K (210-byte blocks of 256: ql[128], qh[64], 16 int8 scales, f16 d; element 128 nn + 32 k + l of a block has its low
+// nibble in ql[64 nn + l + 32 (k & 1)] (high half for k >= 2) and its two high bits at bit 2 k of qh[32 nn + l],
+// src/ggml.rs:774-793) -> T6K records; one thread per lane slot of a record.
+__global__ __launch_bounds__(256) void pack_t6k_kernel(const uint8_t* __restrict__ raw, uint32_t n_out, uint32_t n_in, uint8_t* __restrict__ dst) {
+    const uint32_t nsteps = t6k_steps(n_in), nb = n_in / 256;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x, total = (size_t)row_tiles(n_out) * nsteps * 64;
+    if (idx >= total) return;
+    const uint32_t l = idx & 63, n = l & 15, kq = l >> 4;
+    const size_t recno = idx >> 6, tile = recno / nsteps, st = recno % nsteps, row = tile * 16 + n;
+    uint8_t* rec = dst + recno * T6K_REC;
+    uint32_t lo[4] = {0, 0, 0, 0}, hi[2] = {0, 0};
+    const bool live = row < n_out;
+    const uint8_t* blk = raw + ((live ? row : 0) * nb + st / 2) * 210;
+    const uint32_t nn = st & 1;
+    if (live) {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                const uint32_t wi = 64 * h + 16 * kq + j, k = wi >> 5, e = wi & 31;
+                const uint8_t qb = blk[64 * nn + e + 32 * (k & 1)];
+                const uint32_t lo4 = k < 2 ? (qb & 0xFu) : (qb >> 4), hi2 = (blk[128 + 32 * nn + e] >> (2 * k)) & 3u;
+                lo[2 * h + (j >> 3)] |= lo4 << (8 * (j & 3) + 4 * ((j & 7) >> 2));
+                hi[h] |= hi2 << (8 * (j & 3) + 2 * (j >> 2));
+            }
+    }
+    *reinterpret_cast<uint4*>(rec + 16 * l) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    *reinterpret_cast<uint2*>(rec + 1024 + 8 * l) = make_uint2(hi[0], hi[1]);
+    if (kq == 0) {
+        uint32_t s0 = 0, s1 = 0;
+        uint16_t d = 0;
+        if (live) {
+            for (int i = 0; i < 4; i++) {
+                s0 |= (uint32_t)blk[192 + 8 * nn + i] << (8 * i);
+                s1 |= (uint32_t)blk[192 + 8 * nn + 4 + i] << (8 * i);
+            }
+            d = (uint16_t)(blk[208] | (blk[209] << 8));
+        }
+        *reinterpret_cast<uint2*>(rec + 1536 + 8 * n) = make_uint2(s0, s1);
+        *reinterpret_cast<uint16_t*>(rec + 1664 + 2 * n) = d;
+    }
 }
 
 hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t n_in, const WeightView& d, hipStream_t s) {
@@ -244,10 +275,9 @@ hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t 
         size_t total = (size_t)row_tiles((uint32_t)n_out) * tk4_sbs((uint32_t)n_in) * 128;
         pack_tk4_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
     } else if (fmt == FMT_Q6_K) {
-        size_t nblocks = n_out * (n_in / 256);
-        if (!nblocks) return hipSuccess;
-        repack_q6k_kernel<<<(unsigned)((nblocks + 255) / 256), 256, 0, s>>>(raw, nblocks, p0, const_cast<uint8_t*>(d.p1),
-                                                                           const_cast<uint8_t*>(d.p2), const_cast<uint8_t*>(d.p3));
+        size_t total = (size_t)row_tiles((uint32_t)n_out) * t6k_steps((uint32_t)n_in) * 64;
+        if (!total) return hipSuccess;
+        pack_t6k_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
     } else {
         return hipErrorInvalidValue;
     }

@@ -21,7 +21,7 @@ namespace oxhip {
 //         p1 sc  [n_out][n_in/sgroup] f16 scale; sgroup = 32, or the offset group when every block
 //                                     of a group carries the same scale
 //         p2 off [n_out][n_in/group]  bf16 offsets, optional
-//   Q6_K  p0 ql  [n_out][nb][128], p1 qh [n_out][nb][64], p2 sc [n_out][nb][16] int8, p3 d [n_out][nb] f16
+//   Q6_K  p0      T6K records (layout.hpp)
 //   FP8   p0 q   [n_out][n_in]        e4m3 bytes (row-major, or tile-packed when group == 1: fp8_offset below);
 //         p1 bs f32 [ceil(n_out/br)][ceil(n_in/bc)]
 //   BF16  p0 q   [n_out][n_in]        bf16

@@ -31,14 +31,24 @@ namespace oxhip {
 constexpr uint32_t T8_REC = 1088;
 constexpr uint32_t TK4_REC = 2368;
 constexpr uint32_t T4M_REC = 1152;
+// Q6_K, 16 rows x 128 columns (half a super-block), lane = 16 kq + n, code j of half h = row n, column 64 h + 16 kq + j:
+//   [0, 1024)    low nibbles, 16 bytes per lane: dword 2 h + j / 8, byte j % 4, low nibble if j % 8 < 4, else high
+//   [1024, 1536) the two high bits, 8 bytes per lane: dword h, bits 8 (j % 4) + 2 (j / 4)
+//   [1536, 1664) the 8 int8 scales of row n's 16-column sub-blocks (sub-block 4 h + kq), 8 bytes per row
+//   [1664, 1696) f16 d of row n's super-block
+// so (dword >> 4 i) & 0x0F0F0F0F | ((high >> 2 r) & 0x03030303) << 4 are the four int8 operand dwords of a lane.
+constexpr uint32_t T6K_REC = 1696;
 
 __host__ __device__ inline uint32_t t8_steps(uint32_t n_in) { return (n_in / 32 + 1) / 2; }
 __host__ __device__ inline uint32_t tk4_sbs(uint32_t n_in) { return n_in / 256; }
 __host__ __device__ inline uint32_t t4m_steps(uint32_t n_in) { return (n_in / 32 + 3) / 4; }
+__host__ __device__ inline uint32_t t6k_steps(uint32_t n_in) { return n_in / 128; }
 __host__ __device__ inline uint32_t row_tiles(uint32_t n_out) { return (n_out + 15) / 16; }
 
 __host__ __device__ inline size_t t8_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t8_steps(n_in) * T8_REC; }
 __host__ __device__ inline size_t tk4_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * tk4_sbs(n_in) * TK4_REC; }
 __host__ __device__ inline size_t t4m_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t4m_steps(n_in) * T4M_REC; }
+
+__host__ __device__ inline size_t t6k_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t6k_steps(n_in) * T6K_REC; }
 
 }  // namespace oxhip
