@@ -33,7 +33,7 @@ KERNEL_FMT = {Q8_0: 1, Q4_K: 2, Q6_K: 3}  # template argument in the kernel symb
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # benchmark (KiB per dispatch, FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000: what a 256 MiB device copy
 # reads on the same counters); profiles/decode_batch_kernel_gguf_gemv.md holds the summary.
-TRAFFIC_BYTES = {"decode_batch_kernel": 391953180}
+TRAFFIC_BYTES = {"decode_batch_kernel": 391953180, "decode_batch_kernel/q6k": 200013764}
 
 
 def weight_bytes(kind, n_out, n_in):
@@ -358,7 +358,7 @@ def main():
                    "matmuls_per_step": len(cases), "launches_per_step": 1 if shared else len(cases), "bytes_per_step": step_bytes,
                    "weight_pool_GB_per_shape": args.pool_gb, "activations": "int8 per 32 (quantize_act), resident in HBM"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES.get(dom_symbol) if all(k in (Q8_0, Q4_K) for k in kinds) else None, "kernel": dom_symbol,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES.get(dom_symbol if all(k in (Q8_0, Q4_K) for k in kinds) else dom_symbol + "/q6k"), "kernel": dom_symbol,
                      "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_avg_s * 1e6, 2)},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "detail": detail,
