@@ -95,7 +95,7 @@ void oxhip_free_weight(oxhip_ctx* ctx, oxhip_weight* w);
 size_t oxhip_weight_bytes(const oxhip_weight* w);
 /* Backend::matmul (src/gpu.rs:160; src/cuda.rs:1428-1493): all jobs share x [t, n_in] (host f32);
  * computes every job or none. Routing as matmul_quant_multi_at's (src/kernels.rs:1731-1879): up to 8 tokens the
- * Q8_0 / Q4_K / MLX 4-bit jobs share one launch of the int8 decode kernel (the CPU's decode semantics,
+ * Q8 / Q8_0 / Q4_K / Q6_K / MLX 4-bit jobs share one launch of the int8 decode kernel (the CPU's decode semantics,
  * src/kernels.rs:1908-1928); more than 16 tokens over MLX 4-bit or FP8 (128-column blocks) weights run the bf16
  * matrix-core GEMM; everything else runs the decode kernels over 16 tokens at a time. */
 int oxhip_matmul(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_job* jobs, size_t n_jobs);
@@ -138,7 +138,7 @@ int oxhip_dev_decode(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa
                      void* stream);
 /* Several independent decode matmuls in one call (a decode step issues many small matmuls; what
  * matmul_quant_batch does for the CPU, src/kernels.rs:1937-1994). The jobs must not depend on one another: runs of
- * consecutive jobs of at most 8 tokens over Q8_0 / Q4_K / MLX 4-bit weights share ONE launch (their latency chains
+ * consecutive jobs of at most 8 tokens over Q8 / Q8_0 / Q4_K / Q6_K / MLX 4-bit weights share ONE launch (their latency chains
  * overlap; every job's rows are bit-identical to a launch of its own), the others launch one by one, in order, on
  * `stream`. ev_start / ev_stop (from oxhip_event_create, or NULL) are recorded before / after the launch that
  * holds the job: for jobs that share a launch they bracket the whole shared launch.
@@ -190,7 +190,7 @@ int oxhip_dev_route_top_k(oxhip_ctx* ctx, const float* logits, size_t t, size_t 
 int oxhip_dev_moe(oxhip_ctx* ctx, oxhip_moe* m, const float* x, size_t t, const uint32_t* route_idx, const float* route_w,
                   size_t k, float* y, void* stream);
 /* The exact integer accumulators of the decode kernels, written by the kernels themselves: per
- * block of 32 ([t, n_out, n_in/32]) for Q4, Q8_0 and Q4_K, per 16 ([t, n_out, n_in/16]) for Q6_K.
+ * block of 32 ([t, n_out, n_in/32]) for Q4, Q8, Q8_0 and Q4_K, per 16 ([t, n_out, n_in/16]) for Q6_K.
  * For parity checks (the CPU's per-16 sums add up to the per-32 ones exactly). */
 int oxhip_dev_isums(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa, int32_t* out, void* stream);
 

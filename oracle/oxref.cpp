@@ -711,6 +711,35 @@ void oxref_q4_decode(const uint8_t* q, const uint16_t* sc, const uint16_t* off, 
 }
 
 // ---------------------------------------------------------------------------------------------
+// Q8 (QMatrix: int8 codes, one f32 scale per block of 32)
+// ---------------------------------------------------------------------------------------------
+// dequantize_rows (src/quant.rs:405-419): q as f32 * scale.
+void oxref_q8_dequant_rows(const int8_t* q, const float* scales, size_t n_in, size_t r0, size_t r1, float* out) {
+    size_t bpr = n_in / QBLOCK;
+    for (size_t r = r0; r < r1; r++)
+        for (size_t b = 0; b < bpr; b++)
+            for (size_t j = 0; j < QBLOCK; j++) out[(r - r0) * n_in + b * QBLOCK + j] = (float)q[r * n_in + b * QBLOCK + j] * scales[r * bpr + b];
+}
+
+// QMat::rows_t1 for QMatrix, portable branch (src/kernels.rs:1156-1167): per block the exact int32 dot, then
+// acc += s as f32 * scale_b * xs_b, blocks in order; every token on its own (rows_tc's portable branch, :1207-1212).
+void oxref_q8_decode(const int8_t* q, const float* scales, size_t n_out, size_t n_in, const float* x, size_t t, float* y, int32_t* isums) {
+    QActBuf xa(x, t, n_in);
+    size_t bpr = n_in / QBLOCK;
+    for (size_t c = 0; c < t; c++)
+        for (size_t r = 0; r < n_out; r++) {
+            float acc = 0.0f;
+            for (size_t b = 0; b < bpr; b++) {
+                int32_t sum = 0;
+                for (size_t j = 0; j < QBLOCK; j++) sum += (int32_t)q[r * n_in + b * QBLOCK + j] * (int32_t)xa.q[c * n_in + b * QBLOCK + j];
+                if (isums) isums[(c * n_out + r) * bpr + b] = sum;
+                acc += (float)sum * scales[r * bpr + b] * xa.scales[c * bpr + b];
+            }
+            y[c * n_out + r] = acc;
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
 // GGUF decode, portable definition (src/ggml.rs:1288-1315)
 // ---------------------------------------------------------------------------------------------
 static void gguf_dot_row(uint32_t kind, const uint8_t* row, size_t n_in, const QActBuf& xa, size_t c0,

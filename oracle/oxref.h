@@ -71,6 +71,9 @@ void oxref_dequant_rows_q4(const uint8_t* q, const uint16_t* sc, const uint16_t*
 
 /* Decode (int8 activations).  y is [t][n_out].  isums (optional) receives the exact integer
  * accumulators: Q4 per block of 32 [t][n_out][n_in/32]; GGUF per 16 [t][n_out][n_in/16]. */
+/* Q8 (QMatrix, src/quant.rs:128-133): dequantize_rows (src/quant.rs:405-419) and the portable rows_t1 (src/kernels.rs:1156-1167). */
+void oxref_q8_dequant_rows(const int8_t* q, const float* scales, size_t n_in, size_t r0, size_t r1, float* out);
+void oxref_q8_decode(const int8_t* q, const float* scales, size_t n_out, size_t n_in, const float* x, size_t t, float* y, int32_t* isums);
 void oxref_q4_decode(const uint8_t* q, const uint16_t* sc, const uint16_t* off, size_t group,
                      size_t n_out, size_t n_in, const float* x, size_t t, float* y, int32_t* isums);
 void oxref_q4_decode_avx2(const uint8_t* q, const uint16_t* sc, const uint16_t* off, size_t group,

@@ -50,6 +50,8 @@ def _load():
         "oxref_mlx_dequant_row": (None, [vp, vp, vp, sz, sz, sz, vp]),
         "oxref_dequant_rows_q4": (None, [vp, vp, vp, sz, sz, sz, sz, vp]),
         "oxref_q4_decode": (None, [vp, vp, vp, sz, sz, sz, vp, sz, vp, vp]),
+        "oxref_q8_dequant_rows": (None, [vp, vp, sz, sz, sz, vp]),
+        "oxref_q8_decode": (None, [vp, vp, sz, sz, vp, sz, vp, vp]),
         "oxref_q4_decode_avx2": (None, [vp, vp, vp, sz, sz, sz, vp, sz, vp, C.c_int]),
         "oxref_gguf_decode": (None, [C.c_uint32, vp, sz, sz, vp, sz, vp, vp]),
         "oxref_gguf_decode_avx2": (None, [C.c_uint32, vp, sz, sz, vp, sz, vp, C.c_int]),
@@ -206,6 +208,24 @@ def q4_decode(q, sc, off, group, n_out, n_in, x, t, want_isums=False, avx2=False
         return y
     isums = np.empty((t, n_out, n_in // 32), np.int32) if want_isums else None
     lib.oxref_q4_decode(_p(q), _p(sc), _p(off), group, n_out, n_in, _p(x), t, _p(y), _p(isums))
+    return (y, isums) if want_isums else y
+
+
+def q8_dequant_rows(q, scales, n_out, n_in, r0=0, r1=None):
+    """QMatrix rows as f32 (src/quant.rs:405-419)."""
+    q, scales = _c(q, np.int8), _c(scales, np.float32)
+    r1 = n_out if r1 is None else r1
+    out = np.empty((r1 - r0, n_in), np.float32)
+    lib.oxref_q8_dequant_rows(_p(q), _p(scales), n_in, r0, r1, _p(out))
+    return out
+
+
+def q8_decode(q, scales, n_out, n_in, x, t, want_isums=False):
+    """QMatrix decode product (src/kernels.rs:1156-1167) and, on request, its int32 block sums [t, n_out, n_in/32]."""
+    q, scales, x = _c(q, np.int8), _c(scales, np.float32), _c(x, np.float32)
+    y = np.empty((t, n_out), np.float32)
+    isums = np.empty((t, n_out, n_in // 32), np.int32) if want_isums else None
+    lib.oxref_q8_decode(_p(q), _p(scales), n_out, n_in, _p(x), t, _p(y), _p(isums))
     return (y, isums) if want_isums else y
 
 

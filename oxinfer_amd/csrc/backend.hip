@@ -175,6 +175,19 @@ oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) {
     hipStream_t s = c->stream;
     Planes pl;
     switch (d->kind) {
+        case OXHIP_W_Q8: {  // QMatrix (src/quant.rs:128-133)
+            if (n_in % 32 || !d->scales) return fail("Q8 needs n_in % 32 == 0 and its f32 scales");
+            w->v.fmt = FMT_Q8F;
+            pl.add(0, t8f_bytes((uint32_t)n_out, (uint32_t)n_in));
+            if (!alloc(pl, 1)) return fail("device memory short");
+            Temp q, sc;
+            if (!have_memory(n_out * n_in + n_out * (n_in / 32) * 4) || !q.put(d->data, n_out * n_in, s) || !sc.put(d->scales, n_out * (n_in / 32) * 4, s))
+                return fail("device memory short");
+            if (launch_pack_q8f(static_cast<const int8_t*>(q.p), static_cast<const float*>(sc.p), n_out, n_in, static_cast<uint8_t*>(w->base), s) != hipSuccess)
+                return fail("pack launch failed");
+            if (hipStreamSynchronize(s) != hipSuccess) return fail("pack failed");
+            break;
+        }
         case OXHIP_W_BF16: {
             if (n_in % 8) return fail("bf16 rows must be a multiple of 8");
             w->v.fmt = FMT_BF16;

@@ -295,6 +295,7 @@ hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x
                          const DecodeScratch& sc) {
     switch (w.fmt) {
         case FMT_Q8_0:
+        case FMT_Q8F:
         case FMT_Q4_K:
         case FMT_Q6_K:
         case FMT_Q4M: return launch_decode_mfma(w, xa, t, y, sc, s);
@@ -310,7 +311,7 @@ hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x
 }
 
 hipError_t launch_isums(const WeightView& w, const QActView& xa, size_t t, int32_t* out, hipStream_t s) {
-    if (w.fmt == FMT_Q8_0 || w.fmt == FMT_Q4_K || w.fmt == FMT_Q6_K || w.fmt == FMT_Q4M) return launch_isums_mfma(w, xa, t, nullptr, out, s);
+    if (mfma_decode_format(w.fmt)) return launch_isums_mfma(w, xa, t, nullptr, out, s);
     size_t units = w.n_in / 32;
     size_t total = t * w.n_out * units;
     unsigned grid = (unsigned)((total + 255) / 256);

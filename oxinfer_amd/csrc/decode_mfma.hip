@@ -94,6 +94,11 @@ struct Step<FMT_Q8_0> {
     uint32_t a[2];
 };
 template <>
+struct Step<FMT_Q8F> {
+    uint4 w;
+    uint32_t a[2];
+};
+template <>
 struct Step<FMT_Q4_K> {
     uint4 w;
     uint32_t a[4];
@@ -110,7 +115,7 @@ struct Step<FMT_Q6_K> {
     uint32_t a[1];
 };
 
-// FMT: FMT_Q8_0 / FMT_Q4_K / FMT_Q4M. NT: tokens handled (1, 2, 4 or 8). DUMP: also write the exact
+// FMT: FMT_Q8_0 / FMT_Q8F (the same codes with f32 scales) / FMT_Q4_K / FMT_Q6_K / FMT_Q4M. NT: tokens handled (1, 2, 4 or 8). DUMP: also write the exact
 // integer block sums to `dump` ([t][n_out][n_in/32]) for parity checks.
 // GROUPED: blockIdx.y walks the chunks of a grouped launch (MoE experts over their routed tokens): chunk c is
 // {expert, first row, rows (<= 8 NG)}; the weights are expert's, activation row i of the chunk is row
@@ -128,7 +133,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     static_assert(NG == 1 || (GROUPED && ALDS && !DUMP && NT == 8), "token groups are for grouped launches");
     constexpr int TPAD = NT <= 4 ? 4 : 8;
     constexpr int NI = NT < 4 ? NT : 4;          // accumulator registers that hold live tokens
-    constexpr bool SUMS = FMT != FMT_Q8_0;
+    constexpr bool SUMS = !q8_format(FMT);
     // the wave index and everything derived from it (tile, K range) live in scalar registers: branches on them are
     // scalar, and the load counters the compiler keeps stay exact across them
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -141,8 +146,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     const uint32_t tile = bx * rt + r;
     const uint32_t ntiles = row_tiles(w.n_out);
     // this workgroup's slice of K: steps [S0, S1), blocks [B0, B0 + nbl) (a multiple of 4 blocks)
-    constexpr uint32_t BPS = FMT == FMT_Q8_0 ? 2 : 4;  // blocks of 32 per step
-    const uint32_t nsteps = FMT == FMT_Q8_0   ? t8_steps(w.n_in)
+    constexpr uint32_t BPS = q8_format(FMT) ? 2 : 4;  // blocks of 32 per step
+    const uint32_t nsteps = q8_format(FMT)    ? t8_steps(w.n_in)
                             : FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in)
                             : FMT == FMT_Q6_K ? t6k_steps(w.n_in)
                                               : t4m_steps(w.n_in);
@@ -178,6 +183,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     const uint32_t s0 = S0 + ks * per;
     const uint32_t s1 = tile < ntiles ? min(S1, s0 + per) : 0;  // a tile past the matrix streams nothing
     const uint8_t* base = w.p0 + (size_t)min(tile, ntiles - 1) * (FMT == FMT_Q8_0   ? (size_t)nsteps * T8_REC
+                                                                  : FMT == FMT_Q8F  ? (size_t)nsteps * T8F_REC
                                                                   : FMT == FMT_Q4_K ? (size_t)(nsteps / 2) * TK4_REC
                                                                   : FMT == FMT_Q6_K ? (size_t)nsteps * T6K_REC
                                                                                     : (size_t)nsteps * T4M_REC);
@@ -188,8 +194,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         out[1] = v.y;
     };
     auto load_step = [&](Step<FMT>& st, uint32_t s) {
-        if constexpr (FMT == FMT_Q8_0) {
-            const uint8_t* rec = base + (size_t)s * T8_REC;
+        if constexpr (q8_format(FMT)) {
+            const uint8_t* rec = base + (size_t)s * (FMT == FMT_Q8F ? T8F_REC : T8_REC);
             st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
             if (!ALDS) act2(2 * s + a_half, 8 * kq, st.a);
         } else if constexpr (FMT == FMT_Q4_K) {
@@ -223,11 +229,14 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // kq asks for the words of step `first + kq` (row n of it), and at step first + q every lane takes them from lane
     // 16 q + n. Q8_0: {d of the two blocks}; Q4_K: {four sub-block scales, four mins, (d, dmin)}: this step's four
     // sub-blocks are 4 (s & 1) .. + 3 of the super-block; MLX: {d of the two groups, offsets of the two groups}.
-    constexpr int NM = FMT == FMT_Q8_0 ? 1 : (FMT == FMT_Q4_K || FMT == FMT_Q6_K) ? 3 : 2;
+    constexpr int NM = FMT == FMT_Q8_0 ? 1 : (FMT == FMT_Q4_K || FMT == FMT_Q6_K) ? 3 : 2;  // (Q8F: the two f32 scales)
     const uint32_t slast = max(s1, 1u) - 1;
     auto load_scales = [&](uint32_t* m, uint32_t first) {
         const uint32_t s = min(first + kq, slast);
-        if constexpr (FMT == FMT_Q8_0) {
+        if constexpr (FMT == FMT_Q8F) {
+            m[0] = *reinterpret_cast<const uint32_t*>(base + (size_t)s * T8F_REC + 1024 + 8 * n);
+            m[1] = *reinterpret_cast<const uint32_t*>(base + (size_t)s * T8F_REC + 1028 + 8 * n);
+        } else if constexpr (FMT == FMT_Q8_0) {
             m[0] = *reinterpret_cast<const uint32_t*>(base + (size_t)s * T8_REC + 1024 + 4 * n);
         } else if constexpr (FMT == FMT_Q4_K) {
             const uint8_t* rec = base + (size_t)(s >> 1) * TK4_REC;
@@ -279,8 +288,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     };
     auto compute_step = [&](const Step<FMT>& st, const uint32_t* sw, uint32_t s) {
         const uint4 c = st.w;
-        if constexpr (FMT == FMT_Q8_0) {
-            const float d = f16_bits_to_f32((uint16_t)(d_half ? sw[0] >> 16 : sw[0] & 0xFFFF));
+        if constexpr (q8_format(FMT)) {
+            const float d = FMT == FMT_Q8F ? __uint_as_float(d_half ? sw[NM - 1] : sw[0]) : f16_bits_to_f32((uint16_t)(d_half ? sw[0] >> 16 : sw[0] & 0xFFFF));
             v4i bw = {(int)c.x, (int)c.y, (int)c.z, (int)c.w};
             const uint32_t b = 2 * s + d_half;
 #pragma unroll
@@ -702,6 +711,7 @@ __global__ __launch_bounds__(1024) void decode_batch_kernel(BatchArgs a) {
     const uint32_t bx = blockIdx.x - jb.wg0;
     switch (jb.w.fmt) {
         case FMT_Q8_0: batch_dispatch<FMT_Q8_0>(jb, bx, lds_dyn); break;
+        case FMT_Q8F: batch_dispatch<FMT_Q8F>(jb, bx, lds_dyn); break;
         case FMT_Q4_K: batch_dispatch<FMT_Q4_K>(jb, bx, lds_dyn); break;
         case FMT_Q6_K: batch_dispatch<FMT_Q6_K>(jb, bx, lds_dyn); break;
         case FMT_Q4M: batch_dispatch<FMT_Q4M>(jb, bx, lds_dyn); break;
@@ -810,17 +820,17 @@ hipError_t launch_one(bool alds, dim3 grid, dim3 block, size_t lds, hipStream_t 
 
 template <int FMT>
 constexpr uint32_t steps_of(uint32_t n_in) {
-    return FMT == FMT_Q8_0 ? t8_steps(n_in) : FMT == FMT_Q4_K ? 2 * tk4_sbs(n_in) : FMT == FMT_Q6_K ? t6k_steps(n_in) : t4m_steps(n_in);
+    return q8_format(FMT) ? t8_steps(n_in) : FMT == FMT_Q4_K ? 2 * tk4_sbs(n_in) : FMT == FMT_Q6_K ? t6k_steps(n_in) : t4m_steps(n_in);
 }
 
 template <int FMT, bool DUMP>
 hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* dump, const DecodeScratch& sc, hipStream_t s) {
     const uint32_t ntiles = row_tiles(w.n_out), nsteps = steps_of<FMT>(w.n_in);
-    Shape sh = shape_for(ntiles, nsteps, true, FMT == FMT_Q8_0 ? 64 : 128);
+    Shape sh = shape_for(ntiles, nsteps, true, q8_format(FMT) ? 64 : 128);
     const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
     // slices need scratch: 8 token rows per slice and a counter per row group
     if (sh.ks > 1 && (!sc.partial || !sc.counters || sc.partial_floats < (size_t)sh.ks * 8 * w.n_out || sc.ncounters < groups))
-        sh = shape_for(ntiles, nsteps, false, FMT == FMT_Q8_0 ? 64 : 128);
+        sh = shape_for(ntiles, nsteps, false, q8_format(FMT) ? 64 : 128);
     const uint32_t nblk = w.n_in / 32;
     dim3 grid((ntiles + sh.rt - 1) / sh.rt, sh.ks), block(64 * sh.rt * sh.kw);
     size_t c0 = 0;
@@ -837,7 +847,7 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
         int32_t* du = dump ? dump + c0 * (size_t)w.n_out * nblk * (FMT == FMT_Q6_K ? 2 : 1) : nullptr;
         const int tpad = tc <= 4 ? 4 : 8;
         bool alds;
-        const size_t lds = lds_bytes(FMT != FMT_Q8_0, DUMP, FMT == FMT_Q8_0 ? 2 : 4, nsteps, tpad, sh, &alds);
+        const size_t lds = lds_bytes(!q8_format(FMT), DUMP, q8_format(FMT) ? 2 : 4, nsteps, tpad, sh, &alds);
         if (lds > LDS_MAX) return hipErrorInvalidValue;  // rows too long for the staged activation scales
         const uint32_t tt = (uint32_t)tc;
         hipError_t e;
@@ -870,7 +880,7 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
     const uint32_t ng = max_rows <= 8 ? 1 : (max_rows <= 16 ? 2 : 4);
     if (max_rows > 32) return hipErrorInvalidValue;
     bool alds;
-    const size_t lds = lds_bytes(FMT != FMT_Q8_0, false, FMT == FMT_Q8_0 ? 2 : 4, nsteps, tpad, sh, &alds, ng);
+    const size_t lds = lds_bytes(!q8_format(FMT), false, q8_format(FMT) ? 2 : 4, nsteps, tpad, sh, &alds, ng);
     if (lds > LDS_MAX || (ng > 1 && !alds)) return hipErrorInvalidValue;
     const DecodeScratch none{};
     if (max_rows == 1) return launch_one<FMT, 1, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
@@ -884,7 +894,7 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
 
 namespace {
 uint32_t steps_rt(const WeightView& w) {
-    return w.fmt == FMT_Q8_0   ? steps_of<FMT_Q8_0>(w.n_in)
+    return q8_format(w.fmt)    ? steps_of<FMT_Q8_0>(w.n_in)
            : w.fmt == FMT_Q4_K ? steps_of<FMT_Q4_K>(w.n_in)
            : w.fmt == FMT_Q6_K ? steps_of<FMT_Q6_K>(w.n_in)
                                : steps_of<FMT_Q4M>(w.n_in);
@@ -892,11 +902,11 @@ uint32_t steps_rt(const WeightView& w) {
 }  // namespace
 
 bool decode_batchable(const WeightView& w, size_t t) {
-    if (w.fmt != FMT_Q8_0 && w.fmt != FMT_Q4_K && w.fmt != FMT_Q6_K && w.fmt != FMT_Q4M) return false;
+    if (!mfma_decode_format(w.fmt)) return false;
     if (t < 1 || t > 8) return false;
-    const Shape sh = shape_for(row_tiles(w.n_out), steps_rt(w), true, w.fmt == FMT_Q8_0 ? 64 : 128);  // as a launch of its own: same bits
+    const Shape sh = shape_for(row_tiles(w.n_out), steps_rt(w), true, q8_format(w.fmt) ? 64 : 128);  // as a launch of its own: same bits
     bool alds;
-    const size_t lds = lds_bytes(w.fmt != FMT_Q8_0, false, w.fmt == FMT_Q8_0 ? 2 : 4, steps_rt(w), t <= 4 ? 4 : 8, sh, &alds);
+    const size_t lds = lds_bytes(!q8_format(w.fmt), false, q8_format(w.fmt) ? 2 : 4, steps_rt(w), t <= 4 ? 4 : 8, sh, &alds);
     return alds && lds <= LDS_MAX;
 }
 
@@ -925,9 +935,9 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
         for (uint32_t j = 0; j < a.njobs; j++) {
             const DecodeBatchItem& it = items[i0 + j];
             const uint32_t ntiles = row_tiles(it.w.n_out), nsteps = steps_rt(it.w);
-            const Shape sh = shape_for(ntiles, nsteps, true, it.w.fmt == FMT_Q8_0 ? 64 : 128);
+            const Shape sh = shape_for(ntiles, nsteps, true, q8_format(it.w.fmt) ? 64 : 128);
             bool alds;
-            const size_t l = lds_bytes(it.w.fmt != FMT_Q8_0, false, it.w.fmt == FMT_Q8_0 ? 2 : 4, nsteps, it.t <= 4 ? 4 : 8, sh, &alds);
+            const size_t l = lds_bytes(!q8_format(it.w.fmt), false, q8_format(it.w.fmt) ? 2 : 4, nsteps, it.t <= 4 ? 4 : 8, sh, &alds);
             if (!alds || l > LDS_MAX || it.t < 1 || it.t > 8) return hipErrorInvalidValue;
             const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
             float* partial = nullptr;
@@ -973,6 +983,7 @@ hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, c
 hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, const DecodeScratch& sc, hipStream_t s) {
     switch (w.fmt) {
         case FMT_Q8_0: return run<FMT_Q8_0, false>(w, xa, t, y, nullptr, sc, s);
+        case FMT_Q8F: return run<FMT_Q8F, false>(w, xa, t, y, nullptr, sc, s);
         case FMT_Q4_K: return run<FMT_Q4_K, false>(w, xa, t, y, nullptr, sc, s);
         case FMT_Q6_K: return run<FMT_Q6_K, false>(w, xa, t, y, nullptr, sc, s);
         case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, sc, s);
@@ -984,6 +995,7 @@ hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t,
 hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* out, hipStream_t s) {
     switch (w.fmt) {
         case FMT_Q8_0: return run<FMT_Q8_0, true>(w, xa, t, y, out, DecodeScratch{}, s);
+        case FMT_Q8F: return run<FMT_Q8F, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q4_K: return run<FMT_Q4_K, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q6_K: return run<FMT_Q6_K, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q4M: return run<FMT_Q4M, true>(w, xa, t, y, out, DecodeScratch{}, s);

@@ -38,6 +38,13 @@ __global__ __launch_bounds__(256) void dequantize_kernel(WeightView w, uint32_t 
             v = (float)(int8_t)rec[16 * (kq * 16 + nn) + 8 * h + j] * d;
             break;
         }
+        case FMT_Q8F: {  // q as f32 * scale (src/quant.rs:405-419)
+            uint32_t tile = r >> 4, nn = r & 15, b = c >> 5, st = b >> 1, h = b & 1, e = c & 31, kq = e >> 3, j = e & 7;
+            const uint8_t* rec = w.p0 + ((size_t)tile * t8_steps(n) + st) * T8F_REC;
+            float d = *reinterpret_cast<const float*>(rec + 1024 + 8 * nn + 4 * h);
+            v = (float)(int8_t)rec[16 * (kq * 16 + nn) + 8 * h + j] * d;
+            break;
+        }
         case FMT_Q4_K: {
             uint32_t tile = r >> 4, nn = r & 15, sb = c / 256, e = c % 256, pair = e / 64, hi = (e % 64) / 32, l = e % 32;
             uint32_t st = pair >> 1, jj = pair & 1, kq = l >> 3;
@@ -264,6 +271,36 @@ __global__ __launch_bounds__(256) void pack_t6k_kernel(const uint8_t* __restrict
         *reinterpret_cast<uint2*>(rec + 1536 + 8 * n) = make_uint2(s0, s1);
         *reinterpret_cast<uint16_t*>(rec + 1664 + 2 * n) = d;
     }
+}
+
+// QMatrix (q i8 [n_out][n_in], scales f32 [n_out][n_in/32]) -> T8F records; one thread per lane slot of a record.
+__global__ __launch_bounds__(256) void pack_t8f_kernel(const int8_t* __restrict__ q, const float* __restrict__ scales, uint32_t n_out, uint32_t n_in,
+                                                       uint8_t* __restrict__ dst) {
+    const uint32_t nsteps = t8_steps(n_in), nblk = n_in / 32;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x, total = (size_t)row_tiles(n_out) * nsteps * 64;
+    if (idx >= total) return;
+    const uint32_t l = idx & 63, nn = l & 15, kq = l >> 4;
+    const size_t ts = idx >> 6, tile = ts / nsteps, row = tile * 16 + nn;
+    const uint32_t st = (uint32_t)(ts % nsteps);
+    uint8_t* rec = dst + ts * T8F_REC;
+    uint2 c[2] = {make_uint2(0u, 0u), make_uint2(0u, 0u)};
+    float d[2] = {0.0f, 0.0f};
+    for (uint32_t h = 0; h < 2; h++) {
+        const uint32_t b = 2 * st + h;
+        if (row < n_out && b < nblk) {
+            c[h] = *reinterpret_cast<const uint2*>(q + row * n_in + 32 * b + 8 * kq);
+            d[h] = scales[row * nblk + b];
+        }
+    }
+    *reinterpret_cast<uint4*>(rec + 16 * l) = make_uint4(c[0].x, c[0].y, c[1].x, c[1].y);
+    if (kq == 0) *reinterpret_cast<float2*>(rec + 1024 + 8 * nn) = make_float2(d[0], d[1]);
+}
+
+hipError_t launch_pack_q8f(const int8_t* q, const float* scales, size_t n_out, size_t n_in, uint8_t* dst, hipStream_t s) {
+    const size_t total = (size_t)row_tiles((uint32_t)n_out) * t8_steps((uint32_t)n_in) * 64;
+    if (!total) return hipSuccess;
+    pack_t8f_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(q, scales, (uint32_t)n_out, (uint32_t)n_in, dst);
+    return hipGetLastError();
 }
 
 hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t n_in, const WeightView& d, hipStream_t s) {

@@ -22,11 +22,15 @@ namespace oxhip {
 //                                     of a group carries the same scale
 //         p2 off [n_out][n_in/group]  bf16 offsets, optional
 //   Q6_K  p0      T6K records (layout.hpp)
+//   Q8F   p0      T8F records: QMatrix, int8 codes with one f32 scale per 32
 //   FP8   p0 q   [n_out][n_in]        e4m3 bytes (row-major, or tile-packed when group == 1: fp8_offset below);
 //         p1 bs f32 [ceil(n_out/br)][ceil(n_in/bc)]
 //   BF16  p0 q   [n_out][n_in]        bf16
 // ------------------------------------------------------------------------------------------------
-enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6 };
+enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6, FMT_Q8F = 7 };
+// the formats of the matrix-core decode kernels (decode_mfma.hip); the two Q8 kinds carry no sums or offsets
+inline bool mfma_decode_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F || f == FMT_Q4_K || f == FMT_Q6_K || f == FMT_Q4M; }
+__host__ __device__ constexpr bool q8_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F; }
 
 struct WeightView {
     int fmt;
@@ -70,6 +74,7 @@ __host__ __device__ inline size_t fp8_offset(const WeightView& w, size_t row, si
     return ((row / 16) * nsteps + col / 128) * 2048 + 32 * (((col % 128) / 32) * 16 + row % 16) + col % 32;
 }
 inline bool fp8_tileable(size_t n_in, uint32_t br, uint32_t bc) { return n_in % 128 == 0 && bc % 128 == 0 && br % 16 == 0; }
+hipError_t launch_pack_q8f(const int8_t* q, const float* scales, size_t n_out, size_t n_in, uint8_t* dst, hipStream_t s);
 hipError_t launch_pack_fp8(const uint8_t* raw, size_t n_out, size_t n_in, uint8_t* dst, hipStream_t s);
 
 // Global scratch of the decode kernels that split K across workgroups: `partial` holds slices x 8 token rows of

@@ -29,6 +29,8 @@
 namespace oxhip {
 
 constexpr uint32_t T8_REC = 1088;
+// QMatrix (int8 codes, f32 scale per 32): the T8 codes followed by the two f32 block scales of each of the 16 rows.
+constexpr uint32_t T8F_REC = 1152;
 constexpr uint32_t TK4_REC = 2368;
 constexpr uint32_t T4M_REC = 1152;
 // Q6_K, 16 rows x 128 columns (half a super-block), lane = 16 kq + n, code j of half h = row n, column 64 h + 16 kq + j:
@@ -46,6 +48,7 @@ __host__ __device__ inline uint32_t t6k_steps(uint32_t n_in) { return n_in / 128
 __host__ __device__ inline uint32_t row_tiles(uint32_t n_out) { return (n_out + 15) / 16; }
 
 __host__ __device__ inline size_t t8_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t8_steps(n_in) * T8_REC; }
+__host__ __device__ inline size_t t8f_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t8_steps(n_in) * T8F_REC; }
 __host__ __device__ inline size_t tk4_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * tk4_sbs(n_in) * TK4_REC; }
 __host__ __device__ inline size_t t4m_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t4m_steps(n_in) * T4M_REC; }
 

@@ -258,6 +258,12 @@ class HipBackend:
                        block_scales=_np_ptr(bs), bs_rows=block[0], bs_cols=block[1])
         return self._upload(d, (data, bs))
 
+    def upload_q8(self, q, scales, n_out, n_in):
+        """WeightRef::Q8 (QMatrix, src/quant.rs:128-133): int8 codes, one f32 scale per block of 32."""
+        q, scales = np.ascontiguousarray(q, np.int8), np.ascontiguousarray(scales, np.float32)
+        d = WeightDesc(kind=W_Q8, n_out=n_out, n_in=n_in, data=_np_ptr(q), scales=_np_ptr(scales))
+        return self._upload(d, (q, scales))
+
     def upload_q4(self, q, scales, offsets, group, n_out, n_in):
         """WeightRef::Q4 (src/quant.rs:427-440): nibbles, f16 scales per 32, optional bf16 offsets."""
         q, scales = np.ascontiguousarray(q, np.uint8), np.ascontiguousarray(scales, np.uint16)

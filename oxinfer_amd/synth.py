@@ -29,6 +29,14 @@ def mlx_q4(n_out, n_in, seed, group=64):
     return w, sb, bb
 
 
+def q8_matrix(n_out, n_in, seed):
+    """QMatrix (src/quant.rs:128-133): int8 codes uniform in [-127, 127], f32 scale ~ |N(0, 0.01)| per block of 32."""
+    rng = np.random.default_rng(seed)
+    q = rng.integers(-127, 128, (n_out, n_in), dtype=np.int8)
+    scales = np.abs(rng.normal(0.0, 0.01, (n_out, n_in // 32))).astype(np.float32)
+    return q, scales
+
+
 def gguf_q8_0(n_out, n_in, seed):
     """Q8_0 blocks (34 B): f16 d ~ |N(0, 0.01)|, 32 int8 uniform in [-127, 127]."""
     rng = np.random.default_rng(seed)

@@ -157,6 +157,39 @@ def test_mlx_q4_repack_dequant_isums_decode(be, oxref):
             assert row_err(y, ref) < TOL
 
 
+@pytest.mark.parametrize("t", [1, 3, 8, 13])
+def test_q8_matrix_dequant_isums_decode(be, oxref, t):
+    """QMatrix (WeightRef::Q8, src/quant.rs:128-133): dequantized rows and int32 block sums bit for bit, the product
+    within 1e-3 of the CPU's (src/kernels.rs:1156-1167); a block count that is not a multiple of the step, ragged rows,
+    extreme codes in one row, and one job of a shared launch next to a GGUF one."""
+    from oxinfer_amd import synth
+    n_out, n_in = 45, 1024 + 96
+    q, sc = synth.q8_matrix(n_out, n_in, 31)
+    q[0, :] = 127
+    q[1, :] = -128
+    w = be.upload_q8(q, sc, n_out, n_in)
+    assert w is not None, be.last_error()
+    got = be.dequantize(w).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), oxref.q8_dequant_rows(q, sc, n_out, n_in).view(np.uint32))
+    x = synth.activations(t, n_in, 32 + t)
+    x[0, :] = 3.0  # all activation codes 127 in token 0: the largest sums of a block
+    ref, isum = oxref.q8_decode(q, sc, n_out, n_in, x, t, want_isums=True)
+    xa = be.quantize_act(dev(x))
+    assert np.array_equal(be.isums(w, xa, 32).cpu().numpy(), isum)
+    y = be.decode(w, xa=xa).cpu().numpy()
+    assert row_err(y, ref) < TOL
+    for c in range(min(t, 3)):  # batch invariance
+        y1 = be.decode(w, xa=be.quantize_act(dev(x[c:c + 1]))).cpu().numpy()
+        assert np.array_equal(y1[0].view(np.uint32), y[c].view(np.uint32)), c
+    if t <= 8:  # the host entry point: Q8 and Q8_0 jobs of one call share a launch
+        raw = synth.gguf_q8_0(24, n_in, 33)
+        w2 = be.upload_gguf(Q8_0, raw, 24, n_in)
+        ya, yb = np.full((t, n_out), np.nan, np.float32), np.full((t, 24), np.nan, np.float32)
+        assert be.matmul(x, t, n_in, [(w, ya), (w2, yb)]), be.last_error()
+        assert np.array_equal(ya.view(np.uint32), y.view(np.uint32))
+        assert row_err(yb, oxref.gguf_decode(Q8_0, raw, 24, n_in, x, t)) < TOL
+
+
 def test_q4_without_offsets_and_mixed_scales(be, oxref):
     """A plain Q4_0-layout matrix (no offsets; src/quant.rs:457-513) keeps one scale per block of 32."""
     n_out, n_in = 10, 512

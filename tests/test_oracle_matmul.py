@@ -89,6 +89,26 @@ def test_q4_decode_against_integer_brute_force_and_f64(oxref, t):
     assert row_err(yg, ref) < 1e-4
 
 
+@pytest.mark.parametrize("t", [1, 3])
+def test_q8_matrix_against_integer_brute_force_and_f64(oxref, t):
+    """QMatrix (src/quant.rs:128-133, src/kernels.rs:1156-1167): block sums against numpy integers, the product against
+    the f64 definition from the pinned quantize_act, the dequantized rows exactly (an int8 times an f32 is one rounding)."""
+    from oxinfer_amd import synth
+    n_out, n_in = 40, 384
+    q, sc = synth.q8_matrix(n_out, n_in, 9)
+    x = synth.activations(t, n_in, 10)
+    y, isums = oxref.q8_decode(q, sc, n_out, n_in, x, t, want_isums=True)
+    xq, xs, _, _, _ = oxref.quantize_act(x, t, n_in)
+    isum = (xq.reshape(t, 1, n_in // 32, 32).astype(np.int64) * q.reshape(1, n_out, n_in // 32, 32).astype(np.int64)).sum(axis=3)
+    assert np.array_equal(isums, isum)
+    ref = (isum * sc.astype(np.float64)[None] * xs.reshape(t, 1, -1).astype(np.float64)).sum(axis=2)
+    assert row_err(y, ref) < 1e-4
+    deq = oxref.q8_dequant_rows(q, sc, n_out, n_in)
+    assert np.array_equal(deq, (q.astype(np.float32).reshape(n_out, -1, 32) * sc[:, :, None]).reshape(n_out, n_in))
+    assert np.array_equal(oxref.q8_dequant_rows(q, sc, n_out, n_in, r0=3, r1=5), deq[3:5])
+    assert row_err(y, x.astype(np.float64) @ deq.astype(np.float64).T) < 3e-2  # the int8 activations' bound (src/ggml.rs:1904)
+
+
 def gguf_f64(oxref, kind, data, n_out, n_in, x, t):
     bs, ts = oxref.block_size(kind), oxref.type_size(kind)
     xq, xs, _, _, hs = oxref.quantize_act(x, t, n_in)
