@@ -38,17 +38,38 @@ __global__ __launch_bounds__(256) void pack_a_kernel(const void* __restrict__ x,
     const uint32_t tok = mt * 16 + m;
     uint32_t pk[4] = {0, 0, 0, 0};
     if (tok < t) {
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const uint32_t k = MODE == 1   ? 32 * b + (j < 4 ? 4 * kq + j : 16 + 4 * kq + (j - 4))
-                               : MODE == 2 ? 128 * (b >> 2) + 32 * kq + 8 * (b & 3) + j
-                                           : 32 * b + 8 * kq + j;
-            uint16_t h = 0;
-            if (k < n_in) {
-                if (SRC_BF16) h = reinterpret_cast<const uint16_t*>(x)[(size_t)tok * n_in + k];
-                else h = f32_to_bf16_bits(reinterpret_cast<const float*>(x)[(size_t)tok * n_in + k]);
+        // the lane's 8 values are two runs of 4 consecutive columns (SPLIT) or one run of 8: whole runs are fetched with
+        // one 8- or 16-byte request each (rows are multiples of 8 columns here), a ragged tail value by value
+        const uint32_t k0 = MODE == 1 ? 32 * b + 4 * kq : MODE == 2 ? 128 * (b >> 2) + 32 * kq + 8 * (b & 3) : 32 * b + 8 * kq;
+        const uint32_t k1 = MODE == 1 ? k0 + 16 : k0 + 4;  // first column of the second run of 4
+        const size_t row = (size_t)tok * n_in;
+        if (k1 + 4 <= n_in && n_in % 8 == 0) {
+            if (SRC_BF16) {
+                const uint16_t* xs = reinterpret_cast<const uint16_t*>(x) + row;
+                const uint2 a = *reinterpret_cast<const uint2*>(xs + k0), c = *reinterpret_cast<const uint2*>(xs + k1);
+                pk[0] = a.x;
+                pk[1] = a.y;
+                pk[2] = c.x;
+                pk[3] = c.y;
+            } else {
+                const float* xs = reinterpret_cast<const float*>(x) + row;
+                const float4 a = *reinterpret_cast<const float4*>(xs + k0), c = *reinterpret_cast<const float4*>(xs + k1);
+                pk[0] = f32_to_bf16_bits(a.x) | ((uint32_t)f32_to_bf16_bits(a.y) << 16);
+                pk[1] = f32_to_bf16_bits(a.z) | ((uint32_t)f32_to_bf16_bits(a.w) << 16);
+                pk[2] = f32_to_bf16_bits(c.x) | ((uint32_t)f32_to_bf16_bits(c.y) << 16);
+                pk[3] = f32_to_bf16_bits(c.z) | ((uint32_t)f32_to_bf16_bits(c.w) << 16);
             }
-            pk[j >> 1] |= (uint32_t)h << (16 * (j & 1));
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const uint32_t k = (j < 4 ? k0 : k1 - 4) + j;
+                uint16_t h = 0;
+                if (k < n_in) {
+                    if (SRC_BF16) h = reinterpret_cast<const uint16_t*>(x)[row + k];
+                    else h = f32_to_bf16_bits(reinterpret_cast<const float*>(x)[row + k]);
+                }
+                pk[j >> 1] |= (uint32_t)h << (16 * (j & 1));
+            }
         }
     }
     out[idx] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
