@@ -7,7 +7,7 @@
 namespace oxhip {
 
 // route_top_k: the k largest logits (ties to the lower index, total order on the float bits like
-// f32::total_cmp), weights exp(l - max) / sum over the k. One wavefront per token; n <= 1024.
+// f32::total_cmp), weights exp(l - max) / sum over the k. One wavefront per token; n <= 1024, k <= 64.
 __global__ __launch_bounds__(64) void route_top_k_kernel(const float* __restrict__ logits, uint32_t n, uint32_t k,
                                                          uint32_t* __restrict__ idx, float* __restrict__ wts) {
     const uint32_t tok = blockIdx.x, lane = threadIdx.x;
@@ -22,9 +22,10 @@ __global__ __launch_bounds__(64) void route_top_k_kernel(const float* __restrict
         const int b = live[i] ? __float_as_int(l[j]) : 0;
         key[i] = b ^ (int)(((uint32_t)(b >> 31)) >> 1);  // f32::total_cmp's order as a signed compare
     }
-    float sel[32];
-    uint32_t seli[32];
-    for (uint32_t r = 0; r < k && r < 32; r++) {
+    // round r's winner stays in lane r (a per-thread array indexed by r would turn into long select chains)
+    float mysel = 0.0f;
+    uint32_t myidx = 0;
+    for (uint32_t r = 0; r < k && r < 64; r++) {
         // this lane's best remaining logit (its indices ascend, so ties keep the lower one)
         int bk = 0;
         uint32_t bj = 0xFFFFFFFFu;
@@ -42,24 +43,22 @@ __global__ __launch_bounds__(64) void route_top_k_kernel(const float* __restrict
                 bj = oj;
             }
         }
-        seli[r] = bj;
-        sel[r] = __int_as_float(bk ^ (int)(((uint32_t)(bk >> 31)) >> 1));  // the key's transform is its own inverse
+        if (lane == r) {
+            myidx = bj;
+            mysel = __int_as_float(bk ^ (int)(((uint32_t)(bk >> 31)) >> 1));  // the key's transform is its own inverse
+        }
 #pragma unroll
         for (int i = 0; i < PER; i++)
             if (lane + 64 * i == bj) live[i] = false;
     }
-    if (lane == 0) {
-        const float m = sel[0];
-        float e[32];
-        float s = -0.0f;
-        for (uint32_t r = 0; r < k; r++) {
-            e[r] = expf(sel[r] - m);
-            s += e[r];
-        }
-        for (uint32_t r = 0; r < k; r++) {
-            idx[(size_t)tok * k + r] = seli[r];
-            wts[(size_t)tok * k + r] = e[r] / s;
-        }
+    // weights: exp(l - max) over the k, summed in rank order from -0.0 as the reference does
+    const float m = __shfl(mysel, 0);
+    const float e = lane < k ? expf(mysel - m) : 0.0f;
+    float sum = -0.0f;
+    for (uint32_t r = 0; r < k && r < 64; r++) sum += __shfl(e, (int)r);
+    if (lane < k) {
+        idx[(size_t)tok * k + lane] = myidx;
+        wts[(size_t)tok * k + lane] = e / sum;
     }
 }
 
