@@ -21,6 +21,7 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 // Requests to memory cost the same whether 4 or 64 of a wave's lanes take part, and at a few tokens they, not the bytes
 // of the weights, would bound the kernel. So a token tile's fragments are packed for the smallest TS in {4, 8, 16} that
@@ -74,12 +75,15 @@ __device__ inline uint4 row_take(const uint4& v) {
                       (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v.w, ctrl, 0xf, 0xf, true));
 }
 
+// DIRECT (at most 4 tokens, f32 activations kept exact): `apk` is x itself, [t][n_in] f32: lane 16 kq + n reads the 8
+// columns of token n % 4 and block n / 4 (32 bytes; a token's 16 lanes cover a step's 512 bytes) and splits them into
+// the bf16 value and residual planes in registers; no packing kernel and no scratch.
 // grid x: groups of RT row tiles; grid y: K slices; the workgroup's `kw` waves split the slice's steps and meet in LDS in
 // wave order; with more than one slice the sums go out as f32 partial rows [slice][t][n_out] that a second kernel adds.
 // PF: 128-column steps a wave keeps on request. A step's activation fragments (L2 hits) are requested together with its
 // weights: loads complete in issue order, so fragments asked for any later would make the wave wait for every weight
 // request issued before them and cut the depth of the ring.
-template <int RT, int NTT, int NP, int TS, bool OUT_BF16>
+template <int RT, int NTT, int NP, int TS, bool OUT_BF16, bool DIRECT = false>
 __global__ __launch_bounds__(512) void skinny_fp8_kernel(WeightView w, const uint4* __restrict__ apk, uint32_t t, uint32_t kw,
                                                          void* __restrict__ yv, float* __restrict__ partial) {
     constexpr int CNT = TS / 4, PER = 16 / TS;  // requests per step and plane; blocks b in a request
@@ -102,11 +106,15 @@ __global__ __launch_bounds__(512) void skinny_fp8_kernel(WeightView w, const uin
         wp[r] = w.p0 + fp8_offset(w, row, 32 * kq);
         sp[r] = reinterpret_cast<const float*>(w.p1) + (size_t)(tile * 16 / w.br) * scols;
     }
+    static_assert(!DIRECT || (TS == 4 && NP == 2 && NTT == 1), "direct f32 activations: up to 4 tokens, two planes");
     const uint4* ap = apk + lane;
+    // DIRECT: the lane's 8 columns of a step start at xd + 128 s (absent tokens read token t - 1 and are zeroed)
+    const float* xd = reinterpret_cast<const float*>(apk) + (size_t)min(n & 3u, t - 1) * w.n_in + 32 * kq + 8 * (n >> 2);
+    const bool xlive = (n & 3u) < t;
     struct St {
         uint4 lo[RT], hi[RT];
         float sc[RT];
-        uint4 a[NTT][NP][CNT];
+        uint4 a[NTT][NP][CNT];  // DIRECT: a[0][0][0], a[0][1][0] hold the 8 f32 values until they are split
     };
     auto load = [&](St& st, uint32_t s) {  // s: a step of the matrix
 #pragma unroll
@@ -116,12 +124,34 @@ __global__ __launch_bounds__(512) void skinny_fp8_kernel(WeightView w, const uin
             st.hi[r] = p[1];
             st.sc[r] = sp[r][(128 * s) / w.bc];
         }
+        if (DIRECT) {
+            const uint4* p = reinterpret_cast<const uint4*>(xd + 128 * (size_t)s);
+            st.a[0][0][0] = p[0];
+            st.a[0][NP - 1][0] = p[1];
+        } else {
 #pragma unroll
-        for (int tt = 0; tt < NTT; tt++)
+            for (int tt = 0; tt < NTT; tt++)
 #pragma unroll
-            for (int pl = 0; pl < NP; pl++)
+                for (int pl = 0; pl < NP; pl++)
 #pragma unroll
-                for (int i = 0; i < CNT; i++) st.a[tt][pl][i] = ap[((((size_t)tt * NP + pl) * nsteps + s) * CNT + i) * 64];
+                    for (int i = 0; i < CNT; i++) st.a[tt][pl][i] = ap[((((size_t)tt * NP + pl) * nsteps + s) * CNT + i) * 64];
+        }
+    };
+    // DIRECT: 8 f32 -> the two bf16 planes (round to nearest even; the residual x - bf16(x) is exact in f32)
+    auto split = [&](const St& st, uint4& hi, uint4& lo) {
+        const uint32_t raw[8] = {st.a[0][0][0].x, st.a[0][0][0].y, st.a[0][0][0].z, st.a[0][0][0].w,
+                                 st.a[0][NP - 1][0].x, st.a[0][NP - 1][0].y, st.a[0][NP - 1][0].z, st.a[0][NP - 1][0].w};
+        uint32_t h[4], l[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float x0 = xlive ? __uint_as_float(raw[2 * j]) : 0.0f, x1 = xlive ? __uint_as_float(raw[2 * j + 1]) : 0.0f;
+            const uint32_t hp = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{x0, x1}, bf16x2));
+            const float r0 = x0 - __uint_as_float(hp << 16), r1 = x1 - __uint_as_float(hp & 0xFFFF0000u);
+            h[j] = hp;
+            l[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{r0, r1}, bf16x2));
+        }
+        hi = make_uint4(h[0], h[1], h[2], h[3]);
+        lo = make_uint4(l[0], l[1], l[2], l[3]);
     };
     f32x4 acc[RT][NTT];
 #pragma unroll
@@ -132,8 +162,8 @@ __global__ __launch_bounds__(512) void skinny_fp8_kernel(WeightView w, const uin
     St ring[PF];
 #pragma unroll
     for (int p = 0; p < PF; p++) load(ring[p], gw + stride * min((uint32_t)p, ilast));
-    auto frag = [&](const St& st, int tt, int pl, int b) -> uint4 {
-        const uint4& v = st.a[tt][pl][b / PER];
+    auto frag = [&](const St& st, const uint4* dp, int tt, int pl, int b) -> uint4 {
+        const uint4& v = DIRECT ? dp[pl] : st.a[tt][pl][b / PER];
         switch (TS * (b % PER)) {
             case 4: return row_take<4>(v);
             case 8: return row_take<8>(v);
@@ -142,6 +172,8 @@ __global__ __launch_bounds__(512) void skinny_fp8_kernel(WeightView w, const uin
         }
     };
     auto compute = [&](const St& st) {
+        uint4 dp[2];
+        if (DIRECT) split(st, dp[0], dp[1]);
 #pragma unroll
         for (int r = 0; r < RT; r++) {
             const uint32_t d[8] = {st.lo[r].x, st.lo[r].y, st.lo[r].z, st.lo[r].w, st.hi[r].x, st.hi[r].y, st.hi[r].z, st.hi[r].w};
@@ -159,7 +191,7 @@ __global__ __launch_bounds__(512) void skinny_fp8_kernel(WeightView w, const uin
                 for (int tt = 0; tt < NTT; tt++)
 #pragma unroll
                     for (int pl = 0; pl < NP; pl++)
-                        D[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, frag(st, tt, pl, b)), wb, D[tt], 0, 0, 0);
+                        D[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, frag(st, dp, tt, pl, b)), wb, D[tt], 0, 0, 0);
             }
 #pragma unroll
             for (int tt = 0; tt < NTT; tt++)
@@ -229,14 +261,17 @@ hipError_t launch_skinny_fp8(const WeightView& w, const void* x, bool x_bf16, bo
     if (!skinny_fp8_ok(w, t)) return hipErrorInvalidValue;
     const uint32_t ttiles = (uint32_t)((t + 15) / 16), planes = (!x_bf16 && exact_f32) ? 2 : 1, nsteps = w.n_in / 128;
     const uint32_t ts = t <= 4 ? 4 : t <= 8 ? 8 : 16;
-    const size_t total = (size_t)ttiles * planes * nsteps * (ts / 4) * 64;
+    // up to 4 tokens of exact f32 activations: the kernel reads x itself (rows of whole 16-byte runs)
+    const bool direct = ts == 4 && planes == 2 && w.n_in % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+    const size_t total = direct ? 0 : (size_t)ttiles * planes * nsteps * (ts / 4) * 64;
     const unsigned pgrid = (unsigned)((total + 255) / 256);
-    if (x_bf16) pack_skinny_kernel<true><<<pgrid, 256, 0, s>>>(x, (uint32_t)t, w.n_in, ttiles, planes, nsteps, ts, static_cast<uint4*>(pack));
+    if (!total) {
+    } else if (x_bf16) pack_skinny_kernel<true><<<pgrid, 256, 0, s>>>(x, (uint32_t)t, w.n_in, ttiles, planes, nsteps, ts, static_cast<uint4*>(pack));
     else pack_skinny_kernel<false><<<pgrid, 256, 0, s>>>(x, (uint32_t)t, w.n_in, ttiles, planes, nsteps, ts, static_cast<uint4*>(pack));
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const uint32_t ntiles = (w.n_out + 15) / 16;
-    const uint4* a = static_cast<const uint4*>(pack);
+    const uint4* a = direct ? static_cast<const uint4*>(x) : static_cast<const uint4*>(pack);
     float* partial = reinterpret_cast<float*>(static_cast<uint8_t*>(pack) + frag_bytes(w, t, (int)planes));
     uint32_t slices = 1;
     auto go = [&](auto kern, uint32_t rt, uint32_t ntt) {
@@ -254,7 +289,8 @@ hipError_t launch_skinny_fp8(const WeightView& w, const void* x, bool x_bf16, bo
     auto pick = [&](auto np, auto out) {
         constexpr int NP = decltype(np)::value;
         constexpr bool OB = decltype(out)::value;
-        if (ts == 4) go(skinny_fp8_kernel<1, 1, NP, 4, OB>, 1, 1);
+        if (ts == 4 && NP == 2 && direct) go(skinny_fp8_kernel<1, 1, 2, 4, OB, true>, 1, 1);
+        else if (ts == 4) go(skinny_fp8_kernel<1, 1, NP, 4, OB>, 1, 1);
         else if (ts == 8) go(skinny_fp8_kernel<1, 1, NP, 8, OB>, 1, 1);
         else if (ttiles == 1) go(skinny_fp8_kernel<2, 1, NP, 16, OB>, 2, 1);
         else {
