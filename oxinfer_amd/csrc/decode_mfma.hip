@@ -27,6 +27,7 @@
 // its partial rows in global scratch and the last one to arrive (a counter per row group) adds the slices in slice
 // order: the association of a row's sum depends on the weight's shape only, never on arrival order, and there is
 // no second launch. A workgroup stages only its slice of the activations.
+#include <algorithm>
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
@@ -932,8 +933,28 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
         a.njobs = (uint32_t)(n - i0 < (size_t)BATCH_MAX ? n - i0 : (size_t)BATCH_MAX);
         size_t lds = 0, pf = 0, nc = 0;  // scratch is shared by the jobs of one launch, reused by the next launch
         uint32_t wg = 0, threads = 64;
+        // Block order within the launch. Workgroups start in block order, so the last jobs make the tail of the launch,
+        // when the CUs run dry one after the other: it is shortest when its workgroups do little work per byte and
+        // have no slices to combine. Formats with more instruction work per byte go first (4-bit, 6-bit, 8-bit; the
+        // caller's order within a format), and in the last format present the jobs that slice K go before the others.
+        uint32_t order[BATCH_MAX];
+        {
+            auto cls = [](int fmt) { return q8_format(fmt) ? 2 : fmt == FMT_Q6_K ? 1 : 0; };
+            auto sliced = [](const WeightView& w) {
+                return shape_for(row_tiles(w.n_out), steps_rt(w), true, q8_format(w.fmt) ? 64 : 128).ks > 1;
+            };
+            int last = 0;
+            for (uint32_t j = 0; j < a.njobs; j++) last = std::max(last, cls(items[i0 + j].w.fmt));
+            uint32_t key[BATCH_MAX];
+            for (uint32_t j = 0; j < a.njobs; j++) {
+                const WeightView& w = items[i0 + j].w;
+                key[j] = 2 * cls(w.fmt) + (cls(w.fmt) == last && !sliced(w) ? 1 : 0);
+                order[j] = j;
+            }
+            std::stable_sort(order, order + a.njobs, [&](uint32_t x, uint32_t y) { return key[x] < key[y]; });
+        }
         for (uint32_t j = 0; j < a.njobs; j++) {
-            const DecodeBatchItem& it = items[i0 + j];
+            const DecodeBatchItem& it = items[i0 + order[j]];
             const uint32_t ntiles = row_tiles(it.w.n_out), nsteps = steps_rt(it.w);
             const Shape sh = shape_for(ntiles, nsteps, true, q8_format(it.w.fmt) ? 64 : 128);
             bool alds;
