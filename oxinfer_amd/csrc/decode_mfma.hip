@@ -650,8 +650,16 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         const uint32_t tok = idx / (rt * 16), row = bx * rt * 16 + idx % (rt * 16);
         if (row >= w.n_out) continue;
         const float* p = partial + (size_t)tok * w.n_out + row;
-        float sum = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for (uint32_t z = 1; z < ksplit; z++) sum += __hip_atomic_load(p + (size_t)z * t * w.n_out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // four slices per round trip (a loop of one load per slice waits for each in turn); still added in slice order
+        float sum = 0.0f;
+        for (uint32_t z0 = 0; z0 < ksplit; z0 += 4) {
+            float v[4];
+#pragma unroll
+            for (uint32_t i = 0; i < 4; i++)
+                v[i] = __hip_atomic_load(p + (size_t)min(z0 + i, ksplit - 1) * t * w.n_out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (uint32_t i = 0; i < 4; i++) sum = z0 + i == 0 ? v[i] : z0 + i < ksplit ? sum + v[i] : sum;
+        }
         y[(size_t)tok * w.n_out + row] = sum;
     }
 }
@@ -729,34 +737,47 @@ struct Shape {
 constexpr uint32_t NCU = 256;
 
 // Workgroup shape (rt row tiles x kw waves per tile) and the number of K slices across workgroups (ks): a function of
-// the weight's shape only, so a row's sum is associated the same way whatever the batch or the kind of launch.
+// the weight's shape and format only, so a row's sum is associated the same way whatever the batch or the kind of
+// launch. A cost model fitted to measurements of the Llama-8B MLP shapes (steady streams of launches, single
+// launches and the shared launch of eight):
 //  * A matmul at these sizes is a chain of dependent latencies (stage activations, stream weights, reduce, store)
-//    and only overlaps them when a CU holds several workgroups in different phases: workgroups have at most 8 waves,
-//    and K is sliced until a workgroup's staged activations (11 bytes per column at 8 tokens) leave room for three
-//    workgroups in a CU's 160 KiB.
+//    and only overlaps them when a CU holds two workgroups in different phases (the registers allow no more):
+//    workgroups have at most 8 waves, and K is sliced until two workgroups' staged activations (11 bytes per column
+//    at 8 tokens) fit a CU's 160 KiB. Twice as many slices are also tried: they buy more, smaller workgroups.
+//  * Every further slice costs: its partial rows meet through memory (store, wait, count, and the last one reads
+//    them all), two to three round trips during which the workgroup holds its place and does nothing.
 //  * Among the (rt, kw) left, the pick minimizes the records that pass through the busiest CU when workgroups are
-//    dealt round-robin, and prefers a few records per wave, four or more waves, and little restaging.
-Shape search_shape(uint32_t ntiles, uint32_t nsteps, uint32_t cols_per_step) {
-    uint32_t ks = 1;
-    while (ks < 32 && (size_t)nsteps * cols_per_step * 11 / ks > 48 * 1024 && nsteps / (ks * 2) >= 4) ks *= 2;
-    while (ks > 1 && (nsteps + ks - 1) / ks * (ks - 1) >= nsteps) ks /= 2;  // no empty slice
-    const uint32_t sl = (nsteps + ks - 1) / ks;
-    Shape best{1, 1, ks};
+//    dealt round-robin, and prefers a few records per wave, four or more waves, enough workgroups for every CU, and
+//    little restaging (every workgroup stages its slice of the activations: 11 bytes per column next to the
+//    rt * bytes-per-column of weights it streams).
+Shape search_shape(uint32_t ntiles, uint32_t nsteps, uint32_t cols_per_step, double weight_bytes_per_col) {
+    uint32_t ks0 = 1;
+    while (ks0 < 32 && (size_t)nsteps * cols_per_step * 11 / ks0 > 80 * 1024 && nsteps / (ks0 * 2) >= 4) ks0 *= 2;
+    while (ks0 > 1 && (nsteps + ks0 - 1) / ks0 * (ks0 - 1) >= nsteps) ks0 /= 2;  // no empty slice
+    Shape best{1, 1, ks0};
     double best_cost = 1e300;
-    for (uint32_t kw = 1; kw <= 8; kw *= 2)
-        for (uint32_t rt = 1; rt * kw <= 8; rt++) {
-            const uint32_t per = (sl + kw - 1) / kw;
-            const uint64_t wgs = (uint64_t)((ntiles + rt - 1) / rt) * ks;
-            double cost = (double)((wgs + NCU - 1) / NCU) * rt * per * kw;  // records through the busiest CU
-            if (rt * kw < 4) cost *= 1.0 + 0.10 * (4 - rt * kw);
-            if (per < 8) cost *= 1.0 + 0.03 * (8 - per);    // short streams: the latency chain dominates
-            if (per > 16) cost *= 1.0 + 0.02 * (per - 16);  // long streams: too few waves keep HBM busy
-            cost *= 1.0 + 0.05 / rt + 0.002 * kw;  // every workgroup stages its slice again: larger groups restage less
-            if (cost < best_cost) {
-                best_cost = cost;
-                best = Shape{rt, kw, ks};
+    for (uint32_t ks = ks0; ks <= (ks0 > 1 ? 2 * ks0 : 1u); ks *= 2) {
+        if (ks > ks0 && (ks > 32 || nsteps / ks < 4 || (nsteps + ks - 1) / ks * (ks - 1) >= nsteps)) break;
+        const uint32_t sl = (nsteps + ks - 1) / ks;
+        double slices = 1.0;
+        for (uint32_t k = 1; k < ks; k *= 2) slices *= 1.06;
+        for (uint32_t kw = 1; kw <= 8; kw *= 2)
+            for (uint32_t rt = 1; rt * kw <= 8; rt++) {
+                const uint32_t per = (sl + kw - 1) / kw;
+                const uint64_t wgs = (uint64_t)((ntiles + rt - 1) / rt) * ks;
+                double cost = (double)((wgs + NCU - 1) / NCU) * rt * per * kw;  // records through the busiest CU
+                if (rt * kw < 4) cost *= 1.0 + 0.10 * (4 - rt * kw);
+                if (per < 8) cost *= 1.0 + 0.03 * (8 - per);     // short streams: the latency chain dominates
+                if (per > 16) cost *= 1.0 + 0.001 * (per - 16);  // long streams: fewer waves to keep HBM busy
+                if (wgs < NCU) cost *= 1.05;
+                cost *= 1.0 + 0.25 * 11.0 / (weight_bytes_per_col * rt) + 0.002 * kw;
+                cost *= slices;
+                if (cost < best_cost) {
+                    best_cost = cost;
+                    best = Shape{rt, kw, ks};
+                }
             }
-        }
+    }
     if (const char* e = getenv("OXHIP_DECODE_SHAPE")) {  // developer override for tuning runs: "tiles:steps=rt,kw,ks;..."
         for (const char* p = e; p && *p;) {
             unsigned nt = 0, ns = 0, a = 0, b = 0, c = 0;
@@ -772,14 +793,18 @@ Shape search_shape(uint32_t ntiles, uint32_t nsteps, uint32_t cols_per_step) {
 
 // The search runs once per shape: a decode launch is a few microseconds of GPU time and must not spend as long on
 // the host. Without scratch for the slices (allow_slices false) K stays inside a workgroup.
-Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices, uint32_t cols_per_step = 128) {
+Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices, int fmt) {
+    const uint32_t cols_per_step = q8_format(fmt) ? 64 : 128;
+    // weight bytes per column of a row tile, as the restaging term of the cost sees them: the 8-bit records, and the
+    // 4-bit ones for the 4- and 6-bit formats alike (the 6-bit records are larger but cost as many instructions more)
+    const double bytes_per_col = q8_format(fmt) ? (double)T8_REC / 64 : (double)TK4_REC / 256;
     static std::mutex mu;
     static std::map<uint64_t, Shape> cache;
-    const uint64_t key = ((uint64_t)ntiles << 34) | ((uint64_t)nsteps << 2) | (cols_per_step == 64 ? 2u : 0u) | (allow_slices ? 1u : 0u);
+    const uint64_t key = ((uint64_t)ntiles << 36) | ((uint64_t)nsteps << 4) | ((uint64_t)(fmt & 7) << 1) | (allow_slices ? 1u : 0u);
     std::lock_guard<std::mutex> g(mu);
     auto it = cache.find(key);
     if (it != cache.end()) return it->second;
-    Shape sh = search_shape(ntiles, nsteps, cols_per_step);
+    Shape sh = search_shape(ntiles, nsteps, cols_per_step, bytes_per_col);
     if (!allow_slices) sh.ks = 1;
     cache.emplace(key, sh);
     return sh;
@@ -827,11 +852,11 @@ constexpr uint32_t steps_of(uint32_t n_in) {
 template <int FMT, bool DUMP>
 hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* dump, const DecodeScratch& sc, hipStream_t s) {
     const uint32_t ntiles = row_tiles(w.n_out), nsteps = steps_of<FMT>(w.n_in);
-    Shape sh = shape_for(ntiles, nsteps, true, q8_format(FMT) ? 64 : 128);
+    Shape sh = shape_for(ntiles, nsteps, true, FMT);
     const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
     // slices need scratch: 8 token rows per slice and a counter per row group
     if (sh.ks > 1 && (!sc.partial || !sc.counters || sc.partial_floats < (size_t)sh.ks * 8 * w.n_out || sc.ncounters < groups))
-        sh = shape_for(ntiles, nsteps, false, q8_format(FMT) ? 64 : 128);
+        sh = shape_for(ntiles, nsteps, false, FMT);
     const uint32_t nblk = w.n_in / 32;
     dim3 grid((ntiles + sh.rt - 1) / sh.rt, sh.ks), block(64 * sh.rt * sh.kw);
     size_t c0 = 0;
@@ -905,7 +930,7 @@ uint32_t steps_rt(const WeightView& w) {
 bool decode_batchable(const WeightView& w, size_t t) {
     if (!mfma_decode_format(w.fmt)) return false;
     if (t < 1 || t > 8) return false;
-    const Shape sh = shape_for(row_tiles(w.n_out), steps_rt(w), true, q8_format(w.fmt) ? 64 : 128);  // as a launch of its own: same bits
+    const Shape sh = shape_for(row_tiles(w.n_out), steps_rt(w), true, w.fmt);  // as a launch of its own: same bits
     bool alds;
     const size_t lds = lds_bytes(!q8_format(w.fmt), false, q8_format(w.fmt) ? 2 : 4, steps_rt(w), t <= 4 ? 4 : 8, sh, &alds);
     return alds && lds <= LDS_MAX;
@@ -941,7 +966,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
         {
             auto cls = [](int fmt) { return q8_format(fmt) ? 2 : fmt == FMT_Q6_K ? 1 : 0; };
             auto sliced = [](const WeightView& w) {
-                return shape_for(row_tiles(w.n_out), steps_rt(w), true, q8_format(w.fmt) ? 64 : 128).ks > 1;
+                return shape_for(row_tiles(w.n_out), steps_rt(w), true, w.fmt).ks > 1;
             };
             int last = 0;
             for (uint32_t j = 0; j < a.njobs; j++) last = std::max(last, cls(items[i0 + j].w.fmt));
@@ -956,7 +981,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
         for (uint32_t j = 0; j < a.njobs; j++) {
             const DecodeBatchItem& it = items[i0 + order[j]];
             const uint32_t ntiles = row_tiles(it.w.n_out), nsteps = steps_rt(it.w);
-            const Shape sh = shape_for(ntiles, nsteps, true, q8_format(it.w.fmt) ? 64 : 128);
+            const Shape sh = shape_for(ntiles, nsteps, true, it.w.fmt);
             bool alds;
             const size_t l = lds_bytes(!q8_format(it.w.fmt), false, q8_format(it.w.fmt) ? 2 : 4, nsteps, it.t <= 4 ? 4 : 8, sh, &alds);
             if (!alds || l > LDS_MAX || it.t < 1 || it.t > 8) return hipErrorInvalidValue;
