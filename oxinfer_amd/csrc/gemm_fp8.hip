@@ -33,15 +33,42 @@ __global__ __launch_bounds__(64) void quantize_act_fp8_kernel(const void* __rest
     const uint32_t kb = blockIdx.x % kblocks, mt = blockIdx.x / kblocks;
     const uint32_t tok = mt * 16 + m;
     float v[32];
+    const uint32_t k0 = 128 * kb + 32 * kq;
+    if (tok < t && k0 + 32 <= n_in && n_in % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {  // the lane's 32 columns as whole 16-byte reads
+        if (SRC_BF16) {
+            const uint4* src = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(x) + (size_t)tok * n_in + k0);
 #pragma unroll
-    for (int j = 0; j < 32; j++) {
-        const uint32_t k = 128 * kb + 32 * kq + j;
-        float f = 0.0f;
-        if (tok < t && k < n_in) {
-            if (SRC_BF16) f = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(x)[(size_t)tok * n_in + k]);
-            else f = reinterpret_cast<const float*>(x)[(size_t)tok * n_in + k];
+            for (int q = 0; q < 4; q++) {
+                const uint4 u = src[q];
+                const uint32_t d[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    v[8 * q + 2 * e] = __uint_as_float(d[e] << 16);
+                    v[8 * q + 2 * e + 1] = __uint_as_float(d[e] & 0xFFFF0000u);
+                }
+            }
+        } else {
+            const float4* src = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(x) + (size_t)tok * n_in + k0);
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const float4 f = src[q];
+                v[4 * q] = f.x;
+                v[4 * q + 1] = f.y;
+                v[4 * q + 2] = f.z;
+                v[4 * q + 3] = f.w;
+            }
         }
-        v[j] = f;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 32; j++) {
+            const uint32_t k = k0 + j;
+            float f = 0.0f;
+            if (tok < t && k < n_in) {
+                if (SRC_BF16) f = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(x)[(size_t)tok * n_in + k]);
+                else f = reinterpret_cast<const float*>(x)[(size_t)tok * n_in + k];
+            }
+            v[j] = f;
+        }
     }
     float amax = 0.0f;
 #pragma unroll
@@ -81,7 +108,7 @@ constexpr int F8_NT = 8;   // row tiles per workgroup (128 rows = one scale bloc
 template <bool OUT_BF16>
 __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4* __restrict__ apk, const float* __restrict__ sx,
                                                        uint32_t t, uint32_t mtiles, void* __restrict__ yv) {
-    extern __shared__ uint4 bfrag[];  // [2][8 row tiles][64 lanes][2]
+    extern __shared__ uint4 bfrag[];  // [2][8 row tiles][2 halves][64 lanes]: a lane's two 16-byte halves lie a plane apart (no bank conflicts)
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t n = lane & 15, kq = lane >> 4;
     const uint32_t all_kb = (w.n_in + 127) / 128;
@@ -109,85 +136,117 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
 #pragma unroll
         for (int j = 0; j < F8_NT; j++) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto load_w = [&](uint4 (*r)[2], uint32_t kb) {
-        const size_t col = (size_t)wstep * kb;
+    // Register sets are structs of vector-extension values, indexed only by compile-time constants: HIP's uint4 under
+    // a condition, or a set reached through a pointer, ends up in scratch memory.
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    struct WRegs {
+        u32x4 v[2][2];
+    };
+    struct ARegs {
+        u32x4 v[4][2];
+        f32x4 sx[4];  // the activation scales of the lane's four tokens per tile
+        float sw;     // the weight block's scale
+    };
+    // every request is unconditional and clamped to the last block: a request under a condition makes the compiler
+    // wait for all outstanding ones
+    auto load_w = [&](WRegs& r, uint32_t i_kb) {
+        const size_t col = (size_t)wstep * (kb0 + min(i_kb, nkb - 1));
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            r[i][0] = *reinterpret_cast<const uint4*>(wrow[i] + col);
-            r[i][1] = *reinterpret_cast<const uint4*>(wrow[i] + col + 16);
+            r.v[i][0] = *reinterpret_cast<const u32x4*>(wrow[i] + col);
+            r.v[i][1] = *reinterpret_cast<const u32x4*>(wrow[i] + col + 16);
         }
     };
-    auto store_w = [&](const uint4 (*r)[2], uint32_t buf) {
+    auto store_w = [&](const WRegs& r, uint32_t buf) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            bfrag[((buf * F8_NT + 2 * wave + i) * 64 + lane) * 2] = r[i][0];
-            bfrag[((buf * F8_NT + 2 * wave + i) * 64 + lane) * 2 + 1] = r[i][1];
+            u32x4* dst = reinterpret_cast<u32x4*>(bfrag + (size_t)(buf * F8_NT + 2 * wave + i) * 128 + lane);
+            dst[0] = r.v[i][0];
+            dst[64] = r.v[i][1];
         }
     };
-    auto read_a = [&](uint4 (*dst)[2], uint32_t kb) {
+    auto read_a = [&](ARegs& dst, uint32_t i_kb) {
+        const uint32_t kb = kb0 + min(i_kb, nkb - 1);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            dst[i][0] = abase[i][(size_t)kb * 128];
-            dst[i][1] = abase[i][(size_t)kb * 128 + 1];
+            const u32x4* src = reinterpret_cast<const u32x4*>(abase[i] + (size_t)kb * 128);
+            dst.v[i][0] = src[0];
+            dst.v[i][1] = src[1];
+            dst.sx[i] = *reinterpret_cast<const f32x4*>(sx + (size_t)kb * mtiles * 16 + min(mt0 + i, mtiles - 1) * 16 + 4 * kq);
         }
-    };
-    // per token-tile: s_w * s_x for the 4 tokens this lane's registers hold
-    auto read_f = [&](f32x4* f, uint32_t kb) {
-        const float sw = bs[(size_t)srow * ncb + (128 * kb) / w.bc];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float4 v = *reinterpret_cast<const float4*>(sx + (size_t)kb * mtiles * 16 + min(mt0 + i, mtiles - 1) * 16 + 4 * kq);
-            f[i] = f32x4{v.x * sw, v.y * sw, v.z * sw, v.w * sw};
-        }
+        dst.sw = bs[(size_t)srow * ncb + (128 * kb) / w.bc];
     };
     auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
-    uint4 wr[2][2], a_cur[4][2], a_nxt[4][2];
-    f32x4 f_cur[4], f_nxt[4];
-    load_w(wr, kb0);
-    read_a(a_cur, kb0);
-    read_f(f_cur, kb0);
-    store_w(wr, 0);
-    if (nkb > 1) load_w(wr, kb0 + 1);
+    // Software pipeline, three blocks deep in registers (one wave per SIMD: nothing else hides the latency). At block
+    // i (ring position P = i % 3): the weights of block i + 1 go from registers to the other LDS buffer and their
+    // registers take the request for block i + 4; the matrix instructions run on activation set P and LDS buffer
+    // i & 1; then set P takes the request for block i + 3.
+    WRegs W[3];
+    ARegs A[3];
+    load_w(W[0], 0);
+    read_a(A[0], 0);
+    load_w(W[1], 1);
+    read_a(A[1], 1);
+    load_w(W[2], 2);
+    read_a(A[2], 2);
+    store_w(W[0], 0);
+    load_w(W[0], 3);
     lds_barrier();
-    auto block = [&](uint32_t i_kb, auto more_c) {
-        constexpr bool MORE = decltype(more_c)::value;
-        const uint32_t buf = i_kb & 1, kb = kb0 + i_kb;
-        if (MORE) {
-            read_a(a_nxt, kb + 1);
-            read_f(f_nxt, kb + 1);
-            store_w(wr, buf ^ 1);  // the other buffer was last read two blocks ago, before the previous barrier
-        }
+    auto block = [&](uint32_t i_kb, auto pos) {
+        constexpr int P = decltype(pos)::value, P1 = (P + 1) % 3;
+        const uint32_t buf = i_kb & 1;
+        store_w(W[P1], buf ^ 1);  // the other buffer was last read a block ago, before the previous barrier
+        load_w(W[P1], i_kb + 4);
+        float f[4][4];
 #pragma unroll
-        for (int j = 0; j < F8_NT; j++) {
-            const uint4 b0 = bfrag[((buf * F8_NT + j) * 64 + lane) * 2], b1 = bfrag[((buf * F8_NT + j) * 64 + lane) * 2 + 1];
-            const v8i bb = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+        for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const v8i aa = {(int)a_cur[i][0].x, (int)a_cur[i][0].y, (int)a_cur[i][0].z, (int)a_cur[i][0].w,
-                                (int)a_cur[i][1].x, (int)a_cur[i][1].y, (int)a_cur[i][1].z, (int)a_cur[i][1].w};
+            for (int r = 0; r < 4; r++) f[i][r] = A[P].sx[i][r] * A[P].sw;
+        // the matrix instruction of tile pair k + 1 is issued before the four multiply-adds that take tile pair k's
+        // result into the accumulators: next to each other they would run one after the other
+        f32x4 dprev = {0.0f, 0.0f, 0.0f, 0.0f};
+        u32x4 bq[2][2];  // the row tiles' fragments, read from LDS a tile ahead
+        auto read_b = [&](int j) {
+            const u32x4* bp = reinterpret_cast<const u32x4*>(bfrag + (size_t)(buf * F8_NT + j) * 128 + lane);
+            bq[j & 1][0] = bp[0];
+            bq[j & 1][1] = bp[64];
+        };
+        read_b(0);
+#pragma unroll
+        for (int k = 0; k <= 4 * F8_NT; k++) {
+            const int j = k / 4, i = k % 4;
+            f32x4 d = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (k < 4 * F8_NT) {
+                if (i == 0 && j + 1 < F8_NT) read_b(j + 1);
+                const u32x4 b0 = bq[j & 1][0], b1 = bq[j & 1][1];
+                const v8i bb = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+                const u32x4 a0 = A[P].v[i][0], a1 = A[P].v[i][1];
+                const v8i aa = {(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
                 const f32x4 z = {0.0f, 0.0f, 0.0f, 0.0f};
-                const f32x4 d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aa, bb, z, 0, 0, 0, 127, 0, 127);
-#pragma unroll
-                for (int r = 0; r < 4; r++) acc[i][j][r] = __builtin_fmaf(f_cur[i][r], d[r], acc[i][j][r]);
+                d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aa, bb, z, 0, 0, 0, 127, 0, 127);
             }
-        }
-        if (MORE) {
-            if (i_kb + 2 < nkb) load_w(wr, kb + 2);
-            lds_barrier();
+            if (k > 0) {
+                const int jp = (k - 1) / 4, ip = (k - 1) % 4;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                a_cur[i][0] = a_nxt[i][0];
-                a_cur[i][1] = a_nxt[i][1];
-                f_cur[i] = f_nxt[i];
+                for (int r = 0; r < 4; r++) acc[ip][jp][r] = __builtin_fmaf(f[ip][r], dprev[r], acc[ip][jp][r]);
             }
+            dprev = d;
         }
+        read_a(A[P], i_kb + 3);
+        lds_barrier();
     };
-    using T_ = std::integral_constant<bool, true>;
-    using F_ = std::integral_constant<bool, false>;
+    using P0 = std::integral_constant<int, 0>;
+    using P1_ = std::integral_constant<int, 1>;
+    using P2 = std::integral_constant<int, 2>;
     uint32_t i_kb = 0;
-    for (; i_kb + 1 < nkb; i_kb++) block(i_kb, T_{});
-    block(i_kb, F_{});
+    for (; i_kb + 3 <= nkb; i_kb += 3) {
+        block(i_kb, P0{});
+        block(i_kb + 1, P1_{});
+        block(i_kb + 2, P2{});
+    }
+    if (i_kb < nkb) block(i_kb, P0{});
+    if (i_kb + 1 < nkb) block(i_kb + 1, P1_{});
 
     if (gridDim.z > 1) yv = reinterpret_cast<float*>(yv) + (size_t)blockIdx.z * t * w.n_out;
 #pragma unroll
