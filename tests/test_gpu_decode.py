@@ -326,7 +326,8 @@ def test_decode_batch_shares_a_launch_and_keeps_the_bits(be, oxref):
     import torch
     from oxinfer_amd import synth
     cases = [(Q8_0, 208, 512, 1), (Q4_K, 96, 1024, 8), (Q8_0, 64, 2048, 3), (Q4_K, 176, 512, 2), ("mlx", 80, 640, 5),
-             (Q6_K, 48, 512, 2), (Q4_K, 33, 256, 4), ("mlx", 128, 128, 8)]
+             (Q6_K, 48, 512, 2), (Q4_K, 33, 256, 4), ("mlx", 128, 128, 8),
+             (Q8_0, 48, 14336, 8), (Q4_K, 32, 14336, 1), (Q6_K, 16, 14336, 5)]  # the last three slice K across workgroups
     jobs, alone = [], []
     for i, (kind, n_out, n_in, t) in enumerate(cases):
         if kind == "mlx":
@@ -339,7 +340,7 @@ def test_decode_batch_shares_a_launch_and_keeps_the_bits(be, oxref):
         alone.append(be.decode(w, xa=xa).cpu().numpy())
         y = torch.full((t, n_out), float("nan"), dtype=torch.float32, device="cuda")
         jobs.append((w, xa, None, t, y, None, None))
-    for order in (list(range(len(cases))), list(reversed(range(len(cases)))), [1, 3, 6], [4]):
+    for order in (list(range(len(cases))), list(reversed(range(len(cases)))), [1, 3, 6], [4], [8, 0, 9, 10, 2]):
         for i in order:
             jobs[i][4].fill_(float("nan"))
         be.decode_batch(be.decode_jobs([jobs[i] for i in order]))
