@@ -104,7 +104,7 @@ def fp8_emulation(x, data, scales, oxref):
     return y.astype(np.float32)
 
 
-@pytest.mark.parametrize("n_out,n_in", [(200, 512), (384, 2304)])
+@pytest.mark.parametrize("n_out,n_in", [(200, 512), (384, 2304), (100, 128), (130, 256), (64, 640), (257, 896)])  # 1 to 18 K-blocks: every phase of the kernel's three-deep pipeline
 def test_gemm_fp8_matches_oracle(be, oxref, n_out, n_in):
     import torch
     from oxinfer_amd import synth
