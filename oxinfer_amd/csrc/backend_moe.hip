@@ -91,8 +91,7 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
         if ((v == 8 || v == 16 || v == 32) && t >= 8) max_rows = (uint32_t)v;
     }
     const uint32_t grid_chunks = (uint32_t)((pairs < m->n_exp ? pairs : m->n_exp) + pairs / max_rows + 1);
-    HIP_TRY(launch_moe_plan(route_idx, pairs, k, m->n_exp, max_rows, sc.row_of, sc.src, sc.chunks, sc.nchunks, s), "moe plan launch");
-    HIP_TRY(launch_quantize_act(x, t, h, sc.xa, s), "moe quantize launch");
+    HIP_TRY(launch_moe_front(route_idx, pairs, k, m->n_exp, max_rows, sc.row_of, sc.src, sc.chunks, sc.nchunks, x, t, h, sc.xa, s), "moe plan launch");
     GroupView g{};
     g.chunks = sc.chunks;
     g.nchunks = sc.nchunks;

@@ -132,6 +132,8 @@ hipError_t launch_gemm_fp8(const WeightView& w, const void* apk, const float* sx
 hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, hipStream_t s);
 hipError_t launch_moe_plan(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, uint32_t chunk_rows, int* row_of, int* src,
                            int4* chunks, int* nchunks, hipStream_t s);
+hipError_t launch_moe_front(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, uint32_t chunk_rows, int* row_of, int* src,
+                            int4* chunks, int* nchunks, const float* x, size_t t, size_t h, const oxhip_qact& o, hipStream_t s);
 hipError_t launch_moe_act(const float* g, const float* u, size_t stride, size_t rows, size_t inter, uint32_t kind, float param,
                           float* a, hipStream_t s);
 hipError_t launch_moe_act_quantize(const float* g, const float* u, size_t stride, size_t rows, size_t inter, uint32_t kind, float param,

@@ -2,60 +2,120 @@
 // forward_batched, src/moe.rs:438-617 and :625-828 of the reference; route_top_k, :180-193):
 // routing, the plan that groups (token, expert) pairs by expert, the gated activation with the
 // re-quantization of its output, and the weighted combination in route order.
+#include "act_body.hpp"
 #include "internal.hpp"
 
 namespace oxhip {
 
 // route_top_k: the k largest logits (ties to the lower index, total order on the float bits like
 // f32::total_cmp), weights exp(l - max) / sum over the k. One wavefront per token; n <= 1024, k <= 64.
-__global__ __launch_bounds__(64) void route_top_k_kernel(const float* __restrict__ logits, uint32_t n, uint32_t k,
-                                                         uint32_t* __restrict__ idx, float* __restrict__ wts) {
-    const uint32_t tok = blockIdx.x, lane = threadIdx.x;
+//
+// PER: logits per lane (n <= 64 PER). Up to 256 experts an element's place in the sorted order is counted directly
+// (how many elements beat it: every element is broadcast from its lane in turn, n * PER compares per lane, no
+// dependent lane-to-lane round trips); beyond that k rounds of a wave-wide argmax cost less.
+__device__ __forceinline__ int order_key(float v) {
+    const int b = __float_as_int(v);
+    return b ^ (int)(((uint32_t)(b >> 31)) >> 1);  // f32::total_cmp's order as a signed compare; its own inverse
+}
+
+// NW waves per token. A lone wave issues an instruction every five to eight cycles, so the counting loop is split
+// over the waves (each broadcasts 64 / NW lanes of every register) and the counts meet in LDS; wave 0 finishes.
+template <int PER, int NW>
+__global__ __launch_bounds__(64 * NW) void route_top_k_kernel(const float* __restrict__ logits, uint32_t n, uint32_t k,
+                                                              uint32_t* __restrict__ idx, float* __restrict__ wts) {
+    const uint32_t tok = blockIdx.x, lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const float* l = logits + (size_t)tok * n;
-    constexpr int PER = 16;  // logits per lane
     int key[PER];
     bool live[PER];
 #pragma unroll
     for (int i = 0; i < PER; i++) {
         const uint32_t j = lane + 64 * i;
         live[i] = j < n;
-        const int b = live[i] ? __float_as_int(l[j]) : 0;
-        key[i] = b ^ (int)(((uint32_t)(b >> 31)) >> 1);  // f32::total_cmp's order as a signed compare
+        key[i] = order_key(live[i] ? l[j] : 0.0f);
     }
-    // round r's winner stays in lane r (a per-thread array indexed by r would turn into long select chains)
+    // round r's winner ends up in lane r
     float mysel = 0.0f;
     uint32_t myidx = 0;
-    for (uint32_t r = 0; r < k && r < 64; r++) {
-        // this lane's best remaining logit (its indices ascend, so ties keep the lower one)
-        int bk = 0;
-        uint32_t bj = 0xFFFFFFFFu;
+    if constexpr (PER <= 4) {
+        __shared__ uint32_t rank_s[PER * 64];
+        __shared__ int sel_key[64];
+        __shared__ uint32_t sel_idx[64];
+        if (NW > 1) {
+            for (uint32_t i = threadIdx.x; i < PER * 64; i += 64 * NW) rank_s[i] = 0;
+            __syncthreads();
+        }
+        uint32_t rank[PER];
 #pragma unroll
-        for (int i = 0; i < PER; i++)
-            if (live[i] && (bj == 0xFFFFFFFFu || key[i] > bk)) {
-                bk = key[i];
-                bj = lane + 64 * i;
-            }
-        for (int off = 32; off >= 1; off >>= 1) {
-            const int ok = __shfl_xor(bk, off);
-            const uint32_t oj = __shfl_xor(bj, off);
-            if (oj != 0xFFFFFFFFu && (bj == 0xFFFFFFFFu || ok > bk || (ok == bk && oj < bj))) {
-                bk = ok;
-                bj = oj;
+        for (int i = 0; i < PER; i++) rank[i] = 0;
+        // element j = src + 64 i2 beats element (lane, i) when its key is larger, or equal with a lower index
+        constexpr uint32_t SPAN = 64 / NW;
+#pragma unroll
+        for (int i2 = 0; i2 < PER; i2++) {
+            const uint32_t cnt = min(64u, n > 64u * i2 ? n - 64u * i2 : 0u);  // live lanes of register i2 (uniform)
+            const uint32_t s1 = min(cnt, (wave + 1) * SPAN);
+            for (uint32_t src = wave * SPAN; src < s1; src++) {
+                const int ok = __builtin_amdgcn_readlane(key[i2], (int)src);
+#pragma unroll
+                for (int i = 0; i < PER; i++) {
+                    const bool lower = i2 < i || (i2 == i && src < lane);
+                    rank[i] += (ok > key[i] || (ok == key[i] && lower)) ? 1u : 0u;
+                }
             }
         }
-        if (lane == r) {
-            myidx = bj;
-            mysel = __int_as_float(bk ^ (int)(((uint32_t)(bk >> 31)) >> 1));  // the key's transform is its own inverse
+        if (NW > 1) {
+#pragma unroll
+            for (int i = 0; i < PER; i++)
+                if (rank[i]) atomicAdd(&rank_s[64 * i + lane], rank[i]);
+            __syncthreads();
+            if (wave) return;
+#pragma unroll
+            for (int i = 0; i < PER; i++) rank[i] = rank_s[64 * i + lane];
         }
 #pragma unroll
         for (int i = 0; i < PER; i++)
-            if (lane + 64 * i == bj) live[i] = false;
+            if (live[i] && rank[i] < k && rank[i] < 64) {
+                sel_key[rank[i]] = key[i];
+                sel_idx[rank[i]] = lane + 64 * i;
+            }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): wave 0's LDS writes before its reads below
+        __builtin_amdgcn_wave_barrier();
+        if (lane < k && lane < n) {
+            mysel = __int_as_float(order_key(__int_as_float(sel_key[lane])));
+            myidx = sel_idx[lane];
+        }
+    } else {
+        for (uint32_t r = 0; r < k && r < 64; r++) {
+            // this lane's best remaining logit (its indices ascend, so ties keep the lower one)
+            int bk = 0;
+            uint32_t bj = 0xFFFFFFFFu;
+#pragma unroll
+            for (int i = 0; i < PER; i++)
+                if (live[i] && (bj == 0xFFFFFFFFu || key[i] > bk)) {
+                    bk = key[i];
+                    bj = lane + 64 * i;
+                }
+            for (int off = 32; off >= 1; off >>= 1) {
+                const int ok = __shfl_xor(bk, off);
+                const uint32_t oj = __shfl_xor(bj, off);
+                if (oj != 0xFFFFFFFFu && (bj == 0xFFFFFFFFu || ok > bk || (ok == bk && oj < bj))) {
+                    bk = ok;
+                    bj = oj;
+                }
+            }
+            if (lane == r) {
+                myidx = bj;
+                mysel = __int_as_float(order_key(__int_as_float(bk)));
+            }
+#pragma unroll
+            for (int i = 0; i < PER; i++)
+                if (lane + 64 * i == bj) live[i] = false;
+        }
     }
     // weights: exp(l - max) over the k, summed in rank order from -0.0 as the reference does
-    const float m = __shfl(mysel, 0);
+    const float m = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(mysel)));
     const float e = lane < k ? expf(mysel - m) : 0.0f;
     float sum = -0.0f;
-    for (uint32_t r = 0; r < k && r < 64; r++) sum += __shfl(e, (int)r);
+    for (uint32_t r = 0; r < k && r < 64; r++) sum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), (int)r));
     if (lane < k) {
         idx[(size_t)tok * k + lane] = myidx;
         wts[(size_t)tok * k + lane] = e / sum;
@@ -64,7 +124,9 @@ __global__ __launch_bounds__(64) void route_top_k_kernel(const float* __restrict
 
 hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, hipStream_t s) {
     if (!t) return hipSuccess;
-    route_top_k_kernel<<<(unsigned)t, 64, 0, s>>>(logits, (uint32_t)n, (uint32_t)k, idx, w);
+    if (n <= 128) route_top_k_kernel<2, 8><<<(unsigned)t, 512, 0, s>>>(logits, (uint32_t)n, (uint32_t)k, idx, w);
+    else if (n <= 256) route_top_k_kernel<4, 8><<<(unsigned)t, 512, 0, s>>>(logits, (uint32_t)n, (uint32_t)k, idx, w);
+    else route_top_k_kernel<16, 1><<<(unsigned)t, 64, 0, s>>>(logits, (uint32_t)n, (uint32_t)k, idx, w);
     return hipGetLastError();
 }
 
@@ -75,10 +137,9 @@ hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k,
 //   src[row]           token of a gathered row
 //   chunks[c]          {expert, first row, rows, 0}; *nchunks
 constexpr uint32_t PLAN_LDS_PAIRS = 24 * 1024;  // route entries kept in LDS (96 KiB); longer lists are read from L2
-__global__ __launch_bounds__(1024) void moe_plan_kernel(const uint32_t* __restrict__ route_idx, uint32_t pairs, uint32_t k,
-                                                        uint32_t n_exp, int cr, int* __restrict__ row_of, int* __restrict__ src,
-                                                        int4* __restrict__ chunks, int* __restrict__ nchunks) {
-    extern __shared__ int sh[];
+__device__ __forceinline__ void moe_plan_body(int* sh, const uint32_t* __restrict__ route_idx, uint32_t pairs, uint32_t k, uint32_t n_exp, int cr,
+                                              int* __restrict__ row_of, int* __restrict__ src, int4* __restrict__ chunks,
+                                              int* __restrict__ nchunks) {
     int* cnt = sh;                 // [n_exp]
     int* start = sh + n_exp;       // [n_exp]
     int* cstart = sh + 2 * n_exp;  // [n_exp]
@@ -133,6 +194,29 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const uint32_t* __restri
     }
 }
 
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const uint32_t* __restrict__ route_idx, uint32_t pairs, uint32_t k,
+                                                        uint32_t n_exp, int cr, int* __restrict__ row_of, int* __restrict__ src,
+                                                        int4* __restrict__ chunks, int* __restrict__ nchunks) {
+    extern __shared__ int sh[];
+    moe_plan_body(sh, route_idx, pairs, k, n_exp, cr, row_of, src, chunks, nchunks);
+}
+
+// The plan and the quantization of the layer's input depend only on the layer's arguments, and each is a few
+// microseconds of latency: one launch runs both (workgroup 0 plans, the others quantize one block of 32 per lane).
+__global__ __launch_bounds__(1024) void moe_front_kernel(const uint32_t* __restrict__ route_idx, uint32_t pairs, uint32_t k, uint32_t n_exp,
+                                                         int cr, int* __restrict__ row_of, int* __restrict__ src, int4* __restrict__ chunks,
+                                                         int* __restrict__ nchunks, const float* __restrict__ x, size_t nblocks,
+                                                         int8_t* __restrict__ q, float* __restrict__ scales, int32_t* __restrict__ sums,
+                                                         float* __restrict__ fsums, float* __restrict__ hsums, int32_t* __restrict__ sums16) {
+    extern __shared__ int sh[];
+    if (blockIdx.x == 0) {
+        moe_plan_body(sh, route_idx, pairs, k, n_exp, cr, row_of, src, chunks, nchunks);
+        return;
+    }
+    const size_t b = (size_t)(blockIdx.x - 1) * blockDim.x + threadIdx.x;
+    if (b < nblocks) quantize_act_block(x, b, q, scales, sums, fsums, hsums, sums16);
+}
+
 hipError_t launch_moe_plan(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, uint32_t chunk_rows, int* row_of, int* src,
                            int4* chunks, int* nchunks, hipStream_t s) {
     const size_t lds = 4 * n_exp * sizeof(int) + (pairs <= PLAN_LDS_PAIRS ? pairs * sizeof(uint32_t) : 0);
@@ -141,6 +225,21 @@ hipError_t launch_moe_plan(const uint32_t* route_idx, size_t pairs, size_t k, si
         if (e != hipSuccess) return e;
     }
     moe_plan_kernel<<<1, 1024, lds, s>>>(route_idx, (uint32_t)pairs, (uint32_t)k, (uint32_t)n_exp, (int)chunk_rows, row_of, src, chunks, nchunks);
+    return hipGetLastError();
+}
+
+// Plan + quantize_act(x [t][h]) in one launch when the plan's LDS is small (it is allocated to every workgroup);
+// else two launches.
+hipError_t launch_moe_front(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, uint32_t chunk_rows, int* row_of, int* src,
+                            int4* chunks, int* nchunks, const float* x, size_t t, size_t h, const oxhip_qact& o, hipStream_t s) {
+    const size_t lds = 4 * n_exp * sizeof(int) + pairs * sizeof(uint32_t), nblocks = t * h / 32;
+    if (pairs > 4096 || lds > 32 * 1024 || !nblocks) {
+        hipError_t e = launch_moe_plan(route_idx, pairs, k, n_exp, chunk_rows, row_of, src, chunks, nchunks, s);
+        return e != hipSuccess ? e : launch_quantize_act(x, t, h, o, s);
+    }
+    moe_front_kernel<<<1 + (unsigned)((nblocks + 1023) / 1024), 1024, lds, s>>>(route_idx, (uint32_t)pairs, (uint32_t)k, (uint32_t)n_exp,
+                                                                              (int)chunk_rows, row_of, src, chunks, nchunks, x, nblocks, o.q, o.scales,
+                                                                              o.sums, o.fsums, o.hsums, o.sums16);
     return hipGetLastError();
 }
 
@@ -186,39 +285,55 @@ hipError_t launch_moe_act(const float* g, const float* u, size_t stride, size_t 
     return hipGetLastError();
 }
 
-// The same, followed by quantize_act on the result (src/quant.rs:267-292) without the round trip through memory: one
-// lane per block of 32 of a; bit-identical to moe_act_kernel + quantize_act_kernel. `a` (optional) also keeps the
-// f32 values.
-__global__ __launch_bounds__(64) void moe_act_quantize_kernel(const float* __restrict__ gp, const float* __restrict__ up, size_t stride,
-                                                             size_t rows, uint32_t inter, uint32_t kind, float param,
-                                                             int8_t* __restrict__ q, float* __restrict__ scales, int32_t* __restrict__ sums,
-                                                             float* __restrict__ fsums, float* __restrict__ hsums,
-                                                             int32_t* __restrict__ sums16) {
-    const size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x, bpr = inter / 32;
-    if (b >= rows * bpr) return;
-    const size_t r = b / bpr, j0 = (b % bpr) * 32;
-    const float4* g4 = reinterpret_cast<const float4*>(gp + r * stride + j0);
-    const float4* u4 = reinterpret_cast<const float4*>(up + r * stride + j0);
+// The same, followed by quantize_act on the result (src/quant.rs:267-292) without the round trip through memory;
+// bit-identical to moe_act_kernel + quantize_act_kernel. A workgroup of 256 threads takes 32 blocks of 32: eight
+// neighbouring lanes read one block's gate and up values as whole lines and apply the activation (four values each);
+// the values meet in LDS and one lane per block forms the sums in the reference's order and the int8 codes.
+__global__ __launch_bounds__(256) void moe_act_quantize_kernel(const float* __restrict__ gp, const float* __restrict__ up, size_t stride,
+                                                              size_t rows, uint32_t inter, uint32_t kind, float param,
+                                                              int8_t* __restrict__ q, float* __restrict__ scales, int32_t* __restrict__ sums,
+                                                              float* __restrict__ fsums, float* __restrict__ hsums,
+                                                              int32_t* __restrict__ sums16) {
+    __shared__ float vals[32][36];  // rows padded: the finishing lanes read their blocks 36 words apart
+    const size_t bpr = inter / 32, nblocks = rows * bpr;
+    const size_t b0 = (size_t)blockIdx.x * 32;
+    {
+        const uint32_t lb = threadIdx.x >> 3, part = threadIdx.x & 7;
+        const size_t b = b0 + lb;
+        if (b < nblocks) {
+            const size_t r = b / bpr, j0 = (b % bpr) * 32 + 4 * part;
+            const float4 gg = *reinterpret_cast<const float4*>(gp + r * stride + j0);
+            const float4 uu = *reinterpret_cast<const float4*>(up + r * stride + j0);
+            const float gs[4] = {gg.x, gg.y, gg.z, gg.w}, us[4] = {uu.x, uu.y, uu.z, uu.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float g = gs[e], u = us[e], v;
+                if (kind == 1) {
+                    const float K2 = 2.0f * 0.7978846f;
+                    const float t = K2 * (g + 0.044715f * g * g * g);
+                    v = g / (1.0f + fast_exp(-t)) * u;
+                } else {
+                    if (kind == 2) {
+                        g = fminf(g, param);
+                        u = fminf(fmaxf(u, -param), param);
+                    }
+                    v = g / (1.0f + fast_exp(-g)) * u;
+                }
+                vals[lb][4 * part + e] = v;
+            }
+        }
+    }
+    __syncthreads();
+    const size_t b = b0 + threadIdx.x;
+    if (threadIdx.x >= 32 || b >= nblocks) return;
     float v[32];
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        const float4 gg = g4[i], uu = u4[i];
-        const float gs[4] = {gg.x, gg.y, gg.z, gg.w}, us[4] = {uu.x, uu.y, uu.z, uu.w};
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            float g = gs[e], u = us[e];
-            if (kind == 1) {
-                const float K2 = 2.0f * 0.7978846f;
-                const float t = K2 * (g + 0.044715f * g * g * g);
-                v[4 * i + e] = g / (1.0f + fast_exp(-t)) * u;
-            } else {
-                if (kind == 2) {
-                    g = fminf(g, param);
-                    u = fminf(fmaxf(u, -param), param);
-                }
-                v[4 * i + e] = g / (1.0f + fast_exp(-g)) * u;
-            }
-        }
+        const float4 f = *reinterpret_cast<const float4*>(&vals[threadIdx.x][4 * i]);
+        v[4 * i] = f.x;
+        v[4 * i + 1] = f.y;
+        v[4 * i + 2] = f.z;
+        v[4 * i + 3] = f.w;
     }
     float amax = 0.0f;
 #pragma unroll
@@ -261,7 +376,7 @@ hipError_t launch_moe_act_quantize(const float* g, const float* u, size_t stride
                                    const oxhip_qact& o, hipStream_t s) {
     const size_t blocks = rows * (inter / 32);
     if (!blocks) return hipSuccess;
-    moe_act_quantize_kernel<<<(unsigned)((blocks + 63) / 64), 64, 0, s>>>(g, u, stride, rows, (uint32_t)inter, kind, param, o.q, o.scales, o.sums,
+    moe_act_quantize_kernel<<<(unsigned)((blocks + 31) / 32), 256, 0, s>>>(g, u, stride, rows, (uint32_t)inter, kind, param, o.q, o.scales, o.sums,
                                                                         o.fsums, o.hsums, o.sums16);
     return hipGetLastError();
 }
