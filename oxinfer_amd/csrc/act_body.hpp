@@ -56,4 +56,39 @@ __device__ __forceinline__ void quantize_act_block(const float* __restrict__ x, 
     sums16[2 * b + 1] = s1;
 }
 
+// fast_exp of the reference (src/kernels.rs:2225-2231): clamp, Cody-Waite reduction, degree-6 polynomial,
+// scale by 2^fx through the exponent bits; every operation unfused as written there.
+__device__ __forceinline__ float fast_exp(float x) {
+    x = fminf(fmaxf(x, -87.0f), 88.0f);
+    const float fx = roundf(x * 1.44269504088896340736f);
+    const float r = (x - fx * 0.693359375f) - fx * -2.12194440e-4f;
+    const float p = 1.0f + r * (1.0f + r * (0.5f + r * (0.16666667f + r * (0.041666668f + r * (0.008333334f + r * 0.0013888889f)))));
+    return __int_as_float(((int)fx + 127) << 23) * p;
+}
+
+// Act::apply of one pair (src/moe.rs:18-37, silu_mul / gelu_mul): kind 0 SiLU, 1 GELU-tanh, 2 SiLU with clamp `param`.
+__device__ __forceinline__ float gated_act(float g, float u, uint32_t kind, float param) {
+    if (kind == 1) {
+        const float K2 = 2.0f * 0.7978846f;
+        const float t = K2 * (g + 0.044715f * g * g * g);
+        return g / (1.0f + fast_exp(-t)) * u;
+    }
+    if (kind == 2) {
+        g = fminf(g, param);
+        u = fminf(fmaxf(u, -param), param);
+    }
+    return g / (1.0f + fast_exp(-g)) * u;
+}
+
+// Act::scalar (src/moe.rs:39-46), what the reference's grouped prefill path applies: the exponential of the SiLU
+// kinds is the library's, not fast_exp (GELU-tanh goes through fast_exp in both, src/kernels.rs:2235-2239).
+__device__ __forceinline__ float gated_act_scalar(float g, float u, uint32_t kind, float param) {
+    if (kind == 1) return gated_act(g, u, kind, param);
+    if (kind == 2) {
+        g = fminf(g, param);
+        u = fminf(fmaxf(u, -param), param);
+    }
+    return g / (1.0f + expf(-g)) * u;
+}
+
 }  // namespace oxhip

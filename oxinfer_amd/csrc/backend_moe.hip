@@ -37,6 +37,8 @@ struct Scratch {
     float* a;       // [pairs][inter]
     oxhip_qact aq;  // a quantized
     float* o;       // [pairs][h]
+    void* fx;       // bf16 fragments of the chunks' rows of x, and of a (the prefill form: chunks of up to 16 rows)
+    void* fa;
     uint32_t max_chunks;
     size_t bytes;
 };
@@ -60,6 +62,10 @@ Scratch carve(uint8_t* base, size_t t, size_t pairs, size_t n_exp, size_t h, siz
     s.a = reinterpret_cast<float*>(take(pairs * inter * 4));
     s.aq = carve_qact(take(qact_bytes(pairs, inter)), pairs, inter);
     s.o = reinterpret_cast<float*>(take(pairs * h * 4));
+    const size_t chunks16 = (pairs < n_exp ? pairs : n_exp) + pairs / 16 + 1;
+    const bool prefill = pairs / n_exp >= 6 && h % 128 == 0 && inter % 128 == 0;
+    s.fx = take(prefill ? moe_bf16_frag_bytes(chunks16, h) : 0);
+    s.fa = take(prefill ? moe_bf16_frag_bytes(chunks16, inter) : 0);
     s.bytes = off;
     return s;
 }
@@ -90,34 +96,50 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
         const int v = atoi(e);
         if ((v == 8 || v == 16 || v == 32) && t >= 8) max_rows = (uint32_t)v;
     }
+    // Prefill passes over MLX 4-bit experts (six or more routed rows per expert on average) take the bf16 form: see
+    // moe_bf16.hip. OXHIP_MOE_INT8=1 keeps the integer path (the 1e-3 accuracy class) at any size.
+    const bool fused = m->up.empty();
+    const char* keep_int = getenv("OXHIP_MOE_INT8");
+    const bool bf16_form = avg >= 6 && fused && moe_bf16_ok(m->gate_up[0]->v) && moe_bf16_ok(m->down[0]->v) && !(keep_int && keep_int[0] == '1');
+    if (bf16_form) max_rows = 16;
     const uint32_t grid_chunks = (uint32_t)((pairs < m->n_exp ? pairs : m->n_exp) + pairs / max_rows + 1);
-    HIP_TRY(launch_moe_front(route_idx, pairs, k, m->n_exp, max_rows, sc.row_of, sc.src, sc.chunks, sc.nchunks, x, t, h, sc.xa, s), "moe plan launch");
     GroupView g{};
     g.chunks = sc.chunks;
     g.nchunks = sc.nchunks;
-    // gate / up over the routed rows of x (row i of the gathered order is token src[i])
-    g.rowmap = sc.src;
-    g.bases = m->bases_gu;
-    const bool fused = m->up.empty();
-    HIP_TRY(launch_decode_mfma_grouped(m->gate_up[0]->v, view_of(sc.xa), g, grid_chunks, max_rows, sc.gu, s), "moe gate launch");
-    const float* up_out = sc.gu + inter;
-    size_t stride = 2 * inter;
-    if (!fused) {
-        g.bases = m->bases_up;
-        float* u = sc.gu + pairs * inter;
-        HIP_TRY(launch_decode_mfma_grouped(m->up[0]->v, view_of(sc.xa), g, grid_chunks, max_rows, u, s), "moe up launch");
-        up_out = u;
-        stride = inter;
-    }
-    if (inter % 32 == 0 && stride % 4 == 0) {
-        HIP_TRY(launch_moe_act_quantize(sc.gu, up_out, stride, pairs, inter, m->act_kind, m->act_param, sc.aq, s), "moe act launch");
+    if (bf16_form) {
+        HIP_TRY(launch_moe_plan(route_idx, pairs, k, m->n_exp, max_rows, sc.row_of, sc.src, sc.chunks, sc.nchunks, s), "moe plan launch");
+        HIP_TRY(launch_moe_pack_bf16(x, h, sc.src, sc.chunks, sc.nchunks, grid_chunks, sc.fx, s), "moe pack launch");
+        g.bases = m->bases_gu;
+        HIP_TRY(launch_moe_bf16(m->gate_up[0]->v, g, grid_chunks, sc.fx, sc.gu, s), "moe gate launch");
+        HIP_TRY(launch_moe_act_pack_bf16(sc.gu, sc.gu + inter, 2 * inter, inter, m->act_kind, m->act_param, sc.chunks, sc.nchunks, grid_chunks, sc.fa, s),
+                "moe act launch");
+        g.bases = m->bases_dn;
+        HIP_TRY(launch_moe_bf16(m->down[0]->v, g, grid_chunks, sc.fa, sc.o, s), "moe down launch");
     } else {
-        HIP_TRY(launch_moe_act(sc.gu, up_out, stride, pairs, inter, m->act_kind, m->act_param, sc.a, s), "moe act launch");
-        HIP_TRY(launch_quantize_act(sc.a, pairs, inter, sc.aq, s), "moe quantize launch");
+        HIP_TRY(launch_moe_front(route_idx, pairs, k, m->n_exp, max_rows, sc.row_of, sc.src, sc.chunks, sc.nchunks, x, t, h, sc.xa, s), "moe plan launch");
+        // gate / up over the routed rows of x (row i of the gathered order is token src[i])
+        g.rowmap = sc.src;
+        g.bases = m->bases_gu;
+        HIP_TRY(launch_decode_mfma_grouped(m->gate_up[0]->v, view_of(sc.xa), g, grid_chunks, max_rows, sc.gu, s), "moe gate launch");
+        const float* up_out = sc.gu + inter;
+        size_t stride = 2 * inter;
+        if (!fused) {
+            g.bases = m->bases_up;
+            float* u = sc.gu + pairs * inter;
+            HIP_TRY(launch_decode_mfma_grouped(m->up[0]->v, view_of(sc.xa), g, grid_chunks, max_rows, u, s), "moe up launch");
+            up_out = u;
+            stride = inter;
+        }
+        if (inter % 32 == 0 && stride % 4 == 0) {
+            HIP_TRY(launch_moe_act_quantize(sc.gu, up_out, stride, pairs, inter, m->act_kind, m->act_param, sc.aq, s), "moe act launch");
+        } else {
+            HIP_TRY(launch_moe_act(sc.gu, up_out, stride, pairs, inter, m->act_kind, m->act_param, sc.a, s), "moe act launch");
+            HIP_TRY(launch_quantize_act(sc.a, pairs, inter, sc.aq, s), "moe quantize launch");
+        }
+        g.rowmap = nullptr;
+        g.bases = m->bases_dn;
+        HIP_TRY(launch_decode_mfma_grouped(m->down[0]->v, view_of(sc.aq), g, grid_chunks, max_rows, sc.o, s), "moe down launch");
     }
-    g.rowmap = nullptr;
-    g.bases = m->bases_dn;
-    HIP_TRY(launch_decode_mfma_grouped(m->down[0]->v, view_of(sc.aq), g, grid_chunks, max_rows, sc.o, s), "moe down launch");
     HIP_TRY(launch_moe_combine(sc.o, sc.row_of, route_w, t, k, h, y, s), "moe combine launch");
     return 1;
 }

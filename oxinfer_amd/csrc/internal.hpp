@@ -140,6 +140,14 @@ hipError_t launch_moe_act_quantize(const float* g, const float* u, size_t stride
                                    const oxhip_qact& o, hipStream_t s);
 hipError_t launch_moe_combine(const float* o, const int* row_of, const float* route_w, size_t t, size_t k, size_t h, float* y,
                               hipStream_t s);
+// The bf16 form of the grouped expert matmuls for prefill passes (moe_bf16.hip): MLX 4-bit weights, chunks of <= 16 rows.
+bool moe_bf16_ok(const WeightView& w);
+size_t moe_bf16_frag_bytes(size_t max_chunks, size_t n_in);
+hipError_t launch_moe_pack_bf16(const float* x, size_t n_in, const int* rowmap, const int4* chunks, const int* nchunks, uint32_t max_chunks,
+                                void* frag, hipStream_t s);
+hipError_t launch_moe_act_pack_bf16(const float* g, const float* u, size_t stride, size_t inter, uint32_t kind, float param, const int4* chunks,
+                                    const int* nchunks, uint32_t max_chunks, void* frag, hipStream_t s);
+hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max_chunks, const void* frag, float* out, hipStream_t s);
 
 void set_error(const std::string& msg);
 

@@ -243,16 +243,6 @@ hipError_t launch_moe_front(const uint32_t* route_idx, size_t pairs, size_t k, s
     return hipGetLastError();
 }
 
-// fast_exp of the reference (src/kernels.rs:2225-2231): clamp, Cody-Waite reduction, degree-6 polynomial,
-// scale by 2^fx through the exponent bits; every operation unfused as written there.
-__device__ __forceinline__ float fast_exp(float x) {
-    x = fminf(fmaxf(x, -87.0f), 88.0f);
-    const float fx = roundf(x * 1.44269504088896340736f);
-    const float r = (x - fx * 0.693359375f) - fx * -2.12194440e-4f;
-    const float p = 1.0f + r * (1.0f + r * (0.5f + r * (0.16666667f + r * (0.041666668f + r * (0.008333334f + r * 0.0013888889f)))));
-    return __int_as_float(((int)fx + 127) << 23) * p;
-}
-
 // Act::apply on gathered rows: a = act(g) * u as f32 [rows][inter], with g and u rows `stride` apart (fused
 // gate/up outputs: g = gu, u = gu + inter, stride 2 * inter). kind: 0 SiLU, 1 GELU-tanh, 2 SiLU with clamp
 // `param` (src/moe.rs:18-37, silu_mul / gelu_mul).

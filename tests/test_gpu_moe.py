@@ -93,23 +93,44 @@ def test_moe_mlx_matches_oracle(be, oxref, mlx_experts):
     k = 3
     dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)
     assert dev is not None, be.last_error()
+    import os
     for t in (1, 2, 5, 7, 8, 19, 40):
         x = synth.activations(t, h, 300 + t)
         _, idx, w = make_routes(oxref, t, ne, k, 400 + t)
         y0 = synth.activations(t, h, 500 + t)  # the call adds into y
-        y = y0.copy()
-        assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
         ref = moe_reference(oxref, "mlx", q_gu, q_dn, h, inter, x, idx, w, y0)
-        assert row_err(y - y0, ref - y0) < 1e-3, t
         # the oracle's own MoE driver agrees with the composition above (decode path)
         ref2 = oxref.moe_q4(q_gu, q_dn, 64, h, inter, x, t, idx, w, y0, decode_path=True)
         assert np.array_equal(ref2.view(np.uint32), ref.view(np.uint32))
-        if t >= 8:
-            # from 8 tokens on the CPU takes its grouped f32 path (exact activations, libm exp): the int8
-            # activations of the decode kernels stay within the reference's own bound for them against the
-            # exact product (3e-2, src/ggml.rs:1904)
-            ref3 = oxref.moe_q4(q_gu, q_dn, 64, h, inter, x, t, idx, w, y0, decode_path=False)
+        # from 8 tokens on the CPU takes its grouped f32 path (exact activations, Act::scalar)
+        ref3 = oxref.moe_q4(q_gu, q_dn, 64, h, inter, x, t, idx, w, y0, decode_path=False) if t >= 8 else None
+        # the integer path (int8 activations, the decode kernels' semantics) at every size
+        os.environ["OXHIP_MOE_INT8"] = "1"
+        try:
+            y = y0.copy()
+            assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
+        finally:
+            del os.environ["OXHIP_MOE_INT8"]
+        assert row_err(y - y0, ref - y0) < 1e-3, t
+        if ref3 is not None:
+            # int8 activations against the exact product: within the reference's own bound for them (3e-2, src/ggml.rs:1904)
             assert row_err(y - y0, ref3 - y0) < 3e-2, t
+        # the library's own choice: with six or more routed rows per expert the bf16 form of the grouped matmuls, which
+        # is the grouped f32 path up to the bf16 rounding of x and of the activation's output (2^-9 per element, which
+        # these short rows of 256 and 128 barely average; the bar for the bf16 matrix cores is 2e-2)
+        y = y0.copy()
+        assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
+        if (t * k) // ne >= 6:
+            assert row_err(y - y0, ref3 - y0) < 1e-2, t
+            # with activations that are bf16 values already (the prefill workload's) only the intermediate is rounded
+            import torch
+            xb = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+            refb = oxref.moe_q4(q_gu, q_dn, 64, h, inter, xb, t, idx, w, y0, decode_path=False)
+            yb = y0.copy()
+            assert be.moe(xb, t, h, inter, idx, w, k, dev, yb), be.last_error()
+            assert row_err(yb - y0, refb - y0) < 4e-3, t
+        else:
+            assert row_err(y - y0, ref - y0) < 1e-3, t
 
 
 def test_moe_batched_equals_one_at_a_time(be, oxref, mlx_experts):
