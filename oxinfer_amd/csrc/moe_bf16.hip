@@ -15,6 +15,9 @@
 #include "internal.hpp"
 #include "layout.hpp"
 
+#include <cstdio>
+#include <cstdlib>
+
 namespace oxhip {
 
 namespace {
@@ -61,12 +64,13 @@ __global__ __launch_bounds__(256) void moe_pack_bf16_kernel(const float* __restr
 
 // Workgroup: 8 waves = 8 / kw groups of RT row tiles x kw waves that split the K steps (wave v takes steps v, v + kw, ...)
 // and meet in LDS in wave order. grid x: runs of (8 / kw) RT row tiles; grid y: chunks {expert, first row, rows <= 16}.
-// out [gathered row][n_out] f32.
+// The chunk's fragments (4 KiB per step) are staged into LDS once per workgroup: all eight waves multiply the same
+// rows (each wave asking memory for them costs more than the weights). out [gathered row][n_out] f32.
 template <int RT>
-__global__ __launch_bounds__(512) void moe_bf16_kernel(WeightView w, const uint8_t* const* __restrict__ bases, const int4* __restrict__ chunks,
-                                                       const int* __restrict__ nchunks, const uint4* __restrict__ afrag, uint32_t kw,
-                                                       float* __restrict__ out) {
-    extern __shared__ __align__(16) float red[];  // [wave][RT][64][4]
+__global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const uint8_t* const* __restrict__ bases, const int4* __restrict__ chunks,
+                                                          const int* __restrict__ nchunks, const uint4* __restrict__ afrag, uint32_t kw,
+                                                          float* __restrict__ out) {
+    extern __shared__ __align__(16) float lds[];  // fragments [step][4][64] x 16 B; then the waves' sums [wave][RT][64][4]
     const uint32_t c = blockIdx.y;
     if (c >= (uint32_t)*nchunks) return;  // uniform over the workgroup
     const int4 ch = chunks[c];
@@ -80,13 +84,11 @@ __global__ __launch_bounds__(512) void moe_bf16_kernel(WeightView w, const uint8
     const uint8_t* wp[RT];
 #pragma unroll
     for (int r = 0; r < RT; r++) wp[r] = base + (size_t)min(tile0 + r, ntiles - 1) * t4m_steps(w.n_in) * T4M_REC;
-    const u32x4* ap = reinterpret_cast<const u32x4*>(afrag) + (size_t)c * nsteps * 4 * 64 + lane;
     const uint32_t cnt = (nsteps - kwave + kw - 1) / kw, ilast = cnt - 1;  // kw <= nsteps
 
     struct St {
         u32x4 w[RT];
         uint32_t d[RT], o[RT];
-        u32x4 a[4];
     };
     // every request is unconditional (past the end the last step again): the compiler then knows how many are in flight
     auto load = [&](St& st, uint32_t i) {
@@ -98,22 +100,46 @@ __global__ __launch_bounds__(512) void moe_bf16_kernel(WeightView w, const uint8
             st.d[r] = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
             st.o[r] = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
         }
-#pragma unroll
-        for (int b = 0; b < 4; b++) st.a[b] = ap[((size_t)s * 4 + b) * 64];
     };
+    // the fragments first (L2 hits, needed by every step), then the first weight records, then the fragments go to LDS
+    // while the weights are still on their way
+    const u32x4* src = reinterpret_cast<const u32x4*>(afrag) + (size_t)c * nsteps * 256;
+    u32x4* lf = reinterpret_cast<u32x4*>(lds);
+    constexpr int SG = 4;  // 16-byte pieces a thread holds at a time
+    const uint32_t total = nsteps * 256;
+    constexpr int PF = RT > 2 ? 3 : 4;
+    St ring[PF];
+    for (uint32_t i0 = 0; i0 < total; i0 += 512 * SG) {
+        u32x4 t[SG];
+#pragma unroll
+        for (int k = 0; k < SG; k++) t[k] = src[min(i0 + 512 * k + threadIdx.x, total - 1)];
+        if (i0 == 0) {
+#pragma unroll
+            for (int p = 0; p < PF; p++) load(ring[p], (uint32_t)p);
+        }
+#pragma unroll
+        for (int k = 0; k < SG; k++)
+            if (i0 + 512 * k + threadIdx.x < total) lf[i0 + 512 * k + threadIdx.x] = t[k];
+    }
+    __syncthreads();
+
     f32x4 acc[RT];
 #pragma unroll
     for (int r = 0; r < RT; r++) acc[r] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     const u32x4 one4 = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
     const bf16x8 ones = __builtin_bit_cast(bf16x8, one4);
-    auto compute = [&](const St& st) {
+    auto compute = [&](const St& st, uint32_t i) {
+        const uint32_t s = kwave + kw * i;
+        bf16x8 a[4];
+#pragma unroll
+        for (int b = 0; b < 4; b++) a[b] = __builtin_bit_cast(bf16x8, lf[(s * 4 + b) * 64 + lane]);
         // E[g]: the group's sum of activations per token (every row's offset multiplies it)
         f32x4 E[2];
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             E[g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            E[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, st.a[2 * g]), ones, E[g], 0, 0, 0);
-            E[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, st.a[2 * g + 1]), ones, E[g], 0, 0, 0);
+            E[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[2 * g], ones, E[g], 0, 0, 0);
+            E[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[2 * g + 1], ones, E[g], 0, 0, 0);
         }
 #pragma unroll
         for (int r = 0; r < RT; r++) {
@@ -124,7 +150,7 @@ __global__ __launch_bounds__(512) void moe_bf16_kernel(WeightView w, const uint8
                 const uint32_t wd = st.w[r][b], lo = wd & 0x0F0F0F0Fu, hi = (wd >> 4) & 0x0F0F0F0Fu;
                 const u32x4 wb = {__builtin_amdgcn_perm(0x43434343u, lo, 0x04010400u), __builtin_amdgcn_perm(0x43434343u, lo, 0x04030402u),
                                   __builtin_amdgcn_perm(0x43434343u, hi, 0x04010400u), __builtin_amdgcn_perm(0x43434343u, hi, 0x04030402u)};
-                D[b >> 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, st.a[b]), __builtin_bit_cast(bf16x8, wb), D[b >> 1], 0, 0, 0);
+                D[b >> 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[b], __builtin_bit_cast(bf16x8, wb), D[b >> 1], 0, 0, 0);
             }
 #pragma unroll
             for (int g = 0; g < 2; g++) {
@@ -132,21 +158,19 @@ __global__ __launch_bounds__(512) void moe_bf16_kernel(WeightView w, const uint8
                 const float off = bf16_bits_to_f32((uint16_t)(g ? st.o[r] >> 16 : st.o[r] & 0xFFFF));
                 const float cc = off - 136.0f * d;
 #pragma unroll
-                for (int i = 0; i < 4; i++) acc[r][i] = fmaf(cc, E[g][i], fmaf(d, D[g][i], acc[r][i]));
+                for (int i2 = 0; i2 < 4; i2++) acc[r][i2] = fmaf(cc, E[g][i2], fmaf(d, D[g][i2], acc[r][i2]));
             }
         }
     };
-    constexpr int PF = 2;
-    St ring[PF];
-#pragma unroll
-    for (int p = 0; p < PF; p++) load(ring[p], (uint32_t)p);
     for (uint32_t ib = 0; ib < cnt; ib += PF) {
 #pragma unroll
         for (int p = 0; p < PF; p++) {
-            if (ib + p < cnt) compute(ring[p]);
+            if (ib + p < cnt) compute(ring[p], ib + p);
             load(ring[p], ib + PF + p);
         }
     }
+    __syncthreads();  // the sums overwrite the fragments
+    float* red = lds;
 #pragma unroll
     for (int r = 0; r < RT; r++) *reinterpret_cast<f32x4*>(red + (((size_t)wave * RT + r) * 64 + lane) * 4) = acc[r];
     __syncthreads();
@@ -171,7 +195,8 @@ __global__ __launch_bounds__(512) void moe_bf16_kernel(WeightView w, const uint8
 
 }  // namespace
 
-bool moe_bf16_ok(const WeightView& w) { return w.fmt == FMT_Q4M && w.n_in % 128 == 0 && w.n_in >= 128; }
+// (the fragments of a chunk, 32 bytes per column, must fit the LDS)
+bool moe_bf16_ok(const WeightView& w) { return w.fmt == FMT_Q4M && w.n_in % 128 == 0 && w.n_in >= 128 && w.n_in <= 4096; }
 
 size_t moe_bf16_frag_bytes(size_t max_chunks, size_t n_in) { return max_chunks * (n_in / 128) * 4 * 64 * 16; }
 
@@ -196,13 +221,26 @@ hipError_t launch_moe_act_pack_bf16(const float* g, const float* u, size_t strid
 hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max_chunks, const void* frag, float* out, hipStream_t s) {
     if (!moe_bf16_ok(w)) return hipErrorInvalidValue;
     if (!max_chunks) return hipSuccess;
-    constexpr int RT = 4;
     const uint32_t nsteps = w.n_in / 128, ntiles = row_tiles(w.n_out);
-    const uint32_t kw = nsteps >= 16 ? 2 : 1, ng = 8 / kw;
-    const size_t lds = (size_t)8 * RT * 64 * 16;
-    moe_bf16_kernel<RT><<<dim3((ntiles + ng * RT - 1) / (ng * RT), max_chunks), 512, lds, s>>>(w, g.bases, g.chunks, g.nchunks,
-                                                                                            static_cast<const uint4*>(frag), kw, out);
-    return hipGetLastError();
+    uint32_t rt = 4, kw = nsteps >= 16 ? 2 : 1;
+    if (const char* e = getenv("OXHIP_MOE_BF16")) {  // developer override for tuning runs: "rt,kw"
+        unsigned a = 0, b = 0;
+        if (sscanf(e, "%u,%u", &a, &b) == 2 && (a == 2 || a == 4) && (b == 1 || b == 2 || b == 4 || b == 8) && b <= nsteps) {
+            rt = a;
+            kw = b;
+        }
+    }
+    const uint32_t ng = 8 / kw;
+    const size_t red = (size_t)8 * rt * 64 * 16, fr = (size_t)nsteps * 4096, lds = fr > red ? fr : red;
+    const dim3 grid((ntiles + ng * rt - 1) / (ng * rt), max_chunks);
+    hipError_t e = hipSuccess;
+    auto go = [&](auto kern) {
+        if (lds > 48 * 1024) e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) kern<<<grid, 512, lds, s>>>(w, g.bases, g.chunks, g.nchunks, static_cast<const uint4*>(frag), kw, out);
+    };
+    if (rt == 2) go(moe_bf16_kernel<2>);
+    else go(moe_bf16_kernel<4>);
+    return e != hipSuccess ? e : hipGetLastError();
 }
 
 }  // namespace oxhip
