@@ -88,18 +88,21 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
 
     struct St {
         u32x4 w[RT];
-        uint32_t d[RT], o[RT];
     };
     // every request is unconditional (past the end the last step again): the compiler then knows how many are in flight
     auto load = [&](St& st, uint32_t i) {
         const uint32_t s = kwave + kw * min(i, ilast);
 #pragma unroll
-        for (int r = 0; r < RT; r++) {
-            const uint8_t* rec = wp[r] + (size_t)s * T4M_REC;
-            st.w[r] = *reinterpret_cast<const u32x4*>(rec + 16 * lane);
-            st.d[r] = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
-            st.o[r] = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
-        }
+        for (int r = 0; r < RT; r++) st.w[r] = *reinterpret_cast<const u32x4*>(wp[r] + (size_t)s * T4M_REC + 16 * lane);
+    };
+    // A record's scale words (per row: the two groups' f16 scales at +1024, their bf16 offsets at +1088): a request costs
+    // the memory pipeline the same for 64 bytes as for 1 KiB, so one request per row tile serves two steps: lane group kq
+    // asks for word kq & 1 of step i + (kq >> 1), and at each step every lane takes its row's two words from those lanes.
+    const uint32_t kq = lane >> 4;
+    auto load_scales = [&](uint32_t* sc, uint32_t i) {
+        const uint32_t s = kwave + kw * min(i + (kq >> 1), ilast);
+#pragma unroll
+        for (int r = 0; r < RT; r++) sc[r] = *reinterpret_cast<const uint32_t*>(wp[r] + (size_t)s * T4M_REC + 1024 + 64 * (kq & 1) + 4 * n);
     };
     // the fragments first (L2 hits, needed by every step), then the first weight records, then the fragments go to LDS
     // while the weights are still on their way
@@ -107,15 +110,19 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
     u32x4* lf = reinterpret_cast<u32x4*>(lds);
     constexpr int SG = 4;  // 16-byte pieces a thread holds at a time
     const uint32_t total = nsteps * 256;
-    constexpr int PF = RT > 2 ? 3 : 4;
+    constexpr int PF = RT > 2 ? 2 : 4;  // steps on request (an even number: scales go by pairs of steps)
     St ring[PF];
+    uint32_t scl[PF / 2][RT];
     for (uint32_t i0 = 0; i0 < total; i0 += 512 * SG) {
         u32x4 t[SG];
 #pragma unroll
         for (int k = 0; k < SG; k++) t[k] = src[min(i0 + 512 * k + threadIdx.x, total - 1)];
         if (i0 == 0) {
 #pragma unroll
-            for (int p = 0; p < PF; p++) load(ring[p], (uint32_t)p);
+            for (int p = 0; p < PF; p++) {
+                if (p % 2 == 0) load_scales(scl[p / 2], (uint32_t)p);
+                load(ring[p], (uint32_t)p);
+            }
         }
 #pragma unroll
         for (int k = 0; k < SG; k++)
@@ -128,7 +135,7 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
     for (int r = 0; r < RT; r++) acc[r] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     const u32x4 one4 = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
     const bf16x8 ones = __builtin_bit_cast(bf16x8, one4);
-    auto compute = [&](const St& st, uint32_t i) {
+    auto compute = [&](const St& st, const uint32_t* sc, int odd, uint32_t i) {
         const uint32_t s = kwave + kw * i;
         bf16x8 a[4];
 #pragma unroll
@@ -152,10 +159,12 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
                                   __builtin_amdgcn_perm(0x43434343u, hi, 0x04010400u), __builtin_amdgcn_perm(0x43434343u, hi, 0x04030402u)};
                 D[b >> 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[b], __builtin_bit_cast(bf16x8, wb), D[b >> 1], 0, 0, 0);
             }
+            const uint32_t dw = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(4 * (32 * odd + n)), (int)sc[r]);
+            const uint32_t ow = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(4 * (32 * odd + 16 + n)), (int)sc[r]);
 #pragma unroll
             for (int g = 0; g < 2; g++) {
-                const float d = f16_bits_to_f32((uint16_t)(g ? st.d[r] >> 16 : st.d[r] & 0xFFFF));
-                const float off = bf16_bits_to_f32((uint16_t)(g ? st.o[r] >> 16 : st.o[r] & 0xFFFF));
+                const float d = f16_bits_to_f32((uint16_t)(g ? dw >> 16 : dw & 0xFFFF));
+                const float off = bf16_bits_to_f32((uint16_t)(g ? ow >> 16 : ow & 0xFFFF));
                 const float cc = off - 136.0f * d;
 #pragma unroll
                 for (int i2 = 0; i2 < 4; i2++) acc[r][i2] = fmaf(cc, E[g][i2], fmaf(d, D[g][i2], acc[r][i2]));
@@ -165,8 +174,9 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
     for (uint32_t ib = 0; ib < cnt; ib += PF) {
 #pragma unroll
         for (int p = 0; p < PF; p++) {
-            if (ib + p < cnt) compute(ring[p], ib + p);
+            if (ib + p < cnt) compute(ring[p], scl[p / 2], p % 2, ib + p);
             load(ring[p], ib + PF + p);
+            if (p % 2 == 1) load_scales(scl[p / 2], ib + PF + p - 1);  // both steps of the pair are done with the old words
         }
     }
     __syncthreads();  // the sums overwrite the fragments
@@ -222,7 +232,9 @@ hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max
     if (!moe_bf16_ok(w)) return hipErrorInvalidValue;
     if (!max_chunks) return hipSuccess;
     const uint32_t nsteps = w.n_in / 128, ntiles = row_tiles(w.n_out);
-    uint32_t rt = 4, kw = nsteps >= 16 ? 2 : 1;
+    // a wave streams a whole row of records (kw = 1) unless that leaves fewer workgroups than two per CU
+    uint32_t rt = 4, kw = 1;
+    while (kw < 4 && nsteps / (2 * kw) >= 4 && (uint64_t)((ntiles + (8 / kw) * rt - 1) / ((8 / kw) * rt)) * max_chunks < 512) kw *= 2;
     if (const char* e = getenv("OXHIP_MOE_BF16")) {  // developer override for tuning runs: "rt,kw"
         unsigned a = 0, b = 0;
         if (sscanf(e, "%u,%u", &a, &b) == 2 && (a == 2 || a == 4) && (b == 1 || b == 2 || b == 4 || b == 8) && b <= nsteps) {
