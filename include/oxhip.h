@@ -184,7 +184,12 @@ int oxhip_dev_gemm_isums(oxhip_ctx* ctx, const oxhip_weight* w, const void* x, i
 int oxhip_dev_route_top_k(oxhip_ctx* ctx, const float* logits, size_t t, size_t n_experts, size_t k, uint32_t* idx, float* w,
                           void* stream);
 /* Backend::moe on device buffers: x [t, h] f32, route_idx / route_w [t, k], y [t, h] f32 (added to).
- * One grouped launch per projection over the routed token lists. The scratch it needs lives in
+ * One grouped launch per projection over the routed token lists. Decode-sized passes run the integer kernels on
+ * int8 activations (Experts::forward / forward_batched, src/moe.rs:438-617; within 1e-3 of them); passes with six
+ * or more routed rows per expert over MLX 4-bit experts run the grouped matmuls on the bf16 matrix cores over the
+ * exact rows with Act::scalar between them, which is the reference's grouped prefill form (src/moe.rs:735-827;
+ * within 2e-2 of it: the rows and the activation's output are rounded to bf16). OXHIP_MOE_INT8=1 in the environment
+ * keeps the integer kernels at every size. The scratch it needs lives in
  * `m` and grows on first use (a call with a larger t * k than any before synchronizes and
  * reallocates); calls on one oxhip_moe must not overlap. */
 int oxhip_dev_moe(oxhip_ctx* ctx, oxhip_moe* m, const float* x, size_t t, const uint32_t* route_idx, const float* route_w,
