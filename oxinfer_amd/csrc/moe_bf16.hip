@@ -108,7 +108,7 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
     // while the weights are still on their way
     const u32x4* src = reinterpret_cast<const u32x4*>(afrag) + (size_t)c * nsteps * 256;
     u32x4* lf = reinterpret_cast<u32x4*>(lds);
-    constexpr int SG = 4;  // 16-byte pieces a thread holds at a time
+    constexpr int SG = 8;  // 16-byte pieces a thread holds at a time (2048 columns of 16 rows in one batch)
     const uint32_t total = nsteps * 256;
     constexpr int PF = RT > 2 ? 2 : 4;  // steps on request (an even number: scales go by pairs of steps)
     St ring[PF];
