@@ -55,6 +55,23 @@ def test_route_top_k_matches_oracle_and_definition(be, oxref):
     assert list(idx[0, :2]) == [7, 90] and list(idx[1]) == list(range(k))
 
 
+@pytest.mark.parametrize("ne,k", [(100, 4), (256, 8), (300, 6), (64, 1), (33, 32), (7, 7), (1024, 16)])
+def test_route_top_k_other_sizes(be, oxref, ne, k):
+    """Up to 256 experts the kernel counts ranks, beyond that it runs k rounds of argmax: both against the oracle, with
+    ties (quantized logits) and expert counts that do not fill the lanes."""
+    import torch
+    from oxinfer_amd import synth
+    t = 9
+    logits = synth.router_logits(t, ne, 40 + ne)
+    logits[3:6] = np.round(logits[3:6] * 2.0) / 2.0  # many ties
+    idx, w = be.route_top_k(torch.from_numpy(logits).cuda(), k)
+    idx, w = idx.cpu().numpy().astype(np.uint32), w.cpu().numpy()
+    for i in range(t):
+        ri, rw = oxref.route_top_k(logits[i], k)
+        assert np.array_equal(idx[i], ri), i
+        assert np.allclose(w[i], rw, rtol=1e-6, atol=0), i
+
+
 def moe_reference(oxref, kind, gate_up, down, h, inter, x, idx, w, y0):
     """Each (token, route) pair on the oracle's decode kernels, combined in route order (what
     forward_batched computes row by row, src/moe.rs:438-617)."""
@@ -164,6 +181,28 @@ def test_moe_gguf_experts(be, oxref, kind):
         assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
         ref = moe_reference(oxref, kind, gu, dn, h, inter, x, idx, w, np.zeros((t, h), np.float32))
         assert row_err(y, ref) < 1e-3, t
+
+
+def test_moe_config_shapes(be, oxref):
+    """The benchmark's expert shapes (h 2048, inter 768, top-8) over 16 experts: one token on the integer kernels against
+    the oracle's decode path, 32 tokens (16 routed rows per expert: the bf16 form) against its grouped f32 path."""
+    import torch
+    from oxinfer_amd import synth
+    ne, h, inter, k = 16, 2048, 768, 8
+    raw_gu = [synth.mlx_q4(2 * inter, h, 700 + e) for e in range(ne)]
+    raw_dn = [synth.mlx_q4(h, inter, 800 + e) for e in range(ne)]
+    q_gu = [oxref.from_mlx_q4(*r, 2 * inter, h, 64) for r in raw_gu]
+    q_dn = [oxref.from_mlx_q4(*r, h, inter, 64) for r in raw_dn]
+    dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)
+    assert dev is not None, be.last_error()
+    for t, decode_path, tol in ((1, True, 1e-3), (32, False, 5e-3)):
+        x = synth.activations(t, h, 900 + t, bf16=True)  # bf16 values, as in the workload
+        _, idx, w = make_routes(oxref, t, ne, k, 950 + t)
+        y0 = np.zeros((t, h), np.float32)
+        y = y0.copy()
+        assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
+        ref = oxref.moe_q4(q_gu, q_dn, 64, h, inter, x, t, idx, w, y0, decode_path=decode_path)
+        assert row_err(y, ref) < tol, (t, row_err(y, ref))
 
 
 def test_moe_declines(be, oxref, mlx_experts):
