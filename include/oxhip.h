@@ -140,8 +140,9 @@ int oxhip_dev_decode(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa
  * matmul_quant_batch does for the CPU, src/kernels.rs:1937-1994). The jobs must not depend on one another: runs of
  * consecutive jobs of at most 8 tokens over Q8 / Q8_0 / Q4_K / Q6_K / MLX 4-bit weights share ONE launch (their latency chains
  * overlap; every job's rows are bit-identical to a launch of its own), the others launch one by one, in order, on
- * `stream`. ev_start / ev_stop (from oxhip_event_create, or NULL) are recorded before / after the launch that
- * holds the job: for jobs that share a launch they bracket the whole shared launch.
+ * `stream` (inside a shared launch the library orders the jobs itself). ev_start / ev_stop (from oxhip_event_create, or
+ * NULL) are recorded before / after the launch that holds the job; for jobs that share a launch the first start and the
+ * last stop event take the shared launch's own start and end as the device saw them.
  * The decode entry points use scratch owned by ctx (partial rows of K slices): launches on one ctx must be ordered
  * (one stream, or the caller's own synchronization). */
 typedef struct {

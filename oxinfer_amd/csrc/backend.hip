@@ -394,20 +394,33 @@ int oxhip_dev_decode_batch(oxhip_ctx* c, const oxhip_decode_job* jobs, size_t n_
         size_t e = j;
         while (e < n_jobs && fusable(jobs[e])) e++;
         if (e - j >= 2) {
+            // the first start event and the last stop event of the run bracket the shared launch; any others are
+            // recorded on the stream around it
             items.clear();
+            hipEvent_t e0 = nullptr, e1 = nullptr;
             for (size_t k = j; k < e; k++) {
-                if (jobs[k].ev_start) HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jobs[k].ev_start), s), "event record");
+                if (jobs[k].ev_start) {
+                    if (!e0) e0 = static_cast<hipEvent_t>(jobs[k].ev_start);
+                    else HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jobs[k].ev_start), s), "event record");
+                }
                 items.push_back(DecodeBatchItem{jobs[k].w->v, view_of(*jobs[k].xa), jobs[k].y, (uint32_t)jobs[k].t});
             }
-            const hipError_t err = launch_decode_mfma_batch(items.data(), items.size(), c->dec, s);
+            for (size_t k = e; k-- > j;)
+                if (jobs[k].ev_stop) {
+                    e1 = static_cast<hipEvent_t>(jobs[k].ev_stop);
+                    break;
+                }
+            const hipError_t err = launch_decode_mfma_batch(items.data(), items.size(), c->dec, s, e0, e1);
             if (err == hipErrorOutOfMemory) {  // the scratch does not hold these jobs together: one launch each
+                if (e0) HIP_TRY(hipEventRecord(e0, s), "event record");
                 for (size_t k = j; k < e; k++)
                     if (!oxhip_dev_decode(c, jobs[k].w, jobs[k].xa, jobs[k].x, jobs[k].t, jobs[k].y, stream)) return 0;
+                if (e1) HIP_TRY(hipEventRecord(e1, s), "event record");
             } else {
                 HIP_TRY(err, "decode batch launch");
             }
             for (size_t k = j; k < e; k++)
-                if (jobs[k].ev_stop) HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jobs[k].ev_stop), s), "event record");
+                if (jobs[k].ev_stop && static_cast<hipEvent_t>(jobs[k].ev_stop) != e1) HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jobs[k].ev_stop), s), "event record");
             j = e;
             continue;
         }

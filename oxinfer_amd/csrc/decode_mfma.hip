@@ -36,6 +36,8 @@
 #include <mutex>
 #include <vector>
 
+#include <hip/hip_ext.h>
+
 #include "internal.hpp"
 #include "layout.hpp"
 
@@ -939,7 +941,8 @@ bool decode_batchable(const WeightView& w, size_t t) {
 // Every item must be decode_batchable. Items go out in launches of up to BATCH_MAX jobs; jobs whose shape slices K
 // across workgroups take their partial rows and counters from `sc` (hipErrorOutOfMemory when it is too small:
 // nothing has been launched then and the caller launches the jobs one by one).
-hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s) {
+hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s, hipEvent_t ev_start,
+                                    hipEvent_t ev_stop) {
     static std::atomic<uint64_t> allowed[4];  // whole LDS allowed, one bit per device
     int dev = 0;
     (void)hipGetDevice(&dev);
@@ -1006,12 +1009,22 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
         ldss.push_back(lds);
         threadss.push_back(threads);
     }
+    // Timing events: with one launch they ride on the dispatch itself (its start and end as the device saw them, and no
+    // barrier packets on the stream, which would keep neighbouring launches from overlapping); with several they are
+    // recorded on the stream before the first and after the last.
+    const bool ride = launches.size() == 1 && launches[0].nwg && (ev_start || ev_stop);
+    if (!ride && ev_start) {
+        hipError_t e = hipEventRecord(ev_start, s);
+        if (e != hipSuccess) return e;
+    }
     for (size_t i = 0; i < launches.size(); i++) {
         if (!launches[i].nwg) continue;
-        decode_batch_kernel<<<launches[i].nwg, threadss[i], ldss[i], s>>>(launches[i]);
+        if (ride) hipExtLaunchKernelGGL(decode_batch_kernel, dim3(launches[i].nwg), dim3(threadss[i]), (uint32_t)ldss[i], s, ev_start, ev_stop, 0, launches[i]);
+        else decode_batch_kernel<<<launches[i].nwg, threadss[i], ldss[i], s>>>(launches[i]);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
+    if (!ride && ev_stop) return hipEventRecord(ev_stop, s);
     return hipSuccess;
 }
 

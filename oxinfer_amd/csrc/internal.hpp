@@ -96,7 +96,9 @@ struct DecodeBatchItem {
     uint32_t t;
 };
 bool decode_batchable(const WeightView& w, size_t t);  // the kernel takes it and its activations fit LDS
-hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s);
+// ev_start / ev_stop (optional): timing events around the launches.
+hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s, hipEvent_t ev_start = nullptr,
+                                    hipEvent_t ev_stop = nullptr);
 hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, const DecodeScratch& sc, hipStream_t s);
 hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks,
                                       uint32_t max_rows_per_chunk, float* y, hipStream_t s);
