@@ -100,7 +100,9 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
     // moe_bf16.hip. OXHIP_MOE_INT8=1 keeps the integer path (the 1e-3 accuracy class) at any size.
     const bool fused = m->up.empty();
     const char* keep_int = getenv("OXHIP_MOE_INT8");
-    const bool bf16_form = avg >= 6 && fused && moe_bf16_ok(m->gate_up[0]->v) && moe_bf16_ok(m->down[0]->v) && !(keep_int && keep_int[0] == '1');
+    const size_t grid_chunks16 = (pairs < m->n_exp ? pairs : m->n_exp) + pairs / 16 + 1;
+    const bool bf16_form = avg >= 6 && fused && moe_bf16_ok(m->gate_up[0]->v) && moe_bf16_ok(m->down[0]->v) && !(keep_int && keep_int[0] == '1') &&
+                           reinterpret_cast<uintptr_t>(x) % 16 == 0 && grid_chunks16 <= 65535;
     if (bf16_form) max_rows = 16;
     const uint32_t grid_chunks = (uint32_t)((pairs < m->n_exp ? pairs : m->n_exp) + pairs / max_rows + 1);
     GroupView g{};
