@@ -183,6 +183,24 @@ def test_moe_gguf_experts(be, oxref, kind):
         assert row_err(y, ref) < 1e-3, t
 
 
+def test_moe_prefill_rows_do_not_depend_on_the_batch(be, oxref, mlx_experts):
+    """In the bf16 form too every (token, row) sum is formed on its own in a fixed order: a token's output is
+    bit-identical whichever other tokens share the pass (and its expert's chunks)."""
+    from oxinfer_amd import synth
+    ne, h, inter, raw_gu, raw_dn, _, _ = mlx_experts
+    k, t = 3, 40
+    dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)
+    x = synth.activations(t, h, 21)
+    _, idx, w = make_routes(oxref, t, ne, k, 22)
+    y = np.zeros((t, h), np.float32)
+    assert be.moe(x, t, h, inter, idx, w, k, dev, y)
+    for keep in (np.arange(8, 40), np.arange(0, 40, 2)[:14].repeat(1), np.r_[0:5, 20:33]):
+        assert (len(keep) * k) // ne >= 6  # still the bf16 form
+        ys = np.zeros((len(keep), h), np.float32)
+        assert be.moe(np.ascontiguousarray(x[keep]), len(keep), h, inter, np.ascontiguousarray(idx[keep]), np.ascontiguousarray(w[keep]), k, dev, ys)
+        assert np.array_equal(ys.view(np.uint32), y[keep].view(np.uint32))
+
+
 def test_moe_config_shapes(be, oxref):
     """The benchmark's expert shapes (h 2048, inter 768, top-8) over 16 experts: one token on the integer kernels against
     the oracle's decode path, 32 tokens (16 routed rows per expert: the bf16 form) against its grouped f32 path."""
