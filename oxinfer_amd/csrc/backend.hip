@@ -75,9 +75,9 @@ int oxhip_open(int device, oxhip_ctx** out) {
     auto* c = new oxhip_ctx();
     c->device = device;
     c->name = "hip (" + arch + ")";
-    // 16 MiB of partial rows (32 slices x 8 tokens x 16384 outputs) and 16384 counters, zero between launches
+    // 16 MiB of partial rows (32 slices x 8 tokens x 16384 outputs) and 16384 counters (a line each), zero between launches
     c->dec.partial_floats = (size_t)4 << 20;
-    c->dec.ncounters = 16384;
+    c->dec.ncounters = (size_t)16384 * CTR_STRIDE;
     if (hipMalloc(reinterpret_cast<void**>(&c->dec.partial), c->dec.partial_floats * 4) != hipSuccess ||
         hipMalloc(reinterpret_cast<void**>(&c->dec.counters), c->dec.ncounters * 4) != hipSuccess ||
         hipMemset(c->dec.counters, 0, c->dec.ncounters * 4) != hipSuccess) {

@@ -642,9 +642,9 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
-        const uint32_t seen = __hip_atomic_fetch_add(&counters[bx], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t seen = __hip_atomic_fetch_add(&counters[(size_t)bx * CTR_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         is_last = seen == ksplit - 1;
-        if (seen == ksplit - 1) __hip_atomic_store(&counters[bx], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (seen == ksplit - 1) __hip_atomic_store(&counters[(size_t)bx * CTR_STRIDE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!is_last) return;
@@ -857,7 +857,7 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
     Shape sh = shape_for(ntiles, nsteps, true, FMT);
     const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
     // slices need scratch: 8 token rows per slice and a counter per row group
-    if (sh.ks > 1 && (!sc.partial || !sc.counters || sc.partial_floats < (size_t)sh.ks * 8 * w.n_out || sc.ncounters < groups))
+    if (sh.ks > 1 && (!sc.partial || !sc.counters || sc.partial_floats < (size_t)sh.ks * 8 * w.n_out || sc.ncounters < (size_t)groups * CTR_STRIDE))
         sh = shape_for(ntiles, nsteps, false, FMT);
     const uint32_t nblk = w.n_in / 32;
     dim3 grid((ntiles + sh.rt - 1) / sh.rt, sh.ks), block(64 * sh.rt * sh.kw);
@@ -993,11 +993,11 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
             uint32_t* counters = nullptr;
             if (sh.ks > 1) {
                 const size_t need = (size_t)sh.ks * it.t * it.w.n_out;
-                if (!sc.partial || !sc.counters || pf + need > sc.partial_floats || nc + groups > sc.ncounters) return hipErrorOutOfMemory;
+                if (!sc.partial || !sc.counters || pf + need > sc.partial_floats || nc + (size_t)groups * CTR_STRIDE > sc.ncounters) return hipErrorOutOfMemory;
                 partial = sc.partial + pf;
                 counters = sc.counters + nc;
                 pf += (need + 63) / 64 * 64;
-                nc += groups;
+                nc += (size_t)groups * CTR_STRIDE;
             }
             lds = l > lds ? l : lds;
             threads = 64 * sh.rt * sh.kw > threads ? 64 * sh.rt * sh.kw : threads;

@@ -80,6 +80,9 @@ hipError_t launch_pack_fp8(const uint8_t* raw, size_t n_out, size_t n_in, uint8_
 // Global scratch of the decode kernels that split K across workgroups: `partial` holds slices x 8 token rows of
 // n_out floats, `counters` (zero between launches) one entry per group of row tiles. Launches that share a scratch
 // must be ordered on one stream. Without scratch the kernels keep K inside a workgroup.
+// Arrival counters of the K slices sit one per 128 bytes: atomics on one line take their turn, and neighbouring row
+// groups finish at about the same time.
+constexpr uint32_t CTR_STRIDE = 32;
 struct DecodeScratch {
     float* partial = nullptr;
     uint32_t* counters = nullptr;
