@@ -356,7 +356,8 @@ int oxhip_dev_dequantize(oxhip_ctx* c, const oxhip_weight* w, size_t r0, size_t 
     return 1;
 }
 
-int oxhip_dev_decode(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa, const float* x, size_t t, float* y, void* stream) {
+static int decode_one(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa, const float* x, size_t t, float* y, void* stream,
+                      hipEvent_t ev_start, hipEvent_t ev_stop) {
     if (!c || !w || !y || t == 0 || t > 16) {
         set_error("decode: bad arguments (1 <= t <= 16)");
         return 0;
@@ -374,8 +375,12 @@ int oxhip_dev_decode(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa, 
         }
         v = view_of(*xa);
     }
-    HIP_TRY(launch_decode(w->v, v, x, t, y, static_cast<hipStream_t>(stream), c->dec), "decode launch");
+    HIP_TRY(launch_decode(w->v, v, x, t, y, static_cast<hipStream_t>(stream), c->dec, ev_start, ev_stop), "decode launch");
     return 1;
+}
+
+int oxhip_dev_decode(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa, const float* x, size_t t, float* y, void* stream) {
+    return decode_one(c, w, xa, x, t, y, stream, nullptr, nullptr);
 }
 
 int oxhip_dev_decode_batch(oxhip_ctx* c, const oxhip_decode_job* jobs, size_t n_jobs, void* stream) {
@@ -425,9 +430,7 @@ int oxhip_dev_decode_batch(oxhip_ctx* c, const oxhip_decode_job* jobs, size_t n_
             continue;
         }
         const oxhip_decode_job& jb = jobs[j];
-        if (jb.ev_start) HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jb.ev_start), s), "event record");
-        if (!oxhip_dev_decode(c, jb.w, jb.xa, jb.x, jb.t, jb.y, stream)) return 0;
-        if (jb.ev_stop) HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jb.ev_stop), s), "event record");
+        if (!decode_one(c, jb.w, jb.xa, jb.x, jb.t, jb.y, stream, static_cast<hipEvent_t>(jb.ev_start), static_cast<hipEvent_t>(jb.ev_stop))) return 0;
         j++;
     }
     return 1;

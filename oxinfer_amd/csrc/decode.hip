@@ -291,14 +291,9 @@ hipError_t decode_dense_t(const WeightView& w, const float* x, size_t t, float* 
 
 }  // namespace
 
-hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s,
-                         const DecodeScratch& sc) {
+static hipError_t launch_decode_plain(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s,
+                                      const DecodeScratch& sc) {
     switch (w.fmt) {
-        case FMT_Q8_0:
-        case FMT_Q8F:
-        case FMT_Q4_K:
-        case FMT_Q6_K:
-        case FMT_Q4M: return launch_decode_mfma(w, xa, t, y, sc, s);
         case FMT_Q4: return decode_t<FMT_Q4, 4>(w, xa, t, y, s);
         case FMT_FP8:
             // the matrix-core kernel when the block scales allow it and the caller's scratch holds the packed activations
@@ -308,6 +303,15 @@ hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x
         case FMT_BF16: return decode_dense_t<FMT_BF16, 4>(w, x, t, y, s);
         default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s,
+                         const DecodeScratch& sc, hipEvent_t ev_start, hipEvent_t ev_stop) {
+    if (mfma_decode_format(w.fmt)) return launch_decode_mfma(w, xa, t, y, sc, s, ev_start, ev_stop);
+    hipError_t e = ev_start ? hipEventRecord(ev_start, s) : hipSuccess;
+    if (e == hipSuccess) e = launch_decode_plain(w, xa, x, t, y, s, sc);
+    if (e == hipSuccess && ev_stop) e = hipEventRecord(ev_stop, s);
+    return e;
 }
 
 hipError_t launch_isums(const WeightView& w, const QActView& xa, size_t t, int32_t* out, hipStream_t s) {

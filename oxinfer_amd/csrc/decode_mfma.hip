@@ -826,7 +826,8 @@ size_t lds_bytes(bool sums, bool dump, uint32_t bps, uint32_t nsteps, int tpad, 
 
 template <int FMT, int NT, bool DUMP, bool GROUPED, int NG = 1>
 hipError_t launch_one(bool alds, dim3 grid, dim3 block, size_t lds, hipStream_t s, const WeightView& w, const QActView& v, uint32_t t,
-                      const Shape& sh, float* y, int32_t* dump, const GroupView& g, const DecodeScratch& sc) {
+                      const Shape& sh, float* y, int32_t* dump, const GroupView& g, const DecodeScratch& sc, hipEvent_t ev_start = nullptr,
+                      hipEvent_t ev_stop = nullptr) {
     hipError_t e = hipSuccess;
     auto go = [&](auto kern) {
         // once per kernel and device: allow the whole LDS
@@ -838,7 +839,11 @@ hipError_t launch_one(bool alds, dim3 grid, dim3 block, size_t lds, hipStream_t 
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
             if (e == hipSuccess) allowed[(dev >> 6) & 3].fetch_or(bit, std::memory_order_release);
         }
-        if (e == hipSuccess) kern<<<grid, block, lds, s>>>(w, v, t, sh.rt, sh.kw, y, dump, g, sh.ks, sc.partial, sc.counters);
+        if (e != hipSuccess) return;
+        // timing events ride on the dispatch: its start and end as the device saw them
+        if (ev_start || ev_stop)
+            hipExtLaunchKernelGGL(kern, grid, block, (uint32_t)lds, s, ev_start, ev_stop, 0, w, v, t, sh.rt, sh.kw, y, dump, g, sh.ks, sc.partial, sc.counters);
+        else kern<<<grid, block, lds, s>>>(w, v, t, sh.rt, sh.kw, y, dump, g, sh.ks, sc.partial, sc.counters);
     };
     if (alds) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, true, NG>);
     else if constexpr (NG == 1 && FMT != FMT_Q6_K) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, false, 1>);
@@ -852,7 +857,8 @@ constexpr uint32_t steps_of(uint32_t n_in) {
 }
 
 template <int FMT, bool DUMP>
-hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* dump, const DecodeScratch& sc, hipStream_t s) {
+hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* dump, const DecodeScratch& sc, hipStream_t s,
+               hipEvent_t ev_start = nullptr, hipEvent_t ev_stop = nullptr) {
     const uint32_t ntiles = row_tiles(w.n_out), nsteps = steps_of<FMT>(w.n_in);
     Shape sh = shape_for(ntiles, nsteps, true, FMT);
     const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
@@ -861,6 +867,13 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
         sh = shape_for(ntiles, nsteps, false, FMT);
     const uint32_t nblk = w.n_in / 32;
     dim3 grid((ntiles + sh.rt - 1) / sh.rt, sh.ks), block(64 * sh.rt * sh.kw);
+    // timing events: one launch carries them itself; around several they are recorded on the stream
+    const bool ride = t <= 8;
+    if (!ride && ev_start) {
+        hipError_t e = hipEventRecord(ev_start, s);
+        if (e != hipSuccess) return e;
+    }
+    hipEvent_t e0 = ride ? ev_start : nullptr, e1 = ride ? ev_stop : nullptr;
     size_t c0 = 0;
     while (c0 < t) {
         const size_t tc = t - c0 < 8 ? t - c0 : 8;
@@ -879,13 +892,14 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
         if (lds > LDS_MAX) return hipErrorInvalidValue;  // rows too long for the staged activation scales
         const uint32_t tt = (uint32_t)tc;
         hipError_t e;
-        if (tc == 1) e = launch_one<FMT, 1, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
-        else if (tc == 2 && FMT != FMT_Q4M) e = launch_one<FMT, 2, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
-        else if (tc <= 4) e = launch_one<FMT, 4, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
-        else e = launch_one<FMT, 8, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc);
+        if (tc == 1) e = launch_one<FMT, 1, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
+        else if (tc == 2 && FMT != FMT_Q4M) e = launch_one<FMT, 2, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
+        else if (tc <= 4) e = launch_one<FMT, 4, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
+        else e = launch_one<FMT, 8, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
         if (e != hipSuccess) return e;
         c0 += tc;
     }
+    if (!ride && ev_stop) return hipEventRecord(ev_stop, s);
     return hipSuccess;
 }
 
@@ -1039,13 +1053,14 @@ hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, c
     }
 }
 
-hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, const DecodeScratch& sc, hipStream_t s) {
+hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, const DecodeScratch& sc, hipStream_t s,
+                              hipEvent_t ev_start, hipEvent_t ev_stop) {
     switch (w.fmt) {
-        case FMT_Q8_0: return run<FMT_Q8_0, false>(w, xa, t, y, nullptr, sc, s);
-        case FMT_Q8F: return run<FMT_Q8F, false>(w, xa, t, y, nullptr, sc, s);
-        case FMT_Q4_K: return run<FMT_Q4_K, false>(w, xa, t, y, nullptr, sc, s);
-        case FMT_Q6_K: return run<FMT_Q6_K, false>(w, xa, t, y, nullptr, sc, s);
-        case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, sc, s);
+        case FMT_Q8_0: return run<FMT_Q8_0, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
+        case FMT_Q8F: return run<FMT_Q8F, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
+        case FMT_Q4_K: return run<FMT_Q4_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
+        case FMT_Q6_K: return run<FMT_Q6_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
+        case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
         default: return hipErrorInvalidValue;
     }
 }

@@ -88,8 +88,9 @@ struct DecodeScratch {
     uint32_t* counters = nullptr;
     size_t partial_floats = 0, ncounters = 0;
 };
+// ev_start / ev_stop (optional): timing events around the launches (carried by the launch itself where there is one).
 hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s,
-                         const DecodeScratch& sc = DecodeScratch{});
+                         const DecodeScratch& sc = DecodeScratch{}, hipEvent_t ev_start = nullptr, hipEvent_t ev_stop = nullptr);
 hipError_t launch_isums(const WeightView& w, const QActView& xa, size_t t, int32_t* out, hipStream_t s);
 // Independent matmuls that may share one launch (decode_mfma.hip): each 1..8 tokens over a tile-packed weight.
 struct DecodeBatchItem {
@@ -102,7 +103,8 @@ bool decode_batchable(const WeightView& w, size_t t);  // the kernel takes it an
 // ev_start / ev_stop (optional): timing events around the launches.
 hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s, hipEvent_t ev_start = nullptr,
                                     hipEvent_t ev_stop = nullptr);
-hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, const DecodeScratch& sc, hipStream_t s);
+hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, const DecodeScratch& sc, hipStream_t s,
+                              hipEvent_t ev_start = nullptr, hipEvent_t ev_stop = nullptr);
 hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks,
                                       uint32_t max_rows_per_chunk, float* y, hipStream_t s);
 hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* out, hipStream_t s);
