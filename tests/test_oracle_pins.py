@@ -7,26 +7,18 @@ the mathematics fixes, without running the reference.
 - quantize_act: the scalar definition of src/quant.rs:633-658 including its special cases.
 - decode_i8: the invariant of src/ggml.rs:1663-1681.
 """
+import json
+import os
+
 import numpy as np
 import pytest
 import torch
 
-# (type id, hash) copied from the reference's golden table, src/ggml.rs:1547-1577
-REF_HASHES = {
-    "BF16": (30, 0x767e77c423088e31),
-    "F16": (1, 0xd03c69ee7934955f),
-    "F32": (0, 0x8c4157552256808b),
-    "Q2_K": (10, 0x44b0a081c4b9c71c),
-    "Q4_0": (2, 0xc2ac60f0d9d22bc8),
-    "Q4_1": (3, 0x8a49b60459c03fa2),
-    "Q4_K": (12, 0xde4da39c1d9096b2),
-    "Q5_0": (6, 0x46640e791feaf19f),
-    "Q5_1": (7, 0xb0fd98e61b74d61d),
-    "Q5_K": (13, 0x4be2f59b66cc7042),
-    "Q6_K": (14, 0x20a51cc0feaae638),
-    "Q8_0": (8, 0x3199be3deddf5c1a),
-}
-FIXTURE_ELEMS = 1024
+# (type id, hash): the reference's golden table (src/ggml.rs:1547-1577), kept as a fixture
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_hashes.json")) as _f:
+    _GOLDEN = json.load(_f)
+REF_HASHES = {name: (e["ggml_type"], int(e["fnv1a64"], 16)) for name, e in _GOLDEN["hashes"].items()}
+FIXTURE_ELEMS = _GOLDEN["elements"]
 
 
 def fixture_blocks(oxref, kind):
