@@ -4,6 +4,9 @@ Bars: activation quantization, dequantized weights and the int32 accumulators bi
 outputs within 1e-3 of the oracle's (f32 accumulation), measured like the reference's `row_err`
 (src/cuda.rs:1583-1592): worst error of a token row over that row's largest reference value.
 """
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -66,7 +69,8 @@ def test_quantize_act_bit_exact(be, oxref):
     assert np.array_equal(xa.sums16.cpu().numpy(), s16)
 
 
-REF_HASHES = {Q8_0: 0x3199be3deddf5c1a, Q4_K: 0xde4da39c1d9096b2, Q6_K: 0x20a51cc0feaae638}
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_hashes.json")) as _f:  # src/ggml.rs:1547-1577
+    REF_HASHES = {e["ggml_type"]: int(e["fnv1a64"], 16) for e in json.load(_f)["hashes"].values()}
 
 
 @pytest.mark.parametrize("kind", [Q8_0, Q4_K, Q6_K])
