@@ -248,8 +248,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gguf_gemv", choices=["gguf_gemv", "gguf_gemv_q6k", "mlx_gemv", "mlx_gemm", "moe", "fp8", "copy"],
-                    help="copy = a plain 256 MiB device copy, the known-size kernel that scales the HBM traffic counters")
+    ap.add_argument("--workload", default="gguf_gemv", choices=["gguf_gemv", "gguf_gemv_q6k", "gguf_stream", "mlx_gemv", "mlx_gemm", "moe", "fp8", "copy"],
+                    help="copy = a plain 256 MiB device copy, the known-size kernel that scales the HBM traffic counters; "
+                         "gguf_stream = every GGUF case alone as a steady stream of 192 matmuls handed over in one call")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pool-gb", type=float, default=POOL_BYTES / 1e9)
     ap.add_argument("--variant", default="bf16", choices=["bf16", "i8", "fp8"], help="GEMM variant of mlx_gemm / fp8")
@@ -280,7 +281,7 @@ def main():
         be.close()
         return
     gens = {Q8_0: synth.gguf_q8_0, Q4_K: synth.gguf_q4_k, Q6_K: synth.gguf_q6_k}
-    kinds = [Q8_0, Q4_K] if args.workload == "gguf_gemv" else [Q6_K]
+    kinds = [Q8_0, Q4_K] if args.workload == "gguf_gemv" else [Q6_K] if args.workload == "gguf_gemv_q6k" else [Q8_0, Q4_K, Q6_K]
     cases = gemv_cases(kinds)
 
     # rotating pools of distinct device copies per (format, shape)
@@ -303,6 +304,31 @@ def main():
         c["y"] = torch.empty((c["t"], c["n_out"]), dtype=torch.float32, device="cuda")
         c["pool"] = pools[(c["kind"], c["n_out"], c["n_in"])]
     torch.cuda.synchronize()
+
+    if args.workload == "gguf_stream":
+        # Each case alone, 192 matmuls over rotating weight copies in one call (launches of 16, back to back): what the
+        # kernel streams at when no launch boundary, ramp or tail is in the way. One JSON line; `value` is the mean.
+        detail, tot_b, tot_s = {}, 0.0, 0.0
+        for c in cases:
+            pool = c["pool"]
+            arr = be.decode_jobs([(pool[i % len(pool)], c["xa"], None, c["t"], c["y"], None, None) for i in range(192)])
+            be.decode_batch(arr)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            be.decode_batch(arr)
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / 192
+            detail[c["name"]] = {"us": round(us, 2), "GBs": round(c["bytes"] / us / 1e3, 1), "frac_hbm": round(c["bytes"] / us / 1e3 / HBM_PEAK_GBS, 4)}
+            tot_b += c["bytes"]
+            tot_s += us * 1e-6
+        print(json.dumps({"metric": METRIC, "value": round(tot_b / tot_s / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "higher_is_better": True,
+                          "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+                          "config": {"workload": "GGUF GEMV cases of configs[1] (and Q6_K), each as a steady stream of 192 matmuls in one call"},
+                          "detail": detail}))
+        be.close()
+        return
 
     # The dominant kernel. The jobs of one call share one launch (decode_batch_kernel): that launch is the step, and
     # its events bracket it. (Formats the shared launch does not take would launch one by one: then the largest
