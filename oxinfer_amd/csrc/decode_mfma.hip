@@ -45,6 +45,11 @@ namespace oxhip {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
+// Where slot `slot` (0..63) of row `row` of the LDS operand array sits: the staging stores of a token's consecutive chunks
+// differ only in the row and in slot bits 3 and 5, which alone would put 64 lanes into two bank pairs; mixing the row's
+// low bits into slot bits 0..2 and 4 spreads them over all banks, and a row's 64 slots stay a permutation of the row.
+__device__ __forceinline__ uint32_t opslot(uint32_t row, uint32_t slot) { return slot ^ (row & 7u) ^ ((row & 8u) << 1); }
+
 namespace {
 
 // Records a wave keeps in flight. HBM delivers about 8 TB/s at about 2 us of loaded latency, so some 16 MB must be
@@ -135,6 +140,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                                             float* __restrict__ lds_all) {
     static_assert(NG == 1 || (GROUPED && ALDS && !DUMP && NT == 8), "token groups are for grouped launches");
     constexpr int TPAD = NT <= 4 ? 4 : 8;
+    // the swizzled operand array pays at 8 tokens (where the staging stores are many); at fewer its address math costs more
+    constexpr bool SWZ = NT >= 8;
     constexpr int NI = NT < 4 ? NT : 4;          // accumulator registers that hold live tokens
     constexpr bool SUMS = !q8_format(FMT);
     // the wave index and everything derived from it (tile, K range) live in scalar registers: branches on them are
@@ -273,7 +280,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // `m`: index of the instruction along K (pair of blocks 2 m, 2 m + 1); with ALDS its operand comes from LDS
     auto mfma = [&](v4i bw, uint32_t m, int tg, uint32_t d0, uint32_t d1) -> v4i {
         if (ALDS) {
-            const uint2 av = afr[((size_t)tg * (nbl / 2) + (m - M0)) * 64 + lane];
+            const uint2 av = afr[((size_t)tg * (nbl / 2) + (m - M0)) * 64 + (SWZ ? opslot(m - M0, lane) : lane)];
             d0 = av.x;
             d1 = av.y;
         }
@@ -455,18 +462,20 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     auto act_store = [&](uint32_t tok, uint32_t c, const uint4* v) {
         if (FMT == FMT_Q4M) {
             const uint32_t b = c;
-            uint2* dst = afr + ((size_t)(tok >> 3) * (nbl / 2) + (b >> 1)) * 64 + 8 * (b & 1) + (tok & 7);
-            dst[0] = make_uint2(v[0].x, v[1].x);
-            dst[16] = make_uint2(v[0].y, v[1].y);
-            dst[32] = make_uint2(v[0].z, v[1].z);
-            dst[48] = make_uint2(v[0].w, v[1].w);
+            uint2* dst = afr + ((size_t)(tok >> 3) * (nbl / 2) + (b >> 1)) * 64;
+            const uint32_t s0 = SWZ ? opslot(b >> 1, 8 * (b & 1) + (tok & 7)) : 8 * (b & 1) + (tok & 7);
+            dst[s0] = make_uint2(v[0].x, v[1].x);
+            dst[s0 ^ 16] = make_uint2(v[0].y, v[1].y);
+            dst[s0 ^ 32] = make_uint2(v[0].z, v[1].z);
+            dst[s0 ^ 48] = make_uint2(v[0].w, v[1].w);
         } else if (FMT == FMT_Q6_K) {  // chunk c = columns 16 c ..: sub-block c % 4 of 64-column group c / 4
             reinterpret_cast<uint4*>(afr)[((size_t)(c >> 2) * 8 + (tok & 7)) * 4 + (c & 3)] = make_uint4(v[0].x, v[0].y, v[0].z, v[0].w);
         } else {
             const uint32_t b = c >> 1;
-            uint2* dst = afr + ((size_t)(tok >> 3) * (nbl / 2) + (b >> 1)) * 64 + 32 * (c & 1) + 8 * (b & 1) + (tok & 7);
-            dst[0] = make_uint2(v[0].x, v[0].y);
-            dst[16] = make_uint2(v[0].z, v[0].w);
+            uint2* dst = afr + ((size_t)(tok >> 3) * (nbl / 2) + (b >> 1)) * 64;
+            const uint32_t s0 = SWZ ? opslot(b >> 1, 32 * (c & 1) + 8 * (b & 1) + (tok & 7)) : 32 * (c & 1) + 8 * (b & 1) + (tok & 7);
+            dst[s0] = make_uint2(v[0].x, v[0].y);
+            dst[s0 ^ 16] = make_uint2(v[0].z, v[0].w);
         }
     };
     // scales and sums: unit i = (q = i / nbl, block i % nbl of the slice) with q = TPAD group + token of the group
