@@ -352,3 +352,42 @@ def test_decode_batch_shares_a_launch_and_keeps_the_bits(be, oxref):
         for i in order:
             got = jobs[i][4].cpu().numpy()
             assert np.array_equal(got.view(np.uint32), alone[i].view(np.uint32)), (order, i, cases[i])
+
+
+def test_decode_batch_events(be, oxref):
+    """Timing events of oxhip_dev_decode_batch: a lone job's launch and a shared launch carry them themselves, jobs of
+    other kernels and split runs get them recorded around; either way the interval is positive and the rows unchanged."""
+    import torch
+    from oxinfer_amd import synth
+    rng = np.random.default_rng(31)
+    raw8, _ = oxref.random_blocks(Q8_0, 96 * 1024 // 32, 5)
+    w8 = be.upload_gguf(Q8_0, raw8, 96, 1024)
+    rawk, _ = oxref.random_blocks(Q4_K, 64 * 2048 // 256, 6)
+    wk = be.upload_gguf(Q4_K, rawk, 64, 2048)
+    q = rng.integers(0, 256, (10, 512 // 2), dtype=np.uint8)
+    sc = np.abs(rng.normal(0, 0.01, (10, 512 // 32))).astype(np.float16).view(np.uint16)
+    w4 = be.upload_q4(q, sc, None, 0, 10, 512)  # the planar kernel, not the matrix-core one
+    assert w8 is not None and wk is not None and w4 is not None, be.last_error()
+    xs = {1024: be.quantize_act(torch.from_numpy(synth.activations(13, 1024, 1)).cuda()),
+          2048: be.quantize_act(torch.from_numpy(synth.activations(13, 2048, 2)).cuda()),
+          512: be.quantize_act(torch.from_numpy(synth.activations(13, 512, 3)).cuda())}
+    cases = [(w8, 1024, 96), (wk, 2048, 64), (w4, 512, 10)]
+    for t in (1, 8, 13):  # 13: two launches for the matrix-core kernels
+        plain = [be.decode(w, xa=xs[k], t=t).cpu().numpy() for w, k, _ in cases]
+        # each job alone, with its own pair of events
+        for (w, k, n), want in zip(cases, plain):
+            y = torch.full((t, n), float("nan"), dtype=torch.float32, device="cuda")
+            e0, e1 = be.event(), be.event()
+            be.decode_batch(be.decode_jobs([(w, xs[k], None, t, y, e0, e1)]))
+            torch.cuda.synchronize()
+            assert be.elapsed_ms(e0, e1) > 0.0
+            assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        # all three in one call (the first two share a launch when t <= 8), events on the first and the last job
+        ys = [torch.full((t, n), float("nan"), dtype=torch.float32, device="cuda") for _, _, n in cases]
+        e0, e1, e2, e3 = be.event(), be.event(), be.event(), be.event()
+        be.decode_batch(be.decode_jobs([(cases[0][0], xs[1024], None, t, ys[0], e0, None), (cases[1][0], xs[2048], None, t, ys[1], None, e1),
+                                        (cases[2][0], xs[512], None, t, ys[2], e2, e3)]))
+        torch.cuda.synchronize()
+        assert be.elapsed_ms(e0, e1) > 0.0 and be.elapsed_ms(e2, e3) > 0.0 and be.elapsed_ms(e0, e3) > 0.0
+        for y, want in zip(ys, plain):
+            assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
