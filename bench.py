@@ -252,6 +252,9 @@ def main():
                     help="copy = a plain 256 MiB device copy, the known-size kernel that scales the HBM traffic counters; "
                          "gguf_stream = every GGUF case alone as a steady stream of 192 matmuls handed over in one call")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--event-every", type=int, default=1,
+                    help="gguf_gemv: the launch of every n-th timed step carries the timing events (with n > 1 the launches run closer "
+                         "together: the whole-job figure rises ~3 %, and a timed launch shares the device with its predecessor's tail)")
     ap.add_argument("--pool-gb", type=float, default=POOL_BYTES / 1e9)
     ap.add_argument("--variant", default="bf16", choices=["bf16", "i8", "fp8"], help="GEMM variant of mlx_gemm / fp8")
     ap.add_argument("--tokens", type=int, default=0, help="tokens of the moe (1 or 256) and fp8 (1, 32, 1024) workloads")
@@ -341,9 +344,13 @@ def main():
     per_step = 1 if shared else len(dom)
     dom_symbol = "decode_batch_kernel"
 
-    # One call per step: the job arrays (one per rotation phase) are built once; the dominant launches carry
-    # HIP events recorded by the library on the launch stream.
-    n_ev = args.steps * per_step
+    # One call per step: the job arrays (one per rotation phase) are built once; the dominant launches of every
+    # `--event-every`-th step (default: every step) carry HIP events recorded by the library on the launch stream. An
+    # event pair on a launch leaves a gap of a few microseconds before the next one; without it a launch starts in the
+    # tail of its predecessor, so its own duration reads longer.
+    every = max(1, args.event_every)
+    n_timed = (args.steps + every - 1) // every
+    n_ev = n_timed * per_step
     ev = [(be.event(), be.event()) for _ in range(min(n_ev, 4096))]
 
     def jobs_for(i, timed_slot=None):
@@ -362,7 +369,7 @@ def main():
         return be.decode_jobs(jobs)
 
     warm = [jobs_for(i) for i in range(args.warmup)]
-    timed = [jobs_for(args.warmup + i, i) for i in range(args.steps)]
+    timed = [jobs_for(args.warmup + i, i // every if i % every == 0 else None) for i in range(args.steps)]
     for arr in warm:
         be.decode_batch(arr)
     torch.cuda.synchronize()
@@ -400,7 +407,8 @@ def main():
         "config": {"workload": "configs[1]: GGUF GEMV batch 1 and 8, Llama-8B MLP shapes 4096->14336 and 14336->4096, "
                                + " + ".join(FMT_NAME[k] for k in kinds),
                    "matmuls_per_step": len(cases), "launches_per_step": 1 if shared else len(cases), "bytes_per_step": step_bytes,
-                   "weight_pool_GB_per_shape": args.pool_gb, "activations": "int8 per 32 (quantize_act), resident in HBM"},
+                   "weight_pool_GB_per_shape": args.pool_gb, "activations": "int8 per 32 (quantize_act), resident in HBM",
+                   "events": f"on the launch of every {every}. step ({min(n_ev, len(ev))} timed launches)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES.get(dom_symbol if all(k in (Q8_0, Q4_K) for k in kinds) else dom_symbol + "/q6k"), "kernel": dom_symbol,
                      "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_avg_s * 1e6, 2)},
