@@ -33,7 +33,7 @@ KERNEL_FMT = {Q8_0: 1, Q4_K: 2, Q6_K: 3}  # template argument in the kernel symb
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # benchmark (KiB per dispatch, FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000: what a 256 MiB device copy
 # reads on the same counters); profiles/decode_batch_kernel_gguf_gemv.md holds the summary.
-TRAFFIC_BYTES = {"decode_batch_kernel": 391421998, "decode_batch_kernel/q6k": 200185872}
+TRAFFIC_BYTES = {"decode_batch_kernel": 391571276, "decode_batch_kernel/q6k": 200196474}
 
 
 def weight_bytes(kind, n_out, n_in):
