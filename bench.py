@@ -7,8 +7,10 @@ the next of a rotating pool of distinct weight copies (>= 1.5 GB per format and 
 Infinity Cache cannot serve them; activations are quantized on the device before the timed region
 (the kernels measured are the dequant-fused GEMVs). value = algorithmic bytes of a step / time.
 
-Prints ONE JSON line (see README / DESIGN.md for the fields). `--workload` selects other
-configurations for profiling runs; the default is what the driver records.
+Prints ONE JSON line: metric / value / unit / ms_per_step and the run's parameters, `roofline` (the dominant
+kernel's algorithmic bytes or flops per launch over its mean duration by HIP events, against the published peak, and
+its measured HBM traffic) and `cpu_baseline` (the CPU restatement on the host cores, a bounded sample). `--workload`
+selects other configurations for profiling runs; the default workload is the headline one.
 """
 import argparse
 import json
@@ -32,7 +34,7 @@ FMT_NAME = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
 KERNEL_FMT = {Q8_0: 1, Q4_K: 2, Q6_K: 3}  # template argument in the kernel symbol
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # benchmark (KiB per dispatch, FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000: what a 256 MiB device copy
-# reads on the same counters); profiles/decode_batch_kernel_gguf_gemv.md holds the summary.
+# reads on the same counters); the summaries of those runs are kept under profiles/.
 TRAFFIC_BYTES = {"decode_batch_kernel": 391571276, "decode_batch_kernel/q6k": 200196474}
 
 
@@ -122,7 +124,7 @@ def timed_steps(torch, step, steps, warmup):
 
 def other_workload(args, be, torch, synth):
     """The other configurations of BASELINE.json, one JSON line each (profiling and per-config numbers; the default
-    workload is what the driver records). Weights rotate over >= pool-gb of distinct copies where HBM bounds."""
+    workload is the headline one). Weights rotate over >= pool-gb of distinct copies where HBM bounds."""
     base = {"metric": METRIC, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "data": "synthetic"}
 
