@@ -184,6 +184,28 @@ def other_workload(args, be, torch, synth):
                               "traffic": None, "kernel": "gemm_bf16_kernel<6, false>" if variant == 0 else "gemm_i8_q4m_kernel",
                               "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3 / 2, 2)})
 
+    if args.workload == "gguf_gemm":                     # configs[1]'s weights at configs[2]'s token count: M = 512, both shapes
+        kind, gen = {"q8_0": (Q8_0, synth.gguf_q8_0), "q4_k": (Q4_K, synth.gguf_q4_k), "q6_k": (Q6_K, synth.gguf_q6_k)}[args.format]
+        shapes = [(14336, 4096), (4096, 14336)]
+        ws, xs = [], []
+        for n, k in shapes:
+            raw = gen(n, k, 3)
+            ws.append([be.upload_gguf(kind, raw, n, k) for _ in range(4)])
+            xs.append(torch.from_numpy(synth.activations(512, k, 4, bf16=True)).cuda().to(torch.bfloat16))
+        flops = sum(2 * 512 * n * k for n, k in shapes)
+
+        def step(i):
+            for j in range(2):
+                be.gemm(ws[j][i % 4], xs[j])
+        wall, ms = timed_steps(torch, step, args.steps, args.warmup)
+        ach = flops / (ms * 1e-3) / 1e12
+        return dict(base, value=round(flops * args.steps / wall / 1e12, 2), unit="TFLOP/s", ms_per_step=round(wall / args.steps * 1e3, 5), dtype="bf16",
+                    config={"workload": f"GGUF {args.format.upper()} prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096 (bf16 matrix cores)",
+                            "flops_per_step": flops, "events": "around the two calls of a step (activation packing + GEMM (+ K-slice sum))"},
+                    roofline={"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK["bf16"], "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK["bf16"], 4),
+                              "traffic": None, "kernel": f"gemm_bf16_kernel<{ {'q8_0': 1, 'q4_k': 2, 'q6_k': 3}[args.format]}, false>",
+                              "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3 / 2, 2)})
+
     if args.workload == "moe":                           # configs[3]: 128 experts, top-8, h = 2048, inter = 768
         ne, k, h, inter = 128, 8, 2048, 768
         t = args.tokens or 1
@@ -250,7 +272,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gguf_gemv", choices=["gguf_gemv", "gguf_gemv_q6k", "gguf_stream", "mlx_gemv", "mlx_gemm", "moe", "fp8", "copy"],
+    ap.add_argument("--workload", default="gguf_gemv", choices=["gguf_gemv", "gguf_gemv_q6k", "gguf_stream", "gguf_gemm", "mlx_gemv", "mlx_gemm", "moe", "fp8", "copy"],
                     help="copy = a plain 256 MiB device copy, the known-size kernel that scales the HBM traffic counters; "
                          "gguf_stream = every GGUF case alone as a steady stream of 192 matmuls handed over in one call")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -259,6 +281,7 @@ def main():
                          "together: the whole-job figure rises ~3 %, and a timed launch shares the device with its predecessor's tail)")
     ap.add_argument("--pool-gb", type=float, default=POOL_BYTES / 1e9)
     ap.add_argument("--variant", default="bf16", choices=["bf16", "i8", "fp8"], help="GEMM variant of mlx_gemm / fp8")
+    ap.add_argument("--format", default="q4_k", choices=["q8_0", "q4_k", "q6_k"], help="weight format of the gguf_gemm workload")
     ap.add_argument("--tokens", type=int, default=0, help="tokens of the moe (1 or 256) and fp8 (1, 32, 1024) workloads")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -96,8 +96,8 @@ size_t oxhip_weight_bytes(const oxhip_weight* w);
 /* Backend::matmul (src/gpu.rs:160; src/cuda.rs:1428-1493): all jobs share x [t, n_in] (host f32);
  * computes every job or none. Routing as matmul_quant_multi_at's (src/kernels.rs:1731-1879): up to 8 tokens the
  * Q8 / Q8_0 / Q4_K / Q6_K / MLX 4-bit jobs share one launch of the int8 decode kernel (the CPU's decode semantics,
- * src/kernels.rs:1908-1928); more than 16 tokens over MLX 4-bit or FP8 (128-column blocks) weights run the bf16
- * matrix-core GEMM; everything else runs the decode kernels over 16 tokens at a time. */
+ * src/kernels.rs:1908-1928); more than 16 tokens over MLX 4-bit, Q8, Q8_0, Q4_K, Q6_K or FP8 (128-column blocks)
+ * weights run the bf16 matrix-core GEMM; everything else runs the decode kernels over 16 tokens at a time. */
 int oxhip_matmul(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_job* jobs, size_t n_jobs);
 /* Backend::matvec_rows (src/gpu.rs:165): t in 1..=4. */
 int oxhip_matvec_rows(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_rows_job* jobs, size_t n_jobs);
@@ -163,7 +163,8 @@ float oxhip_event_elapsed_ms(void* start, void* stop);
 /* Prefill: y [t, n_out] = x [t, n_in] W^T on the matrix cores (what matmul_quant_multi's GEMM paths compute,
  * src/kernels.rs:1774-1847). x_dtype / y_dtype: OXHIP_F32 or OXHIP_BF16. variant:
  *   OXHIP_GEMM_BF16  weights dequantized to bf16 (through LDS), bf16 MFMA, f32 accumulation (the x86 CPU's
- *                    f32 GEMM rounded to bf16 operands); MLX 4-bit weights;
+ *                    f32 GEMM rounded to bf16 operands); MLX 4-bit, Q8, Q8_0, Q4_K and Q6_K weights (the rows
+ *                    that dequantize_row yields, src/ggml.rs:630-793, rounded to bf16);
  *                    also FP8 weights whose rows are multiples of 128 (e4m3 x block scale rounded to bf16);
  *   OXHIP_GEMM_I8    MLX 4-bit weights on the int8 matrix cores: activations quantized per token and block of 32
  *                    as quantize_act does, exact int32 block sums, f32 rescale by the block and activation scales,

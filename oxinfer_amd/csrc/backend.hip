@@ -540,7 +540,7 @@ int oxhip_matmul(oxhip_ctx* c, const float* x, size_t t, size_t n_in, oxhip_job*
             fused.push_back(DecodeBatchItem{w->v, view_of(xa), yd + offs[j], (uint32_t)t});
             continue;
         }
-        const bool gemm = t > 16 && (w->v.fmt == FMT_Q4M || (w->v.fmt == FMT_FP8 && w->v.br % 16 == 0 && w->v.bc % 128 == 0 && n_in % 128 == 0));
+        const bool gemm = t > 16 && gemm_bf16_ok(w->v);
         if (gemm) {
             if (!gemm_bf16_run(c, w, c->x.p, false, t, yd + offs[j], false, s)) {
                 (void)hipStreamSynchronize(s);

@@ -7,9 +7,9 @@ namespace oxhip {
 
 // Packs x and runs the bf16 GEMM; the packed activations live in ctx scratch.
 int gemm_bf16_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf16, size_t t, void* y, bool y_bf16, hipStream_t s) {
-    const bool fp8 = w->v.fmt == FMT_FP8 && w->v.br % 16 == 0 && w->v.bc % 128 == 0 && w->v.n_in % 128 == 0;
-    if (w->v.fmt != FMT_Q4M && !fp8) {
-        set_error("gemm: the bf16 variant runs MLX 4-bit weights and FP8 weights whose rows are multiples of 128");
+    const bool fp8 = w->v.fmt == FMT_FP8;
+    if (!gemm_bf16_ok(w->v)) {
+        set_error("gemm: the bf16 variant runs MLX 4-bit, Q8, Q8_0, Q4_K and Q6_K weights and FP8 weights whose rows are multiples of 128");
         return 0;
     }
     if (fp8 && skinny_fp8_ok(w->v, t)) {  // up to 32 tokens: bandwidth-bound, one pass over the weights
@@ -35,7 +35,7 @@ int gemm_bf16_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf1
             return 0;
         }
     }
-    HIP_TRY(launch_pack_a(x, x_bf16, fp8 ? 2 : 1, t, w->v.n_in, mtiles, kblocks, c->gemm_ws.p, s), "gemm pack launch");
+    HIP_TRY(launch_pack_a(x, x_bf16, gemm_bf16_pack_mode(w->v), t, w->v.n_in, mtiles, kblocks, c->gemm_ws.p, s), "gemm pack launch");
     float* partial = reinterpret_cast<float*>(static_cast<uint8_t*>(c->gemm_ws.p) + pack_bytes);
     HIP_TRY(launch_gemm_bf16(w->v, c->gemm_ws.p, t, mtiles, y, y_bf16, partial, s), "gemm launch");
     return 1;

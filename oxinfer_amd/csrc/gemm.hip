@@ -1,5 +1,6 @@
 // Prefill GEMM, variant (a): weights dequantized to bf16 on the way to the matrix cores, bf16 MFMA with f32
-// accumulation. y[t][n_out] = x[t][n_in] * W^T for the tile-packed MLX 4-bit format.
+// accumulation. y[t][n_out] = x[t][n_in] * W^T for the tile-packed MLX 4-bit, Q8_0 / Q8, Q4_K and Q6_K formats (and
+// FP8 bytes with block scales).
 //
 // The CPU computes this product from the f32-dequantized rows with one fused multiply-add chain per output
 // (matmul_quant_block_prefill + gemm_8x8, src/kernels.rs:1998-2038, src/kernels_x86.rs:296-324 of the reference);
@@ -10,7 +11,9 @@
 //   B (weights): each K-step of 128 the four waves dequantize the step's 8 row tiles (two each) from the packed
 //     records into bf16 MFMA fragments in LDS (double-buffered, one barrier per step); every wave then reads all
 //     8 x 4 fragments with ds_read_b128. A weight is dequantized once per workgroup: (code - 8) * d + offset in
-//     f32 as one fma(code, d, offset - 8 d), rounded to bf16.
+//     f32 as one fma(code, d, offset - 8 d), rounded to bf16. The GGUF formats likewise, from their own records:
+//     Q8_0 q * d, Q4_K (d * sc) * nibble - dmin * mn, Q6_K (d * sc) * (code - 32) (dequantize_row, src/ggml.rs:707-793
+//     of the reference), each as one fma over the unsigned code.
 //   A (activations): packed beforehand (pack_a_kernel) into MFMA fragments, one 1 KiB record per (16 tokens,
 //     block of 32) in the K order the weight fragments use, so a wave fetches its fragment with one coalesced
 //     16-byte-per-lane load straight from global memory / L2, a block ahead of its use.
@@ -28,6 +31,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // 16 mtile + m at K positions 32 b + 4 kq + {0..3} then 32 b + 16 + 4 kq + {0..3} (SPLIT, the order of the
 // nibble pairs of Q4 bytes) or 32 b + 8 kq + {0..7}. Tokens past t and columns past n_in are zero.
 // MODE 2 (FP8 weights read 32 row bytes per lane): block kb = 4 s + b of step s holds columns 128 s + 32 kq + 8 b + j.
+// MODE 3 (Q6_K records: a lane owns 16 consecutive columns of each half step): block kb = 4 s + 2 h + e holds columns
+// 128 s + 64 h + 16 kq + 8 e + j.
 template <int MODE, bool SRC_BF16>
 __global__ __launch_bounds__(256) void pack_a_kernel(const void* __restrict__ x, uint32_t t, uint32_t n_in, uint32_t mtiles,
                                                      uint32_t kblocks, uint4* __restrict__ out) {
@@ -40,7 +45,10 @@ __global__ __launch_bounds__(256) void pack_a_kernel(const void* __restrict__ x,
     if (tok < t) {
         // the lane's 8 values are two runs of 4 consecutive columns (SPLIT) or one run of 8: whole runs are fetched with
         // one 8- or 16-byte request each (rows are multiples of 8 columns here), a ragged tail value by value
-        const uint32_t k0 = MODE == 1 ? 32 * b + 4 * kq : MODE == 2 ? 128 * (b >> 2) + 32 * kq + 8 * (b & 3) : 32 * b + 8 * kq;
+        const uint32_t k0 = MODE == 1   ? 32 * b + 4 * kq
+                            : MODE == 2 ? 128 * (b >> 2) + 32 * kq + 8 * (b & 3)
+                            : MODE == 3 ? 128 * (b >> 2) + 64 * ((b >> 1) & 1) + 16 * kq + 8 * (b & 1)
+                                        : 32 * b + 8 * kq;
         const uint32_t k1 = MODE == 1 ? k0 + 16 : k0 + 4;  // first column of the second run of 4
         const size_t row = (size_t)tok * n_in;
         if (k1 + 4 <= n_in && n_in % 8 == 0) {
@@ -88,12 +96,19 @@ hipError_t launch_pack_a(const void* x, bool src_bf16, int mode, size_t t, size_
     } else if (mode == 2) {
         if (src_bf16) pack_a_kernel<2, true><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
         else pack_a_kernel<2, false><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
+    } else if (mode == 3) {
+        if (src_bf16) pack_a_kernel<3, true><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
+        else pack_a_kernel<3, false><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
     } else {
         if (src_bf16) pack_a_kernel<0, true><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
         else pack_a_kernel<0, false><<<grid, 256, 0, s>>>(x, tt, kk, mt, kb, o);
     }
     return hipGetLastError();
 }
+
+#ifndef OXHIP_GEMM_EARLY_RAW
+#define OXHIP_GEMM_EARLY_RAW 1
+#endif
 
 namespace {
 
@@ -108,10 +123,8 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
 }
 
-// One dword of a T4M chunk (4 bytes of one block: low nibbles = elements 4 kq + i, high = 16 + 4 kq + i) -> the
-// lane's 8 bf16 of that block.
-__device__ __forceinline__ uint4 dequant_q4m(uint32_t w, float d, float c) {
-    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+// Eight unsigned byte codes (the bytes of lo, then of hi) -> 8 bf16 of code * d + c.
+__device__ __forceinline__ uint4 dequant_u8x8(uint32_t lo, uint32_t hi, float d, float c) {
     float f[8];
     f[0] = __builtin_fmaf((float)(lo & 0xFF), d, c);
     f[1] = __builtin_fmaf((float)((lo >> 8) & 0xFF), d, c);
@@ -123,6 +136,11 @@ __device__ __forceinline__ uint4 dequant_q4m(uint32_t w, float d, float c) {
     f[7] = __builtin_fmaf((float)(hi >> 24), d, c);
     return make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
 }
+// One dword of a T4M chunk (4 bytes of one block: low nibbles = elements 4 kq + i, high = 16 + 4 kq + i) -> the
+// lane's 8 bf16 of that block.
+__device__ __forceinline__ uint4 dequant_q4m(uint32_t w, float d, float c) {
+    return dequant_u8x8(w & 0x0F0F0F0Fu, (w >> 4) & 0x0F0F0F0Fu, d, c);
+}
 
 }  // namespace
 
@@ -130,7 +148,7 @@ __device__ __forceinline__ uint4 dequant_q4m(uint32_t w, float d, float c) {
 // kblocks = 4 * steps. OUT_BF16: y is bf16 [t][n_out], else f32.
 // With gridDim.z > 1 the K-steps are split over z and each slice writes its partial sums as f32 to
 // yv + z * t * n_out (a second kernel adds the slices in order).
-// FMT: FMT_Q4M (tile-packed MLX 4-bit) or FMT_FP8 (row-major e4m3 bytes with 128 x 128 block scales: the bytes are
+// FMT: FMT_Q4M (tile-packed MLX 4-bit), FMT_Q8_0 / FMT_Q8F / FMT_Q4_K / FMT_Q6_K (their tile records) or FMT_FP8 (e4m3 bytes with 128 x 128 block scales: the bytes are
 // exact in bf16, the block scale multiplies in f32 before the rounding, and a lane takes 32 consecutive row bytes
 // per step, which pack_a's mode 2 mirrors on the activation side).
 template <int FMT, bool OUT_BF16>
@@ -155,6 +173,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
         const uint32_t tile = min(nt0 + 2 * wave + i, ntiles - 1);
         if (FMT == FMT_Q4M) {
             wbase[i] = w.p0 + ((size_t)tile * all_steps + step0) * T4M_REC;
+        } else if (q8_format(FMT)) {  // the tile's records; load_raw indexes them from the matrix's first step
+            wbase[i] = w.p0 + (size_t)tile * t8_steps(w.n_in) * (FMT == FMT_Q8F ? T8F_REC : T8_REC);
+        } else if (FMT == FMT_Q4_K) {
+            wbase[i] = w.p0 + (size_t)tile * tk4_sbs(w.n_in) * TK4_REC;
+        } else if (FMT == FMT_Q6_K) {
+            wbase[i] = w.p0 + (size_t)tile * t6k_steps(w.n_in) * T6K_REC;
         } else {
             const uint32_t row = min(tile * 16 + n, w.n_out - 1);
             wbase[i] = w.p0 + fp8_offset(w, row, 128 * (size_t)step0 + 32 * (lane >> 4));
@@ -173,38 +197,110 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
         for (int j = 0; j < WG_NT; j++) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
     struct Raw {
-        uint4 c, c2;      // Q4M: one chunk; FP8: 32 row bytes
-        uint32_t dd, oo;  // Q4M: scales, offsets; FP8: dd = the block scale's bits
+        uint4 c, c2;    // Q4M, Q4_K: one chunk; Q8: the chunks of the step's two records; Q6_K: low nibbles, high bit pairs; FP8: 32 row bytes
+        uint32_t m[4];  // the row's scale words (Q4M: scales, offsets; FP8: the block scale's bits)
     };
-    auto load_raw = [&](Raw* r, uint32_t s) {
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
+    auto load_raw_tile = [&](Raw* r, int i, uint32_t s) {  // the records of the wave's row tile i at step s
+        {
             if (FMT == FMT_Q4M) {
                 const uint8_t* rec = wbase[i] + (size_t)s * T4M_REC;
                 r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
-                r[i].dd = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
-                r[i].oo = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
+                r[i].m[0] = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
+                r[i].m[1] = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
+            } else if (q8_format(FMT)) {  // a step of 128 columns is two records of 64 (past the row's last record: that one again,
+                                          // which dequant_tile zeroes: nothing here may depend on a loaded value, or the request
+                                          // would be waited for where it is made)
+                constexpr uint32_t REC = FMT == FMT_Q8F ? T8F_REC : T8_REC;
+                const uint32_t nrec = t8_steps(w.n_in);
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const uint8_t* rec = wbase[i] + (size_t)min(2 * (step0 + s) + h, nrec - 1) * REC;
+                    const uint4 v = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+                    if (h) r[i].c2 = v;
+                    else r[i].c = v;
+                    if (FMT == FMT_Q8F) {
+                        const uint2 sc = *reinterpret_cast<const uint2*>(rec + 1024 + 8 * n);
+                        r[i].m[2 * h] = sc.x;
+                        r[i].m[2 * h + 1] = sc.y;
+                    } else {
+                        r[i].m[h] = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
+                    }
+                }
+            } else if (FMT == FMT_Q4_K) {  // half a super-block record: sub-blocks 4 (sa & 1) .. + 3
+                const uint32_t sa = step0 + s;
+                const uint8_t* rec = wbase[i] + (size_t)(sa >> 1) * TK4_REC;
+                r[i].c = *reinterpret_cast<const uint4*>(rec + (sa & 1) * 1024 + 16 * lane);
+                r[i].m[0] = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 4 * (sa & 1));
+                r[i].m[1] = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 8 + 4 * (sa & 1));
+                r[i].m[2] = *reinterpret_cast<const uint32_t*>(rec + 2304 + 4 * n);
+            } else if (FMT == FMT_Q6_K) {
+                const uint8_t* rec = wbase[i] + (size_t)(step0 + s) * T6K_REC;
+                r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+                const uint2 hb = *reinterpret_cast<const uint2*>(rec + 1024 + 8 * lane);
+                r[i].c2.x = hb.x;
+                r[i].c2.y = hb.y;
+                const uint2 sc = *reinterpret_cast<const uint2*>(rec + 1536 + 8 * n);
+                r[i].m[0] = sc.x;
+                r[i].m[1] = sc.y;
+                r[i].m[2] = *reinterpret_cast<const uint16_t*>(rec + 1664 + 2 * n);
             } else {
                 const uint8_t* p = wbase[i] + (w.group == 1 ? 2048 : 128) * (size_t)s;
                 r[i].c = *reinterpret_cast<const uint4*>(p);
                 r[i].c2 = *reinterpret_cast<const uint4*>(p + 16);
-                r[i].dd = __float_as_uint(sbase[i][(128 * s) / w.bc]);
+                r[i].m[0] = __float_as_uint(sbase[i][(128 * s) / w.bc]);
             }
         }
     };
-    auto dequant_tile = [&](const Raw& r, int i, uint32_t buf) {  // one of the wave's two row tiles, 4 blocks
+    auto load_raw = [&](Raw* r, uint32_t s) {
+        load_raw_tile(r, 0, s);
+        load_raw_tile(r, 1, s);
+    };
+    // `s`: the step the records belong to (of this slice)
+    auto dequant_tile = [&](const Raw& r, int i, uint32_t buf, uint32_t s) {  // one of the wave's two row tiles, 4 blocks
+        uint4* dst = bfrag + ((size_t)(buf * 4) * WG_NT + 2 * wave + i) * 64 + lane;  // block b: + b * WG_NT * 64
         if (FMT == FMT_Q4M) {
             const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
             for (int b = 0; b < 4; b++) {
                 const int g = b >> 1;
-                const float d = f16_bits_to_f32((uint16_t)(g ? r.dd >> 16 : r.dd & 0xFFFF));
-                const float off = bf16_bits_to_f32((uint16_t)(g ? r.oo >> 16 : r.oo & 0xFFFF));
-                bfrag[((buf * 4 + b) * WG_NT + 2 * wave + i) * 64 + lane] = dequant_q4m(cw[b], d, off - 8.0f * d);
+                const float d = f16_bits_to_f32((uint16_t)(g ? r.m[0] >> 16 : r.m[0] & 0xFFFF));
+                const float off = bf16_bits_to_f32((uint16_t)(g ? r.m[1] >> 16 : r.m[1] & 0xFFFF));
+                dst[b * WG_NT * 64] = dequant_q4m(cw[b], d, off - 8.0f * d);
+            }
+        } else if (q8_format(FMT)) {  // block b = 2 h + e: codes 8 kq .. + 7 of block e of record h; q * d as (q + 128) * d - 128 d
+            const uint32_t cw[8] = {r.c.x, r.c.y, r.c.z, r.c.w, r.c2.x, r.c2.y, r.c2.z, r.c2.w};
+            const bool past = 2 * (step0 + s) + 1 >= t8_steps(w.n_in);  // the step's second record lies past the row
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const int h = b >> 1, e = b & 1;
+                float d = FMT == FMT_Q8F ? __uint_as_float(r.m[b]) : f16_bits_to_f32((uint16_t)(e ? r.m[h] >> 16 : r.m[h] & 0xFFFF));
+                if (h && past) d = 0.0f;
+                dst[b * WG_NT * 64] = dequant_u8x8(cw[2 * b] ^ 0x80808080u, cw[2 * b + 1] ^ 0x80808080u, d, -128.0f * d);
+            }
+        } else if (FMT == FMT_Q4_K) {  // block b = 2 jj + e: the low (e = 0) or high nibbles of the chunk's byte pair jj
+            const float d = f16_bits_to_f32((uint16_t)(r.m[2] & 0xFFFF)), dmin = f16_bits_to_f32((uint16_t)(r.m[2] >> 16));
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const int jj = b >> 1, e = b & 1;
+                const uint32_t lo = jj ? r.c.z : r.c.x, hi = jj ? r.c.w : r.c.y;
+                const float sc = (float)((r.m[0] >> (8 * b)) & 0xFF), mn = (float)((r.m[1] >> (8 * b)) & 0xFF);
+                dst[b * WG_NT * 64] = dequant_u8x8((lo >> (4 * e)) & 0x0F0F0F0Fu, (hi >> (4 * e)) & 0x0F0F0F0Fu, d * sc, -(dmin * mn));
+            }
+        } else if (FMT == FMT_Q6_K) {  // block b = 2 h + e: codes 8 e .. + 7 of the lane's 16 columns of half h
+            const float d = f16_bits_to_f32((uint16_t)(r.m[2] & 0xFFFF));
+            const uint32_t kq = lane >> 4;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const int h = b >> 1, e = b & 1;
+                const uint32_t src = e ? (h ? r.c.w : r.c.y) : (h ? r.c.z : r.c.x), hh = (h ? r.c2.y : r.c2.x) >> (4 * e);
+                const uint32_t w0 = (src & 0x0F0F0F0Fu) | ((hh & 0x03030303u) << 4);
+                const uint32_t w1 = ((src >> 4) & 0x0F0F0F0Fu) | (((hh >> 2) & 0x03030303u) << 4);
+                const float dsc = d * (float)(int)(int8_t)((r.m[h] >> (8 * kq)) & 0xFF);
+                dst[b * WG_NT * 64] = dequant_u8x8(w0, w1, dsc, -32.0f * dsc);
             }
         } else {
             const uint32_t cw[8] = {r.c.x, r.c.y, r.c.z, r.c.w, r.c2.x, r.c2.y, r.c2.z, r.c2.w};
-            const float sc = __uint_as_float(r.dd);
+            const float sc = __uint_as_float(r.m[0]);
 #pragma unroll
             for (int b = 0; b < 4; b++) {  // bytes 8 b .. 8 b + 7 of the lane's 32
                 const f32x2 v0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)cw[2 * b], false);
@@ -213,7 +309,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
                 const f32x2 v3 = __builtin_amdgcn_cvt_pk_f32_fp8((int)cw[2 * b + 1], true);
                 const uint32_t o[4] = {pack_bf16(v0.x * sc, v0.y * sc), pack_bf16(v1.x * sc, v1.y * sc),
                                        pack_bf16(v2.x * sc, v2.y * sc), pack_bf16(v3.x * sc, v3.y * sc)};
-                bfrag[((buf * 4 + b) * WG_NT + 2 * wave + i) * 64 + lane] = make_uint4(o[0], o[1], o[2], o[3]);
+                dst[b * WG_NT * 64] = make_uint4(o[0], o[1], o[2], o[3]);
             }
         }
     };
@@ -232,14 +328,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     // memory a whole K-step (four blocks, ~2000 MFMA cycles) ahead; the packed records of the next step two blocks
     // before they are dequantized into the other LDS buffer. Each fragment has one home, refilled in place right after
     // its last use.
+    constexpr bool EARLY_RAW = OXHIP_GEMM_EARLY_RAW;
     Raw raw[2];
     load_raw(raw, 0);
     uint4 a_cur[AR][4], b_cur[WG_NT];
     const uint32_t last = nsteps - 1, last_blk = 4 * nsteps - 1;
 #pragma unroll
     for (int b = 0; b < AR; b++) read_a(a_cur[b], min((uint32_t)b, last_blk));
-    dequant_tile(raw[0], 0, 0);
-    dequant_tile(raw[1], 1, 0);
+    dequant_tile(raw[0], 0, 0, 0);
+    dequant_tile(raw[1], 1, 0, 0);
     load_raw(raw, min(1u, last));
     lds_barrier();
     read_b(b_cur, 0, 0);
@@ -262,9 +359,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
                 else b_cur[j] = bfrag[(((buf ^ 1) * 4) * WG_NT + j) * 64 + lane];
             }
             read_a(a_cur[b % AR], min(4 * s + b + AR, last_blk));
-            if (b == 0) dequant_tile(raw[0], 0, buf ^ 1);
-            if (b == 1) dequant_tile(raw[1], 1, buf ^ 1);
-            if (b == 2) load_raw(raw, min(s + 2, last));
+            if (EARLY_RAW) {  // a tile's records of the step after next are requested as soon as its registers are free
+                if (b < 2) {
+                    dequant_tile(raw[b], b, buf ^ 1, min(s + 1, last));
+                    load_raw_tile(raw, b, min(s + 2, last));
+                }
+            } else {
+                if (b == 0) dequant_tile(raw[0], 0, buf ^ 1, min(s + 1, last));
+                if (b == 1) dequant_tile(raw[1], 1, buf ^ 1, min(s + 1, last));
+                if (b == 2) load_raw(raw, min(s + 2, last));
+            }
         }
     }
     // D[token 4 kq + r][row n] per tile
@@ -343,12 +447,27 @@ hipError_t launch_gemm_reduce(const float* partial, size_t n, uint32_t slices, v
 }
 
 // `partial`: scratch of slices * t * n_out floats when gemm_k_slices() > 1.
+// The formats the kernel dequantizes: tile-packed MLX 4-bit, Q8_0 / Q8, Q4_K, Q6_K, and FP8 rows of whole 128-column
+// steps with scale blocks of 16 k rows x 128 k columns.
+bool gemm_bf16_ok(const WeightView& w) {
+    if (w.fmt == FMT_Q4M || q8_format(w.fmt)) return true;
+    if (w.fmt == FMT_Q4_K || w.fmt == FMT_Q6_K) return w.n_in % 256 == 0;
+    return w.fmt == FMT_FP8 && w.br % 16 == 0 && w.bc % 128 == 0 && w.n_in % 128 == 0;
+}
+// pack_a's MODE for the format's fragments
+int gemm_bf16_pack_mode(const WeightView& w) { return w.fmt == FMT_Q4M ? 1 : w.fmt == FMT_FP8 ? 2 : w.fmt == FMT_Q6_K ? 3 : 0; }
+
 hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                             hipStream_t s) {
-    if (w.fmt == FMT_Q4M) return run_gemm_bf16<FMT_Q4M>(w, apk, t, mtiles, y, out_bf16, partial, s);
-    if (w.fmt == FMT_FP8 && w.br % 16 == 0 && w.bc % 128 == 0 && w.n_in % 128 == 0)
-        return run_gemm_bf16<FMT_FP8>(w, apk, t, mtiles, y, out_bf16, partial, s);
-    return hipErrorInvalidValue;
+    if (!gemm_bf16_ok(w)) return hipErrorInvalidValue;
+    switch (w.fmt) {
+        case FMT_Q4M: return run_gemm_bf16<FMT_Q4M>(w, apk, t, mtiles, y, out_bf16, partial, s);
+        case FMT_Q8_0: return run_gemm_bf16<FMT_Q8_0>(w, apk, t, mtiles, y, out_bf16, partial, s);
+        case FMT_Q8F: return run_gemm_bf16<FMT_Q8F>(w, apk, t, mtiles, y, out_bf16, partial, s);
+        case FMT_Q4_K: return run_gemm_bf16<FMT_Q4_K>(w, apk, t, mtiles, y, out_bf16, partial, s);
+        case FMT_Q6_K: return run_gemm_bf16<FMT_Q6_K>(w, apk, t, mtiles, y, out_bf16, partial, s);
+        default: return run_gemm_bf16<FMT_FP8>(w, apk, t, mtiles, y, out_bf16, partial, s);
+    }
 }
 
 }  // namespace oxhip

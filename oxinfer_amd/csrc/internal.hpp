@@ -119,6 +119,8 @@ hipError_t launch_q4_scale_groups(const uint16_t* sc32, size_t n_out, size_t n_i
 hipError_t launch_pack_a(const void* x, bool src_bf16, int mode, size_t t, size_t n_in, size_t mtiles, size_t kblocks, void* out,
                          hipStream_t s);
 uint32_t gemm_k_slices(const WeightView& w, size_t mtiles);
+bool gemm_bf16_ok(const WeightView& w);        // the bf16 matrix-core GEMM dequantizes this weight's format and shape
+int gemm_bf16_pack_mode(const WeightView& w);  // launch_pack_a's mode for its activation fragments
 // decode_fp8.hip: FP8 weights at up to 32 tokens on the bf16 matrix cores
 bool skinny_fp8_ok(const WeightView& w, size_t t);
 size_t skinny_fp8_pack_bytes(const WeightView& w, size_t t, int planes);

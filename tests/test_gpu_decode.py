@@ -267,17 +267,28 @@ def test_fp8_rows_scale_blocks(oxref, be):
 
 
 def test_host_matmul_matches_device_path_and_declines(be, oxref):
+    from oxinfer_amd import synth
     n_in = 512
     raws = [(k, n, oxref.random_blocks(k, n * n_in // oxref.block_size(k), 31 + k)[0]) for k, n in ((Q4_K, 24), (Q6_K, 8), (Q8_0, 40))]
     ws = [be.upload_gguf(k, raw, n, n_in) for k, n, raw in raws]
-    for t in (1, 3, 9, 16, 17, 40):   # up to 8 tokens the Q4_K and Q8_0 jobs share a launch; past 16 the rows go in slices
+    # up to 8 tokens the Q4_K and Q8_0 jobs share a launch; 9 to 16 run the decode kernels; past 16 every format takes
+    # the prefill GEMM on the exact rows, as the CPU does past its decode limit (src/kernels.rs:1774-1847): bf16 matrix
+    # cores, 2e-2 of the f32 product
+    for t in (1, 3, 9, 16, 17, 40):
         x = lcg_input(t, n_in, 40 + t, oxref)
         ys = [np.full((t, n), np.nan, np.float32) for _, n, _ in raws]
         assert be.matmul(x, t, n_in, list(zip(ws, ys))), be.last_error()
         for (k, n, raw), y in zip(raws, ys):
-            assert row_err(y, oxref.gguf_decode(k, raw, n, n_in, x, t)) < TOL
-    # more than 16 tokens over MLX 4-bit and FP8 weights take the prefill GEMM (bf16 matrix cores: 2e-2 of the f32 product)
-    from oxinfer_amd import synth
+            if t <= 16:
+                assert row_err(y, oxref.gguf_decode(k, raw, n, n_in, x, t)) < TOL
+            else:  # (a token has as few as 8 outputs here, all of which may cancel: the bound is on the terms' size)
+                wf = oxref.dequantize_rows(k, raw, n, n_in)
+                terms = (np.abs(x).astype(np.float64) @ np.abs(wf).astype(np.float64).T).max(axis=1)
+                ref = oxref.gemm_quant(k, raw, None, None, n, n_in, x, t)
+                assert float((np.abs(y - ref).max(axis=1) / terms).max()) < 2e-2 / 8
+                xb, wb = synth.bf16_round(x).astype(np.float64), synth.bf16_round(wf).astype(np.float64)
+                assert row_err(y, (xb @ wb.T).astype(np.float32)) < TOL
+    # and so do MLX 4-bit and FP8 weights
     t, n_out = 40, 48
     wq, sc, bi = synth.mlx_q4(n_out, n_in, 3)
     q, s16, off = oxref.from_mlx_q4(wq, sc, bi, n_out, n_in, 64)

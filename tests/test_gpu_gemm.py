@@ -66,6 +66,93 @@ def test_gemm_bf16_row_magnitudes_and_f32_inputs(be, oxref):
     assert row_err(y, ref) < 2e-2
 
 
+GGUF_KINDS = {"Q8_0": 8, "Q4_K": 12, "Q6_K": 14}
+
+
+def gguf_raw(name, n_out, n_in, seed):
+    from oxinfer_amd import synth
+    return {"Q8_0": synth.gguf_q8_0, "Q4_K": synth.gguf_q4_k, "Q6_K": synth.gguf_q6_k}[name](n_out, n_in, seed)
+
+
+# 4352 columns = 34 steps of 128: K slices of 9 steps, so slices start inside a Q4_K super-block record; 1120 and 96
+# columns (Q8_0 only): a last step of one record, and of one block
+@pytest.mark.parametrize("name,n_out,n_in", [(k, n, c) for k in GGUF_KINDS for n, c in ((37, 1024), (256, 512), (200, 256), (130, 4352))]
+                         + [("Q8_0", 100, 96), ("Q8_0", 64, 1120)])
+def test_gemm_bf16_gguf_matches_oracle(be, oxref, name, n_out, n_in):
+    """The GGUF formats on the bf16 matrix cores: within 2e-2 of the CPU's prefill product over the rows that
+    dequantize_row yields (src/ggml.rs:630-793, src/kernels.rs:1998-2038), and 1e-3 of the same product with both
+    operands rounded to bf16, which is what the kernel computes."""
+    import torch
+    from oxinfer_amd import synth
+    kind = GGUF_KINDS[name]
+    raw = gguf_raw(name, n_out, n_in, 17)
+    w = be.upload_gguf(kind, raw, n_out, n_in)
+    assert w is not None, be.last_error()
+    wb = synth.bf16_round(oxref.dequantize_rows(kind, raw, n_out, n_in)).astype(np.float64)
+    for t in (1, 16, 37, 150, 300, 513):
+        x = synth.activations(t, n_in, 200 + t, bf16=True)
+        ref = oxref.gemm_quant(kind, raw, None, None, n_out, n_in, x, t)
+        exact_bf16 = (x.astype(np.float64) @ wb.T).astype(np.float32)
+        for xd in (torch.from_numpy(x).cuda(), torch.from_numpy(x).cuda().to(torch.bfloat16)):
+            y = be.gemm(w, xd).cpu().numpy()
+            assert row_err(y, ref) < 2e-2, (t, xd.dtype)
+            assert row_err(y, exact_bf16) < 1e-3, (t, xd.dtype)
+    yb = be.gemm(w, torch.from_numpy(x).cuda(), out_bf16=True).float().cpu().numpy()
+    assert row_err(yb, ref) < 2e-2
+
+
+def test_gemm_bf16_gguf_reference_fixtures(be, oxref):
+    """The reference's own block fixtures (random_blocks, src/ggml.rs:1446-1496: every bit pattern of codes and packed
+    scales, signed Q6_K scales, d of either sign) through the GEMM."""
+    import torch
+    from oxinfer_amd import synth
+    n_out, n_in, t = 48, 1024, 64
+    for kind in GGUF_KINDS.values():
+        raw = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 77 + kind)[0]
+        w = be.upload_gguf(kind, raw, n_out, n_in)
+        wb = synth.bf16_round(oxref.dequantize_rows(kind, raw, n_out, n_in)).astype(np.float64)
+        x = synth.activations(t, n_in, 78, bf16=True)
+        y = be.gemm(w, torch.from_numpy(x).cuda()).cpu().numpy()
+        assert row_err(y, (x.astype(np.float64) @ wb.T).astype(np.float32)) < 1e-3, kind
+        assert row_err(y, oxref.gemm_quant(kind, raw, None, None, n_out, n_in, x, t)) < 2e-2, kind
+
+
+@pytest.mark.parametrize("n_out,n_in", [(40, 640), (130, 96)])
+def test_gemm_bf16_q8_matrix_matches_oracle(be, oxref, n_out, n_in):
+    """QMatrix (int8 codes, f32 scale per 32; src/quant.rs:128-133) through the same kernel."""
+    import torch
+    from oxinfer_amd import synth
+    q, sc = synth.q8_matrix(n_out, n_in, 23)
+    w = be.upload_q8(q, sc, n_out, n_in)
+    assert w is not None, be.last_error()
+    wf = oxref.q8_dequant_rows(q, sc, n_out, n_in)
+    for t in (17, 260):
+        x = synth.activations(t, n_in, 300 + t, bf16=True)
+        y = be.gemm(w, torch.from_numpy(x).cuda()).cpu().numpy()
+        assert row_err(y, oxref.gemm_f32(wf, n_out, n_in, x, t)) < 2e-2
+        assert row_err(y, (x.astype(np.float64) @ synth.bf16_round(wf).astype(np.float64).T).astype(np.float32)) < 1e-3
+
+
+@pytest.mark.parametrize("name", list(GGUF_KINDS))
+def test_gemm_gguf_full_size_sampled_rows(be, oxref, name):
+    """The Llama-8B MLP shape 512 x 4096 -> 14336 with GGUF weights: a sample of output rows against the oracle."""
+    import torch
+    from oxinfer_amd import synth
+    n_out, n_in, t = 14336, 4096, 512
+    kind = GGUF_KINDS[name]
+    raw = gguf_raw(name, n_out, n_in, 13)
+    w = be.upload_gguf(kind, raw, n_out, n_in)
+    assert w is not None, be.last_error()
+    x = synth.activations(t, n_in, 14, bf16=True)
+    y = be.gemm(w, torch.from_numpy(x).cuda().to(torch.bfloat16)).cpu().numpy()
+    rows = np.r_[0:4, 7165:7171, n_out - 4:n_out, np.random.default_rng(1).integers(0, n_out, 18)]
+    rb = oxref.row_bytes(kind, n_in)
+    sub = np.concatenate([raw[r * rb:(r + 1) * rb] for r in rows])
+    ref = oxref.gemm_quant(kind, sub, None, None, len(rows), n_in, x, t)
+    m = np.maximum(np.abs(y).max(axis=1), 1e-30)
+    assert float((np.abs(y[:, rows] - ref).max(axis=1) / m).max()) < 2e-2
+
+
 def test_gemm_full_size_sampled_rows(be, oxref):
     """The benchmark shape 512 x 4096 -> 14336: a sample of output rows against the oracle."""
     import torch
