@@ -192,7 +192,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     const uint32_t per = (S1 - S0 + kw - 1) >> kwsh;
     const uint32_t s0 = S0 + ks * per;
     const uint32_t s1 = tile < ntiles ? min(S1, s0 + per) : 0;  // a tile past the matrix streams nothing
-    const uint8_t* base = w.p0 + (size_t)min(tile, ntiles - 1) * (FMT == FMT_Q8_0   ? (size_t)nsteps * T8_REC
+    // (typed as global memory: a grouped launch reads w.p0 from the table of expert bases)
+    const gbytes base = as_global(w.p0) + (size_t)min(tile, ntiles - 1) * (FMT == FMT_Q8_0   ? (size_t)nsteps * T8_REC
                                                                   : FMT == FMT_Q8F  ? (size_t)nsteps * T8F_REC
                                                                   : FMT == FMT_Q4_K ? (size_t)(nsteps / 2) * TK4_REC
                                                                   : FMT == FMT_Q6_K ? (size_t)nsteps * T6K_REC
@@ -205,24 +206,24 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     };
     auto load_step = [&](Step<FMT>& st, uint32_t s) {
         if constexpr (q8_format(FMT)) {
-            const uint8_t* rec = base + (size_t)s * (FMT == FMT_Q8F ? T8F_REC : T8_REC);
-            st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+            const gbytes rec = base + (size_t)s * (FMT == FMT_Q8F ? T8F_REC : T8_REC);
+            st.w = gload<uint4>(rec + 16 * lane);
             if (!ALDS) act2(2 * s + a_half, 8 * kq, st.a);
         } else if constexpr (FMT == FMT_Q4_K) {
-            const uint8_t* rec = base + (size_t)(s >> 1) * TK4_REC;
-            st.w = *reinterpret_cast<const uint4*>(rec + (s & 1) * 1024 + 16 * lane);
+            const gbytes rec = base + (size_t)(s >> 1) * TK4_REC;
+            st.w = gload<uint4>(rec + (s & 1) * 1024 + 16 * lane);
             if (!ALDS) {
                 act2(4 * s + a_half, 8 * kq, st.a);
                 act2(4 * s + 2 + a_half, 8 * kq, st.a + 2);
             }
         } else if constexpr (FMT == FMT_Q6_K) {
             static_assert(FMT != FMT_Q6_K || ALDS, "Q6_K takes its activations from LDS");
-            const uint8_t* rec = base + (size_t)s * T6K_REC;
-            st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
-            st.h = *reinterpret_cast<const uint2*>(rec + 1024 + 8 * lane);
+            const gbytes rec = base + (size_t)s * T6K_REC;
+            st.w = gload<uint4>(rec + 16 * lane);
+            st.h = gload<uint2>(rec + 1024 + 8 * lane);
         } else {
-            const uint8_t* rec = base + (size_t)s * T4M_REC;
-            st.w = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+            const gbytes rec = base + (size_t)s * T4M_REC;
+            st.w = gload<uint4>(rec + 16 * lane);
             if (!ALDS) {
 #pragma unroll
                 for (int g = 0; g < 2; g++) {  // positions 4 kq.. and 16 + 4 kq.. of block 4 s + 2 g + half
@@ -244,24 +245,24 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     auto load_scales = [&](uint32_t* m, uint32_t first) {
         const uint32_t s = min(first + kq, slast);
         if constexpr (FMT == FMT_Q8F) {
-            m[0] = *reinterpret_cast<const uint32_t*>(base + (size_t)s * T8F_REC + 1024 + 8 * n);
-            m[1] = *reinterpret_cast<const uint32_t*>(base + (size_t)s * T8F_REC + 1028 + 8 * n);
+            m[0] = gload<uint32_t>(base + (size_t)s * T8F_REC + 1024 + 8 * n);
+            m[1] = gload<uint32_t>(base + (size_t)s * T8F_REC + 1028 + 8 * n);
         } else if constexpr (FMT == FMT_Q8_0) {
-            m[0] = *reinterpret_cast<const uint32_t*>(base + (size_t)s * T8_REC + 1024 + 4 * n);
+            m[0] = gload<uint32_t>(base + (size_t)s * T8_REC + 1024 + 4 * n);
         } else if constexpr (FMT == FMT_Q4_K) {
-            const uint8_t* rec = base + (size_t)(s >> 1) * TK4_REC;
-            m[0] = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 4 * (s & 1));
-            m[1] = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
-            m[2] = *reinterpret_cast<const uint32_t*>(rec + 2304 + 4 * n);
+            const gbytes rec = base + (size_t)(s >> 1) * TK4_REC;
+            m[0] = gload<uint32_t>(rec + 2048 + 16 * n + 4 * (s & 1));
+            m[1] = gload<uint32_t>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
+            m[2] = gload<uint32_t>(rec + 2304 + 4 * n);
         } else if constexpr (FMT == FMT_Q6_K) {  // {scales of sub-blocks 0..3, of 4..7, d}
-            const uint8_t* rec = base + (size_t)s * T6K_REC;
-            m[0] = *reinterpret_cast<const uint32_t*>(rec + 1536 + 8 * n);
-            m[1] = *reinterpret_cast<const uint32_t*>(rec + 1540 + 8 * n);
-            m[2] = *reinterpret_cast<const uint16_t*>(rec + 1664 + 2 * n);
+            const gbytes rec = base + (size_t)s * T6K_REC;
+            m[0] = gload<uint32_t>(rec + 1536 + 8 * n);
+            m[1] = gload<uint32_t>(rec + 1540 + 8 * n);
+            m[2] = gload<uint16_t>(rec + 1664 + 2 * n);
         } else {
-            const uint8_t* rec = base + (size_t)s * T4M_REC;
-            m[0] = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
-            m[1] = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
+            const gbytes rec = base + (size_t)s * T4M_REC;
+            m[0] = gload<uint32_t>(rec + 1024 + 4 * n);
+            m[1] = gload<uint32_t>(rec + 1088 + 4 * n);
         }
     };
     const int take0 = (int)(4 * n);  // byte index of lane n for the lane-to-lane read; + 64 q: lane 16 q + n

@@ -163,6 +163,35 @@ void set_error(const std::string& msg);
 // ------------------------------------------------------------------------------------------------
 // Device helpers
 // ------------------------------------------------------------------------------------------------
+// A pointer that a kernel reads from memory (a table of per-expert bases) carries no address space, and loads through
+// it would be flat: those count as LDS traffic as well as memory traffic, so every wait for an LDS read would also wait
+// for all the weight records in flight. Weight streams therefore go through pointers typed as global memory.
+typedef const __attribute__((address_space(1))) uint8_t* gbytes;
+__device__ __forceinline__ gbytes as_global(const uint8_t* p) { return (gbytes)p; }
+template <int BYTES>
+struct GWord;
+template <>
+struct GWord<2> {
+    typedef uint16_t type;
+};
+template <>
+struct GWord<4> {
+    typedef uint32_t type;
+};
+template <>
+struct GWord<8> {
+    typedef uint32_t type __attribute__((ext_vector_type(2)));
+};
+template <>
+struct GWord<16> {
+    typedef uint32_t type __attribute__((ext_vector_type(4)));
+};
+template <class T>
+__device__ __forceinline__ T gload(gbytes p) {  // one request of sizeof(T) bytes
+    typedef typename GWord<sizeof(T)>::type W;
+    const W v = *reinterpret_cast<const __attribute__((address_space(1))) W*>(p);
+    return __builtin_bit_cast(T, v);
+}
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);  // exact
 }

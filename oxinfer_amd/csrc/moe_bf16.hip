@@ -80,8 +80,8 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
     const uint32_t nsteps = w.n_in / 128, ntiles = row_tiles(w.n_out);
     const uint32_t ng = 8 / kw, rg = wave / kw, kwave = wave % kw;
     const uint32_t tile0 = (blockIdx.x * ng + rg) * RT;
-    const uint8_t* base = bases[ch.x];
-    const uint8_t* wp[RT];
+    const gbytes base = as_global(bases[ch.x]);
+    gbytes wp[RT];
 #pragma unroll
     for (int r = 0; r < RT; r++) wp[r] = base + (size_t)min(tile0 + r, ntiles - 1) * t4m_steps(w.n_in) * T4M_REC;
     const uint32_t cnt = (nsteps - kwave + kw - 1) / kw, ilast = cnt - 1;  // kw <= nsteps
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
     auto load = [&](St& st, uint32_t i) {
         const uint32_t s = kwave + kw * min(i, ilast);
 #pragma unroll
-        for (int r = 0; r < RT; r++) st.w[r] = *reinterpret_cast<const u32x4*>(wp[r] + (size_t)s * T4M_REC + 16 * lane);
+        for (int r = 0; r < RT; r++) st.w[r] = gload<u32x4>(wp[r] + (size_t)s * T4M_REC + 16 * lane);
     };
     // A record's scale words (per row: the two groups' f16 scales at +1024, their bf16 offsets at +1088): a request costs
     // the memory pipeline the same for 64 bytes as for 1 KiB, so one request per row tile serves two steps: lane group kq
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
     auto load_scales = [&](uint32_t* sc, uint32_t i) {
         const uint32_t s = kwave + kw * min(i + (kq >> 1), ilast);
 #pragma unroll
-        for (int r = 0; r < RT; r++) sc[r] = *reinterpret_cast<const uint32_t*>(wp[r] + (size_t)s * T4M_REC + 1024 + 64 * (kq & 1) + 4 * n);
+        for (int r = 0; r < RT; r++) sc[r] = gload<uint32_t>(wp[r] + (size_t)s * T4M_REC + 1024 + 64 * (kq & 1) + 4 * n);
     };
     // the fragments first (L2 hits, needed by every step), then the first weight records, then the fragments go to LDS
     // while the weights are still on their way
