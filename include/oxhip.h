@@ -41,7 +41,7 @@ enum {
 };
 
 /* GGUF type ids handled (src/ggml.rs:42-93). */
-enum { OXHIP_GGML_Q8_0 = 8, OXHIP_GGML_Q4_K = 12, OXHIP_GGML_Q6_K = 14, OXHIP_GGML_F8E4M3 = 0x1000 };
+enum { OXHIP_GGML_Q4_0 = 2, OXHIP_GGML_Q8_0 = 8, OXHIP_GGML_Q4_K = 12, OXHIP_GGML_Q6_K = 14, OXHIP_GGML_F8E4M3 = 0x1000 };
 
 typedef struct {
     uint32_t kind;            /* OXHIP_W_* */

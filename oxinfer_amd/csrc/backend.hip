@@ -281,6 +281,29 @@ oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) {
                 }
                 break;
             }
+            if (d->ggml_type == OXHIP_GGML_Q4_0) {
+                // Q4_0 (18 B per 32: f16 d, then 16 bytes whose byte j holds elements j and j + 16; src/ggml.rs:675-683) is
+                // the Q4Matrix layout with the scale inside the block: split it into codes and scales and take that path
+                if (n_in % 32) return fail("Q4_0 rows must be whole blocks of 32");
+                const size_t nb = n_out * (n_in / 32);
+                std::vector<uint8_t> q(nb * 16);
+                std::vector<uint16_t> sc(nb);
+                const uint8_t* src = static_cast<const uint8_t*>(d->data);
+                for (size_t b = 0; b < nb; b++) {
+                    std::memcpy(&sc[b], src + 18 * b, 2);
+                    std::memcpy(&q[16 * b], src + 18 * b + 2, 16);
+                }
+                oxhip_weight_desc d2{};
+                d2.kind = OXHIP_W_Q4;
+                d2.n_out = n_out;
+                d2.n_in = n_in;
+                d2.data = q.data();
+                d2.scales = sc.data();
+                delete w;
+                oxhip_weight* w2 = oxhip_upload(c, &d2);
+                if (w2) w2->v.br = 1;
+                return w2;
+            }
             size_t raw_bytes;
             int np;
             if (d->ggml_type == OXHIP_GGML_Q8_0) {

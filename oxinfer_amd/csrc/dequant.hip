@@ -28,7 +28,8 @@ __global__ __launch_bounds__(256) void dequantize_kernel(WeightView w, uint32_t 
             int nib = j < 16 ? (byte & 0x0F) : (byte >> 4);
             float d = f16_bits_to_f32(reinterpret_cast<const uint16_t*>(w.p1)[r * (n / w.sgroup) + c / w.sgroup]);
             float m = w.group ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(w.p2)[r * (n / w.group) + c / w.group]) : 0.0f;
-            v = (float)(nib - 8) * d + m;
+            v = (float)(nib - 8) * d;
+            if (!w.br) v += m;  // Q4Matrix adds its offset, 0 without one (src/quant.rs:586-606); GGUF Q4_0 adds nothing (src/ggml.rs:675-683)
             break;
         }
         case FMT_Q8_0: {

@@ -41,7 +41,7 @@ struct WeightView {
     const uint8_t* p3;
     uint32_t sgroup;  // Q4: elements per scale
     uint32_t group;   // Q4: elements per offset (0: none)
-    uint32_t br, bc;  // FP8 block scale geometry
+    uint32_t br, bc;  // FP8 block scale geometry; planar Q4: br = 1 marks GGUF Q4_0 blocks (dequantized without an offset term)
 };
 
 struct QActView {

@@ -12,7 +12,7 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-Q8_0, Q4_K, Q6_K = 8, 12, 14
+Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
 TOL = 1e-3
 
 
@@ -73,7 +73,7 @@ with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "re
     REF_HASHES = {e["ggml_type"]: int(e["fnv1a64"], 16) for e in json.load(_f)["hashes"].values()}
 
 
-@pytest.mark.parametrize("kind", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q6_K])
 def test_gguf_dequant_matches_ggml_hash_on_device(be, oxref, kind):
     """The device dequantizer reproduces the reference's golden hashes (src/ggml.rs:1547-1577)."""
     raw, _ = oxref.random_blocks(kind, 1024 // oxref.block_size(kind), 1000 + kind)
@@ -83,7 +83,7 @@ def test_gguf_dequant_matches_ggml_hash_on_device(be, oxref, kind):
     assert oxref.fnv1a_f32(y) == REF_HASHES[kind]
 
 
-@pytest.mark.parametrize("kind", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q6_K])
 def test_gguf_dequant_and_isums_bit_exact(be, oxref, kind):
     n_out, n_in, t = 37, 3 * 256, 5
     raw, seed = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 13 + kind)
@@ -103,7 +103,7 @@ def test_gguf_dequant_and_isums_bit_exact(be, oxref, kind):
         assert np.array_equal(be.isums(w, xa, 32).cpu().numpy(), isums.reshape(t, n_out, -1, 2).sum(axis=3))
 
 
-@pytest.mark.parametrize("kind", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q6_K])
 @pytest.mark.parametrize("t", [1, 2, 3, 5, 8, 11, 16])
 def test_gguf_decode_matches_oracle(be, oxref, kind, t):
     # rows not a multiple of the wave's row group; Q8_0 with a block count that is not a multiple of 4
@@ -122,7 +122,7 @@ def test_gguf_decode_matches_oracle(be, oxref, kind, t):
         assert np.array_equal(y1[0].view(np.uint32), y[c].view(np.uint32)), c
 
 
-@pytest.mark.parametrize("kind", [Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q6_K])
 def test_gguf_decode_row_magnitudes(be, oxref, kind):
     n_out, n_in, t = 64, 4096, 4
     raw, seed = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 5 + kind)
@@ -308,7 +308,7 @@ def test_host_matmul_matches_device_path_and_declines(be, oxref):
 
 
 def test_upload_declines(be):
-    assert be.upload_gguf(2, np.zeros(18 * 4, np.uint8), 1, 128) is None  # Q4_0: no device kernels
+    assert be.upload_gguf(13, np.zeros(176, np.uint8), 1, 256) is None  # Q5_K: no device kernels
     assert "no device kernels" in be.last_error()
     assert be.upload_gguf(Q4_K, np.zeros(144, np.uint8), 1, 256) is not None
 
