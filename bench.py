@@ -304,7 +304,7 @@ def main():
         print(json.dumps({"workload": "copy", "bytes_read": n, "bytes_written": n, "launches": args.warmup + args.steps}))
         return
     be = HipBackend(0)
-    if args.workload in ("mlx_gemv", "mlx_gemm", "moe", "fp8"):
+    if args.workload in ("mlx_gemv", "mlx_gemm", "gguf_gemm", "moe", "fp8"):
         print(json.dumps(other_workload(args, be, torch, synth)))
         be.close()
         return
