@@ -139,7 +139,8 @@ void oxhip_free_weight(oxhip_ctx* c, oxhip_weight* w) {
     delete w;
 }
 
-oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) {
+// `q4_0_blocks`: the planar Q4 data of this call are GGUF Q4_0 blocks split by the caller below (no offset term at all)
+static oxhip_weight* upload_weight(oxhip_ctx* c, const oxhip_weight_desc* d, bool q4_0_blocks) {
     if (!c || !d || !d->data) {
         set_error("upload: null argument");
         return nullptr;
@@ -300,9 +301,7 @@ oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) {
                 d2.data = q.data();
                 d2.scales = sc.data();
                 delete w;
-                oxhip_weight* w2 = oxhip_upload(c, &d2);
-                if (w2) w2->v.br = 1;
-                return w2;
+                return upload_weight(c, &d2, true);
             }
             size_t raw_bytes;
             int np;
@@ -338,12 +337,14 @@ oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) {
         default: return fail("weight kind " + std::to_string(d->kind) + " has no device kernels");
     }
     if (hipStreamSynchronize(s) != hipSuccess) return fail("upload failed");
-    if (w->v.fmt == FMT_Q4 && w->v.group == 64 && w->v.sgroup == 64) {
-        // one scale and one offset per 64 (MLX checkpoints): tile-packed for the matrix cores
+    const bool q40 = q4_0_blocks && w->v.fmt == FMT_Q4;
+    if (q40) w->v.br = 1;  // (kept should the tile packing below be skipped for lack of memory)
+    if ((w->v.fmt == FMT_Q4 && w->v.group == 64 && w->v.sgroup == 64) || q40) {
+        // one scale and one offset per 64 (MLX checkpoints), or GGUF Q4_0's scale per 32: tile-packed for the matrix cores
         const size_t bytes = t4m_bytes((uint32_t)n_out, (uint32_t)n_in);
         void* packed = nullptr;
         if (have_memory(bytes) && hipMalloc(&packed, bytes) == hipSuccess) {
-            if (launch_pack_q4m(w->v.p0, reinterpret_cast<const uint16_t*>(w->v.p1), reinterpret_cast<const uint16_t*>(w->v.p2), n_out,
+            if (launch_pack_q4m(w->v.p0, reinterpret_cast<const uint16_t*>(w->v.p1), q40 ? nullptr : reinterpret_cast<const uint16_t*>(w->v.p2), n_out,
                                 n_in, static_cast<uint8_t*>(packed), s) != hipSuccess ||
                 hipStreamSynchronize(s) != hipSuccess) {
                 (void)hipFree(packed);
@@ -352,13 +353,15 @@ oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) {
             (void)hipFree(w->base);
             w->base = packed;
             w->bytes = bytes;
-            w->v.fmt = FMT_Q4M;
+            w->v.fmt = q40 ? FMT_Q40 : FMT_Q4M;
             w->v.p0 = static_cast<const uint8_t*>(packed);
             w->v.p1 = w->v.p2 = nullptr;
         }
     }
     return w;
 }
+
+oxhip_weight* oxhip_upload(oxhip_ctx* c, const oxhip_weight_desc* d) { return upload_weight(c, d, false); }
 
 // ---- device-pointer entry points ---------------------------------------------------------------
 int oxhip_dev_quantize_act(oxhip_ctx* c, const float* x, size_t t, size_t n_in, const oxhip_qact* out, void* stream) {

@@ -117,6 +117,11 @@ struct Step<FMT_Q4M> {
     uint32_t a[4];
 };
 template <>
+struct Step<FMT_Q40> {
+    uint4 w;
+    uint32_t a[4];
+};
+template <>
 struct Step<FMT_Q6_K> {
     uint4 w;   // low nibbles
     uint2 h;   // high bit pairs
@@ -401,8 +406,10 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                 v4i bw = {(int)(w0 & 0x0F0F0F0Fu), (int)((w0 >> 4) & 0x0F0F0F0Fu), (int)(w1 & 0x0F0F0F0Fu),
                           (int)((w1 >> 4) & 0x0F0F0F0Fu)};
                 const uint32_t b = 4 * s + 2 * g + d_half;
-                const float d = f16_bits_to_f32((uint16_t)(g ? sw[0] >> 16 : sw[0] & 0xFFFF));
-                const float off = bf16_bits_to_f32((uint16_t)(g ? sw[1] >> 16 : sw[1] & 0xFFFF));
+                // MLX: the group's scale and offset; Q4_0: the lane's block's own scale (word g, half d_half), no offset
+                const float d = FMT == FMT_Q40 ? f16_bits_to_f32((uint16_t)(d_half ? sw[g] >> 16 : sw[g] & 0xFFFF))
+                                               : f16_bits_to_f32((uint16_t)(g ? sw[0] >> 16 : sw[0] & 0xFFFF));
+                const float off = FMT == FMT_Q40 ? 0.0f : bf16_bits_to_f32((uint16_t)(g ? sw[1] >> 16 : sw[1] & 0xFFFF));
                 const float dz = b < nblk ? d : 0.0f, offz = b < nblk ? off : 0.0f;
 #pragma unroll
                 for (int tg = 0; tg < NG; tg++) {
@@ -414,7 +421,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                     // zeros (as a select, not a branch: a divergent branch here makes every step wait for all requests)
 #pragma unroll
                     for (int i = 0; i < NI; i++)
-                        acc[tg][i] = fmaf(offz, m.fs[i], fmaf(dz, fmaf(m.xs[i], (float)U[i], m.c[i]), acc[tg][i]));
+                        acc[tg][i] = FMT == FMT_Q40 ? fmaf(dz, fmaf(m.xs[i], (float)U[i], m.c[i]), acc[tg][i])
+                                                    : fmaf(offz, m.fs[i], fmaf(dz, fmaf(m.xs[i], (float)U[i], m.c[i]), acc[tg][i]));
                     if (DUMP) {
                         int isum[4] = {U[0] - 8 * m.su[0], U[1] - 8 * m.su[1], U[2] - 8 * m.su[2], U[3] - 8 * m.su[3]};
                         dump_block(b, isum);
@@ -437,11 +445,11 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // the weights' lane group kq pairs with (Q4: positions 4 kq.. and 16 + 4 kq..; else 8 kq..). A thread moves 16
     // (Q4: 32) consecutive bytes of one token's row, so the global reads are whole lines. Absent tokens and a padding
     // block keep whatever LDS holds: those products meet zero weights or are dropped.
-    constexpr int AU = FMT == FMT_Q4M ? 2 : 1;  // 16-byte loads per unit of staging work
+    constexpr int AU = t4m_format(FMT) ? 2 : 1;  // 16-byte loads per unit of staging work
     // Unit i of the staging work is (token i / adiv, chunk i % adiv); a thread takes units tid, tid + nthr, ...: one
     // division for its first unit, then carries (a division per unit would be most of the instructions of a wave that
     // only streams some fifteen records).
-    const uint32_t adiv = max(FMT == FMT_Q4M ? nb : 2 * nb, 1u);
+    const uint32_t adiv = max(t4m_format(FMT) ? nb : 2 * nb, 1u);
     auto advance = [](uint32_t& q, uint32_t& r, uint32_t dq, uint32_t dr, uint32_t dv) {
         r += dr;
         q += dq;
@@ -452,7 +460,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     };
     const uint32_t a_dq = nthr / adiv, a_dr = nthr - a_dq * adiv;
     auto act_load = [&](uint32_t tok, uint32_t c, uint4* v) {  // tok < t; c: chunk (Q4M: block) within the slice
-        if (FMT == FMT_Q4M) {
+        if (t4m_format(FMT)) {
             const uint4* xb = reinterpret_cast<const uint4*>(xa.q + src_row(tok) * w.n_in + (size_t)(B0 + c) * 32);
             v[0] = xb[0];
             v[1] = xb[1];
@@ -461,7 +469,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         }
     };
     auto act_store = [&](uint32_t tok, uint32_t c, const uint4* v) {
-        if (FMT == FMT_Q4M) {
+        if (t4m_format(FMT)) {
             const uint32_t b = c;
             uint2* dst = afr + ((size_t)(tok >> 3) * (nbl / 2) + (b >> 1)) * 64;
             const uint32_t s0 = SWZ ? opslot(b >> 1, 8 * (b & 1) + (tok & 7)) : 8 * (b & 1) + (tok & 7);
@@ -718,7 +726,7 @@ __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid,
     const GroupView none{};
     const uint32_t bx = bid >> __builtin_ctz(jb.ks), by = bid & (jb.ks - 1);  // the slices of a row group are neighbours in launch order (ks: a power of two)
     if (jb.t == 1) decode_body<FMT, 1, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
-    else if (jb.t == 2 && FMT != FMT_Q4M) decode_body<FMT, 2, false, false, true>(  // (MLX at 2 tokens: the 4-token body, which fits the registers)
+    else if (jb.t == 2 && !t4m_format(FMT)) decode_body<FMT, 2, false, false, true>(  // (MLX at 2 tokens: the 4-token body, which fits the registers)
         jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
     else if (jb.t <= 4) decode_body<FMT, 4, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
     else decode_body<FMT, 8, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
@@ -736,6 +744,7 @@ __global__ __launch_bounds__(1024) void decode_batch_kernel(BatchArgs a) {
         case FMT_Q4_K: batch_dispatch<FMT_Q4_K>(jb, bx, lds_dyn); break;
         case FMT_Q6_K: batch_dispatch<FMT_Q6_K>(jb, bx, lds_dyn); break;
         case FMT_Q4M: batch_dispatch<FMT_Q4M>(jb, bx, lds_dyn); break;
+        case FMT_Q40: batch_dispatch<FMT_Q40>(jb, bx, lds_dyn); break;
         default: break;
     }
 }
@@ -903,7 +912,7 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
         const uint32_t tt = (uint32_t)tc;
         hipError_t e;
         if (tc == 1) e = launch_one<FMT, 1, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
-        else if (tc == 2 && FMT != FMT_Q4M) e = launch_one<FMT, 2, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
+        else if (tc == 2 && !t4m_format(FMT)) e = launch_one<FMT, 2, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
         else if (tc <= 4) e = launch_one<FMT, 4, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
         else e = launch_one<FMT, 8, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
         if (e != hipSuccess) return e;
@@ -1071,6 +1080,7 @@ hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t,
         case FMT_Q4_K: return run<FMT_Q4_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
         case FMT_Q6_K: return run<FMT_Q6_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
         case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
+        case FMT_Q40: return run<FMT_Q40, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
         default: return hipErrorInvalidValue;
     }
 }
@@ -1083,6 +1093,7 @@ hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, 
         case FMT_Q4_K: return run<FMT_Q4_K, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q6_K: return run<FMT_Q6_K, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q4M: return run<FMT_Q4M, true>(w, xa, t, y, out, DecodeScratch{}, s);
+        case FMT_Q40: return run<FMT_Q40, true>(w, xa, t, y, out, DecodeScratch{}, s);
         default: return hipErrorInvalidValue;
     }
 }

@@ -69,6 +69,15 @@ __global__ __launch_bounds__(256) void dequantize_kernel(WeightView w, uint32_t 
             v = (float)(nib - 8) * d + m;
             break;
         }
+        case FMT_Q40: {  // (nib - 8) * d, no offset term (src/ggml.rs:675-683)
+            uint32_t tile = r >> 4, nn = r & 15, b = c >> 5, st = b >> 2, bi = b & 3, e = c & 31, hi = e >> 4, pp = e & 15, kq = pp >> 2;
+            const uint8_t* rec = w.p0 + ((size_t)tile * t4m_steps(n) + st) * T4M_REC;
+            uint8_t byte = rec[16 * (kq * 16 + nn) + 4 * bi + (pp & 3)];
+            int nib = hi ? (byte >> 4) : (byte & 0xF);
+            float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(rec + (bi < 2 ? 1024 : 1088) + 4 * nn + 2 * (bi & 1)));
+            v = (float)(nib - 8) * d;
+            break;
+        }
         case FMT_Q6_K: {
             const uint32_t tile = r >> 4, nn = r & 15, st = c >> 7, wi = c & 127, h = wi >> 6, kq = (wi & 63) >> 4, j = wi & 15;
             const uint8_t* rec = w.p0 + ((size_t)tile * t6k_steps(n) + st) * T6K_REC;
@@ -189,7 +198,10 @@ __global__ __launch_bounds__(256) void pack_q4m_kernel(const uint8_t* __restrict
         uint32_t d = 0, o = 0;
         for (uint32_t g = 0; g < 2; g++) {
             uint32_t grp = 2 * st + g;
-            if (row < n_out && grp < n_in / 64) {
+            if (!off) {  // Q4_0: a scale per 32; d = blocks 0 and 1 of the step, o = blocks 2 and 3
+                if (row < n_out && 4 * st + g < nblk) d |= (uint32_t)sc[row * nblk + 4 * st + g] << (16 * g);
+                if (row < n_out && 4 * st + 2 + g < nblk) o |= (uint32_t)sc[row * nblk + 4 * st + 2 + g] << (16 * g);
+            } else if (row < n_out && grp < n_in / 64) {
                 d |= (uint32_t)sc[row * (n_in / 64) + grp] << (16 * g);
                 o |= (uint32_t)off[row * (n_in / 64) + grp] << (16 * g);
             }

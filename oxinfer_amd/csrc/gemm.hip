@@ -171,7 +171,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
 #pragma unroll
     for (int i = 0; i < 2; i++) {
         const uint32_t tile = min(nt0 + 2 * wave + i, ntiles - 1);
-        if (FMT == FMT_Q4M) {
+        if (t4m_format(FMT)) {
             wbase[i] = w.p0 + ((size_t)tile * all_steps + step0) * T4M_REC;
         } else if (q8_format(FMT)) {  // the tile's records; load_raw indexes them from the matrix's first step
             wbase[i] = w.p0 + (size_t)tile * t8_steps(w.n_in) * (FMT == FMT_Q8F ? T8F_REC : T8_REC);
@@ -202,7 +202,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     };
     auto load_raw_tile = [&](Raw* r, int i, uint32_t s) {  // the records of the wave's row tile i at step s
         {
-            if (FMT == FMT_Q4M) {
+            if (t4m_format(FMT)) {
                 const uint8_t* rec = wbase[i] + (size_t)s * T4M_REC;
                 r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
                 r[i].m[0] = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
@@ -258,7 +258,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     // `s`: the step the records belong to (of this slice)
     auto dequant_tile = [&](const Raw& r, int i, uint32_t buf, uint32_t s) {  // one of the wave's two row tiles, 4 blocks
         uint4* dst = bfrag + ((size_t)(buf * 4) * WG_NT + 2 * wave + i) * 64 + lane;  // block b: + b * WG_NT * 64
-        if (FMT == FMT_Q4M) {
+        if (FMT == FMT_Q40) {  // the block's own scale: word b / 2, half b % 2; (nib - 8) * d
+            const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const float d = f16_bits_to_f32((uint16_t)((b & 1) ? r.m[b >> 1] >> 16 : r.m[b >> 1] & 0xFFFF));
+                dst[b * WG_NT * 64] = dequant_q4m(cw[b], d, -8.0f * d);
+            }
+        } else if (FMT == FMT_Q4M) {
             const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
             for (int b = 0; b < 4; b++) {
@@ -447,21 +454,22 @@ hipError_t launch_gemm_reduce(const float* partial, size_t n, uint32_t slices, v
 }
 
 // `partial`: scratch of slices * t * n_out floats when gemm_k_slices() > 1.
-// The formats the kernel dequantizes: tile-packed MLX 4-bit, Q8_0 / Q8, Q4_K, Q6_K, and FP8 rows of whole 128-column
+// The formats the kernel dequantizes: tile-packed MLX 4-bit and Q4_0, Q8_0 / Q8, Q4_K, Q6_K, and FP8 rows of whole 128-column
 // steps with scale blocks of 16 k rows x 128 k columns.
 bool gemm_bf16_ok(const WeightView& w) {
-    if (w.fmt == FMT_Q4M || q8_format(w.fmt)) return true;
+    if (t4m_format(w.fmt) || q8_format(w.fmt)) return true;
     if (w.fmt == FMT_Q4_K || w.fmt == FMT_Q6_K) return w.n_in % 256 == 0;
     return w.fmt == FMT_FP8 && w.br % 16 == 0 && w.bc % 128 == 0 && w.n_in % 128 == 0;
 }
 // pack_a's MODE for the format's fragments
-int gemm_bf16_pack_mode(const WeightView& w) { return w.fmt == FMT_Q4M ? 1 : w.fmt == FMT_FP8 ? 2 : w.fmt == FMT_Q6_K ? 3 : 0; }
+int gemm_bf16_pack_mode(const WeightView& w) { return t4m_format(w.fmt) ? 1 : w.fmt == FMT_FP8 ? 2 : w.fmt == FMT_Q6_K ? 3 : 0; }
 
 hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                             hipStream_t s) {
     if (!gemm_bf16_ok(w)) return hipErrorInvalidValue;
     switch (w.fmt) {
         case FMT_Q4M: return run_gemm_bf16<FMT_Q4M>(w, apk, t, mtiles, y, out_bf16, partial, s);
+        case FMT_Q40: return run_gemm_bf16<FMT_Q40>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q8_0: return run_gemm_bf16<FMT_Q8_0>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q8F: return run_gemm_bf16<FMT_Q8F>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q4_K: return run_gemm_bf16<FMT_Q4_K>(w, apk, t, mtiles, y, out_bf16, partial, s);

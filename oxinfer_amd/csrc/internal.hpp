@@ -22,14 +22,17 @@ namespace oxhip {
 //                                     of a group carries the same scale
 //         p2 off [n_out][n_in/group]  bf16 offsets, optional
 //   Q6_K  p0      T6K records (layout.hpp)
+//   Q40   p0      T4M records of GGUF Q4_0: the four f16 block scales of a row where MLX keeps two scales and two offsets
 //   Q8F   p0      T8F records: QMatrix, int8 codes with one f32 scale per 32
 //   FP8   p0 q   [n_out][n_in]        e4m3 bytes (row-major, or tile-packed when group == 1: fp8_offset below);
 //         p1 bs f32 [ceil(n_out/br)][ceil(n_in/bc)]
 //   BF16  p0 q   [n_out][n_in]        bf16
 // ------------------------------------------------------------------------------------------------
-enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6, FMT_Q8F = 7 };
+enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6, FMT_Q8F = 7, FMT_Q40 = 8 };
 // the formats of the matrix-core decode kernels (decode_mfma.hip); the two Q8 kinds carry no sums or offsets
-inline bool mfma_decode_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F || f == FMT_Q4_K || f == FMT_Q6_K || f == FMT_Q4M; }
+inline bool mfma_decode_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F || f == FMT_Q4_K || f == FMT_Q6_K || f == FMT_Q4M || f == FMT_Q40; }
+// the two 4-bit formats in T4M records (MLX: a scale and an offset per 64; GGUF Q4_0: a scale per 32)
+__host__ __device__ constexpr bool t4m_format(int f) { return f == FMT_Q4M || f == FMT_Q40; }
 __host__ __device__ constexpr bool q8_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F; }
 
 struct WeightView {
@@ -109,6 +112,7 @@ hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, c
                                       uint32_t max_rows_per_chunk, float* y, hipStream_t s);
 hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* out, hipStream_t s);
 hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t n_in, const WeightView& dst, hipStream_t s);
+// off == nullptr: `sc` holds one scale per 32 (Q4_0) and the record keeps all four of a row's step
 hipError_t launch_pack_q4m(const uint8_t* q, const uint16_t* sc, const uint16_t* off, size_t n_out, size_t n_in, uint8_t* dst,
                            hipStream_t s);
 hipError_t launch_repack_mlx_q4(const uint32_t* w, const uint16_t* scales, const uint16_t* biases, size_t n_out,

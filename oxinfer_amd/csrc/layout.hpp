@@ -22,6 +22,8 @@
 //                  (low nibble: element 4 kq + j, high nibble: element 16 + 4 kq + j)
 //               d[n][2] f16 (blocks 0-1, blocks 2-3)                                  64 B
 //               off[n][2] bf16                                                        64 B
+//   GGUF Q4_0 in the same records: d[n][4] f16, the scales of blocks 0-1 where MLX has its scales and of blocks 2-3
+//   where it has its offsets.
 #pragma once
 #include <stddef.h>
 #include <stdint.h>

@@ -37,6 +37,16 @@ def q8_matrix(n_out, n_in, seed):
     return q, scales
 
 
+def gguf_q4_0(n_out, n_in, seed):
+    """Q4_0 blocks (18 B): f16 d ~ |N(0, 0.01)|, 32 nibbles uniform (byte j = elements j and j + 16)."""
+    rng = np.random.default_rng(seed)
+    nb = n_out * n_in // 32
+    blk = np.empty((nb, 18), np.uint8)
+    blk[:, :2] = np.abs(rng.normal(0.0, 0.01, nb)).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    blk[:, 2:] = rng.integers(0, 256, (nb, 16), dtype=np.uint8)
+    return blk.reshape(-1)
+
+
 def gguf_q8_0(n_out, n_in, seed):
     """Q8_0 blocks (34 B): f16 d ~ |N(0, 0.01)|, 32 int8 uniform in [-127, 127]."""
     rng = np.random.default_rng(seed)
