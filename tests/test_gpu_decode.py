@@ -402,3 +402,47 @@ def test_decode_batch_events(be, oxref):
         assert be.elapsed_ms(e0, e1) > 0.0 and be.elapsed_ms(e2, e3) > 0.0 and be.elapsed_ms(e0, e3) > 0.0
         for y, want in zip(ys, plain):
             assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_works_from_another_thread_and_concurrent_calls_do_not_mix(be, oxref):
+    """The Backend surface is Send + Sync (src/gpu.rs:151): a call from another thread, on weights uploaded here, and eight
+    threads calling at once, each with its own input, get their own rows (src/cuda.rs:2048-2077, :2411-2439). A call's
+    rows are a function of its inputs alone, so they must equal the rows of the same call made alone, bit for bit."""
+    import threading
+    from oxinfer_amd import synth
+    n_out, n_in = 64, 512
+    raw = oxref.random_blocks(Q4_K, n_out * n_in // 256, 91)[0]
+    wq, sc, bi = synth.mlx_q4(n_out, n_in, 92)
+    ws = [be.upload_gguf(Q4_K, raw, n_out, n_in), be.upload_mlx_q4(wq, sc, bi, 64, n_out, n_in)]
+    cases = []
+    for i in range(8):
+        t = (3, 40)[i % 2]  # the shared decode launch, and the prefill GEMM with its scratch in the context
+        x = synth.activations(t, n_in, 300 + i)
+        ys = [np.full((t, n_out), np.nan, np.float32) for _ in ws]
+        assert be.matmul(x, t, n_in, list(zip(ws, ys))), be.last_error()
+        assert row_err(ys[0], oxref.gguf_decode(Q4_K, raw, n_out, n_in, x, t) if t <= 16 else oxref.gemm_quant(Q4_K, raw, None, None, n_out, n_in, x, t)) < 2e-2
+        cases.append((t, x, ys))
+    errors = []
+
+    def worker(t, x, want, rounds):
+        try:
+            for _ in range(rounds):
+                ys = [np.full((t, n_out), np.nan, np.float32) for _ in ws]
+                if not be.matmul(x, t, n_in, list(zip(ws, ys))):
+                    raise AssertionError("declined: " + be.last_error())
+                for y, w0 in zip(ys, want):
+                    if not np.array_equal(y.view(np.uint32), w0.view(np.uint32)):
+                        raise AssertionError(f"rows of another call (t = {t})")
+        except Exception as e:  # reported by the main thread
+            errors.append(e)
+
+    th = threading.Thread(target=worker, args=(*cases[0], 1))
+    th.start()
+    th.join()
+    assert not errors, errors
+    threads = [threading.Thread(target=worker, args=(*c, 8)) for c in cases]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
