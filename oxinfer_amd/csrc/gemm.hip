@@ -112,7 +112,7 @@ hipError_t launch_pack_a(const void* x, bool src_bf16, int mode, size_t t, size_
 
 namespace {
 
-constexpr int WG_MT = 16;  // token tiles per workgroup (256 tokens), 4 per wave
+
 constexpr int WG_NT = 8;   // row tiles per workgroup (128 rows)
 constexpr int AR = 4;      // blocks of A fragments held ahead (a whole K-step: two starve the FP8 shapes, whose activations do not stay in L2)
 
@@ -151,7 +151,7 @@ __device__ __forceinline__ uint4 dequant_q4m(uint32_t w, float d, float c) {
 // FMT: FMT_Q4M (tile-packed MLX 4-bit), FMT_Q8_0 / FMT_Q8F / FMT_Q4_K / FMT_Q6_K (their tile records) or FMT_FP8 (e4m3 bytes with 128 x 128 block scales: the bytes are
 // exact in bf16, the block scale multiplies in f32 before the rounding, and a lane takes 32 consecutive row bytes
 // per step, which pack_a's mode 2 mirrors on the activation side).
-template <int FMT, bool OUT_BF16>
+template <int FMT, bool OUT_BF16, int NV>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint4* __restrict__ apk, uint32_t t, uint32_t mtiles,
                                                         void* __restrict__ yv) {
     extern __shared__ uint4 bfrag[];  // [2][4 blocks][8 row tiles][64 lanes]
@@ -163,7 +163,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     const uint32_t nsteps = min(all_steps, step0 + per_z) - step0;
     const uint32_t ntiles = row_tiles(w.n_out);
     const uint32_t nt0 = blockIdx.x * WG_NT;               // first row tile of the workgroup
-    const uint32_t mt0 = blockIdx.y * WG_MT + wave * 4;    // first token tile of the wave
+    // the wave's token tiles: mt0, mt0 + 4, ... (NV of them: 4, or 1 when the whole launch has at most 64 tokens per
+    // workgroup row, so that a few tokens do not pay for 256)
+    const uint32_t mt0 = blockIdx.y * (4 * NV) + wave;
 
     // the two row tiles this wave dequantizes
     const uint8_t* wbase[2];
@@ -186,13 +188,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
         }
     }
     // A fragments of the wave's 4 token tiles (tiles past the end repeat the last one; their rows are not stored)
-    const uint4* abase[4];
+    const uint4* abase[NV];
 #pragma unroll
-    for (int i = 0; i < 4; i++) abase[i] = apk + ((size_t)min(mt0 + i, mtiles - 1) * kblocks + 4 * step0) * 64 + lane;
+    for (int i = 0; i < NV; i++) abase[i] = apk + ((size_t)min(mt0 + 4 * i, mtiles - 1) * kblocks + 4 * step0) * 64 + lane;
 
-    f32x4 acc[4][WG_NT];
+    f32x4 acc[NV][WG_NT];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < NV; i++)
 #pragma unroll
         for (int j = 0; j < WG_NT; j++) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
@@ -326,7 +328,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     };
     auto read_a = [&](uint4* dst, uint32_t blk) {  // the A fragments of block `blk` of this slice
 #pragma unroll
-        for (int i = 0; i < 4; i++) dst[i] = abase[i][(size_t)blk * 64];
+        for (int i = 0; i < NV; i++) dst[i] = abase[i][(size_t)blk * 64];
     };
     // LDS traffic only: outstanding global loads (the prefetches) stay in flight across the barrier
     auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
@@ -338,7 +340,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     constexpr bool EARLY_RAW = OXHIP_GEMM_EARLY_RAW;
     Raw raw[2];
     load_raw(raw, 0);
-    uint4 a_cur[AR][4], b_cur[WG_NT];
+    uint4 a_cur[AR][NV], b_cur[WG_NT];
     const uint32_t last = nsteps - 1, last_blk = 4 * nsteps - 1;
 #pragma unroll
     for (int b = 0; b < AR; b++) read_a(a_cur[b], min((uint32_t)b, last_blk));
@@ -360,7 +362,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
             for (int j = 0; j < WG_NT; j++) {
                 const bf16x8 bb = __builtin_bit_cast(bf16x8, b_cur[j]);
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                for (int i = 0; i < NV; i++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_cur[b % AR][i]), bb, acc[i][j], 0, 0, 0);
                 if (b < 3) b_cur[j] = bfrag[((buf * 4 + b + 1) * WG_NT + j) * 64 + lane];
                 else b_cur[j] = bfrag[(((buf ^ 1) * 4) * WG_NT + j) * 64 + lane];
@@ -382,14 +384,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     const uint32_t kq = lane >> 4;
     if (gridDim.z > 1) yv = reinterpret_cast<float*>(yv) + (size_t)blockIdx.z * t * w.n_out;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < NV; i++) {
 #pragma unroll
         for (int j = 0; j < WG_NT; j++) {
             const uint32_t row = (nt0 + j) * 16 + n;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const uint32_t tok = (mt0 + i) * 16 + 4 * kq + r;
-                if (tok < t && row < w.n_out && mt0 + i < mtiles) {
+                const uint32_t tok = (mt0 + 4 * i) * 16 + 4 * kq + r;
+                if (tok < t && row < w.n_out && mt0 + 4 * i < mtiles) {
                     if (OUT_BF16) reinterpret_cast<uint16_t*>(yv)[(size_t)tok * w.n_out + row] = f32_to_bf16_bits(acc[i][j][r]);
                     else reinterpret_cast<float*>(yv)[(size_t)tok * w.n_out + row] = acc[i][j][r];
                 }
@@ -410,32 +412,44 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restric
 }
 
 // K slices for a launch: enough workgroups to cover the CUs while each keeps at least 8 steps.
+// Token tiles per wave: one when the launch has at most four (64 tokens), else four.
+static int gemm_nv(size_t mtiles) { return mtiles <= 4 ? 1 : 4; }
+
 uint32_t gemm_k_slices(const WeightView& w, size_t mtiles) {
-    const uint32_t wgs = ((row_tiles(w.n_out) + WG_NT - 1) / WG_NT) * (uint32_t)((mtiles + WG_MT - 1) / WG_MT);
+    const uint32_t per_wg = 4 * gemm_nv(mtiles);
+    const uint32_t wgs = ((row_tiles(w.n_out) + WG_NT - 1) / WG_NT) * (uint32_t)((mtiles + per_wg - 1) / per_wg);
     const uint32_t steps = (w.n_in + 127) / 128;
     uint32_t z = 1;
-    while (z < 8 && wgs * z * 2 <= 256 && steps / (z * 2) >= 8) z *= 2;
+    // (one token tile per wave: a K-step is short, two workgroups fit a CU, and what counts is requests in flight)
+    const uint32_t places = gemm_nv(mtiles) == 1 ? 512 : 256, min_steps = gemm_nv(mtiles) == 1 ? 4 : 8;
+    while (z < 8 && wgs * z * 2 <= places && steps / (z * 2) >= min_steps) {
+        // every slice must own a step: the kernel gives slice i the steps from i * ceil(steps / z) (33 steps in 8 slices
+        // of 5 would start the last one past the end)
+        const uint32_t z2 = z * 2, per = (steps + z2 - 1) / z2;
+        if ((z2 - 1) * per >= steps) break;
+        z = z2;
+    }
     return z;
 }
 
 namespace {
-template <int FMT>
-hipError_t run_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
+template <int FMT, int NV>
+hipError_t run_gemm_bf16_nv(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                          hipStream_t s) {
     const uint32_t slices = gemm_k_slices(w, mtiles);
-    dim3 grid((row_tiles(w.n_out) + WG_NT - 1) / WG_NT, (unsigned)((mtiles + WG_MT - 1) / WG_MT), slices);
+    dim3 grid((row_tiles(w.n_out) + WG_NT - 1) / WG_NT, (unsigned)((mtiles + 4 * NV - 1) / (4 * NV)), slices);
     const size_t lds = 2 * 4 * WG_NT * 64 * 16;  // 64 KiB
     const bool direct_bf16 = out_bf16 && slices == 1;
     void* dst = slices > 1 ? static_cast<void*>(partial) : y;
     hipError_t e;
     if (direct_bf16) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, true, NV>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        gemm_bf16_kernel<FMT, true><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
+        gemm_bf16_kernel<FMT, true, NV><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
     } else {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, false, NV>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        gemm_bf16_kernel<FMT, false><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
+        gemm_bf16_kernel<FMT, false, NV><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
     }
     e = hipGetLastError();
     if (e != hipSuccess || slices == 1) return e;
@@ -443,6 +457,12 @@ hipError_t run_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t 
     if (out_bf16) gemm_reduce_kernel<true><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
     else gemm_reduce_kernel<false><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
     return hipGetLastError();
+}
+template <int FMT>
+hipError_t run_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
+                         hipStream_t s) {
+    if (gemm_nv(mtiles) == 1) return run_gemm_bf16_nv<FMT, 1>(w, apk, t, mtiles, y, out_bf16, partial, s);
+    return run_gemm_bf16_nv<FMT, 4>(w, apk, t, mtiles, y, out_bf16, partial, s);
 }
 }  // namespace
 
