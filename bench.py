@@ -181,7 +181,7 @@ def other_workload(args, be, torch, synth):
                     config={"workload": f"configs[2]: MLX 4-bit g64 prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096, variant {args.variant}",
                             "flops_per_step": flops, "events": "around the two calls of a step (activation packing + GEMM (+ K-slice sum))"},
                     roofline={"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4),
-                              "traffic": None, "kernel": "gemm_bf16_kernel<6, false>" if variant == 0 else "gemm_i8_q4m_kernel",
+                              "traffic": None, "kernel": "gemm_bf16_kernel<6, false, 4>" if variant == 0 else "gemm_i8_q4m_kernel",
                               "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3 / 2, 2)})
 
     if args.workload == "gguf_gemm":                     # configs[1]'s weights at configs[2]'s token count: M = 512, both shapes
@@ -203,7 +203,7 @@ def other_workload(args, be, torch, synth):
                     config={"workload": f"GGUF {args.format.upper()} prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096 (bf16 matrix cores)",
                             "flops_per_step": flops, "events": "around the two calls of a step (activation packing + GEMM (+ K-slice sum))"},
                     roofline={"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK["bf16"], "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK["bf16"], 4),
-                              "traffic": None, "kernel": f"gemm_bf16_kernel<{ {'q8_0': 1, 'q4_k': 2, 'q6_k': 3}[args.format]}, false>",
+                              "traffic": None, "kernel": f"gemm_bf16_kernel<{ {'q8_0': 1, 'q4_k': 2, 'q6_k': 3}[args.format]}, false, 4>",
                               "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3 / 2, 2)})
 
     if args.workload == "moe":                           # configs[3]: 128 experts, top-8, h = 2048, inter = 768
@@ -253,7 +253,7 @@ def other_workload(args, be, torch, synth):
         kern = "skinny_fp8_kernel<*, 1, 2, *, false> (+ pack_skinny_kernel)"
     else:
         step = lambda i: be.gemm(ws[i % len(ws)], xb, variant=variant, out_bf16=True)
-        kern = ("skinny_fp8_kernel<4, 2, 1, 16, true> (+ pack_skinny_kernel, gemm_reduce_kernel)" if m <= 32 else "gemm_bf16_kernel<4, true>") if variant == 0 else "gemm_fp8_kernel<true>"
+        kern = ("skinny_fp8_kernel<4, 2, 1, 16, true> (+ pack_skinny_kernel, gemm_reduce_kernel)" if m <= 32 else "gemm_bf16_kernel<4, true, 4>") if variant == 0 else "gemm_fp8_kernel<true>"
     wall, ms = timed_steps(torch, step, args.steps, args.warmup)
     flops, nbytes = 2 * m * n * k, n * k + scales.size * 4 + m * k * 2 + m * n * 2
     hbm = m <= 64
