@@ -6,8 +6,9 @@
 // (matmul_quant_block_prefill + gemm_8x8, src/kernels.rs:1998-2038, src/kernels_x86.rs:296-324 of the reference);
 // here weights and activations are rounded to bf16 first, so results agree to bf16 precision, not bit for bit.
 //
-// Work split: a workgroup of 4 waves owns 256 tokens x 128 weight rows; wave v owns tokens 64 v .. 64 v + 63 and
-// all 128 rows (4 x 8 MFMA tiles of 16 x 16, 128 accumulator registers).
+// Work split: a workgroup of 4 waves owns 256 tokens x 128 weight rows; wave v owns the token tiles v, v + 4, v + 8,
+// v + 12 of the workgroup's sixteen and all 128 rows (4 x 8 MFMA tiles of 16 x 16, 128 accumulator registers). A
+// launch of at most 64 tokens gives each wave one token tile (64 tokens x 128 rows per workgroup).
 //   B (weights): each K-step of 128 the four waves dequantize the step's 8 row tiles (two each) from the packed
 //     records into bf16 MFMA fragments in LDS (double-buffered, one barrier per step); every wave then reads all
 //     8 x 4 fragments with ds_read_b128. A weight is dequantized once per workgroup: (code - 8) * d + offset in
