@@ -22,7 +22,7 @@ struct oxhip_moe {
 
 namespace {
 
-bool mfma_format(const oxhip_weight* w) { return w->v.fmt == FMT_Q8_0 || w->v.fmt == FMT_Q4_K || w->v.fmt == FMT_Q4M; }
+bool mfma_format(const oxhip_weight* w) { return w->v.fmt == FMT_Q8_0 || w->v.fmt == FMT_Q4_K || t4m_format(w->v.fmt); }
 
 size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 
@@ -214,7 +214,7 @@ oxhip_moe* oxhip_upload_moe(oxhip_ctx* c, const oxhip_weight_desc* gate_up, cons
             if (w->v.fmt != v[0]->v.fmt || !mfma_format(w)) return false;
         return true;
     };
-    if (!same(m->gate_up) || !same(m->down) || (up && !same(m->up))) return fail("experts must share one of the formats the grouped kernel runs (Q8_0, Q4_K, MLX Q4)");
+    if (!same(m->gate_up) || !same(m->down) || (up && !same(m->up))) return fail("experts must share one of the formats the grouped kernel runs (Q8_0, Q4_K, Q4_0, MLX Q4)");
     auto table = [&](const std::vector<oxhip_weight*>& v, const uint8_t*** out) {
         std::vector<const uint8_t*> host(v.size());
         for (size_t i = 0; i < v.size(); i++) host[i] = v[i]->v.p0;

@@ -1068,6 +1068,7 @@ hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, c
         case FMT_Q8_0: return run_grouped<FMT_Q8_0>(w, xa, g, max_chunks, max_rows_per_chunk, y, s);
         case FMT_Q4_K: return run_grouped<FMT_Q4_K>(w, xa, g, max_chunks, max_rows_per_chunk, y, s);
         case FMT_Q4M: return run_grouped<FMT_Q4M>(w, xa, g, max_chunks, max_rows_per_chunk, y, s);
+        case FMT_Q40: return run_grouped<FMT_Q40>(w, xa, g, max_chunks, max_rows_per_chunk, y, s);
         default: return hipErrorInvalidValue;
     }
 }

@@ -6,7 +6,7 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-Q8_0, Q4_K = 8, 12
+Q4_0, Q8_0, Q4_K = 2, 8, 12
 
 
 @pytest.fixture(scope="module")
@@ -166,7 +166,7 @@ def test_moe_batched_equals_one_at_a_time(be, oxref, mlx_experts):
         assert np.array_equal(y1[0].view(np.uint32), y[i].view(np.uint32)), i
 
 
-@pytest.mark.parametrize("kind", [Q8_0, Q4_K])
+@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K])
 def test_moe_gguf_experts(be, oxref, kind):
     from oxinfer_amd import synth
     ne, h, inter, k = 4, 256, 256, 2
@@ -174,7 +174,7 @@ def test_moe_gguf_experts(be, oxref, kind):
     dn = [oxref.random_blocks(kind, h * inter // oxref.block_size(kind), 20 + e)[0] for e in range(ne)]
     dev = be.upload_moe([be.desc_gguf(kind, g, 2 * inter, h) for g in gu], [be.desc_gguf(kind, d, h, inter) for d in dn], h, inter)
     assert dev is not None, be.last_error()
-    for t in (1, 3, 11):
+    for t in (1, 3, 11, 40):  # (40: twenty rows per expert, chunks of 32 rows on four accumulator sets)
         x = synth.activations(t, h, 30 + t)
         _, idx, w = make_routes(oxref, t, ne, k, 40 + t)
         y = np.zeros((t, h), np.float32)
