@@ -136,6 +136,15 @@ int oxhip_dev_dequantize(oxhip_ctx* ctx, const oxhip_weight* w, size_t r0, size_
  * (`dense`, src/ggml.rs:1370): they take f32 rows `x` instead and `xa` may be NULL. */
 int oxhip_dev_decode(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa, const float* x, size_t t, float* y,
                      void* stream);
+/* oxhip_dev_decode for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc); it has no counterpart in the reference. The same kernels and the same
+ * bits as oxhip_dev_decode over the quantized formats of the matrix-core decode kernel (Q8, Q8_0, Q4_0, Q4_K, Q6_K,
+ * MLX 4-bit; 1 <= t <= 16), but the partial rows and arrival counters of shapes that slice K live in an array the
+ * library holds statically on every GPU (4 MiB + 256 KiB, kept until the process ends), and the call allocates and
+ * frees nothing on the device. Declined (0, nothing written) when the weight needs more than that: K slices x 8 x
+ * n_out floats of partial rows beyond 4 MiB, or more than 2048 row groups. All calls on one GPU share the array:
+ * calls that overlap on one GPU (other streams, other threads, other contexts) race; order them. */
+int oxhip_dev_decode_noalloc(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa, size_t t, float* y, void* stream);
 /* Several independent decode matmuls in one call (a decode step issues many small matmuls; what
  * matmul_quant_batch does for the CPU, src/kernels.rs:1937-1994). The jobs must not depend on one another: runs of
  * consecutive jobs of at most 8 tokens over Q8 / Q8_0 / Q4_K / Q6_K / MLX 4-bit weights share ONE launch (their latency chains

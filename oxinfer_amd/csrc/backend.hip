@@ -13,6 +13,21 @@ void set_error(const std::string& m) { g_err = m; }
 
 using namespace oxhip;
 
+// Scratch of the allocation-free decode entry point (oxhip_dev_decode_noalloc): partial rows of the K slices, then
+// their arrival counters. Every GPU the library runs on holds its own copy of this array until the process ends.
+constexpr size_t NOALLOC_PARTIAL_FLOATS = (size_t)1 << 20;       // 4 MiB
+constexpr size_t NOALLOC_COUNTERS = (size_t)2048 * CTR_STRIDE;   // 2048 row groups, a 128-byte line each: 256 KiB
+static __device__ __align__(256) unsigned char scratch[NOALLOC_PARTIAL_FLOATS * 4 + NOALLOC_COUNTERS * 4];
+// The array's address on each device (the name above is only a host-side stand-in for it), looked up by oxhip_open.
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static void* g_scratch_ptr[NOALLOC_MAX_DEVICES];
+static std::mutex g_scratch_mu;
+
+__global__ void fill_zero_kernel(uint32_t* p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
 namespace {
 
 struct Planes {
@@ -64,6 +79,14 @@ int oxhip_open(int device, oxhip_ctx** out) {
         return 0;
     }
     HIP_TRY(hipSetDevice(device), "hipSetDevice");
+    if (device < NOALLOC_MAX_DEVICES) {  // once per device, with that device current
+        std::lock_guard<std::mutex> g(g_scratch_mu);
+        if (!g_scratch_ptr[device]) {
+            void* ptr = nullptr;
+            HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+            g_scratch_ptr[device] = ptr;
+        }
+    }
     hipDeviceProp_t prop;
     HIP_TRY(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties");
     std::string arch = prop.gcnArchName;
@@ -407,6 +430,48 @@ static int decode_one(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa,
 
 int oxhip_dev_decode(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa, const float* x, size_t t, float* y, void* stream) {
     return decode_one(c, w, xa, x, t, y, stream, nullptr, nullptr);
+}
+
+int oxhip_dev_decode_noalloc(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa, size_t t, float* y, void* stream) {
+    if (!c || !w || !xa || !y || t == 0 || t > 16) {
+        set_error("decode_noalloc: bad arguments (1 <= t <= 16)");
+        return 0;
+    }
+    if (!mfma_decode_format(w->v.fmt)) {
+        set_error("decode_noalloc: only the quantized formats of the matrix-core decode kernel (Q8, Q8_0, Q4_0, Q4_K, Q6_K, MLX 4-bit)");
+        return 0;
+    }
+    if (xa->n_in != w->v.n_in || xa->t < t) {
+        set_error("decode_noalloc: quantized activations of another shape");
+        return 0;
+    }
+    void* ptr = c->device < NOALLOC_MAX_DEVICES ? g_scratch_ptr[c->device] : nullptr;
+    if (!ptr) {
+        set_error("decode_noalloc: no static scratch on device " + std::to_string(c->device));
+        return 0;
+    }
+    size_t need_p = 0, need_c = 0;
+    decode_scratch_need(w->v, &need_p, &need_c);
+    if (need_p > NOALLOC_PARTIAL_FLOATS || need_c > NOALLOC_COUNTERS) {
+        set_error("decode_noalloc: [" + std::to_string(w->v.n_out) + ", " + std::to_string(w->v.n_in) + "] needs " + std::to_string(need_p * 4) +
+                  " bytes of partial rows and " + std::to_string(need_c / CTR_STRIDE) + " row-group counters; the static scratch holds " +
+                  std::to_string(NOALLOC_PARTIAL_FLOATS * 4) + " bytes and " + std::to_string(NOALLOC_COUNTERS / CTR_STRIDE) + " counters");
+        return 0;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    DecodeScratch sc;
+    sc.partial = static_cast<float*>(ptr);
+    sc.counters = reinterpret_cast<uint32_t*>(static_cast<unsigned char*>(ptr) + NOALLOC_PARTIAL_FLOATS * 4);
+    sc.partial_floats = NOALLOC_PARTIAL_FLOATS;
+    sc.ncounters = NOALLOC_COUNTERS;
+    if (need_c) {
+        // the array keeps what the last call (of any caller on this GPU) left: the counters must start at zero. A small
+        // kernel, not a memset: memset nodes captured into a graph have replayed wrongly.
+        fill_zero_kernel<<<(unsigned)((need_c + 255) / 256), 256, 0, s>>>(sc.counters, need_c);
+        HIP_TRY(hipGetLastError(), "decode_noalloc: counter clear launch");
+    }
+    HIP_TRY(launch_decode_mfma(w->v, view_of(*xa), t, y, sc, s), "decode_noalloc launch");
+    return 1;
 }
 
 int oxhip_dev_decode_batch(oxhip_ctx* c, const oxhip_decode_job* jobs, size_t n_jobs, void* stream) {

@@ -971,6 +971,18 @@ bool decode_batchable(const WeightView& w, size_t t) {
     return alds && lds <= LDS_MAX;
 }
 
+// Scratch a launch of this weight alone takes when its shape slices K across workgroups (floats of partial rows,
+// arrival counters); both zero when K stays inside a workgroup.
+void decode_scratch_need(const WeightView& w, size_t* partial_floats, size_t* ncounters) {
+    *partial_floats = *ncounters = 0;
+    if (!mfma_decode_format(w.fmt)) return;
+    const uint32_t ntiles = row_tiles(w.n_out);
+    const Shape sh = shape_for(ntiles, steps_rt(w), true, w.fmt);
+    if (sh.ks <= 1) return;
+    *partial_floats = (size_t)sh.ks * 8 * w.n_out;
+    *ncounters = (size_t)((ntiles + sh.rt - 1) / sh.rt) * CTR_STRIDE;
+}
+
 // Every item must be decode_batchable. Items go out in launches of up to BATCH_MAX jobs; jobs whose shape slices K
 // across workgroups take their partial rows and counters from `sc` (hipErrorOutOfMemory when it is too small:
 // nothing has been launched then and the caller launches the jobs one by one).

@@ -102,6 +102,7 @@ struct DecodeBatchItem {
     float* y;
     uint32_t t;
 };
+void decode_scratch_need(const WeightView& w, size_t* partial_floats, size_t* ncounters);  // of a launch that slices K; else zeros
 bool decode_batchable(const WeightView& w, size_t t);  // the kernel takes it and its activations fit LDS
 // ev_start / ev_stop (optional): timing events around the launches.
 hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s, hipEvent_t ev_start = nullptr,

@@ -76,6 +76,7 @@ def load_library():
         "oxhip_dev_quantize_act": (C.c_int, [vp, vp, sz, sz, C.POINTER(QActC), vp]),
         "oxhip_dev_dequantize": (C.c_int, [vp, vp, sz, sz, vp, vp]),
         "oxhip_dev_decode": (C.c_int, [vp, vp, C.POINTER(QActC), vp, sz, vp, vp]),
+        "oxhip_dev_decode_noalloc": (C.c_int, [vp, vp, C.POINTER(QActC), sz, vp, vp]),
         "oxhip_dev_isums": (C.c_int, [vp, vp, C.POINTER(QActC), vp, vp]),
         "oxhip_dev_decode_batch": (C.c_int, [vp, C.POINTER(DecodeJob), sz, vp]),
         "oxhip_dev_gemm": (C.c_int, [vp, vp, vp, C.c_int, sz, vp, C.c_int, C.c_int, vp]),
@@ -327,6 +328,15 @@ class HipBackend:
         if not ok:
             raise RuntimeError(self.last_error())
         return y
+
+    def decode_noalloc(self, w, xa, t=None, y=None):
+        """oxhip_dev_decode_noalloc: the decode kernels over the library's static scratch. False = declined."""
+        import torch
+        t = t or xa.t
+        if y is None:
+            y = torch.empty((t, w.n_out), dtype=torch.float32, device=f"cuda:{self.device}")
+        ok = self.lib.oxhip_dev_decode_noalloc(self.ctx, w.handle, C.byref(xa.c), t, y.data_ptr(), self._stream())
+        return y if ok else None
 
     def decode_jobs(self, jobs):
         """Builds a reusable job array for decode_batch: jobs = [(DeviceWeight, QAct | None, x | None, t, y, ev0, ev1)]."""
