@@ -102,12 +102,21 @@ int oxhip_matmul(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_jo
 /* Backend::matvec_rows (src/gpu.rs:165): t in 1..=4. */
 int oxhip_matvec_rows(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_rows_job* jobs, size_t n_jobs);
 
-/* Backend::upload_moe / upload_moe_transient (src/gpu.rs:206-231): expert e has gate_up[e]
- * ([2*inter, h] fused, or [inter, h] when `up` is given) and down[e] ([h, inter]). */
+/* Backend::upload_moe (src/gpu.rs:206-216): expert e has gate_up[e] ([2*inter, h] fused, or [inter, h] when `up` is
+ * given) and down[e] ([h, inter]). Backend::upload_moe_transient (src/gpu.rs:221-231: experts uploaded for one pass and
+ * dropped after it) is this call followed by oxhip_free_moe once the pass has returned: uploads here never share or
+ * cache device memory between calls, so a transient layer costs exactly its upload and nothing stays behind. */
 oxhip_moe* oxhip_upload_moe(oxhip_ctx* ctx, const oxhip_weight_desc* gate_up, const oxhip_weight_desc* up,
                             const oxhip_weight_desc* down, size_t n_experts, size_t h, size_t inter,
                             uint32_t act_kind, float act_param);
 void oxhip_free_moe(oxhip_ctx* ctx, oxhip_moe* m);
+/* The arithmetic of prefill-sized passes (a property of the layer, as `act` is; the reference picks by token count
+ * alone, src/moe.rs:625-640): OXHIP_MOE_AUTO follows the reference's split (decode-sized passes on int8 activations,
+ * passes with six or more routed rows per expert over MLX 4-bit experts on the exact rows, bf16 matrix cores);
+ * OXHIP_MOE_INT8 keeps the integer kernels (int8 activations, exact int32 block sums) at every size. Must not overlap
+ * a pass over the same oxhip_moe. */
+enum { OXHIP_MOE_AUTO = 0, OXHIP_MOE_INT8 = 1 };
+int oxhip_moe_set_mode(oxhip_moe* m, uint32_t mode);
 /* Backend::moe (src/gpu.rs:237-248) with `routes` flattened as CUDA's moe_run does
  * (src/cuda.rs:802-838): token i goes through experts route_idx[i*k .. i*k+k] with weights
  * route_w[...]; y[i] += sum_j w_j * down(act(gate x) * up x), in route order. */
@@ -199,7 +208,7 @@ int oxhip_dev_route_top_k(oxhip_ctx* ctx, const float* logits, size_t t, size_t 
  * int8 activations (Experts::forward / forward_batched, src/moe.rs:438-617; within 1e-3 of them); passes with six
  * or more routed rows per expert over MLX 4-bit experts run the grouped matmuls on the bf16 matrix cores over the
  * exact rows with Act::scalar between them, which is the reference's grouped prefill form (src/moe.rs:735-827;
- * within 2e-2 of it: the rows and the activation's output are rounded to bf16). OXHIP_MOE_INT8=1 in the environment
+ * within 2e-2 of it: the rows and the activation's output are rounded to bf16); oxhip_moe_set_mode(m, OXHIP_MOE_INT8)
  * keeps the integer kernels at every size. The scratch it needs lives in
  * `m` and grows on first use (a call with a larger t * k than any before synchronizes and
  * reallocates); calls on one oxhip_moe must not overlap. */

@@ -581,18 +581,17 @@ int oxhip_matmul(oxhip_ctx* c, const float* x, size_t t, size_t n_in, oxhip_job*
         set_error("matmul: device memory short");
         return 0;
     }
-    hipEvent_t e0, e1, e2, e3;
-    HIP_TRY(hipEventCreate(&e0), "event");
-    HIP_TRY(hipEventCreate(&e1), "event");
-    HIP_TRY(hipEventCreate(&e2), "event");
-    HIP_TRY(hipEventCreate(&e3), "event");
+    hipEvent_t e0 = nullptr, e1 = nullptr, e2 = nullptr, e3 = nullptr;
     auto done = [&](int rc) {
-        (void)hipEventDestroy(e0);
-        (void)hipEventDestroy(e1);
-        (void)hipEventDestroy(e2);
-        (void)hipEventDestroy(e3);
+        for (hipEvent_t e : {e0, e1, e2, e3})
+            if (e) (void)hipEventDestroy(e);
         return rc;
     };
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess || hipEventCreate(&e2) != hipSuccess ||
+        hipEventCreate(&e3) != hipSuccess) {
+        set_error("matmul: hipEventCreate failed");
+        return done(0);
+    }
     // Everything is computed into device staging first; y is written only once all jobs ran.
     (void)hipEventRecord(e0, s);
     if (hipMemcpyAsync(c->x.p, x, t * n_in * 4, hipMemcpyHostToDevice, s) != hipSuccess) {

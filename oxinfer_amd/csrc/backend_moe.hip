@@ -18,6 +18,7 @@ struct oxhip_moe {
     const uint8_t** bases_dn = nullptr;
     DevBuf ws;                           // scratch of one pass
     size_t ws_pairs = 0, ws_t = 0;
+    uint32_t mode = OXHIP_MOE_AUTO;      // oxhip_moe_set_mode
 };
 
 namespace {
@@ -43,10 +44,12 @@ struct Scratch {
     size_t bytes;
 };
 
-// (sized for chunks of 8 rows, the most there can be)
+// The chunk table holds the most chunks any plan can cut: an expert with c routed rows yields ceil(c / rows per chunk)
+// chunks, at most c of them (chunks of one row, a one-token pass) plus one per expert in use. Every part grows with t
+// and pairs, so a buffer sized for the largest of each serves any smaller pass.
 Scratch carve(uint8_t* base, size_t t, size_t pairs, size_t n_exp, size_t h, size_t inter) {
     Scratch s{};
-    s.max_chunks = (uint32_t)((pairs < n_exp ? pairs : n_exp) + pairs / 8 + 1);
+    s.max_chunks = (uint32_t)((pairs < n_exp ? pairs : n_exp) + pairs + 1);
     size_t off = 0;
     auto take = [&](size_t bytes) {
         uint8_t* p = base ? base + off : nullptr;
@@ -92,18 +95,32 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
     uint32_t max_rows = (uint32_t)(t < 8 ? t : 8);
     const size_t avg = pairs / m->n_exp;
     if (avg >= 6 && mfma_format(m->gate_up[0])) max_rows = avg >= 20 ? 32 : 16;
-    if (const char* e = getenv("OXHIP_MOE_CHUNK")) {  // developer override for tuning runs
+#ifdef OXHIP_TUNING  // tuning builds only: rows per chunk in OXHIP_MOE_CHUNK
+    if (const char* e = getenv("OXHIP_MOE_CHUNK")) {
         const int v = atoi(e);
         if ((v == 8 || v == 16 || v == 32) && t >= 8) max_rows = (uint32_t)v;
     }
+#endif
     // Prefill passes over MLX 4-bit experts (six or more routed rows per expert on average) take the bf16 form: see
-    // moe_bf16.hip. OXHIP_MOE_INT8=1 keeps the integer path (the 1e-3 accuracy class) at any size.
+    // moe_bf16.hip. OXHIP_MOE_INT8 (oxhip_moe_set_mode) keeps the integer path (the 1e-3 accuracy class) at any size.
     const bool fused = m->up.empty();
-    const char* keep_int = getenv("OXHIP_MOE_INT8");
     const size_t grid_chunks16 = (pairs < m->n_exp ? pairs : m->n_exp) + pairs / 16 + 1;
-    const bool bf16_form = avg >= 6 && fused && moe_bf16_ok(m->gate_up[0]->v) && moe_bf16_ok(m->down[0]->v) && !(keep_int && keep_int[0] == '1') &&
+    const bool bf16_form = avg >= 6 && fused && moe_bf16_ok(m->gate_up[0]->v) && moe_bf16_ok(m->down[0]->v) && m->mode != OXHIP_MOE_INT8 &&
                            reinterpret_cast<uintptr_t>(x) % 16 == 0 && grid_chunks16 <= 65535;
     if (bf16_form) max_rows = 16;
+    if (!bf16_form) {
+        // The grouped integer kernel stages a chunk's activations in LDS, one set per group of 8 rows: long rows take
+        // smaller chunks (checked for every projection before anything is launched).
+        auto fits = [&](uint32_t rows) {
+            return decode_grouped_fits(m->gate_up[0]->v, rows) && decode_grouped_fits(m->down[0]->v, rows) &&
+                   (fused || decode_grouped_fits(m->up[0]->v, rows));
+        };
+        while (max_rows > 8 && !fits(max_rows)) max_rows /= 2;
+        if (!fits(max_rows)) {
+            set_error("moe: rows of these experts are too long for the grouped kernel's staging");
+            return 0;
+        }
+    }
     const uint32_t grid_chunks = (uint32_t)((pairs < m->n_exp ? pairs : m->n_exp) + pairs / max_rows + 1);
     GroupView g{};
     g.chunks = sc.chunks;
@@ -224,6 +241,15 @@ oxhip_moe* oxhip_upload_moe(oxhip_ctx* c, const oxhip_weight_desc* gate_up, cons
     if (!table(m->gate_up, &m->bases_gu) || !table(m->down, &m->bases_dn) || (up && !table(m->up, &m->bases_up)))
         return fail("device memory short");
     return m;
+}
+
+int oxhip_moe_set_mode(oxhip_moe* m, uint32_t mode) {
+    if (!m || mode > OXHIP_MOE_INT8) {
+        set_error("moe_set_mode: bad arguments");
+        return 0;
+    }
+    m->mode = mode;
+    return 1;
 }
 
 int oxhip_dev_route_top_k(oxhip_ctx* c, const float* logits, size_t t, size_t n_experts, size_t k, uint32_t* idx, float* w, void* stream) {

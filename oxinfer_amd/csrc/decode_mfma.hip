@@ -799,16 +799,18 @@ Shape search_shape(uint32_t ntiles, uint32_t nsteps, uint32_t cols_per_step, dou
                 }
             }
     }
-    if (const char* e = getenv("OXHIP_DECODE_SHAPE")) {  // developer override for tuning runs: "tiles:steps=rt,kw,ks;..."
+#ifdef OXHIP_TUNING  // tuning builds only (never the shipped library): "tiles:steps=rt,kw,ks;..." in OXHIP_DECODE_SHAPE
+    if (const char* e = getenv("OXHIP_DECODE_SHAPE")) {
         for (const char* p = e; p && *p;) {
             unsigned nt = 0, ns = 0, a = 0, b = 0, c = 0;
             if (sscanf(p, "%u:%u=%u,%u,%u", &nt, &ns, &a, &b, &c) == 5 && nt == ntiles && ns == nsteps && a >= 1 && b >= 1 && c >= 1 &&
-                (b & (b - 1)) == 0 && (c & (c - 1)) == 0 && a * b <= 16)  // kw and ks: powers of two
+                (b & (b - 1)) == 0 && (c & (c - 1)) == 0 && a * b <= 16 && c <= 32 && (nsteps + c - 1) / c * (c - 1) < nsteps)  // kw, ks: powers of two; no empty slice
                 best = Shape{a, b, c};
             p = strchr(p, ';');
             if (p) p++;
         }
     }
+#endif
     return best;
 }
 
@@ -821,7 +823,9 @@ Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices, int fmt) {
     const double bytes_per_col = q8_format(fmt) ? (double)T8_REC / 64 : (double)TK4_REC / 256;
     static std::mutex mu;
     static std::map<uint64_t, Shape> cache;
-    const uint64_t key = ((uint64_t)ntiles << 36) | ((uint64_t)nsteps << 4) | ((uint64_t)(fmt & 7) << 1) | (allow_slices ? 1u : 0u);
+    // ntiles and nsteps are below 2^27 (n_out, n_in < 2^31): 27 + 27 + 8 bits of format + 1
+    static_assert(FMT_Q40 < 256, "the key keeps 8 bits of the format");
+    const uint64_t key = ((uint64_t)ntiles << 36) | ((uint64_t)nsteps << 9) | ((uint64_t)(fmt & 0xFF) << 1) | (allow_slices ? 1u : 0u);
     std::lock_guard<std::mutex> g(mu);
     auto it = cache.find(key);
     if (it != cache.end()) return it->second;
@@ -932,10 +936,12 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
     uint32_t gkw = 1;
     while (gkw < 8 && nsteps / (gkw * 2) >= 16) gkw *= 2;
     Shape sh{8 / gkw, gkw, 1};
-    if (const char* e = getenv("OXHIP_GROUPED_SHAPE")) {  // developer override for tuning runs: "rt,kw"
+#ifdef OXHIP_TUNING  // tuning builds only: "rt,kw" in OXHIP_GROUPED_SHAPE
+    if (const char* e = getenv("OXHIP_GROUPED_SHAPE")) {
         unsigned a = 0, b = 0;
-        if (sscanf(e, "%u,%u", &a, &b) == 2 && a >= 1 && b >= 1 && (b & (b - 1)) == 0 && a * b <= 16) sh = Shape{a, b, 1};
+        if (sscanf(e, "%u,%u", &a, &b) == 2 && a >= 1 && b >= 1 && (b & (b - 1)) == 0 && a * b <= 8) sh = Shape{a, b, 1};
     }
+#endif
     dim3 grid((ntiles + sh.rt - 1) / sh.rt, max_chunks), block(64 * sh.rt * sh.kw);
     const int tpad = max_rows <= 4 ? 4 : 8;
     const uint32_t ng = max_rows <= 8 ? 1 : (max_rows <= 16 ? 2 : 4);
@@ -1071,6 +1077,19 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     }
     if (!ride && ev_stop) return hipEventRecord(ev_stop, s);
     return hipSuccess;
+}
+
+// Whether a grouped launch with chunks of up to max_rows rows fits this weight's staged activations into LDS.
+bool decode_grouped_fits(const WeightView& w, uint32_t max_rows) {
+    if (!mfma_decode_format(w.fmt) || max_rows < 1 || max_rows > 32) return false;
+    const uint32_t nsteps = steps_rt(w);
+    uint32_t gkw = 1;
+    while (gkw < 8 && nsteps / (gkw * 2) >= 16) gkw *= 2;
+    const Shape sh{8 / gkw, gkw, 1};
+    const uint32_t ng = max_rows <= 8 ? 1 : (max_rows <= 16 ? 2 : 4);
+    bool alds;
+    const size_t lds = lds_bytes(!q8_format(w.fmt), false, q8_format(w.fmt) ? 2 : 4, nsteps, max_rows <= 4 ? 4 : 8, sh, &alds, ng);
+    return lds <= LDS_MAX && (alds || (ng == 1 && w.fmt != FMT_Q6_K));
 }
 
 hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks,

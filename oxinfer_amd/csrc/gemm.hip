@@ -185,7 +185,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
         } else {
             const uint32_t row = min(tile * 16 + n, w.n_out - 1);
             wbase[i] = w.p0 + fp8_offset(w, row, 128 * (size_t)step0 + 32 * (lane >> 4));
-            sbase[i] = reinterpret_cast<const float*>(w.p1) + (size_t)(tile * 16 / w.br) * ((w.n_in + w.bc - 1) / w.bc) + step0;
+            sbase[i] = reinterpret_cast<const float*>(w.p1) + (size_t)(tile * 16 / w.br) * ((w.n_in + w.bc - 1) / w.bc);  // indexed by the absolute column block
         }
     }
     // A fragments of the wave's 4 token tiles (tiles past the end repeat the last one; their rows are not stored)
@@ -250,7 +250,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
                 const uint8_t* p = wbase[i] + (w.group == 1 ? 2048 : 128) * (size_t)s;
                 r[i].c = *reinterpret_cast<const uint4*>(p);
                 r[i].c2 = *reinterpret_cast<const uint4*>(p + 16);
-                r[i].m[0] = __float_as_uint(sbase[i][(128 * s) / w.bc]);
+                r[i].m[0] = __float_as_uint(sbase[i][(128 * (step0 + s)) / w.bc]);
             }
         }
     };

@@ -259,10 +259,12 @@ constexpr Tile TILES[] = {{2, 8, 2}, {2, 4, 1}, {2, 2, 1}};
 constexpr int NTILES = sizeof(TILES) / sizeof(TILES[0]);
 
 int pick_tile(uint32_t ntiles, uint32_t ttiles) {
-    if (const char* e = getenv("OXHIP_I8_TILE")) {  // developer override for tuning runs
+#ifdef OXHIP_TUNING  // tuning builds only: tile index in OXHIP_I8_TILE
+    if (const char* e = getenv("OXHIP_I8_TILE")) {
         const int v = atoi(e);
         if (v >= 0 && v < NTILES) return v;
     }
+#endif
     int best = 0;
     uint64_t best_cost = ~0ull;
     for (int i = 0; i < NTILES; i++) {

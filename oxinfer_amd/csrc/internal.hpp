@@ -111,6 +111,7 @@ hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t,
                               hipEvent_t ev_start = nullptr, hipEvent_t ev_stop = nullptr);
 hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks,
                                       uint32_t max_rows_per_chunk, float* y, hipStream_t s);
+bool decode_grouped_fits(const WeightView& w, uint32_t max_rows_per_chunk);  // LDS holds a chunk's staged activations
 hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* out, hipStream_t s);
 hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t n_in, const WeightView& dst, hipStream_t s);
 // off == nullptr: `sc` holds one scale per 32 (Q4_0) and the record keeps all four of a row's step

@@ -235,13 +235,15 @@ hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max
     // a wave streams a whole row of records (kw = 1) unless that leaves fewer workgroups than two per CU
     uint32_t rt = 4, kw = 1;
     while (kw < 4 && nsteps / (2 * kw) >= 4 && (uint64_t)((ntiles + (8 / kw) * rt - 1) / ((8 / kw) * rt)) * max_chunks < 512) kw *= 2;
-    if (const char* e = getenv("OXHIP_MOE_BF16")) {  // developer override for tuning runs: "rt,kw"
+#ifdef OXHIP_TUNING  // tuning builds only: "rt,kw" in OXHIP_MOE_BF16
+    if (const char* e = getenv("OXHIP_MOE_BF16")) {
         unsigned a = 0, b = 0;
         if (sscanf(e, "%u,%u", &a, &b) == 2 && (a == 2 || a == 4) && (b == 1 || b == 2 || b == 4 || b == 8) && b <= nsteps) {
             rt = a;
             kw = b;
         }
     }
+#endif
     const uint32_t ng = 8 / kw;
     const size_t red = (size_t)8 * rt * 64 * 16, fr = (size_t)nsteps * 4096, lds = fr > red ? fr : red;
     const dim3 grid((ntiles + ng * rt - 1) / (ng * rt), max_chunks);

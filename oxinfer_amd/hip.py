@@ -84,6 +84,7 @@ def load_library():
         "oxhip_matvec_rows": (C.c_int, [vp, vp, sz, sz, C.POINTER(RowsJob), sz]),
         "oxhip_upload_moe": (vp, [vp, C.POINTER(WeightDesc), C.POINTER(WeightDesc), C.POINTER(WeightDesc), sz, sz, sz, C.c_uint32, C.c_float]),
         "oxhip_free_moe": (None, [vp, vp]),
+        "oxhip_moe_set_mode": (C.c_int, [vp, C.c_uint32]),
         "oxhip_moe_forward": (C.c_int, [vp, vp, sz, sz, sz, vp, vp, sz, vp, vp]),
         "oxhip_dev_route_top_k": (C.c_int, [vp, vp, sz, sz, sz, vp, vp, vp]),
         "oxhip_dev_moe": (C.c_int, [vp, vp, vp, sz, vp, vp, sz, vp, vp]),
@@ -124,6 +125,11 @@ class DeviceMoe:
     def __init__(self, be, handle, n_exp, h, inter):
         self.be, self.handle, self.n_exp, self.h, self.inter = be, handle, n_exp, h, inter
 
+    def set_mode(self, mode):
+        """MOE_AUTO: the reference's split by pass size; MOE_INT8: the integer kernels at every size."""
+        if not load_library().oxhip_moe_set_mode(self.handle, mode):
+            raise RuntimeError(self.be.last_error())
+
     def __del__(self):
         if getattr(self, "handle", None) and self.be.ctx:
             load_library().oxhip_free_moe(self.be.ctx, self.handle)
@@ -131,6 +137,7 @@ class DeviceMoe:
 
 
 ACT_SILU, ACT_GELU_TANH, ACT_SILU_CLAMP = 0, 1, 2
+MOE_AUTO, MOE_INT8 = 0, 1
 
 
 class QAct:

@@ -266,6 +266,42 @@ def test_fp8_rows_scale_blocks(oxref, be):
     assert row_err(be.decode(w, x=dev(x)).cpu().numpy(), ref) < TOL
 
 
+@pytest.mark.parametrize("n_out,n_in", [(200, 512), (37, 1064), (4096, 4096)])
+def test_bf16_weights(be, oxref, n_out, n_in):
+    """WeightRef::Bf16 (src/gpu.rs:16): bf16 rows widen exactly (bf16_to_f32, src/kernels.rs:16-18) and the product
+    accumulates in f32 over f32 activations (matmul_multi, src/kernels.rs:59-192): dequantized rows bit for bit, outputs
+    within 1e-3 of the CPU's f32 product and of the f64 one, at every token count of the decode entry point, through
+    the host surface past it, and declined where the reference's layout cannot be met."""
+    from oxinfer_amd import synth
+    rng = np.random.default_rng(n_out + n_in)
+    wf = rng.normal(0.0, 0.02, (n_out, n_in)).astype(np.float32)
+    wf[0, :8] = [0.0, -0.0, 1.0, -1.0, 3.3895314e38, -3.3895314e38, 1e-40, 9.1835e-41]  # the extremes of bf16, subnormals
+    wf = synth.bf16_round(wf)
+    wbits = (wf.view(np.uint32) >> 16).astype(np.uint16)
+    w = be.upload_bf16(wbits, n_out, n_in)
+    assert w is not None, be.last_error()
+    got = be.dequantize(w, 0, min(n_out, 64)).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), wf[:64].view(np.uint32))
+    wf[0, :8] = 0.0  # (keep the products finite for the comparisons below)
+    wbits = (wf.view(np.uint32) >> 16).astype(np.uint16)
+    w = be.upload_bf16(wbits, n_out, n_in)
+    for t in ((1, 2, 3, 4, 5, 7, 16) if n_out < 4096 else (1, 8)):
+        x = lcg_input(t, n_in, 60 + t, oxref)
+        y = be.decode(w, x=dev(x)).cpu().numpy()
+        assert row_err(y, oxref.gemm_f32(wf, n_out, n_in, x, t)) < TOL
+        assert row_err(y, (x.astype(np.float64) @ wf.astype(np.float64).T).astype(np.float32)) < TOL
+    if n_out < 4096:
+        t = 21  # the host surface walks longer batches 16 tokens at a time
+        x = lcg_input(t, n_in, 99, oxref)
+        yh = np.full((t, n_out), np.nan, np.float32)
+        if n_in % 32 == 0:
+            assert be.matmul(x, t, n_in, [(w, yh)]), be.last_error()
+            assert row_err(yh, oxref.gemm_f32(wf, n_out, n_in, x, t)) < TOL
+        else:
+            assert not be.matmul(x, t, n_in, [(w, yh)]) and np.isnan(yh).all()
+    assert be.upload_bf16(np.zeros((3, 12), np.uint16), 3, 12) is None  # rows must be whole 16-byte units
+
+
 def test_host_matmul_matches_device_path_and_declines(be, oxref):
     from oxinfer_amd import synth
     n_in = 512
@@ -313,7 +349,7 @@ def test_upload_declines(be):
     assert be.upload_gguf(Q4_K, np.zeros(144, np.uint8), 1, 256) is not None
 
 
-@pytest.mark.parametrize("kind,n_out,n_in", [(Q8_0, 14336, 4096), (Q4_K, 14336, 4096), (Q4_K, 4096, 14336), (Q6_K, 4096, 14336)])
+@pytest.mark.parametrize("kind,n_out,n_in", [(Q8_0, 14336, 4096), (Q8_0, 4096, 14336), (Q4_K, 14336, 4096), (Q4_K, 4096, 14336), (Q6_K, 14336, 4096), (Q6_K, 4096, 14336)])
 def test_full_size_rows_against_oracle(be, oxref, kind, n_out, n_in):
     """The benchmark shapes: a sample of rows of the full-size product against the oracle, plus properties
     that hold at any size: the all-ones-activation row sums and batch invariance."""
@@ -333,6 +369,39 @@ def test_full_size_rows_against_oracle(be, oxref, kind, n_out, n_in):
     assert float((np.abs(y[:, rows] - ref).max(axis=1) / m).max()) < TOL
     y1 = be.decode(w, xa=be.quantize_act(dev(x[3:4]))).cpu().numpy()
     assert np.array_equal(y1[0].view(np.uint32), y[3].view(np.uint32))
+
+
+def test_mlx_gemv_config_shape_against_oracle(be, oxref):
+    """BASELINE configs[0] at its full size: MLX 4-bit g64 [4096, 4096] (bias = -8 scale), one token of N(0, 1). Every
+    row: the int32 block sums bit for bit, the outputs within 1e-3 of the CPU decode product (from_mlx_q4 then the Q4
+    decode kernel, src/quant.rs:518-563, src/kernels_x86.rs:447-474), the dequantized rows bit for bit; and the same
+    rows from the shared launch of a layer's four 4096 x 4096 matmuls."""
+    import torch
+    from oxinfer_amd import synth
+    n = k = 4096
+    wq, sc, bi = synth.mlx_q4(n, k, 1)
+    w = be.upload_mlx_q4(wq, sc, bi, 64, n, k)
+    assert w is not None, be.last_error()
+    q, s16, off = oxref.from_mlx_q4(wq, sc, bi, n, k, 64)
+    assert not off.any()  # bias = -8 scale: the offsets b + 8 s vanish exactly
+    got = be.dequantize(w, 1000, 1064).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), oxref.dequant_rows_q4(q, s16, off, 64, n, k, 1000, 1064).view(np.uint32))
+    x = synth.activations(1, k, 2)
+    xa = be.quantize_act(dev(x))
+    ref, isums = oxref.q4_decode(q, s16, off, 64, n, k, x, 1, want_isums=True)
+    assert np.array_equal(be.isums(w, xa, 32).cpu().numpy(), isums)
+    y = be.decode(w, xa=xa).cpu().numpy()
+    assert row_err(y, ref) < TOL
+    # against the exact f32 product over the dequantized rows: the int8 activations' own bound (src/ggml.rs:1904)
+    exact = (x.astype(np.float64) @ oxref.dequant_rows_q4(q, s16, off, 64, n, k).astype(np.float64).T).astype(np.float32)
+    assert row_err(y, exact) < 3e-2
+    ws = [w] + [be.upload_mlx_q4(*synth.mlx_q4(n, k, 10 + i), 64, n, k) for i in range(3)]
+    ys = [torch.full((1, n), float("nan"), dtype=torch.float32, device="cuda") for _ in ws]
+    be.decode_batch(be.decode_jobs([(wi, xa, None, 1, yi, None, None) for wi, yi in zip(ws, ys)]))
+    torch.cuda.synchronize()
+    assert np.array_equal(ys[0].cpu().numpy().view(np.uint32), y.view(np.uint32))
+    for wi, yi in zip(ws[1:], ys[1:]):
+        assert np.array_equal(yi.cpu().numpy().view(np.uint32), be.decode(wi, xa=xa).cpu().numpy().view(np.uint32))
 
 
 def test_decode_batch_shares_a_launch_and_keeps_the_bits(be, oxref):

@@ -133,19 +133,21 @@ def test_gemm_bf16_q8_matrix_matches_oracle(be, oxref, n_out, n_in):
         assert row_err(y, (x.astype(np.float64) @ synth.bf16_round(wf).astype(np.float64).T).astype(np.float32)) < 1e-3
 
 
+@pytest.mark.parametrize("n_out,n_in", [(14336, 4096), (4096, 14336)])
 @pytest.mark.parametrize("name", list(GGUF_KINDS))
-def test_gemm_gguf_full_size_sampled_rows(be, oxref, name):
-    """The Llama-8B MLP shape 512 x 4096 -> 14336 with GGUF weights: a sample of output rows against the oracle."""
+def test_gemm_gguf_full_size_sampled_rows(be, oxref, name, n_out, n_in):
+    """The Llama-8B MLP shapes 512 x 4096 -> 14336 and 512 x 14336 -> 4096 (the K-sliced route) with GGUF weights: a
+    sample of output rows against the oracle."""
     import torch
     from oxinfer_amd import synth
-    n_out, n_in, t = 14336, 4096, 512
+    t = 512
     kind = GGUF_KINDS[name]
     raw = gguf_raw(name, n_out, n_in, 13)
     w = be.upload_gguf(kind, raw, n_out, n_in)
     assert w is not None, be.last_error()
     x = synth.activations(t, n_in, 14, bf16=True)
     y = be.gemm(w, torch.from_numpy(x).cuda().to(torch.bfloat16)).cpu().numpy()
-    rows = np.r_[0:4, 7165:7171, n_out - 4:n_out, np.random.default_rng(1).integers(0, n_out, 18)]
+    rows = np.r_[0:4, n_out // 2 - 3:n_out // 2 + 3, n_out - 4:n_out, np.random.default_rng(1).integers(0, n_out, 18)]
     rb = oxref.row_bytes(kind, n_in)
     sub = np.concatenate([raw[r * rb:(r + 1) * rb] for r in rows])
     ref = oxref.gemm_quant(kind, sub, None, None, len(rows), n_in, x, t)
@@ -153,42 +155,66 @@ def test_gemm_gguf_full_size_sampled_rows(be, oxref, name):
     assert float((np.abs(y[:, rows] - ref).max(axis=1) / m).max()) < 2e-2
 
 
-def test_gemm_full_size_sampled_rows(be, oxref):
-    """The benchmark shape 512 x 4096 -> 14336: a sample of output rows against the oracle."""
+@pytest.mark.parametrize("n_out,n_in", [(14336, 4096), (4096, 14336)])
+def test_gemm_full_size_sampled_rows(be, oxref, n_out, n_in):
+    """BASELINE configs[2] variant (a) at both shapes, 512 x 4096 -> 14336 and 512 x 14336 -> 4096 (K sliced across
+    workgroups, slices summed by a second kernel): a sample of output rows against the oracle."""
     import torch
     from oxinfer_amd import synth
-    n_out, n_in, t = 14336, 4096, 512
+    t = 512
     wq, sc, bi = synth.mlx_q4(n_out, n_in, 11)
     w = be.upload_mlx_q4(wq, sc, bi, 64, n_out, n_in)
     assert w is not None, be.last_error()
     x = synth.activations(t, n_in, 12, bf16=True)
     y = be.gemm(w, torch.from_numpy(x).cuda().to(torch.bfloat16)).cpu().numpy()
-    rows = np.r_[0:4, 7165:7171, n_out - 4:n_out, np.random.default_rng(1).integers(0, n_out, 18)]
+    rows = np.r_[0:4, n_out // 2 - 3:n_out // 2 + 3, n_out - 4:n_out, np.random.default_rng(1).integers(0, n_out, 18)]
     q, s16, off = oxref.from_mlx_q4(wq[rows], sc[rows], bi[rows], len(rows), n_in, 64)
     ref = oxref.gemm_quant(-1, q, s16, off, len(rows), n_in, x, t)
     m = np.maximum(np.abs(y).max(axis=1), 1e-30)
     assert float((np.abs(y[:, rows] - ref).max(axis=1) / m).max()) < 2e-2
 
 
-def fp8_emulation(x, data, scales, oxref):
+def fp8_emulation(x, data, scales, oxref, rows=None):
     """What the fp8 kernel computes, in f64: activations quantized to e4m3 per token and 128 columns (scale =
-    amax / 448, RNE), exact products, both scales applied per 128 x 128 block."""
+    amax / 448, RNE), exact products, both scales applied per 128 x 128 block. `rows`: only these weight rows."""
     import torch
     t, n_in = x.shape
-    n_out = data.shape[0]
+    rows = np.arange(data.shape[0]) if rows is None else np.asarray(rows)
     table = np.array([oxref.e4m3_to_f32(b) for b in range(256)], np.float64)
-    wq = table[data]
-    y = np.zeros((t, n_out))
+    wq = table[data[rows]]
+    y = np.zeros((t, len(rows)))
     for kb in range(n_in // 128):
         xb = x[:, 128 * kb:128 * kb + 128]
         amax = np.abs(xb).max(axis=1, keepdims=True).astype(np.float32)
         inv = np.where(amax > 0, np.float32(448.0) / np.maximum(amax, np.float32(1e-38)), np.float32(0)).astype(np.float32)
         q = torch.from_numpy(np.clip(xb * inv, -448, 448).astype(np.float32)).to(torch.float8_e4m3fn).to(torch.float32).numpy().astype(np.float64)
         sxv = (amax / np.float32(448.0)).astype(np.float64)
-        for rb in range((n_out + 127) // 128):
-            rows = slice(128 * rb, min(n_out, 128 * rb + 128))
-            y[:, rows] += (q @ wq[rows, 128 * kb:128 * kb + 128].T) * sxv * float(scales[rb, kb])
+        y += (q @ wq[:, 128 * kb:128 * kb + 128].T) * sxv * scales[rows // 128, kb].astype(np.float64)[None, :]
     return y.astype(np.float32)
+
+
+# What e4m3 activations cost against the CPU's f32 product, from the format alone. An activation scaled into its
+# tile's range moves by at most half an ulp of a 3-bit mantissa, 2^-4 of its value (2^-10 of the scaled unit in the
+# subnormal range, i.e. amax * 2^-10 / 448), so every output obeys |y - ref| <= sum_k |w_k| max(2^-4 |x_k|, amax_k 2^-10 / 448).
+# With roundings independent and uniform within half an ulp the error's rms is at most 2^-4 / sqrt(3) = 0.036 of the
+# output's rms at any row length (signal and error both grow as sqrt(K)): the recipe's error does not average out, and
+# measured it is 0.02-0.035 of a row's largest output, which is why this variant cannot meet the 2e-2 bar of the bf16
+# matrix cores and is not the default.
+E4M3_HALF_ULP = 2.0 ** -4
+E4M3_RMS = E4M3_HALF_ULP / np.sqrt(3.0)
+
+
+def fp8_activation_checks(y, ref, x, wf):
+    """Asserts the two bounds above for outputs y [t, rows] against ref = x wf^T."""
+    t, n_in = x.shape
+    ax = np.abs(x).astype(np.float64)
+    tile_amax = ax.reshape(t, n_in // 128, 128).max(axis=2, keepdims=True)
+    dx = np.maximum(E4M3_HALF_ULP * ax.reshape(t, n_in // 128, 128), tile_amax * 2.0 ** -10 / 448.0).reshape(t, n_in)
+    aw = np.abs(wf).astype(np.float64)
+    bound = dx @ aw.T + 1e-3 * (ax @ aw.T)  # (f32 accumulation and the rounding of the scales)
+    assert (np.abs(y.astype(np.float64) - ref) <= bound).all()
+    rms = lambda a: float(np.sqrt(np.mean(np.square(a.astype(np.float64)))))
+    assert rms(y - ref) <= E4M3_RMS * rms(ref), rms(y - ref) / rms(ref)
 
 
 @pytest.mark.parametrize("n_out,n_in", [(200, 512), (384, 2304), (100, 128), (130, 256), (64, 640), (257, 896)])  # 1 to 18 K-blocks: every phase of the kernel's three-deep pipeline
@@ -198,6 +224,7 @@ def test_gemm_fp8_matches_oracle(be, oxref, n_out, n_in):
     data, scales = synth.fp8_e4m3(n_out, n_in, 11)
     w = be.upload_fp8(data, scales, n_out, n_in)
     assert w is not None, be.last_error()
+    wf = oxref.fp8_dequant_rows(data, scales, n_out, n_in)
     for t in (1, 17, 32, 100, 300):
         x = synth.activations(t, n_in, 60 + t, bf16=True)
         ref = oxref.gemm_quant(oxref.F8E4M3, data, scales, None, n_out, n_in, x, t)
@@ -206,17 +233,38 @@ def test_gemm_fp8_matches_oracle(be, oxref, n_out, n_in):
             # bf16 activations on the bf16 matrix cores (e4m3 x block scale rounded to bf16): the parity path
             y0 = be.gemm(w, xd, variant=0).cpu().numpy()
             assert row_err(y0, ref) < 2e-2, (t, xd.dtype)
-            # e4m3 activations on the fp8 matrix cores: exact against its own definition; against the CPU's f32
-            # product the 3 mantissa bits of every activation leave an error of a few percent of the row's
-            # magnitude that does not shrink with the row length (signal and error both grow as sqrt(K)), so this
-            # variant is an explicit choice of the caller and only sanity-bounded here
+            # e4m3 activations on the fp8 matrix cores: exact against its own definition (1e-3); against the CPU's
+            # f32 product it is held to what the e4m3 rounding of the activations allows and no more
             y = be.gemm(w, xd, variant=2).cpu().numpy()
             assert row_err(y, emu) < 1e-3, (t, xd.dtype)
-            assert row_err(y, ref) < 8e-2, (t, xd.dtype)
+            fp8_activation_checks(y, ref, x, wf)
         yb = be.gemm(w, torch.from_numpy(x).cuda(), variant=2, out_bf16=True).float().cpu().numpy()
         assert row_err(yb, emu) < 1e-2
         yb0 = be.gemm(w, torch.from_numpy(x).cuda(), variant=0, out_bf16=True).float().cpu().numpy()
         assert row_err(yb0, ref) < 2e-2
+
+
+def test_gemm_fp8_wide_scale_blocks_and_k_slices(be, oxref):
+    """Scale blocks of 128 x 256: two K-steps share a scale, and with K sliced across workgroups a slice's first step
+    may sit in the second half of a block. 64 x 4096 at 100 tokens runs sliced; 200 x 1024 does not."""
+    import torch
+    from oxinfer_amd import synth
+    for n_out, n_in, t in ((64, 4096, 100), (200, 1024, 300), (64, 4096, 24)):  # 24 tokens: the skinny kernel
+        data, _ = synth.fp8_e4m3(n_out, n_in, 71)
+        scales = np.abs(np.random.default_rng(72).normal(0.0, 0.01, (-(-n_out // 128), n_in // 256))).astype(np.float32)
+        w = be.upload_fp8(data, scales, n_out, n_in, block=(128, 256))
+        assert w is not None, be.last_error()
+        want = oxref.fp8_dequant_rows(data, scales, n_out, n_in, 128, 256)
+        assert np.array_equal(be.dequantize(w).cpu().numpy().view(np.uint32), want.view(np.uint32))
+        x = synth.activations(t, n_in, 73, bf16=True)
+        ref = oxref.gemm_quant(oxref.F8E4M3, data, scales, None, n_out, n_in, x, t, brows=128, bcols=256)
+        y = be.gemm(w, torch.from_numpy(x).cuda().to(torch.bfloat16), variant=0).cpu().numpy()
+        assert row_err(y, ref) < 2e-2, (n_out, n_in, t)
+        xb, wb = x.astype(np.float64), synth.bf16_round(want).astype(np.float64)
+        if t > 32:  # the GEMM rounds e4m3 x scale to bf16: tight against that product
+            assert row_err(y, (xb @ wb.T).astype(np.float32)) < 1e-3, (n_out, n_in, t)
+        y1 = be.decode(w, x=torch.from_numpy(x[:3]).cuda()).cpu().numpy()
+        assert row_err(y1, ref[:3]) < 1e-3
 
 
 def test_gemm_fp8_declines_other_shapes(be):
@@ -229,10 +277,36 @@ def test_gemm_fp8_declines_other_shapes(be):
             be.gemm(w, torch.zeros((4, 320), device="cuda"), variant=variant)
 
 
+def test_gemm_fp8_config_m1024_sampled_rows(be, oxref):
+    """BASELINE configs[4] at M = 1024, [7168, 18432]: sampled rows of both variants. bf16 activations on the bf16 matrix
+    cores within 2e-2 of the CPU's f32 product (dequantize_rows then the f32 GEMM, src/ggml.rs:433-444); the literal
+    recipe (activations to e4m3 per 1 x 128, fp8 matrix cores) within 1e-3 of its own f64 definition and within what
+    the e4m3 rounding allows of the CPU product."""
+    import torch
+    from oxinfer_amd import synth
+    n_out, n_in, m = 7168, 18432, 1024
+    data, scales = synth.fp8_e4m3(n_out, n_in, 51)
+    w = be.upload_fp8(data, scales, n_out, n_in)
+    assert w is not None, be.last_error()
+    rows = np.r_[0:3, 127:130, n_out - 3:n_out, np.random.default_rng(3).integers(0, n_out, 12)]
+    x = synth.activations(m, n_in, 52, bf16=True)
+    xd = torch.from_numpy(x).cuda().to(torch.bfloat16)
+    wf = np.stack([oxref.fp8_dequant_rows(data, scales, n_out, n_in, r0=int(r), r1=int(r) + 1)[0] for r in rows])
+    ref = oxref.gemm_f32(wf, len(rows), n_in, x, m)
+    y = be.gemm(w, xd, variant=0).cpu().numpy()
+    mx = np.maximum(np.abs(y).max(axis=1), 1e-30)
+    assert float((np.abs(y[:, rows] - ref).max(axis=1) / mx).max()) < 2e-2
+    yb = be.gemm(w, xd, variant=0, out_bf16=True).float().cpu().numpy()  # the config's output type
+    assert float((np.abs(yb[:, rows] - ref).max(axis=1) / mx).max()) < 2e-2
+    y8 = be.gemm(w, xd, variant=2).cpu().numpy()
+    assert row_err(y8[:, rows], fp8_emulation(x, data, scales, oxref, rows)) < 1e-3
+    fp8_activation_checks(y8[:, rows], ref, x, wf)
+
+
 def test_gemm_fp8_full_size_sampled_rows(be, oxref):
     """The benchmark shape [7168, 18432] at M = 32: sampled rows against the CPU's f32 product within 2e-2 (bf16
-    activations; the e4m3-activation variant is sanity-bounded), and
-    the float-stored decode path (exact f32 activations) at M = 1 within 1e-3."""
+    activations; the e4m3-activation variant within 1e-3 of its own definition and within what the e4m3 rounding of the
+    activations allows of the CPU product), and the float-stored decode path (exact f32 activations) at M = 1 within 1e-3."""
     import torch
     from oxinfer_amd import synth
     n_out, n_in = 7168, 18432
@@ -249,9 +323,8 @@ def test_gemm_fp8_full_size_sampled_rows(be, oxref):
     ref = oxref.gemm_f32(wf, len(rows), n_in, x, 32)
     m = np.maximum(np.abs(y).max(axis=1), 1e-30)
     assert float((np.abs(y[:, rows] - ref).max(axis=1) / m).max()) < 2e-2
-    e8 = float((np.abs(y8[:, rows] - ref).max(axis=1) / m).max())
-    print(f"fp8-activation variant at K=18432: {e8:.4f}")
-    assert e8 < 8e-2
+    assert row_err(y8[:, rows], fp8_emulation(x, data, scales, oxref, rows)) < 1e-3
+    fp8_activation_checks(y8[:, rows], ref, x, wf)
     y1 = be.decode(w, x=torch.from_numpy(x[:1]).cuda()).cpu().numpy()
     assert float(np.abs(y1[0, rows] - ref[0]).max() / np.abs(y1).max()) < 1e-3
 

@@ -110,7 +110,7 @@ def test_moe_mlx_matches_oracle(be, oxref, mlx_experts):
     k = 3
     dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)
     assert dev is not None, be.last_error()
-    import os
+    from oxinfer_amd import hip
     for t in (1, 2, 5, 7, 8, 19, 40):
         x = synth.activations(t, h, 300 + t)
         _, idx, w = make_routes(oxref, t, ne, k, 400 + t)
@@ -122,12 +122,12 @@ def test_moe_mlx_matches_oracle(be, oxref, mlx_experts):
         # from 8 tokens on the CPU takes its grouped f32 path (exact activations, Act::scalar)
         ref3 = oxref.moe_q4(q_gu, q_dn, 64, h, inter, x, t, idx, w, y0, decode_path=False) if t >= 8 else None
         # the integer path (int8 activations, the decode kernels' semantics) at every size
-        os.environ["OXHIP_MOE_INT8"] = "1"
+        dev.set_mode(hip.MOE_INT8)
         try:
             y = y0.copy()
             assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
         finally:
-            del os.environ["OXHIP_MOE_INT8"]
+            dev.set_mode(hip.MOE_AUTO)
         assert row_err(y - y0, ref - y0) < 1e-3, t
         if ref3 is not None:
             # int8 activations against the exact product: within the reference's own bound for them (3e-2, src/ggml.rs:1904)
@@ -221,6 +221,98 @@ def test_moe_config_shapes(be, oxref):
         assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
         ref = oxref.moe_q4(q_gu, q_dn, 64, h, inter, x, t, idx, w, y0, decode_path=decode_path)
         assert row_err(y, ref) < tol, (t, row_err(y, ref))
+
+
+@pytest.fixture(scope="module")
+def config_experts(oxref):
+    """BASELINE configs[3]: 128 experts of [1536, 2048] + [2048, 768], MLX 4-bit g64."""
+    from oxinfer_amd import synth
+    ne, h, inter = 128, 2048, 768
+    raw_gu = [synth.mlx_q4(2 * inter, h, 1100 + e) for e in range(ne)]
+    raw_dn = [synth.mlx_q4(h, inter, 1300 + e) for e in range(ne)]
+    q_gu = [oxref.from_mlx_q4(*r, 2 * inter, h, 64) for r in raw_gu]
+    q_dn = [oxref.from_mlx_q4(*r, h, inter, 64) for r in raw_dn]
+    return ne, h, inter, raw_gu, raw_dn, q_gu, q_dn
+
+
+def test_moe_config_128_experts(be, oxref, config_experts):
+    """BASELINE configs[3] at its full size: 128 experts, top-8, h 2048, inter 768, bf16-valued activations, routing
+    on the device. T = 1 (8 experts, the integer kernels) against the oracle's decode path (forward_batched,
+    src/moe.rs:438-617) within 1e-3; T = 256 (2048 routed rows, 16 per expert on average: the bf16 form) against the
+    grouped f32 path (src/moe.rs:735-827) on a sample of tokens (a token's row depends on its own routes only) within
+    1e-2, and the integer kernels at that size within the reference's bound for int8 activations (3e-2, src/ggml.rs:1904)."""
+    import torch
+    from oxinfer_amd import hip, synth
+    ne, h, inter, raw_gu, raw_dn, q_gu, q_dn = config_experts
+    k = 8
+    dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)
+    assert dev is not None, be.last_error()
+    for t in (1, 256):
+        x = synth.activations(t, h, 1500 + t, bf16=True)
+        logits = synth.router_logits(t, ne, 1600 + t)
+        idx_d, w_d = be.route_top_k(torch.from_numpy(logits).cuda(), k)
+        idx, w = idx_d.cpu().numpy().astype(np.uint32), w_d.cpu().numpy()
+        for i in range(t):  # the device's routing is the oracle's (src/moe.rs:180-193)
+            ri, rw = oxref.route_top_k(logits[i], k)
+            assert np.array_equal(idx[i], ri) and np.allclose(w[i], rw, rtol=1e-6, atol=0)
+        y = torch.zeros((t, h), dtype=torch.float32, device="cuda")
+        be.dev_moe(dev, torch.from_numpy(x).cuda(), idx_d, w_d, y)
+        y = y.cpu().numpy()
+        sample = np.arange(t) if t == 1 else np.r_[0:3, 100:103, 253:256, np.random.default_rng(5).integers(0, t, 7)]
+        xs, si, sw = np.ascontiguousarray(x[sample]), np.ascontiguousarray(idx[sample]), np.ascontiguousarray(w[sample])
+        y0 = np.zeros((len(sample), h), np.float32)
+        if t == 1:
+            ref = oxref.moe_q4(q_gu, q_dn, 64, h, inter, xs, 1, si, sw, y0, decode_path=True)
+            assert row_err(y, ref) < 1e-3, row_err(y, ref)
+        else:
+            assert len(set(idx.reshape(-1).tolist())) == ne  # every expert is in use
+            ref = oxref.moe_q4(q_gu, q_dn, 64, h, inter, xs, len(sample), si, sw, y0, decode_path=False)
+            assert row_err(y[sample], ref) < 1e-2, row_err(y[sample], ref)
+            dev.set_mode(hip.MOE_INT8)
+            try:
+                yi = torch.zeros((t, h), dtype=torch.float32, device="cuda")
+                be.dev_moe(dev, torch.from_numpy(x).cuda(), idx_d, w_d, yi)
+                yi = yi.cpu().numpy()
+            finally:
+                dev.set_mode(hip.MOE_AUTO)
+            assert row_err(yi[sample], ref) < 3e-2
+            refi = oxref.moe_q4(q_gu, q_dn, 64, h, inter, xs[:4], 4, si[:4], sw[:4], y0[:4], decode_path=True)
+            assert row_err(yi[sample[:4]], refi) < 1e-3
+
+
+def test_moe_long_rows_take_smaller_chunks(be, oxref):
+    """Experts of the Llama-8B MLP shape (h 4096, inter 14336) in GGUF Q8_0: a prefill-sized pass (20 routed rows per
+    expert and more) would take chunks of 32 rows, whose staged activations do not fit the LDS at these row lengths;
+    the pass must still run on the device, on smaller chunks, and match the oracle's decode kernels row by row."""
+    from oxinfer_amd import synth
+    ne, h, inter, k, t = 2, 4096, 14336, 2, 24
+    gu = [synth.gguf_q8_0(2 * inter, h, 2100 + e) for e in range(ne)]
+    dn = [synth.gguf_q8_0(h, inter, 2200 + e) for e in range(ne)]
+    dev = be.upload_moe([be.desc_gguf(Q8_0, g, 2 * inter, h) for g in gu], [be.desc_gguf(Q8_0, d, h, inter) for d in dn], h, inter)
+    assert dev is not None, be.last_error()
+    x = synth.activations(t, h, 2300)
+    idx = np.tile(np.array([[0, 1]], np.uint32), (t, 1))
+    w = np.tile(np.array([[0.75, 0.25]], np.float32), (t, 1))
+    y = np.zeros((t, h), np.float32)
+    assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
+    sample = [0, 7, 23]
+    ref = moe_reference(oxref, Q8_0, gu, dn, h, inter, x[sample], idx[sample], w[sample], np.zeros((len(sample), h), np.float32))
+    assert row_err(y[sample], ref) < 1e-3
+
+
+def test_moe_duplicate_routes_within_a_token(be, oxref, mlx_experts):
+    """Routes that name one expert several times (nothing in Backend::moe forbids them): one token whose eight routes all
+    go to expert 0 cuts eight one-row chunks, more than there are experts."""
+    from oxinfer_amd import synth
+    ne, h, inter, raw_gu, raw_dn, q_gu, q_dn = mlx_experts
+    dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)
+    x = synth.activations(1, h, 77)
+    idx = np.zeros((1, 8), np.uint32)
+    w = np.full((1, 8), 0.125, np.float32)
+    y = np.zeros((1, h), np.float32)
+    assert be.moe(x, 1, h, inter, idx, w, 8, dev, y), be.last_error()
+    ref = moe_reference(oxref, "mlx", q_gu, q_dn, h, inter, x, idx, w, np.zeros((1, h), np.float32))
+    assert row_err(y, ref) < 1e-3
 
 
 def test_moe_declines(be, oxref, mlx_experts):
