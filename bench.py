@@ -1,20 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-weight matmul path on one MI355X.
 
-Default workload = BASELINE.json configs[1]: GGUF GEMV at batch 1 and 8 over Llama-8B MLP shapes
-(4096->14336 and 14336->4096) in Q8_0 and Q4_K. One step = the eight matmuls of that set, each on
-the next of a rotating pool of distinct weight copies (>= 1.5 GB per format and shape) so the 256 MB
-Infinity Cache cannot serve them; activations are quantized on the device before the timed region
-(the kernels measured are the dequant-fused GEMVs). value = algorithmic bytes of a step / time.
+Headline workload = BASELINE.json configs[1]: GGUF GEMV at batch 1 and 8 over Llama-8B MLP shapes
+(4096->14336 and 14336->4096) in Q8_0 and Q4_K. One step = the activation quantization of the four inputs (one
+launch) and the eight matmuls of that set (one launch), each matmul on the next of a rotating pool of distinct
+weight copies (>= 1.5 GB per format and shape) so the 256 MB Infinity Cache cannot serve them; the f32 inputs are
+resident in HBM when the timed region starts. value = algorithmic bytes of a step / wall time per step.
 
 Prints ONE JSON line: metric / value / unit / ms_per_step and the run's parameters, `roofline` (the dominant
-kernel's algorithmic bytes or flops per launch over its mean duration by HIP events, against the published peak, and
-its measured HBM traffic) and `cpu_baseline` (the CPU restatement on the host cores, a bounded sample). `--workload`
-selects other configurations for profiling runs; the default workload is the headline one.
+kernel's algorithmic bytes per launch over its mean duration by HIP events, against the published peak, and its
+measured HBM traffic from the kept profile), `cpu_baseline` (the CPU restatement on the host cores, a bounded
+sample) and `per_config`: every other configuration of BASELINE.json measured in the same run (value, dominant
+kernel, mean time, roofline fraction, and its own CPU baseline). `--workload` runs one configuration alone (for
+profiling runs) and prints that configuration's full line.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -26,16 +29,29 @@ if ROOT not in sys.path:
 
 METRIC = "quant GEMV GB/s (% of 8 TB/s); quant GEMM TFLOPS (% MFMA peak); vs CPU"
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK = {"bf16": 2500.0, "i8": 5000.0, "fp8": 5000.0}
 POOL_BYTES = 1.5e9
 
 Q8_0, Q4_K, Q6_K = 8, 12, 14
 ROW_BYTES = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
 FMT_NAME = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
-KERNEL_FMT = {Q8_0: 1, Q4_K: 2, Q6_K: 3}  # template argument in the kernel symbol
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
-# benchmark (KiB per dispatch, FETCH_SIZE scaled by 2.000 and WRITE_SIZE by 1.000: what a 256 MiB device copy
-# reads on the same counters); the summaries of those runs are kept under profiles/.
-TRAFFIC_BYTES = {"decode_batch_kernel": 391571276, "decode_batch_kernel/q6k": 200196474}
+
+
+def profile_traffic(profile, kernel):
+    """HBM bytes per launch of `kernel` from the kept rocprofv3 summary `profiles/<profile>` (its table of scaled
+    FETCH_SIZE + WRITE_SIZE per dispatch); None when the summary or the row is missing."""
+    try:
+        text = open(os.path.join(ROOT, "profiles", profile)).read()
+    except OSError:
+        return None
+    sect = text.split("## HBM traffic", 1)
+    if len(sect) < 2:
+        return None
+    for line in sect[1].splitlines():
+        m = re.match(r"\|\s*`" + re.escape(kernel) + r"`\s*\|.*\|\s*(\d+)\s*\|\s*$", line)
+        if m:
+            return int(m.group(1))
+    return None
 
 
 def weight_bytes(kind, n_out, n_in):
@@ -65,17 +81,29 @@ def gemv_cases(kinds):
     return cases
 
 
-def cpu_baseline(cases, gens, seconds=20.0):
-    """The oracle's AVX2 restatement of the reference's x86 decode kernels, scheduled like
-    matmul_quant_multi_at over all host cores, on the same eight matmuls: best of 5 per case over rotating
-    weight copies (so the caches do not help). Tokens up to 8 take the int-dot kernels, as with
-    set_decode_max_tokens(8) in the reference's kernel_bench."""
+def best_of(fn, min_reps, seconds):
+    """Best wall time of fn(i) over at least min_reps runs and about `seconds` of them."""
+    best, reps, t_start = float("inf"), 0, time.time()
+    while reps < min_reps or (reps < 200 and time.time() - t_start < seconds):
+        t0 = time.perf_counter()
+        fn(reps)
+        best = min(best, time.perf_counter() - t0)
+        reps += 1
+    return best, reps
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# CPU baselines: the oracle's C++ restatement of the reference's x86 kernels, on all host cores (kind "port": the
+# reference is Rust and cannot be built here). Each is a bounded sample of its configuration.
+# ---------------------------------------------------------------------------------------------------------------
+def cpu_gguf_gemv(cases, gens, seconds=16.0):
+    """The AVX2 restatement of kernels_ggml_x86 scheduled like matmul_quant_multi_at over all host cores, on the same
+    eight matmuls: best of >= 5 per case over rotating weight copies (so the caches do not help). Tokens up to 8 take
+    the int-dot kernels, as with set_decode_max_tokens(8) in the reference's kernel_bench."""
     from oracle import oxref
     from oxinfer_amd import synth
     threads = oxref.hw_threads()
-    total_bytes, total_s, per = 0, 0.0, {}
-    t_start = time.time()
-    host = {}
+    total_bytes, total_s, per, host = 0, 0.0, {}, {}
     for c in cases:
         key = (c["kind"], c["n_out"], c["n_in"])
         if key not in host:
@@ -83,26 +111,103 @@ def cpu_baseline(cases, gens, seconds=20.0):
             ncopies = max(2, int(np.ceil(4.0e8 / raw.size)))  # 0.4 GB per shape: well past the host caches
             host[key] = [raw] + [raw.copy() for _ in range(ncopies - 1)]
         x = synth.activations(c["t"], c["n_in"], 5)
-        best = float("inf")
         copies = host[key]
-        reps = 0
-        while reps < 5 or (reps < 50 and time.time() - t_start < seconds * 0.1):
-            raw = copies[reps % len(copies)]
-            t0 = time.perf_counter()
-            oxref.gguf_decode(c["kind"], raw, c["n_out"], c["n_in"], x, c["t"], avx2=True, threads=threads)
-            best = min(best, time.perf_counter() - t0)
-            reps += 1
+        best, _ = best_of(lambda i: oxref.gguf_decode(c["kind"], copies[i % len(copies)], c["n_out"], c["n_in"], x, c["t"], avx2=True, threads=threads),
+                          5, seconds / len(cases))
         per[c["name"]] = round(weight_bytes(c["kind"], c["n_out"], c["n_in"]) / best / 1e9, 2)
         total_bytes += c["bytes"]
         total_s += best
     return {"value": round(total_bytes / total_s / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": "the 8 matmuls of one step, best of >=5 runs each over rotating weight copies; C++ AVX2 "
+            "sample": "the 8 matmuls of one step, best of >= 5 runs each over rotating weight copies; C++ AVX2 "
                       "restatement of kernels_ggml_x86 (int8 dot path, decode_max_tokens >= 8), activation "
                       "quantization included",
             "per_case_weight_GBs": per}
 
 
-MFMA_PEAK = {"bf16": 2500.0, "i8": 5000.0, "fp8": 5000.0}
+def cpu_mlx_gemv(seconds=3.0):
+    from oracle import oxref
+    from oxinfer_amd import synth
+    n = k = 4096
+    q, s16, off = oxref.from_mlx_q4(*synth.mlx_q4(n, k, 1), n, k, 64)
+    copies = [(q.copy(), s16.copy(), off.copy()) for _ in range(40)]  # 0.4 GB
+    x = synth.activations(1, k, 2)
+    threads = oxref.hw_threads()
+    best, reps = best_of(lambda i: oxref.q4_decode(*copies[i % len(copies)], 64, n, k, x, 1, avx2=True, threads=threads), 20, seconds)
+    nbytes = int(n * k * 0.5625) + k * 4 + n * 4
+    return {"value": round(nbytes / best / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"the whole matmul, best of {reps} runs over 40 rotating weight copies; AVX2 restatement of q4_dot_rows_tc_avx2 + add_offsets "
+                      "(src/kernels_x86.rs:476-519), activation quantization included"}
+
+
+def cpu_mlx_gemm(seconds=6.0):
+    """The x86 prefill path (dequantize 8 rows, f32 FMA GEMM; src/kernels.rs:1998-2038) over both shapes; the reference's
+    int8 GEMM is aarch64-only, so on these host cores this is the CPU path of both variants."""
+    from oracle import oxref
+    from oxinfer_amd import synth
+    threads = oxref.hw_threads()
+    total_f, total_s = 0.0, 0.0
+    for n, k in ((14336, 4096), (4096, 14336)):
+        q, s16, off = oxref.from_mlx_q4(*synth.mlx_q4(n, k, 3), n, k, 64)
+        x = synth.activations(512, k, 4, bf16=True)
+        best, _ = best_of(lambda i: oxref.gemm_quant(-1, q, s16, off, n, k, x, 512, threads=threads), 2, seconds / 2)
+        total_f += 2.0 * 512 * n * k
+        total_s += best
+    return {"value": round(total_f / total_s / 1e12, 3), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "both shapes whole, best of >= 2 runs each; restatement of matmul_quant_block_prefill + gemm_8x8_avx2 "
+                      "(dequantize 8 rows to f32, one fma chain per output)"}
+
+
+def cpu_moe(t, experts, seconds=4.0):
+    from oracle import oxref
+    from oxinfer_amd import synth
+    ne, k, h, inter = 128, 8, 2048, 768
+    q_gu = [oxref.from_mlx_q4(*g, 2 * inter, h, 64) for g in experts[0]]
+    q_dn = [oxref.from_mlx_q4(*d, h, inter, 64) for d in experts[1]]
+    x = synth.activations(t, h, 5, bf16=True)
+    logits = synth.router_logits(t, ne, 6)
+    idx = np.zeros((t, k), np.uint32)
+    w = np.zeros((t, k), np.float32)
+    for i in range(t):
+        idx[i], w[i] = oxref.route_top_k(logits[i], k)
+    y0 = np.zeros((t, h), np.float32)
+    threads = oxref.hw_threads()
+    touched = len(set(idx.reshape(-1).tolist()))
+    if t < 8:
+        fn = lambda i: oxref.moe_q4(q_gu, q_dn, 64, h, inter, x, t, idx, w, y0, decode_path=True, avx2=True, threads=threads)
+        what = "the whole pass (8 experts stay in the host caches), AVX2 int8 decode kernels in one parallel region per projection (forward_batched + matmul_quant_batch)"
+    else:
+        fn = lambda i: oxref.moe_q4(q_gu, q_dn, 64, h, inter, x, t, idx, w, y0, decode_path=False)
+        what = "the whole pass, grouped f32 path (dequantize + f32 FMA GEMM per expert, Act::scalar), experts in parallel"
+    best, reps = best_of(fn, 3, seconds)
+    nbytes = touched * int((2 * inter * h + h * inter) * 0.5625)
+    return {"value": round(nbytes / best / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{what}; best of {reps} runs", "tflops": round(2 * t * k * (2 * inter * h + h * inter) / best / 1e12, 4)}
+
+
+def cpu_fp8(m, data, scales, seconds=6.0):
+    """dequantize_rows + the f32 GEMM (float-stored matrices take the f32 path at every M, src/kernels.rs:1802). At
+    M = 1024 a quarter of the rows is timed (the work is uniform over rows) and scaled."""
+    from oracle import oxref
+    from oxinfer_amd import synth
+    n, k = data.shape
+    rows = n if m < 1024 else n // 4
+    x = synth.activations(m, k, 8, bf16=True)
+    threads = oxref.hw_threads()
+    sub = np.ascontiguousarray(data[:rows])
+    best, reps = best_of(lambda i: oxref.gemm_quant(oxref.F8E4M3, sub, scales, None, rows, k, x, m, threads=threads), 2, seconds)
+    flops = 2.0 * m * rows * k
+    hbm = m <= 64
+    val = (rows * k + m * k * 4 + m * rows * 4) / best / 1e9 if hbm else flops / best / 1e12
+    return {"value": round(val, 3), "unit": "GB/s" if hbm else "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"rows 0..{rows} of {n} (all columns), best of {reps} runs; restatement of dequantize_rows (e4m3 x block scale) + gemm_8x8_avx2"}
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# GPU legs. Each returns the configuration's full line.
+# ---------------------------------------------------------------------------------------------------------------
+def base_line(steps, warmup):
+    return {"metric": METRIC, "n_gpus": 1, "steps": steps, "warmup": warmup, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "data": "synthetic"}
 
 
 def timed_steps(torch, step, steps, warmup):
@@ -122,27 +227,28 @@ def timed_steps(torch, step, steps, warmup):
     return wall, float(np.mean([a.elapsed_time(b) for a, b in ev]))
 
 
-def other_workload(args, be, torch, synth):
-    """The other configurations of BASELINE.json, one JSON line each (profiling and per-config numbers; the default
-    workload is the headline one). Weights rotate over >= pool-gb of distinct copies where HBM bounds."""
-    base = {"metric": METRIC, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
-            "scaling": "weak", "vs_baseline": None, "data": "synthetic"}
+def make_pool(make, nbytes, pool_gb):
+    return [make() for _ in range(max(2, int(np.ceil(pool_gb * 1e9 / nbytes))))]
 
-    def pool(make, nbytes):
-        return [make() for _ in range(max(2, int(np.ceil(args.pool_gb * 1e9 / nbytes))))]
 
-    if args.workload == "mlx_gemv":                      # configs[0]: N = K = 4096, T = 1
-        n = k = 4096
-        wq, sc, bi = synth.mlx_q4(n, k, 1)
-        ws = pool(lambda: be.upload_mlx_q4(wq, sc, bi, 64, n, k), n * k * 0.5625)
-        xa = be.quantize_act(torch.from_numpy(synth.activations(1, k, 2)).cuda())
-        y = torch.empty((1, n), dtype=torch.float32, device="cuda")
-        nbytes = int(n * k * 0.5625) + k * (1 + 4 / 32 + 8 / 32) + n * 4
-        # the library's own events: for a single launch they ride on the dispatch (its start and end on the device)
-        # (on every fourth step: an event pair costs the host more than this launch takes)
-        evs = [(be.event(), be.event()) if i % 4 == 0 else (None, None) for i in range(args.steps)]
-        warm = [be.decode_jobs([(ws[i % len(ws)], xa, None, 1, y, None, None)]) for i in range(args.warmup)]
-        timed = [be.decode_jobs([(ws[(args.warmup + i) % len(ws)], xa, None, 1, y, evs[i][0], evs[i][1])]) for i in range(args.steps)]
+def bench_mlx_gemv(be, torch, synth, steps, warmup, pool_gb):
+    """configs[0]: N = K = 4096, T = 1. Three figures: the single launch over rotating copies (cold HBM; `value` and
+    `roofline`), the shared launch of a layer's four 4096 x 4096 matmuls (q/k/v/o) over rotating copies, and the
+    single launch on one copy (cache-resident)."""
+    n = k = 4096
+    wq, sc, bi = synth.mlx_q4(n, k, 1)
+    ws = make_pool(lambda: be.upload_mlx_q4(wq, sc, bi, 64, n, k), n * k * 0.5625, pool_gb)
+    x = torch.from_numpy(synth.activations(1, k, 2)).cuda()
+    xa = be.quantize_act(x)
+    ys = [torch.empty((1, n), dtype=torch.float32, device="cuda") for _ in range(4)]
+    nbytes = int(n * k * 0.5625) + k * (1 + 4 / 32 + 8 / 32) + n * 4
+
+    def run(jobs_of, per_call):
+        # the library's own events ride on the dispatch (its start and end on the device), on every fourth step: an
+        # event pair costs the host more than this launch takes
+        evs = [(be.event(), be.event()) if i % 4 == 0 else (None, None) for i in range(steps)]
+        warm = [be.decode_jobs(jobs_of(i, None, None)) for i in range(warmup)]
+        timed = [be.decode_jobs(jobs_of(warmup + i, *evs[i])) for i in range(steps)]
         for arr in warm:
             be.decode_batch(arr)
         torch.cuda.synchronize()
@@ -152,119 +258,307 @@ def other_workload(args, be, torch, synth):
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
         ms = float(np.mean([be.elapsed_ms(a, b) for a, b in evs if a is not None]))
-        ach = nbytes / (ms * 1e-3) / 1e9
-        return dict(base, value=round(nbytes * args.steps / wall / 1e9, 2), unit="GB/s", ms_per_step=round(wall / args.steps * 1e3, 5),
-                    dtype="int8", config={"workload": "configs[0]: MLX 4-bit g64 GEMV 4096 -> 4096, T = 1", "bytes_per_step": nbytes,
-                                          "events": "carried by the launch itself, on every fourth step"},
-                    roofline={"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                              "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "decode_mfma_kernel<6, 1, ...>",
-                              "bytes_per_launch": nbytes, "avg_launch_us": round(ms * 1e3, 2)})
+        return wall, ms
 
-    if args.workload == "mlx_gemm":                      # configs[2]: M = 512, both shapes, variant (a) or (b)
-        variant = {"bf16": 0, "i8": 1}[args.variant]
-        shapes = [(14336, 4096), (4096, 14336)]
-        ws, xs = [], []
-        for n, k in shapes:
-            wq, sc, bi = synth.mlx_q4(n, k, 3)
-            ws.append([be.upload_mlx_q4(wq, sc, bi, 64, n, k) for _ in range(4)])
-            xs.append(torch.from_numpy(synth.activations(512, k, 4, bf16=True)).cuda().to(torch.bfloat16))
-        flops = sum(2 * 512 * n * k for n, k in shapes)
+    single = lambda i, e0, e1: [(ws[i % len(ws)], xa, None, 1, ys[0], e0, e1)]
+    four = lambda i, e0, e1: [(ws[(4 * i + j) % len(ws)], xa, None, 1, ys[j], e0 if j == 0 else None, e1 if j == 3 else None) for j in range(4)]
+    hot = lambda i, e0, e1: [(ws[0], xa, None, 1, ys[0], e0, e1)]
+    wall, ms = run(single, 1)
+    _, ms4 = run(four, 4)
+    _, msh = run(hot, 1)
+    ach = nbytes / (ms * 1e-3) / 1e9
+    line = dict(base_line(steps, warmup), value=round(nbytes * steps / wall / 1e9, 2), unit="GB/s", ms_per_step=round(wall / steps * 1e3, 5),
+                dtype="int8", config={"workload": "configs[0]: MLX 4-bit g64 GEMV 4096 -> 4096, T = 1", "bytes_per_step": nbytes,
+                                      "events": "carried by the launch itself, on every fourth step"},
+                roofline={"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "decode_mfma_kernel<6, 1, ...>",
+                          "bytes_per_launch": nbytes, "avg_launch_us": round(ms * 1e3, 2)})
+    line["shared_launch_of_4"] = {"what": "a layer's four 4096 x 4096 matmuls (q, k, v, o) in one oxhip_dev_decode_batch launch, rotating copies (cold HBM)",
+                                  "kernel": "decode_batch_kernel", "avg_launch_us": round(ms4 * 1e3, 2), "GBs": round(4 * nbytes / (ms4 * 1e-3) / 1e9, 1),
+                                  "frac_hbm": round(4 * nbytes / (ms4 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    line["cache_resident"] = {"what": "the single launch on one weight copy (9.4 MB stays in the 256 MB Infinity Cache)",
+                              "avg_launch_us": round(msh * 1e3, 2), "GBs": round(nbytes / (msh * 1e-3) / 1e9, 1)}
+    return line
 
-        def step(i):
-            for j in range(2):
-                be.gemm(ws[j][i % 4], xs[j], variant=variant)
-        wall, ms = timed_steps(torch, step, args.steps, args.warmup)
-        ach = flops / (ms * 1e-3) / 1e12
-        peak = MFMA_PEAK[args.variant]
-        return dict(base, value=round(flops * args.steps / wall / 1e12, 2), unit="TFLOP/s", ms_per_step=round(wall / args.steps * 1e3, 5),
-                    dtype="bf16" if variant == 0 else "int8",
-                    config={"workload": f"configs[2]: MLX 4-bit g64 prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096, variant {args.variant}",
-                            "flops_per_step": flops, "events": "around the two calls of a step (activation packing + GEMM (+ K-slice sum))"},
-                    roofline={"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4),
-                              "traffic": None, "kernel": "gemm_bf16_kernel<6, false, 4>" if variant == 0 else "gemm_i8_q4m_kernel",
-                              "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3 / 2, 2)})
 
-    if args.workload == "gguf_gemm":                     # configs[1]'s weights at configs[2]'s token count: M = 512, both shapes
-        kind, gen = {"q8_0": (Q8_0, synth.gguf_q8_0), "q4_k": (Q4_K, synth.gguf_q4_k), "q6_k": (Q6_K, synth.gguf_q6_k)}[args.format]
-        shapes = [(14336, 4096), (4096, 14336)]
-        ws, xs = [], []
-        for n, k in shapes:
-            raw = gen(n, k, 3)
-            ws.append([be.upload_gguf(kind, raw, n, k) for _ in range(4)])
-            xs.append(torch.from_numpy(synth.activations(512, k, 4, bf16=True)).cuda().to(torch.bfloat16))
-        flops = sum(2 * 512 * n * k for n, k in shapes)
+def bench_mlx_gemm(be, torch, synth, steps, warmup, variant_name):
+    """configs[2]: M = 512, both shapes, variant (a) bf16 or (b) i8."""
+    variant = {"bf16": 0, "i8": 1}[variant_name]
+    shapes = [(14336, 4096), (4096, 14336)]
+    ws, xs = [], []
+    for n, k in shapes:
+        wq, sc, bi = synth.mlx_q4(n, k, 3)
+        ws.append([be.upload_mlx_q4(wq, sc, bi, 64, n, k) for _ in range(4)])
+        xs.append(torch.from_numpy(synth.activations(512, k, 4, bf16=True)).cuda().to(torch.bfloat16))
+    flops = sum(2 * 512 * n * k for n, k in shapes)
 
-        def step(i):
-            for j in range(2):
-                be.gemm(ws[j][i % 4], xs[j])
-        wall, ms = timed_steps(torch, step, args.steps, args.warmup)
-        ach = flops / (ms * 1e-3) / 1e12
-        return dict(base, value=round(flops * args.steps / wall / 1e12, 2), unit="TFLOP/s", ms_per_step=round(wall / args.steps * 1e3, 5), dtype="bf16",
-                    config={"workload": f"GGUF {args.format.upper()} prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096 (bf16 matrix cores)",
-                            "flops_per_step": flops, "events": "around the two calls of a step (activation packing + GEMM (+ K-slice sum))"},
-                    roofline={"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK["bf16"], "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK["bf16"], 4),
-                              "traffic": None, "kernel": f"gemm_bf16_kernel<{ {'q8_0': 1, 'q4_k': 2, 'q6_k': 3}[args.format]}, false, 4>",
-                              "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3 / 2, 2)})
+    def step(i):
+        for j in range(2):
+            be.gemm(ws[j][i % 4], xs[j], variant=variant)
+    wall, ms = timed_steps(torch, step, steps, warmup)
+    ach = flops / (ms * 1e-3) / 1e12
+    peak = MFMA_PEAK[variant_name]
+    roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4),
+            "traffic": None, "kernel": "gemm_bf16_kernel<6, false, 4>" if variant == 0 else "gemm_i8_q4m_kernel",
+            "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3 / 2, 2)}
+    if variant == 1:
+        # one activation scale per token and block of 32: every int8 matrix instruction (16 x 16 x 32) is followed by a
+        # conversion and a multiply-add per accumulator and the scale products, >= 8 VALU cycles-worth next to its 8:
+        # the variant's semantics bound it near a fifth of the int8 peak
+        roof["ceiling"] = {"frac_of_peak": 0.2, "why": "per-(token, 32-block) f32 rescale: >= 8 VALU instructions per mfma_i32_16x16x32_i8"}
+    return dict(base_line(steps, warmup), value=round(flops * steps / wall / 1e12, 2), unit="TFLOP/s", ms_per_step=round(wall / steps * 1e3, 5),
+                dtype="bf16" if variant == 0 else "int8",
+                config={"workload": f"configs[2]: MLX 4-bit g64 prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096, variant {variant_name}",
+                        "flops_per_step": flops, "events": "around the two calls of a step (activation packing + GEMM (+ K-slice sum))"},
+                roofline=roof)
 
-    if args.workload == "moe":                           # configs[3]: 128 experts, top-8, h = 2048, inter = 768
-        ne, k, h, inter = 128, 8, 2048, 768
-        t = args.tokens or 1
-        gu = [synth.mlx_q4(2 * inter, h, 100 + e) for e in range(ne)]
-        dn = [synth.mlx_q4(h, inter, 300 + e) for e in range(ne)]
-        expert_bytes = int((2 * inter * h + h * inter) * 0.5625)
-        devs = pool(lambda: be.upload_moe([be.desc_mlx_q4(*g, 64, 2 * inter, h) for g in gu],
-                                          [be.desc_mlx_q4(*d, 64, h, inter) for d in dn], h, inter), ne * expert_bytes)
-        x = torch.from_numpy(synth.activations(t, h, 5, bf16=True)).cuda()
-        logits = torch.from_numpy(synth.router_logits(t, ne, 6)).cuda()
-        idx, w = be.route_top_k(logits, k)
-        touched = len(set(idx.cpu().numpy().reshape(-1).tolist()))
-        y = torch.zeros((t, h), dtype=torch.float32, device="cuda")
-        nbytes = touched * expert_bytes
-        flops = 2 * t * k * (2 * inter * h + h * inter)
-        # six or more routed rows per expert: the library takes the bf16 form of the grouped matmuls (the reference's prefill form)
-        prefill_form = (t * k) // ne >= 6 and os.environ.get("OXHIP_MOE_INT8") != "1"
 
-        def step(i):
-            be.route_top_k(logits, k)
-            be.dev_moe(devs[i % len(devs)], x, idx, w, y)
-        wall, ms = timed_steps(torch, step, args.steps, args.warmup)
-        ach = nbytes / (ms * 1e-3) / 1e9
-        return dict(base, value=round(nbytes * args.steps / wall / 1e9, 2), unit="GB/s", ms_per_step=round(wall / args.steps * 1e3, 5),
-                    dtype="int8" if prefill_form is False else "bf16",
-                    config={"workload": f"configs[3]: MoE 128 experts top-8, h 2048, inter 768, MLX 4-bit g64, T = {t}",
-                            "experts_touched": touched, "bytes_per_step": nbytes, "flops_per_step": flops,
-                            "events": "around routing + the MoE call (" + ("plan + quantize, grouped gate_up, activation + quantize, grouped down, combine)"
-                                                                           if not prefill_form else "plan, bf16 fragments of x, grouped gate_up, activation as bf16 fragments, grouped down, combine)")},
-                    roofline={"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                              "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "moe_bf16_kernel<4> (grouped)" if prefill_form else "decode_mfma_kernel<6, *, false, true, true> (grouped)",
-                              "bytes_per_launch": nbytes, "avg_launch_us": round(ms * 1e3, 2)},
-                    tflops=round(flops / (ms * 1e-3) / 1e12, 2))
+def bench_gguf_gemm(be, torch, synth, steps, warmup, fmt):
+    """configs[1]'s weights at configs[2]'s token count: M = 512, both shapes."""
+    kind, gen = {"q8_0": (Q8_0, synth.gguf_q8_0), "q4_k": (Q4_K, synth.gguf_q4_k), "q6_k": (Q6_K, synth.gguf_q6_k)}[fmt]
+    shapes = [(14336, 4096), (4096, 14336)]
+    ws, xs = [], []
+    for n, k in shapes:
+        raw = gen(n, k, 3)
+        ws.append([be.upload_gguf(kind, raw, n, k) for _ in range(4)])
+        xs.append(torch.from_numpy(synth.activations(512, k, 4, bf16=True)).cuda().to(torch.bfloat16))
+    flops = sum(2 * 512 * n * k for n, k in shapes)
 
-    # configs[4]: FP8 E4M3 [7168, 18432] with 128 x 128 block scales, bf16 activations, bf16 out
+    def step(i):
+        for j in range(2):
+            be.gemm(ws[j][i % 4], xs[j])
+    wall, ms = timed_steps(torch, step, steps, warmup)
+    ach = flops / (ms * 1e-3) / 1e12
+    return dict(base_line(steps, warmup), value=round(flops * steps / wall / 1e12, 2), unit="TFLOP/s", ms_per_step=round(wall / steps * 1e3, 5), dtype="bf16",
+                config={"workload": f"GGUF {fmt.upper()} prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096 (bf16 matrix cores)",
+                        "flops_per_step": flops, "events": "around the two calls of a step (activation packing + GEMM (+ K-slice sum))"},
+                roofline={"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK["bf16"], "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK["bf16"], 4),
+                          "traffic": None, "kernel": f"gemm_bf16_kernel<{ {'q8_0': 1, 'q4_k': 2, 'q6_k': 3}[fmt]}, false, 4>",
+                          "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3 / 2, 2)})
+
+
+def moe_experts(synth):
+    ne, h, inter = 128, 2048, 768
+    return ([synth.mlx_q4(2 * inter, h, 100 + e) for e in range(ne)], [synth.mlx_q4(h, inter, 300 + e) for e in range(ne)])
+
+
+def bench_moe(be, torch, synth, steps, warmup, pool_gb, t, experts, int8=False):
+    """configs[3]: 128 experts, top-8, h = 2048, inter = 768; a step = routing + the MoE pass."""
+    from oxinfer_amd import hip
+    ne, k, h, inter = 128, 8, 2048, 768
+    gu, dn = experts
+    expert_bytes = int((2 * inter * h + h * inter) * 0.5625)
+    devs = make_pool(lambda: be.upload_moe([be.desc_mlx_q4(*g, 64, 2 * inter, h) for g in gu],
+                                           [be.desc_mlx_q4(*d, 64, h, inter) for d in dn], h, inter), ne * expert_bytes, pool_gb)
+    if int8:
+        for d in devs:
+            d.set_mode(hip.MOE_INT8)
+    x = torch.from_numpy(synth.activations(t, h, 5, bf16=True)).cuda()
+    logits = torch.from_numpy(synth.router_logits(t, ne, 6)).cuda()
+    idx, w = be.route_top_k(logits, k)
+    touched = len(set(idx.cpu().numpy().reshape(-1).tolist()))
+    y = torch.zeros((t, h), dtype=torch.float32, device="cuda")
+    nbytes = touched * expert_bytes
+    flops = 2 * t * k * (2 * inter * h + h * inter)
+    # six or more routed rows per expert: the library takes the bf16 form of the grouped matmuls (the reference's prefill form)
+    prefill_form = (t * k) // ne >= 6 and not int8
+
+    def step(i):
+        be.route_top_k(logits, k)
+        be.dev_moe(devs[i % len(devs)], x, idx, w, y)
+    wall, ms = timed_steps(torch, step, steps, warmup)
+    ach = nbytes / (ms * 1e-3) / 1e9
+    return dict(base_line(steps, warmup), value=round(nbytes * steps / wall / 1e9, 2), unit="GB/s", ms_per_step=round(wall / steps * 1e3, 5),
+                dtype="bf16" if prefill_form else "int8",
+                config={"workload": f"configs[3]: MoE 128 experts top-8, h 2048, inter 768, MLX 4-bit g64, T = {t}",
+                        "experts_touched": touched, "bytes_per_step": nbytes, "flops_per_step": flops,
+                        "events": "around routing + the MoE call"},
+                roofline={"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+                          "kernel": "moe_bf16_kernel<4> (grouped)" if prefill_form else "decode_mfma_kernel<6, *, false, true, true> (grouped)",
+                          "bytes_per_launch": nbytes, "avg_launch_us": round(ms * 1e3, 2)},
+                tflops=round(flops / (ms * 1e-3) / 1e12, 2))
+
+
+def fp8_weights(synth):
+    return synth.fp8_e4m3(7168, 18432, 7)
+
+
+def bench_fp8(be, torch, synth, steps, warmup, pool_gb, m, variant_name, weights):
+    """configs[4]: FP8 E4M3 [7168, 18432] with 128 x 128 block scales, bf16 activations, bf16 out."""
     n, k = 7168, 18432
-    m = args.tokens or 1024
-    data, scales = synth.fp8_e4m3(n, k, 7)
-    ws = pool(lambda: be.upload_fp8(data, scales, n, k), n * k)
+    data, scales = weights
+    ws = make_pool(lambda: be.upload_fp8(data, scales, n, k), n * k, pool_gb)
     x32 = torch.from_numpy(synth.activations(m, k, 8, bf16=True)).cuda()
     xb = x32.to(torch.bfloat16)
-    variant = {"bf16": 0, "fp8": 2}.get(args.variant, 0)
+    variant = {"bf16": 0, "fp8": 2}.get(variant_name, 0)
     if m <= 16:
         step = lambda i: be.decode(ws[i % len(ws)], x=x32)
         kern = "skinny_fp8_kernel<*, 1, 2, *, false> (+ pack_skinny_kernel)"
     else:
         step = lambda i: be.gemm(ws[i % len(ws)], xb, variant=variant, out_bf16=True)
         kern = ("skinny_fp8_kernel<4, 2, 1, 16, true> (+ pack_skinny_kernel, gemm_reduce_kernel)" if m <= 32 else "gemm_bf16_kernel<4, true, 4>") if variant == 0 else "gemm_fp8_kernel<true>"
-    wall, ms = timed_steps(torch, step, args.steps, args.warmup)
+    wall, ms = timed_steps(torch, step, steps, warmup)
     flops, nbytes = 2 * m * n * k, n * k + scales.size * 4 + m * k * 2 + m * n * 2
     hbm = m <= 64
     ach = nbytes / (ms * 1e-3) / 1e9 if hbm else flops / (ms * 1e-3) / 1e12
     peak = HBM_PEAK_GBS if hbm else MFMA_PEAK["bf16" if variant == 0 else "fp8"]
-    return dict(base, value=round((nbytes / 1e9 if hbm else flops / 1e12) * args.steps / wall, 2), unit="GB/s" if hbm else "TFLOP/s",
-                ms_per_step=round(wall / args.steps * 1e3, 5), dtype="fp8 weights, " + ("f32" if m <= 16 else ("bf16" if variant == 0 else "fp8")) + " activations",
-                config={"workload": f"configs[4]: FP8 E4M3 block-scaled GEMM [7168, 18432], M = {m}, variant {args.variant if m > 16 else 'decode'}",
+    return dict(base_line(steps, warmup), value=round((nbytes / 1e9 if hbm else flops / 1e12) * steps / wall, 2), unit="GB/s" if hbm else "TFLOP/s",
+                ms_per_step=round(wall / steps * 1e3, 5), dtype="fp8 weights, " + ("f32" if m <= 16 else ("bf16" if variant == 0 else "fp8")) + " activations",
+                config={"workload": f"configs[4]: FP8 E4M3 block-scaled GEMM [7168, 18432], M = {m}, variant {variant_name if m > 16 else 'decode'}",
                         "bytes_per_step": nbytes, "flops_per_step": flops},
                 roofline={"bound": "hbm" if hbm else "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "GB/s" if hbm else "TFLOP/s",
                           "frac": round(ach / peak, 4), "traffic": None, "kernel": kern, "avg_launch_us": round(ms * 1e3, 2)})
+
+
+def bench_gguf_gemv(args, be, torch, synth, kinds, gens):
+    """configs[1] (or its Q6_K counterpart): the headline line, without the CPU leg."""
+    from oxinfer_amd.hip import QAct
+    cases = gemv_cases(kinds)
+    pools = {}
+    for c in cases:
+        key = (c["kind"], c["n_out"], c["n_in"])
+        if key in pools:
+            continue
+        raw = gens[c["kind"]](c["n_out"], c["n_in"], 1)
+        pools[key] = []
+        for _ in range(max(2, int(np.ceil(args.pool_gb * 1e9 / raw.size)))):
+            w = be.upload_gguf(c["kind"], raw, c["n_out"], c["n_in"])
+            if w is None:
+                raise RuntimeError(be.last_error())
+            pools[key].append(w)
+    # the step's inputs: one f32 matrix per (batch, width), shared by the formats like a layer's gate and up share theirs
+    inputs = {}
+    for c in cases:
+        key = (c["t"], c["n_in"])
+        if key not in inputs:
+            x = torch.from_numpy(synth.activations(c["t"], c["n_in"], 5)).cuda()
+            inputs[key] = (x, QAct(c["t"], c["n_in"], x.device))
+        c["xa"] = inputs[key][1]
+        c["y"] = torch.empty((c["t"], c["n_out"]), dtype=torch.float32, device="cuda")
+        c["pool"] = pools[(c["kind"], c["n_out"], c["n_in"])]
+    qjobs = be.quantize_jobs(list(inputs.values()))
+    be.quantize_act_batch(qjobs)
+    torch.cuda.synchronize()
+
+    if args.workload == "gguf_stream":
+        # Each case alone, 192 matmuls over rotating weight copies in one call (launches of 16, back to back): what the
+        # kernel streams at when no launch boundary, ramp or tail is in the way. `value` is the mean.
+        detail, tot_b, tot_s = {}, 0.0, 0.0
+        for c in cases:
+            pool = c["pool"]
+            arr = be.decode_jobs([(pool[i % len(pool)], c["xa"], None, c["t"], c["y"], None, None) for i in range(192)])
+            be.decode_batch(arr)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            be.decode_batch(arr)
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / 192
+            detail[c["name"]] = {"us": round(us, 2), "GBs": round(c["bytes"] / us / 1e3, 1), "frac_hbm": round(c["bytes"] / us / 1e3 / HBM_PEAK_GBS, 4)}
+            tot_b += c["bytes"]
+            tot_s += us * 1e-6
+        return {"metric": METRIC, "value": round(tot_b / tot_s / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "higher_is_better": True,
+                "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+                "config": {"workload": "GGUF GEMV cases of configs[1] (and Q6_K), each as a steady stream of 192 matmuls in one call"},
+                "detail": detail}, cases
+
+    # The dominant kernel: the jobs of one call share one launch (decode_batch_kernel); that launch carries HIP events
+    # recorded by the library on the launch stream, on every `--event-every`-th step (default: every step). An event
+    # pair on a launch leaves a gap of a few microseconds before the next one; without it a launch starts in the tail of
+    # its predecessor, so its own duration reads longer.
+    dom_symbol = "decode_batch_kernel"
+    every = max(1, args.event_every)
+    n_ev = (args.steps + every - 1) // every
+    ev = [(be.event(), be.event()) for _ in range(min(n_ev, 4096))]
+
+    def jobs_for(i, timed_slot=None):
+        jobs = []
+        for n, c in enumerate(cases):
+            w = c["pool"][(2 * i + (c["t"] > 1)) % len(c["pool"])]
+            e0 = e1 = None
+            if timed_slot is not None:
+                pair = ev[timed_slot % len(ev)]
+                e0 = pair[0] if n == 0 else None
+                e1 = pair[1] if n == len(cases) - 1 else None
+            jobs.append((w, c["xa"], None, c["t"], c["y"], e0, e1))
+        return be.decode_jobs(jobs)
+
+    def run(with_quantize):
+        warm = [jobs_for(i) for i in range(args.warmup)]
+        timed = [jobs_for(args.warmup + i, i // every if i % every == 0 else None) for i in range(args.steps)]
+        for arr in warm:
+            if with_quantize:
+                be.quantize_act_batch(qjobs)
+            be.decode_batch(arr)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for arr in timed:
+            if with_quantize:
+                be.quantize_act_batch(qjobs)
+            be.decode_batch(arr)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        return elapsed, [be.elapsed_ms(a, b) for a, b in ev[:min(n_ev, len(ev))]]
+
+    elapsed_k, _ = run(False)      # the matmul launches alone (activations quantized beforehand)
+    elapsed, dom_ms = run(True)    # the whole step: quantize the four inputs, then the eight matmuls
+    step_bytes = sum(c["bytes"] for c in cases) + sum(x.numel() * 4 for x, _ in inputs.values())
+    dom_bytes = float(sum(c["bytes"] for c in cases))
+    value = step_bytes * args.steps / elapsed / 1e9
+    dom_avg_s = float(np.mean(dom_ms)) / 1e3
+    achieved = dom_bytes / dom_avg_s / 1e9
+
+    # per-case detail (untimed pass, one event pair per launch)
+    detail = {}
+    for c in cases:
+        ms = []
+        for i in range(30):
+            w = c["pool"][i % len(c["pool"])]
+            arr = be.decode_jobs([(w, c["xa"], None, c["t"], c["y"], ev[0][0], ev[0][1])])
+            be.decode_batch(arr)
+            ms.append(be.elapsed_ms(ev[0][0], ev[0][1]))
+        us = float(np.median(ms)) * 1e3
+        detail[c["name"]] = {"us": round(us, 2), "GBs": round(c["bytes"] / us / 1e3, 1),
+                             "frac_hbm": round(c["bytes"] / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+    q6k = kinds == [Q6_K]
+    traffic = profile_traffic("decode_batch_kernel_q6k_gemv.md" if q6k else "decode_batch_kernel_gguf_gemv.md", dom_symbol) if kinds in ([Q8_0, Q4_K], [Q6_K]) else None
+    out = dict(base_line(args.steps, args.warmup), value=round(value, 2), unit="GB/s", ms_per_step=round(elapsed / args.steps * 1e3, 5), dtype="int8",
+               config={"workload": "configs[1]: GGUF GEMV batch 1 and 8, Llama-8B MLP shapes 4096->14336 and 14336->4096, "
+                                   + " + ".join(FMT_NAME[k] for k in kinds),
+                       "matmuls_per_step": len(cases), "launches_per_step": 2, "bytes_per_step": step_bytes,
+                       "weight_pool_GB_per_shape": args.pool_gb,
+                       "activations": "f32 in HBM; quantize_act (int8 per 32) of the step's four inputs is one launch inside the timed step",
+                       "events": f"on the matmul launch of every {every}. step ({min(n_ev, len(ev))} timed launches)"},
+               roofline={"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": dom_symbol,
+                         "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_avg_s * 1e6, 2)},
+               frac_of_hbm_peak=round(value / HBM_PEAK_GBS, 4),
+               matmul_launches_only={"what": "the same steps with the activations quantized beforehand (the matmul launches back to back)",
+                                     "value": round(dom_bytes * args.steps / elapsed_k / 1e9, 2), "unit": "GB/s",
+                                     "ms_per_step": round(elapsed_k / args.steps * 1e3, 5)},
+               detail=detail)
+    return out, cases
+
+
+def summary(line, cpu):
+    """A configuration's entry of `per_config`."""
+    r = line["roofline"]
+    e = {"workload": line["config"]["workload"], "value": line["value"], "unit": line["unit"], "ms_per_step": line["ms_per_step"],
+         "dtype": line["dtype"], "kernel": r["kernel"], "avg_us": r["avg_launch_us"], "bound": r["bound"],
+         "roofline_frac": r["frac"], "achieved": r["achieved"], "peak": r["peak"], "steps": line["steps"]}
+    for k in ("ceiling",):
+        if k in r:
+            e[k] = r[k]
+    for k in ("shared_launch_of_4", "cache_resident", "tflops"):
+        if k in line:
+            e[k] = line[k]
+    e["cpu_baseline"] = cpu
+    if cpu and cpu["unit"] == line["unit"] and cpu["value"]:
+        e["gpu_over_cpu"] = round(r["achieved"] / cpu["value"], 1)
+    return e
 
 
 def main():
@@ -272,17 +566,20 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gguf_gemv", choices=["gguf_gemv", "gguf_gemv_q6k", "gguf_stream", "gguf_gemm", "mlx_gemv", "mlx_gemm", "moe", "fp8", "copy"],
-                    help="copy = a plain 256 MiB device copy, the known-size kernel that scales the HBM traffic counters; "
+    ap.add_argument("--workload", default="all", choices=["all", "gguf_gemv", "gguf_gemv_q6k", "gguf_stream", "gguf_gemm", "mlx_gemv", "mlx_gemm", "moe", "fp8", "copy"],
+                    help="all (default) = the headline configs[1] line with every other configuration in per_config; gguf_gemv = the headline alone; "
+                         "copy = a plain 256 MiB device copy, the known-size kernel that scales the HBM traffic counters; "
                          "gguf_stream = every GGUF case alone as a steady stream of 192 matmuls handed over in one call")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--event-every", type=int, default=1,
                     help="gguf_gemv: the launch of every n-th timed step carries the timing events (with n > 1 the launches run closer "
-                         "together: the whole-job figure rises ~3 %, and a timed launch shares the device with its predecessor's tail)")
+                         "together, and a timed launch shares the device with its predecessor's tail)")
     ap.add_argument("--pool-gb", type=float, default=POOL_BYTES / 1e9)
     ap.add_argument("--variant", default="bf16", choices=["bf16", "i8", "fp8"], help="GEMM variant of mlx_gemm / fp8")
     ap.add_argument("--format", default="q4_k", choices=["q8_0", "q4_k", "q6_k"], help="weight format of the gguf_gemm workload")
     ap.add_argument("--tokens", type=int, default=0, help="tokens of the moe (1 or 256) and fp8 (1, 32, 1024) workloads")
+    ap.add_argument("--moe-int8", action="store_true", help="moe: keep the integer kernels at every size (oxhip_moe_set_mode)")
+    ap.add_argument("--config-steps", type=int, default=40, help="all: timed steps of each per_config entry")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1 (nothing here uses a second device)", file=sys.stderr)
@@ -304,145 +601,53 @@ def main():
         print(json.dumps({"workload": "copy", "bytes_read": n, "bytes_written": n, "launches": args.warmup + args.steps}))
         return
     be = HipBackend(0)
-    if args.workload in ("mlx_gemv", "mlx_gemm", "gguf_gemm", "moe", "fp8"):
-        print(json.dumps(other_workload(args, be, torch, synth)))
-        be.close()
-        return
+    cpu = not args.no_cpu
     gens = {Q8_0: synth.gguf_q8_0, Q4_K: synth.gguf_q4_k, Q6_K: synth.gguf_q6_k}
-    kinds = [Q8_0, Q4_K] if args.workload == "gguf_gemv" else [Q6_K] if args.workload == "gguf_gemv_q6k" else [Q8_0, Q4_K, Q6_K]
-    cases = gemv_cases(kinds)
-
-    # rotating pools of distinct device copies per (format, shape)
-    pools = {}
-    for c in cases:
-        key = (c["kind"], c["n_out"], c["n_in"])
-        if key in pools:
-            continue
-        raw = gens[c["kind"]](c["n_out"], c["n_in"], 1)
-        n = max(2, int(np.ceil(args.pool_gb * 1e9 / raw.size)))
-        pools[key] = []
-        for _ in range(n):
-            w = be.upload_gguf(c["kind"], raw, c["n_out"], c["n_in"])
-            if w is None:
-                raise RuntimeError(be.last_error())
-            pools[key].append(w)
-    for c in cases:
-        x = torch.from_numpy(synth.activations(c["t"], c["n_in"], 5)).cuda()
-        c["xa"] = be.quantize_act(x)
-        c["y"] = torch.empty((c["t"], c["n_out"]), dtype=torch.float32, device="cuda")
-        c["pool"] = pools[(c["kind"], c["n_out"], c["n_in"])]
-    torch.cuda.synchronize()
-
-    if args.workload == "gguf_stream":
-        # Each case alone, 192 matmuls over rotating weight copies in one call (launches of 16, back to back): what the
-        # kernel streams at when no launch boundary, ramp or tail is in the way. One JSON line; `value` is the mean.
-        detail, tot_b, tot_s = {}, 0.0, 0.0
-        for c in cases:
-            pool = c["pool"]
-            arr = be.decode_jobs([(pool[i % len(pool)], c["xa"], None, c["t"], c["y"], None, None) for i in range(192)])
-            be.decode_batch(arr)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            be.decode_batch(arr)
-            e1.record()
-            torch.cuda.synchronize()
-            us = e0.elapsed_time(e1) * 1e3 / 192
-            detail[c["name"]] = {"us": round(us, 2), "GBs": round(c["bytes"] / us / 1e3, 1), "frac_hbm": round(c["bytes"] / us / 1e3 / HBM_PEAK_GBS, 4)}
-            tot_b += c["bytes"]
-            tot_s += us * 1e-6
-        print(json.dumps({"metric": METRIC, "value": round(tot_b / tot_s / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "higher_is_better": True,
-                          "vs_baseline": None, "dtype": "int8", "data": "synthetic",
-                          "config": {"workload": "GGUF GEMV cases of configs[1] (and Q6_K), each as a steady stream of 192 matmuls in one call"},
-                          "detail": detail}))
-        be.close()
-        return
-
-    # The dominant kernel. The jobs of one call share one launch (decode_batch_kernel): that launch is the step, and
-    # its events bracket it. (Formats the shared launch does not take would launch one by one: then the largest
-    # matmul at the larger batch is timed.)
-    shared = all(k in (Q8_0, Q4_K, Q6_K) for k in kinds)
-    dom_kind = kinds[0]
-    for c in cases:
-        c["dom"] = shared or (c["kind"] == dom_kind and c["t"] == 8)
-    dom = [c for c in cases if c["dom"]]
-    per_step = 1 if shared else len(dom)
-    dom_symbol = "decode_batch_kernel"
-
-    # One call per step: the job arrays (one per rotation phase) are built once; the dominant launches of every
-    # `--event-every`-th step (default: every step) carry HIP events recorded by the library on the launch stream. An
-    # event pair on a launch leaves a gap of a few microseconds before the next one; without it a launch starts in the
-    # tail of its predecessor, so its own duration reads longer.
-    every = max(1, args.event_every)
-    n_timed = (args.steps + every - 1) // every
-    n_ev = n_timed * per_step
-    ev = [(be.event(), be.event()) for _ in range(min(n_ev, 4096))]
-
-    def jobs_for(i, timed_slot=None):
-        jobs, k = [], 0
-        for n, c in enumerate(cases):
-            w = c["pool"][(2 * i + (c["t"] > 1)) % len(c["pool"])]
-            e0 = e1 = None
-            if timed_slot is not None and shared:
-                pair = ev[timed_slot % len(ev)]
-                e0 = pair[0] if n == 0 else None
-                e1 = pair[1] if n == len(cases) - 1 else None
-            elif timed_slot is not None and c["dom"]:
-                e0, e1 = ev[(timed_slot * per_step + k) % len(ev)]
-                k += 1
-            jobs.append((w, c["xa"], None, c["t"], c["y"], e0, e1))
-        return be.decode_jobs(jobs)
-
-    warm = [jobs_for(i) for i in range(args.warmup)]
-    timed = [jobs_for(args.warmup + i, i // every if i % every == 0 else None) for i in range(args.steps)]
-    for arr in warm:
-        be.decode_batch(arr)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for arr in timed:
-        be.decode_batch(arr)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    used = min(n_ev, len(ev))
-    dom_ms = [be.elapsed_ms(a, b) for a, b in ev[:used]]
-
-    step_bytes = sum(c["bytes"] for c in cases)
-    value = step_bytes * args.steps / elapsed / 1e9
-    dom_avg_s = float(np.mean(dom_ms)) / 1e3
-    dom_bytes = float(step_bytes) if shared else float(np.mean([c["bytes"] for c in dom]))
-    achieved = dom_bytes / dom_avg_s / 1e9
-
-    # per-case detail (untimed pass, one event pair per launch)
-    detail = {}
-    for c in cases:
-        ms = []
-        for i in range(30):
-            w = c["pool"][i % len(c["pool"])]
-            arr = be.decode_jobs([(w, c["xa"], None, c["t"], c["y"], ev[0][0], ev[0][1])])
-            be.decode_batch(arr)
-            ms.append(be.elapsed_ms(ev[0][0], ev[0][1]))
-        us = float(np.median(ms)) * 1e3
-        detail[c["name"]] = {"us": round(us, 2), "GBs": round(c["bytes"] / us / 1e3, 1),
-                             "frac_hbm": round(c["bytes"] / us / 1e3 / HBM_PEAK_GBS, 4)}
-
-    out = {
-        "metric": METRIC, "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(elapsed / args.steps * 1e3, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
-        "config": {"workload": "configs[1]: GGUF GEMV batch 1 and 8, Llama-8B MLP shapes 4096->14336 and 14336->4096, "
-                               + " + ".join(FMT_NAME[k] for k in kinds),
-                   "matmuls_per_step": len(cases), "launches_per_step": 1 if shared else len(cases), "bytes_per_step": step_bytes,
-                   "weight_pool_GB_per_shape": args.pool_gb, "activations": "int8 per 32 (quantize_act), resident in HBM",
-                   "events": f"on the launch of every {every}. step ({min(n_ev, len(ev))} timed launches)"},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES.get(dom_symbol if all(k in (Q8_0, Q4_K) for k in kinds) else dom_symbol + "/q6k"), "kernel": dom_symbol,
-                     "bytes_per_launch": dom_bytes, "avg_launch_us": round(dom_avg_s * 1e6, 2)},
-        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-        "detail": detail,
-    }
-    if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(cases, gens)
-    print(json.dumps(out))
+    w = args.workload
+    if w == "mlx_gemv":
+        line = bench_mlx_gemv(be, torch, synth, args.steps, args.warmup, args.pool_gb)
+        if cpu:
+            line["cpu_baseline"] = cpu_mlx_gemv()
+    elif w == "mlx_gemm":
+        line = bench_mlx_gemm(be, torch, synth, args.steps, args.warmup, args.variant)
+        if cpu:
+            line["cpu_baseline"] = cpu_mlx_gemm()
+    elif w == "gguf_gemm":
+        line = bench_gguf_gemm(be, torch, synth, args.steps, args.warmup, args.format)
+    elif w == "moe":
+        ex = moe_experts(synth)
+        line = bench_moe(be, torch, synth, args.steps, args.warmup, args.pool_gb, args.tokens or 1, ex, args.moe_int8)
+        if cpu:
+            line["cpu_baseline"] = cpu_moe(args.tokens or 1, ex)
+    elif w == "fp8":
+        wts = fp8_weights(synth)
+        line = bench_fp8(be, torch, synth, args.steps, args.warmup, args.pool_gb, args.tokens or 1024, args.variant, wts)
+        if cpu:
+            line["cpu_baseline"] = cpu_fp8(args.tokens or 1024, *wts)
+    else:
+        kinds = [Q6_K] if w == "gguf_gemv_q6k" else [Q8_0, Q4_K, Q6_K] if w == "gguf_stream" else [Q8_0, Q4_K]
+        line, cases = bench_gguf_gemv(args, be, torch, synth, kinds, gens)
+        if cpu and w != "gguf_stream":
+            line["cpu_baseline"] = cpu_gguf_gemv(cases, gens)
+        if w == "all":
+            # every other configuration, measured in this same run (GPU leg, then its CPU leg)
+            ks, kw = args.config_steps, max(3, args.config_steps // 8)
+            per = {}
+            l = bench_mlx_gemv(be, torch, synth, 4 * ks, 4 * kw, args.pool_gb)
+            per["configs[0] MLX GEMV T=1"] = summary(l, cpu_mlx_gemv() if cpu else None)
+            cg = cpu_mlx_gemm() if cpu else None
+            per["configs[2a] MLX GEMM M=512 bf16 MFMA"] = summary(bench_mlx_gemm(be, torch, synth, ks, kw, "bf16"), cg)
+            per["configs[2b] MLX GEMM M=512 int8 MFMA"] = summary(bench_mlx_gemm(be, torch, synth, ks, kw, "i8"), cg)
+            ex = moe_experts(synth)
+            per["configs[3] MoE T=1"] = summary(bench_moe(be, torch, synth, 2 * ks, 2 * kw, args.pool_gb, 1, ex), cpu_moe(1, ex) if cpu else None)
+            per["configs[3] MoE T=256"] = summary(bench_moe(be, torch, synth, ks, kw, args.pool_gb, 256, ex), cpu_moe(256, ex) if cpu else None)
+            del ex
+            wts = fp8_weights(synth)
+            for m in (1, 32, 1024):
+                per[f"configs[4] FP8 M={m}"] = summary(bench_fp8(be, torch, synth, ks, kw, args.pool_gb, m, "bf16", wts), cpu_fp8(m, *wts) if cpu else None)
+            per["configs[4] FP8 M=1024 fp8 MFMA"] = summary(bench_fp8(be, torch, synth, ks, kw, args.pool_gb, 1024, "fp8", wts), per["configs[4] FP8 M=1024"]["cpu_baseline"])
+            line["per_config"] = per
+    print(json.dumps(line))
     be.close()
 
 

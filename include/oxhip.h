@@ -138,6 +138,14 @@ typedef struct {
 
 /* quant::quantize_act (src/quant.rs:294-343) on device rows x [t, n_in] f32. */
 int oxhip_dev_quantize_act(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, const oxhip_qact* out, void* stream);
+/* The same for several activation matrices in one launch (a decode step quantizes the input of each group of matmuls:
+ * QAct::new per input, src/quant.rs:294-343; every launch costs its latency whatever its size). */
+typedef struct {
+    const float* x; /* device, [t, n_in] f32 */
+    size_t t, n_in;
+    const oxhip_qact* out;
+} oxhip_quant_job;
+int oxhip_dev_quantize_act_batch(oxhip_ctx* ctx, const oxhip_quant_job* jobs, size_t n_jobs, void* stream);
 /* QMat::dequantize_rows (src/kernels.rs:1336, src/ggml.rs:409-459): rows r0..r1 as f32 [r1-r0, n_in]. */
 int oxhip_dev_dequantize(oxhip_ctx* ctx, const oxhip_weight* w, size_t r0, size_t r1, float* out, void* stream);
 /* The decode kernels (QMat::rows_t1 / rows_tc, src/kernels.rs:1339-1369, src/ggml.rs:1319-1354):

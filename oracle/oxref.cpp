@@ -11,6 +11,7 @@
 #include <condition_variable>
 #include <cstring>
 #include <functional>
+#include <memory>
 #include <mutex>
 #include <thread>
 #include <vector>
@@ -1275,5 +1276,98 @@ void oxref_moe_q4(const oxref_q4_ref* gate_up, const oxref_q4_ref* down, size_t 
             const float* o = &outs[(ti * k + j) * h];
             for (size_t i = 0; i < h; i++) y[ti * h + i] += w * o[i];
         }
+}
+
+// The decode-sized MoE pass as the x86 CPU schedules it, for the timed baseline (values as oxref_moe_q4's decode
+// path up to the AVX2 kernels' f32 order): activations quantized once per expert's rows, every expert's matmul cut
+// into row blocks of one shared parallel region (matmul_quant_batch, src/kernels.rs:1937-1994), the AVX2 decode
+// kernels per block (src/kernels_x86.rs:476-519), silu_mul (src/kernels.rs:2188-2198), requantize, down, combine in
+// route order (src/moe.rs:608-615).
+void oxref_moe_q4_avx2(const oxref_q4_ref* gate_up, const oxref_q4_ref* down, size_t ne, size_t group,
+                       size_t h, size_t inter, const float* x, size_t t, const uint32_t* route_idx,
+                       const float* route_w, size_t k, float* y, int threads) {
+#if defined(__AVX2__)
+    std::vector<std::vector<std::pair<size_t, size_t>>> by(ne);
+    for (size_t ti = 0; ti < t; ti++)
+        for (size_t j = 0; j < k; j++) by[route_idx[ti * k + j]].emplace_back(ti, j);
+    std::vector<size_t> used;
+    for (size_t e = 0; e < ne; e++)
+        if (!by[e].empty()) used.push_back(e);
+    struct Job {
+        size_t e, n;
+        std::vector<float> xs, gu, a, o;
+        std::unique_ptr<QActBuf> xa, aq;
+        std::vector<std::vector<float>> gs;
+    };
+    std::vector<Job> jobs(used.size());
+    for (size_t u = 0; u < used.size(); u++) {
+        Job& jb = jobs[u];
+        jb.e = used[u];
+        jb.n = by[jb.e].size();
+        jb.xs.resize(jb.n * h);
+        for (size_t i = 0; i < jb.n; i++) std::memcpy(&jb.xs[i * h], x + by[jb.e][i].first * h, h * 4);
+        jb.xa.reset(new QActBuf(jb.xs.data(), jb.n, h));
+        jb.gu.resize(jb.n * 2 * inter);
+        jb.a.resize(jb.n * inter);
+        jb.o.resize(jb.n * h);
+    }
+    struct Block {
+        size_t u, r0, r1;
+    };
+    auto run_phase = [&](bool second) {
+        const size_t n_out = second ? h : 2 * inter, n_in = second ? inter : h;
+        const size_t bytes_per_row = n_in / 2 + n_in / 32 * 2 + n_in / group * 2;
+        const size_t rpb = rows_per_block(jobs.size() * n_out * bytes_per_row, jobs.size() * n_out, threads);
+        std::vector<Block> blocks;
+        for (size_t u = 0; u < jobs.size(); u++) {
+            Job& jb = jobs[u];
+            const QActBuf& xa = second ? *jb.aq : *jb.xa;
+            jb.gs.assign(jb.n, std::vector<float>());
+            for (size_t c = 0; c < jb.n; c++) q4_group_sums(xa, c, group, jb.gs[c]);
+            for (size_t r = 0; r < n_out; r += rpb) blocks.push_back(Block{u, r, std::min(n_out, r + rpb)});
+        }
+        pool(threads).run(blocks.size(), [&](size_t b) {
+            const Block& bl = blocks[b];
+            Job& jb = jobs[bl.u];
+            const oxref_q4_ref& w = second ? down[jb.e] : gate_up[jb.e];
+            const QActBuf& xa = second ? *jb.aq : *jb.xa;
+            float* out = second ? jb.o.data() : jb.gu.data();
+            for (size_t c = 0; c < jb.n;) {
+                size_t tc = std::min<size_t>(jb.n - c, 2);
+                if (tc == 1) q4_rows_avx2<1>(w.q, w.sc, n_out, n_in, xa, c, out, bl.r0, bl.r1);
+                else q4_rows_avx2<2>(w.q, w.sc, n_out, n_in, xa, c, out, bl.r0, bl.r1);
+                c += tc;
+            }
+            if (w.off)
+                for (size_t c = 0; c < jb.n; c++)
+                    for (size_t r = bl.r0; r < bl.r1; r++)
+                        out[c * n_out + r] += dot_bf16_lanes(w.off + r * (n_in / group), jb.gs[c].data(), n_in / group);
+        });
+    };
+    run_phase(false);
+    pool(threads).run(jobs.size(), [&](size_t u) {
+        Job& jb = jobs[u];
+        for (size_t i = 0; i < jb.n; i++) {
+            float* g = &jb.gu[i * 2 * inter];
+            oxref_silu_mul(g, g + inter, inter);
+            std::memcpy(&jb.a[i * inter], g, inter * 4);
+        }
+        jb.aq.reset(new QActBuf(jb.a.data(), jb.n, inter));
+    });
+    run_phase(true);
+    for (size_t ti = 0; ti < t; ti++)
+        for (size_t j = 0; j < k; j++) {
+            const size_t e = route_idx[ti * k + j];
+            size_t u = std::lower_bound(used.begin(), used.end(), e) - used.begin();
+            size_t i = 0;
+            while (by[e][i] != std::make_pair(ti, j)) i++;
+            const float w = route_w[ti * k + j];
+            const float* o = &jobs[u].o[i * h];
+            for (size_t c = 0; c < h; c++) y[ti * h + c] += w * o[c];
+        }
+#else
+    (void)threads;
+    oxref_moe_q4(gate_up, down, ne, group, h, inter, x, t, route_idx, route_w, k, y, 1);
+#endif
 }
 

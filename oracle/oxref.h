@@ -111,6 +111,11 @@ void oxref_moe_q4(const oxref_q4_ref* gate_up, const oxref_q4_ref* down, size_t 
                   size_t h, size_t inter, const float* x, size_t t, const uint32_t* route_idx,
                   const float* route_w, size_t k, float* y, int decode_path);
 
+/* The decode-sized pass scheduled and vectorized as the x86 CPU does it (timed baseline). */
+void oxref_moe_q4_avx2(const oxref_q4_ref* gate_up, const oxref_q4_ref* down, size_t ne, size_t group,
+                       size_t h, size_t inter, const float* x, size_t t, const uint32_t* route_idx,
+                       const float* route_w, size_t k, float* y, int threads);
+
 int oxref_hw_threads(void);
 
 #ifdef __cplusplus

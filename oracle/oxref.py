@@ -62,6 +62,7 @@ def _load():
         "oxref_silu_mul": (None, [vp, vp, sz]),
         "oxref_route_top_k": (None, [vp, sz, sz, vp, vp]),
         "oxref_moe_q4": (None, [vp, vp, sz, sz, sz, sz, vp, sz, vp, vp, sz, vp, C.c_int]),
+        "oxref_moe_q4_avx2": (None, [vp, vp, sz, sz, sz, sz, vp, sz, vp, vp, sz, vp, C.c_int]),
         "oxref_hw_threads": (C.c_int, []),
     }
     for name, (res, args) in sig.items():
@@ -288,8 +289,9 @@ class _Q4Ref(C.Structure):
     _fields_ = [("q", C.c_void_p), ("sc", C.c_void_p), ("off", C.c_void_p)]
 
 
-def moe_q4(gate_up, down, group, h, inter, x, t, route_idx, route_w, y, decode_path):
-    """gate_up / down: lists of (q, sc, off) numpy triples per expert. Adds into y ([t, h] f32) and returns it."""
+def moe_q4(gate_up, down, group, h, inter, x, t, route_idx, route_w, y, decode_path, avx2=False, threads=None):
+    """gate_up / down: lists of (q, sc, off) numpy triples per expert. Adds into y ([t, h] f32) and returns it.
+    avx2: the decode path scheduled and vectorized as the x86 CPU runs it (the timed baseline)."""
     ne = len(gate_up)
     keep = []
 
@@ -306,5 +308,9 @@ def moe_q4(gate_up, down, group, h, inter, x, t, route_idx, route_w, y, decode_p
     route_idx, route_w = _c(route_idx, np.uint32), _c(route_w, np.float32)
     k = route_idx.size // t
     y = np.array(y, np.float32, copy=True)
+    if avx2:
+        assert decode_path
+        lib.oxref_moe_q4_avx2(gu, dn, ne, group, h, inter, _p(x), t, _p(route_idx), _p(route_w), k, _p(y), threads or hw_threads())
+        return y
     lib.oxref_moe_q4(gu, dn, ne, group, h, inter, _p(x), t, _p(route_idx), _p(route_w), k, _p(y), int(decode_path))
     return y

@@ -19,6 +19,55 @@ __global__ __launch_bounds__(64) void quantize_act_kernel(const float* __restric
     quantize_act_block(x, b, q, scales, sums, fsums, hsums, sums16);
 }
 
+// Several activation matrices in one launch (a decode step quantizes the input of every group of matmuls; each launch
+// is a few microseconds of latency whatever its size).
+struct QuantBatchArgs {
+    uint32_t njobs;
+    uint32_t first[QUANT_BATCH_MAX + 1];  // first lane-block of job j; first[njobs] = total
+    const float* x[QUANT_BATCH_MAX];
+    int8_t* q[QUANT_BATCH_MAX];
+    float* scales[QUANT_BATCH_MAX];
+    int32_t* sums[QUANT_BATCH_MAX];
+    float* fsums[QUANT_BATCH_MAX];
+    float* hsums[QUANT_BATCH_MAX];
+    int32_t* sums16[QUANT_BATCH_MAX];
+};
+
+__global__ __launch_bounds__(64) void quantize_act_batch_kernel(QuantBatchArgs a) {
+    const uint32_t b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= a.first[a.njobs]) return;
+    uint32_t j = 0;
+    while (j + 1 < a.njobs && b >= a.first[j + 1]) j++;
+    quantize_act_block(a.x[j], (size_t)(b - a.first[j]), a.q[j], a.scales[j], a.sums[j], a.fsums[j], a.hsums[j], a.sums16[j]);
+}
+
+hipError_t launch_quantize_act_batch(const float* const* x, const size_t* t, const size_t* n_in, const oxhip_qact* o, size_t n, hipStream_t s) {
+    for (size_t i0 = 0; i0 < n; i0 += QUANT_BATCH_MAX) {
+        QuantBatchArgs a{};
+        a.njobs = (uint32_t)(n - i0 < (size_t)QUANT_BATCH_MAX ? n - i0 : (size_t)QUANT_BATCH_MAX);
+        uint32_t total = 0;
+        for (uint32_t j = 0; j < a.njobs; j++) {
+            const size_t nb = t[i0 + j] * n_in[i0 + j] / 32;
+            if (total + nb > 0x7FFFFFFFu) return hipErrorInvalidValue;
+            a.first[j] = total;
+            total += (uint32_t)nb;
+            a.x[j] = x[i0 + j];
+            a.q[j] = o[i0 + j].q;
+            a.scales[j] = o[i0 + j].scales;
+            a.sums[j] = o[i0 + j].sums;
+            a.fsums[j] = o[i0 + j].fsums;
+            a.hsums[j] = o[i0 + j].hsums;
+            a.sums16[j] = o[i0 + j].sums16;
+        }
+        a.first[a.njobs] = total;
+        if (!total) continue;
+        quantize_act_batch_kernel<<<(total + 63) / 64, 64, 0, s>>>(a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
 hipError_t launch_quantize_act(const float* x, size_t t, size_t n_in, const oxhip_qact& o, hipStream_t s) {
     size_t nblocks = t * n_in / 32;
     if (nblocks == 0) return hipSuccess;

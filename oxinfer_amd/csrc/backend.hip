@@ -396,6 +396,28 @@ int oxhip_dev_quantize_act(oxhip_ctx* c, const float* x, size_t t, size_t n_in, 
     return 1;
 }
 
+int oxhip_dev_quantize_act_batch(oxhip_ctx* c, const oxhip_quant_job* jobs, size_t n_jobs, void* stream) {
+    if (!c || (!jobs && n_jobs)) {
+        set_error("quantize_act_batch: bad arguments");
+        return 0;
+    }
+    std::vector<const float*> xs(n_jobs);
+    std::vector<size_t> ts(n_jobs), ns(n_jobs);
+    std::vector<oxhip_qact> outs(n_jobs);
+    for (size_t j = 0; j < n_jobs; j++) {
+        if (!jobs[j].x || !jobs[j].out || jobs[j].n_in % 32) {
+            set_error("quantize_act_batch: job " + std::to_string(j) + ": bad arguments (n_in must be a multiple of 32)");
+            return 0;
+        }
+        xs[j] = jobs[j].x;
+        ts[j] = jobs[j].t;
+        ns[j] = jobs[j].n_in;
+        outs[j] = *jobs[j].out;
+    }
+    HIP_TRY(launch_quantize_act_batch(xs.data(), ts.data(), ns.data(), outs.data(), n_jobs, static_cast<hipStream_t>(stream)), "quantize_act_batch launch");
+    return 1;
+}
+
 int oxhip_dev_dequantize(oxhip_ctx* c, const oxhip_weight* w, size_t r0, size_t r1, float* out, void* stream) {
     if (!c || !w || !out || r0 > r1 || r1 > w->v.n_out) {
         set_error("dequantize: bad arguments");

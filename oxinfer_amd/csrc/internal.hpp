@@ -66,6 +66,8 @@ struct GroupView {
 
 // Launchers (each returns hipSuccess or the launch error).
 hipError_t launch_quantize_act(const float* x, size_t t, size_t n_in, const oxhip_qact& out, hipStream_t s);
+constexpr int QUANT_BATCH_MAX = 16;  // matrices per launch of the batched form
+hipError_t launch_quantize_act_batch(const float* const* x, const size_t* t, const size_t* n_in, const oxhip_qact* o, size_t n, hipStream_t s);
 hipError_t launch_dequantize(const WeightView& w, size_t r0, size_t r1, float* out, hipStream_t s);
 // FP8 weights are tile-packed (WeightView::group == 1) when their rows are whole 128-column steps and the scale blocks
 // are multiples of 16 rows x 128 columns: record (tile of 16 rows, step of 128 columns) is 2048 contiguous bytes, lane

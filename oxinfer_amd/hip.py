@@ -32,6 +32,10 @@ class DecodeJob(C.Structure):
                 ("ev_start", C.c_void_p), ("ev_stop", C.c_void_p)]
 
 
+class QuantJob(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("t", C.c_size_t), ("n_in", C.c_size_t), ("out", C.c_void_p)]
+
+
 class RowsJob(C.Structure):
     _fields_ = [("w", C.c_void_p), ("up", C.c_void_p), ("n_out", C.c_size_t), ("y", C.c_void_p)]
 
@@ -74,6 +78,7 @@ def load_library():
         "oxhip_weight_bytes": (sz, [vp]),
         "oxhip_matmul": (C.c_int, [vp, vp, sz, sz, C.POINTER(Job), sz]),
         "oxhip_dev_quantize_act": (C.c_int, [vp, vp, sz, sz, C.POINTER(QActC), vp]),
+        "oxhip_dev_quantize_act_batch": (C.c_int, [vp, C.POINTER(QuantJob), sz, vp]),
         "oxhip_dev_dequantize": (C.c_int, [vp, vp, sz, sz, vp, vp]),
         "oxhip_dev_decode": (C.c_int, [vp, vp, C.POINTER(QActC), vp, sz, vp, vp]),
         "oxhip_dev_decode_noalloc": (C.c_int, [vp, vp, C.POINTER(QActC), sz, vp, vp]),
@@ -315,6 +320,17 @@ class HipBackend:
         if not self.lib.oxhip_dev_quantize_act(self.ctx, x.data_ptr(), t, n_in, C.byref(out.c), self._stream()):
             raise RuntimeError(self.last_error())
         return out
+
+    def quantize_jobs(self, pairs):
+        """A reusable job array for quantize_act_batch: pairs = [(x f32 [t, n_in] on the device, QAct)]."""
+        arr = (QuantJob * len(pairs))()
+        for i, (x, out) in enumerate(pairs):
+            arr[i] = QuantJob(x.data_ptr(), x.shape[0], x.shape[1], C.addressof(out.c))
+        return arr
+
+    def quantize_act_batch(self, arr):
+        if not self.lib.oxhip_dev_quantize_act_batch(self.ctx, arr, len(arr), self._stream()):
+            raise RuntimeError(self.last_error())
 
     def dequantize(self, w, r0=0, r1=None):
         import torch

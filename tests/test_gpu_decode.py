@@ -69,6 +69,24 @@ def test_quantize_act_bit_exact(be, oxref):
     assert np.array_equal(xa.sums16.cpu().numpy(), s16)
 
 
+def test_quantize_act_batch_bit_exact(be, oxref):
+    """Several matrices in one launch: every output equal to the reference's, as for one at a time."""
+    from oxinfer_amd.hip import QAct
+    shapes = [(1, 4096), (8, 4096), (3, 96), (1, 14336), (5, 32)] * 4  # 20 jobs: two launches
+    xs = [lcg_input(t, n, 200 + i, oxref) for i, (t, n) in enumerate(shapes)]
+    xd = [dev(x) for x in xs]
+    outs = [QAct(t, n, "cuda") for t, n in shapes]
+    be.quantize_act_batch(be.quantize_jobs(list(zip(xd, outs))))
+    for x, (t, n), xa in zip(xs, shapes, outs):
+        q, scales, sums, fsums, hsums = oxref.quantize_act(x, t, n)
+        assert np.array_equal(xa.q.cpu().numpy(), q)
+        assert np.array_equal(xa.scales.cpu().numpy().view(np.uint32), scales.view(np.uint32))
+        assert np.array_equal(xa.sums.cpu().numpy(), sums)
+        assert np.array_equal(xa.fsums.cpu().numpy().view(np.uint32), fsums.view(np.uint32))
+        assert np.array_equal(xa.hsums.cpu().numpy().view(np.uint32), hsums.view(np.uint32))
+        assert np.array_equal(xa.sums16.cpu().numpy(), q.astype(np.int32).reshape(t, n // 16, 16).sum(axis=2))
+
+
 with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_hashes.json")) as _f:  # src/ggml.rs:1547-1577
     REF_HASHES = {e["ggml_type"]: int(e["fnv1a64"], 16) for e in json.load(_f)["hashes"].values()}
 

@@ -258,3 +258,8 @@ def test_moe_against_the_f64_definition(oxref):
     y1 = synth.activations(t, h, 3)
     dec1 = oxref.moe_q4(gu, dn, 64, h, inter, x, t, idx, w, y1, decode_path=True)
     assert np.abs(dec1 - (y1 + dec)).max() < 1e-5
+    # the baseline's AVX2-scheduled decode pass is the same computation up to the f32 order inside the kernels
+    fast = oxref.moe_q4(gu, dn, 64, h, inter, x, t, idx, w, y0, decode_path=True, avx2=True, threads=4)
+    assert row_err(fast - y0, dec - y0) < 1e-5
+    one = oxref.moe_q4(gu, dn, 64, h, inter, x[:1], 1, idx[:1], w[:1], y0[:1], decode_path=True, avx2=True, threads=3)
+    assert row_err(one, dec[:1] - y0[:1]) < 1e-5
