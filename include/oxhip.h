@@ -73,6 +73,21 @@ typedef struct {
 /* `MoeAct` (src/gpu.rs:35-54); the CPU-only kinds are declined like the reference's backends do. */
 enum { OXHIP_ACT_SILU = 0, OXHIP_ACT_GELU_TANH = 1, OXHIP_ACT_SILU_CLAMP = 2 };
 
+/* ---- detection --------------------------------------------------------------------------- */
+/* platform::gpu::cuda::probe (src/platform.rs:446-482) for HIP devices, the source of a `GpuInfo { kind: GpuKind::Hip, .. }`
+ * (src/platform.rs:25-34): fills up to `cap` entries and returns the number of devices the runtime reports (0 without a
+ * driver or a device; never an error). `usable`: this library holds code for the device's architecture (gfx950);
+ * oxhip_open declines the others. */
+typedef struct {
+    int index;
+    char name[256];        /* marketing name */
+    char arch[64];         /* e.g. "gfx950" */
+    uint64_t memory_bytes; /* device-local memory */
+    char driver[64];       /* runtime version, architecture, CU count */
+    int usable;
+} oxhip_gpu_info;
+int oxhip_probe(oxhip_gpu_info* out, int cap);
+
 /* ---- life cycle -------------------------------------------------------------------------- */
 /* CudaBackend::new (src/cuda.rs:448-570). 1 on success; 0 when the device cannot start. */
 int oxhip_open(int device, oxhip_ctx** out);
@@ -169,8 +184,9 @@ int oxhip_dev_decode_noalloc(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_
  * `stream` (inside a shared launch the library orders the jobs itself). ev_start / ev_stop (from oxhip_event_create, or
  * NULL) are recorded before / after the launch that holds the job; for jobs that share a launch the first start and the
  * last stop event take the shared launch's own start and end as the device saw them.
- * The decode entry points use scratch owned by ctx (partial rows of K slices): launches on one ctx must be ordered
- * (one stream, or the caller's own synchronization). */
+ * The device-pointer entry points keep their scratch (partial rows of K slices, packed GEMM activations) per calling
+ * stream, created on a stream's first call: calls on one stream are ordered and share it, calls on different streams
+ * may overlap one another and the host-pointer surface. */
 typedef struct {
     const oxhip_weight* w;
     const oxhip_qact* xa; /* quantized weights */
@@ -199,7 +215,7 @@ float oxhip_event_elapsed_ms(void* start, void* stop);
  *   OXHIP_GEMM_FP8   FP8 weights with 128 x 128 block scales: activations quantized on the device to e4m3 per token
  *                    and 128 columns (scale amax / 448), fp8 MFMA, the two scales applied to each block's f32
  *                    partial sum (the reference has no activation-FP8 path: parity is against its f32 product);
- * Packed activations live in scratch owned by ctx (grown on first use; calls on one ctx must not overlap). */
+ * Packed activations live in the calling stream's scratch (grown on first use). */
 enum { OXHIP_F32 = 0, OXHIP_BF16 = 1 };
 enum { OXHIP_GEMM_BF16 = 0, OXHIP_GEMM_I8 = 1, OXHIP_GEMM_FP8 = 2 };
 int oxhip_dev_gemm(oxhip_ctx* ctx, const oxhip_weight* w, const void* x, int x_dtype, size_t t, void* y, int y_dtype, int variant,
@@ -222,6 +238,48 @@ int oxhip_dev_route_top_k(oxhip_ctx* ctx, const float* logits, size_t t, size_t 
  * reallocates); calls on one oxhip_moe must not overlap. */
 int oxhip_dev_moe(oxhip_ctx* ctx, oxhip_moe* m, const float* x, size_t t, const uint32_t* route_idx, const float* route_w,
                   size_t k, float* y, void* stream);
+/* ---- device-resident ops of the single-token decode graph (src/gpu_decode.rs:52-340) ---------------------------
+ * What a `DecodePlan` (src/gpu_decode.rs:572-587) runs between the embedding lookup and the logits, on buffers that
+ * stay in HBM: a plan built on these issues a token's linears and its MoE layer back to back on one stream, with no
+ * host round trip (the reference measured that per-matmul offload of decode loses, docs/platforms.md:115-117). */
+/* The arena of a plan (src/cuda_decode.rs:1044-1049: one zeroed device allocation; `View`s are offsets into it,
+ * src/gpu_decode.rs:17-33). buf_write / buf_read copy between host memory and the arena and wait for the copy. */
+void* oxhip_buf_alloc(oxhip_ctx* ctx, size_t bytes);
+void oxhip_buf_free(oxhip_ctx* ctx, void* buf);
+int oxhip_buf_write(oxhip_ctx* ctx, void* dst, const void* src_host, size_t bytes, void* stream);
+int oxhip_buf_read(oxhip_ctx* ctx, void* dst_host, const void* src, size_t bytes, void* stream);
+/* Op::Norm feeding a linear (src/gpu_decode.rs:53-66; rmsnorm, src/kernels.rs:2107-2123, then QAct::new,
+ * src/quant.rs:294-343): v = (x * r) * w with r = (mean(x^2) + eps)^(-1/2), weights f32 (`w_f32`), bf16 (`w_bf16`) or
+ * none; v goes to `out` ([t, n] f32, optional) and, quantized exactly as quantize_act quantizes it, to `q` (optional).
+ * The squares are summed in f64 in a fixed order (the CPU's one-after-the-other f32 sum cannot be repeated in
+ * parallel): r is within an ulp or two of the CPU's, the quantization of v is bit-exact. */
+int oxhip_dev_rmsnorm_quantize(oxhip_ctx* ctx, const float* x, const float* w_f32, const uint16_t* w_bf16, float eps, size_t t, size_t n,
+                               float* out, const oxhip_qact* q, void* stream);
+/* Op::Linear with its LinMode (src/gpu_decode.rs:37-50, :67-77): y [t, n_out] f32 on the device, t <= 16.
+ *   STORE      y  = W x
+ *   ADD        y += W x                        (residual)
+ *   SILU_PAIR  y  = silu(W x) * (W2 x)         (silu_mul, src/kernels.rs:2188-2198)
+ *   GELU_PAIR  y  = gelu_tanh(W x) * (W2 x)    (gelu_mul, src/kernels.rs:2234-2257)
+ *   ADD_GATED  y += sigmoid(gate[token]) * W x (a gated shared expert; `gate` one f32 per token on the device)
+ * Inputs as oxhip_dev_decode's: `xa` for quantized weights, f32 rows `x` for float-stored ones. The matrices of a
+ * pair share shape and format (pairable, src/gpu_decode.rs:340-349). The store / add / gated modes are the decode
+ * kernels' own output stage; a pair runs both products in one launch and the gate as a second one. */
+enum { OXHIP_LIN_STORE = 0, OXHIP_LIN_ADD = 1, OXHIP_LIN_SILU_PAIR = 2, OXHIP_LIN_GELU_PAIR = 3, OXHIP_LIN_ADD_GATED = 4 };
+int oxhip_dev_linear(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_weight* w2, const oxhip_qact* xa, const float* x, size_t t,
+                     float* y, uint32_t mode, const float* gate, void* stream);
+/* Op::Glu (src/gpu_decode.rs:231-239): y = silu(g) * u or gelu_tanh(g) * u over n values, for pairs of different formats. */
+int oxhip_dev_glu(oxhip_ctx* ctx, const float* g, const float* u, size_t n, int gelu, float* y, void* stream);
+/* Op::Route (src/gpu_decode.rs:154-172): logits [t, n_exp (+1)] = router [n_exp, h] (f32) . x, with `gate` ([h]) one
+ * more logit behind them; then route_top_k over the first n_exp (ties to the lower index) into `sel`: the k expert
+ * ids of every token ([t, k] u32), then their k softmax weights ([t, k] f32 bits) -- for one token "k ids then k
+ * weights" -- times expert_scale[id] when given. All pointers on the device. */
+int oxhip_dev_route(oxhip_ctx* ctx, const float* x, const float* router, const float* gate, size_t t, size_t n_exp, size_t h, size_t k,
+                    float* logits, uint32_t* sel, const float* expert_scale, void* stream);
+/* Op::Experts (src/gpu_decode.rs:318-337): the routed experts chosen in `sel` (as oxhip_dev_route writes it) over
+ * x [t, h]: y += (add) or y = the weighted sum of down_e(act(gate_e x) * up_e x), in route order. The activation
+ * (SiLU / GELU-tanh) is the layer's (oxhip_upload_moe). */
+int oxhip_dev_experts(oxhip_ctx* ctx, oxhip_moe* m, const float* x, size_t t, const uint32_t* sel, size_t k, float* y, int add, void* stream);
+
 /* The exact integer accumulators of the decode kernels, written by the kernels themselves: per
  * block of 32 ([t, n_out, n_in/32]) for Q4, Q8, Q8_0 and Q4_K, per 16 ([t, n_out, n_in/16]) for Q6_K.
  * For parity checks (the CPU's per-16 sums add up to the per-32 ones exactly). */

@@ -9,7 +9,7 @@ CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "liboxinfer_hip.so")
 OBJ = os.path.join(HERE, "build")
 
-SOURCES = ["act.hip", "dequant.hip", "decode.hip", "decode_mfma.hip", "decode_fp8.hip", "moe.hip", "moe_bf16.hip", "gemm.hip", "gemm_fp8.hip", "gemm_i8.hip", "backend.hip", "backend_moe.hip", "backend_gemm.hip"]
+SOURCES = ["act.hip", "dequant.hip", "decode.hip", "decode_mfma.hip", "decode_fp8.hip", "moe.hip", "moe_bf16.hip", "gemm.hip", "gemm_fp8.hip", "gemm_i8.hip", "backend.hip", "backend_moe.hip", "backend_gemm.hip", "graph_ops.hip", "backend_graph.hip"]
 
 # -ffp-contract=off: multiply-adds fuse only where the source says fmaf (the bit-exact dequantizers
 # need the reference's unfused operations). Packed-FP32 instructions are switched off.
@@ -35,13 +35,16 @@ def hipcc():
     raise RuntimeError("hipcc not found")
 
 
-def build(verbose=False):
+def build(verbose=False, tuning=False):
+    """tuning=True compiles the developer overrides in (-DOXHIP_TUNING: environment variables that override tile shapes
+    and orders, for measurement scripts); the library that ships is always built without them."""
     os.makedirs(OBJ, exist_ok=True)
     cc = hipcc()
+    extra_all = ["-DOXHIP_TUNING"] if tuning else []
 
     def one(src):
         obj = os.path.join(OBJ, src.replace(".hip", ".o"))
-        cmd = [cc, *FLAGS, *EXTRA.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [cc, *FLAGS, *extra_all, *EXTRA.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         # the host pass does not know the device-only target feature; that warning is harmless
         err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
@@ -60,4 +63,4 @@ def build(verbose=False):
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, tuning="--tuning" in sys.argv[1:]))

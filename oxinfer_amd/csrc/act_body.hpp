@@ -5,19 +5,10 @@
 
 namespace oxhip {
 
-__device__ __forceinline__ void quantize_act_block(const float* __restrict__ x, size_t b, int8_t* __restrict__ q, float* __restrict__ scales,
-                                                   int32_t* __restrict__ sums, float* __restrict__ fsums, float* __restrict__ hsums,
-                                                   int32_t* __restrict__ sums16) {
-    const float4* src = reinterpret_cast<const float4*>(x + b * 32);
-    float v[32];
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        float4 f = src[i];
-        v[4 * i] = f.x;
-        v[4 * i + 1] = f.y;
-        v[4 * i + 2] = f.z;
-        v[4 * i + 3] = f.w;
-    }
+// (the block's 32 values already in registers: block b of the output arrays)
+__device__ __forceinline__ void quantize_act_values(const float* v, size_t b, int8_t* __restrict__ q, float* __restrict__ scales,
+                                                    int32_t* __restrict__ sums, float* __restrict__ fsums, float* __restrict__ hsums,
+                                                    int32_t* __restrict__ sums16) {
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < 32; i++) amax = fmaxf(amax, fabsf(v[i]));
@@ -54,6 +45,22 @@ __device__ __forceinline__ void quantize_act_block(const float* __restrict__ x, 
     hsums[2 * b + 1] = h1;
     sums16[2 * b] = s0;
     sums16[2 * b + 1] = s1;
+}
+
+__device__ __forceinline__ void quantize_act_block(const float* __restrict__ x, size_t b, int8_t* __restrict__ q, float* __restrict__ scales,
+                                                   int32_t* __restrict__ sums, float* __restrict__ fsums, float* __restrict__ hsums,
+                                                   int32_t* __restrict__ sums16) {
+    const float4* src = reinterpret_cast<const float4*>(x + b * 32);
+    float v[32];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        float4 f = src[i];
+        v[4 * i] = f.x;
+        v[4 * i + 1] = f.y;
+        v[4 * i + 2] = f.z;
+        v[4 * i + 3] = f.w;
+    }
+    quantize_act_values(v, b, q, scales, sums, fsums, hsums, sums16);
 }
 
 // fast_exp of the reference (src/kernels.rs:2225-2231): clamp, Cody-Waite reduction, degree-6 polynomial,

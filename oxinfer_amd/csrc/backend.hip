@@ -69,6 +69,32 @@ extern "C" {
 
 const char* oxhip_last_error(void) { return g_err.c_str(); }
 
+int oxhip_probe(oxhip_gpu_info* out, int cap) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();  // no driver or no device: not an error of the caller's
+        return 0;
+    }
+    int rt = 0;
+    (void)hipRuntimeGetVersion(&rt);
+    for (int d = 0; d < n && out && d < cap; d++) {
+        oxhip_gpu_info& g = out[d];
+        std::memset(&g, 0, sizeof g);
+        g.index = d;
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, d) != hipSuccess) continue;
+        std::snprintf(g.name, sizeof g.name, "%s", prop.name);
+        std::string arch = prop.gcnArchName;
+        arch = arch.substr(0, arch.find(':'));
+        std::snprintf(g.arch, sizeof g.arch, "%s", arch.c_str());
+        g.memory_bytes = prop.totalGlobalMem;
+        std::snprintf(g.driver, sizeof g.driver, "HIP runtime %d.%d, %s, %d CUs", rt / 10000000, (rt / 100000) % 100, arch.c_str(),
+                      prop.multiProcessorCount);
+        g.usable = arch == "gfx950";
+    }
+    return n;
+}
+
 int oxhip_open(int device, oxhip_ctx** out) {
     if (!out) return 0;
     *out = nullptr;
@@ -129,6 +155,7 @@ void oxhip_close(oxhip_ctx* c) {
     c->xq.release();
     c->y.release();
     c->gemm_ws.release();
+    free_stream_scratch(c);
     (void)hipFree(c->dec.partial);
     (void)hipFree(c->dec.counters);
     (void)hipStreamDestroy(c->stream);
@@ -446,7 +473,13 @@ static int decode_one(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa,
         }
         v = view_of(*xa);
     }
-    HIP_TRY(launch_decode(w->v, v, x, t, y, static_cast<hipStream_t>(stream), c->dec, ev_start, ev_stop), "decode launch");
+    HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
+    StreamScratch* sc = scratch_for(c, static_cast<hipStream_t>(stream));
+    if (!sc) {
+        set_error("decode: device memory short");
+        return 0;
+    }
+    HIP_TRY(launch_decode(w->v, v, x, t, y, static_cast<hipStream_t>(stream), sc->dec, ev_start, ev_stop), "decode launch");
     return 1;
 }
 
@@ -502,6 +535,12 @@ int oxhip_dev_decode_batch(oxhip_ctx* c, const oxhip_decode_job* jobs, size_t n_
         return 0;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
+    HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
+    StreamScratch* ssc = scratch_for(c, s);
+    if (!ssc) {
+        set_error("decode_batch: device memory short");
+        return 0;
+    }
     // Runs of jobs that the matrix-core decode kernel takes share one launch; the others go out one by one.
     auto fusable = [&](const oxhip_decode_job& jb) {
         return jb.w && jb.xa && jb.y && !is_dense(jb.w) && jb.xa->n_in == jb.w->v.n_in && jb.xa->t >= jb.t && decode_batchable(jb.w->v, jb.t);
@@ -521,14 +560,14 @@ int oxhip_dev_decode_batch(oxhip_ctx* c, const oxhip_decode_job* jobs, size_t n_
                     if (!e0) e0 = static_cast<hipEvent_t>(jobs[k].ev_start);
                     else HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(jobs[k].ev_start), s), "event record");
                 }
-                items.push_back(DecodeBatchItem{jobs[k].w->v, view_of(*jobs[k].xa), jobs[k].y, (uint32_t)jobs[k].t});
+                items.push_back(DecodeBatchItem{jobs[k].w->v, view_of(*jobs[k].xa), jobs[k].y, (uint32_t)jobs[k].t, Epi{}});
             }
             for (size_t k = e; k-- > j;)
                 if (jobs[k].ev_stop) {
                     e1 = static_cast<hipEvent_t>(jobs[k].ev_stop);
                     break;
                 }
-            const hipError_t err = launch_decode_mfma_batch(items.data(), items.size(), c->dec, s, e0, e1);
+            const hipError_t err = launch_decode_mfma_batch(items.data(), items.size(), ssc->dec, s, e0, e1);
             if (err == hipErrorOutOfMemory) {  // the scratch does not hold these jobs together: one launch each
                 if (e0) HIP_TRY(hipEventRecord(e0, s), "event record");
                 for (size_t k = j; k < e; k++)
@@ -649,12 +688,12 @@ int oxhip_matmul(oxhip_ctx* c, const float* x, size_t t, size_t n_in, oxhip_job*
     for (size_t j = 0; j < n_jobs; j++) {
         const oxhip_weight* w = jobs[j].w;
         if (t <= 8 && !is_dense(w) && decode_batchable(w->v, t)) {
-            fused.push_back(DecodeBatchItem{w->v, view_of(xa), yd + offs[j], (uint32_t)t});
+            fused.push_back(DecodeBatchItem{w->v, view_of(xa), yd + offs[j], (uint32_t)t, Epi{}});
             continue;
         }
         const bool gemm = t > 16 && gemm_bf16_ok(w->v);
         if (gemm) {
-            if (!gemm_bf16_run(c, w, c->x.p, false, t, yd + offs[j], false, s)) {
+            if (!gemm_bf16_run(c->gemm_ws, w, c->x.p, false, t, yd + offs[j], false, s)) {
                 (void)hipStreamSynchronize(s);
                 return done(0);
             }

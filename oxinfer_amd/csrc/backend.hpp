@@ -3,6 +3,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <map>
 #include <string>
 #include <vector>
 
@@ -45,6 +46,15 @@ struct DevBuf {
     }
 };
 
+// Scratch of the device-pointer entry points on one stream: the decode kernels' K-slice rows and counters, the
+// products of a gate / up pair (and of formats whose kernels only store) before their epilogue, the prefill GEMMs'
+// packed activations.
+struct StreamScratch {
+    DecodeScratch dec;
+    DevBuf tmp;
+    DevBuf gemm_ws;
+};
+
 }  // namespace oxhip
 
 struct oxhip_weight {
@@ -60,15 +70,20 @@ struct oxhip_ctx {
     std::mutex mu;  // serializes the host-pointer surface (staging is shared), as Mutex<Staging> does
     oxhip::DevBuf x, xq, y;
     oxhip::DevBuf gemm_ws;  // packed activations of the prefill GEMMs
-    oxhip::DecodeScratch dec;  // partial rows and counters of the decode kernels that split K across workgroups
+    oxhip::DecodeScratch dec;  // partial rows and counters of the decode kernels that split K across workgroups (host surface, on `stream`)
+    std::mutex smu;            // guards per_stream
+    std::map<hipStream_t, oxhip::StreamScratch*> per_stream;  // the device-pointer entry points' scratch, by calling stream
     double ms_in = 0, ms_gpu = 0, ms_out = 0;
     size_t calls = 0;
 };
 
 namespace oxhip {
 
-// backend_gemm.hip: packs x and runs the bf16-matrix-core GEMM (1 = done, 0 = declined with the error set)
-int gemm_bf16_run(oxhip_ctx* c, const oxhip_weight* w, const void* x, bool x_bf16, size_t t, void* y, bool y_bf16, hipStream_t s);
+// backend_gemm.hip: packs x into `ws` and runs the bf16-matrix-core GEMM (1 = done, 0 = declined with the error set)
+int gemm_bf16_run(DevBuf& ws, const oxhip_weight* w, const void* x, bool x_bf16, size_t t, void* y, bool y_bf16, hipStream_t s);
+// backend_graph.hip: the calling stream's scratch (created on the stream's first call; nullptr when memory is short)
+StreamScratch* scratch_for(oxhip_ctx* c, hipStream_t s);
+void free_stream_scratch(oxhip_ctx* c);
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 

@@ -1,0 +1,208 @@
+// Device-resident ops of the reference's single-token decode graph (src/gpu_decode.rs:52-340), so that a token's
+// linears and its MoE layer run back to back on buffers that stay in HBM: Op::Linear with its LinMode, Op::Norm fused
+// with the quantization of the next linear's input, Op::Route, Op::Experts, Op::Glu, and the arena they work in.
+#include <algorithm>
+
+#include "backend.hpp"
+
+using namespace oxhip;
+
+namespace oxhip {
+
+// The scratch of the device-pointer entry points, one set per stream: launches on one stream are ordered, so they may
+// share; launches on different streams may overlap and must not.
+StreamScratch* scratch_for(oxhip_ctx* c, hipStream_t s) {
+    std::lock_guard<std::mutex> g(c->smu);
+    auto it = c->per_stream.find(s);
+    if (it != c->per_stream.end()) return it->second;
+    auto* sc = new StreamScratch();
+    sc->dec.partial_floats = c->dec.partial_floats;
+    sc->dec.ncounters = c->dec.ncounters;
+    if (hipMalloc(reinterpret_cast<void**>(&sc->dec.partial), sc->dec.partial_floats * 4) != hipSuccess ||
+        hipMalloc(reinterpret_cast<void**>(&sc->dec.counters), sc->dec.ncounters * 4) != hipSuccess ||
+        hipMemset(sc->dec.counters, 0, sc->dec.ncounters * 4) != hipSuccess) {
+        if (sc->dec.partial) (void)hipFree(sc->dec.partial);
+        if (sc->dec.counters) (void)hipFree(sc->dec.counters);
+        delete sc;
+        return nullptr;
+    }
+    c->per_stream.emplace(s, sc);
+    return sc;
+}
+
+void free_stream_scratch(oxhip_ctx* c) {
+    std::lock_guard<std::mutex> g(c->smu);
+    for (auto& kv : c->per_stream) {
+        (void)hipFree(kv.second->dec.partial);
+        (void)hipFree(kv.second->dec.counters);
+        kv.second->tmp.release();
+        kv.second->gemm_ws.release();
+        delete kv.second;
+    }
+    c->per_stream.clear();
+}
+
+}  // namespace oxhip
+
+extern "C" {
+
+void* oxhip_buf_alloc(oxhip_ctx* c, size_t bytes) {
+    if (!c || !bytes) {
+        set_error("buf_alloc: bad arguments");
+        return nullptr;
+    }
+    void* p = nullptr;
+    if (hipSetDevice(c->device) != hipSuccess || hipMalloc(&p, bytes) != hipSuccess) {
+        set_error("buf_alloc: device memory short");
+        return nullptr;
+    }
+    if (hipMemset(p, 0, bytes) != hipSuccess) {
+        (void)hipFree(p);
+        set_error("buf_alloc: clearing failed");
+        return nullptr;
+    }
+    return p;
+}
+
+void oxhip_buf_free(oxhip_ctx* c, void* p) {
+    if (!p) return;
+    if (c) (void)hipSetDevice(c->device);
+    (void)hipFree(p);
+}
+
+int oxhip_buf_write(oxhip_ctx* c, void* dst, const void* src, size_t bytes, void* stream) {
+    if (!c || !dst || !src) {
+        set_error("buf_write: null argument");
+        return 0;
+    }
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)), "buf_write");
+    HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "buf_write");  // the host buffer may be reused at once
+    return 1;
+}
+
+int oxhip_buf_read(oxhip_ctx* c, void* dst, const void* src, size_t bytes, void* stream) {
+    if (!c || !dst || !src) {
+        set_error("buf_read: null argument");
+        return 0;
+    }
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)), "buf_read");
+    HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "buf_read");
+    return 1;
+}
+
+int oxhip_dev_rmsnorm_quantize(oxhip_ctx* c, const float* x, const float* w_f32, const uint16_t* w_bf16, float eps, size_t t, size_t n,
+                               float* out, const oxhip_qact* q, void* stream) {
+    if (!c || !x || (!out && !q) || n % 32 || (w_f32 && w_bf16) || (q && (q->n_in != n || q->t < t))) {
+        set_error("rmsnorm_quantize: bad arguments (n must be a multiple of 32, one kind of weights, outputs of the input's shape)");
+        return 0;
+    }
+    HIP_TRY(launch_rmsnorm_quantize(x, w_f32, w_bf16, eps, t, n, out, q, static_cast<hipStream_t>(stream)), "rmsnorm_quantize launch");
+    return 1;
+}
+
+int oxhip_dev_glu(oxhip_ctx* c, const float* g, const float* u, size_t n, int gelu, float* y, void* stream) {
+    if (!c || !g || !u || !y) {
+        set_error("glu: null argument");
+        return 0;
+    }
+    HIP_TRY(launch_glu(g, u, n, gelu != 0, y, static_cast<hipStream_t>(stream)), "glu launch");
+    return 1;
+}
+
+int oxhip_dev_linear(oxhip_ctx* c, const oxhip_weight* w, const oxhip_weight* w2, const oxhip_qact* xa, const float* x, size_t t, float* y,
+                     uint32_t mode, const float* gate, void* stream) {
+    if (!c || !w || !y || t == 0 || t > 16 || mode > OXHIP_LIN_ADD_GATED) {
+        set_error("linear: bad arguments (1 <= t <= 16)");
+        return 0;
+    }
+    const bool pair = mode == OXHIP_LIN_SILU_PAIR || mode == OXHIP_LIN_GELU_PAIR;
+    if (pair != (w2 != nullptr) || (mode == OXHIP_LIN_ADD_GATED) != (gate != nullptr)) {
+        set_error("linear: the pair modes take a second matrix, the gated mode a gate, the others neither");
+        return 0;
+    }
+    if (pair && (w2->v.n_in != w->v.n_in || w2->v.n_out != w->v.n_out || w2->v.fmt != w->v.fmt)) {
+        set_error("linear: the matrices of a pair share shape and storage format (pairable, src/gpu_decode.rs:340-349)");
+        return 0;
+    }
+    QActView v{};
+    if (is_dense(w)) {
+        if (!x) {
+            set_error("linear: float-stored weights take f32 rows");
+            return 0;
+        }
+    } else {
+        if (!xa || xa->n_in != w->v.n_in || xa->t < t) {
+            set_error("linear: quantized activations missing or of another shape");
+            return 0;
+        }
+        v = view_of(*xa);
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
+    StreamScratch* sc = scratch_for(c, s);
+    if (!sc) {
+        set_error("linear: device memory short");
+        return 0;
+    }
+    const size_t n_out = w->v.n_out;
+    Epi epi;
+    epi.mode = mode == OXHIP_LIN_ADD ? EPI_ADD : mode == OXHIP_LIN_ADD_GATED ? EPI_ADD_GATED : EPI_STORE;
+    epi.gate = gate;
+    if (!pair) {
+        if (mfma_decode_format(w->v.fmt)) {
+            HIP_TRY(launch_decode_mfma(w->v, v, t, y, sc->dec, s, nullptr, nullptr, epi), "linear launch");
+            return 1;
+        }
+        if (epi.mode == EPI_STORE) {
+            HIP_TRY(launch_decode(w->v, v, x, t, y, s, sc->dec), "linear launch");
+            return 1;
+        }
+        // formats whose kernels only store: the product goes to scratch, the mode is a small kernel of its own
+        if (!sc->tmp.grow(t * n_out * 4)) {
+            set_error("linear: device memory short");
+            return 0;
+        }
+        float* tmp = static_cast<float*>(sc->tmp.p);
+        HIP_TRY(launch_decode(w->v, v, x, t, tmp, s, sc->dec), "linear launch");
+        HIP_TRY(launch_epilogue(tmp, t, n_out, y, epi, s), "linear epilogue launch");
+        return 1;
+    }
+    // y = act(W x) * (W2 x): both products in one shared launch where the kernel takes them, then the gate
+    if (!sc->tmp.grow(2 * t * n_out * 4)) {
+        set_error("linear: device memory short");
+        return 0;
+    }
+    float* g = static_cast<float*>(sc->tmp.p);
+    float* u = g + t * n_out;
+    if (t <= 8 && decode_batchable(w->v, t)) {
+        DecodeBatchItem items[2] = {{w->v, v, g, (uint32_t)t, Epi{}}, {w2->v, v, u, (uint32_t)t, Epi{}}};
+        hipError_t e = launch_decode_mfma_batch(items, 2, sc->dec, s);
+        if (e == hipErrorOutOfMemory) {
+            HIP_TRY(launch_decode(w->v, v, x, t, g, s, sc->dec), "linear launch");
+            HIP_TRY(launch_decode(w2->v, v, x, t, u, s, sc->dec), "linear launch");
+        } else {
+            HIP_TRY(e, "linear launch");
+        }
+    } else {
+        HIP_TRY(launch_decode(w->v, v, x, t, g, s, sc->dec), "linear launch");
+        HIP_TRY(launch_decode(w2->v, v, x, t, u, s, sc->dec), "linear launch");
+    }
+    HIP_TRY(launch_glu(g, u, t * n_out, mode == OXHIP_LIN_GELU_PAIR, y, s), "linear gate launch");
+    return 1;
+}
+
+int oxhip_dev_route(oxhip_ctx* c, const float* x, const float* router, const float* gate, size_t t, size_t n_exp, size_t h, size_t k,
+                    float* logits, uint32_t* sel, const float* expert_scale, void* stream) {
+    if (!c || !x || !router || !logits || !sel || !t || !k || k > 32 || k > n_exp || n_exp > 1024 || !h) {
+        set_error("route: bad arguments (k <= 32, k <= n_experts <= 1024)");
+        return 0;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    HIP_TRY(launch_router_logits(x, router, gate, t, n_exp, h, logits, s), "router launch");
+    // sel: the k ids of every token, then their k weights (for one token: k ids then k weights, src/gpu_decode.rs:158-160)
+    HIP_TRY(launch_route_top_k(logits, t, n_exp, k, sel, reinterpret_cast<float*>(sel + t * k), s, n_exp + (gate ? 1 : 0), expert_scale),
+            "route_top_k launch");
+    return 1;
+}
+
+}  // extern "C"

@@ -74,7 +74,7 @@ Scratch carve(uint8_t* base, size_t t, size_t pairs, size_t n_exp, size_t h, siz
 }
 
 int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t* route_idx, const float* route_w, size_t k,
-            float* y, hipStream_t s) {
+            float* y, hipStream_t s, bool add = true) {
     const size_t pairs = t * k, h = m->h, inter = m->inter;
     if (!pairs) return 1;
     if (pairs > m->ws_pairs || t > m->ws_t) {
@@ -159,7 +159,7 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
         g.bases = m->bases_dn;
         HIP_TRY(launch_decode_mfma_grouped(m->down[0]->v, view_of(sc.aq), g, grid_chunks, max_rows, sc.o, s), "moe down launch");
     }
-    HIP_TRY(launch_moe_combine(sc.o, sc.row_of, route_w, t, k, h, y, s), "moe combine launch");
+    HIP_TRY(launch_moe_combine(sc.o, sc.row_of, route_w, t, k, h, y, s, add), "moe combine launch");
     return 1;
 }
 
@@ -268,6 +268,15 @@ int oxhip_dev_moe(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const ui
         return 0;
     }
     return moe_run(c, m, x, t, route_idx, route_w, k, y, static_cast<hipStream_t>(stream));
+}
+
+int oxhip_dev_experts(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t* sel, size_t k, float* y, int add, void* stream) {
+    if (!c || !m || !x || !sel || !y || !k || !t) {
+        set_error("experts: bad arguments");
+        return 0;
+    }
+    HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
+    return moe_run(c, m, x, t, sel, reinterpret_cast<const float*>(sel + t * k), k, y, static_cast<hipStream_t>(stream), add != 0);
 }
 
 int oxhip_moe_forward(oxhip_ctx* c, const float* x, size_t t, size_t h, size_t inter, const uint32_t* route_idx, const float* route_w,

@@ -142,7 +142,7 @@ template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS, int NG = 1>
 __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw, float* __restrict__ y,
                                             int32_t* __restrict__ dump, GroupView grp, uint32_t ksplit, float* __restrict__ partial,
                                             uint32_t* __restrict__ counters, uint32_t bx, uint32_t by, uint32_t nthr,
-                                            float* __restrict__ lds_all) {
+                                            float* __restrict__ lds_all, Epi epi = Epi{}) {
     static_assert(NG == 1 || (GROUPED && ALDS && !DUMP && NT == 8), "token groups are for grouped launches");
     constexpr int TPAD = NT <= 4 ? 4 : 8;
     // the swizzled operand array pays at 8 tokens (where the staging stores are many); at fewer its address math costs more
@@ -639,6 +639,12 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                 if (d_tok0 + i < (uint32_t)TPAD) red[(((size_t)wave * NG + g) * TPAD + d_tok0 + i) * 16 + n] = acc[g][i];
     }
     __syncthreads();
+    // how a finished sum goes out (uniform branches)
+    auto emit = [&](float* dst, float v, uint32_t tok) {
+        if (epi.mode == EPI_STORE) *dst = v;
+        else if (epi.mode == EPI_ADD) *dst = *dst + v;
+        else *dst = *dst + (1.0f / (1.0f + expf(-epi.gate[tok]))) * v;
+    };
     // the waves of a tile in order; with one slice that is the result, else this slice's partial rows
     float* out = ksplit > 1 ? partial + (size_t)slice * t * w.n_out : y;
     for (uint32_t idx = threadIdx.x; idx < rt * NG * TPAD * 16; idx += nthr) {
@@ -649,7 +655,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         for (uint32_t k = 0; k < kw; k++) sum += red[((((size_t)rr * kw + k) * NG + g) * TPAD + (idx / 16) % TPAD) * 16 + nn];
         // partial rows go out as device-scope stores (written through to memory, where the other XCDs' L2s see them)
         if (ksplit > 1) __hip_atomic_store(out + (size_t)tok * w.n_out + row, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        else out[(size_t)tok * w.n_out + row] = sum;
+        else emit(out + (size_t)tok * w.n_out + row, sum, tok);
     }
     if (GROUPED || ksplit == 1 || !y) return;  // uniform over the workgroup
     // The last workgroup of this row group to get here adds the slices in slice order; the counter returns to zero
@@ -680,7 +686,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
 #pragma unroll
             for (uint32_t i = 0; i < 4; i++) sum = z0 + i == 0 ? v[i] : z0 + i < ksplit ? sum + v[i] : sum;
         }
-        y[(size_t)tok * w.n_out + row] = sum;
+        emit(y + (size_t)tok * w.n_out + row, sum, tok);
     }
 }
 
@@ -693,10 +699,10 @@ __global__ __launch_bounds__(GROUPED ? 512 : 1024) void decode_mfma_kernel(Weigh
                                                                            uint32_t kw, float* __restrict__ y,
                                                                            int32_t* __restrict__ dump, GroupView grp, uint32_t ksplit,
                                                                            float* __restrict__ partial,
-                                                                           uint32_t* __restrict__ counters) {
+                                                                           uint32_t* __restrict__ counters, Epi epi) {
     extern __shared__ __align__(16) float lds_dyn[];
     decode_body<FMT, NT, DUMP, GROUPED, ALDS, NG>(w, xa, t, rt, kw, y, dump, grp, ksplit, partial, counters, blockIdx.x, blockIdx.y,
-                                                  blockDim.x, lds_dyn);
+                                                  blockDim.x, lds_dyn, epi);
 }
 
 // Several independent matmuls in one launch (the jobs of one Backend::matmul call, src/gpu.rs:160: Q/K/V, gate/up ...):
@@ -713,6 +719,7 @@ struct BatchJob {
     float* partial;      // this job's share of the scratch (K slices across workgroups)
     uint32_t* counters;
     uint32_t t, rt, kw, ks, wg0;
+    Epi epi;
 };
 struct BatchArgs {
     uint32_t njobs, nwg;
@@ -725,11 +732,11 @@ __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid,
     if (threadIdx.x >= nthr) return;  // whole waves (nthr is a multiple of 64), before any barrier
     const GroupView none{};
     const uint32_t bx = bid >> __builtin_ctz(jb.ks), by = bid & (jb.ks - 1);  // the slices of a row group are neighbours in launch order (ks: a power of two)
-    if (jb.t == 1) decode_body<FMT, 1, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
+    if (jb.t == 1) decode_body<FMT, 1, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi);
     else if (jb.t == 2 && !t4m_format(FMT)) decode_body<FMT, 2, false, false, true>(  // (MLX at 2 tokens: the 4-token body, which fits the registers)
-        jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
-    else if (jb.t <= 4) decode_body<FMT, 4, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
-    else decode_body<FMT, 8, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds);
+        jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi);
+    else if (jb.t <= 4) decode_body<FMT, 4, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi);
+    else decode_body<FMT, 8, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi);
 }
 
 __global__ __launch_bounds__(1024) void decode_batch_kernel(BatchArgs a) {
@@ -850,7 +857,7 @@ size_t lds_bytes(bool sums, bool dump, uint32_t bps, uint32_t nsteps, int tpad, 
 template <int FMT, int NT, bool DUMP, bool GROUPED, int NG = 1>
 hipError_t launch_one(bool alds, dim3 grid, dim3 block, size_t lds, hipStream_t s, const WeightView& w, const QActView& v, uint32_t t,
                       const Shape& sh, float* y, int32_t* dump, const GroupView& g, const DecodeScratch& sc, hipEvent_t ev_start = nullptr,
-                      hipEvent_t ev_stop = nullptr) {
+                      hipEvent_t ev_stop = nullptr, const Epi& epi = Epi{}) {
     hipError_t e = hipSuccess;
     auto go = [&](auto kern) {
         // once per kernel and device: allow the whole LDS
@@ -865,8 +872,8 @@ hipError_t launch_one(bool alds, dim3 grid, dim3 block, size_t lds, hipStream_t 
         if (e != hipSuccess) return;
         // timing events ride on the dispatch: its start and end as the device saw them
         if (ev_start || ev_stop)
-            hipExtLaunchKernelGGL(kern, grid, block, (uint32_t)lds, s, ev_start, ev_stop, 0, w, v, t, sh.rt, sh.kw, y, dump, g, sh.ks, sc.partial, sc.counters);
-        else kern<<<grid, block, lds, s>>>(w, v, t, sh.rt, sh.kw, y, dump, g, sh.ks, sc.partial, sc.counters);
+            hipExtLaunchKernelGGL(kern, grid, block, (uint32_t)lds, s, ev_start, ev_stop, 0, w, v, t, sh.rt, sh.kw, y, dump, g, sh.ks, sc.partial, sc.counters, epi);
+        else kern<<<grid, block, lds, s>>>(w, v, t, sh.rt, sh.kw, y, dump, g, sh.ks, sc.partial, sc.counters, epi);
     };
     if (alds) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, true, NG>);
     else if constexpr (NG == 1 && FMT != FMT_Q6_K) go(decode_mfma_kernel<FMT, NT, DUMP, GROUPED, false, 1>);
@@ -881,7 +888,7 @@ constexpr uint32_t steps_of(uint32_t n_in) {
 
 template <int FMT, bool DUMP>
 hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* dump, const DecodeScratch& sc, hipStream_t s,
-               hipEvent_t ev_start = nullptr, hipEvent_t ev_stop = nullptr) {
+               hipEvent_t ev_start = nullptr, hipEvent_t ev_stop = nullptr, const Epi& epi0 = Epi{}) {
     const uint32_t ntiles = row_tiles(w.n_out), nsteps = steps_of<FMT>(w.n_in);
     Shape sh = shape_for(ntiles, nsteps, true, FMT);
     const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
@@ -914,11 +921,13 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
         const size_t lds = lds_bytes(!q8_format(FMT), DUMP, q8_format(FMT) ? 2 : 4, nsteps, tpad, sh, &alds);
         if (lds > LDS_MAX) return hipErrorInvalidValue;  // rows too long for the staged activation scales
         const uint32_t tt = (uint32_t)tc;
+        Epi epi = epi0;
+        if (epi.gate) epi.gate += c0;
         hipError_t e;
-        if (tc == 1) e = launch_one<FMT, 1, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
-        else if (tc == 2 && !t4m_format(FMT)) e = launch_one<FMT, 2, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
-        else if (tc <= 4) e = launch_one<FMT, 4, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
-        else e = launch_one<FMT, 8, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1);
+        if (tc == 1) e = launch_one<FMT, 1, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1, epi);
+        else if (tc == 2 && !t4m_format(FMT)) e = launch_one<FMT, 2, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1, epi);
+        else if (tc <= 4) e = launch_one<FMT, 4, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1, epi);
+        else e = launch_one<FMT, 8, DUMP, false>(alds, grid, block, lds, s, w, v, tt, sh, yo, du, GroupView{}, sc, e0, e1, epi);
         if (e != hipSuccess) return e;
         c0 += tc;
     }
@@ -1052,7 +1061,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
             }
             lds = l > lds ? l : lds;
             threads = 64 * sh.rt * sh.kw > threads ? 64 * sh.rt * sh.kw : threads;
-            a.j[j] = BatchJob{it.w, it.xa, it.y, partial, counters, it.t, sh.rt, sh.kw, sh.ks, wg};
+            a.j[j] = BatchJob{it.w, it.xa, it.y, partial, counters, it.t, sh.rt, sh.kw, sh.ks, wg, it.epi};
             wg += groups * sh.ks;
         }
         a.nwg = wg;
@@ -1105,14 +1114,14 @@ hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, c
 }
 
 hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, const DecodeScratch& sc, hipStream_t s,
-                              hipEvent_t ev_start, hipEvent_t ev_stop) {
+                              hipEvent_t ev_start, hipEvent_t ev_stop, const Epi& epi) {
     switch (w.fmt) {
-        case FMT_Q8_0: return run<FMT_Q8_0, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
-        case FMT_Q8F: return run<FMT_Q8F, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
-        case FMT_Q4_K: return run<FMT_Q4_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
-        case FMT_Q6_K: return run<FMT_Q6_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
-        case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
-        case FMT_Q40: return run<FMT_Q40, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop);
+        case FMT_Q8_0: return run<FMT_Q8_0, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
+        case FMT_Q8F: return run<FMT_Q8F, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
+        case FMT_Q4_K: return run<FMT_Q4_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
+        case FMT_Q6_K: return run<FMT_Q6_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
+        case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
+        case FMT_Q40: return run<FMT_Q40, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
         default: return hipErrorInvalidValue;
     }
 }

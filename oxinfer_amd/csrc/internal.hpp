@@ -56,6 +56,14 @@ struct QActView {
     const int32_t* sums16;
 };
 
+// How a decode matmul writes its rows (LinMode of the reference's decode graph, src/gpu_decode.rs:37-50): y = v,
+// y += v (a residual), or y += sigmoid(gate[token]) * v (a gated shared expert).
+enum : uint32_t { EPI_STORE = 0, EPI_ADD = 1, EPI_ADD_GATED = 2 };
+struct Epi {
+    uint32_t mode = EPI_STORE;
+    const float* gate = nullptr;  // EPI_ADD_GATED: one f32 per token
+};
+
 // A grouped launch (MoE): chunk c = {expert, first row, rows (<= 8), 0}; see decode_mfma.hip.
 struct GroupView {
     const uint8_t* const* bases;  // per expert: tile-packed weights
@@ -96,6 +104,9 @@ struct DecodeScratch {
 // ev_start / ev_stop (optional): timing events around the launches (carried by the launch itself where there is one).
 hipError_t launch_decode(const WeightView& w, const QActView& xa, const float* x, size_t t, float* y, hipStream_t s,
                          const DecodeScratch& sc = DecodeScratch{}, hipEvent_t ev_start = nullptr, hipEvent_t ev_stop = nullptr);
+// y <- epi(y, v) over n values of t tokens ([t][n], v likewise): the epilogue as a kernel of its own, for the formats whose
+// decode kernels only store.
+hipError_t launch_epilogue(const float* v, size_t t, size_t n, float* y, const Epi& epi, hipStream_t s);
 hipError_t launch_isums(const WeightView& w, const QActView& xa, size_t t, int32_t* out, hipStream_t s);
 // Independent matmuls that may share one launch (decode_mfma.hip): each 1..8 tokens over a tile-packed weight.
 struct DecodeBatchItem {
@@ -103,6 +114,7 @@ struct DecodeBatchItem {
     QActView xa;
     float* y;
     uint32_t t;
+    Epi epi{};
 };
 void decode_scratch_need(const WeightView& w, size_t* partial_floats, size_t* ncounters);  // of a launch that slices K; else zeros
 bool decode_batchable(const WeightView& w, size_t t);  // the kernel takes it and its activations fit LDS
@@ -110,7 +122,7 @@ bool decode_batchable(const WeightView& w, size_t t);  // the kernel takes it an
 hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s, hipEvent_t ev_start = nullptr,
                                     hipEvent_t ev_stop = nullptr);
 hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, const DecodeScratch& sc, hipStream_t s,
-                              hipEvent_t ev_start = nullptr, hipEvent_t ev_stop = nullptr);
+                              hipEvent_t ev_start = nullptr, hipEvent_t ev_stop = nullptr, const Epi& epi = Epi{});
 hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks,
                                       uint32_t max_rows_per_chunk, float* y, hipStream_t s);
 bool decode_grouped_fits(const WeightView& w, uint32_t max_rows_per_chunk);  // LDS holds a chunk's staged activations
@@ -146,7 +158,8 @@ hipError_t launch_quantize_act_fp8(const void* x, bool src_bf16, size_t t, size_
 uint32_t gemm_fp8_k_slices(const WeightView& w, size_t mtiles);
 hipError_t launch_gemm_fp8(const WeightView& w, const void* apk, const float* sx, size_t t, size_t mtiles, void* y, bool out_bf16,
                            float* partial, hipStream_t s);
-hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, hipStream_t s);
+hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, hipStream_t s, size_t stride = 0,
+                              const float* expert_scale = nullptr);
 hipError_t launch_moe_plan(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, uint32_t chunk_rows, int* row_of, int* src,
                            int4* chunks, int* nchunks, hipStream_t s);
 hipError_t launch_moe_front(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, uint32_t chunk_rows, int* row_of, int* src,
@@ -156,7 +169,13 @@ hipError_t launch_moe_act(const float* g, const float* u, size_t stride, size_t 
 hipError_t launch_moe_act_quantize(const float* g, const float* u, size_t stride, size_t rows, size_t inter, uint32_t kind, float param,
                                    const oxhip_qact& o, hipStream_t s);
 hipError_t launch_moe_combine(const float* o, const int* row_of, const float* route_w, size_t t, size_t k, size_t h, float* y,
-                              hipStream_t s);
+                              hipStream_t s, bool add = true);
+// decode-graph kernels (graph_ops.hip)
+hipError_t launch_glu(const float* g, const float* u, size_t n, bool gelu, float* y, hipStream_t s);
+hipError_t launch_router_logits(const float* x, const float* router, const float* gate, size_t t, size_t n_exp, size_t h, float* logits,
+                                hipStream_t s);
+hipError_t launch_rmsnorm_quantize(const float* x, const float* w_f32, const uint16_t* w_bf16, float eps, size_t t, size_t n, float* out,
+                                   const oxhip_qact* q, hipStream_t s);
 // The bf16 form of the grouped expert matmuls for prefill passes (moe_bf16.hip): MLX 4-bit weights, chunks of <= 16 rows.
 bool moe_bf16_ok(const WeightView& w);
 size_t moe_bf16_frag_bytes(size_t max_chunks, size_t n_in);

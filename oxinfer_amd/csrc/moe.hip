@@ -21,10 +21,11 @@ __device__ __forceinline__ int order_key(float v) {
 // NW waves per token. A lone wave issues an instruction every five to eight cycles, so the counting loop is split
 // over the waves (each broadcasts 64 / NW lanes of every register) and the counts meet in LDS; wave 0 finishes.
 template <int PER, int NW>
-__global__ __launch_bounds__(64 * NW) void route_top_k_kernel(const float* __restrict__ logits, uint32_t n, uint32_t k,
-                                                              uint32_t* __restrict__ idx, float* __restrict__ wts) {
+__global__ __launch_bounds__(64 * NW) void route_top_k_kernel(const float* __restrict__ logits, uint32_t stride, uint32_t n, uint32_t k,
+                                                              uint32_t* __restrict__ idx, float* __restrict__ wts,
+                                                              const float* __restrict__ expert_scale) {
     const uint32_t tok = blockIdx.x, lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const float* l = logits + (size_t)tok * n;
+    const float* l = logits + (size_t)tok * stride;
     int key[PER];
     bool live[PER];
 #pragma unroll
@@ -118,15 +119,19 @@ __global__ __launch_bounds__(64 * NW) void route_top_k_kernel(const float* __res
     for (uint32_t r = 0; r < k && r < 64; r++) sum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), (int)r));
     if (lane < k) {
         idx[(size_t)tok * k + lane] = myidx;
-        wts[(size_t)tok * k + lane] = e / sum;
+        // (per-expert factors multiply the weights after the softmax, src/gpu_decode.rs:167-168)
+        wts[(size_t)tok * k + lane] = expert_scale ? e / sum * expert_scale[myidx] : e / sum;
     }
 }
 
-hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, hipStream_t s) {
+// `stride`: floats between the logit rows of consecutive tokens (>= n; the decode graph keeps one more logit behind them).
+hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, hipStream_t s, size_t stride,
+                              const float* expert_scale) {
     if (!t) return hipSuccess;
-    if (n <= 128) route_top_k_kernel<2, 8><<<(unsigned)t, 512, 0, s>>>(logits, (uint32_t)n, (uint32_t)k, idx, w);
-    else if (n <= 256) route_top_k_kernel<4, 8><<<(unsigned)t, 512, 0, s>>>(logits, (uint32_t)n, (uint32_t)k, idx, w);
-    else route_top_k_kernel<16, 1><<<(unsigned)t, 64, 0, s>>>(logits, (uint32_t)n, (uint32_t)k, idx, w);
+    const uint32_t st = (uint32_t)(stride ? stride : n);
+    if (n <= 128) route_top_k_kernel<2, 8><<<(unsigned)t, 512, 0, s>>>(logits, st, (uint32_t)n, (uint32_t)k, idx, w, expert_scale);
+    else if (n <= 256) route_top_k_kernel<4, 8><<<(unsigned)t, 512, 0, s>>>(logits, st, (uint32_t)n, (uint32_t)k, idx, w, expert_scale);
+    else route_top_k_kernel<16, 1><<<(unsigned)t, 64, 0, s>>>(logits, st, (uint32_t)n, (uint32_t)k, idx, w, expert_scale);
     return hipGetLastError();
 }
 
@@ -374,11 +379,11 @@ hipError_t launch_moe_act_quantize(const float* g, const float* u, size_t stride
 // y[i] += w_j * o[row_of(i, j)] for j in route order: axpy per expert, multiply then add (src/moe.rs:608-615).
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ o, const int* __restrict__ row_of,
                                                           const float* __restrict__ route_w, uint32_t t, uint32_t k, uint32_t h,
-                                                          float* __restrict__ y) {
+                                                          float* __restrict__ y, bool add) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)t * h) return;
     uint32_t tok = i / h, c = i % h;
-    float acc = y[i];
+    float acc = add ? y[i] : 0.0f;
     for (uint32_t j = 0; j < k; j++) {
         const float w = route_w[(size_t)tok * k + j];
         acc = acc + w * o[(size_t)row_of[(size_t)tok * k + j] * h + c];
@@ -387,10 +392,10 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 }
 
 hipError_t launch_moe_combine(const float* o, const int* row_of, const float* route_w, size_t t, size_t k, size_t h, float* y,
-                              hipStream_t s) {
+                              hipStream_t s, bool add) {
     size_t total = t * h;
     if (!total) return hipSuccess;
-    moe_combine_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(o, row_of, route_w, (uint32_t)t, (uint32_t)k, (uint32_t)h, y);
+    moe_combine_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(o, row_of, route_w, (uint32_t)t, (uint32_t)k, (uint32_t)h, y, add);
     return hipGetLastError();
 }
 

@@ -32,6 +32,11 @@ class DecodeJob(C.Structure):
                 ("ev_start", C.c_void_p), ("ev_stop", C.c_void_p)]
 
 
+class GpuInfo(C.Structure):
+    _fields_ = [("index", C.c_int), ("name", C.c_char * 256), ("arch", C.c_char * 64), ("memory_bytes", C.c_uint64),
+                ("driver", C.c_char * 64), ("usable", C.c_int)]
+
+
 class QuantJob(C.Structure):
     _fields_ = [("x", C.c_void_p), ("t", C.c_size_t), ("n_in", C.c_size_t), ("out", C.c_void_p)]
 
@@ -67,6 +72,7 @@ def load_library():
     lib = C.CDLL(_SO)
     vp, sz = C.c_void_p, C.c_size_t
     sig = {
+        "oxhip_probe": (C.c_int, [C.POINTER(GpuInfo), C.c_int]),
         "oxhip_open": (C.c_int, [C.c_int, C.POINTER(vp)]),
         "oxhip_close": (None, [vp]),
         "oxhip_name": (C.c_char_p, [vp]),
@@ -93,6 +99,15 @@ def load_library():
         "oxhip_moe_forward": (C.c_int, [vp, vp, sz, sz, sz, vp, vp, sz, vp, vp]),
         "oxhip_dev_route_top_k": (C.c_int, [vp, vp, sz, sz, sz, vp, vp, vp]),
         "oxhip_dev_moe": (C.c_int, [vp, vp, vp, sz, vp, vp, sz, vp, vp]),
+        "oxhip_buf_alloc": (vp, [vp, sz]),
+        "oxhip_buf_free": (None, [vp, vp]),
+        "oxhip_buf_write": (C.c_int, [vp, vp, vp, sz, vp]),
+        "oxhip_buf_read": (C.c_int, [vp, vp, vp, sz, vp]),
+        "oxhip_dev_rmsnorm_quantize": (C.c_int, [vp, vp, vp, vp, C.c_float, sz, sz, vp, C.POINTER(QActC), vp]),
+        "oxhip_dev_linear": (C.c_int, [vp, vp, vp, C.POINTER(QActC), vp, sz, vp, C.c_uint32, vp, vp]),
+        "oxhip_dev_glu": (C.c_int, [vp, vp, vp, sz, C.c_int, vp, vp]),
+        "oxhip_dev_route": (C.c_int, [vp, vp, vp, vp, sz, sz, sz, sz, vp, vp, vp, vp]),
+        "oxhip_dev_experts": (C.c_int, [vp, vp, vp, sz, vp, sz, vp, C.c_int, vp]),
         "oxhip_event_create": (vp, []),
         "oxhip_event_destroy": (None, [vp]),
         "oxhip_event_elapsed_ms": (C.c_float, [vp, vp]),
@@ -106,6 +121,15 @@ def load_library():
 
 def _np_ptr(a):
     return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def probe():
+    """platform::gpu::cuda::probe for HIP devices (src/platform.rs:446-482): a list of dicts like `GpuInfo`."""
+    lib = load_library()
+    arr = (GpuInfo * 16)()
+    n = lib.oxhip_probe(arr, 16)
+    return [dict(kind="hip", index=g.index, name=g.name.decode(), arch=g.arch.decode(), memory_bytes=int(g.memory_bytes),
+                 driver=g.driver.decode(), usable=bool(g.usable)) for g in arr[:min(n, 16)]]
 
 
 class DeviceWeight:
@@ -143,6 +167,7 @@ class DeviceMoe:
 
 ACT_SILU, ACT_GELU_TANH, ACT_SILU_CLAMP = 0, 1, 2
 MOE_AUTO, MOE_INT8 = 0, 1
+LIN_STORE, LIN_ADD, LIN_SILU_PAIR, LIN_GELU_PAIR, LIN_ADD_GATED = 0, 1, 2, 3, 4
 
 
 class QAct:
@@ -360,6 +385,53 @@ class HipBackend:
             y = torch.empty((t, w.n_out), dtype=torch.float32, device=f"cuda:{self.device}")
         ok = self.lib.oxhip_dev_decode_noalloc(self.ctx, w.handle, C.byref(xa.c), t, y.data_ptr(), self._stream())
         return y if ok else None
+
+    # ---- decode-graph ops (device tensors; Op::Norm / Linear / Route / Experts of src/gpu_decode.rs) -----------
+    def rmsnorm_quantize(self, x, w=None, eps=1e-6, want_out=True, want_q=True):
+        """x [t, n] f32 -> (normed [t, n] f32 or None, QAct or None); w: f32 or bf16 device tensor [n], or None."""
+        import torch
+        t, n = x.shape
+        out = torch.empty_like(x) if want_out else None
+        q = QAct(t, n, x.device) if want_q else None
+        wf = w.data_ptr() if w is not None and w.dtype == torch.float32 else None
+        wb = w.data_ptr() if w is not None and w.dtype == torch.bfloat16 else None
+        ok = self.lib.oxhip_dev_rmsnorm_quantize(self.ctx, x.data_ptr(), wf, wb, eps, t, n, out.data_ptr() if want_out else None,
+                                                 C.byref(q.c) if want_q else None, self._stream())
+        if not ok:
+            raise RuntimeError(self.last_error())
+        return out, q
+
+    def linear(self, w, y, xa=None, x=None, t=None, mode=LIN_STORE, w2=None, gate=None):
+        """Op::Linear on device tensors; y [t, n_out] f32 is written or added to according to `mode`. False = declined."""
+        t = t or (xa.t if xa is not None else x.shape[0])
+        return bool(self.lib.oxhip_dev_linear(self.ctx, w.handle, w2.handle if w2 is not None else None,
+                                              C.byref(xa.c) if xa is not None else None, x.data_ptr() if x is not None else None, t,
+                                              y.data_ptr(), mode, gate.data_ptr() if gate is not None else None, self._stream()))
+
+    def glu(self, g, u, gelu=False):
+        import torch
+        y = torch.empty_like(g)
+        if not self.lib.oxhip_dev_glu(self.ctx, g.data_ptr(), u.data_ptr(), g.numel(), int(gelu), y.data_ptr(), self._stream()):
+            raise RuntimeError(self.last_error())
+        return y
+
+    def route(self, x, router, k, gate=None, expert_scale=None):
+        """Op::Route: x [t, h], router [n_exp, h] f32 -> (logits [t, n_exp (+1)], sel int32 [2, t, k]: ids, then weight bits)."""
+        import torch
+        t, h = x.shape
+        n_exp = router.shape[0]
+        logits = torch.empty((t, n_exp + (1 if gate is not None else 0)), dtype=torch.float32, device=x.device)
+        sel = torch.empty((2, t, k), dtype=torch.int32, device=x.device)
+        ok = self.lib.oxhip_dev_route(self.ctx, x.data_ptr(), router.data_ptr(), gate.data_ptr() if gate is not None else None, t, n_exp, h, k,
+                                      logits.data_ptr(), sel.data_ptr(), expert_scale.data_ptr() if expert_scale is not None else None, self._stream())
+        if not ok:
+            raise RuntimeError(self.last_error())
+        return logits, sel
+
+    def experts(self, dev, x, sel, y, add=True):
+        """Op::Experts: the experts chosen in `sel` (as route() returns it) over x [t, h]; y += or y =."""
+        _, t, k = sel.shape
+        return bool(self.lib.oxhip_dev_experts(self.ctx, dev.handle, x.data_ptr(), t, sel.data_ptr(), k, y.data_ptr(), int(add), self._stream()))
 
     def decode_jobs(self, jobs):
         """Builds a reusable job array for decode_batch: jobs = [(DeviceWeight, QAct | None, x | None, t, y, ev0, ev1)]."""

@@ -40,6 +40,14 @@ def test_open_declines_without_a_device(lib):
     assert lib.oxhip_last_error()  # says why
 
 
+def test_probe_without_a_device_reports_none(lib):
+    import torch
+    from oxinfer_amd import hip
+    if torch.cuda.is_available():
+        pytest.skip("a device is present")
+    assert hip.probe() == []
+
+
 def test_null_arguments_decline(lib):
     assert lib.oxhip_upload(None, None) is None
     assert lib.oxhip_matmul(None, None, 0, 0, None, 0) == 0

@@ -44,6 +44,14 @@ def lcg_input(t, n, seed, oxref):
     return x * mags[np.arange(t) % 4][:, None]
 
 
+def test_probe_lists_the_device(be):
+    """The GpuKind::Hip probe (beside platform::gpu::cuda::probe, src/platform.rs:446-482)."""
+    from oxinfer_amd import hip
+    gpus = hip.probe()
+    assert len(gpus) >= 1 and gpus[0]["index"] == 0 and gpus[0]["arch"] == "gfx950" and gpus[0]["usable"]
+    assert gpus[0]["memory_bytes"] > 200 * 2 ** 30 and gpus[0]["name"] and "gfx950" in gpus[0]["driver"]
+
+
 def test_name_and_wants(be):
     assert be.name() == "hip (gfx950)"
     assert be.wants(4096, 4096, 1) and not be.wants(64, 40, 1) and not be.wants(64, 64, 0)

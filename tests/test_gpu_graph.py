@@ -1,0 +1,240 @@
+"""GPU parity of the device-resident decode-graph ops (Op::Norm / Linear / Glu / Route / Experts of the reference's
+src/gpu_decode.rs) against compositions of the CPU oracle, through the C ABI. Everything stays on the device between
+the ops; the bar is that of the decode path (1e-3 of a row's largest value, f32 accumulation)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def be():
+    import torch
+    assert torch.cuda.is_available(), "the gpu tests need a device"
+    from oxinfer_amd import HipBackend
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def row_err(y, ref):
+    m = np.maximum(np.abs(ref).max(axis=1), 1e-30)
+    return float((np.abs(y - ref).max(axis=1) / m).max())
+
+
+def rmsnorm_ref(x, w, eps):
+    """rmsnorm of the reference (src/kernels.rs:2107-2123): squares summed one after the other in f32, r = ss^(-1/2),
+    out = (x * r) * w."""
+    out = np.empty_like(x)
+    for i, row in enumerate(x):
+        sq = (row * row).astype(np.float32)
+        ss = np.add.accumulate(sq, dtype=np.float32)[-1] / np.float32(row.size) + np.float32(eps)
+        r = np.float32(ss) ** np.float32(-0.5)
+        out[i] = (row * r) * w if w is not None else row * r
+    return out.astype(np.float32)
+
+
+def weights(be, oxref, kind, n_out, n_in, seed):
+    """(device weight, decode(x, t) on the oracle) for one storage format."""
+    from oxinfer_amd import synth
+    if kind == "mlx":
+        wq, sc, bi = synth.mlx_q4(n_out, n_in, seed)
+        rng = np.random.default_rng(seed + 1)
+        sf = (sc.astype(np.uint32) << 16).view(np.float32)
+        bi = synth.bf16_bits((np.float32(-8.0) * sf + 0.01 * rng.uniform(-1, 1, sc.shape)).astype(np.float32))
+        q, s16, off = oxref.from_mlx_q4(wq, sc, bi, n_out, n_in, 64)
+        return be.upload_mlx_q4(wq, sc, bi, 64, n_out, n_in), lambda x, t: oxref.q4_decode(q, s16, off, 64, n_out, n_in, x, t)
+    if kind == "q4":  # planar Q4 without offsets: the v_dot4 kernel, whose output stage only stores
+        rng = np.random.default_rng(seed)
+        q = rng.integers(0, 256, (n_out, n_in // 2), dtype=np.uint8)
+        sc = np.abs(rng.normal(0, 0.01, (n_out, n_in // 32))).astype(np.float16).view(np.uint16)
+        sc[:, 1::2] = sc[:, 0::2] + 1  # scales differ inside a group: stays planar
+        return be.upload_q4(q, sc, None, 0, n_out, n_in), lambda x, t: oxref.q4_decode(q, sc, None, 32, n_out, n_in, x, t)
+    if kind == "bf16":
+        wf = synth.bf16_round(np.random.default_rng(seed).normal(0.0, 0.02, (n_out, n_in)).astype(np.float32))
+        return be.upload_bf16((wf.view(np.uint32) >> 16).astype(np.uint16), n_out, n_in), lambda x, t: oxref.gemm_f32(wf, n_out, n_in, x, t)
+    if kind == "fp8":
+        data, scales = synth.fp8_e4m3(n_out, n_in, seed)
+        return be.upload_fp8(data, scales, n_out, n_in), lambda x, t: oxref.gemm_quant(oxref.F8E4M3, data, scales, None, n_out, n_in, x, t)
+    raw, _ = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), seed)
+    return be.upload_gguf(kind, raw, n_out, n_in), lambda x, t: oxref.gguf_decode(kind, raw, n_out, n_in, x, t)
+
+
+@pytest.mark.parametrize("kind,n_out,n_in", [(Q4_K, 53, 768), (Q8_0, 40, 864), (Q6_K, 24, 512), (Q4_0, 33, 1120), ("mlx", 37, 640),
+                                             (Q4_K, 32, 14336), (Q8_0, 48, 14336),  # K sliced across workgroups
+                                             ("q4", 10, 512), ("bf16", 21, 520), ("fp8", 200, 512)])
+def test_linear_store_add_gated(be, oxref, kind, n_out, n_in):
+    """LinMode Store / Add / AddGated (src/gpu_decode.rs:37-50) over every storage format, 1 to 16 tokens."""
+    import torch
+    from oxinfer_amd import hip, synth
+    w, ref_of = weights(be, oxref, kind, n_out, n_in, 500)
+    assert w is not None, be.last_error()
+    dense = kind in ("bf16", "fp8")
+    for t in (1, 3, 8, 11, 16):
+        x = synth.activations(t, n_in, 510 + t, bf16=dense)
+        ref = ref_of(x, t)
+        xd = dev(x)
+        args = dict(x=xd) if dense else dict(xa=be.quantize_act(xd))
+        y0 = synth.activations(t, n_out, 520 + t) * np.abs(ref).max()
+        g = np.linspace(-3.0, 3.0, t).astype(np.float32)
+        y = torch.full((t, n_out), float("nan"), device="cuda")
+        assert be.linear(w, y, t=t, mode=hip.LIN_STORE, **args), be.last_error()
+        assert row_err(y.cpu().numpy(), ref) < TOL, t
+        y = dev(y0)
+        assert be.linear(w, y, t=t, mode=hip.LIN_ADD, **args), be.last_error()
+        assert row_err(y.cpu().numpy() - y0, ref) < TOL, t
+        y = dev(y0)
+        assert be.linear(w, y, t=t, mode=hip.LIN_ADD_GATED, gate=dev(g), **args), be.last_error()
+        sig = (1.0 / (1.0 + np.exp(-g.astype(np.float64)))).astype(np.float32)[:, None]
+        assert row_err(y.cpu().numpy() - y0, sig * ref) < TOL, t
+    # the modes must come with their operands, and only with them
+    xa1 = be.quantize_act(dev(synth.activations(1, n_in, 1))) if not dense else None
+    x1 = dev(synth.activations(1, n_in, 1)) if dense else None
+    y = torch.full((1, n_out), 7.0, device="cuda")
+    assert not be.linear(w, y, xa=xa1, x=x1, t=1, mode=hip.LIN_ADD_GATED)
+    assert not be.linear(w, y, xa=xa1, x=x1, t=1, mode=hip.LIN_STORE, gate=y)
+    assert not be.linear(w, y, xa=xa1, x=x1, t=1, mode=hip.LIN_SILU_PAIR)
+    assert not be.linear(w, y, xa=xa1, x=x1, t=17, mode=hip.LIN_STORE)
+    assert float(y.min()) == 7.0 and float(y.max()) == 7.0  # declined: nothing written
+
+
+@pytest.mark.parametrize("kind,n_out,n_in", [(Q4_K, 96, 512), (Q8_0, 40, 864), ("mlx", 80, 640), (Q4_K, 32, 14336), ("q4", 10, 512), ("bf16", 21, 520)])
+def test_linear_pairs(be, oxref, kind, n_out, n_in):
+    """LinMode SiluPair / GeluPair: y = act(W x) * (W2 x) with silu_mul / gelu_mul (src/kernels.rs:2188-2198, :2234-2257)."""
+    import torch
+    from oxinfer_amd import hip, synth
+    w, ref_w = weights(be, oxref, kind, n_out, n_in, 600)
+    u, ref_u = weights(be, oxref, kind, n_out, n_in, 601)
+    dense = kind == "bf16"
+    for t in (1, 4, 8, 13):
+        x = synth.activations(t, n_in, 610 + t, bf16=dense) * np.float32(3.0)
+        g_ref, u_ref = ref_w(x, t), ref_u(x, t)
+        xd = dev(x)
+        args = dict(x=xd) if dense else dict(xa=be.quantize_act(xd))
+        y = torch.full((t, n_out), float("nan"), device="cuda")
+        assert be.linear(w, y, t=t, mode=hip.LIN_SILU_PAIR, w2=u, **args), be.last_error()
+        assert row_err(y.cpu().numpy(), oxref.silu_mul(g_ref, u_ref)) < TOL, t
+        y = torch.full((t, n_out), float("nan"), device="cuda")
+        assert be.linear(w, y, t=t, mode=hip.LIN_GELU_PAIR, w2=u, **args), be.last_error()
+        g64 = g_ref.astype(np.float64)
+        with np.errstate(over="ignore"):  # exp overflows to inf for very negative gates: the quotient is -0.0, as on the device
+            gelu = g64 / (1.0 + np.exp(-2.0 * 0.7978846 * (g64 + 0.044715 * g64 ** 3))) * u_ref
+        assert row_err(y.cpu().numpy(), gelu.astype(np.float32)) < TOL, t
+        # Op::Glu on the two products computed apart gives the same rows as the pair
+        gd, ud = torch.empty((t, n_out), device="cuda"), torch.empty((t, n_out), device="cuda")
+        assert be.linear(w, gd, t=t, **args) and be.linear(u, ud, t=t, **args)
+        assert np.array_equal(be.glu(gd, ud, gelu=True).cpu().numpy().view(np.uint32), y.cpu().numpy().view(np.uint32))
+    if not dense:  # a second matrix of another storage format is not pairable: declined, nothing written
+        other, _ = weights(be, oxref, Q8_0 if kind != Q8_0 else Q4_0, n_out, n_in, 602)
+        y = torch.full((1, n_out), 7.0, device="cuda")
+        assert not be.linear(w, y, t=1, mode=hip.LIN_SILU_PAIR, w2=other, xa=be.quantize_act(dev(synth.activations(1, n_in, 1))))
+        assert float(y.min()) == 7.0 and float(y.max()) == 7.0
+
+
+@pytest.mark.parametrize("n", [4096, 96, 14336])
+def test_rmsnorm_quantize(be, oxref, n):
+    """Op::Norm fused with the quantization of the next linear's input: the normed row within a few ulp of rmsnorm's
+    (src/kernels.rs:2107-2123; its one-after-the-other sum of squares is not repeatable in parallel), and the QAct
+    exactly quantize_act's of that row (src/quant.rs:243-343), bit for bit."""
+    import torch
+    from oxinfer_amd import synth
+    t = 5
+    v, _ = oxref.lcg_stream(n, t * n)
+    x = ((v >> 7).astype(np.float64) / float(1 << 24) - 0.5).astype(np.float32).reshape(t, n)
+    x *= np.array([1e-3, 1.0, 300.0, 2e5, 1.0], np.float32)[:, None]
+    x[4] = 0.0  # an all-zero row: r = eps^(-1/2), every output 0
+    rng = np.random.default_rng(n)
+    wf = (1.0 + 0.1 * rng.normal(size=n)).astype(np.float32)
+    wb = synth.bf16_round(wf)
+    for eps in (1e-6, 1e-5):
+        for w_host, w_dev in ((None, None), (wf, dev(wf)), (wb, dev(wb).to(torch.bfloat16))):
+            out, qa = be.rmsnorm_quantize(dev(x), w_dev, eps)
+            out = out.cpu().numpy()
+            ref = rmsnorm_ref(x, w_host, eps)
+            assert np.allclose(out, ref, rtol=2e-5, atol=0)  # (the f32 running sum of n squares is off by up to ~sqrt(n) ulp)
+            q, scales, sums, fsums, hsums = oxref.quantize_act(out, t, n)
+            assert np.array_equal(qa.q.cpu().numpy(), q)
+            assert np.array_equal(qa.scales.cpu().numpy().view(np.uint32), scales.view(np.uint32))
+            assert np.array_equal(qa.sums.cpu().numpy(), sums)
+            assert np.array_equal(qa.fsums.cpu().numpy().view(np.uint32), fsums.view(np.uint32))
+            assert np.array_equal(qa.hsums.cpu().numpy().view(np.uint32), hsums.view(np.uint32))
+            assert np.array_equal(qa.sums16.cpu().numpy(), q.astype(np.int32).reshape(t, n // 16, 16).sum(axis=2))
+            # without the f32 output the codes are the same
+            _, qb = be.rmsnorm_quantize(dev(x), w_dev, eps, want_out=False)
+            assert np.array_equal(qb.q.cpu().numpy(), q) and np.array_equal(qb.scales.cpu().numpy().view(np.uint32), scales.view(np.uint32))
+
+
+@pytest.mark.parametrize("ne,h,k", [(128, 2048, 8), (6, 256, 3), (300, 130, 6)])
+def test_route(be, oxref, ne, h, k):
+    """Op::Route (src/gpu_decode.rs:154-172): the router's logits (and the shared expert's gate logit behind them), then
+    route_top_k over the experts' logits (src/moe.rs:180-193) into sel."""
+    from oxinfer_amd import synth
+    t = 3
+    rng = np.random.default_rng(ne)
+    router = rng.normal(0, 0.05, (ne, h)).astype(np.float32)
+    gate = rng.normal(0, 0.05, h).astype(np.float32)
+    scale = (0.5 + rng.uniform(size=ne)).astype(np.float32)
+    x = synth.activations(t, h, 7)
+    for with_gate, with_scale in ((False, False), (True, False), (True, True)):
+        logits, sel = be.route(dev(x), dev(router), k, gate=dev(gate) if with_gate else None, expert_scale=dev(scale) if with_scale else None)
+        logits, sel = logits.cpu().numpy(), sel.cpu().numpy()
+        want = x.astype(np.float64) @ router.astype(np.float64).T
+        assert np.abs(logits[:, :ne] - want).max() < 1e-5 * max(1.0, np.abs(want).max())
+        if with_gate:
+            assert np.abs(logits[:, ne] - x.astype(np.float64) @ gate.astype(np.float64)).max() < 1e-5
+        ids, wts = sel[0].view(np.uint32), sel[1].view(np.float32)
+        for i in range(t):
+            ri, rw = oxref.route_top_k(np.ascontiguousarray(logits[i, :ne]), k)
+            assert np.array_equal(ids[i], ri), i
+            assert np.allclose(wts[i], rw * (scale[ri] if with_scale else 1.0), rtol=1e-6, atol=0), i
+
+
+@pytest.mark.parametrize("ne,h,inter,k", [(6, 256, 128, 3), (16, 2048, 768, 8)])
+def test_layer_chain_stays_on_the_device(be, oxref, ne, h, inter, k):
+    """One token through residual linear (Add) -> RMSNorm + quantize -> Route -> Experts (add), every op on device
+    buffers on one stream, against the same chain composed from the oracle's pieces."""
+    import torch
+    from oxinfer_amd import hip, synth
+    raw_gu = [synth.mlx_q4(2 * inter, h, 3100 + e) for e in range(ne)]
+    raw_dn = [synth.mlx_q4(h, inter, 3200 + e) for e in range(ne)]
+    q_gu = [oxref.from_mlx_q4(*r, 2 * inter, h, 64) for r in raw_gu]
+    q_dn = [oxref.from_mlx_q4(*r, h, inter, 64) for r in raw_dn]
+    moe = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)
+    assert moe is not None, be.last_error()
+    wo_raw = synth.gguf_q4_k(h, h, 3300)
+    wo = be.upload_gguf(Q4_K, wo_raw, h, h)
+    rng = np.random.default_rng(3400 + ne)
+    router = rng.normal(0, 0.2, (ne, h)).astype(np.float32)
+    wn = (1.0 + 0.1 * rng.normal(size=h)).astype(np.float32)
+    for t in (1, 4):
+        x0 = synth.activations(t, h, 3500 + t)
+        resid = synth.activations(t, h, 3600 + t)
+        # device: four launches of the library per op group, nothing read back in between
+        y = dev(resid)
+        assert be.linear(wo, y, xa=be.quantize_act(dev(x0)), t=t, mode=hip.LIN_ADD), be.last_error()
+        normed, qa = be.rmsnorm_quantize(y, dev(wn), 1e-6)
+        logits, sel = be.route(normed, dev(router), k)
+        assert be.experts(moe, normed, sel, y, add=True), be.last_error()
+        torch.cuda.synchronize()
+        # oracle
+        y1 = resid + oxref.gguf_decode(Q4_K, wo_raw, h, h, x0, t)
+        n1 = rmsnorm_ref(y1, wn, 1e-6)
+        idx = np.zeros((t, k), np.uint32)
+        w = np.zeros((t, k), np.float32)
+        for i in range(t):
+            idx[i], w[i] = oxref.route_top_k((n1[i].astype(np.float64) @ router.astype(np.float64).T).astype(np.float32), k)
+        assert np.array_equal(sel[0].cpu().numpy().view(np.uint32), idx)
+        y2 = oxref.moe_q4(q_gu, q_dn, 64, h, inter, n1, t, idx, w, y1, decode_path=True)
+        assert row_err(y.cpu().numpy(), y2) < TOL, (t, row_err(y.cpu().numpy(), y2))
+        # Experts with add = false writes the experts' sum alone
+        only = torch.full((t, h), float("nan"), device="cuda")
+        assert be.experts(moe, normed, sel, only, add=False)
+        assert row_err(only.cpu().numpy(), y2 - y1) < TOL
