@@ -40,7 +40,7 @@ def build(verbose=False, tuning=False):
     and orders, for measurement scripts); the library that ships is always built without them."""
     os.makedirs(OBJ, exist_ok=True)
     cc = hipcc()
-    extra_all = ["-DOXHIP_TUNING"] if tuning else []
+    extra_all = (["-DOXHIP_TUNING"] + os.environ.get("OXHIP_EXP_FLAGS", "").split()) if tuning else []
 
     def one(src):
         obj = os.path.join(OBJ, src.replace(".hip", ".o"))

@@ -44,6 +44,7 @@
 namespace oxhip {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 // Where slot `slot` (0..63) of row `row` of the LDS operand array sits: the staging stores of a token's consecutive chunks
 // differ only in the row and in slot bits 3 and 5, which alone would put 64 lanes into two bank pairs; mixing the row's
@@ -57,36 +58,20 @@ namespace {
 template <int FMT, int NT>
 constexpr int pf_for() { return FMT == FMT_Q6_K ? 4 : 8; }  // Q6_K records are 1.7 KiB and its step needs the registers
 
-struct Meta4 {
-    float xs[4];
-    float c[4];
-    float fs[4];
-    int su[4];
-};
-
-// The kernels evaluate a block's contribution with the fewest f32 operations per (row, token):
-//   Q8_0:  d * (xs * I)
-//   Q4_K:  d * sc * (xs * U + c) - dmin * mn * fs,   c = 8 * (fs - xs * su)      [U = sum of unsigned nibbles * q]
-//   MLX:   d * (xs * U + c) + off * fs,              c = -8 * xs * su
-// which equal the reference's (s * xs) * (U - 8 su) + m * fs (src/ggml.rs:1288-1315, src/kernels.rs:1287-1297)
-// up to f32 rounding; the integer sums U - 8 su themselves are exact (and are what the DUMP variant writes).
-// LDS: xs | c | fs | su, each [nbl][TPAD] over the workgroup's nbl blocks from b0 (c, fs only for the formats with
-// sums; su only for DUMP)
-// `as`: floats per array (xs, c, fs, su in turn); `at`: index of the lane's first token in its block's row
-template <bool SUMS, bool DUMP>
-__device__ __forceinline__ void load_meta(const float* lds, uint32_t as, uint32_t at, Meta4& m) {
+// The kernels evaluate a block's contribution as the reference does (src/ggml.rs:1288-1315, src/kernels.rs:1287-1297):
+//   Q8_0:        d * (xs * I)                                  I = sum of codes * activation codes (exact)
+//   4-bit:       (s / 16) * (xs * I16) + m * fs                I16 = 16 * sum of (nibble - 8) * activation codes (exact)
+//                Q4_K: s = d * sc, m = 8 s - dmin * mn (decode_i8's s and m);  MLX: s = d, m = the group's offset
+// up to the order of the f32 operations. The centred nibbles go to the matrix cores as the int8 values 16 * (nibble - 8)
+// (a nibble moved to the top of its byte with its top bit flipped), so the integer sum needs no correction by the
+// activations' own sums; the DUMP variant writes I16 / 16. The m * fs terms of a step's four blocks are one more
+// matrix instruction (f32, 16 x 16 x 4: rows = tokens, K = the four blocks), straight into the accumulators.
+// LDS metadata: xs [nbl][TPAD], and for the formats with mins or offsets fs [nbl][TPAD], over the workgroup's nbl
+// blocks from b0. Q6_K keeps its own three arrays (see its step).
+// `at`: index of the lane's first token in its block's row
+__device__ __forceinline__ void load_xs(const float* lds, uint32_t at, float* xs) {
     const float4 x = *reinterpret_cast<const float4*>(lds + at);
-    m.xs[0] = x.x; m.xs[1] = x.y; m.xs[2] = x.z; m.xs[3] = x.w;
-    if (SUMS) {
-        const float4 c = *reinterpret_cast<const float4*>(lds + (size_t)as + at);
-        const float4 f = *reinterpret_cast<const float4*>(lds + (size_t)2 * as + at);
-        m.c[0] = c.x; m.c[1] = c.y; m.c[2] = c.z; m.c[3] = c.w;
-        m.fs[0] = f.x; m.fs[1] = f.y; m.fs[2] = f.z; m.fs[3] = f.w;
-        if (DUMP) {
-            const int4 q = *reinterpret_cast<const int4*>(lds + (size_t)3 * as + at);
-            m.su[0] = q.x; m.su[1] = q.y; m.su[2] = q.z; m.su[3] = q.w;
-        }
-    }
+    xs[0] = x.x; xs[1] = x.y; xs[2] = x.z; xs[3] = x.w;
 }
 
 }  // namespace
@@ -148,7 +133,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // the swizzled operand array pays at 8 tokens (where the staging stores are many); at fewer its address math costs more
     constexpr bool SWZ = NT >= 8;
     constexpr int NI = NT < 4 ? NT : 4;          // accumulator registers that hold live tokens
-    constexpr bool SUMS = !q8_format(FMT);
+    constexpr bool MINS = FMT == FMT_Q4_K || FMT == FMT_Q4M;   // m * fs terms (Q4_0 has none)
+    constexpr int NARR = q8_format(FMT) || FMT == FMT_Q40 ? 1 : FMT == FMT_Q6_K ? (DUMP ? 4 : 3) : 2;  // metadata arrays
     // the wave index and everything derived from it (tile, K range) live in scalar registers: branches on them are
     // scalar, and the load counters the compiler keeps stay exact across them
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -175,7 +161,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     uint2* afr = reinterpret_cast<uint2*>(lds_all);  // [NG][nbl / 2][64]
     float* lds = lds_all + (ALDS ? (size_t)NG * (nbl / 2) * 128 : 0);
     const uint32_t nm = nbl * TPAD, as = NG * nm;  // scale entries of a token group; floats per array
-    float* red = ALDS ? lds_all : lds + (size_t)(SUMS ? (DUMP ? 4 : 3) : 1) * as;  // [rt * kw][NG][TPAD][16]
+    float* red = ALDS ? lds_all : lds + (size_t)NARR * as;  // [rt * kw][NG][TPAD][16]
     uint32_t row0 = 0;  // first activation / output row of this launch unit
     if (GROUPED) {
         if (by >= (uint32_t)*grp.nchunks) return;  // uniform over the workgroup
@@ -193,6 +179,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     const uint32_t amask0 = a_half ? 0u : 0xFFFFFFFFu, amask1 = ~amask0;
     // D role: this lane's registers are tokens 4 (kq & 1) + i of block parity kq >> 1
     const uint32_t d_half = kq >> 1, d_tok0 = 4 * (kq & 1);
+    // Q4_K: the bytes this lane takes from a step's {scales, mins} words (v_perm_b32: 0..3 = the scales, 4..7 = the mins)
+    const uint32_t q4k_sel = d_half | ((2 + d_half) << 8) | (kq << 16) | ((4 + kq) << 24);
 
     const uint32_t per = (S1 - S0 + kw - 1) >> kwsh;
     const uint32_t s0 = S0 + ks * per;
@@ -281,19 +269,37 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     for (int g = 0; g < NG; g++)
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[g][i] = 0.0f;
+    // the m * fs terms accumulate on their own (a chain of matrix instructions that depends on nothing else) and join at the end
+    v4f macc[MINS ? NG : 1];
+#pragma unroll
+    for (int g = 0; g < (MINS ? NG : 1); g++) macc[g] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
     // Q6_K: every lane group sums its own 16-column sub-block for tokens 4 tg + i
     float acc6a[4] = {0.0f, 0.0f, 0.0f, 0.0f}, acc6b[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // tg = 0, 1
     // `m`: index of the instruction along K (pair of blocks 2 m, 2 m + 1); with ALDS its operand comes from LDS
     auto mfma = [&](v4i bw, uint32_t m, int tg, uint32_t d0, uint32_t d1) -> v4i {
+        v4i c = {0, 0, 0, 0};
         if (ALDS) {
             const uint2 av = afr[((size_t)tg * (nbl / 2) + (m - M0)) * 64 + (SWZ ? opslot(m - M0, lane) : lane)];
             d0 = av.x;
             d1 = av.y;
         }
         v4i a = {(int)(d0 & amask0), (int)(d1 & amask0), (int)(d0 & amask1), (int)(d1 & amask1)};
-        v4i c = {0, 0, 0, 0};
         return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bw, c, 0, 0, 0);
     };
+    // The m * fs terms of the step's four blocks (blocks b4 .. b4 + 3): rows = tokens (8 .. 15: none), K = the blocks;
+    // this lane supplies fs of (token n, block b4 + kq) and `mk`, row n's m of block b4 + kq. D[4 kq + i][n]: the lane
+    // groups 0 and 1 receive the tokens their accumulators hold, the others zeros.
+    auto mins = [&](uint32_t b4, float mk) {
+        if constexpr (MINS) {
+            const uint32_t at = (min(b4 + kq, nblk - 1) - B0) * TPAD + min(n, (uint32_t)TPAD - 1);
+#pragma unroll
+            for (int tg = 0; tg < NG; tg++) {
+                const float f = lds[(size_t)as + tg * nm + at];
+                macc[tg] = __builtin_amdgcn_mfma_f32_16x16x4f32(n < (uint32_t)TPAD ? f : 0.0f, mk, macc[tg], 0, 0, 0);
+            }
+        }
+    };
+    constexpr uint32_t CENTRE = 0x88888888u, TOPN = 0xF0F0F0F0u;
     auto dump_block = [&](uint32_t b, const int* isum) {
         if (!DUMP) return;
         const uint32_t row = tile * 16 + n;
@@ -311,49 +317,43 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
 #pragma unroll
             for (int tg = 0; tg < NG; tg++) {
                 v4i D = mfma(bw, s, tg, st.a[0], st.a[1]);
-                Meta4 m;
-                load_meta<SUMS, DUMP>(lds, as, tg * nm + (min(b, nblk - 1) - B0) * TPAD + d_tok0, m);
+                float xs[4];
+                load_xs(lds, tg * nm + (min(b, nblk - 1) - B0) * TPAD + d_tok0, xs);
                 int isum[4] = {D.x, D.y, D.z, D.w};
 #pragma unroll
-                for (int i = 0; i < NI; i++) acc[tg][i] = fmaf(d, m.xs[i] * (float)isum[i], acc[tg][i]);
+                for (int i = 0; i < NI; i++) acc[tg][i] = fmaf(d, xs[i] * (float)isum[i], acc[tg][i]);
                 dump_block(b, isum);
             }
         } else if constexpr (FMT == FMT_Q4_K) {
-            const float d = f16_bits_to_f32((uint16_t)(sw[2] & 0xFFFF)), ndmin = -f16_bits_to_f32((uint16_t)(sw[2] >> 16));
-            float P[NG][4], Q[NG][4];
-#pragma unroll
-            for (int tg = 0; tg < NG; tg++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) P[tg][i] = Q[tg][i] = 0.0f;
+            // sw[0]: the step's four sub-block scales, sw[1]: its four mins (bytes), sw[2]: (d, dmin). One byte permute
+            // gathers this lane's four: the scales of its two blocks (sub-blocks d_half and 2 + d_half of the step) and,
+            // for the mins' matrix instruction, the scale and min of sub-block kq.
+            const float d = f16_bits_to_f32((uint16_t)(sw[2] & 0xFFFF)), dmin = f16_bits_to_f32((uint16_t)(sw[2] >> 16));
+            const uint32_t pk = __builtin_amdgcn_perm(sw[1], sw[0], q4k_sel);
+            const float d16 = d * 0.0625f;
+            const float dsc[2] = {d16 * (float)(pk & 0xFF), d16 * (float)((pk >> 8) & 0xFF)};
+            // decode_i8's m of sub-block kq: 8 s - dmin * mn (src/ggml.rs:1046-1073)
+            const float mk = fmaf(8.0f * d, (float)((pk >> 16) & 0xFF), -(dmin * (float)(pk >> 24)));
 #pragma unroll
             for (int pr = 0; pr < 2; pr++) {  // the two byte pairs of the lane's chunk
-                const uint32_t lo = pr ? c.z : c.x, hi = pr ? c.w : c.y;
-                v4i bw = {(int)(lo & 0x0F0F0F0Fu), (int)(hi & 0x0F0F0F0Fu), (int)((lo >> 4) & 0x0F0F0F0Fu),
-                          (int)((hi >> 4) & 0x0F0F0F0Fu)};
+                const uint32_t x0 = (pr ? c.z : c.x) ^ CENTRE, x1 = (pr ? c.w : c.y) ^ CENTRE;
+                v4i bw = {(int)((x0 << 4) & TOPN), (int)((x1 << 4) & TOPN), (int)(x0 & TOPN), (int)(x1 & TOPN)};
                 const uint32_t b = 4 * s + 2 * pr + d_half;  // global index of this lane's block of 32
-                const uint32_t q = 2 * pr + d_half;
-                const float sc = (float)((sw[0] >> (8 * q)) & 0xFF), mn = (float)((sw[1] >> (8 * q)) & 0xFF);
 #pragma unroll
                 for (int tg = 0; tg < NG; tg++) {
                     v4i D = mfma(bw, 2 * s + pr, tg, st.a[2 * pr], st.a[2 * pr + 1]);
-                    Meta4 m;
-                    load_meta<SUMS, DUMP>(lds, as, tg * nm + (b - B0) * TPAD + d_tok0, m);
-                    const int U[4] = {D.x, D.y, D.z, D.w};
+                    float xs[4];
+                    load_xs(lds, tg * nm + (b - B0) * TPAD + d_tok0, xs);
+                    const int I[4] = {D.x, D.y, D.z, D.w};
 #pragma unroll
-                    for (int i = 0; i < NI; i++) {
-                        P[tg][i] = fmaf(sc, fmaf(m.xs[i], (float)U[i], m.c[i]), P[tg][i]);
-                        Q[tg][i] = fmaf(mn, m.fs[i], Q[tg][i]);
-                    }
+                    for (int i = 0; i < NI; i++) acc[tg][i] = fmaf(dsc[pr], xs[i] * (float)I[i], acc[tg][i]);
                     if (DUMP) {
-                        int isum[4] = {U[0] - 8 * m.su[0], U[1] - 8 * m.su[1], U[2] - 8 * m.su[2], U[3] - 8 * m.su[3]};
+                        int isum[4] = {I[0] >> 4, I[1] >> 4, I[2] >> 4, I[3] >> 4};
                         dump_block(b, isum);
                     }
                 }
             }
-#pragma unroll
-            for (int tg = 0; tg < NG; tg++)
-#pragma unroll
-                for (int i = 0; i < NI; i++) acc[tg][i] = fmaf(ndmin, Q[tg][i], fmaf(d, P[tg][i], acc[tg][i]));
+            mins(4 * s, mk);
         } else if constexpr (FMT == FMT_Q6_K) {
             // Scales go per 16 columns, so an instruction's 16 operand slots are (sub-block sb, token t4): lane group kq
             // supplies sub-block kq's 16 activations of token t4 in the slots with sb = kq and zeros elsewhere, and lane
@@ -402,32 +402,32 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         } else {
 #pragma unroll
             for (int g = 0; g < 2; g++) {  // the two groups of 64 of the step
-                const uint32_t w0 = g ? c.z : c.x, w1 = g ? c.w : c.y;  // blocks 2 g, 2 g + 1
-                v4i bw = {(int)(w0 & 0x0F0F0F0Fu), (int)((w0 >> 4) & 0x0F0F0F0Fu), (int)(w1 & 0x0F0F0F0Fu),
-                          (int)((w1 >> 4) & 0x0F0F0F0Fu)};
+                const uint32_t x0 = (g ? c.z : c.x) ^ CENTRE, x1 = (g ? c.w : c.y) ^ CENTRE;  // blocks 2 g, 2 g + 1
+                v4i bw = {(int)((x0 << 4) & TOPN), (int)(x0 & TOPN), (int)((x1 << 4) & TOPN), (int)(x1 & TOPN)};
                 const uint32_t b = 4 * s + 2 * g + d_half;
-                // MLX: the group's scale and offset; Q4_0: the lane's block's own scale (word g, half d_half), no offset
+                // MLX: the group's scale; Q4_0: the lane's block's own scale (word g, half d_half)
                 const float d = FMT == FMT_Q40 ? f16_bits_to_f32((uint16_t)(d_half ? sw[g] >> 16 : sw[g] & 0xFFFF))
                                                : f16_bits_to_f32((uint16_t)(g ? sw[0] >> 16 : sw[0] & 0xFFFF));
-                const float off = FMT == FMT_Q40 ? 0.0f : bf16_bits_to_f32((uint16_t)(g ? sw[1] >> 16 : sw[1] & 0xFFFF));
-                const float dz = b < nblk ? d : 0.0f, offz = b < nblk ? off : 0.0f;
+                // padding blocks hold zero codes (which centre to -8) and zero scales: they add zeros (as a select, not a
+                // branch: a divergent branch here makes every step wait for all requests)
+                const float dz = b < nblk ? d * 0.0625f : 0.0f;
 #pragma unroll
                 for (int tg = 0; tg < NG; tg++) {
                     v4i D = mfma(bw, 2 * s + g, tg, st.a[2 * g], st.a[2 * g + 1]);
-                    Meta4 m;
-                    load_meta<SUMS, DUMP>(lds, as, tg * nm + (min(b, nblk - 1) - B0) * TPAD + d_tok0, m);
-                    const int U[4] = {D.x, D.y, D.z, D.w};
-                    // padding blocks hold zero codes and zero scales, but their staged sums are a real block's: they add
-                    // zeros (as a select, not a branch: a divergent branch here makes every step wait for all requests)
+                    float xs[4];
+                    load_xs(lds, tg * nm + (min(b, nblk - 1) - B0) * TPAD + d_tok0, xs);
+                    const int I[4] = {D.x, D.y, D.z, D.w};
 #pragma unroll
-                    for (int i = 0; i < NI; i++)
-                        acc[tg][i] = FMT == FMT_Q40 ? fmaf(dz, fmaf(m.xs[i], (float)U[i], m.c[i]), acc[tg][i])
-                                                    : fmaf(offz, m.fs[i], fmaf(dz, fmaf(m.xs[i], (float)U[i], m.c[i]), acc[tg][i]));
+                    for (int i = 0; i < NI; i++) acc[tg][i] = fmaf(dz, xs[i] * (float)I[i], acc[tg][i]);
                     if (DUMP) {
-                        int isum[4] = {U[0] - 8 * m.su[0], U[1] - 8 * m.su[1], U[2] - 8 * m.su[2], U[3] - 8 * m.su[3]};
+                        int isum[4] = {I[0] >> 4, I[1] >> 4, I[2] >> 4, I[3] >> 4};
                         dump_block(b, isum);
                     }
                 }
+            }
+            if constexpr (FMT == FMT_Q4M) {  // the offset of block kq's group of 64, times the block's exact activation sum
+                const float off = bf16_bits_to_f32((uint16_t)(kq >> 1 ? sw[1] >> 16 : sw[1] & 0xFFFF));
+                mins(4 * s, 4 * s + kq < nblk ? off : 0.0f);
             }
         }
     };
@@ -503,9 +503,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             r.sq2 = live ? xa.sums16[2 * src + 1] : 0;
             r.f = 0.0f;
         } else {
-            r.sq = SUMS && live ? xa.sums[src] : 0;
-            r.sq2 = 0;
-            r.f = SUMS && live ? xa.fsums[src] : 0.0f;
+            r.sq = r.sq2 = 0;
+            r.f = MINS && live ? xa.fsums[src] : 0.0f;
         }
     };
     auto meta_store = [&](uint32_t q, uint32_t b, const MetaReg& r) {
@@ -515,10 +514,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             lds[(size_t)as + at] = -32.0f * (r.x * (float)r.sq);
             lds[(size_t)2 * as + at] = -32.0f * (r.x * (float)r.sq2);
             if (DUMP) reinterpret_cast<int*>(lds)[(size_t)3 * as + at] = (r.sq & 0xFFFF) | (r.sq2 << 16);
-        } else if (SUMS) {
-            lds[(size_t)as + at] = FMT == FMT_Q4_K ? 8.0f * (r.f - r.x * (float)r.sq) : -8.0f * (r.x * (float)r.sq);
-            lds[(size_t)2 * as + at] = r.f;
-            if (DUMP) reinterpret_cast<int*>(lds)[(size_t)3 * as + at] = r.sq;
+        } else if (MINS) {
+            lds[(size_t)as + at] = r.f;
         }
     };
     uint4 sa[SA];
@@ -624,6 +621,12 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             acc[0][i] = (kq & 1) ? b : a;
         }
     } else {
+        if constexpr (MINS) {
+#pragma unroll
+            for (int g = 0; g < NG; g++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[g][i] += macc[g][i];
+        }
         // the two block parities of a token meet across lane groups kq and kq ^ 2
 #pragma unroll
         for (int g = 0; g < NG; g++)
@@ -844,10 +847,13 @@ Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices, int fmt) {
 
 constexpr size_t LDS_MAX = 160 * 1024 - 256;  // dynamic LDS on offer (the kernel also holds a static word)
 
-// Dynamic LDS of a launch; `alds` comes back false when the operand-order activations do not fit.
-size_t lds_bytes(bool sums, bool dump, uint32_t bps, uint32_t nsteps, int tpad, const Shape& sh, bool* alds, uint32_t ng = 1) {
+// Dynamic LDS of a launch; `alds` comes back false when the operand-order activations do not fit (they are then read
+// from L2 per record).
+size_t lds_bytes(int fmt, bool dump, uint32_t nsteps, int tpad, const Shape& sh, bool* alds, uint32_t ng = 1) {
+    const uint32_t bps = q8_format(fmt) ? 2 : 4;
     const uint32_t nbl = bps * ((nsteps + sh.ks - 1) / sh.ks);  // blocks of a slice
-    const size_t meta = (size_t)(sums ? (dump ? 4 : 3) : 1) * ng * nbl * tpad * 4, red = (size_t)sh.rt * sh.kw * ng * tpad * 16 * 4;
+    const uint32_t narr = q8_format(fmt) || fmt == FMT_Q40 ? 1 : fmt == FMT_Q6_K ? (dump ? 4 : 3) : 2;  // metadata arrays
+    const size_t meta = (size_t)narr * ng * nbl * tpad * 4, red = (size_t)sh.rt * sh.kw * ng * tpad * 16 * 4;
     const size_t act = (size_t)ng * (nbl / 2) * 512;
     const size_t with = act + meta > red ? act + meta : red;  // the partial sums reuse the activations' space
     *alds = with <= LDS_MAX;
@@ -918,7 +924,7 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
         int32_t* du = dump ? dump + c0 * (size_t)w.n_out * nblk * (FMT == FMT_Q6_K ? 2 : 1) : nullptr;
         const int tpad = tc <= 4 ? 4 : 8;
         bool alds;
-        const size_t lds = lds_bytes(!q8_format(FMT), DUMP, q8_format(FMT) ? 2 : 4, nsteps, tpad, sh, &alds);
+        const size_t lds = lds_bytes(FMT, DUMP, nsteps, tpad, sh, &alds);
         if (lds > LDS_MAX) return hipErrorInvalidValue;  // rows too long for the staged activation scales
         const uint32_t tt = (uint32_t)tc;
         Epi epi = epi0;
@@ -956,7 +962,7 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
     const uint32_t ng = max_rows <= 8 ? 1 : (max_rows <= 16 ? 2 : 4);
     if (max_rows > 32) return hipErrorInvalidValue;
     bool alds;
-    const size_t lds = lds_bytes(!q8_format(FMT), false, q8_format(FMT) ? 2 : 4, nsteps, tpad, sh, &alds, ng);
+    const size_t lds = lds_bytes(FMT, false, nsteps, tpad, sh, &alds, ng);
     if (lds > LDS_MAX || (ng > 1 && !alds)) return hipErrorInvalidValue;
     const DecodeScratch none{};
     if (max_rows == 1) return launch_one<FMT, 1, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
@@ -982,7 +988,7 @@ bool decode_batchable(const WeightView& w, size_t t) {
     if (t < 1 || t > 8) return false;
     const Shape sh = shape_for(row_tiles(w.n_out), steps_rt(w), true, w.fmt);  // as a launch of its own: same bits
     bool alds;
-    const size_t lds = lds_bytes(!q8_format(w.fmt), false, q8_format(w.fmt) ? 2 : 4, steps_rt(w), t <= 4 ? 4 : 8, sh, &alds);
+    const size_t lds = lds_bytes(w.fmt, false, steps_rt(w), t <= 4 ? 4 : 8, sh, &alds);
     return alds && lds <= LDS_MAX;
 }
 
@@ -1046,7 +1052,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
             const uint32_t ntiles = row_tiles(it.w.n_out), nsteps = steps_rt(it.w);
             const Shape sh = shape_for(ntiles, nsteps, true, it.w.fmt);
             bool alds;
-            const size_t l = lds_bytes(!q8_format(it.w.fmt), false, q8_format(it.w.fmt) ? 2 : 4, nsteps, it.t <= 4 ? 4 : 8, sh, &alds);
+            const size_t l = lds_bytes(it.w.fmt, false, nsteps, it.t <= 4 ? 4 : 8, sh, &alds);
             if (!alds || l > LDS_MAX || it.t < 1 || it.t > 8) return hipErrorInvalidValue;
             const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
             float* partial = nullptr;
@@ -1097,7 +1103,7 @@ bool decode_grouped_fits(const WeightView& w, uint32_t max_rows) {
     const Shape sh{8 / gkw, gkw, 1};
     const uint32_t ng = max_rows <= 8 ? 1 : (max_rows <= 16 ? 2 : 4);
     bool alds;
-    const size_t lds = lds_bytes(!q8_format(w.fmt), false, q8_format(w.fmt) ? 2 : 4, nsteps, max_rows <= 4 ? 4 : 8, sh, &alds, ng);
+    const size_t lds = lds_bytes(w.fmt, false, nsteps, max_rows <= 4 ? 4 : 8, sh, &alds, ng);
     return lds <= LDS_MAX && (alds || (ng == 1 && w.fmt != FMT_Q6_K));
 }
 
