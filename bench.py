@@ -363,9 +363,10 @@ def bench_moe(be, torch, synth, steps, warmup, pool_gb, t, experts, int8=False):
     # six or more routed rows per expert: the library takes the bf16 form of the grouped matmuls (the reference's prefill form)
     prefill_form = (t * k) // ne >= 6 and not int8
 
-    def step(i):
-        be.route_top_k(logits, k)
-        be.dev_moe(devs[i % len(devs)], x, idx, w, y)
+    sel = torch.empty((2, t, k), dtype=torch.int32, device="cuda")
+
+    def step(i):  # routing (top-k of the logits) and the experts, one library call
+        be.moe_routed(devs[i % len(devs)], x, logits, k, y, sel=sel)
     wall, ms = timed_steps(torch, step, steps, warmup)
     ach = nbytes / (ms * 1e-3) / 1e9
     return dict(base_line(steps, warmup), value=round(nbytes * steps / wall / 1e9, 2), unit="GB/s", ms_per_step=round(wall / steps * 1e3, 5),

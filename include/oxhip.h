@@ -280,6 +280,15 @@ int oxhip_dev_route(oxhip_ctx* ctx, const float* x, const float* router, const f
  * (SiLU / GELU-tanh) is the layer's (oxhip_upload_moe). */
 int oxhip_dev_experts(oxhip_ctx* ctx, oxhip_moe* m, const float* x, size_t t, const uint32_t* sel, size_t k, float* y, int add, void* stream);
 
+/* Op::Route's top-k and Op::Experts in one call, for plans that keep the router's logits on the device: `logits`
+ * [t] rows of n_experts (rows `logit_stride` floats apart; 0 = n_experts), as oxhip_dev_route leaves them; `sel`
+ * receives the routes (ids [t, k], then weights [t, k]) and y the experts' weighted sum (added or stored). For one
+ * token over fused gate / up experts the pass is three launches: routing + input quantization; gate / up with the
+ * activation and its quantization in the launch's output stage; down with the route-order combination done by the last
+ * workgroup of each row group to finish. */
+int oxhip_dev_moe_routed(oxhip_ctx* ctx, oxhip_moe* m, const float* x, size_t t, const float* logits, size_t logit_stride, size_t k,
+                         const float* expert_scale, uint32_t* sel, float* y, int add, void* stream);
+
 /* The exact integer accumulators of the decode kernels, written by the kernels themselves: per
  * block of 32 ([t, n_out, n_in/32]) for Q4, Q8, Q8_0 and Q4_K, per 16 ([t, n_out, n_in/16]) for Q6_K.
  * For parity checks (the CPU's per-16 sums add up to the per-32 ones exactly). */

@@ -27,6 +27,8 @@ bool mfma_format(const oxhip_weight* w) { return w->v.fmt == FMT_Q8_0 || w->v.fm
 
 size_t up256(size_t v) { return (v + 255) / 256 * 256; }
 
+constexpr size_t COMB_GROUPS = 4096;  // row groups of the down projection that may meet through counters (h <= 65536)
+
 // The scratch of one pass, carved from one allocation.
 struct Scratch {
     int* row_of;
@@ -40,6 +42,7 @@ struct Scratch {
     float* o;       // [pairs][h]
     void* fx;       // bf16 fragments of the chunks' rows of x, and of a (the prefill form: chunks of up to 16 rows)
     void* fa;
+    uint32_t* counters;  // arrival counters of the down launch's row groups (zero between launches)
     uint32_t max_chunks;
     size_t bytes;
 };
@@ -56,6 +59,8 @@ Scratch carve(uint8_t* base, size_t t, size_t pairs, size_t n_exp, size_t h, siz
         off += up256(bytes);
         return p;
     };
+    // (the counters first: their place must not depend on the pass's size, they stay zero from one pass to the next)
+    s.counters = reinterpret_cast<uint32_t*>(take((size_t)COMB_GROUPS * CTR_STRIDE * 4));
     s.row_of = reinterpret_cast<int*>(take(pairs * 4));
     s.src = reinterpret_cast<int*>(take(pairs * 4));
     s.chunks = reinterpret_cast<int4*>(take((size_t)s.max_chunks * 16));
@@ -73,10 +78,21 @@ Scratch carve(uint8_t* base, size_t t, size_t pairs, size_t n_exp, size_t h, siz
     return s;
 }
 
+// Routing inside the pass: with `logits` ([t] rows `logit_stride` apart) the top-k of every token is formed first, into
+// route_idx / route_w (then outputs: [t, k] each).
+struct RouteIn {
+    const float* logits = nullptr;
+    size_t stride = 0;
+    const float* expert_scale = nullptr;
+};
+
 int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t* route_idx, const float* route_w, size_t k,
-            float* y, hipStream_t s, bool add = true) {
+            float* y, hipStream_t s, bool add = true, const RouteIn& rin = RouteIn{}) {
     const size_t pairs = t * k, h = m->h, inter = m->inter;
     if (!pairs) return 1;
+    uint32_t* ridx_out = const_cast<uint32_t*>(route_idx);
+    float* rw_out = const_cast<float*>(route_w);
+    bool routed = rin.logits == nullptr;  // the routes are there (given, or already formed)
     if (pairs > m->ws_pairs || t > m->ws_t) {
         (void)hipStreamSynchronize(s);  // an earlier pass may still read the old scratch
         const size_t np = pairs > m->ws_pairs ? pairs : m->ws_pairs, nt = t > m->ws_t ? t : m->ws_t;
@@ -88,6 +104,8 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
         }
         m->ws_pairs = np;
         m->ws_t = nt;
+        // the arrival counters start at zero (every launch leaves them so); the buffer moved, and its layout with it
+        HIP_TRY(hipMemsetAsync(m->ws.p, 0, m->ws.cap, s), "moe scratch clear");
     }
     Scratch sc = carve(static_cast<uint8_t*>(m->ws.p), t, pairs, m->n_exp, h, inter);
     // Rows per chunk: one pass over an expert's weights serves a whole chunk, so chunks grow with the rows an expert
@@ -125,6 +143,13 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
     GroupView g{};
     g.chunks = sc.chunks;
     g.nchunks = sc.nchunks;
+    // One token over fused gate / up experts needs no plan: chunk j is route j (see GroupView::direct); its routing
+    // and the quantization of x share a launch, and the pass is three launches.
+    const bool direct = !bf16_form && t == 1 && fused && decode_grouped_glu_ok(m->gate_up[0]->v, inter) && row_tiles((uint32_t)h) <= COMB_GROUPS;
+    if (!routed && !(direct && m->n_exp <= 256)) {
+        HIP_TRY(launch_route_top_k(rin.logits, t, m->n_exp, k, ridx_out, rw_out, s, rin.stride, rin.expert_scale), "route_top_k launch");
+        routed = true;
+    }
     if (bf16_form) {
         HIP_TRY(launch_moe_plan(route_idx, pairs, k, m->n_exp, max_rows, sc.row_of, sc.src, sc.chunks, sc.nchunks, s), "moe plan launch");
         HIP_TRY(launch_moe_pack_bf16(x, h, sc.src, sc.chunks, sc.nchunks, grid_chunks, sc.fx, s), "moe pack launch");
@@ -135,10 +160,36 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
         g.bases = m->bases_dn;
         HIP_TRY(launch_moe_bf16(m->down[0]->v, g, grid_chunks, sc.fa, sc.o, s), "moe down launch");
     } else {
-        HIP_TRY(launch_moe_front(route_idx, pairs, k, m->n_exp, max_rows, sc.row_of, sc.src, sc.chunks, sc.nchunks, x, t, h, sc.xa, s), "moe plan launch");
+        if (direct) {
+            if (!routed) HIP_TRY(launch_route_quantize(rin.logits, 1, m->n_exp, k, ridx_out, rw_out, rin.stride, rin.expert_scale, x, h, sc.xa, s), "route + quantize launch");
+            else HIP_TRY(launch_quantize_act(x, 1, h, sc.xa, s), "moe quantize launch");
+            g.direct = route_idx;
+            g.direct_n = (uint32_t)k;
+            g.direct_x0 = 1;
+        } else {
+            HIP_TRY(launch_moe_front(route_idx, pairs, k, m->n_exp, max_rows, sc.row_of, sc.src, sc.chunks, sc.nchunks, x, t, h, sc.xa, s), "moe plan launch");
+        }
         // gate / up over the routed rows of x (row i of the gathered order is token src[i])
-        g.rowmap = sc.src;
+        g.rowmap = direct ? nullptr : sc.src;
         g.bases = m->bases_gu;
+        // fused gate / up experts whose launch pairs gate and up tiles: the activation and the quantization of its output
+        // are the launch's own output stage; the down launch then also combines (the last workgroup of a row group to
+        // finish adds the routed rows in route order): three launches for a decode-sized pass
+        const bool glu_fused = fused && decode_grouped_glu_ok(m->gate_up[0]->v, inter);
+        const bool comb_fused = row_tiles((uint32_t)h) <= COMB_GROUPS;
+        if (glu_fused) {
+            GroupView gg = g;
+            gg.glu_inter = (uint32_t)inter;
+            gg.act_kind = m->act_kind;
+            gg.act_param = m->act_param;
+            gg.aq_q = sc.aq.q;
+            gg.aq_scales = sc.aq.scales;
+            gg.aq_sums = sc.aq.sums;
+            gg.aq_fsums = sc.aq.fsums;
+            gg.aq_hsums = sc.aq.hsums;
+            gg.aq_sums16 = sc.aq.sums16;
+            HIP_TRY(launch_decode_mfma_grouped(m->gate_up[0]->v, view_of(sc.xa), gg, grid_chunks, max_rows, sc.gu, s), "moe gate launch");
+        } else {
         HIP_TRY(launch_decode_mfma_grouped(m->gate_up[0]->v, view_of(sc.xa), g, grid_chunks, max_rows, sc.gu, s), "moe gate launch");
         const float* up_out = sc.gu + inter;
         size_t stride = 2 * inter;
@@ -155,9 +206,21 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
             HIP_TRY(launch_moe_act(sc.gu, up_out, stride, pairs, inter, m->act_kind, m->act_param, sc.a, s), "moe act launch");
             HIP_TRY(launch_quantize_act(sc.a, pairs, inter, sc.aq, s), "moe quantize launch");
         }
+        }
         g.rowmap = nullptr;
         g.bases = m->bases_dn;
+        g.direct_x0 = 0;
+        if (comb_fused) {
+            g.comb_y = y;
+            g.row_of = direct ? nullptr : sc.row_of;
+            g.route_w = route_w;
+            g.comb_t = (uint32_t)t;
+            g.comb_k = (uint32_t)k;
+            g.comb_add = add ? 1u : 0u;
+            g.comb_counters = sc.counters;
+        }
         HIP_TRY(launch_decode_mfma_grouped(m->down[0]->v, view_of(sc.aq), g, grid_chunks, max_rows, sc.o, s), "moe down launch");
+        if (comb_fused) return 1;
     }
     HIP_TRY(launch_moe_combine(sc.o, sc.row_of, route_w, t, k, h, y, s, add), "moe combine launch");
     return 1;
@@ -277,6 +340,20 @@ int oxhip_dev_experts(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, cons
     }
     HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
     return moe_run(c, m, x, t, sel, reinterpret_cast<const float*>(sel + t * k), k, y, static_cast<hipStream_t>(stream), add != 0);
+}
+
+int oxhip_dev_moe_routed(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const float* logits, size_t logit_stride, size_t k,
+                         const float* expert_scale, uint32_t* sel, float* y, int add, void* stream) {
+    if (!c || !m || !x || !logits || !sel || !y || !k || !t || k > 32 || k > m->n_exp || m->n_exp > 1024 || (logit_stride && logit_stride < m->n_exp)) {
+        set_error("moe_routed: bad arguments (k <= 32, k <= n_experts <= 1024)");
+        return 0;
+    }
+    HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
+    RouteIn rin;
+    rin.logits = logits;
+    rin.stride = logit_stride;
+    rin.expert_scale = expert_scale;
+    return moe_run(c, m, x, t, sel, reinterpret_cast<const float*>(sel + t * k), k, y, static_cast<hipStream_t>(stream), add != 0, rin);
 }
 
 int oxhip_moe_forward(oxhip_ctx* c, const float* x, size_t t, size_t h, size_t inter, const uint32_t* route_idx, const float* route_w,

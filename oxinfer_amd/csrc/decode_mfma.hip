@@ -38,6 +38,7 @@
 
 #include <hip/hip_ext.h>
 
+#include "act_body.hpp"
 #include "internal.hpp"
 #include "layout.hpp"
 
@@ -144,8 +145,11 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // known at run time costs some twenty instructions even when it is the same for the whole wave
     const uint32_t kwsh = (uint32_t)__builtin_ctz(kw), kssh = (uint32_t)__builtin_ctz(ksplit);
     const uint32_t r = wave >> kwsh, ks = wave & (kw - 1);
-    const uint32_t tile = bx * rt + r;
-    const uint32_t ntiles = row_tiles(w.n_out);
+    // (fused gate / up experts: the first rt / 2 tiles of the workgroup are gate tiles, the others the up tiles of the same rows)
+    const bool glu = GROUPED && grp.glu_inter != 0;
+    const uint32_t ghalf = rt >> 1, gtiles = grp.glu_inter / 16;
+    const uint32_t tile = !glu ? bx * rt + r : r < ghalf ? bx * ghalf + r : gtiles + bx * ghalf + (r - ghalf);
+    const uint32_t ntiles = glu && r < ghalf ? gtiles : row_tiles(w.n_out);
     // this workgroup's slice of K: steps [S0, S1), blocks [B0, B0 + nbl) (a multiple of 4 blocks)
     constexpr uint32_t BPS = q8_format(FMT) ? 2 : 4;  // blocks of 32 per step
     const uint32_t nsteps = q8_format(FMT)    ? t8_steps(w.n_in)
@@ -164,14 +168,24 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     float* red = ALDS ? lds_all : lds + (size_t)NARR * as;  // [rt * kw][NG][TPAD][16]
     uint32_t row0 = 0;  // first activation / output row of this launch unit
     if (GROUPED) {
-        if (by >= (uint32_t)*grp.nchunks) return;  // uniform over the workgroup
-        const int4 ch = grp.chunks[by];
-        w.p0 = grp.bases[ch.x];
-        row0 = (uint32_t)ch.y;
-        t = (uint32_t)ch.z;
+        if (grp.direct) {
+            if (by >= grp.direct_n) return;  // uniform over the workgroup
+            w.p0 = grp.bases[grp.direct[by]];
+            row0 = by;
+            t = 1;
+        } else {
+            if (by >= (uint32_t)*grp.nchunks) return;  // uniform over the workgroup
+            const int4 ch = grp.chunks[by];
+            w.p0 = grp.bases[ch.x];
+            row0 = (uint32_t)ch.y;
+            t = (uint32_t)ch.z;
+        }
         y += (size_t)row0 * w.n_out;
     }
-    auto src_row = [&](uint32_t i) -> size_t { return GROUPED && grp.rowmap ? (size_t)grp.rowmap[row0 + i] : (size_t)row0 + i; };
+    auto src_row = [&](uint32_t i) -> size_t {
+        if (GROUPED && grp.direct && grp.direct_x0) return 0;
+        return GROUPED && grp.rowmap ? (size_t)grp.rowmap[row0 + i] : (size_t)row0 + i;
+    };
 
     // A role: slot n of this lane = (half, token); tokens past t read token t - 1 (their sums are dropped)
     const uint32_t a_half = n >> 3, a_tok = min(n & 7u, t - 1);
@@ -648,6 +662,75 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         else if (epi.mode == EPI_ADD) *dst = *dst + v;
         else *dst = *dst + (1.0f / (1.0f + expf(-epi.gate[tok]))) * v;
     };
+    if constexpr (GROUPED && !DUMP) {
+        if (glu) {
+            // a [token][rt / 2 * 16 rows of inter] = act(gate) * up behind the partial sums in LDS, then one lane per (token,
+            // block of 32) quantizes its block exactly as quantize_act does (sequential sums in element order)
+            float* aval = red + (size_t)rt * kw * NG * TPAD * 16;  // [NG * TPAD][ghalf * 16]
+            const uint32_t cols = ghalf * 16;
+            for (uint32_t idx = threadIdx.x; idx < ghalf * NG * TPAD * 16; idx += nthr) {
+                const uint32_t rr = idx / (NG * TPAD * 16), gt = (idx / 16) % (NG * TPAD), nn = idx % 16;
+                const uint32_t g = gt / TPAD, tl = gt % TPAD;
+                float gs = 0.0f, us = 0.0f;
+                for (uint32_t k = 0; k < kw; k++) {
+                    gs += red[((((size_t)rr * kw + k) * NG + g) * TPAD + tl) * 16 + nn];
+                    us += red[((((size_t)(ghalf + rr) * kw + k) * NG + g) * TPAD + tl) * 16 + nn];
+                }
+                aval[(size_t)gt * cols + rr * 16 + nn] = gated_act(gs, us, grp.act_kind, grp.act_param);
+            }
+            __syncthreads();
+            // quantize_act's arithmetic (act_body.hpp) with 32 lanes per block: the maximum, the codes and the integer sums do
+            // not depend on the order; the f32 sums do, and lane 0 (block and first half) and lane 16 (second half) of a block
+            // form them one element after the other as the reference does. (A lone lane walking the whole block is a
+            // microsecond and a half of dependent instructions at the end of every workgroup.)
+            const uint32_t bpw = cols / 32, bpr = grp.glu_inter / 32;  // blocks of the workgroup; blocks of a row
+            for (uint32_t idx = threadIdx.x; idx < NG * TPAD * bpw * 32; idx += nthr) {
+                const uint32_t e = idx & 31, u = idx >> 5, gt = u / bpw, bl = u % bpw, tok = 8 * (gt / TPAD) + gt % TPAD;
+                const uint32_t blk = bx * bpw + bl;
+                const bool live = tok < t && blk < bpr;  // uniform over the 32 lanes of a block
+                const float* src = aval + (size_t)gt * cols + bl * 32;
+                const float v = src[e];
+                float amax = fabsf(v);
+#pragma unroll
+                for (int off = 16; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+                const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+                const float rr = roundf(v * inv);  // half away from zero
+                const int iv = rr != rr ? 0 : (int)fminf(fmaxf(rr, -128.0f), 127.0f);
+                int s16 = iv;  // the integer sum of the lane's half of the block
+#pragma unroll
+                for (int off = 8; off >= 1; off >>= 1) s16 += __shfl_xor(s16, off);
+                const int s_other = __shfl_xor(s16, 16);
+                float fsum = -0.0f, h0 = -0.0f;  // Rust's iter().sum() starts from -0.0
+                if ((e & 15) == 0) {
+                    if (e == 0) {
+#pragma unroll
+                        for (int i = 0; i < 16; i++) fsum += src[i];
+                        h0 = fsum;
+#pragma unroll
+                        for (int i = 16; i < 32; i++) fsum += src[i];
+                    } else {
+#pragma unroll
+                        for (int i = 16; i < 32; i++) h0 += src[i];
+                    }
+                }
+                if (!live) continue;
+                const size_t gb = (size_t)(row0 + tok) * bpr + blk;
+                grp.aq_q[gb * 32 + e] = (int8_t)iv;
+                if (e == 0) {
+                    grp.aq_scales[gb] = amax / 127.0f;
+                    grp.aq_sums[gb] = s16 + s_other;
+                    grp.aq_fsums[gb] = fsum;
+                    grp.aq_hsums[2 * gb] = h0;
+                    grp.aq_sums16[2 * gb] = s16;
+                } else if (e == 16) {
+                    grp.aq_hsums[2 * gb + 1] = h0;
+                    grp.aq_sums16[2 * gb + 1] = s16;
+                }
+            }
+            return;
+        }
+    }
+    const bool combine = GROUPED && grp.comb_y != nullptr;
     // the waves of a tile in order; with one slice that is the result, else this slice's partial rows
     float* out = ksplit > 1 ? partial + (size_t)slice * t * w.n_out : y;
     for (uint32_t idx = threadIdx.x; idx < rt * NG * TPAD * 16; idx += nthr) {
@@ -657,10 +740,47 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         float sum = 0.0f;
         for (uint32_t k = 0; k < kw; k++) sum += red[((((size_t)rr * kw + k) * NG + g) * TPAD + (idx / 16) % TPAD) * 16 + nn];
         // partial rows go out as device-scope stores (written through to memory, where the other XCDs' L2s see them)
-        if (ksplit > 1) __hip_atomic_store(out + (size_t)tok * w.n_out + row, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (ksplit > 1 || combine) __hip_atomic_store(out + (size_t)tok * w.n_out + row, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else emit(out + (size_t)tok * w.n_out + row, sum, tok);
     }
-    if (GROUPED || ksplit == 1 || !y) return;  // uniform over the workgroup
+    if constexpr (GROUPED) {
+        if (!combine) return;
+        // The chunks of a row group meet like K slices do (below): the last workgroup to arrive, of all the launch's chunks,
+        // adds every token's routed rows in route order (multiply, then add: src/moe.rs:608-615).
+        __shared__ uint32_t last_chunk;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const uint32_t total = grp.direct ? grp.direct_n : (uint32_t)*grp.nchunks;
+            const uint32_t seen = __hip_atomic_fetch_add(&grp.comb_counters[(size_t)bx * CTR_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_chunk = seen == total - 1;
+            if (seen == total - 1) __hip_atomic_store(&grp.comb_counters[(size_t)bx * CTR_STRIDE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!last_chunk) return;
+        const float* o = y - (size_t)row0 * w.n_out;  // the gathered rows from row 0
+        for (uint32_t idx = threadIdx.x; idx < rt * 16 * grp.comb_t; idx += nthr) {
+            const uint32_t tok = idx / (rt * 16), row = bx * rt * 16 + idx % (rt * 16);
+            if (row >= w.n_out) continue;
+            float acc_y = grp.comb_add ? grp.comb_y[(size_t)tok * w.n_out + row] : 0.0f;
+            for (uint32_t j0 = 0; j0 < grp.comb_k; j0 += 4) {  // four routes per round trip, added in route order
+                float v[4], wt[4];
+#pragma unroll
+                for (uint32_t i = 0; i < 4; i++) {
+                    const uint32_t j = min(j0 + i, grp.comb_k - 1);
+                    const int rw = grp.row_of ? grp.row_of[(size_t)tok * grp.comb_k + j] : (int)j;
+                    wt[i] = grp.route_w[(size_t)tok * grp.comb_k + j];
+                    v[i] = __hip_atomic_load(o + (size_t)rw * w.n_out + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (uint32_t i = 0; i < 4; i++)
+                    if (j0 + i < grp.comb_k) acc_y = acc_y + wt[i] * v[i];
+            }
+            grp.comb_y[(size_t)tok * w.n_out + row] = acc_y;
+        }
+        return;
+    }
+    if (ksplit == 1 || !y) return;  // uniform over the workgroup
     // The last workgroup of this row group to get here adds the slices in slice order; the counter returns to zero
     // for the next launch. Every access to the partial rows and the counter is a device-scope atomic access, and each
     // thread waits for its stores to complete before the workgroup's arrival is counted, so no cache-wide write-back
@@ -962,7 +1082,15 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
     const uint32_t ng = max_rows <= 8 ? 1 : (max_rows <= 16 ? 2 : 4);
     if (max_rows > 32) return hipErrorInvalidValue;
     bool alds;
-    const size_t lds = lds_bytes(FMT, false, nsteps, tpad, sh, &alds, ng);
+    size_t lds = lds_bytes(FMT, false, nsteps, tpad, sh, &alds, ng);
+    if (g.glu_inter) {
+        // gate and up tiles in pairs, whole blocks of 32 rows per workgroup; act(gate) * up sits behind the partial sums
+        if (sh.rt % 4 || g.glu_inter % 32 || w.n_out != 2 * g.glu_inter) return hipErrorInvalidValue;
+        grid.x = (g.glu_inter / 16 + sh.rt / 2 - 1) / (sh.rt / 2);
+        const size_t red = (size_t)sh.rt * sh.kw * ng * tpad * 16 * 4, aval = (size_t)ng * tpad * (sh.rt / 2) * 16 * 4;
+        if (alds) lds = std::max(lds, red + aval);
+        else lds += aval;
+    }
     if (lds > LDS_MAX || (ng > 1 && !alds)) return hipErrorInvalidValue;
     const DecodeScratch none{};
     if (max_rows == 1) return launch_one<FMT, 1, false, true>(alds, grid, block, lds, s, w, xa, 0u, sh, y, nullptr, g, none);
@@ -1092,6 +1220,16 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     }
     if (!ride && ev_stop) return hipEventRecord(ev_stop, s);
     return hipSuccess;
+}
+
+// Whether the grouped launch of fused gate / up experts can pair its gate and up tiles per workgroup (and so apply the
+// activation and the quantization itself): its shape gives a workgroup a multiple of four row tiles.
+bool decode_grouped_glu_ok(const WeightView& w, size_t inter) {
+    if (!mfma_decode_format(w.fmt) || w.fmt == FMT_Q6_K || inter % 32 || w.n_out != 2 * inter) return false;
+    const uint32_t nsteps = steps_rt(w);
+    uint32_t gkw = 1;
+    while (gkw < 8 && nsteps / (gkw * 2) >= 16) gkw *= 2;
+    return (8 / gkw) % 4 == 0;
 }
 
 // Whether a grouped launch with chunks of up to max_rows rows fits this weight's staged activations into LDS.

@@ -70,6 +70,32 @@ struct GroupView {
     const int4* chunks;
     const int* nchunks;           // device scalar: chunks in use (the grid covers the worst case)
     const int* rowmap;            // optional: activation row of each gathered row
+    // Fused gate / up experts ([2 inter, n_in]: gate rows, then up rows), glu_inter = inter != 0: a workgroup's row tiles
+    // are rt / 2 gate tiles and the up tiles of the same rows; instead of the products it writes act(gate) * up, quantized
+    // as quantize_act quantizes it, into the QAct `aq` ([gathered rows][inter]) -- the input of the down projection.
+    uint32_t glu_inter = 0;
+    uint32_t act_kind = 0;
+    float act_param = 0.0f;
+    int8_t* aq_q = nullptr;
+    float* aq_scales = nullptr;
+    int32_t* aq_sums = nullptr;
+    float* aq_fsums = nullptr;
+    float* aq_hsums = nullptr;
+    int32_t* aq_sums16 = nullptr;
+    // The down projection with the combination inside (comb_y != nullptr): the products go to the gathered rows `y` as
+    // always; the last workgroup of a row group to finish (arrival counter per row group, zero between launches) then
+    // adds them into comb_y [comb_t, n_out] in route order: comb_y[i] (+)= sum_j route_w[i k + j] * y[row_of[i k + j]].
+    float* comb_y = nullptr;
+    const int* row_of = nullptr;
+    const float* route_w = nullptr;
+    uint32_t comb_t = 0, comb_k = 0;
+    uint32_t comb_add = 1;
+    uint32_t* comb_counters = nullptr;
+    // A one-token pass needs no plan: with direct != nullptr chunk c is {expert direct[c], gathered row c, one row} for
+    // c < direct_n, every gathered row of the gate / up launch reads token 0 (direct_x0), and route j's row is row j.
+    const uint32_t* direct = nullptr;
+    uint32_t direct_n = 0;
+    uint32_t direct_x0 = 0;
 };
 
 // Launchers (each returns hipSuccess or the launch error).
@@ -125,7 +151,8 @@ hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t,
                               hipEvent_t ev_start = nullptr, hipEvent_t ev_stop = nullptr, const Epi& epi = Epi{});
 hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks,
                                       uint32_t max_rows_per_chunk, float* y, hipStream_t s);
-bool decode_grouped_fits(const WeightView& w, uint32_t max_rows_per_chunk);  // LDS holds a chunk's staged activations
+bool decode_grouped_fits(const WeightView& w, uint32_t max_rows_per_chunk);
+bool decode_grouped_glu_ok(const WeightView& w, size_t inter);  // the grouped launch can apply act(gate) * up and quantize it itself  // LDS holds a chunk's staged activations
 hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* out, hipStream_t s);
 hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t n_in, const WeightView& dst, hipStream_t s);
 // off == nullptr: `sc` holds one scale per 32 (Q4_0) and the record keeps all four of a row's step
@@ -160,6 +187,10 @@ hipError_t launch_gemm_fp8(const WeightView& w, const void* apk, const float* sx
                            float* partial, hipStream_t s);
 hipError_t launch_route_top_k(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, hipStream_t s, size_t stride = 0,
                               const float* expert_scale = nullptr);
+// route_top_k of t rows of logits and quantize_act of x [t][h] in one launch (the two are independent and each is a few
+// microseconds of latency); n <= 256.
+hipError_t launch_route_quantize(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, size_t stride,
+                                 const float* expert_scale, const float* x, size_t h, const oxhip_qact& o, hipStream_t s);
 hipError_t launch_moe_plan(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, uint32_t chunk_rows, int* row_of, int* src,
                            int4* chunks, int* nchunks, hipStream_t s);
 hipError_t launch_moe_front(const uint32_t* route_idx, size_t pairs, size_t k, size_t n_exp, uint32_t chunk_rows, int* row_of, int* src,

@@ -21,10 +21,10 @@ __device__ __forceinline__ int order_key(float v) {
 // NW waves per token. A lone wave issues an instruction every five to eight cycles, so the counting loop is split
 // over the waves (each broadcasts 64 / NW lanes of every register) and the counts meet in LDS; wave 0 finishes.
 template <int PER, int NW>
-__global__ __launch_bounds__(64 * NW) void route_top_k_kernel(const float* __restrict__ logits, uint32_t stride, uint32_t n, uint32_t k,
-                                                              uint32_t* __restrict__ idx, float* __restrict__ wts,
-                                                              const float* __restrict__ expert_scale) {
-    const uint32_t tok = blockIdx.x, lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+__device__ __forceinline__ void route_top_k_body(const float* __restrict__ logits, uint32_t stride, uint32_t n, uint32_t k,
+                                                 uint32_t* __restrict__ idx, float* __restrict__ wts,
+                                                 const float* __restrict__ expert_scale, uint32_t tok) {
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const float* l = logits + (size_t)tok * stride;
     int key[PER];
     bool live[PER];
@@ -122,6 +122,45 @@ __global__ __launch_bounds__(64 * NW) void route_top_k_kernel(const float* __res
         // (per-expert factors multiply the weights after the softmax, src/gpu_decode.rs:167-168)
         wts[(size_t)tok * k + lane] = expert_scale ? e / sum * expert_scale[myidx] : e / sum;
     }
+}
+
+template <int PER, int NW>
+__global__ __launch_bounds__(64 * NW) void route_top_k_kernel(const float* __restrict__ logits, uint32_t stride, uint32_t n, uint32_t k,
+                                                              uint32_t* __restrict__ idx, float* __restrict__ wts,
+                                                              const float* __restrict__ expert_scale) {
+    route_top_k_body<PER, NW>(logits, stride, n, k, idx, wts, expert_scale, blockIdx.x);
+}
+
+// Workgroups 0 .. t - 1 route a token each; the others quantize one block of 32 of x per lane.
+template <int PER>
+__global__ __launch_bounds__(512) void route_quantize_kernel(const float* __restrict__ logits, uint32_t stride, uint32_t n, uint32_t k,
+                                                             uint32_t* __restrict__ idx, float* __restrict__ wts,
+                                                             const float* __restrict__ expert_scale, uint32_t t, const float* __restrict__ x,
+                                                             size_t nblocks, int8_t* __restrict__ q, float* __restrict__ scales,
+                                                             int32_t* __restrict__ sums, float* __restrict__ fsums, float* __restrict__ hsums,
+                                                             int32_t* __restrict__ sums16) {
+    if (blockIdx.x < t) {
+        route_top_k_body<PER, 8>(logits, stride, n, k, idx, wts, expert_scale, blockIdx.x);
+        return;
+    }
+    const size_t b = (size_t)(blockIdx.x - t) * blockDim.x + threadIdx.x;
+    if (b < nblocks) quantize_act_block(x, b, q, scales, sums, fsums, hsums, sums16);
+}
+
+hipError_t launch_route_quantize(const float* logits, size_t t, size_t n, size_t k, uint32_t* idx, float* w, size_t stride,
+                                 const float* expert_scale, const float* x, size_t h, const oxhip_qact& o, hipStream_t s) {
+    if (!t) return hipSuccess;
+    if (n > 256) return hipErrorInvalidValue;
+    const uint32_t st = (uint32_t)(stride ? stride : n);
+    const size_t nblocks = t * h / 32;
+    const unsigned grid = (unsigned)(t + (nblocks + 511) / 512);
+    if (n <= 128)
+        route_quantize_kernel<2><<<grid, 512, 0, s>>>(logits, st, (uint32_t)n, (uint32_t)k, idx, w, expert_scale, (uint32_t)t, x, nblocks, o.q, o.scales,
+                                                     o.sums, o.fsums, o.hsums, o.sums16);
+    else
+        route_quantize_kernel<4><<<grid, 512, 0, s>>>(logits, st, (uint32_t)n, (uint32_t)k, idx, w, expert_scale, (uint32_t)t, x, nblocks, o.q, o.scales,
+                                                     o.sums, o.fsums, o.hsums, o.sums16);
+    return hipGetLastError();
 }
 
 // `stride`: floats between the logit rows of consecutive tokens (>= n; the decode graph keeps one more logit behind them).

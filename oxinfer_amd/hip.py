@@ -108,6 +108,7 @@ def load_library():
         "oxhip_dev_glu": (C.c_int, [vp, vp, vp, sz, C.c_int, vp, vp]),
         "oxhip_dev_route": (C.c_int, [vp, vp, vp, vp, sz, sz, sz, sz, vp, vp, vp, vp]),
         "oxhip_dev_experts": (C.c_int, [vp, vp, vp, sz, vp, sz, vp, C.c_int, vp]),
+        "oxhip_dev_moe_routed": (C.c_int, [vp, vp, vp, sz, vp, sz, sz, vp, vp, vp, C.c_int, vp]),
         "oxhip_event_create": (vp, []),
         "oxhip_event_destroy": (None, [vp]),
         "oxhip_event_elapsed_ms": (C.c_float, [vp, vp]),
@@ -432,6 +433,19 @@ class HipBackend:
         """Op::Experts: the experts chosen in `sel` (as route() returns it) over x [t, h]; y += or y =."""
         _, t, k = sel.shape
         return bool(self.lib.oxhip_dev_experts(self.ctx, dev.handle, x.data_ptr(), t, sel.data_ptr(), k, y.data_ptr(), int(add), self._stream()))
+
+    def moe_routed(self, dev, x, logits, k, y, sel=None, add=True, expert_scale=None):
+        """Top-k of `logits` [t, n_exp (+...)] and the routed experts over x [t, h] in one call; returns sel [2, t, k]."""
+        import torch
+        t = x.shape[0]
+        if sel is None:
+            sel = torch.empty((2, t, k), dtype=torch.int32, device=x.device)
+        ok = self.lib.oxhip_dev_moe_routed(self.ctx, dev.handle, x.data_ptr(), t, logits.data_ptr(), logits.shape[1], k,
+                                           expert_scale.data_ptr() if expert_scale is not None else None, sel.data_ptr(), y.data_ptr(),
+                                           int(add), self._stream())
+        if not ok:
+            raise RuntimeError(self.last_error())
+        return sel
 
     def decode_jobs(self, jobs):
         """Builds a reusable job array for decode_batch: jobs = [(DeviceWeight, QAct | None, x | None, t, y, ev0, ev1)]."""

@@ -258,6 +258,11 @@ def test_moe_config_128_experts(be, oxref, config_experts):
         y = torch.zeros((t, h), dtype=torch.float32, device="cuda")
         be.dev_moe(dev, torch.from_numpy(x).cuda(), idx_d, w_d, y)
         y = y.cpu().numpy()
+        # routing inside the pass (one call: top-k of the logits, then the experts): the same routes and the same rows
+        y2 = torch.zeros((t, h), dtype=torch.float32, device="cuda")
+        sel = be.moe_routed(dev, torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda(), k, y2).cpu().numpy()
+        assert np.array_equal(sel[0].view(np.uint32), idx) and np.array_equal(sel[1].view(np.float32).view(np.uint32), w.view(np.uint32))
+        assert np.array_equal(y2.cpu().numpy().view(np.uint32), y.view(np.uint32))
         sample = np.arange(t) if t == 1 else np.r_[0:3, 100:103, 253:256, np.random.default_rng(5).integers(0, t, 7)]
         xs, si, sw = np.ascontiguousarray(x[sample]), np.ascontiguousarray(idx[sample]), np.ascontiguousarray(w[sample])
         y0 = np.zeros((len(sample), h), np.float32)
