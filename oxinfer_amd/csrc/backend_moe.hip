@@ -175,8 +175,11 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
         // fused gate / up experts whose launch pairs gate and up tiles: the activation and the quantization of its output
         // are the launch's own output stage; the down launch then also combines (the last workgroup of a row group to
         // finish adds the routed rows in route order): three launches for a decode-sized pass
-        const bool glu_fused = fused && decode_grouped_glu_ok(m->gate_up[0]->v, inter);
-        const bool comb_fused = row_tiles((uint32_t)h) <= COMB_GROUPS;
+        // (decode-sized passes only: a large pass has enough rows to fill launches of their own, and its combination is
+        // too much work for the one workgroup per row group that would do it)
+        const bool small = t <= 8;
+        const bool glu_fused = small && fused && decode_grouped_glu_ok(m->gate_up[0]->v, inter);
+        const bool comb_fused = small && row_tiles((uint32_t)h) <= COMB_GROUPS;
         if (glu_fused) {
             GroupView gg = g;
             gg.glu_inter = (uint32_t)inter;

@@ -1061,6 +1061,17 @@ hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int3
     return hipSuccess;
 }
 
+// The workgroup of a grouped launch: rows are split over up to eight waves of 16 records or more (kw: a function of the
+// weight alone, since it fixes the order of a row's sum), and a workgroup takes as many row tiles as eight waves allow,
+// because every workgroup stages its chunk's activations. Decode-sized passes (chunks of at most 8 rows: little to stage,
+// few chunks) take at most four tiles: smaller workgroups spread a pass of 8 experts over more CUs (24.8 -> 23.0 us).
+Shape grouped_shape(uint32_t nsteps, uint32_t max_rows) {
+    uint32_t gkw = 1;
+    while (gkw < 8 && nsteps / (gkw * 2) >= 16) gkw *= 2;
+    const uint32_t rt = 8 / gkw;
+    return Shape{max_rows <= 8 && rt > 4 ? 4u : rt, gkw, 1};
+}
+
 template <int FMT>
 hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView& g, uint32_t max_chunks, uint32_t max_rows,
                        float* y, hipStream_t s) {
@@ -1068,9 +1079,7 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
     // grid y walks the chunks (no K slices across workgroups). Every workgroup stages its chunk's activations, so it
     // takes as many row tiles as 8 waves allow, each wave keeping 16 records or more where K is long enough. The shape depends on the
     // weight alone, so a token's row is bit-identical whatever else is in the group.
-    uint32_t gkw = 1;
-    while (gkw < 8 && nsteps / (gkw * 2) >= 16) gkw *= 2;
-    Shape sh{8 / gkw, gkw, 1};
+    Shape sh = grouped_shape(nsteps, max_rows);
 #ifdef OXHIP_TUNING  // tuning builds only: "rt,kw" in OXHIP_GROUPED_SHAPE
     if (const char* e = getenv("OXHIP_GROUPED_SHAPE")) {
         unsigned a = 0, b = 0;
@@ -1226,19 +1235,14 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
 // activation and the quantization itself): its shape gives a workgroup a multiple of four row tiles.
 bool decode_grouped_glu_ok(const WeightView& w, size_t inter) {
     if (!mfma_decode_format(w.fmt) || w.fmt == FMT_Q6_K || inter % 32 || w.n_out != 2 * inter) return false;
-    const uint32_t nsteps = steps_rt(w);
-    uint32_t gkw = 1;
-    while (gkw < 8 && nsteps / (gkw * 2) >= 16) gkw *= 2;
-    return (8 / gkw) % 4 == 0;
+    return grouped_shape(steps_rt(w), 8).rt % 4 == 0 && grouped_shape(steps_rt(w), 32).rt % 4 == 0;
 }
 
 // Whether a grouped launch with chunks of up to max_rows rows fits this weight's staged activations into LDS.
 bool decode_grouped_fits(const WeightView& w, uint32_t max_rows) {
     if (!mfma_decode_format(w.fmt) || max_rows < 1 || max_rows > 32) return false;
     const uint32_t nsteps = steps_rt(w);
-    uint32_t gkw = 1;
-    while (gkw < 8 && nsteps / (gkw * 2) >= 16) gkw *= 2;
-    const Shape sh{8 / gkw, gkw, 1};
+    const Shape sh = grouped_shape(nsteps, max_rows);
     const uint32_t ng = max_rows <= 8 ? 1 : (max_rows <= 16 ? 2 : 4);
     bool alds;
     const size_t lds = lds_bytes(w.fmt, false, nsteps, max_rows <= 4 ? 4 : 8, sh, &alds, ng);
