@@ -266,6 +266,16 @@ def bench_mlx_gemv(be, torch, synth, steps, warmup, pool_gb):
     wall, ms = run(single, 1)
     _, ms4 = run(four, 4)
     _, msh = run(hot, 1)
+    # a steady stream: 192 matmuls over rotating copies handed over in one call (shared launches of 16, back to back)
+    arr = be.decode_jobs([(ws[i % len(ws)], xa, None, 1, ys[i % 4], None, None) for i in range(192)])
+    be.decode_batch(arr)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    be.decode_batch(arr)
+    e1.record()
+    torch.cuda.synchronize()
+    us_stream = e0.elapsed_time(e1) * 1e3 / 192
     ach = nbytes / (ms * 1e-3) / 1e9
     line = dict(base_line(steps, warmup), value=round(nbytes * steps / wall / 1e9, 2), unit="GB/s", ms_per_step=round(wall / steps * 1e3, 5),
                 dtype="int8", config={"workload": "configs[0]: MLX 4-bit g64 GEMV 4096 -> 4096, T = 1", "bytes_per_step": nbytes,
@@ -276,6 +286,9 @@ def bench_mlx_gemv(be, torch, synth, steps, warmup, pool_gb):
     line["shared_launch_of_4"] = {"what": "a layer's four 4096 x 4096 matmuls (q, k, v, o) in one oxhip_dev_decode_batch launch, rotating copies (cold HBM)",
                                   "kernel": "decode_batch_kernel", "avg_launch_us": round(ms4 * 1e3, 2), "GBs": round(4 * nbytes / (ms4 * 1e-3) / 1e9, 1),
                                   "frac_hbm": round(4 * nbytes / (ms4 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    line["steady_stream"] = {"what": "192 matmuls over rotating copies in one call (launches of 16 back to back): what the kernel streams at without launch boundaries",
+                             "us_per_matmul": round(us_stream, 2), "GBs": round(nbytes / us_stream / 1e3, 1),
+                             "frac_hbm": round(nbytes / us_stream / 1e3 / HBM_PEAK_GBS, 4)}
     line["cache_resident"] = {"what": "the single launch on one weight copy (9.4 MB stays in the 256 MB Infinity Cache)",
                               "avg_launch_us": round(msh * 1e3, 2), "GBs": round(nbytes / (msh * 1e-3) / 1e9, 1)}
     return line
@@ -553,7 +566,7 @@ def summary(line, cpu):
     for k in ("ceiling",):
         if k in r:
             e[k] = r[k]
-    for k in ("shared_launch_of_4", "cache_resident", "tflops"):
+    for k in ("shared_launch_of_4", "steady_stream", "cache_resident", "tflops"):
         if k in line:
             e[k] = line[k]
     e["cpu_baseline"] = cpu
