@@ -41,7 +41,7 @@ enum {
 };
 
 /* GGUF type ids handled (src/ggml.rs:42-93). */
-enum { OXHIP_GGML_Q4_0 = 2, OXHIP_GGML_Q8_0 = 8, OXHIP_GGML_Q4_K = 12, OXHIP_GGML_Q6_K = 14, OXHIP_GGML_F8E4M3 = 0x1000 };
+enum { OXHIP_GGML_Q4_0 = 2, OXHIP_GGML_Q8_0 = 8, OXHIP_GGML_Q4_K = 12, OXHIP_GGML_Q5_K = 13, OXHIP_GGML_Q6_K = 14, OXHIP_GGML_F8E4M3 = 0x1000 };
 
 typedef struct {
     uint32_t kind;            /* OXHIP_W_* */
@@ -110,8 +110,8 @@ void oxhip_free_weight(oxhip_ctx* ctx, oxhip_weight* w);
 size_t oxhip_weight_bytes(const oxhip_weight* w);
 /* Backend::matmul (src/gpu.rs:160; src/cuda.rs:1428-1493): all jobs share x [t, n_in] (host f32);
  * computes every job or none. Routing as matmul_quant_multi_at's (src/kernels.rs:1731-1879): up to 8 tokens the
- * Q8 / Q8_0 / Q4_K / Q6_K / MLX 4-bit jobs share one launch of the int8 decode kernel (the CPU's decode semantics,
- * src/kernels.rs:1908-1928); more than 16 tokens over MLX 4-bit, Q8, Q8_0, Q4_K, Q6_K or FP8 (128-column blocks)
+ * Q8 / Q8_0 / Q4_K / Q5_K / Q6_K / MLX 4-bit jobs share one launch of the int8 decode kernel (the CPU's decode semantics,
+ * src/kernels.rs:1908-1928); more than 16 tokens over MLX 4-bit, Q8, Q8_0, Q4_K, Q5_K, Q6_K or FP8 (128-column blocks)
  * weights run the bf16 matrix-core GEMM; everything else runs the decode kernels over 16 tokens at a time. */
 int oxhip_matmul(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_job* jobs, size_t n_jobs);
 /* Backend::matvec_rows (src/gpu.rs:165): t in 1..=4. */
@@ -170,7 +170,7 @@ int oxhip_dev_decode(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa
                      void* stream);
 /* oxhip_dev_decode for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc); it has no counterpart in the reference. The same kernels and the same
- * bits as oxhip_dev_decode over the quantized formats of the matrix-core decode kernel (Q8, Q8_0, Q4_0, Q4_K, Q6_K,
+ * bits as oxhip_dev_decode over the quantized formats of the matrix-core decode kernel (Q8, Q8_0, Q4_0, Q4_K, Q5_K, Q6_K,
  * MLX 4-bit; 1 <= t <= 16), but the partial rows and arrival counters of shapes that slice K live in an array the
  * library holds statically on every GPU (4 MiB + 256 KiB, kept until the process ends), and the call allocates and
  * frees nothing on the device. Declined (0, nothing written) when the weight needs more than that: K slices x 8 x
@@ -179,7 +179,7 @@ int oxhip_dev_decode(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa
 int oxhip_dev_decode_noalloc(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa, size_t t, float* y, void* stream);
 /* Several independent decode matmuls in one call (a decode step issues many small matmuls; what
  * matmul_quant_batch does for the CPU, src/kernels.rs:1937-1994). The jobs must not depend on one another: runs of
- * consecutive jobs of at most 8 tokens over Q8 / Q8_0 / Q4_K / Q6_K / MLX 4-bit weights share ONE launch (their latency chains
+ * consecutive jobs of at most 8 tokens over Q8 / Q8_0 / Q4_K / Q5_K / Q6_K / MLX 4-bit weights share ONE launch (their latency chains
  * overlap; every job's rows are bit-identical to a launch of its own), the others launch one by one, in order, on
  * `stream` (inside a shared launch the library orders the jobs itself). ev_start / ev_stop (from oxhip_event_create, or
  * NULL) are recorded before / after the launch that holds the job; for jobs that share a launch the first start and the
@@ -205,7 +205,7 @@ float oxhip_event_elapsed_ms(void* start, void* stop);
 /* Prefill: y [t, n_out] = x [t, n_in] W^T on the matrix cores (what matmul_quant_multi's GEMM paths compute,
  * src/kernels.rs:1774-1847). x_dtype / y_dtype: OXHIP_F32 or OXHIP_BF16. variant:
  *   OXHIP_GEMM_BF16  weights dequantized to bf16 (through LDS), bf16 MFMA, f32 accumulation (the x86 CPU's
- *                    f32 GEMM rounded to bf16 operands); MLX 4-bit, Q8, Q8_0, Q4_K and Q6_K weights (the rows
+ *                    f32 GEMM rounded to bf16 operands); MLX 4-bit, Q8, Q8_0, Q4_K, Q5_K and Q6_K weights (the rows
  *                    that dequantize_row yields, src/ggml.rs:630-793, rounded to bf16);
  *                    also FP8 weights whose rows are multiples of 128 (e4m3 x block scale rounded to bf16);
  *   OXHIP_GEMM_I8    MLX 4-bit weights on the int8 matrix cores: activations quantized per token and block of 32
@@ -290,7 +290,7 @@ int oxhip_dev_moe_routed(oxhip_ctx* ctx, oxhip_moe* m, const float* x, size_t t,
                          const float* expert_scale, uint32_t* sel, float* y, int add, void* stream);
 
 /* The exact integer accumulators of the decode kernels, written by the kernels themselves: per
- * block of 32 ([t, n_out, n_in/32]) for Q4, Q8, Q8_0 and Q4_K, per 16 ([t, n_out, n_in/16]) for Q6_K.
+ * block of 32 ([t, n_out, n_in/32]) for Q4, Q8, Q8_0, Q4_K and Q5_K, per 16 ([t, n_out, n_in/16]) for Q6_K.
  * For parity checks (the CPU's per-16 sums add up to the per-32 ones exactly). */
 int oxhip_dev_isums(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa, int32_t* out, void* stream);
 

@@ -9,7 +9,7 @@ namespace oxhip {
 int gemm_bf16_run(DevBuf& ws, const oxhip_weight* w, const void* x, bool x_bf16, size_t t, void* y, bool y_bf16, hipStream_t s) {
     const bool fp8 = w->v.fmt == FMT_FP8;
     if (!gemm_bf16_ok(w->v)) {
-        set_error("gemm: the bf16 variant runs MLX 4-bit, Q8, Q8_0, Q4_K and Q6_K weights and FP8 weights whose rows are multiples of 128");
+        set_error("gemm: the bf16 variant runs MLX 4-bit, Q8, Q8_0, Q4_K, Q5_K and Q6_K weights and FP8 weights whose rows are multiples of 128");
         return 0;
     }
     if (fp8 && skinny_fp8_ok(w->v, t)) {  // up to 32 tokens: bandwidth-bound, one pass over the weights

@@ -98,6 +98,12 @@ struct Step<FMT_Q4_K> {
     uint32_t a[4];
 };
 template <>
+struct Step<FMT_Q5_K> {
+    uint4 w;
+    uint32_t h;  // the fifth bits of the lane's 32 codes
+    uint32_t a[4];
+};
+template <>
 struct Step<FMT_Q4M> {
     uint4 w;
     uint32_t a[4];
@@ -134,7 +140,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // the swizzled operand array pays at 8 tokens (where the staging stores are many); at fewer its address math costs more
     constexpr bool SWZ = NT >= 8;
     constexpr int NI = NT < 4 ? NT : 4;          // accumulator registers that hold live tokens
-    constexpr bool MINS = FMT == FMT_Q4_K || FMT == FMT_Q4M;   // m * fs terms (Q4_0 has none)
+    constexpr bool MINS = k45_format(FMT) || FMT == FMT_Q4M;   // m * fs terms (Q4_0 has none)
     constexpr int NARR = q8_format(FMT) || FMT == FMT_Q40 ? 1 : FMT == FMT_Q6_K ? (DUMP ? 4 : 3) : 2;  // metadata arrays
     // the wave index and everything derived from it (tile, K range) live in scalar registers: branches on them are
     // scalar, and the load counters the compiler keeps stay exact across them
@@ -152,8 +158,9 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     const uint32_t ntiles = glu && r < ghalf ? gtiles : row_tiles(w.n_out);
     // this workgroup's slice of K: steps [S0, S1), blocks [B0, B0 + nbl) (a multiple of 4 blocks)
     constexpr uint32_t BPS = q8_format(FMT) ? 2 : 4;  // blocks of 32 per step
+    constexpr uint32_t K45_REC = FMT == FMT_Q5_K ? TK5_REC : TK4_REC;
     const uint32_t nsteps = q8_format(FMT)    ? t8_steps(w.n_in)
-                            : FMT == FMT_Q4_K ? 2 * tk4_sbs(w.n_in)
+                            : k45_format(FMT) ? 2 * tk4_sbs(w.n_in)
                             : FMT == FMT_Q6_K ? t6k_steps(w.n_in)
                                               : t4m_steps(w.n_in);
     const uint32_t slice = GROUPED ? 0 : by;
@@ -202,7 +209,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // (typed as global memory: a grouped launch reads w.p0 from the table of expert bases)
     const gbytes base = as_global(w.p0) + (size_t)min(tile, ntiles - 1) * (FMT == FMT_Q8_0   ? (size_t)nsteps * T8_REC
                                                                   : FMT == FMT_Q8F  ? (size_t)nsteps * T8F_REC
-                                                                  : FMT == FMT_Q4_K ? (size_t)(nsteps / 2) * TK4_REC
+                                                                  : k45_format(FMT) ? (size_t)(nsteps / 2) * K45_REC
                                                                   : FMT == FMT_Q6_K ? (size_t)nsteps * T6K_REC
                                                                                     : (size_t)nsteps * T4M_REC);
 
@@ -216,9 +223,10 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             const gbytes rec = base + (size_t)s * (FMT == FMT_Q8F ? T8F_REC : T8_REC);
             st.w = gload<uint4>(rec + 16 * lane);
             if (!ALDS) act2(2 * s + a_half, 8 * kq, st.a);
-        } else if constexpr (FMT == FMT_Q4_K) {
-            const gbytes rec = base + (size_t)(s >> 1) * TK4_REC;
+        } else if constexpr (k45_format(FMT)) {
+            const gbytes rec = base + (size_t)(s >> 1) * K45_REC;
             st.w = gload<uint4>(rec + (s & 1) * 1024 + 16 * lane);
+            if constexpr (FMT == FMT_Q5_K) st.h = gload<uint32_t>(rec + TK4_REC + (s & 1) * 256 + 4 * lane);
             if (!ALDS) {
                 act2(4 * s + a_half, 8 * kq, st.a);
                 act2(4 * s + 2 + a_half, 8 * kq, st.a + 2);
@@ -247,7 +255,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // kq asks for the words of step `first + kq` (row n of it), and at step first + q every lane takes them from lane
     // 16 q + n. Q8_0: {d of the two blocks}; Q4_K: {four sub-block scales, four mins, (d, dmin)}: this step's four
     // sub-blocks are 4 (s & 1) .. + 3 of the super-block; MLX: {d of the two groups, offsets of the two groups}.
-    constexpr int NM = FMT == FMT_Q8_0 ? 1 : (FMT == FMT_Q4_K || FMT == FMT_Q6_K) ? 3 : 2;  // (Q8F: the two f32 scales)
+    constexpr int NM = FMT == FMT_Q8_0 ? 1 : (k45_format(FMT) || FMT == FMT_Q6_K) ? 3 : 2;  // (Q8F: the two f32 scales)
     const uint32_t slast = max(s1, 1u) - 1;
     auto load_scales = [&](uint32_t* m, uint32_t first) {
         const uint32_t s = min(first + kq, slast);
@@ -256,8 +264,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             m[1] = gload<uint32_t>(base + (size_t)s * T8F_REC + 1028 + 8 * n);
         } else if constexpr (FMT == FMT_Q8_0) {
             m[0] = gload<uint32_t>(base + (size_t)s * T8_REC + 1024 + 4 * n);
-        } else if constexpr (FMT == FMT_Q4_K) {
-            const gbytes rec = base + (size_t)(s >> 1) * TK4_REC;
+        } else if constexpr (k45_format(FMT)) {
+            const gbytes rec = base + (size_t)(s >> 1) * K45_REC;
             m[0] = gload<uint32_t>(rec + 2048 + 16 * n + 4 * (s & 1));
             m[1] = gload<uint32_t>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
             m[2] = gload<uint32_t>(rec + 2304 + 4 * n);
@@ -338,20 +346,31 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                 for (int i = 0; i < NI; i++) acc[tg][i] = fmaf(d, xs[i] * (float)isum[i], acc[tg][i]);
                 dump_block(b, isum);
             }
-        } else if constexpr (FMT == FMT_Q4_K) {
+        } else if constexpr (k45_format(FMT)) {
             // sw[0]: the step's four sub-block scales, sw[1]: its four mins (bytes), sw[2]: (d, dmin). One byte permute
             // gathers this lane's four: the scales of its two blocks (sub-blocks d_half and 2 + d_half of the step) and,
             // for the mins' matrix instruction, the scale and min of sub-block kq.
             const float d = f16_bits_to_f32((uint16_t)(sw[2] & 0xFFFF)), dmin = f16_bits_to_f32((uint16_t)(sw[2] >> 16));
             const uint32_t pk = __builtin_amdgcn_perm(sw[1], sw[0], q4k_sel);
-            const float d16 = d * 0.0625f;
+            // Q5_K: the codes centre on 16 and go to the matrix cores as 8 (code - 16): the nibble in bits 3..6 of its
+            // byte, the inverted fifth bit on top
+            constexpr bool FIVE = FMT == FMT_Q5_K;
+            const float d16 = d * (FIVE ? 0.125f : 0.0625f);
             const float dsc[2] = {d16 * (float)(pk & 0xFF), d16 * (float)((pk >> 8) & 0xFF)};
-            // decode_i8's m of sub-block kq: 8 s - dmin * mn (src/ggml.rs:1046-1073)
-            const float mk = fmaf(8.0f * d, (float)((pk >> 16) & 0xFF), -(dmin * (float)(pk >> 24)));
+            // decode_i8's m of sub-block kq: 8 s - dmin * mn, 16 s for Q5_K (src/ggml.rs:1046-1073)
+            const float mk = fmaf((FIVE ? 16.0f : 8.0f) * d, (float)((pk >> 16) & 0xFF), -(dmin * (float)(pk >> 24)));
 #pragma unroll
             for (int pr = 0; pr < 2; pr++) {  // the two byte pairs of the lane's chunk
-                const uint32_t x0 = (pr ? c.z : c.x) ^ CENTRE, x1 = (pr ? c.w : c.y) ^ CENTRE;
-                v4i bw = {(int)((x0 << 4) & TOPN), (int)((x1 << 4) & TOPN), (int)(x0 & TOPN), (int)(x1 & TOPN)};
+                v4i bw;
+                if constexpr (FIVE) {
+                    constexpr uint32_t NIB = 0x78787878u, TOP = 0x80808080u;
+                    const uint32_t x0 = pr ? c.z : c.x, x1 = pr ? c.w : c.y, hb = ~st.h;
+                    bw = v4i{(int)(((x0 << 3) & NIB) | ((hb << (7 - 4 * pr)) & TOP)), (int)(((x1 << 3) & NIB) | ((hb << (6 - 4 * pr)) & TOP)),
+                             (int)(((x0 >> 1) & NIB) | ((hb << (5 - 4 * pr)) & TOP)), (int)(((x1 >> 1) & NIB) | ((hb << (4 - 4 * pr)) & TOP))};
+                } else {
+                    const uint32_t x0 = (pr ? c.z : c.x) ^ CENTRE, x1 = (pr ? c.w : c.y) ^ CENTRE;
+                    bw = v4i{(int)((x0 << 4) & TOPN), (int)((x1 << 4) & TOPN), (int)(x0 & TOPN), (int)(x1 & TOPN)};
+                }
                 const uint32_t b = 4 * s + 2 * pr + d_half;  // global index of this lane's block of 32
 #pragma unroll
                 for (int tg = 0; tg < NG; tg++) {
@@ -362,7 +381,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
 #pragma unroll
                     for (int i = 0; i < NI; i++) acc[tg][i] = fmaf(dsc[pr], xs[i] * (float)I[i], acc[tg][i]);
                     if (DUMP) {
-                        int isum[4] = {I[0] >> 4, I[1] >> 4, I[2] >> 4, I[3] >> 4};
+                        constexpr int SH = FIVE ? 3 : 4;
+                        int isum[4] = {I[0] >> SH, I[1] >> SH, I[2] >> SH, I[3] >> SH};
                         dump_block(b, isum);
                     }
                 }
@@ -862,6 +882,13 @@ __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid,
     else decode_body<FMT, 8, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi);
 }
 
+// FSET: the formats compiled in, one bit per Fmt. The compiler allocates registers over the whole kernel, so every
+// format in it costs the others (a seventh format made the three common GGUF ones 15 % slower): a launch takes the
+// smallest of the sets below that holds all its jobs' formats.
+constexpr uint32_t fbit(int f) { return 1u << f; }
+constexpr uint32_t FSET_GGUF = fbit(FMT_Q8_0) | fbit(FMT_Q4_K) | fbit(FMT_Q6_K), FSET_MLX = fbit(FMT_Q4M),
+                   FSET_ALL = FSET_GGUF | FSET_MLX | fbit(FMT_Q8F) | fbit(FMT_Q5_K) | fbit(FMT_Q40);
+template <uint32_t FSET>
 __global__ __launch_bounds__(1024) void decode_batch_kernel(BatchArgs a) {
     extern __shared__ __align__(16) float lds_dyn[];
     uint32_t j = 0;
@@ -869,12 +896,13 @@ __global__ __launch_bounds__(1024) void decode_batch_kernel(BatchArgs a) {
     const BatchJob& jb = a.j[j];
     const uint32_t bx = blockIdx.x - jb.wg0;
     switch (jb.w.fmt) {
-        case FMT_Q8_0: batch_dispatch<FMT_Q8_0>(jb, bx, lds_dyn); break;
-        case FMT_Q8F: batch_dispatch<FMT_Q8F>(jb, bx, lds_dyn); break;
-        case FMT_Q4_K: batch_dispatch<FMT_Q4_K>(jb, bx, lds_dyn); break;
-        case FMT_Q6_K: batch_dispatch<FMT_Q6_K>(jb, bx, lds_dyn); break;
-        case FMT_Q4M: batch_dispatch<FMT_Q4M>(jb, bx, lds_dyn); break;
-        case FMT_Q40: batch_dispatch<FMT_Q40>(jb, bx, lds_dyn); break;
+        case FMT_Q8_0: if constexpr (FSET & fbit(FMT_Q8_0)) batch_dispatch<FMT_Q8_0>(jb, bx, lds_dyn); break;
+        case FMT_Q8F: if constexpr (FSET & fbit(FMT_Q8F)) batch_dispatch<FMT_Q8F>(jb, bx, lds_dyn); break;
+        case FMT_Q4_K: if constexpr (FSET & fbit(FMT_Q4_K)) batch_dispatch<FMT_Q4_K>(jb, bx, lds_dyn); break;
+        case FMT_Q5_K: if constexpr (FSET & fbit(FMT_Q5_K)) batch_dispatch<FMT_Q5_K>(jb, bx, lds_dyn); break;
+        case FMT_Q6_K: if constexpr (FSET & fbit(FMT_Q6_K)) batch_dispatch<FMT_Q6_K>(jb, bx, lds_dyn); break;
+        case FMT_Q4M: if constexpr (FSET & fbit(FMT_Q4M)) batch_dispatch<FMT_Q4M>(jb, bx, lds_dyn); break;
+        case FMT_Q40: if constexpr (FSET & fbit(FMT_Q40)) batch_dispatch<FMT_Q40>(jb, bx, lds_dyn); break;
         default: break;
     }
 }
@@ -950,11 +978,11 @@ Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices, int fmt) {
     const uint32_t cols_per_step = q8_format(fmt) ? 64 : 128;
     // weight bytes per column of a row tile, as the restaging term of the cost sees them: the 8-bit records, and the
     // 4-bit ones for the 4- and 6-bit formats alike (the 6-bit records are larger but cost as many instructions more)
-    const double bytes_per_col = q8_format(fmt) ? (double)T8_REC / 64 : (double)TK4_REC / 256;
+    const double bytes_per_col = q8_format(fmt) ? (double)T8_REC / 64 : fmt == FMT_Q5_K ? (double)TK5_REC / 256 : (double)TK4_REC / 256;
     static std::mutex mu;
     static std::map<uint64_t, Shape> cache;
     // ntiles and nsteps are below 2^27 (n_out, n_in < 2^31): 27 + 27 + 8 bits of format + 1
-    static_assert(FMT_Q40 < 256, "the key keeps 8 bits of the format");
+    static_assert(FMT_Q5_K < 256, "the key keeps 8 bits of the format");
     const uint64_t key = ((uint64_t)ntiles << 36) | ((uint64_t)nsteps << 9) | ((uint64_t)(fmt & 0xFF) << 1) | (allow_slices ? 1u : 0u);
     std::lock_guard<std::mutex> g(mu);
     auto it = cache.find(key);
@@ -1009,7 +1037,7 @@ hipError_t launch_one(bool alds, dim3 grid, dim3 block, size_t lds, hipStream_t 
 
 template <int FMT>
 constexpr uint32_t steps_of(uint32_t n_in) {
-    return q8_format(FMT) ? t8_steps(n_in) : FMT == FMT_Q4_K ? 2 * tk4_sbs(n_in) : FMT == FMT_Q6_K ? t6k_steps(n_in) : t4m_steps(n_in);
+    return q8_format(FMT) ? t8_steps(n_in) : k45_format(FMT) ? 2 * tk4_sbs(n_in) : FMT == FMT_Q6_K ? t6k_steps(n_in) : t4m_steps(n_in);
 }
 
 template <int FMT, bool DUMP>
@@ -1114,7 +1142,7 @@ hipError_t run_grouped(const WeightView& w, const QActView& xa, const GroupView&
 namespace {
 uint32_t steps_rt(const WeightView& w) {
     return q8_format(w.fmt)    ? steps_of<FMT_Q8_0>(w.n_in)
-           : w.fmt == FMT_Q4_K ? steps_of<FMT_Q4_K>(w.n_in)
+           : k45_format(w.fmt) ? steps_of<FMT_Q4_K>(w.n_in)
            : w.fmt == FMT_Q6_K ? steps_of<FMT_Q6_K>(w.n_in)
                                : steps_of<FMT_Q4M>(w.n_in);
 }
@@ -1151,9 +1179,11 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     (void)hipGetDevice(&dev);
     const uint64_t bit = 1ull << (dev & 63);
     if (!(allowed[(dev >> 6) & 3].load(std::memory_order_acquire) & bit)) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(decode_batch_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)LDS_MAX);
-        if (e != hipSuccess) return e;
+        for (const void* k : {reinterpret_cast<const void*>(decode_batch_kernel<FSET_GGUF>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_MLX>),
+                              reinterpret_cast<const void*>(decode_batch_kernel<FSET_ALL>)}) {
+            hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
+            if (e != hipSuccess) return e;
+        }
         allowed[(dev >> 6) & 3].fetch_or(bit, std::memory_order_release);
     }
     std::vector<BatchArgs> launches;
@@ -1222,8 +1252,15 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     }
     for (size_t i = 0; i < launches.size(); i++) {
         if (!launches[i].nwg) continue;
-        if (ride) hipExtLaunchKernelGGL(decode_batch_kernel, dim3(launches[i].nwg), dim3(threadss[i]), (uint32_t)ldss[i], s, ev_start, ev_stop, 0, launches[i]);
-        else decode_batch_kernel<<<launches[i].nwg, threadss[i], ldss[i], s>>>(launches[i]);
+        uint32_t fset = 0;
+        for (uint32_t j = 0; j < launches[i].njobs; j++) fset |= fbit(launches[i].j[j].w.fmt);
+        auto go = [&](auto kern) {
+            if (ride) hipExtLaunchKernelGGL(kern, dim3(launches[i].nwg), dim3(threadss[i]), (uint32_t)ldss[i], s, ev_start, ev_stop, 0, launches[i]);
+            else kern<<<launches[i].nwg, threadss[i], ldss[i], s>>>(launches[i]);
+        };
+        if (!(fset & ~FSET_GGUF)) go(decode_batch_kernel<FSET_GGUF>);
+        else if (!(fset & ~FSET_MLX)) go(decode_batch_kernel<FSET_MLX>);
+        else go(decode_batch_kernel<FSET_ALL>);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -1267,6 +1304,7 @@ hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t,
         case FMT_Q8_0: return run<FMT_Q8_0, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
         case FMT_Q8F: return run<FMT_Q8F, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
         case FMT_Q4_K: return run<FMT_Q4_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
+        case FMT_Q5_K: return run<FMT_Q5_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
         case FMT_Q6_K: return run<FMT_Q6_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
         case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
         case FMT_Q40: return run<FMT_Q40, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
@@ -1280,6 +1318,7 @@ hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, 
         case FMT_Q8_0: return run<FMT_Q8_0, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q8F: return run<FMT_Q8F, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q4_K: return run<FMT_Q4_K, true>(w, xa, t, y, out, DecodeScratch{}, s);
+        case FMT_Q5_K: return run<FMT_Q5_K, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q6_K: return run<FMT_Q6_K, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q4M: return run<FMT_Q4M, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q40: return run<FMT_Q40, true>(w, xa, t, y, out, DecodeScratch{}, s);

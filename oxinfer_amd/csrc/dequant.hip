@@ -6,6 +6,7 @@
 //   Q4    ((nib - 8) as f32) * d + m                      src/quant.rs:586-606
 //   Q8_0  (q as f32) * d                                  src/ggml.rs:707-712
 //   Q4_K  (d * sc) * v - (dmin * mn), v the raw nibble    src/ggml.rs:750-773
+//   Q5_K  the same with v = nibble + 16 * fifth bit       src/ggml.rs:750-773
 //   Q6_K  (d * sc) * q, q = 6-bit code - 32               src/ggml.rs:774-793
 //   FP8   e4m3(byte) * block scale                        src/ggml.rs:282-293, :433-444
 //   MLX 4-bit -> Q4 + offsets                             src/quant.rs:518-563
@@ -46,12 +47,17 @@ __global__ __launch_bounds__(256) void dequantize_kernel(WeightView w, uint32_t 
             v = (float)(int8_t)rec[16 * (kq * 16 + nn) + 8 * h + j] * d;
             break;
         }
-        case FMT_Q4_K: {
+        case FMT_Q4_K:
+        case FMT_Q5_K: {
             uint32_t tile = r >> 4, nn = r & 15, sb = c / 256, e = c % 256, pair = e / 64, hi = (e % 64) / 32, l = e % 32;
             uint32_t st = pair >> 1, jj = pair & 1, kq = l >> 3;
-            const uint8_t* rec = w.p0 + ((size_t)tile * tk4_sbs(n) + sb) * TK4_REC;
+            const uint8_t* rec = w.p0 + ((size_t)tile * tk4_sbs(n) + sb) * (w.fmt == FMT_Q5_K ? TK5_REC : TK4_REC);
             uint8_t byte = rec[st * 1024 + 16 * (kq * 16 + nn) + 8 * jj + (l & 7)];
             uint32_t q = hi ? (byte >> 4) : (byte & 0xF);
+            if (w.fmt == FMT_Q5_K) {  // the fifth bit adds 16 (src/ggml.rs:765-768)
+                const uint32_t hb = *reinterpret_cast<const uint32_t*>(rec + TK4_REC + 256 * st + 4 * (kq * 16 + nn));
+                q += 16 * ((hb >> (8 * (l & 3) + 4 * jj + 2 * hi + ((l & 7) >> 2))) & 1);
+            }
             uint32_t sc = rec[2048 + 16 * nn + 2 * pair + hi], mn = rec[2048 + 16 * nn + 8 + 2 * pair + hi];
             float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(rec + 2304 + 4 * nn));
             float dmin = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(rec + 2304 + 4 * nn + 2));
@@ -138,7 +144,10 @@ __global__ __launch_bounds__(256) void pack_t8_kernel(const uint8_t* __restrict_
     if (kq == 0) *reinterpret_cast<uint32_t*>(rec + 1024 + 4 * nn) = d[0] | ((uint32_t)d[1] << 16);
 }
 
+// FIVE: Q5_K blocks (d, dmin, scales[12], qh[32], qs[128]: src/ggml.rs:753-757) into TK5 records
+template <bool FIVE>
 __global__ __launch_bounds__(256) void pack_tk4_kernel(const uint8_t* __restrict__ raw, uint32_t n_out, uint32_t n_in, uint8_t* __restrict__ dst) {
+    constexpr uint32_t REC = FIVE ? TK5_REC : TK4_REC, BLK = FIVE ? 176 : 144, QS = FIVE ? 48 : 16;
     const uint32_t nsb = tk4_sbs(n_in);
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     size_t total = (size_t)row_tiles(n_out) * nsb * 128;  // two steps of 64 chunks per super-block
@@ -148,13 +157,22 @@ __global__ __launch_bounds__(256) void pack_tk4_kernel(const uint8_t* __restrict
     uint32_t sb = tsb % nsb;
     size_t tile = tsb / nsb;
     size_t row = tile * 16 + nn;
-    uint8_t* rec = dst + tsb * TK4_REC;
-    const uint8_t* src = raw + (row * nsb + sb) * 144;
+    uint8_t* rec = dst + tsb * REC;
+    const uint8_t* src = raw + (row * nsb + sb) * BLK;
     uint32_t out[4] = {0, 0, 0, 0};
     if (row < n_out)
         for (uint32_t jj = 0; jj < 2; jj++)
-            for (int j = 0; j < 8; j++) out[2 * jj + j / 4] |= (uint32_t)src[16 + 32 * (2 * st + jj) + 8 * kq + j] << (8 * (j & 3));
+            for (int j = 0; j < 8; j++) out[2 * jj + j / 4] |= (uint32_t)src[QS + 32 * (2 * st + jj) + 8 * kq + j] << (8 * (j & 3));
     *reinterpret_cast<uint4*>(rec + st * 1024 + 16 * l) = make_uint4(out[0], out[1], out[2], out[3]);
+    if (FIVE) {  // qh[l'] bit 2 j' + h: the fifth bit of element l' of sub-block 2 j' + h (j' = 2 st + jj)
+        uint32_t hb = 0;
+        if (row < n_out)
+            for (uint32_t jj = 0; jj < 2; jj++)
+                for (uint32_t hi = 0; hi < 2; hi++)
+                    for (uint32_t j = 0; j < 8; j++)
+                        hb |= (((uint32_t)src[16 + 8 * kq + j] >> (2 * (2 * st + jj) + hi)) & 1u) << (8 * (j & 3) + 4 * jj + 2 * hi + (j >> 2));
+        *reinterpret_cast<uint32_t*>(rec + TK4_REC + 256 * st + 4 * l) = hb;
+    }
     if (kq == 0 && st == 0) {
         uint32_t sc[2] = {0, 0}, mn[2] = {0, 0}, dd = 0;
         if (row < n_out) {
@@ -321,9 +339,11 @@ hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t 
     if (fmt == FMT_Q8_0) {
         size_t total = (size_t)row_tiles((uint32_t)n_out) * t8_steps((uint32_t)n_in) * 64;
         pack_t8_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
-    } else if (fmt == FMT_Q4_K) {
+    } else if (k45_format(fmt)) {
         size_t total = (size_t)row_tiles((uint32_t)n_out) * tk4_sbs((uint32_t)n_in) * 128;
-        pack_tk4_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
+        if (!total) return hipSuccess;
+        if (fmt == FMT_Q5_K) pack_tk4_kernel<true><<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
+        else pack_tk4_kernel<false><<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
     } else if (fmt == FMT_Q6_K) {
         size_t total = (size_t)row_tiles((uint32_t)n_out) * t6k_steps((uint32_t)n_in) * 64;
         if (!total) return hipSuccess;

@@ -178,8 +178,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
             wbase[i] = w.p0 + ((size_t)tile * all_steps + step0) * T4M_REC;
         } else if (q8_format(FMT)) {  // the tile's records; load_raw indexes them from the matrix's first step
             wbase[i] = w.p0 + (size_t)tile * t8_steps(w.n_in) * (FMT == FMT_Q8F ? T8F_REC : T8_REC);
-        } else if (FMT == FMT_Q4_K) {
-            wbase[i] = w.p0 + (size_t)tile * tk4_sbs(w.n_in) * TK4_REC;
+        } else if (k45_format(FMT)) {
+            wbase[i] = w.p0 + (size_t)tile * tk4_sbs(w.n_in) * (FMT == FMT_Q5_K ? TK5_REC : TK4_REC);
         } else if (FMT == FMT_Q6_K) {
             wbase[i] = w.p0 + (size_t)tile * t6k_steps(w.n_in) * T6K_REC;
         } else {
@@ -229,10 +229,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
                         r[i].m[h] = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
                     }
                 }
-            } else if (FMT == FMT_Q4_K) {  // half a super-block record: sub-blocks 4 (sa & 1) .. + 3
+            } else if (k45_format(FMT)) {  // half a super-block record: sub-blocks 4 (sa & 1) .. + 3
                 const uint32_t sa = step0 + s;
-                const uint8_t* rec = wbase[i] + (size_t)(sa >> 1) * TK4_REC;
+                const uint8_t* rec = wbase[i] + (size_t)(sa >> 1) * (FMT == FMT_Q5_K ? TK5_REC : TK4_REC);
                 r[i].c = *reinterpret_cast<const uint4*>(rec + (sa & 1) * 1024 + 16 * lane);
+                if (FMT == FMT_Q5_K) r[i].c2.x = *reinterpret_cast<const uint32_t*>(rec + TK4_REC + (sa & 1) * 256 + 4 * lane);
                 r[i].m[0] = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 4 * (sa & 1));
                 r[i].m[1] = *reinterpret_cast<const uint32_t*>(rec + 2048 + 16 * n + 8 + 4 * (sa & 1));
                 r[i].m[2] = *reinterpret_cast<const uint32_t*>(rec + 2304 + 4 * n);
@@ -287,14 +288,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
                 if (h && past) d = 0.0f;
                 dst[b * WG_NT * 64] = dequant_u8x8(cw[2 * b] ^ 0x80808080u, cw[2 * b + 1] ^ 0x80808080u, d, -128.0f * d);
             }
-        } else if (FMT == FMT_Q4_K) {  // block b = 2 jj + e: the low (e = 0) or high nibbles of the chunk's byte pair jj
+        } else if (k45_format(FMT)) {  // block b = 2 jj + e: the low (e = 0) or high nibbles of the chunk's byte pair jj
             const float d = f16_bits_to_f32((uint16_t)(r.m[2] & 0xFFFF)), dmin = f16_bits_to_f32((uint16_t)(r.m[2] >> 16));
 #pragma unroll
             for (int b = 0; b < 4; b++) {
                 const int jj = b >> 1, e = b & 1;
                 const uint32_t lo = jj ? r.c.z : r.c.x, hi = jj ? r.c.w : r.c.y;
                 const float sc = (float)((r.m[0] >> (8 * b)) & 0xFF), mn = (float)((r.m[1] >> (8 * b)) & 0xFF);
-                dst[b * WG_NT * 64] = dequant_u8x8((lo >> (4 * e)) & 0x0F0F0F0Fu, (hi >> (4 * e)) & 0x0F0F0F0Fu, d * sc, -(dmin * mn));
+                uint32_t w0 = (lo >> (4 * e)) & 0x0F0F0F0Fu, w1 = (hi >> (4 * e)) & 0x0F0F0F0Fu;
+                if (FMT == FMT_Q5_K) {  // the fifth bits of the block's two dwords: bits 8 k + 2 b and 8 k + 2 b + 1 of the plane
+                    w0 |= ((r.c2.x >> (2 * b)) & 0x01010101u) << 4;
+                    w1 |= ((r.c2.x >> (2 * b + 1)) & 0x01010101u) << 4;
+                }
+                dst[b * WG_NT * 64] = dequant_u8x8(w0, w1, d * sc, -(dmin * mn));
             }
         } else if (FMT == FMT_Q6_K) {  // block b = 2 h + e: codes 8 e .. + 7 of the lane's 16 columns of half h
             const float d = f16_bits_to_f32((uint16_t)(r.m[2] & 0xFFFF));
@@ -479,7 +485,7 @@ hipError_t launch_gemm_reduce(const float* partial, size_t n, uint32_t slices, v
 // steps with scale blocks of 16 k rows x 128 k columns.
 bool gemm_bf16_ok(const WeightView& w) {
     if (t4m_format(w.fmt) || q8_format(w.fmt)) return true;
-    if (w.fmt == FMT_Q4_K || w.fmt == FMT_Q6_K) return w.n_in % 256 == 0;
+    if (k45_format(w.fmt) || w.fmt == FMT_Q6_K) return w.n_in % 256 == 0;
     return w.fmt == FMT_FP8 && w.br % 16 == 0 && w.bc % 128 == 0 && w.n_in % 128 == 0;
 }
 // pack_a's MODE for the format's fragments
@@ -494,6 +500,7 @@ hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size
         case FMT_Q8_0: return run_gemm_bf16<FMT_Q8_0>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q8F: return run_gemm_bf16<FMT_Q8F>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q4_K: return run_gemm_bf16<FMT_Q4_K>(w, apk, t, mtiles, y, out_bf16, partial, s);
+        case FMT_Q5_K: return run_gemm_bf16<FMT_Q5_K>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q6_K: return run_gemm_bf16<FMT_Q6_K>(w, apk, t, mtiles, y, out_bf16, partial, s);
         default: return run_gemm_bf16<FMT_FP8>(w, apk, t, mtiles, y, out_bf16, partial, s);
     }

@@ -22,18 +22,21 @@ namespace oxhip {
 //                                     of a group carries the same scale
 //         p2 off [n_out][n_in/group]  bf16 offsets, optional
 //   Q6_K  p0      T6K records (layout.hpp)
+//   Q5_K  p0      TK5 records (layout.hpp)
 //   Q40   p0      T4M records of GGUF Q4_0: the four f16 block scales of a row where MLX keeps two scales and two offsets
 //   Q8F   p0      T8F records: QMatrix, int8 codes with one f32 scale per 32
 //   FP8   p0 q   [n_out][n_in]        e4m3 bytes (row-major, or tile-packed when group == 1: fp8_offset below);
 //         p1 bs f32 [ceil(n_out/br)][ceil(n_in/bc)]
 //   BF16  p0 q   [n_out][n_in]        bf16
 // ------------------------------------------------------------------------------------------------
-enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6, FMT_Q8F = 7, FMT_Q40 = 8 };
+enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6, FMT_Q8F = 7, FMT_Q40 = 8, FMT_Q5_K = 9 };
 // the formats of the matrix-core decode kernels (decode_mfma.hip); the two Q8 kinds carry no sums or offsets
-inline bool mfma_decode_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F || f == FMT_Q4_K || f == FMT_Q6_K || f == FMT_Q4M || f == FMT_Q40; }
+inline bool mfma_decode_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F || f == FMT_Q4_K || f == FMT_Q6_K || f == FMT_Q4M || f == FMT_Q40 || f == FMT_Q5_K; }
 // the two 4-bit formats in T4M records (MLX: a scale and an offset per 64; GGUF Q4_0: a scale per 32)
 __host__ __device__ constexpr bool t4m_format(int f) { return f == FMT_Q4M || f == FMT_Q40; }
 __host__ __device__ constexpr bool q8_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F; }
+// the K-quants in super-block records with 6-bit scales and mins (Q5_K: the Q4_K record and a plane of fifth bits)
+__host__ __device__ constexpr bool k45_format(int f) { return f == FMT_Q4_K || f == FMT_Q5_K; }
 
 struct WeightView {
     int fmt;

@@ -17,6 +17,9 @@
 //                  (low nibble: sub-block 2 (2 t + jj), high nibble: the next one)
 //               sc[n][8], mn[n][8] bytes (the 6-bit scales and mins, unpacked)       256 B
 //               d[n], dmin[n] f16                                                     64 B
+//   Q5_K (TK5)  the TK4 record followed by the fifth bits, 2880 B:
+//               hbit[256 t + 4 l] (a dword): bit 8 k + i = fifth bit of the code in byte k of the lane's operand dword i
+//                  of step t, i = 4 jj + 2 (high nibble) + (j / 4), k = j % 4, for the codes byte 8 jj + j    512 B
 //   Q4 with one scale and one offset per 64 (MLX; T4M)  step = 4 blocks (128 K), record 1152 B:
 //               codes[16 l + 4 b + j] = q[row n][block 4 s + b][4 kq + j]           1024 B
 //                  (low nibble: element 4 kq + j, high nibble: element 16 + 4 kq + j)
@@ -34,6 +37,7 @@ constexpr uint32_t T8_REC = 1088;
 // QMatrix (int8 codes, f32 scale per 32): the T8 codes followed by the two f32 block scales of each of the 16 rows.
 constexpr uint32_t T8F_REC = 1152;
 constexpr uint32_t TK4_REC = 2368;
+constexpr uint32_t TK5_REC = TK4_REC + 512;
 constexpr uint32_t T4M_REC = 1152;
 // Q6_K, 16 rows x 128 columns (half a super-block), lane = 16 kq + n, code j of half h = row n, column 64 h + 16 kq + j:
 //   [0, 1024)    low nibbles, 16 bytes per lane: dword 2 h + j / 8, byte j % 4, low nibble if j % 8 < 4, else high
@@ -52,6 +56,7 @@ __host__ __device__ inline uint32_t row_tiles(uint32_t n_out) { return (n_out + 
 __host__ __device__ inline size_t t8_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t8_steps(n_in) * T8_REC; }
 __host__ __device__ inline size_t t8f_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t8_steps(n_in) * T8F_REC; }
 __host__ __device__ inline size_t tk4_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * tk4_sbs(n_in) * TK4_REC; }
+__host__ __device__ inline size_t tk5_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * tk4_sbs(n_in) * TK5_REC; }
 __host__ __device__ inline size_t t4m_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t4m_steps(n_in) * T4M_REC; }
 
 __host__ __device__ inline size_t t6k_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t6k_steps(n_in) * T6K_REC; }

@@ -79,6 +79,18 @@ def gguf_q4_k(n_out, n_in, seed):
     return blk.reshape(-1)
 
 
+def gguf_q5_k(n_out, n_in, seed):
+    """Q5_K super-blocks (176 B): the Q4_K header, then 32 bytes of fifth bits and 128 of nibbles, uniform."""
+    rng = np.random.default_rng(seed)
+    nb = n_out * n_in // 256
+    blk = np.empty((nb, 176), np.uint8)
+    blk[:, 0:2] = np.abs(rng.normal(0.0, 0.005, nb)).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    blk[:, 2:4] = np.abs(rng.normal(0.0, 0.005, nb)).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    blk[:, 4:16] = pack_k4_scales(rng.integers(0, 64, (nb, 8)), rng.integers(0, 64, (nb, 8)))
+    blk[:, 16:] = rng.integers(0, 256, (nb, 160), dtype=np.uint8)
+    return blk.reshape(-1)
+
+
 def gguf_q6_k(n_out, n_in, seed):
     """Q6_K super-blocks (210 B): ql, qh uniform bits, int8 scales uniform, f16 d ~ +-|N(0, 0.005)|."""
     rng = np.random.default_rng(seed)

@@ -66,12 +66,12 @@ def test_gemm_bf16_row_magnitudes_and_f32_inputs(be, oxref):
     assert row_err(y, ref) < 2e-2
 
 
-GGUF_KINDS = {"Q4_0": 2, "Q8_0": 8, "Q4_K": 12, "Q6_K": 14}
+GGUF_KINDS = {"Q4_0": 2, "Q8_0": 8, "Q4_K": 12, "Q5_K": 13, "Q6_K": 14}
 
 
 def gguf_raw(name, n_out, n_in, seed):
     from oxinfer_amd import synth
-    return {"Q4_0": synth.gguf_q4_0, "Q8_0": synth.gguf_q8_0, "Q4_K": synth.gguf_q4_k, "Q6_K": synth.gguf_q6_k}[name](n_out, n_in, seed)
+    return {"Q4_0": synth.gguf_q4_0, "Q8_0": synth.gguf_q8_0, "Q4_K": synth.gguf_q4_k, "Q5_K": synth.gguf_q5_k, "Q6_K": synth.gguf_q6_k}[name](n_out, n_in, seed)
 
 
 # 4352 columns = 34 steps of 128: K slices of 9 steps, so slices start inside a Q4_K super-block record; 1120 and 96
