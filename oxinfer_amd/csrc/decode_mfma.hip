@@ -313,7 +313,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // groups 0 and 1 receive the tokens their accumulators hold, the others zeros.
     auto mins = [&](uint32_t b4, float mk) {
         if constexpr (MINS) {
-            const uint32_t at = (min(b4 + kq, nblk - 1) - B0) * TPAD + min(n, (uint32_t)TPAD - 1);
+            // (a block past the row lies inside the slice's arrays all the same, staged as zero)
+            const uint32_t at = (b4 + kq - B0) * TPAD + min(n, (uint32_t)TPAD - 1);
 #pragma unroll
             for (int tg = 0; tg < NG; tg++) {
                 const float f = lds[(size_t)as + tg * nm + at];
@@ -321,7 +322,11 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             }
         }
     };
-    constexpr uint32_t CENTRE = 0x88888888u, TOPN = 0xF0F0F0F0u;
+    // a nibble moved to the top of its byte with its top bit flipped: one three-input bit operation per operand dword
+    // (plus the shift for the low nibbles)
+    constexpr uint32_t TOPB = 0x80808080u, TOPN = 0xF0F0F0F0u;
+    auto centre_lo = [](uint32_t x) { return (int)(((x << 4) & TOPN) ^ TOPB); };
+    auto centre_hi = [](uint32_t x) { return (int)((x & TOPN) ^ TOPB); };
     auto dump_block = [&](uint32_t b, const int* isum) {
         if (!DUMP) return;
         const uint32_t row = tile * 16 + n;
@@ -368,8 +373,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                     bw = v4i{(int)(((x0 << 3) & NIB) | ((hb << (7 - 4 * pr)) & TOP)), (int)(((x1 << 3) & NIB) | ((hb << (6 - 4 * pr)) & TOP)),
                              (int)(((x0 >> 1) & NIB) | ((hb << (5 - 4 * pr)) & TOP)), (int)(((x1 >> 1) & NIB) | ((hb << (4 - 4 * pr)) & TOP))};
                 } else {
-                    const uint32_t x0 = (pr ? c.z : c.x) ^ CENTRE, x1 = (pr ? c.w : c.y) ^ CENTRE;
-                    bw = v4i{(int)((x0 << 4) & TOPN), (int)((x1 << 4) & TOPN), (int)(x0 & TOPN), (int)(x1 & TOPN)};
+                    const uint32_t x0 = pr ? c.z : c.x, x1 = pr ? c.w : c.y;
+                    bw = v4i{centre_lo(x0), centre_lo(x1), centre_hi(x0), centre_hi(x1)};
                 }
                 const uint32_t b = 4 * s + 2 * pr + d_half;  // global index of this lane's block of 32
 #pragma unroll
@@ -436,8 +441,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         } else {
 #pragma unroll
             for (int g = 0; g < 2; g++) {  // the two groups of 64 of the step
-                const uint32_t x0 = (g ? c.z : c.x) ^ CENTRE, x1 = (g ? c.w : c.y) ^ CENTRE;  // blocks 2 g, 2 g + 1
-                v4i bw = {(int)((x0 << 4) & TOPN), (int)(x0 & TOPN), (int)((x1 << 4) & TOPN), (int)(x1 & TOPN)};
+                const uint32_t x0 = g ? c.z : c.x, x1 = g ? c.w : c.y;  // blocks 2 g, 2 g + 1
+                v4i bw = {centre_lo(x0), centre_hi(x0), centre_lo(x1), centre_hi(x1)};
                 const uint32_t b = 4 * s + 2 * g + d_half;
                 // MLX: the group's scale; Q4_0: the lane's block's own scale (word g, half d_half)
                 const float d = FMT == FMT_Q40 ? f16_bits_to_f32((uint16_t)(d_half ? sw[g] >> 16 : sw[g] & 0xFFFF))
