@@ -48,7 +48,7 @@ def profile_traffic(profile, kernel):
     if len(sect) < 2:
         return None
     for line in sect[1].splitlines():
-        m = re.match(r"\|\s*`" + re.escape(kernel) + r"`\s*\|.*\|\s*(\d+)\s*\|\s*$", line)
+        m = re.match(r"\|\s*`" + re.escape(kernel) + r"(?:<[^`]*>)?`\s*\|.*\|\s*(\d+)\s*\|\s*$", line)
         if m:
             return int(m.group(1))
     return None
