@@ -888,11 +888,11 @@ __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid,
 }
 
 // FSET: the formats compiled in, one bit per Fmt. The compiler allocates registers over the whole kernel, so every
-// format in it costs the others (a seventh format made the three common GGUF ones 15 % slower): a launch takes the
-// smallest of the sets below that holds all its jobs' formats.
+// format in it costs the others (a seventh format made the common GGUF ones 15 % slower, and Q6_K beside Q8_0 and Q4_K
+// spilled registers inside its loop): a launch takes the smallest of the sets below that holds all its jobs' formats.
 constexpr uint32_t fbit(int f) { return 1u << f; }
-constexpr uint32_t FSET_GGUF = fbit(FMT_Q8_0) | fbit(FMT_Q4_K) | fbit(FMT_Q6_K), FSET_MLX = fbit(FMT_Q4M),
-                   FSET_ALL = FSET_GGUF | FSET_MLX | fbit(FMT_Q8F) | fbit(FMT_Q5_K) | fbit(FMT_Q40);
+constexpr uint32_t FSET_GGUF = fbit(FMT_Q8_0) | fbit(FMT_Q4_K), FSET_Q6K = fbit(FMT_Q6_K), FSET_MLX = fbit(FMT_Q4M),
+                   FSET_ALL = FSET_GGUF | FSET_Q6K | FSET_MLX | fbit(FMT_Q8F) | fbit(FMT_Q5_K) | fbit(FMT_Q40);
 template <uint32_t FSET>
 __global__ __launch_bounds__(1024) void decode_batch_kernel(BatchArgs a) {
     extern __shared__ __align__(16) float lds_dyn[];
@@ -1184,7 +1184,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     (void)hipGetDevice(&dev);
     const uint64_t bit = 1ull << (dev & 63);
     if (!(allowed[(dev >> 6) & 3].load(std::memory_order_acquire) & bit)) {
-        for (const void* k : {reinterpret_cast<const void*>(decode_batch_kernel<FSET_GGUF>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_MLX>),
+        for (const void* k : {reinterpret_cast<const void*>(decode_batch_kernel<FSET_GGUF>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_MLX>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_Q6K>),
                               reinterpret_cast<const void*>(decode_batch_kernel<FSET_ALL>)}) {
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
             if (e != hipSuccess) return e;
@@ -1265,6 +1265,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
         };
         if (!(fset & ~FSET_GGUF)) go(decode_batch_kernel<FSET_GGUF>);
         else if (!(fset & ~FSET_MLX)) go(decode_batch_kernel<FSET_MLX>);
+        else if (!(fset & ~FSET_Q6K)) go(decode_batch_kernel<FSET_Q6K>);
         else go(decode_batch_kernel<FSET_ALL>);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
