@@ -41,7 +41,7 @@ enum {
 };
 
 /* GGUF type ids handled (src/ggml.rs:42-93). */
-enum { OXHIP_GGML_Q4_0 = 2, OXHIP_GGML_Q8_0 = 8, OXHIP_GGML_Q4_K = 12, OXHIP_GGML_Q5_K = 13, OXHIP_GGML_Q6_K = 14, OXHIP_GGML_F8E4M3 = 0x1000 };
+enum { OXHIP_GGML_Q4_0 = 2, OXHIP_GGML_Q8_0 = 8, OXHIP_GGML_Q4_K = 12, OXHIP_GGML_Q5_K = 13, OXHIP_GGML_Q6_K = 14, OXHIP_GGML_MXFP4 = 39, OXHIP_GGML_F8E4M3 = 0x1000 };
 
 typedef struct {
     uint32_t kind;            /* OXHIP_W_* */
@@ -110,8 +110,8 @@ void oxhip_free_weight(oxhip_ctx* ctx, oxhip_weight* w);
 size_t oxhip_weight_bytes(const oxhip_weight* w);
 /* Backend::matmul (src/gpu.rs:160; src/cuda.rs:1428-1493): all jobs share x [t, n_in] (host f32);
  * computes every job or none. Routing as matmul_quant_multi_at's (src/kernels.rs:1731-1879): up to 8 tokens the
- * Q8 / Q8_0 / Q4_K / Q5_K / Q6_K / MLX 4-bit jobs share one launch of the int8 decode kernel (the CPU's decode semantics,
- * src/kernels.rs:1908-1928); more than 16 tokens over MLX 4-bit, Q8, Q8_0, Q4_K, Q5_K, Q6_K or FP8 (128-column blocks)
+ * Q8 / Q8_0 / Q4_K / Q5_K / Q6_K / MXFP4 / MLX 4-bit jobs share one launch of the int8 decode kernel (the CPU's decode semantics,
+ * src/kernels.rs:1908-1928); more than 16 tokens over MLX 4-bit, Q8, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4 or FP8 (128-column blocks)
  * weights run the bf16 matrix-core GEMM; everything else runs the decode kernels over 16 tokens at a time. */
 int oxhip_matmul(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_job* jobs, size_t n_jobs);
 /* Backend::matvec_rows (src/gpu.rs:165): t in 1..=4. */
@@ -171,7 +171,7 @@ int oxhip_dev_decode(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_qact* xa
 /* oxhip_dev_decode for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc); it has no counterpart in the reference. The same kernels and the same
  * bits as oxhip_dev_decode over the quantized formats of the matrix-core decode kernel (Q8, Q8_0, Q4_0, Q4_K, Q5_K, Q6_K,
- * MLX 4-bit; 1 <= t <= 16), but the partial rows and arrival counters of shapes that slice K live in an array the
+ * MXFP4, MLX 4-bit; 1 <= t <= 16), but the partial rows and arrival counters of shapes that slice K live in an array the
  * library holds statically on every GPU (4 MiB + 256 KiB, kept until the process ends), and the call allocates and
  * frees nothing on the device. Declined (0, nothing written) when the weight needs more than that: K slices x 8 x
  * n_out floats of partial rows beyond 4 MiB, or more than 2048 row groups. All calls on one GPU share the array:

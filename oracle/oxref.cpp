@@ -233,7 +233,7 @@ float oxref_bf16_to_f32(uint16_t h) { return bits_f32((uint32_t)h << 16); }  // 
 size_t oxref_block_size(uint32_t kind) {
     switch (kind) {
         case OXREF_F32: case OXREF_F16: case OXREF_BF16: case OXREF_F8E4M3: return 1;
-        case OXREF_Q4_0: case OXREF_Q4_1: case OXREF_Q5_0: case OXREF_Q5_1: case OXREF_Q8_0: return 32;
+        case OXREF_Q4_0: case OXREF_Q4_1: case OXREF_Q5_0: case OXREF_Q5_1: case OXREF_Q8_0: case OXREF_MXFP4: return 32;
         case OXREF_Q2_K: case OXREF_Q4_K: case OXREF_Q5_K: case OXREF_Q6_K: return QK_K;
         default: return 0;
     }
@@ -252,6 +252,7 @@ size_t oxref_type_size(uint32_t kind) {
         case OXREF_Q4_K: return 144;
         case OXREF_Q5_K: return 176;
         case OXREF_Q6_K: return 210;
+        case OXREF_MXFP4: return 17;
         default: return 0;
     }
 }
@@ -312,6 +313,7 @@ void oxref_random_blocks(uint32_t kind, size_t nb, uint64_t* seed, uint8_t* out)
                 put_f16(b, 2, rnd_scale(seed, false));
                 break;
             case OXREF_Q6_K: put_f16(b, 208, rnd_scale(seed, true)); break;
+            case OXREF_MXFP4: b[0] = (uint8_t)(118 + oxref_lcg(seed) % 7); break;  // src/ggml.rs:1491
             default: put_f16(b, 0, rnd_scale(seed, true)); break;
         }
     }
@@ -326,8 +328,13 @@ uint64_t oxref_fnv1a_f32(const float* v, size_t n) {
     return h;
 }
 
+// MXFP4: E2M1 values stored doubled (src/ggml_tables.rs:1896) and half the value of the block's E8M0 scale byte,
+// 2^(e - 128) (src/ggml.rs:466-475: the two smallest codes are subnormal f32 values).
+static const int8_t KVALUES_MXFP4[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+static float e8m0_half(uint8_t e) { return e < 2 ? bits_f32(0x00200000u << e) : bits_f32(((uint32_t)e - 1) << 23); }
+
 // ---------------------------------------------------------------------------------------------
-// dequantize_row (src/ggml.rs:630-793)
+// dequantize_row (src/ggml.rs:630-793; MXFP4 :922-928)
 // ---------------------------------------------------------------------------------------------
 void oxref_dequantize_row(uint32_t kind, const uint8_t* src, size_t n, float* out) {
     switch (kind) {
@@ -355,6 +362,14 @@ void oxref_dequantize_row(uint32_t kind, const uint8_t* src, size_t n, float* ou
                 for (int j = 0; j < 16; j++) {
                     y[j] = (float)((int)(b[2 + j] & 0xF) - 8) * d;
                     y[j + 16] = (float)((int)(b[2 + j] >> 4) - 8) * d;
+                }
+                break;
+            }
+            case OXREF_MXFP4: {
+                float d = e8m0_half(b[0]);
+                for (int j = 0; j < 16; j++) {
+                    y[j] = d * (float)KVALUES_MXFP4[b[1 + j] & 0xF];
+                    y[j + 16] = d * (float)KVALUES_MXFP4[b[1 + j] >> 4];
                 }
                 break;
             }
@@ -489,6 +504,13 @@ int oxref_decode_i8(uint32_t kind, const uint8_t* b, int8_t* q, float* s, float*
         case OXREF_Q8_0:
             for (int j = 0; j < 32; j++) q[j] = (int8_t)b[2 + j];
             s[0] = s[1] = f16at(b, 0);
+            return 0;
+        case OXREF_MXFP4:  // src/ggml.rs:1209-1216
+            s[0] = s[1] = e8m0_half(b[0]);
+            for (int j = 0; j < 16; j++) {
+                q[j] = KVALUES_MXFP4[b[1 + j] & 0xF];
+                q[j + 16] = KVALUES_MXFP4[b[1 + j] >> 4];
+            }
             return 0;
         case OXREF_Q2_K: {
             float d = f16at(b, 80), mn = f16at(b, 82);

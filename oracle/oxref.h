@@ -33,7 +33,7 @@ extern "C" {
 enum {
     OXREF_F32 = 0, OXREF_F16 = 1, OXREF_Q4_0 = 2, OXREF_Q4_1 = 3, OXREF_Q5_0 = 6, OXREF_Q5_1 = 7,
     OXREF_Q8_0 = 8, OXREF_Q2_K = 10, OXREF_Q3_K = 11, OXREF_Q4_K = 12, OXREF_Q5_K = 13,
-    OXREF_Q6_K = 14, OXREF_BF16 = 30, OXREF_F8E4M3 = 0x1000
+    OXREF_Q6_K = 14, OXREF_BF16 = 30, OXREF_MXFP4 = 39, OXREF_F8E4M3 = 0x1000
 };
 
 /* conversions (half crate 2.7.1 semantics: IEEE RNE) */

@@ -13,9 +13,9 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "liboxref.so")
 
 F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 = 0, 1, 2, 3, 6, 7, 8
-Q2_K, Q4_K, Q5_K, Q6_K, BF16, F8E4M3 = 10, 12, 13, 14, 30, 0x1000
+Q2_K, Q4_K, Q5_K, Q6_K, BF16, MXFP4, F8E4M3 = 10, 12, 13, 14, 30, 39, 0x1000
 NAMES = {F32: "F32", F16: "F16", Q4_0: "Q4_0", Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q8_0: "Q8_0",
-         Q2_K: "Q2_K", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", BF16: "BF16"}
+         Q2_K: "Q2_K", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", BF16: "BF16", MXFP4: "MXFP4"}
 
 
 def build():

@@ -373,6 +373,12 @@ static oxhip_weight* upload_weight(oxhip_ctx* c, const oxhip_weight_desc* d, boo
                 pl.add(0, tk5_bytes((uint32_t)n_out, (uint32_t)n_in));
                 raw_bytes = n_out * (n_in / 256) * 176;
                 np = 1;
+            } else if (d->ggml_type == OXHIP_GGML_MXFP4) {
+                if (n_in % 32) return fail("MXFP4 rows must be whole blocks of 32");
+                w->v.fmt = FMT_MXFP4;
+                pl.add(0, t4x_bytes((uint32_t)n_out, (uint32_t)n_in));
+                raw_bytes = n_out * (n_in / 32) * 17;
+                np = 1;
             } else if (d->ggml_type == OXHIP_GGML_Q6_K) {
                 if (n_in % 256) return fail("Q6_K rows must be whole blocks of 256");
                 w->v.fmt = FMT_Q6_K;
@@ -499,7 +505,7 @@ int oxhip_dev_decode_noalloc(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qa
         return 0;
     }
     if (!mfma_decode_format(w->v.fmt)) {
-        set_error("decode_noalloc: only the quantized formats of the matrix-core decode kernel (Q8, Q8_0, Q4_0, Q4_K, Q5_K, Q6_K, MLX 4-bit)");
+        set_error("decode_noalloc: only the quantized formats of the matrix-core decode kernel (Q8, Q8_0, Q4_0, Q4_K, Q5_K, Q6_K, MXFP4, MLX 4-bit)");
         return 0;
     }
     if (xa->n_in != w->v.n_in || xa->t < t) {

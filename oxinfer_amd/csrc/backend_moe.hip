@@ -297,7 +297,7 @@ oxhip_moe* oxhip_upload_moe(oxhip_ctx* c, const oxhip_weight_desc* gate_up, cons
             if (w->v.fmt != v[0]->v.fmt || !mfma_format(w)) return false;
         return true;
     };
-    if (!same(m->gate_up) || !same(m->down) || (up && !same(m->up))) return fail("experts must share one of the formats the grouped kernel runs (Q8_0, Q4_K, Q4_0, MLX Q4)");
+    if (!same(m->gate_up) || !same(m->down) || (up && !same(m->up))) return fail("experts must share one of the formats the grouped kernel runs (Q8_0, Q4_K, Q4_0, MXFP4, MLX Q4)");
     auto table = [&](const std::vector<oxhip_weight*>& v, const uint8_t*** out) {
         std::vector<const uint8_t*> host(v.size());
         for (size_t i = 0; i < v.size(); i++) host[i] = v[i]->v.p0;

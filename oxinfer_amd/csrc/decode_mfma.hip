@@ -114,6 +114,11 @@ struct Step<FMT_Q40> {
     uint32_t a[4];
 };
 template <>
+struct Step<FMT_MXFP4> {
+    uint4 w;
+    uint32_t a[4];
+};
+template <>
 struct Step<FMT_Q6_K> {
     uint4 w;   // low nibbles
     uint2 h;   // high bit pairs
@@ -141,7 +146,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     constexpr bool SWZ = NT >= 8;
     constexpr int NI = NT < 4 ? NT : 4;          // accumulator registers that hold live tokens
     constexpr bool MINS = k45_format(FMT) || FMT == FMT_Q4M;   // m * fs terms (Q4_0 has none)
-    constexpr int NARR = q8_format(FMT) || FMT == FMT_Q40 ? 1 : FMT == FMT_Q6_K ? (DUMP ? 4 : 3) : 2;  // metadata arrays
+    constexpr int NARR = q8_format(FMT) || FMT == FMT_Q40 || FMT == FMT_MXFP4 ? 1 : FMT == FMT_Q6_K ? (DUMP ? 4 : 3) : 2;  // metadata arrays
     // the wave index and everything derived from it (tile, K range) live in scalar registers: branches on them are
     // scalar, and the load counters the compiler keeps stay exact across them
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -158,7 +163,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     const uint32_t ntiles = glu && r < ghalf ? gtiles : row_tiles(w.n_out);
     // this workgroup's slice of K: steps [S0, S1), blocks [B0, B0 + nbl) (a multiple of 4 blocks)
     constexpr uint32_t BPS = q8_format(FMT) ? 2 : 4;  // blocks of 32 per step
-    constexpr uint32_t K45_REC = FMT == FMT_Q5_K ? TK5_REC : TK4_REC;
+    constexpr uint32_t K45_REC = FMT == FMT_Q5_K ? TK5_REC : TK4_REC, T4_REC = FMT == FMT_MXFP4 ? T4X_REC : T4M_REC;
     const uint32_t nsteps = q8_format(FMT)    ? t8_steps(w.n_in)
                             : k45_format(FMT) ? 2 * tk4_sbs(w.n_in)
                             : FMT == FMT_Q6_K ? t6k_steps(w.n_in)
@@ -211,7 +216,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                                                                   : FMT == FMT_Q8F  ? (size_t)nsteps * T8F_REC
                                                                   : k45_format(FMT) ? (size_t)(nsteps / 2) * K45_REC
                                                                   : FMT == FMT_Q6_K ? (size_t)nsteps * T6K_REC
-                                                                                    : (size_t)nsteps * T4M_REC);
+                                                                                    : (size_t)nsteps * T4_REC);
 
     auto act2 = [&](uint32_t b, uint32_t pos, uint32_t* out) {  // 8 consecutive activations of block b
         const uint2 v = *reinterpret_cast<const uint2*>(xrow + min(b, nblk - 1) * 32 + pos);
@@ -237,7 +242,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             st.w = gload<uint4>(rec + 16 * lane);
             st.h = gload<uint2>(rec + 1024 + 8 * lane);
         } else {
-            const gbytes rec = base + (size_t)s * T4M_REC;
+            const gbytes rec = base + (size_t)s * T4_REC;
             st.w = gload<uint4>(rec + 16 * lane);
             if (!ALDS) {
 #pragma unroll
@@ -255,7 +260,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // kq asks for the words of step `first + kq` (row n of it), and at step first + q every lane takes them from lane
     // 16 q + n. Q8_0: {d of the two blocks}; Q4_K: {four sub-block scales, four mins, (d, dmin)}: this step's four
     // sub-blocks are 4 (s & 1) .. + 3 of the super-block; MLX: {d of the two groups, offsets of the two groups}.
-    constexpr int NM = FMT == FMT_Q8_0 ? 1 : (k45_format(FMT) || FMT == FMT_Q6_K) ? 3 : 2;  // (Q8F: the two f32 scales)
+    constexpr int NM = FMT == FMT_Q8_0 || FMT == FMT_MXFP4 ? 1 : (k45_format(FMT) || FMT == FMT_Q6_K) ? 3 : 2;  // (Q8F: the two f32 scales)
     const uint32_t slast = max(s1, 1u) - 1;
     auto load_scales = [&](uint32_t* m, uint32_t first) {
         const uint32_t s = min(first + kq, slast);
@@ -274,6 +279,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             m[0] = gload<uint32_t>(rec + 1536 + 8 * n);
             m[1] = gload<uint32_t>(rec + 1540 + 8 * n);
             m[2] = gload<uint16_t>(rec + 1664 + 2 * n);
+        } else if constexpr (FMT == FMT_MXFP4) {  // the four scale bytes of row n's blocks
+            m[0] = gload<uint32_t>(base + (size_t)s * T4X_REC + 1024 + 4 * n);
         } else {
             const gbytes rec = base + (size_t)s * T4M_REC;
             m[0] = gload<uint32_t>(rec + 1024 + 4 * n);
@@ -442,14 +449,20 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
 #pragma unroll
             for (int g = 0; g < 2; g++) {  // the two groups of 64 of the step
                 const uint32_t x0 = g ? c.z : c.x, x1 = g ? c.w : c.y;  // blocks 2 g, 2 g + 1
-                v4i bw = {centre_lo(x0), centre_hi(x0), centre_lo(x1), centre_hi(x1)};
+                constexpr bool MX = FMT == FMT_MXFP4;  // table codes: the int8 operand is the code's doubled value itself
+                constexpr uint32_t NIB = 0x0F0F0F0Fu;
+                v4i bw = MX ? v4i{(int)mxfp4_values<0>(x0 & NIB), (int)mxfp4_values<0>((x0 >> 4) & NIB), (int)mxfp4_values<0>(x1 & NIB),
+                                  (int)mxfp4_values<0>((x1 >> 4) & NIB)}
+                            : v4i{centre_lo(x0), centre_hi(x0), centre_lo(x1), centre_hi(x1)};
                 const uint32_t b = 4 * s + 2 * g + d_half;
-                // MLX: the group's scale; Q4_0: the lane's block's own scale (word g, half d_half)
-                const float d = FMT == FMT_Q40 ? f16_bits_to_f32((uint16_t)(d_half ? sw[g] >> 16 : sw[g] & 0xFFFF))
-                                               : f16_bits_to_f32((uint16_t)(g ? sw[0] >> 16 : sw[0] & 0xFFFF));
+                // MLX: the group's scale; Q4_0: the lane's block's own scale (word g, half d_half); MXFP4: its scale byte
+                float d;
+                if constexpr (MX) d = e8m0_half((sw[0] >> (8 * (2 * g + d_half))) & 0xFF);
+                else if constexpr (FMT == FMT_Q40) d = f16_bits_to_f32((uint16_t)(d_half ? sw[g] >> 16 : sw[g] & 0xFFFF));
+                else d = f16_bits_to_f32((uint16_t)(g ? sw[0] >> 16 : sw[0] & 0xFFFF));
                 // padding blocks hold zero codes (which centre to -8) and zero scales: they add zeros (as a select, not a
                 // branch: a divergent branch here makes every step wait for all requests)
-                const float dz = b < nblk ? d * 0.0625f : 0.0f;
+                const float dz = b < nblk ? (MX ? d : d * 0.0625f) : 0.0f;
 #pragma unroll
                 for (int tg = 0; tg < NG; tg++) {
                     v4i D = mfma(bw, 2 * s + g, tg, st.a[2 * g], st.a[2 * g + 1]);
@@ -459,7 +472,8 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
 #pragma unroll
                     for (int i = 0; i < NI; i++) acc[tg][i] = fmaf(dz, xs[i] * (float)I[i], acc[tg][i]);
                     if (DUMP) {
-                        int isum[4] = {I[0] >> 4, I[1] >> 4, I[2] >> 4, I[3] >> 4};
+                        constexpr int SH = MX ? 0 : 4;
+                        int isum[4] = {I[0] >> SH, I[1] >> SH, I[2] >> SH, I[3] >> SH};
                         dump_block(b, isum);
                     }
                 }
@@ -892,7 +906,7 @@ __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid,
 // spilled registers inside its loop): a launch takes the smallest of the sets below that holds all its jobs' formats.
 constexpr uint32_t fbit(int f) { return 1u << f; }
 constexpr uint32_t FSET_GGUF = fbit(FMT_Q8_0) | fbit(FMT_Q4_K), FSET_Q6K = fbit(FMT_Q6_K), FSET_MLX = fbit(FMT_Q4M),
-                   FSET_ALL = FSET_GGUF | FSET_Q6K | FSET_MLX | fbit(FMT_Q8F) | fbit(FMT_Q5_K) | fbit(FMT_Q40);
+                   FSET_ALL = FSET_GGUF | FSET_Q6K | FSET_MLX | fbit(FMT_Q8F) | fbit(FMT_Q5_K) | fbit(FMT_Q40) | fbit(FMT_MXFP4);
 template <uint32_t FSET>
 __global__ __launch_bounds__(1024) void decode_batch_kernel(BatchArgs a) {
     extern __shared__ __align__(16) float lds_dyn[];
@@ -908,6 +922,7 @@ __global__ __launch_bounds__(1024) void decode_batch_kernel(BatchArgs a) {
         case FMT_Q6_K: if constexpr (FSET & fbit(FMT_Q6_K)) batch_dispatch<FMT_Q6_K>(jb, bx, lds_dyn); break;
         case FMT_Q4M: if constexpr (FSET & fbit(FMT_Q4M)) batch_dispatch<FMT_Q4M>(jb, bx, lds_dyn); break;
         case FMT_Q40: if constexpr (FSET & fbit(FMT_Q40)) batch_dispatch<FMT_Q40>(jb, bx, lds_dyn); break;
+        case FMT_MXFP4: if constexpr (FSET & fbit(FMT_MXFP4)) batch_dispatch<FMT_MXFP4>(jb, bx, lds_dyn); break;
         default: break;
     }
 }
@@ -987,7 +1002,7 @@ Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices, int fmt) {
     static std::mutex mu;
     static std::map<uint64_t, Shape> cache;
     // ntiles and nsteps are below 2^27 (n_out, n_in < 2^31): 27 + 27 + 8 bits of format + 1
-    static_assert(FMT_Q5_K < 256, "the key keeps 8 bits of the format");
+    static_assert(FMT_MXFP4 < 256, "the key keeps 8 bits of the format");
     const uint64_t key = ((uint64_t)ntiles << 36) | ((uint64_t)nsteps << 9) | ((uint64_t)(fmt & 0xFF) << 1) | (allow_slices ? 1u : 0u);
     std::lock_guard<std::mutex> g(mu);
     auto it = cache.find(key);
@@ -1005,7 +1020,7 @@ constexpr size_t LDS_MAX = 160 * 1024 - 256;  // dynamic LDS on offer (the kerne
 size_t lds_bytes(int fmt, bool dump, uint32_t nsteps, int tpad, const Shape& sh, bool* alds, uint32_t ng = 1) {
     const uint32_t bps = q8_format(fmt) ? 2 : 4;
     const uint32_t nbl = bps * ((nsteps + sh.ks - 1) / sh.ks);  // blocks of a slice
-    const uint32_t narr = q8_format(fmt) || fmt == FMT_Q40 ? 1 : fmt == FMT_Q6_K ? (dump ? 4 : 3) : 2;  // metadata arrays
+    const uint32_t narr = q8_format(fmt) || fmt == FMT_Q40 || fmt == FMT_MXFP4 ? 1 : fmt == FMT_Q6_K ? (dump ? 4 : 3) : 2;  // metadata arrays
     const size_t meta = (size_t)narr * ng * nbl * tpad * 4, red = (size_t)sh.rt * sh.kw * ng * tpad * 16 * 4;
     const size_t act = (size_t)ng * (nbl / 2) * 512;
     const size_t with = act + meta > red ? act + meta : red;  // the partial sums reuse the activations' space
@@ -1300,6 +1315,7 @@ hipError_t launch_decode_mfma_grouped(const WeightView& w, const QActView& xa, c
         case FMT_Q4_K: return run_grouped<FMT_Q4_K>(w, xa, g, max_chunks, max_rows_per_chunk, y, s);
         case FMT_Q4M: return run_grouped<FMT_Q4M>(w, xa, g, max_chunks, max_rows_per_chunk, y, s);
         case FMT_Q40: return run_grouped<FMT_Q40>(w, xa, g, max_chunks, max_rows_per_chunk, y, s);
+        case FMT_MXFP4: return run_grouped<FMT_MXFP4>(w, xa, g, max_chunks, max_rows_per_chunk, y, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -1314,6 +1330,7 @@ hipError_t launch_decode_mfma(const WeightView& w, const QActView& xa, size_t t,
         case FMT_Q6_K: return run<FMT_Q6_K, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
         case FMT_Q4M: return run<FMT_Q4M, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
         case FMT_Q40: return run<FMT_Q40, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
+        case FMT_MXFP4: return run<FMT_MXFP4, false>(w, xa, t, y, nullptr, sc, s, ev_start, ev_stop, epi);
         default: return hipErrorInvalidValue;
     }
 }
@@ -1328,6 +1345,7 @@ hipError_t launch_isums_mfma(const WeightView& w, const QActView& xa, size_t t, 
         case FMT_Q6_K: return run<FMT_Q6_K, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q4M: return run<FMT_Q4M, true>(w, xa, t, y, out, DecodeScratch{}, s);
         case FMT_Q40: return run<FMT_Q40, true>(w, xa, t, y, out, DecodeScratch{}, s);
+        case FMT_MXFP4: return run<FMT_MXFP4, true>(w, xa, t, y, out, DecodeScratch{}, s);
         default: return hipErrorInvalidValue;
     }
 }

@@ -8,6 +8,7 @@
 //   Q4_K  (d * sc) * v - (dmin * mn), v the raw nibble    src/ggml.rs:750-773
 //   Q5_K  the same with v = nibble + 16 * fifth bit       src/ggml.rs:750-773
 //   Q6_K  (d * sc) * q, q = 6-bit code - 32               src/ggml.rs:774-793
+//   MXFP4 2^(e - 128) * doubled E2M1 value               src/ggml.rs:922-928
 //   FP8   e4m3(byte) * block scale                        src/ggml.rs:282-293, :433-444
 //   MLX 4-bit -> Q4 + offsets                             src/quant.rs:518-563
 #include "internal.hpp"
@@ -73,6 +74,15 @@ __global__ __launch_bounds__(256) void dequantize_kernel(WeightView w, uint32_t 
             float d = f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(rec + 1024 + 4 * nn + 2 * (bi >> 1)));
             float m = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(rec + 1088 + 4 * nn + 2 * (bi >> 1)));
             v = (float)(nib - 8) * d + m;
+            break;
+        }
+        case FMT_MXFP4: {
+            uint32_t tile = r >> 4, nn = r & 15, b = c >> 5, st = b >> 2, bi = b & 3, e = c & 31, hi = e >> 4, pp = e & 15, kq = pp >> 2;
+            const uint8_t* rec = w.p0 + ((size_t)tile * t4m_steps(n) + st) * T4X_REC;
+            uint8_t byte = rec[16 * (kq * 16 + nn) + 4 * bi + (pp & 3)];
+            const uint32_t code = hi ? (byte >> 4) : (byte & 0xF);
+            const int kv = (int)(int8_t)(mxfp4_values<0>(code) & 0xFF);
+            v = e8m0_half(rec[1024 + 4 * nn + bi]) * (float)kv;
             break;
         }
         case FMT_Q40: {  // (nib - 8) * d, no offset term (src/ggml.rs:675-683)
@@ -229,6 +239,28 @@ __global__ __launch_bounds__(256) void pack_q4m_kernel(const uint8_t* __restrict
     }
 }
 
+// GGUF MXFP4 blocks (scale byte, 16 code bytes: src/ggml.rs:922-928) -> T4X records; one thread per lane slot of a record.
+__global__ __launch_bounds__(256) void pack_t4x_kernel(const uint8_t* __restrict__ raw, uint32_t n_out, uint32_t n_in, uint8_t* __restrict__ dst) {
+    const uint32_t nsteps = t4m_steps(n_in), nblk = n_in / 32;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x, total = (size_t)row_tiles(n_out) * nsteps * 64;
+    if (idx >= total) return;
+    const uint32_t l = idx & 63, nn = l & 15, kq = l >> 4;
+    const size_t ts = idx >> 6, tile = ts / nsteps, row = tile * 16 + nn;
+    const uint32_t st = (uint32_t)(ts % nsteps);
+    uint8_t* rec = dst + ts * T4X_REC;
+    uint32_t out[4] = {0, 0, 0, 0}, sc = 0;
+    for (uint32_t b = 0; b < 4; b++) {
+        const uint32_t blk = 4 * st + b;
+        if (row < n_out && blk < nblk) {
+            const uint8_t* src = raw + (row * nblk + blk) * 17;
+            for (uint32_t j = 0; j < 4; j++) out[b] |= (uint32_t)src[1 + 4 * kq + j] << (8 * j);
+            sc |= (uint32_t)src[0] << (8 * b);
+        }
+    }
+    *reinterpret_cast<uint4*>(rec + 16 * l) = make_uint4(out[0], out[1], out[2], out[3]);
+    if (kq == 0) *reinterpret_cast<uint32_t*>(rec + 1024 + 4 * nn) = sc;
+}
+
 hipError_t launch_pack_q4m(const uint8_t* q, const uint16_t* sc, const uint16_t* off, size_t n_out, size_t n_in, uint8_t* dst,
                            hipStream_t s) {
     size_t total = (size_t)row_tiles((uint32_t)n_out) * t4m_steps((uint32_t)n_in) * 64;
@@ -344,6 +376,10 @@ hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t 
         if (!total) return hipSuccess;
         if (fmt == FMT_Q5_K) pack_tk4_kernel<true><<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
         else pack_tk4_kernel<false><<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
+    } else if (fmt == FMT_MXFP4) {
+        size_t total = (size_t)row_tiles((uint32_t)n_out) * t4m_steps((uint32_t)n_in) * 64;
+        if (!total) return hipSuccess;
+        pack_t4x_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
     } else if (fmt == FMT_Q6_K) {
         size_t total = (size_t)row_tiles((uint32_t)n_out) * t6k_steps((uint32_t)n_in) * 64;
         if (!total) return hipSuccess;

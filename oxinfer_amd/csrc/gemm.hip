@@ -175,7 +175,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     for (int i = 0; i < 2; i++) {
         const uint32_t tile = min(nt0 + 2 * wave + i, ntiles - 1);
         if (t4m_format(FMT)) {
-            wbase[i] = w.p0 + ((size_t)tile * all_steps + step0) * T4M_REC;
+            wbase[i] = w.p0 + ((size_t)tile * all_steps + step0) * (FMT == FMT_MXFP4 ? T4X_REC : T4M_REC);
         } else if (q8_format(FMT)) {  // the tile's records; load_raw indexes them from the matrix's first step
             wbase[i] = w.p0 + (size_t)tile * t8_steps(w.n_in) * (FMT == FMT_Q8F ? T8F_REC : T8_REC);
         } else if (k45_format(FMT)) {
@@ -206,10 +206,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     auto load_raw_tile = [&](Raw* r, int i, uint32_t s) {  // the records of the wave's row tile i at step s
         {
             if (t4m_format(FMT)) {
-                const uint8_t* rec = wbase[i] + (size_t)s * T4M_REC;
+                const uint8_t* rec = wbase[i] + (size_t)s * (FMT == FMT_MXFP4 ? T4X_REC : T4M_REC);
                 r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
                 r[i].m[0] = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
-                r[i].m[1] = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
+                if (FMT != FMT_MXFP4) r[i].m[1] = *reinterpret_cast<const uint32_t*>(rec + 1088 + 4 * n);
             } else if (q8_format(FMT)) {  // a step of 128 columns is two records of 64 (past the row's last record: that one again,
                                           // which dequant_tile zeroes: nothing here may depend on a loaded value, or the request
                                           // would be waited for where it is made)
@@ -262,7 +262,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     // `s`: the step the records belong to (of this slice)
     auto dequant_tile = [&](const Raw& r, int i, uint32_t buf, uint32_t s) {  // one of the wave's two row tiles, 4 blocks
         uint4* dst = bfrag + ((size_t)(buf * 4) * WG_NT + 2 * wave + i) * 64 + lane;  // block b: + b * WG_NT * 64
-        if (FMT == FMT_Q40) {  // the block's own scale: word b / 2, half b % 2; (nib - 8) * d
+        if (FMT == FMT_MXFP4) {  // the code's doubled value + 12 as an unsigned byte, times the block's power of two: exact in bf16
+            const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const float d = e8m0_half((r.m[0] >> (8 * b)) & 0xFF);
+                dst[b * WG_NT * 64] = dequant_u8x8(mxfp4_values<12>(cw[b] & 0x0F0F0F0Fu), mxfp4_values<12>((cw[b] >> 4) & 0x0F0F0F0Fu), d, -12.0f * d);
+            }
+        } else if (FMT == FMT_Q40) {  // the block's own scale: word b / 2, half b % 2; (nib - 8) * d
             const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
             for (int b = 0; b < 4; b++) {
@@ -497,6 +504,7 @@ hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size
     switch (w.fmt) {
         case FMT_Q4M: return run_gemm_bf16<FMT_Q4M>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q40: return run_gemm_bf16<FMT_Q40>(w, apk, t, mtiles, y, out_bf16, partial, s);
+        case FMT_MXFP4: return run_gemm_bf16<FMT_MXFP4>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q8_0: return run_gemm_bf16<FMT_Q8_0>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q8F: return run_gemm_bf16<FMT_Q8F>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q4_K: return run_gemm_bf16<FMT_Q4_K>(w, apk, t, mtiles, y, out_bf16, partial, s);

@@ -23,17 +23,19 @@ namespace oxhip {
 //         p2 off [n_out][n_in/group]  bf16 offsets, optional
 //   Q6_K  p0      T6K records (layout.hpp)
 //   Q5_K  p0      TK5 records (layout.hpp)
+//   MXFP4 p0      T4X records (layout.hpp)
 //   Q40   p0      T4M records of GGUF Q4_0: the four f16 block scales of a row where MLX keeps two scales and two offsets
 //   Q8F   p0      T8F records: QMatrix, int8 codes with one f32 scale per 32
 //   FP8   p0 q   [n_out][n_in]        e4m3 bytes (row-major, or tile-packed when group == 1: fp8_offset below);
 //         p1 bs f32 [ceil(n_out/br)][ceil(n_in/bc)]
 //   BF16  p0 q   [n_out][n_in]        bf16
 // ------------------------------------------------------------------------------------------------
-enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6, FMT_Q8F = 7, FMT_Q40 = 8, FMT_Q5_K = 9 };
+enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6, FMT_Q8F = 7, FMT_Q40 = 8, FMT_Q5_K = 9, FMT_MXFP4 = 10 };
 // the formats of the matrix-core decode kernels (decode_mfma.hip); the two Q8 kinds carry no sums or offsets
-inline bool mfma_decode_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F || f == FMT_Q4_K || f == FMT_Q6_K || f == FMT_Q4M || f == FMT_Q40 || f == FMT_Q5_K; }
+inline bool mfma_decode_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F || f == FMT_Q4_K || f == FMT_Q6_K || f == FMT_Q4M || f == FMT_Q40 || f == FMT_Q5_K || f == FMT_MXFP4; }
 // the two 4-bit formats in T4M records (MLX: a scale and an offset per 64; GGUF Q4_0: a scale per 32)
-__host__ __device__ constexpr bool t4m_format(int f) { return f == FMT_Q4M || f == FMT_Q40; }
+// (and MXFP4 in the same geometry: 4-bit table codes with a power-of-two scale byte per 32)
+__host__ __device__ constexpr bool t4m_format(int f) { return f == FMT_Q4M || f == FMT_Q40 || f == FMT_MXFP4; }
 __host__ __device__ constexpr bool q8_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F; }
 // the K-quants in super-block records with 6-bit scales and mins (Q5_K: the Q4_K record and a plane of fifth bits)
 __host__ __device__ constexpr bool k45_format(int f) { return f == FMT_Q4_K || f == FMT_Q5_K; }
@@ -293,6 +295,23 @@ __device__ __forceinline__ void scale_min_k4(uint32_t i, uint32_t d0, uint32_t d
         mn = (c >> 4) | ((b >> 6) << 4);
     }
 }
+
+// MXFP4: four E2M1 codes (one per byte, 0..15) -> their doubled values {0, 1, 2, 3, 4, 6, 8, 12} with the sign of bit 3
+// (src/ggml_tables.rs:1896) plus BIAS, as four bytes: a byte permute per sign over an 8-byte table, then a select.
+template <int BIAS>
+__device__ __forceinline__ uint32_t mxfp4_values(uint32_t codes) {
+    constexpr uint32_t B4 = (uint32_t)(BIAS & 0xFF) * 0x01010101u;
+    constexpr uint32_t PLO = 0x03020100u + B4, PHI = 0x0C080604u + B4;                    // BIAS + {0, 1, 2, 3}, {4, 6, 8, 12}
+    constexpr uint32_t NLO = (B4 - 0x03020100u) & 0xFFFFFFFFu, NHI = B4 - 0x0C080604u;  // BIAS - ..., bytewise when BIAS >= 12
+    constexpr uint32_t NLO0 = 0xFDFEFF00u, NHI0 = 0xF4F8FAFCu;                            // BIAS 0: {0, -1, -2, -3}, {-4, -6, -8, -12} as int8
+    const uint32_t sel = codes & 0x07070707u;
+    const uint32_t pos = __builtin_amdgcn_perm(PHI, PLO, sel);
+    const uint32_t neg = __builtin_amdgcn_perm(BIAS ? NHI : NHI0, BIAS ? NLO : NLO0, sel);
+    const uint32_t m = ((codes >> 3) & 0x01010101u) * 0xFFu;
+    return (pos & ~m) | (neg & m);
+}
+// Half the value of an E8M0 scale byte, 2^(e - 128) (src/ggml.rs:466-475; exact for every e, subnormal for e < 2).
+__device__ __forceinline__ float e8m0_half(uint32_t e) { return ldexpf(1.0f, (int)e - 128); }
 
 __device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
 

@@ -27,6 +27,8 @@
 //               off[n][2] bf16                                                        64 B
 //   GGUF Q4_0 in the same records: d[n][4] f16, the scales of blocks 0-1 where MLX has its scales and of blocks 2-3
 //   where it has its offsets.
+//   MXFP4 (T4X) the T4M codes (byte j of a block: elements j and j + 16, as in the file) followed by the four E8M0 scale
+//               bytes of each row's blocks, record 1088 B
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
@@ -39,6 +41,7 @@ constexpr uint32_t T8F_REC = 1152;
 constexpr uint32_t TK4_REC = 2368;
 constexpr uint32_t TK5_REC = TK4_REC + 512;
 constexpr uint32_t T4M_REC = 1152;
+constexpr uint32_t T4X_REC = 1088;
 // Q6_K, 16 rows x 128 columns (half a super-block), lane = 16 kq + n, code j of half h = row n, column 64 h + 16 kq + j:
 //   [0, 1024)    low nibbles, 16 bytes per lane: dword 2 h + j / 8, byte j % 4, low nibble if j % 8 < 4, else high
 //   [1024, 1536) the two high bits, 8 bytes per lane: dword h, bits 8 (j % 4) + 2 (j / 4)
@@ -57,6 +60,7 @@ __host__ __device__ inline size_t t8_bytes(uint32_t n_out, uint32_t n_in) { retu
 __host__ __device__ inline size_t t8f_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t8_steps(n_in) * T8F_REC; }
 __host__ __device__ inline size_t tk4_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * tk4_sbs(n_in) * TK4_REC; }
 __host__ __device__ inline size_t tk5_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * tk4_sbs(n_in) * TK5_REC; }
+__host__ __device__ inline size_t t4x_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t4m_steps(n_in) * T4X_REC; }
 __host__ __device__ inline size_t t4m_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t4m_steps(n_in) * T4M_REC; }
 
 __host__ __device__ inline size_t t6k_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t6k_steps(n_in) * T6K_REC; }

@@ -13,8 +13,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "liboxinfer_hip.so")
 
 W_BF16, W_Q8, W_Q4, W_GGUF, W_MLX_Q4 = 0, 1, 2, 3, 4
-GGML_Q4_0, GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_F8E4M3 = 2, 8, 12, 13, 14, 0x1000
-GGML_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q4_K: (256, 144), GGML_Q5_K: (256, 176), GGML_Q6_K: (256, 210)}
+GGML_Q4_0, GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_MXFP4, GGML_F8E4M3 = 2, 8, 12, 13, 14, 39, 0x1000
+GGML_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q4_K: (256, 144), GGML_Q5_K: (256, 176), GGML_Q6_K: (256, 210), GGML_MXFP4: (32, 17)}
 
 
 class WeightDesc(C.Structure):

@@ -91,6 +91,15 @@ def gguf_q5_k(n_out, n_in, seed):
     return blk.reshape(-1)
 
 
+def gguf_mxfp4(n_out, n_in, seed):
+    """MXFP4 blocks (17 B): an E8M0 scale byte 2^-12..2^-5 (as half values), 16 bytes of E2M1 codes, uniform."""
+    rng = np.random.default_rng(seed)
+    nb = n_out * n_in // 32
+    blk = rng.integers(0, 256, (nb, 17), dtype=np.uint8)
+    blk[:, 0] = rng.integers(116, 124, nb, dtype=np.uint8)
+    return blk.reshape(-1)
+
+
 def gguf_q6_k(n_out, n_in, seed):
     """Q6_K super-blocks (210 B): ql, qh uniform bits, int8 scales uniform, f16 d ~ +-|N(0, 0.005)|."""
     rng = np.random.default_rng(seed)

@@ -12,7 +12,7 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14
+Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4 = 2, 8, 12, 13, 14, 39
 TOL = 1e-3
 
 
@@ -99,7 +99,7 @@ with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "re
     REF_HASHES = {e["ggml_type"]: int(e["fnv1a64"], 16) for e in json.load(_f)["hashes"].values()}
 
 
-@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4])
 def test_gguf_dequant_matches_ggml_hash_on_device(be, oxref, kind):
     """The device dequantizer reproduces the reference's golden hashes (src/ggml.rs:1547-1577)."""
     raw, _ = oxref.random_blocks(kind, 1024 // oxref.block_size(kind), 1000 + kind)
@@ -109,7 +109,7 @@ def test_gguf_dequant_matches_ggml_hash_on_device(be, oxref, kind):
     assert oxref.fnv1a_f32(y) == REF_HASHES[kind]
 
 
-@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4])
 def test_gguf_dequant_and_isums_bit_exact(be, oxref, kind):
     n_out, n_in, t = 37, 3 * 256, 5
     raw, seed = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 13 + kind)
@@ -129,7 +129,7 @@ def test_gguf_dequant_and_isums_bit_exact(be, oxref, kind):
         assert np.array_equal(be.isums(w, xa, 32).cpu().numpy(), isums.reshape(t, n_out, -1, 2).sum(axis=3))
 
 
-@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4])
 @pytest.mark.parametrize("t", [1, 2, 3, 5, 8, 11, 16])
 def test_gguf_decode_matches_oracle(be, oxref, kind, t):
     # rows not a multiple of the wave's row group; Q8_0 with a block count that is not a multiple of 4
@@ -148,7 +148,7 @@ def test_gguf_decode_matches_oracle(be, oxref, kind, t):
         assert np.array_equal(y1[0].view(np.uint32), y[c].view(np.uint32)), c
 
 
-@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4])
 def test_gguf_decode_row_magnitudes(be, oxref, kind):
     n_out, n_in, t = 64, 4096, 4
     raw, seed = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 5 + kind)
@@ -376,12 +376,12 @@ def test_upload_declines(be):
     assert be.upload_gguf(Q4_K, np.zeros(144, np.uint8), 1, 256) is not None
 
 
-@pytest.mark.parametrize("kind,n_out,n_in", [(Q8_0, 14336, 4096), (Q8_0, 4096, 14336), (Q4_K, 14336, 4096), (Q4_K, 4096, 14336), (Q6_K, 14336, 4096), (Q6_K, 4096, 14336), (Q5_K, 4096, 14336)])
+@pytest.mark.parametrize("kind,n_out,n_in", [(Q8_0, 14336, 4096), (Q8_0, 4096, 14336), (Q4_K, 14336, 4096), (Q4_K, 4096, 14336), (Q6_K, 14336, 4096), (Q6_K, 4096, 14336), (Q5_K, 4096, 14336), (MXFP4, 14336, 4096)])
 def test_full_size_rows_against_oracle(be, oxref, kind, n_out, n_in):
     """The benchmark shapes: a sample of rows of the full-size product against the oracle, plus properties
     that hold at any size: the all-ones-activation row sums and batch invariance."""
     from oxinfer_amd import synth
-    gen = {Q8_0: synth.gguf_q8_0, Q4_K: synth.gguf_q4_k, Q5_K: synth.gguf_q5_k, Q6_K: synth.gguf_q6_k}[kind]
+    gen = {Q8_0: synth.gguf_q8_0, Q4_K: synth.gguf_q4_k, Q5_K: synth.gguf_q5_k, Q6_K: synth.gguf_q6_k, MXFP4: synth.gguf_mxfp4}[kind]
     raw = gen(n_out, n_in, 1000 + kind)
     w = be.upload_gguf(kind, raw, n_out, n_in)
     assert w is not None, be.last_error()
@@ -439,7 +439,7 @@ def test_decode_batch_shares_a_launch_and_keeps_the_bits(be, oxref):
     cases = [(Q8_0, 208, 512, 1), (Q4_K, 96, 1024, 8), (Q8_0, 64, 2048, 3), (Q4_K, 176, 512, 2), ("mlx", 80, 640, 5),
              (Q6_K, 48, 512, 2), (Q4_K, 33, 256, 4), ("mlx", 128, 128, 8),
              (Q8_0, 48, 14336, 8), (Q4_K, 32, 14336, 1), (Q6_K, 16, 14336, 5),  # these three slice K across workgroups
-             (Q5_K, 72, 768, 7), (Q5_K, 40, 14336, 1)]
+             (Q5_K, 72, 768, 7), (Q5_K, 40, 14336, 1), (MXFP4, 56, 1120, 6)]
     jobs, alone = [], []
     for i, (kind, n_out, n_in, t) in enumerate(cases):
         if kind == "mlx":
@@ -452,7 +452,7 @@ def test_decode_batch_shares_a_launch_and_keeps_the_bits(be, oxref):
         alone.append(be.decode(w, xa=xa).cpu().numpy())
         y = torch.full((t, n_out), float("nan"), dtype=torch.float32, device="cuda")
         jobs.append((w, xa, None, t, y, None, None))
-    for order in (list(range(len(cases))), list(reversed(range(len(cases)))), [1, 3, 6], [4], [8, 0, 9, 10, 2], [11, 5, 12]):
+    for order in (list(range(len(cases))), list(reversed(range(len(cases)))), [1, 3, 6], [4], [8, 0, 9, 10, 2], [11, 5, 12], [13, 4], [13]):
         for i in order:
             jobs[i][4].fill_(float("nan"))
         be.decode_batch(be.decode_jobs([jobs[i] for i in order]))

@@ -66,18 +66,18 @@ def test_gemm_bf16_row_magnitudes_and_f32_inputs(be, oxref):
     assert row_err(y, ref) < 2e-2
 
 
-GGUF_KINDS = {"Q4_0": 2, "Q8_0": 8, "Q4_K": 12, "Q5_K": 13, "Q6_K": 14}
+GGUF_KINDS = {"Q4_0": 2, "Q8_0": 8, "Q4_K": 12, "Q5_K": 13, "Q6_K": 14, "MXFP4": 39}
 
 
 def gguf_raw(name, n_out, n_in, seed):
     from oxinfer_amd import synth
-    return {"Q4_0": synth.gguf_q4_0, "Q8_0": synth.gguf_q8_0, "Q4_K": synth.gguf_q4_k, "Q5_K": synth.gguf_q5_k, "Q6_K": synth.gguf_q6_k}[name](n_out, n_in, seed)
+    return {"Q4_0": synth.gguf_q4_0, "Q8_0": synth.gguf_q8_0, "Q4_K": synth.gguf_q4_k, "Q5_K": synth.gguf_q5_k, "Q6_K": synth.gguf_q6_k, "MXFP4": synth.gguf_mxfp4}[name](n_out, n_in, seed)
 
 
 # 4352 columns = 34 steps of 128: K slices of 9 steps, so slices start inside a Q4_K super-block record; 1120 and 96
 # columns (Q8_0 only): a last step of one record, and of one block
 @pytest.mark.parametrize("name,n_out,n_in", [(k, n, c) for k in GGUF_KINDS for n, c in ((37, 1024), (256, 512), (200, 256), (130, 4352))]
-                         + [("Q8_0", 100, 96), ("Q8_0", 64, 1120), ("Q4_0", 100, 96), ("Q4_0", 64, 1120)])
+                         + [("Q8_0", 100, 96), ("Q8_0", 64, 1120), ("Q4_0", 100, 96), ("Q4_0", 64, 1120), ("MXFP4", 64, 1120)])
 def test_gemm_bf16_gguf_matches_oracle(be, oxref, name, n_out, n_in):
     """The GGUF formats on the bf16 matrix cores: within 2e-2 of the CPU's prefill product over the rows that
     dequantize_row yields (src/ggml.rs:630-793, src/kernels.rs:1998-2038), and 1e-3 of the same product with both

@@ -6,7 +6,7 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-Q4_0, Q8_0, Q4_K = 2, 8, 12
+Q4_0, Q8_0, Q4_K, MXFP4 = 2, 8, 12, 39
 
 
 @pytest.fixture(scope="module")
@@ -166,7 +166,7 @@ def test_moe_batched_equals_one_at_a_time(be, oxref, mlx_experts):
         assert np.array_equal(y1[0].view(np.uint32), y[i].view(np.uint32)), i
 
 
-@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K])
+@pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, MXFP4])
 def test_moe_gguf_experts(be, oxref, kind):
     from oxinfer_amd import synth
     ne, h, inter, k = 4, 256, 256, 2

@@ -5,7 +5,7 @@ tests state (src/kernels.rs:2484-2488, src/ggml.rs:1712-1747, :1904, src/cuda.rs
 import numpy as np
 import pytest
 
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+Q8_0, Q4_K, Q5_K, Q6_K, MXFP4 = 8, 12, 13, 14, 39
 
 
 def row_err(y, ref):
@@ -130,7 +130,7 @@ def gguf_f64(oxref, kind, data, n_out, n_in, x, t):
     return y, isums
 
 
-@pytest.mark.parametrize("kind", [Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("kind", [Q8_0, Q4_K, Q5_K, Q6_K, MXFP4])
 def test_gguf_decode_against_integer_brute_force_and_f64(oxref, kind):
     from oxinfer_amd import synth
     n_out, n_in, t = 12, 512, 3
@@ -177,7 +177,7 @@ def test_prefill_gemm_is_the_f64_product_of_the_dequantized_rows(oxref):
     ref = x.astype(np.float64) @ wf.astype(np.float64).T
     assert row_err(oxref.gemm_quant(-1, q, s16, off, n_out, n_in, x, t), ref) < 1e-4      # src/cuda.rs:1684-1685
     assert row_err(oxref.gemm_f32(wf, n_out, n_in, x, t), ref) < 1e-4
-    for kind in (Q8_0, Q4_K, Q5_K, Q6_K):
+    for kind in (Q8_0, Q4_K, Q5_K, Q6_K, MXFP4):
         data, _ = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 5)
         ref = x.astype(np.float64) @ oxref.dequantize_rows(kind, data, n_out, n_in).astype(np.float64).T
         assert row_err(oxref.gemm_quant(kind, data, None, None, n_out, n_in, x, t), ref) < 1e-4
