@@ -226,12 +226,12 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     auto load_step = [&](Step<FMT>& st, uint32_t s) {
         if constexpr (q8_format(FMT)) {
             const gbytes rec = base + (size_t)s * (FMT == FMT_Q8F ? T8F_REC : T8_REC);
-            st.w = gload<uint4>(rec + 16 * lane);
+            st.w = gload_once<uint4>(rec + 16 * lane);
             if (!ALDS) act2(2 * s + a_half, 8 * kq, st.a);
         } else if constexpr (k45_format(FMT)) {
             const gbytes rec = base + (size_t)(s >> 1) * K45_REC;
-            st.w = gload<uint4>(rec + (s & 1) * 1024 + 16 * lane);
-            if constexpr (FMT == FMT_Q5_K) st.h = gload<uint32_t>(rec + TK4_REC + (s & 1) * 256 + 4 * lane);
+            st.w = gload_once<uint4>(rec + (s & 1) * 1024 + 16 * lane);
+            if constexpr (FMT == FMT_Q5_K) st.h = gload_once<uint32_t>(rec + TK4_REC + (s & 1) * 256 + 4 * lane);
             if (!ALDS) {
                 act2(4 * s + a_half, 8 * kq, st.a);
                 act2(4 * s + 2 + a_half, 8 * kq, st.a + 2);
@@ -239,11 +239,11 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         } else if constexpr (FMT == FMT_Q6_K) {
             static_assert(FMT != FMT_Q6_K || ALDS, "Q6_K takes its activations from LDS");
             const gbytes rec = base + (size_t)s * T6K_REC;
-            st.w = gload<uint4>(rec + 16 * lane);
-            st.h = gload<uint2>(rec + 1024 + 8 * lane);
+            st.w = gload_once<uint4>(rec + 16 * lane);
+            st.h = gload_once<uint2>(rec + 1024 + 8 * lane);
         } else {
             const gbytes rec = base + (size_t)s * T4_REC;
-            st.w = gload<uint4>(rec + 16 * lane);
+            st.w = gload_once<uint4>(rec + 16 * lane);
             if (!ALDS) {
 #pragma unroll
                 for (int g = 0; g < 2; g++) {  // positions 4 kq.. and 16 + 4 kq.. of block 4 s + 2 g + half
@@ -265,26 +265,26 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     auto load_scales = [&](uint32_t* m, uint32_t first) {
         const uint32_t s = min(first + kq, slast);
         if constexpr (FMT == FMT_Q8F) {
-            m[0] = gload<uint32_t>(base + (size_t)s * T8F_REC + 1024 + 8 * n);
-            m[1] = gload<uint32_t>(base + (size_t)s * T8F_REC + 1028 + 8 * n);
+            m[0] = gload_once<uint32_t>(base + (size_t)s * T8F_REC + 1024 + 8 * n);
+            m[1] = gload_once<uint32_t>(base + (size_t)s * T8F_REC + 1028 + 8 * n);
         } else if constexpr (FMT == FMT_Q8_0) {
-            m[0] = gload<uint32_t>(base + (size_t)s * T8_REC + 1024 + 4 * n);
+            m[0] = gload_once<uint32_t>(base + (size_t)s * T8_REC + 1024 + 4 * n);
         } else if constexpr (k45_format(FMT)) {
             const gbytes rec = base + (size_t)(s >> 1) * K45_REC;
-            m[0] = gload<uint32_t>(rec + 2048 + 16 * n + 4 * (s & 1));
-            m[1] = gload<uint32_t>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
-            m[2] = gload<uint32_t>(rec + 2304 + 4 * n);
+            m[0] = gload_once<uint32_t>(rec + 2048 + 16 * n + 4 * (s & 1));
+            m[1] = gload_once<uint32_t>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
+            m[2] = gload_once<uint32_t>(rec + 2304 + 4 * n);
         } else if constexpr (FMT == FMT_Q6_K) {  // {scales of sub-blocks 0..3, of 4..7, d}
             const gbytes rec = base + (size_t)s * T6K_REC;
-            m[0] = gload<uint32_t>(rec + 1536 + 8 * n);
-            m[1] = gload<uint32_t>(rec + 1540 + 8 * n);
-            m[2] = gload<uint16_t>(rec + 1664 + 2 * n);
+            m[0] = gload_once<uint32_t>(rec + 1536 + 8 * n);
+            m[1] = gload_once<uint32_t>(rec + 1540 + 8 * n);
+            m[2] = gload_once<uint16_t>(rec + 1664 + 2 * n);
         } else if constexpr (FMT == FMT_MXFP4) {  // the four scale bytes of row n's blocks
-            m[0] = gload<uint32_t>(base + (size_t)s * T4X_REC + 1024 + 4 * n);
+            m[0] = gload_once<uint32_t>(base + (size_t)s * T4X_REC + 1024 + 4 * n);
         } else {
             const gbytes rec = base + (size_t)s * T4M_REC;
-            m[0] = gload<uint32_t>(rec + 1024 + 4 * n);
-            m[1] = gload<uint32_t>(rec + 1088 + 4 * n);
+            m[0] = gload_once<uint32_t>(rec + 1024 + 4 * n);
+            m[1] = gload_once<uint32_t>(rec + 1088 + 4 * n);
         }
     };
     const int take0 = (int)(4 * n);  // byte index of lane n for the lane-to-lane read; + 64 q: lane 16 q + n

@@ -281,9 +281,9 @@ __global__ __launch_bounds__(256) void pack_fp8_kernel(const uint8_t* __restrict
         a = src[0];
         b = src[1];
     }
-    uint4* out = reinterpret_cast<uint4*>(dst + rec * 2048 + 32 * l);
+    uint4* out = reinterpret_cast<uint4*>(dst + rec * 2048 + 16 * l);
     out[0] = a;
-    out[1] = b;
+    out[64] = b;
 }
 
 hipError_t launch_pack_fp8(const uint8_t* raw, size_t n_out, size_t n_in, uint8_t* dst, hipStream_t s) {

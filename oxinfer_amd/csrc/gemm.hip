@@ -250,7 +250,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
             } else {
                 const uint8_t* p = wbase[i] + (w.group == 1 ? 2048 : 128) * (size_t)s;
                 r[i].c = *reinterpret_cast<const uint4*>(p);
-                r[i].c2 = *reinterpret_cast<const uint4*>(p + 16);
+                r[i].c2 = *reinterpret_cast<const uint4*>(p + fp8_second_chunk(w));
                 r[i].m[0] = __float_as_uint(sbase[i][(128 * (step0 + s)) / w.bc]);
             }
         }

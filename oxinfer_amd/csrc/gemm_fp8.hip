@@ -125,6 +125,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
 #pragma unroll
     for (int i = 0; i < 2; i++) wrow[i] = w.p0 + fp8_offset(w, min((nt0 + 2 * wave + i) * 16 + n, w.n_out - 1), 32 * kq);
     const uint32_t wstep = w.group == 1 ? 2048 : 128;  // bytes between a lane's chunks of consecutive 128-column steps
+    const uint32_t whi = fp8_second_chunk(w);
     const uint4* abase[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) abase[i] = apk + ((size_t)min(mt0 + i, mtiles - 1) * all_kb * 64 + lane) * 2;
@@ -154,7 +155,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             r.v[i][0] = *reinterpret_cast<const u32x4*>(wrow[i] + col);
-            r.v[i][1] = *reinterpret_cast<const u32x4*>(wrow[i] + col + 16);
+            r.v[i][1] = *reinterpret_cast<const u32x4*>(wrow[i] + col + whi);
         }
     };
     auto store_w = [&](const WRegs& r, uint32_t buf) {
