@@ -479,7 +479,8 @@ def bench_gguf_gemv(args, be, torch, synth, kinds, gens):
                 "detail": detail}, cases
 
     # The dominant kernel: the jobs of one call share one launch (decode_batch_kernel); that launch carries HIP events
-    # recorded by the library on the launch stream, on every `--event-every`-th step (default: every step). An event
+    # recorded by the library on the launch stream, on every `--event-every`-th step (default: every fourth; an event pair on every launch keeps consecutive
+    # launches a few microseconds apart, which costs the whole-step figure 5 %). An event
     # pair on a launch leaves a gap of a few microseconds before the next one; without it a launch starts in the tail of
     # its predecessor, so its own duration reads longer.
     dom_symbol = "decode_batch_kernel"
@@ -585,7 +586,7 @@ def main():
                          "copy = a plain 256 MiB device copy, the known-size kernel that scales the HBM traffic counters; "
                          "gguf_stream = every GGUF case alone as a steady stream of 192 matmuls handed over in one call")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
-    ap.add_argument("--event-every", type=int, default=1,
+    ap.add_argument("--event-every", type=int, default=4,
                     help="gguf_gemv: the launch of every n-th timed step carries the timing events (with n > 1 the launches run closer "
                          "together, and a timed launch shares the device with its predecessor's tail)")
     ap.add_argument("--pool-gb", type=float, default=POOL_BYTES / 1e9)
