@@ -114,6 +114,7 @@ hipError_t launch_pack_a(const void* x, bool src_bf16, int mode, size_t t, size_
 namespace {
 
 
+typedef uint32_t u32x4g __attribute__((ext_vector_type(4)));
 constexpr int WG_NT = 8;   // row tiles per workgroup (128 rows)
 constexpr int AR = 4;      // blocks of A fragments held ahead (a whole K-step: two starve the FP8 shapes, whose activations do not stay in L2)
 
@@ -125,16 +126,25 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 }
 
 // Eight unsigned byte codes (the bytes of lo, then of hi) -> 8 bf16 of code * d + c.
+template <int K>
+__device__ __forceinline__ float byte_f32(uint32_t x) {  // byte K of x as f32: one conversion that selects the byte itself
+    float f;
+    if constexpr (K == 0) asm("v_cvt_f32_ubyte0_e32 %0, %1" : "=v"(f) : "v"(x));
+    else if constexpr (K == 1) asm("v_cvt_f32_ubyte1_e32 %0, %1" : "=v"(f) : "v"(x));
+    else if constexpr (K == 2) asm("v_cvt_f32_ubyte2_e32 %0, %1" : "=v"(f) : "v"(x));
+    else asm("v_cvt_f32_ubyte3_e32 %0, %1" : "=v"(f) : "v"(x));
+    return f;
+}
 __device__ __forceinline__ uint4 dequant_u8x8(uint32_t lo, uint32_t hi, float d, float c) {
     float f[8];
-    f[0] = __builtin_fmaf((float)(lo & 0xFF), d, c);
-    f[1] = __builtin_fmaf((float)((lo >> 8) & 0xFF), d, c);
-    f[2] = __builtin_fmaf((float)((lo >> 16) & 0xFF), d, c);
-    f[3] = __builtin_fmaf((float)(lo >> 24), d, c);
-    f[4] = __builtin_fmaf((float)(hi & 0xFF), d, c);
-    f[5] = __builtin_fmaf((float)((hi >> 8) & 0xFF), d, c);
-    f[6] = __builtin_fmaf((float)((hi >> 16) & 0xFF), d, c);
-    f[7] = __builtin_fmaf((float)(hi >> 24), d, c);
+    f[0] = __builtin_fmaf(byte_f32<0>(lo), d, c);
+    f[1] = __builtin_fmaf(byte_f32<1>(lo), d, c);
+    f[2] = __builtin_fmaf(byte_f32<2>(lo), d, c);
+    f[3] = __builtin_fmaf(byte_f32<3>(lo), d, c);
+    f[4] = __builtin_fmaf(byte_f32<0>(hi), d, c);
+    f[5] = __builtin_fmaf(byte_f32<1>(hi), d, c);
+    f[6] = __builtin_fmaf(byte_f32<2>(hi), d, c);
+    f[7] = __builtin_fmaf(byte_f32<3>(hi), d, c);
     return make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
 }
 // One dword of a T4M chunk (4 bytes of one block: low nibbles = elements 4 kq + i, high = 16 + 4 kq + i) -> the
@@ -156,7 +166,7 @@ template <int FMT, bool OUT_BF16, int NV>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint4* __restrict__ apk, uint32_t t, uint32_t mtiles,
                                                         void* __restrict__ yv) {
     extern __shared__ uint4 bfrag[];  // [2][4 blocks][8 row tiles][64 lanes]
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t n = lane & 15;
     const uint32_t all_steps = (w.n_in + 127) / 128, kblocks = 4 * all_steps;  // == t4m_steps(n_in)
     const uint32_t per_z = (all_steps + gridDim.z - 1) / gridDim.z;
@@ -191,7 +201,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     // A fragments of the wave's 4 token tiles (tiles past the end repeat the last one; their rows are not stored)
     const uint4* abase[NV];
 #pragma unroll
-    for (int i = 0; i < NV; i++) abase[i] = apk + ((size_t)min(mt0 + 4 * i, mtiles - 1) * kblocks + 4 * step0) * 64 + lane;
+    for (int i = 0; i < NV; i++) abase[i] = apk + ((size_t)min(mt0 + 4 * i, mtiles - 1) * kblocks + 4 * step0) * 64;  // (the same in every lane)
 
     f32x4 acc[NV][WG_NT];
 #pragma unroll
@@ -342,7 +352,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     };
     auto read_a = [&](uint4* dst, uint32_t blk) {  // the A fragments of block `blk` of this slice
 #pragma unroll
-        for (int i = 0; i < NV; i++) dst[i] = abase[i][(size_t)blk * 64];
+        for (int i = 0; i < NV; i++) {
+            // the block's base is the same in every lane: kept in scalar registers, the request takes it with the lane's 32-bit offset
+            const uint64_t pa = reinterpret_cast<uint64_t>(abase[i] + (size_t)blk * 64);
+            const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)pa), hi = __builtin_amdgcn_readfirstlane((uint32_t)(pa >> 32));
+            dst[i] = __builtin_bit_cast(uint4, reinterpret_cast<const __attribute__((address_space(1))) u32x4g*>(((uint64_t)hi << 32) | lo)[lane]);
+        }
     };
     // LDS traffic only: outstanding global loads (the prefetches) stay in flight across the barrier
     auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
