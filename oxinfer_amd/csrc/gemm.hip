@@ -6,10 +6,15 @@
 // (matmul_quant_block_prefill + gemm_8x8, src/kernels.rs:1998-2038, src/kernels_x86.rs:296-324 of the reference);
 // here weights and activations are rounded to bf16 first, so results agree to bf16 precision, not bit for bit.
 //
-// Work split: a workgroup of 4 waves owns 256 tokens x 128 weight rows; wave v owns the token tiles v, v + 4, v + 8,
-// v + 12 of the workgroup's sixteen and all 128 rows (4 x 8 MFMA tiles of 16 x 16, 128 accumulator registers). A
-// launch of at most 64 tokens gives each wave one token tile (64 tokens x 128 rows per workgroup).
-//   B (weights): each K-step of 128 the four waves dequantize the step's 8 row tiles (two each) from the packed
+// Work split: a workgroup of 8 waves (two per SIMD) owns 256 tokens x 128 weight rows; wave v owns the token tiles v
+// and v + 8 of the workgroup's sixteen and all 128 rows (2 x 8 MFMA tiles of 16 x 16, 64 accumulator registers). One
+// wave per SIMD issues a matrix instruction about every 30 cycles with this loop's vector, LDS and memory
+// instructions between them; a second wave fills the pipe while the first dequantizes, provided the two do not
+// dequantize at the same time: the waves 0-3 do so in a step's first block, the waves 4-7 in its second. Sharing the
+// token dimension keeps the activation requests at one per fragment and workgroup (sharing the rows instead would
+// request every fragment twice and run into the vector memory path's 64 bytes per cycle and CU). A
+// launch of at most 64 tokens runs 4 waves with one token tile each (64 tokens x 128 rows per workgroup).
+//   B (weights): each K-step of 128 the waves dequantize the step's 8 row tiles (one each; two each with 4 waves) from the packed
 //     records into bf16 MFMA fragments in LDS (double-buffered, one barrier per step); every wave then reads all
 //     8 x 4 fragments with ds_read_b128. A weight is dequantized once per workgroup: (code - 8) * d + offset in
 //     f32 as one fma(code, d, offset - 8 d), rounded to bf16. The GGUF formats likewise, from their own records:
@@ -162,28 +167,29 @@ __device__ __forceinline__ uint4 dequant_q4m(uint32_t w, float d, float c) {
 // FMT: FMT_Q4M (tile-packed MLX 4-bit), FMT_Q8_0 / FMT_Q8F / FMT_Q4_K / FMT_Q6_K (their tile records) or FMT_FP8 (e4m3 bytes with 128 x 128 block scales: the bytes are
 // exact in bf16, the block scale multiplies in f32 before the rounding, and a lane takes 32 consecutive row bytes
 // per step, which pack_a's mode 2 mirrors on the activation side).
-template <int FMT, bool OUT_BF16, int NV>
-__global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint4* __restrict__ apk, uint32_t t, uint32_t mtiles,
+template <int FMT, bool OUT_BF16, int NV, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, const uint4* __restrict__ apk, uint32_t t, uint32_t mtiles,
                                                         void* __restrict__ yv) {
     extern __shared__ uint4 bfrag[];  // [2][4 blocks][8 row tiles][64 lanes]
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t n = lane & 15;
+    constexpr int DT = WG_NT / WAVES;  // row tiles a wave dequantizes
     const uint32_t all_steps = (w.n_in + 127) / 128, kblocks = 4 * all_steps;  // == t4m_steps(n_in)
     const uint32_t per_z = (all_steps + gridDim.z - 1) / gridDim.z;
     const uint32_t step0 = blockIdx.z * per_z;              // this slice's K-steps: step0 .. step0 + nsteps
     const uint32_t nsteps = min(all_steps, step0 + per_z) - step0;
     const uint32_t ntiles = row_tiles(w.n_out);
     const uint32_t nt0 = blockIdx.x * WG_NT;               // first row tile of the workgroup
-    // the wave's token tiles: mt0, mt0 + 4, ... (NV of them: 4, or 1 when the whole launch has at most 64 tokens per
+    // the wave's token tiles: mt0, mt0 + WAVES, ... (NV of them: 2, or 1 when the whole launch has at most 64 tokens per
     // workgroup row, so that a few tokens do not pay for 256)
-    const uint32_t mt0 = blockIdx.y * (4 * NV) + wave;
+    const uint32_t mt0 = blockIdx.y * (WAVES * NV) + wave;
 
-    // the two row tiles this wave dequantizes
+    // the row tiles this wave dequantizes
     const uint8_t* wbase[2];
     const float* sbase[2] = {nullptr, nullptr};  // FP8: the block scales of the tile's rows
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const uint32_t tile = min(nt0 + 2 * wave + i, ntiles - 1);
+    for (int i = 0; i < DT; i++) {
+        const uint32_t tile = min(nt0 + DT * wave + i, ntiles - 1);
         if (t4m_format(FMT)) {
             wbase[i] = w.p0 + ((size_t)tile * all_steps + step0) * (FMT == FMT_MXFP4 ? T4X_REC : T4M_REC);
         } else if (q8_format(FMT)) {  // the tile's records; load_raw indexes them from the matrix's first step
@@ -198,10 +204,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
             sbase[i] = reinterpret_cast<const float*>(w.p1) + (size_t)(tile * 16 / w.br) * ((w.n_in + w.bc - 1) / w.bc);  // indexed by the absolute column block
         }
     }
-    // A fragments of the wave's 4 token tiles (tiles past the end repeat the last one; their rows are not stored)
+    // A fragments of the wave's token tiles (tiles past the end repeat the last one; their rows are not stored)
     const uint4* abase[NV];
 #pragma unroll
-    for (int i = 0; i < NV; i++) abase[i] = apk + ((size_t)min(mt0 + 4 * i, mtiles - 1) * kblocks + 4 * step0) * 64;  // (the same in every lane)
+    for (int i = 0; i < NV; i++) abase[i] = apk + ((size_t)min(mt0 + WAVES * i, mtiles - 1) * kblocks + 4 * step0) * 64;  // (the same in every lane)
 
     f32x4 acc[NV][WG_NT];
 #pragma unroll
@@ -267,11 +273,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     };
     auto load_raw = [&](Raw* r, uint32_t s) {
         load_raw_tile(r, 0, s);
-        load_raw_tile(r, 1, s);
+        if (DT == 2) load_raw_tile(r, 1, s);
     };
     // `s`: the step the records belong to (of this slice)
-    auto dequant_tile = [&](const Raw& r, int i, uint32_t buf, uint32_t s) {  // one of the wave's two row tiles, 4 blocks
-        uint4* dst = bfrag + ((size_t)(buf * 4) * WG_NT + 2 * wave + i) * 64 + lane;  // block b: + b * WG_NT * 64
+    auto dequant_tile = [&](const Raw& r, int i, uint32_t buf, uint32_t s) {  // one of the wave's row tiles, 4 blocks
+        uint4* dst = bfrag + ((size_t)(buf * 4) * WG_NT + DT * wave + i) * 64 + lane;  // block b: + b * WG_NT * 64
         if (FMT == FMT_MXFP4) {  // the code's doubled value + 12 as an unsigned byte, times the block's power of two: exact in bf16
             const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
@@ -367,19 +373,20 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
     // before they are dequantized into the other LDS buffer. Each fragment has one home, refilled in place right after
     // its last use.
     constexpr bool EARLY_RAW = OXHIP_GEMM_EARLY_RAW;
-    Raw raw[2];
+    Raw raw[DT];
     load_raw(raw, 0);
     uint4 a_cur[AR][NV], b_cur[WG_NT];
     const uint32_t last = nsteps - 1, last_blk = 4 * nsteps - 1;
 #pragma unroll
     for (int b = 0; b < AR; b++) read_a(a_cur[b], min((uint32_t)b, last_blk));
     dequant_tile(raw[0], 0, 0, 0);
-    dequant_tile(raw[1], 1, 0, 0);
+    if (DT == 2) dequant_tile(raw[DT - 1], 1, 0, 0);
     load_raw(raw, min(1u, last));
     lds_barrier();
     read_b(b_cur, 0, 0);
     // One K-step; every step does the same work, so that the loop is one body whose accumulators stay in place: the
-    // records of the next step are dequantized into the other LDS buffer during blocks 0 and 1, block 3 refills from
+    // records of the next step are dequantized into the other LDS buffer during blocks 0 and 1 (with 8 waves: block 0
+    // by the waves 0-3, block 1 by the waves 4-7, which share their SIMDs with them), block 3 refills from
     // that buffer after the barrier, and the step after next is requested during block 2. Past the end the indices
     // repeat the last step: a little work that nobody reads, instead of separate loop tails.
     for (uint32_t s = 0; s < nsteps; s++) {
@@ -397,14 +404,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
                 else b_cur[j] = bfrag[(((buf ^ 1) * 4) * WG_NT + j) * 64 + lane];
             }
             read_a(a_cur[b % AR], min(4 * s + b + AR, last_blk));
-            if (EARLY_RAW) {  // a tile's records of the step after next are requested as soon as its registers are free
+            if (DT == 1) {
+                if (b == (int)(wave >> 2)) {
+                    dequant_tile(raw[0], 0, buf ^ 1, min(s + 1, last));
+                    load_raw_tile(raw, 0, min(s + 2, last));
+                }
+            } else if (EARLY_RAW) {  // a tile's records of the step after next are requested as soon as its registers are free
                 if (b < 2) {
-                    dequant_tile(raw[b], b, buf ^ 1, min(s + 1, last));
+                    dequant_tile(raw[b < DT ? b : 0], b, buf ^ 1, min(s + 1, last));
                     load_raw_tile(raw, b, min(s + 2, last));
                 }
             } else {
                 if (b == 0) dequant_tile(raw[0], 0, buf ^ 1, min(s + 1, last));
-                if (b == 1) dequant_tile(raw[1], 1, buf ^ 1, min(s + 1, last));
+                if (b == 1) dequant_tile(raw[DT - 1], 1, buf ^ 1, min(s + 1, last));
                 if (b == 2) load_raw(raw, min(s + 2, last));
             }
         }
@@ -419,8 +431,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(WeightView w, const uint
             const uint32_t row = (nt0 + j) * 16 + n;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const uint32_t tok = (mt0 + 4 * i) * 16 + 4 * kq + r;
-                if (tok < t && row < w.n_out && mt0 + 4 * i < mtiles) {
+                const uint32_t tok = (mt0 + WAVES * i) * 16 + 4 * kq + r;
+                if (tok < t && row < w.n_out && mt0 + WAVES * i < mtiles) {
                     if (OUT_BF16) reinterpret_cast<uint16_t*>(yv)[(size_t)tok * w.n_out + row] = f32_to_bf16_bits(acc[i][j][r]);
                     else reinterpret_cast<float*>(yv)[(size_t)tok * w.n_out + row] = acc[i][j][r];
                 }
@@ -441,11 +453,13 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restric
 }
 
 // K slices for a launch: enough workgroups to cover the CUs while each keeps at least 8 steps.
-// Token tiles per wave: one when the launch has at most four (64 tokens), else four.
-static int gemm_nv(size_t mtiles) { return mtiles <= 4 ? 1 : 4; }
+// Token tiles per wave and waves per workgroup: one tile and four waves when the launch has at most four tiles (64 tokens),
+// else two tiles and eight waves.
+static int gemm_nv(size_t mtiles) { return mtiles <= 4 ? 1 : 2; }
+static int gemm_waves(size_t mtiles) { return mtiles <= 4 ? 4 : 8; }
 
 uint32_t gemm_k_slices(const WeightView& w, size_t mtiles) {
-    const uint32_t per_wg = 4 * gemm_nv(mtiles);
+    const uint32_t per_wg = gemm_waves(mtiles) * gemm_nv(mtiles);
     const uint32_t wgs = ((row_tiles(w.n_out) + WG_NT - 1) / WG_NT) * (uint32_t)((mtiles + per_wg - 1) / per_wg);
     const uint32_t steps = (w.n_in + 127) / 128;
     uint32_t z = 1;
@@ -465,20 +479,21 @@ namespace {
 template <int FMT, int NV>
 hipError_t run_gemm_bf16_nv(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                          hipStream_t s) {
+    constexpr int WAVES = NV == 1 ? 4 : 8;
     const uint32_t slices = gemm_k_slices(w, mtiles);
-    dim3 grid((row_tiles(w.n_out) + WG_NT - 1) / WG_NT, (unsigned)((mtiles + 4 * NV - 1) / (4 * NV)), slices);
+    dim3 grid((row_tiles(w.n_out) + WG_NT - 1) / WG_NT, (unsigned)((mtiles + WAVES * NV - 1) / (WAVES * NV)), slices);
     const size_t lds = 2 * 4 * WG_NT * 64 * 16;  // 64 KiB
     const bool direct_bf16 = out_bf16 && slices == 1;
     void* dst = slices > 1 ? static_cast<void*>(partial) : y;
     hipError_t e;
     if (direct_bf16) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, true, NV>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, true, NV, WAVES>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        gemm_bf16_kernel<FMT, true, NV><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
+        gemm_bf16_kernel<FMT, true, NV, WAVES><<<grid, 64 * WAVES, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
     } else {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, false, NV>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, false, NV, WAVES>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        gemm_bf16_kernel<FMT, false, NV><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
+        gemm_bf16_kernel<FMT, false, NV, WAVES><<<grid, 64 * WAVES, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
     }
     e = hipGetLastError();
     if (e != hipSuccess || slices == 1) return e;
@@ -491,7 +506,7 @@ template <int FMT>
 hipError_t run_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                          hipStream_t s) {
     if (gemm_nv(mtiles) == 1) return run_gemm_bf16_nv<FMT, 1>(w, apk, t, mtiles, y, out_bf16, partial, s);
-    return run_gemm_bf16_nv<FMT, 4>(w, apk, t, mtiles, y, out_bf16, partial, s);
+    return run_gemm_bf16_nv<FMT, 2>(w, apk, t, mtiles, y, out_bf16, partial, s);
 }
 }  // namespace
 
