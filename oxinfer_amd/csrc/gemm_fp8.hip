@@ -8,8 +8,9 @@
 // a whole scale block, and the two scales multiply that partial sum on its way into the f32 accumulator. Results
 // agree with the CPU to fp8-activation precision (the 2e-2 bar), not bit for bit.
 //
-// Work split as in gemm.hip: a workgroup of 4 waves owns 256 tokens x 128 rows (one row of scale blocks); per
-// K-block of 128 the four waves copy the 8 row tiles' bytes (2 KiB each, two tiles per wave) into LDS as MFMA
+// Work split as in gemm.hip: a workgroup of 8 waves owns 256 tokens x 128 rows (one row of scale blocks), each wave
+// two token tiles and all the rows; per
+// K-block of 128 the waves copy the 8 row tiles' bytes (2 KiB each, one tile per wave) into LDS as MFMA
 // fragments (lane = 16 kq + n holds row n's bytes 32 kq .. 32 kq + 31, which are contiguous in the row-major
 // weights, so no repacking at upload) and every wave reads all 8; activation fragments come packed from global
 // memory. K may be split over workgroups (gridDim.z) when the output is narrow.
@@ -101,12 +102,15 @@ hipError_t launch_quantize_act_fp8(const void* x, bool src_bf16, size_t t, size_
 }
 
 namespace {
-constexpr int F8_MT = 16;  // token tiles per workgroup (4 per wave)
+constexpr int F8_MT = 16;  // token tiles per workgroup
 constexpr int F8_NT = 8;   // row tiles per workgroup (128 rows = one scale block row)
+constexpr int F8_WAVES = 8;              // waves per workgroup: two per SIMD, so that one issues matrix instructions while the other scales and accumulates
+constexpr int F8_TW = F8_MT / F8_WAVES;  // token tiles per wave
+constexpr int F8_RW = F8_NT / F8_WAVES;  // row tiles whose bytes a wave copies
 }  // namespace
 
 template <bool OUT_BF16>
-__global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4* __restrict__ apk, const float* __restrict__ sx,
+__global__ __launch_bounds__(64 * F8_WAVES) void gemm_fp8_kernel(WeightView w, const uint4* __restrict__ apk, const float* __restrict__ sx,
                                                        uint32_t t, uint32_t mtiles, void* __restrict__ yv) {
     extern __shared__ uint4 bfrag[];  // [2][8 row tiles][2 halves][64 lanes]: a lane's two 16-byte halves lie a plane apart (no bank conflicts)
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -116,24 +120,24 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
     const uint32_t kb0 = blockIdx.z * per_z;
     const uint32_t nkb = min(all_kb, kb0 + per_z) - kb0;
     const uint32_t nt0 = blockIdx.x * F8_NT;
-    const uint32_t mt0 = blockIdx.y * F8_MT + wave * 4;
+    const uint32_t mt0 = blockIdx.y * F8_MT + wave * F8_TW;
     const uint32_t ncb = (w.n_in + w.bc - 1) / w.bc;
     const float* bs = reinterpret_cast<const float*>(w.p1);
 
     // the two row tiles whose bytes this wave copies: row pointers of this lane (rows past the end repeat the last)
-    const uint8_t* wrow[2];
+    const uint8_t* wrow[F8_RW];
 #pragma unroll
-    for (int i = 0; i < 2; i++) wrow[i] = w.p0 + fp8_offset(w, min((nt0 + 2 * wave + i) * 16 + n, w.n_out - 1), 32 * kq);
+    for (int i = 0; i < F8_RW; i++) wrow[i] = w.p0 + fp8_offset(w, min((nt0 + F8_RW * wave + i) * 16 + n, w.n_out - 1), 32 * kq);
     const uint32_t wstep = w.group == 1 ? 2048 : 128;  // bytes between a lane's chunks of consecutive 128-column steps
     const uint32_t whi = fp8_second_chunk(w);
-    const uint4* abase[4];
+    const uint4* abase[F8_TW];
 #pragma unroll
-    for (int i = 0; i < 4; i++) abase[i] = apk + ((size_t)min(mt0 + i, mtiles - 1) * all_kb * 64 + lane) * 2;
+    for (int i = 0; i < F8_TW; i++) abase[i] = apk + ((size_t)min(mt0 + i, mtiles - 1) * all_kb * 64 + lane) * 2;
     const uint32_t srow = min(nt0 * 16, w.n_out - 1) / w.br;  // the workgroup's 128 rows lie in one scale block row
 
-    f32x4 acc[4][F8_NT];
+    f32x4 acc[F8_TW][F8_NT];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < F8_TW; i++)
 #pragma unroll
         for (int j = 0; j < F8_NT; j++) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
@@ -141,11 +145,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
     // a condition, or a set reached through a pointer, ends up in scratch memory.
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     struct WRegs {
-        u32x4 v[2][2];
+        u32x4 v[F8_RW][2];
     };
     struct ARegs {
-        u32x4 v[4][2];
-        f32x4 sx[4];  // the activation scales of the lane's four tokens per tile
+        u32x4 v[F8_TW][2];
+        f32x4 sx[F8_TW];  // the activation scales of the lane's four tokens per tile
         float sw;     // the weight block's scale
     };
     // every request is unconditional and clamped to the last block: a request under a condition makes the compiler
@@ -153,15 +157,15 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
     auto load_w = [&](WRegs& r, uint32_t i_kb) {
         const size_t col = (size_t)wstep * (kb0 + min(i_kb, nkb - 1));
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < F8_RW; i++) {
             r.v[i][0] = *reinterpret_cast<const u32x4*>(wrow[i] + col);
             r.v[i][1] = *reinterpret_cast<const u32x4*>(wrow[i] + col + whi);
         }
     };
     auto store_w = [&](const WRegs& r, uint32_t buf) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            u32x4* dst = reinterpret_cast<u32x4*>(bfrag + (size_t)(buf * F8_NT + 2 * wave + i) * 128 + lane);
+        for (int i = 0; i < F8_RW; i++) {
+            u32x4* dst = reinterpret_cast<u32x4*>(bfrag + (size_t)(buf * F8_NT + F8_RW * wave + i) * 128 + lane);
             dst[0] = r.v[i][0];
             dst[64] = r.v[i][1];
         }
@@ -169,7 +173,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
     auto read_a = [&](ARegs& dst, uint32_t i_kb) {
         const uint32_t kb = kb0 + min(i_kb, nkb - 1);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < F8_TW; i++) {
             const u32x4* src = reinterpret_cast<const u32x4*>(abase[i] + (size_t)kb * 128);
             dst.v[i][0] = src[0];
             dst.v[i][1] = src[1];
@@ -179,7 +183,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
     };
     auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
-    // Software pipeline, three blocks deep in registers (one wave per SIMD: nothing else hides the latency). At block
+    // Software pipeline, three blocks deep in registers. At block
     // i (ring position P = i % 3): the weights of block i + 1 go from registers to the other LDS buffer and their
     // registers take the request for block i + 4; the matrix instructions run on activation set P and LDS buffer
     // i & 1; then set P takes the request for block i + 3.
@@ -199,9 +203,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
         const uint32_t buf = i_kb & 1;
         store_w(W[P1], buf ^ 1);  // the other buffer was last read a block ago, before the previous barrier
         load_w(W[P1], i_kb + 4);
-        float f[4][4];
+        float f[F8_TW][4];
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < F8_TW; i++)
 #pragma unroll
             for (int r = 0; r < 4; r++) f[i][r] = A[P].sx[i][r] * A[P].sw;
         // the matrix instruction of tile pair k + 1 is issued before the four multiply-adds that take tile pair k's
@@ -215,10 +219,10 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
         };
         read_b(0);
 #pragma unroll
-        for (int k = 0; k <= 4 * F8_NT; k++) {
-            const int j = k / 4, i = k % 4;
+        for (int k = 0; k <= F8_TW * F8_NT; k++) {
+            const int j = k / F8_TW, i = k % F8_TW;
             f32x4 d = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (k < 4 * F8_NT) {
+            if (k < F8_TW * F8_NT) {
                 if (i == 0 && j + 1 < F8_NT) read_b(j + 1);
                 const u32x4 b0 = bq[j & 1][0], b1 = bq[j & 1][1];
                 const v8i bb = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
@@ -228,7 +232,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
                 d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(aa, bb, z, 0, 0, 0, 127, 0, 127);
             }
             if (k > 0) {
-                const int jp = (k - 1) / 4, ip = (k - 1) % 4;
+                const int jp = (k - 1) / F8_TW, ip = (k - 1) % F8_TW;
 #pragma unroll
                 for (int r = 0; r < 4; r++) acc[ip][jp][r] = __builtin_fmaf(f[ip][r], dprev[r], acc[ip][jp][r]);
             }
@@ -251,7 +255,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_kernel(WeightView w, const uint4
 
     if (gridDim.z > 1) yv = reinterpret_cast<float*>(yv) + (size_t)blockIdx.z * t * w.n_out;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < F8_TW; i++) {
 #pragma unroll
         for (int j = 0; j < F8_NT; j++) {
             const uint32_t row = (nt0 + j) * 16 + n;
@@ -293,8 +297,8 @@ hipError_t launch_gemm_fp8(const WeightView& w, const void* apk, const float* sx
     const size_t lds = 2 * F8_NT * 64 * 32;  // 32 KiB
     const bool direct_bf16 = out_bf16 && slices == 1;
     void* dst = slices > 1 ? static_cast<void*>(partial) : y;
-    if (direct_bf16) gemm_fp8_kernel<true><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), sx, (uint32_t)t, (uint32_t)mtiles, dst);
-    else gemm_fp8_kernel<false><<<grid, 256, lds, s>>>(w, static_cast<const uint4*>(apk), sx, (uint32_t)t, (uint32_t)mtiles, dst);
+    if (direct_bf16) gemm_fp8_kernel<true><<<grid, 64 * F8_WAVES, lds, s>>>(w, static_cast<const uint4*>(apk), sx, (uint32_t)t, (uint32_t)mtiles, dst);
+    else gemm_fp8_kernel<false><<<grid, 64 * F8_WAVES, lds, s>>>(w, static_cast<const uint4*>(apk), sx, (uint32_t)t, (uint32_t)mtiles, dst);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || slices == 1) return e;
     const size_t n = t * (size_t)w.n_out;
