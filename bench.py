@@ -227,6 +227,34 @@ def timed_steps(torch, step, steps, warmup):
     return wall, float(np.mean([a.elapsed_time(b) for a, b in ev]))
 
 
+def timed_gemm_steps(be, torch, calls, steps, warmup):
+    """calls(i) -> the step's GEMM calls as (weight, x, kwargs). Two passes of W untimed and K timed steps: a plain one
+    for the wall time and the whole step by events around it, then one in which the library records events right
+    before and after each call's matrix kernel (their recording costs the stream a few microseconds per call, which is
+    why the first pass does without). Returns (wall seconds, mean milliseconds of a step, mean milliseconds of one
+    call's matrix kernel)."""
+    def step(i):
+        for w, x, kw in calls(i):
+            be.gemm(w, x, **kw)
+    wall, step_ms = timed_steps(torch, step, steps, warmup)
+    n = len(calls(0))
+    kev = [[(be.event(), be.event()) for _ in range(n)] for _ in range(steps)]
+    for i in range(steps):
+        for (w, x, kw), e in zip(calls(warmup + i), kev[i]):
+            be.gemm(w, x, events=e, **kw)
+    torch.cuda.synchronize()
+    kern_ms = float(np.mean([be.elapsed_ms(a, b) for row in kev for a, b in row]))
+    for row in kev:
+        for a, b in row:
+            be.lib.oxhip_event_destroy(a)
+            be.lib.oxhip_event_destroy(b)
+    return wall, step_ms, kern_ms
+
+
+GEMM_EVENTS = ("recorded by the library right before and after each call's matrix kernel (oxhip_dev_gemm_timed) in a second pass; "
+               "value, ms_per_step and call_us are the first pass's whole calls: activation packing or quantization + that kernel (+ K-slice sum)")
+
+
 def make_pool(make, nbytes, pool_gb):
     return [make() for _ in range(max(2, int(np.ceil(pool_gb * 1e9 / nbytes))))]
 
@@ -305,15 +333,13 @@ def bench_mlx_gemm(be, torch, synth, steps, warmup, variant_name):
         xs.append(torch.from_numpy(synth.activations(512, k, 4, bf16=True)).cuda().to(torch.bfloat16))
     flops = sum(2 * 512 * n * k for n, k in shapes)
 
-    def step(i):
-        for j in range(2):
-            be.gemm(ws[j][i % 4], xs[j], variant=variant)
-    wall, ms = timed_steps(torch, step, steps, warmup)
-    ach = flops / (ms * 1e-3) / 1e12
+    calls = lambda i: [(ws[j][i % 4], xs[j], {"variant": variant}) for j in range(2)]
+    wall, step_ms, ms = timed_gemm_steps(be, torch, calls, steps, warmup)
+    ach = flops / 2 / (ms * 1e-3) / 1e12
     peak = MFMA_PEAK[variant_name]
     roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4),
             "traffic": None, "kernel": "gemm_bf16_kernel<6, false, 2, 8>" if variant == 0 else "gemm_i8_q4m_kernel",
-            "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3 / 2, 2)}
+            "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3, 2), "call_us": round(step_ms * 1e3 / 2, 2)}
     if variant == 1:
         # one activation scale per token and block of 32: every int8 matrix instruction (16 x 16 x 32) is followed by a
         # conversion and a multiply-add per accumulator and the scale products, >= 8 VALU cycles-worth next to its 8:
@@ -322,7 +348,7 @@ def bench_mlx_gemm(be, torch, synth, steps, warmup, variant_name):
     return dict(base_line(steps, warmup), value=round(flops * steps / wall / 1e12, 2), unit="TFLOP/s", ms_per_step=round(wall / steps * 1e3, 5),
                 dtype="bf16" if variant == 0 else "int8",
                 config={"workload": f"configs[2]: MLX 4-bit g64 prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096, variant {variant_name}",
-                        "flops_per_step": flops, "events": "around the two calls of a step (activation packing + GEMM (+ K-slice sum))"},
+                        "flops_per_step": flops, "events": GEMM_EVENTS},
                 roofline=roof)
 
 
@@ -337,17 +363,15 @@ def bench_gguf_gemm(be, torch, synth, steps, warmup, fmt):
         xs.append(torch.from_numpy(synth.activations(512, k, 4, bf16=True)).cuda().to(torch.bfloat16))
     flops = sum(2 * 512 * n * k for n, k in shapes)
 
-    def step(i):
-        for j in range(2):
-            be.gemm(ws[j][i % 4], xs[j])
-    wall, ms = timed_steps(torch, step, steps, warmup)
-    ach = flops / (ms * 1e-3) / 1e12
+    calls = lambda i: [(ws[j][i % 4], xs[j], {}) for j in range(2)]
+    wall, step_ms, ms = timed_gemm_steps(be, torch, calls, steps, warmup)
+    ach = flops / 2 / (ms * 1e-3) / 1e12
     return dict(base_line(steps, warmup), value=round(flops * steps / wall / 1e12, 2), unit="TFLOP/s", ms_per_step=round(wall / steps * 1e3, 5), dtype="bf16",
                 config={"workload": f"GGUF {fmt.upper()} prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096 (bf16 matrix cores)",
-                        "flops_per_step": flops, "events": "around the two calls of a step (activation packing + GEMM (+ K-slice sum))"},
+                        "flops_per_step": flops, "events": GEMM_EVENTS},
                 roofline={"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK["bf16"], "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK["bf16"], 4),
                           "traffic": None, "kernel": f"gemm_bf16_kernel<{ {'q8_0': 1, 'q4_k': 2, 'q6_k': 3}[fmt]}, false, 2, 8>",
-                          "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3 / 2, 2)})
+                          "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3, 2), "call_us": round(step_ms * 1e3 / 2, 2)})
 
 
 def moe_experts(synth):
@@ -406,13 +430,19 @@ def bench_fp8(be, torch, synth, steps, warmup, pool_gb, m, variant_name, weights
     x32 = torch.from_numpy(synth.activations(m, k, 8, bf16=True)).cuda()
     xb = x32.to(torch.bfloat16)
     variant = {"bf16": 0, "fp8": 2}.get(variant_name, 0)
+    call_ms = None
     if m <= 16:
         step = lambda i: be.decode(ws[i % len(ws)], x=x32)
         kern = "skinny_fp8_kernel<*, 1, 2, *, false> (+ pack_skinny_kernel)"
-    else:
+        wall, ms = timed_steps(torch, step, steps, warmup)
+    elif m <= 32 and variant == 0:
         step = lambda i: be.gemm(ws[i % len(ws)], xb, variant=variant, out_bf16=True)
-        kern = ("skinny_fp8_kernel<4, 2, 1, 16, true> (+ pack_skinny_kernel, gemm_reduce_kernel)" if m <= 32 else "gemm_bf16_kernel<4, true, 2, 8>") if variant == 0 else "gemm_fp8_kernel<true>"
-    wall, ms = timed_steps(torch, step, steps, warmup)
+        kern = "skinny_fp8_kernel<4, 2, 1, 16, true> (+ pack_skinny_kernel, gemm_reduce_kernel)"
+        wall, ms = timed_steps(torch, step, steps, warmup)
+    else:
+        kern = "gemm_bf16_kernel<4, true, 2, 8>" if variant == 0 else "gemm_fp8_kernel<true>"
+        calls = lambda i: [(ws[i % len(ws)], xb, {"variant": variant, "out_bf16": True})]
+        wall, call_ms, ms = timed_gemm_steps(be, torch, calls, steps, warmup)
     flops, nbytes = 2 * m * n * k, n * k + scales.size * 4 + m * k * 2 + m * n * 2
     hbm = m <= 64
     ach = nbytes / (ms * 1e-3) / 1e9 if hbm else flops / (ms * 1e-3) / 1e12
@@ -420,9 +450,10 @@ def bench_fp8(be, torch, synth, steps, warmup, pool_gb, m, variant_name, weights
     return dict(base_line(steps, warmup), value=round((nbytes / 1e9 if hbm else flops / 1e12) * steps / wall, 2), unit="GB/s" if hbm else "TFLOP/s",
                 ms_per_step=round(wall / steps * 1e3, 5), dtype="fp8 weights, " + ("f32" if m <= 16 else ("bf16" if variant == 0 else "fp8")) + " activations",
                 config={"workload": f"configs[4]: FP8 E4M3 block-scaled GEMM [7168, 18432], M = {m}, variant {variant_name if m > 16 else 'decode'}",
-                        "bytes_per_step": nbytes, "flops_per_step": flops},
+                        "bytes_per_step": nbytes, "flops_per_step": flops, **({"events": GEMM_EVENTS} if call_ms is not None else {})},
                 roofline={"bound": "hbm" if hbm else "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "GB/s" if hbm else "TFLOP/s",
-                          "frac": round(ach / peak, 4), "traffic": None, "kernel": kern, "avg_launch_us": round(ms * 1e3, 2)})
+                          "frac": round(ach / peak, 4), "traffic": None, "kernel": kern, "avg_launch_us": round(ms * 1e3, 2),
+                          **({"call_us": round(call_ms * 1e3, 2)} if call_ms is not None else {})})
 
 
 def bench_gguf_gemv(args, be, torch, synth, kinds, gens):

@@ -220,6 +220,12 @@ enum { OXHIP_F32 = 0, OXHIP_BF16 = 1 };
 enum { OXHIP_GEMM_BF16 = 0, OXHIP_GEMM_I8 = 1, OXHIP_GEMM_FP8 = 2 };
 int oxhip_dev_gemm(oxhip_ctx* ctx, const oxhip_weight* w, const void* x, int x_dtype, size_t t, void* y, int y_dtype, int variant,
                    void* stream);
+/* oxhip_dev_gemm with two events (from oxhip_event_create; either may be NULL) recorded on `stream` right before and right
+ * after the variant's matrix kernel, i.e. after the activation packing or quantization launch and before the K-slice sum: the
+ * kernel's own duration as the device saw it, for measurement without a profiler (Backend::stats-style; no counterpart in
+ * the reference's trait). The FP8 skinny path (up to 32 tokens) counts its packing launch and its kernel as one. */
+int oxhip_dev_gemm_timed(oxhip_ctx* ctx, const oxhip_weight* w, const void* x, int x_dtype, size_t t, void* y, int y_dtype, int variant,
+                         void* stream, void* ev_start, void* ev_stop);
 /* The exact int32 block sums of the OXHIP_GEMM_I8 variant, [t, n_out, n_in/32], written by the GEMM kernel itself
  * (kernels_i8gemm's `block` accumulators, src/kernels_i8gemm.rs:249-334). For parity checks. */
 int oxhip_dev_gemm_isums(oxhip_ctx* ctx, const oxhip_weight* w, const void* x, int x_dtype, size_t t, int32_t* out, void* stream);

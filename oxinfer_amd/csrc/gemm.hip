@@ -486,6 +486,7 @@ hipError_t run_gemm_bf16_nv(const WeightView& w, const void* apk, size_t t, size
     const bool direct_bf16 = out_bf16 && slices == 1;
     void* dst = slices > 1 ? static_cast<void*>(partial) : y;
     hipError_t e;
+    span_start(s);
     if (direct_bf16) {
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, true, NV, WAVES>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
@@ -496,6 +497,7 @@ hipError_t run_gemm_bf16_nv(const WeightView& w, const void* apk, size_t t, size
         gemm_bf16_kernel<FMT, false, NV, WAVES><<<grid, 64 * WAVES, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
     }
     e = hipGetLastError();
+    span_stop(s);
     if (e != hipSuccess || slices == 1) return e;
     const size_t n = t * (size_t)w.n_out;
     if (out_bf16) gemm_reduce_kernel<true><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);

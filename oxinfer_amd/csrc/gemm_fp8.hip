@@ -297,9 +297,11 @@ hipError_t launch_gemm_fp8(const WeightView& w, const void* apk, const float* sx
     const size_t lds = 2 * F8_NT * 64 * 32;  // 32 KiB
     const bool direct_bf16 = out_bf16 && slices == 1;
     void* dst = slices > 1 ? static_cast<void*>(partial) : y;
+    span_start(s);
     if (direct_bf16) gemm_fp8_kernel<true><<<grid, 64 * F8_WAVES, lds, s>>>(w, static_cast<const uint4*>(apk), sx, (uint32_t)t, (uint32_t)mtiles, dst);
     else gemm_fp8_kernel<false><<<grid, 64 * F8_WAVES, lds, s>>>(w, static_cast<const uint4*>(apk), sx, (uint32_t)t, (uint32_t)mtiles, dst);
     hipError_t e = hipGetLastError();
+    span_stop(s);
     if (e != hipSuccess || slices == 1) return e;
     const size_t n = t * (size_t)w.n_out;
     if (out_bf16) gemm_fp8_reduce_kernel<true><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);

@@ -337,11 +337,13 @@ hipError_t launch_gemm_i8(const WeightView& w, const void* frag, const void* xs,
     const float2* x2 = static_cast<const float2*>(xs);
     const float* f1 = static_cast<const float*>(fs);
     const uint32_t tt = (uint32_t)t, ng = (uint32_t)ngrp;
+    span_start(s);
     switch (pick) {
         case 0: launch_tile<2, 8, 2>(grid, s, w, f, x2, f1, tt, ng, y, dump); break;
         case 1: launch_tile<2, 4, 1>(grid, s, w, f, x2, f1, tt, ng, y, dump); break;
         default: launch_tile<2, 2, 1>(grid, s, w, f, x2, f1, tt, ng, y, dump); break;
     }
+    span_stop(s);
     return hipGetLastError();
 }
 

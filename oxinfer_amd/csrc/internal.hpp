@@ -182,6 +182,18 @@ size_t skinny_fp8_pack_bytes(const WeightView& w, size_t t, int planes);
 hipError_t launch_skinny_fp8(const WeightView& w, const void* x, bool x_bf16, bool exact_f32, size_t t, void* y, bool y_bf16, void* pack,
                              hipStream_t s);
 hipError_t launch_gemm_reduce(const float* partial, size_t n, uint32_t slices, void* y, bool out_bf16, hipStream_t s);
+// Events a caller wants around the matrix kernel of the GEMM it is about to launch on this thread (oxhip_dev_gemm_timed): the
+// launchers record them right before and right after that kernel, inside the activation packing and the K-slice sum.
+struct KernelSpan {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+extern thread_local KernelSpan g_kernel_span;
+inline void span_start(hipStream_t s) {
+    if (g_kernel_span.start) (void)hipEventRecord(g_kernel_span.start, s);
+}
+inline void span_stop(hipStream_t s) {
+    if (g_kernel_span.stop) (void)hipEventRecord(g_kernel_span.stop, s);
+}
 void gemm_i8_geometry(const WeightView& w, size_t t, size_t* slots, size_t* ngrp);
 uint32_t gemm_i8_k_slices(const WeightView& w, size_t t);
 hipError_t launch_quantize_pack_i8(const void* x, bool src_bf16, size_t t, const WeightView& w, void* frag, void* xs, void* fs, hipStream_t s);

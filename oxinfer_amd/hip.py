@@ -91,6 +91,7 @@ def load_library():
         "oxhip_dev_isums": (C.c_int, [vp, vp, C.POINTER(QActC), vp, vp]),
         "oxhip_dev_decode_batch": (C.c_int, [vp, C.POINTER(DecodeJob), sz, vp]),
         "oxhip_dev_gemm": (C.c_int, [vp, vp, vp, C.c_int, sz, vp, C.c_int, C.c_int, vp]),
+        "oxhip_dev_gemm_timed": (C.c_int, [vp, vp, vp, C.c_int, sz, vp, C.c_int, C.c_int, vp, vp, vp]),
         "oxhip_dev_gemm_isums": (C.c_int, [vp, vp, vp, C.c_int, sz, vp, vp]),
         "oxhip_matvec_rows": (C.c_int, [vp, vp, sz, sz, C.POINTER(RowsJob), sz]),
         "oxhip_upload_moe": (vp, [vp, C.POINTER(WeightDesc), C.POINTER(WeightDesc), C.POINTER(WeightDesc), sz, sz, sz, C.c_uint32, C.c_float]),
@@ -468,14 +469,20 @@ class HipBackend:
     def elapsed_ms(self, a, b):
         return self.lib.oxhip_event_elapsed_ms(a, b)
 
-    def gemm(self, w, x, variant=0, out_bf16=False):
-        """Prefill GEMM on device tensors: x [t, n_in] f32 or bf16 -> y [t, n_out] f32 (or bf16)."""
+    def gemm(self, w, x, variant=0, out_bf16=False, events=None):
+        """Prefill GEMM on device tensors: x [t, n_in] f32 or bf16 -> y [t, n_out] f32 (or bf16). `events`: a pair from
+        event() that the library records right before and after the variant's matrix kernel."""
         import torch
         t = x.shape[0]
         y = torch.empty((t, w.n_out), dtype=torch.bfloat16 if out_bf16 else torch.float32, device=x.device)
         xd = 1 if x.dtype == torch.bfloat16 else 0
         assert x.dtype in (torch.bfloat16, torch.float32) and x.is_contiguous()
-        if not self.lib.oxhip_dev_gemm(self.ctx, w.handle, x.data_ptr(), xd, t, y.data_ptr(), int(out_bf16), variant, self._stream()):
+        if events is None:
+            ok = self.lib.oxhip_dev_gemm(self.ctx, w.handle, x.data_ptr(), xd, t, y.data_ptr(), int(out_bf16), variant, self._stream())
+        else:
+            ok = self.lib.oxhip_dev_gemm_timed(self.ctx, w.handle, x.data_ptr(), xd, t, y.data_ptr(), int(out_bf16), variant, self._stream(),
+                                               events[0], events[1])
+        if not ok:
             raise RuntimeError(self.last_error())
         return y
 

@@ -53,6 +53,32 @@ def test_gemm_bf16_matches_oracle(be, oxref, n_out, n_in):
         assert row_err(yb, ref) < 2e-2
 
 
+def test_gemm_timed_records_the_kernel_and_changes_nothing(be, oxref):
+    """oxhip_dev_gemm_timed: the same bytes as oxhip_dev_gemm for every variant, and the two events end up recorded in order
+    (a span inside the whole call's)."""
+    import torch
+    from oxinfer_amd import synth
+    raw, _ = mlx_case(oxref, 200, 1024, 11)
+    w = be.upload_mlx_q4(*raw, 64, 200, 1024)
+    data, scales = synth.fp8_e4m3(256, 512, 5)
+    wf = be.upload_fp8(data, scales, 256, 512)
+    for wt, variant, n_in in ((w, 0, 1024), (w, 1, 1024), (wf, 0, 512), (wf, 2, 512)):
+        for t in (20, 300):  # 300 tokens of 1024 columns: K slices, so the span ends before the slice sum
+            x = torch.from_numpy(synth.activations(t, n_in, 3 + t, bf16=True)).cuda().to(torch.bfloat16)
+            e0, e1 = be.event(), be.event()
+            o0, o1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            plain = be.gemm(wt, x, variant=variant)
+            o0.record()
+            timed = be.gemm(wt, x, variant=variant, events=(e0, e1))
+            o1.record()
+            torch.cuda.synchronize()
+            assert torch.equal(plain, timed), (variant, t)
+            span, whole = be.elapsed_ms(e0, e1), o0.elapsed_time(o1)
+            assert 0.0 < span <= whole + 0.02, (variant, t, span, whole)  # (two clocks' readings: 20 us of slack)
+            be.lib.oxhip_event_destroy(e0)
+            be.lib.oxhip_event_destroy(e1)
+
+
 def test_gemm_bf16_row_magnitudes_and_f32_inputs(be, oxref):
     """Token rows of magnitude 1e-3 / 1 / 300 / 2e5 (src/cuda.rs:1579-1581); f32 inputs are rounded to bf16."""
     import torch
