@@ -120,7 +120,7 @@ namespace {
 
 
 typedef uint32_t u32x4g __attribute__((ext_vector_type(4)));
-constexpr int WG_NT = 8;   // row tiles per workgroup (128 rows)
+constexpr int WG_NT = 8;   // row tiles per workgroup (128 rows), or 7 where that fills more CUs (gemm_row_tiles)
 constexpr int AR = 4;      // blocks of A fragments held ahead (a whole K-step: two starve the FP8 shapes, whose activations do not stay in L2)
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -167,19 +167,19 @@ __device__ __forceinline__ uint4 dequant_q4m(uint32_t w, float d, float c) {
 // FMT: FMT_Q4M (tile-packed MLX 4-bit), FMT_Q8_0 / FMT_Q8F / FMT_Q4_K / FMT_Q6_K (their tile records) or FMT_FP8 (e4m3 bytes with 128 x 128 block scales: the bytes are
 // exact in bf16, the block scale multiplies in f32 before the rounding, and a lane takes 32 consecutive row bytes
 // per step, which pack_a's mode 2 mirrors on the activation side).
-template <int FMT, bool OUT_BF16, int NV, int WAVES>
+template <int FMT, bool OUT_BF16, int NV, int WAVES, int NT>
 __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, const uint4* __restrict__ apk, uint32_t t, uint32_t mtiles,
                                                         void* __restrict__ yv) {
-    extern __shared__ uint4 bfrag[];  // [2][4 blocks][8 row tiles][64 lanes]
+    extern __shared__ uint4 bfrag[];  // [2][4 blocks][NT row tiles][64 lanes]
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t n = lane & 15;
-    constexpr int DT = WG_NT / WAVES;  // row tiles a wave dequantizes
+    constexpr int DT = (NT + WAVES - 1) / WAVES;  // row tiles a wave dequantizes (with NT = 7 the last wave has one fewer)
     const uint32_t all_steps = (w.n_in + 127) / 128, kblocks = 4 * all_steps;  // == t4m_steps(n_in)
     const uint32_t per_z = (all_steps + gridDim.z - 1) / gridDim.z;
     const uint32_t step0 = blockIdx.z * per_z;              // this slice's K-steps: step0 .. step0 + nsteps
     const uint32_t nsteps = min(all_steps, step0 + per_z) - step0;
     const uint32_t ntiles = row_tiles(w.n_out);
-    const uint32_t nt0 = blockIdx.x * WG_NT;               // first row tile of the workgroup
+    const uint32_t nt0 = blockIdx.x * NT;               // first row tile of the workgroup
     // the wave's token tiles: mt0, mt0 + WAVES, ... (NV of them: 2, or 1 when the whole launch has at most 64 tokens per
     // workgroup row, so that a few tokens do not pay for 256)
     const uint32_t mt0 = blockIdx.y * (WAVES * NV) + wave;
@@ -209,18 +209,18 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
 #pragma unroll
     for (int i = 0; i < NV; i++) abase[i] = apk + ((size_t)min(mt0 + WAVES * i, mtiles - 1) * kblocks + 4 * step0) * 64;  // (the same in every lane)
 
-    f32x4 acc[NV][WG_NT];
+    f32x4 acc[NV][NT];
 #pragma unroll
     for (int i = 0; i < NV; i++)
 #pragma unroll
-        for (int j = 0; j < WG_NT; j++) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
     struct Raw {
         uint4 c, c2;    // Q4M, Q4_K: one chunk; Q8: the chunks of the step's two records; Q6_K: low nibbles, high bit pairs; FP8: 32 row bytes
         uint32_t m[4];  // the row's scale words (Q4M: scales, offsets; FP8: the block scale's bits)
     };
     auto load_raw_tile = [&](Raw* r, int i, uint32_t s) {  // the records of the wave's row tile i at step s
-        {
+        if (NT % WAVES == 0 || DT * wave + i < NT) {  // (with NT = 7 the eighth wave has no tile)
             if (t4m_format(FMT)) {
                 const uint8_t* rec = wbase[i] + (size_t)s * (FMT == FMT_MXFP4 ? T4X_REC : T4M_REC);
                 r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
@@ -277,20 +277,21 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
     };
     // `s`: the step the records belong to (of this slice)
     auto dequant_tile = [&](const Raw& r, int i, uint32_t buf, uint32_t s) {  // one of the wave's row tiles, 4 blocks
-        uint4* dst = bfrag + ((size_t)(buf * 4) * WG_NT + DT * wave + i) * 64 + lane;  // block b: + b * WG_NT * 64
+        if (NT % WAVES != 0 && DT * wave + i >= NT) return;
+        uint4* dst = bfrag + ((size_t)(buf * 4) * NT + DT * wave + i) * 64 + lane;  // block b: + b * NT * 64
         if (FMT == FMT_MXFP4) {  // the code's doubled value + 12 as an unsigned byte, times the block's power of two: exact in bf16
             const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
             for (int b = 0; b < 4; b++) {
                 const float d = e8m0_half((r.m[0] >> (8 * b)) & 0xFF);
-                dst[b * WG_NT * 64] = dequant_u8x8(mxfp4_values<12>(cw[b] & 0x0F0F0F0Fu), mxfp4_values<12>((cw[b] >> 4) & 0x0F0F0F0Fu), d, -12.0f * d);
+                dst[b * NT * 64] = dequant_u8x8(mxfp4_values<12>(cw[b] & 0x0F0F0F0Fu), mxfp4_values<12>((cw[b] >> 4) & 0x0F0F0F0Fu), d, -12.0f * d);
             }
         } else if (FMT == FMT_Q40) {  // the block's own scale: word b / 2, half b % 2; (nib - 8) * d
             const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
             for (int b = 0; b < 4; b++) {
                 const float d = f16_bits_to_f32((uint16_t)((b & 1) ? r.m[b >> 1] >> 16 : r.m[b >> 1] & 0xFFFF));
-                dst[b * WG_NT * 64] = dequant_q4m(cw[b], d, -8.0f * d);
+                dst[b * NT * 64] = dequant_q4m(cw[b], d, -8.0f * d);
             }
         } else if (FMT == FMT_Q4M) {
             const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
@@ -299,7 +300,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
                 const int g = b >> 1;
                 const float d = f16_bits_to_f32((uint16_t)(g ? r.m[0] >> 16 : r.m[0] & 0xFFFF));
                 const float off = bf16_bits_to_f32((uint16_t)(g ? r.m[1] >> 16 : r.m[1] & 0xFFFF));
-                dst[b * WG_NT * 64] = dequant_q4m(cw[b], d, off - 8.0f * d);
+                dst[b * NT * 64] = dequant_q4m(cw[b], d, off - 8.0f * d);
             }
         } else if (q8_format(FMT)) {  // block b = 2 h + e: codes 8 kq .. + 7 of block e of record h; q * d as (q + 128) * d - 128 d
             const uint32_t cw[8] = {r.c.x, r.c.y, r.c.z, r.c.w, r.c2.x, r.c2.y, r.c2.z, r.c2.w};
@@ -309,7 +310,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
                 const int h = b >> 1, e = b & 1;
                 float d = FMT == FMT_Q8F ? __uint_as_float(r.m[b]) : f16_bits_to_f32((uint16_t)(e ? r.m[h] >> 16 : r.m[h] & 0xFFFF));
                 if (h && past) d = 0.0f;
-                dst[b * WG_NT * 64] = dequant_u8x8(cw[2 * b] ^ 0x80808080u, cw[2 * b + 1] ^ 0x80808080u, d, -128.0f * d);
+                dst[b * NT * 64] = dequant_u8x8(cw[2 * b] ^ 0x80808080u, cw[2 * b + 1] ^ 0x80808080u, d, -128.0f * d);
             }
         } else if (k45_format(FMT)) {  // block b = 2 jj + e: the low (e = 0) or high nibbles of the chunk's byte pair jj
             const float d = f16_bits_to_f32((uint16_t)(r.m[2] & 0xFFFF)), dmin = f16_bits_to_f32((uint16_t)(r.m[2] >> 16));
@@ -323,7 +324,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
                     w0 |= ((r.c2.x >> (2 * b)) & 0x01010101u) << 4;
                     w1 |= ((r.c2.x >> (2 * b + 1)) & 0x01010101u) << 4;
                 }
-                dst[b * WG_NT * 64] = dequant_u8x8(w0, w1, d * sc, -(dmin * mn));
+                dst[b * NT * 64] = dequant_u8x8(w0, w1, d * sc, -(dmin * mn));
             }
         } else if (FMT == FMT_Q6_K) {  // block b = 2 h + e: codes 8 e .. + 7 of the lane's 16 columns of half h
             const float d = f16_bits_to_f32((uint16_t)(r.m[2] & 0xFFFF));
@@ -335,7 +336,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
                 const uint32_t w0 = (src & 0x0F0F0F0Fu) | ((hh & 0x03030303u) << 4);
                 const uint32_t w1 = ((src >> 4) & 0x0F0F0F0Fu) | (((hh >> 2) & 0x03030303u) << 4);
                 const float dsc = d * (float)(int)(int8_t)((r.m[h] >> (8 * kq)) & 0xFF);
-                dst[b * WG_NT * 64] = dequant_u8x8(w0, w1, dsc, -32.0f * dsc);
+                dst[b * NT * 64] = dequant_u8x8(w0, w1, dsc, -32.0f * dsc);
             }
         } else {
             const uint32_t cw[8] = {r.c.x, r.c.y, r.c.z, r.c.w, r.c2.x, r.c2.y, r.c2.z, r.c2.w};
@@ -348,13 +349,13 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
                 const f32x2 v3 = __builtin_amdgcn_cvt_pk_f32_fp8((int)cw[2 * b + 1], true);
                 const uint32_t o[4] = {pack_bf16(v0.x * sc, v0.y * sc), pack_bf16(v1.x * sc, v1.y * sc),
                                        pack_bf16(v2.x * sc, v2.y * sc), pack_bf16(v3.x * sc, v3.y * sc)};
-                dst[b * WG_NT * 64] = make_uint4(o[0], o[1], o[2], o[3]);
+                dst[b * NT * 64] = make_uint4(o[0], o[1], o[2], o[3]);
             }
         }
     };
     auto read_b = [&](uint4* dst, uint32_t buf, uint32_t b) {
 #pragma unroll
-        for (int j = 0; j < WG_NT; j++) dst[j] = bfrag[((buf * 4 + b) * WG_NT + j) * 64 + lane];
+        for (int j = 0; j < NT; j++) dst[j] = bfrag[((buf * 4 + b) * NT + j) * 64 + lane];
     };
     auto read_a = [&](uint4* dst, uint32_t blk) {  // the A fragments of block `blk` of this slice
 #pragma unroll
@@ -375,7 +376,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
     constexpr bool EARLY_RAW = OXHIP_GEMM_EARLY_RAW;
     Raw raw[DT];
     load_raw(raw, 0);
-    uint4 a_cur[AR][NV], b_cur[WG_NT];
+    uint4 a_cur[AR][NV], b_cur[NT];
     const uint32_t last = nsteps - 1, last_blk = 4 * nsteps - 1;
 #pragma unroll
     for (int b = 0; b < AR; b++) read_a(a_cur[b], min((uint32_t)b, last_blk));
@@ -395,13 +396,13 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
         for (int b = 0; b < 4; b++) {
             if (b == 3) lds_barrier();  // the other buffer is complete, and nobody still reads this one
 #pragma unroll
-            for (int j = 0; j < WG_NT; j++) {
+            for (int j = 0; j < NT; j++) {
                 const bf16x8 bb = __builtin_bit_cast(bf16x8, b_cur[j]);
 #pragma unroll
                 for (int i = 0; i < NV; i++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a_cur[b % AR][i]), bb, acc[i][j], 0, 0, 0);
-                if (b < 3) b_cur[j] = bfrag[((buf * 4 + b + 1) * WG_NT + j) * 64 + lane];
-                else b_cur[j] = bfrag[(((buf ^ 1) * 4) * WG_NT + j) * 64 + lane];
+                if (b < 3) b_cur[j] = bfrag[((buf * 4 + b + 1) * NT + j) * 64 + lane];
+                else b_cur[j] = bfrag[(((buf ^ 1) * 4) * NT + j) * 64 + lane];
             }
             read_a(a_cur[b % AR], min(4 * s + b + AR, last_blk));
             if (DT == 1) {
@@ -427,7 +428,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
 #pragma unroll
     for (int i = 0; i < NV; i++) {
 #pragma unroll
-        for (int j = 0; j < WG_NT; j++) {
+        for (int j = 0; j < NT; j++) {
             const uint32_t row = (nt0 + j) * 16 + n;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
@@ -458,9 +459,9 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restric
 static int gemm_nv(size_t mtiles) { return mtiles <= 4 ? 1 : 2; }
 static int gemm_waves(size_t mtiles) { return mtiles <= 4 ? 4 : 8; }
 
-uint32_t gemm_k_slices(const WeightView& w, size_t mtiles) {
+static uint32_t k_slices_for(const WeightView& w, size_t mtiles, uint32_t nt) {
     const uint32_t per_wg = gemm_waves(mtiles) * gemm_nv(mtiles);
-    const uint32_t wgs = ((row_tiles(w.n_out) + WG_NT - 1) / WG_NT) * (uint32_t)((mtiles + per_wg - 1) / per_wg);
+    const uint32_t wgs = ((row_tiles(w.n_out) + nt - 1) / nt) * (uint32_t)((mtiles + per_wg - 1) / per_wg);
     const uint32_t steps = (w.n_in + 127) / 128;
     uint32_t z = 1;
     // (one token tile per wave: a K-step is short, two workgroups fit a CU, and what counts is requests in flight)
@@ -475,26 +476,38 @@ uint32_t gemm_k_slices(const WeightView& w, size_t mtiles) {
     return z;
 }
 
+// Row tiles per workgroup: 8, or 7 where that puts more workgroups on the 256 CUs without a second round of them or more
+// K slices (14336 rows x 512 tokens: 256 workgroups of 112 rows instead of 224 of 128, 62 -> 57 us).
+static int gemm_row_tiles(const WeightView& w, size_t mtiles) {
+    if (gemm_nv(mtiles) == 1) return WG_NT;
+    const uint32_t per_wg = gemm_waves(mtiles) * gemm_nv(mtiles), cols = (uint32_t)((mtiles + per_wg - 1) / per_wg);
+    const uint32_t z8 = k_slices_for(w, mtiles, 8), z7 = k_slices_for(w, mtiles, 7);
+    const uint32_t w8 = ((row_tiles(w.n_out) + 7) / 8) * cols * z8, w7 = ((row_tiles(w.n_out) + 6) / 7) * cols * z7;
+    return z7 == z8 && w7 <= 256 && w7 > w8 ? 7 : WG_NT;
+}
+
+uint32_t gemm_k_slices(const WeightView& w, size_t mtiles) { return k_slices_for(w, mtiles, (uint32_t)gemm_row_tiles(w, mtiles)); }
+
 namespace {
-template <int FMT, int NV>
+template <int FMT, int NV, int NT>
 hipError_t run_gemm_bf16_nv(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                          hipStream_t s) {
     constexpr int WAVES = NV == 1 ? 4 : 8;
     const uint32_t slices = gemm_k_slices(w, mtiles);
-    dim3 grid((row_tiles(w.n_out) + WG_NT - 1) / WG_NT, (unsigned)((mtiles + WAVES * NV - 1) / (WAVES * NV)), slices);
-    const size_t lds = 2 * 4 * WG_NT * 64 * 16;  // 64 KiB
+    dim3 grid((row_tiles(w.n_out) + NT - 1) / NT, (unsigned)((mtiles + WAVES * NV - 1) / (WAVES * NV)), slices);
+    const size_t lds = 2 * 4 * NT * 64 * 16;  // 64 KiB with 8 row tiles
     const bool direct_bf16 = out_bf16 && slices == 1;
     void* dst = slices > 1 ? static_cast<void*>(partial) : y;
     hipError_t e;
     span_start(s);
     if (direct_bf16) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, true, NV, WAVES>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, true, NV, WAVES, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        gemm_bf16_kernel<FMT, true, NV, WAVES><<<grid, 64 * WAVES, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
+        gemm_bf16_kernel<FMT, true, NV, WAVES, NT><<<grid, 64 * WAVES, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
     } else {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, false, NV, WAVES>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<FMT, false, NV, WAVES, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        gemm_bf16_kernel<FMT, false, NV, WAVES><<<grid, 64 * WAVES, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
+        gemm_bf16_kernel<FMT, false, NV, WAVES, NT><<<grid, 64 * WAVES, lds, s>>>(w, static_cast<const uint4*>(apk), (uint32_t)t, (uint32_t)mtiles, dst);
     }
     e = hipGetLastError();
     span_stop(s);
@@ -507,8 +520,9 @@ hipError_t run_gemm_bf16_nv(const WeightView& w, const void* apk, size_t t, size
 template <int FMT>
 hipError_t run_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                          hipStream_t s) {
-    if (gemm_nv(mtiles) == 1) return run_gemm_bf16_nv<FMT, 1>(w, apk, t, mtiles, y, out_bf16, partial, s);
-    return run_gemm_bf16_nv<FMT, 2>(w, apk, t, mtiles, y, out_bf16, partial, s);
+    if (gemm_nv(mtiles) == 1) return run_gemm_bf16_nv<FMT, 1, WG_NT>(w, apk, t, mtiles, y, out_bf16, partial, s);
+    if (gemm_row_tiles(w, mtiles) == 7) return run_gemm_bf16_nv<FMT, 2, 7>(w, apk, t, mtiles, y, out_bf16, partial, s);
+    return run_gemm_bf16_nv<FMT, 2, WG_NT>(w, apk, t, mtiles, y, out_bf16, partial, s);
 }
 }  // namespace
 
