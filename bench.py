@@ -338,7 +338,7 @@ def bench_mlx_gemm(be, torch, synth, steps, warmup, variant_name):
     ach = flops / 2 / (ms * 1e-3) / 1e12
     peak = MFMA_PEAK[variant_name]
     roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4),
-            "traffic": None, "kernel": "gemm_bf16_kernel<6, false, 2, 8>" if variant == 0 else "gemm_i8_q4m_kernel",
+            "traffic": None, "kernel": "gemm_bf16_kernel<6, false, 2, 8, 7|8>" if variant == 0 else "gemm_i8_q4m_kernel",
             "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3, 2), "call_us": round(step_ms * 1e3 / 2, 2)}
     if variant == 1:
         # one activation scale per token and block of 32: every int8 matrix instruction (16 x 16 x 32) is followed by a
@@ -370,7 +370,7 @@ def bench_gguf_gemm(be, torch, synth, steps, warmup, fmt):
                 config={"workload": f"GGUF {fmt.upper()} prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096 (bf16 matrix cores)",
                         "flops_per_step": flops, "events": GEMM_EVENTS},
                 roofline={"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK["bf16"], "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK["bf16"], 4),
-                          "traffic": None, "kernel": f"gemm_bf16_kernel<{ {'q8_0': 1, 'q4_k': 2, 'q6_k': 3}[fmt]}, false, 2, 8>",
+                          "traffic": None, "kernel": f"gemm_bf16_kernel<{ {'q8_0': 1, 'q4_k': 2, 'q6_k': 3}[fmt]}, false, 2, 8, 7|8>",
                           "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3, 2), "call_us": round(step_ms * 1e3 / 2, 2)})
 
 
@@ -440,7 +440,7 @@ def bench_fp8(be, torch, synth, steps, warmup, pool_gb, m, variant_name, weights
         kern = "skinny_fp8_kernel<4, 2, 1, 16, true> (+ pack_skinny_kernel, gemm_reduce_kernel)"
         wall, ms = timed_steps(torch, step, steps, warmup)
     else:
-        kern = "gemm_bf16_kernel<4, true, 2, 8>" if variant == 0 else "gemm_fp8_kernel<true>"
+        kern = "gemm_bf16_kernel<4, true, 2, 8, 7>" if variant == 0 else "gemm_fp8_kernel<true>"
         calls = lambda i: [(ws[i % len(ws)], xb, {"variant": variant, "out_bf16": True})]
         wall, call_ms, ms = timed_gemm_steps(be, torch, calls, steps, warmup)
     flops, nbytes = 2 * m * n * k, n * k + scales.size * 4 + m * k * 2 + m * n * 2
