@@ -32,7 +32,7 @@ def mlx_case(oxref, n_out, n_in, seed):
     return (wq, sc, bi), (q, s16, off)
 
 
-@pytest.mark.parametrize("n_out,n_in", [(37, 4160), (256, 512), (200, 64)])
+@pytest.mark.parametrize("n_out,n_in", [(37, 4160), (256, 512), (200, 64), (900, 384)])  # (900 rows past 64 tokens: 112-row workgroups, a ragged last one)
 def test_gemm_bf16_matches_oracle(be, oxref, n_out, n_in):
     import torch
     from oxinfer_amd import synth
