@@ -625,7 +625,7 @@ def main():
     ap.add_argument("--format", default="q4_k", choices=["q8_0", "q4_k", "q6_k"], help="weight format of the gguf_gemm workload")
     ap.add_argument("--tokens", type=int, default=0, help="tokens of the moe (1 or 256) and fp8 (1, 32, 1024) workloads")
     ap.add_argument("--moe-int8", action="store_true", help="moe: keep the integer kernels at every size (oxhip_moe_set_mode)")
-    ap.add_argument("--config-steps", type=int, default=40, help="all: timed steps of each per_config entry")
+    ap.add_argument("--config-steps", type=int, default=200, help="all: timed steps of each per_config entry")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1 (nothing here uses a second device)", file=sys.stderr)
