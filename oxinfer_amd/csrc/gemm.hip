@@ -476,14 +476,18 @@ static uint32_t k_slices_for(const WeightView& w, size_t mtiles, uint32_t nt) {
     return z;
 }
 
-// Row tiles per workgroup: 8, or 7 where that puts more workgroups on the 256 CUs without a second round of them or more
-// K slices (14336 rows x 512 tokens: 256 workgroups of 112 rows instead of 224 of 128, 62 -> 57 us).
+// Row tiles per workgroup: 8, or 7 where that costs less by this count: rounds of workgroups over the 256 CUs x row tiles
+// per workgroup x K-steps per slice (14336 rows x 512 tokens: one round of 256 workgroups of 112 rows instead of 224 of 128,
+// 63 -> 60 us; x 1024 tokens: two full rounds of 256 instead of 256 + 192).
 static int gemm_row_tiles(const WeightView& w, size_t mtiles) {
     if (gemm_nv(mtiles) == 1) return WG_NT;
     const uint32_t per_wg = gemm_waves(mtiles) * gemm_nv(mtiles), cols = (uint32_t)((mtiles + per_wg - 1) / per_wg);
-    const uint32_t z8 = k_slices_for(w, mtiles, 8), z7 = k_slices_for(w, mtiles, 7);
-    const uint32_t w8 = ((row_tiles(w.n_out) + 7) / 8) * cols * z8, w7 = ((row_tiles(w.n_out) + 6) / 7) * cols * z7;
-    return z7 == z8 && w7 <= 256 && w7 > w8 ? 7 : WG_NT;
+    const uint32_t steps = (w.n_in + 127) / 128;
+    auto cost = [&](uint32_t nt) {
+        const uint32_t z = k_slices_for(w, mtiles, nt), wgs = ((row_tiles(w.n_out) + nt - 1) / nt) * cols * z;
+        return (uint64_t)((wgs + 255) / 256) * nt * ((steps + z - 1) / z);
+    };
+    return cost(7) < cost(8) ? 7 : WG_NT;
 }
 
 uint32_t gemm_k_slices(const WeightView& w, size_t mtiles) { return k_slices_for(w, mtiles, (uint32_t)gemm_row_tiles(w, mtiles)); }
