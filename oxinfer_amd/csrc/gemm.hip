@@ -13,7 +13,8 @@
 // dequantize at the same time: the waves 0-3 do so in a step's first block, the waves 4-7 in its second. Sharing the
 // token dimension keeps the activation requests at one per fragment and workgroup (sharing the rows instead would
 // request every fragment twice and run into the vector memory path's 64 bytes per cycle and CU). A
-// launch of at most 64 tokens runs 4 waves with one token tile each (64 tokens x 128 rows per workgroup).
+// launch of at most 64 tokens runs 4 waves with one token tile each (64 tokens x 128 rows per workgroup), one of 65 to
+// 128 tokens 8 waves with one tile each (34 -> 27 us on the Llama-8B MLP shapes against two tiles per wave).
 //   B (weights): each K-step of 128 the waves dequantize the step's 8 row tiles (one each; two each with 4 waves) from the packed
 //     records into bf16 MFMA fragments in LDS (double-buffered, one barrier per step); every wave then reads all
 //     8 x 4 fragments with ds_read_b128. A weight is dequantized once per workgroup: (code - 8) * d + offset in
@@ -455,9 +456,9 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restric
 
 // K slices for a launch: enough workgroups to cover the CUs while each keeps at least 8 steps.
 // Token tiles per wave and waves per workgroup: one tile and four waves when the launch has at most four tiles (64 tokens),
-// else two tiles and eight waves.
-static int gemm_nv(size_t mtiles) { return mtiles <= 4 ? 1 : 2; }
-static int gemm_waves(size_t mtiles) { return mtiles <= 4 ? 4 : 8; }
+// one tile and eight waves up to eight tiles (128 tokens), else two tiles and eight waves.
+static int gemm_nv(size_t mtiles) { return mtiles <= 8 ? 1 : 2; }
+static int gemm_waves(size_t mtiles) { return mtiles <= 4 ? 4 : 8; }  // (5 to 8 token tiles: eight waves of one tile each)
 
 static uint32_t k_slices_for(const WeightView& w, size_t mtiles, uint32_t nt) {
     const uint32_t per_wg = gemm_waves(mtiles) * gemm_nv(mtiles);
@@ -493,10 +494,9 @@ static int gemm_row_tiles(const WeightView& w, size_t mtiles) {
 uint32_t gemm_k_slices(const WeightView& w, size_t mtiles) { return k_slices_for(w, mtiles, (uint32_t)gemm_row_tiles(w, mtiles)); }
 
 namespace {
-template <int FMT, int NV, int NT>
+template <int FMT, int NV, int NT, int WAVES = (NV == 1 ? 4 : 8)>
 hipError_t run_gemm_bf16_nv(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                          hipStream_t s) {
-    constexpr int WAVES = NV == 1 ? 4 : 8;
     const uint32_t slices = gemm_k_slices(w, mtiles);
     dim3 grid((row_tiles(w.n_out) + NT - 1) / NT, (unsigned)((mtiles + WAVES * NV - 1) / (WAVES * NV)), slices);
     const size_t lds = 2 * 4 * NT * 64 * 16;  // 64 KiB with 8 row tiles
@@ -524,7 +524,8 @@ hipError_t run_gemm_bf16_nv(const WeightView& w, const void* apk, size_t t, size
 template <int FMT>
 hipError_t run_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                          hipStream_t s) {
-    if (gemm_nv(mtiles) == 1) return run_gemm_bf16_nv<FMT, 1, WG_NT>(w, apk, t, mtiles, y, out_bf16, partial, s);
+    if (gemm_nv(mtiles) == 1 && gemm_waves(mtiles) == 4) return run_gemm_bf16_nv<FMT, 1, WG_NT>(w, apk, t, mtiles, y, out_bf16, partial, s);
+    if (gemm_nv(mtiles) == 1) return run_gemm_bf16_nv<FMT, 1, WG_NT, 8>(w, apk, t, mtiles, y, out_bf16, partial, s);
     if (gemm_row_tiles(w, mtiles) == 7) return run_gemm_bf16_nv<FMT, 2, 7>(w, apk, t, mtiles, y, out_bf16, partial, s);
     return run_gemm_bf16_nv<FMT, 2, WG_NT>(w, apk, t, mtiles, y, out_bf16, partial, s);
 }

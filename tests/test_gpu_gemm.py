@@ -41,7 +41,7 @@ def test_gemm_bf16_matches_oracle(be, oxref, n_out, n_in):
     assert w is not None, be.last_error()
     wf = oxref.dequant_rows_q4(q, s16, off, 64, n_out, n_in)
     wb = synth.bf16_round(wf).astype(np.float64)
-    for t in (1, 15, 16, 37, 64, 150, 300, 513):
+    for t in (1, 15, 16, 37, 64, 65, 100, 128, 150, 300, 513):  # (one token tile per wave up to 128 tokens, two past them)
         x = synth.activations(t, n_in, 100 + t, bf16=True)
         ref = oxref.gemm_quant(-1, q, s16, off, n_out, n_in, x, t)
         exact_bf16 = (x.astype(np.float64) @ wb.T).astype(np.float32)
@@ -115,7 +115,7 @@ def test_gemm_bf16_gguf_matches_oracle(be, oxref, name, n_out, n_in):
     w = be.upload_gguf(kind, raw, n_out, n_in)
     assert w is not None, be.last_error()
     wb = synth.bf16_round(oxref.dequantize_rows(kind, raw, n_out, n_in)).astype(np.float64)
-    for t in (1, 16, 37, 150, 300, 513):
+    for t in (1, 16, 37, 100, 150, 300, 513):
         x = synth.activations(t, n_in, 200 + t, bf16=True)
         ref = oxref.gemm_quant(kind, raw, None, None, n_out, n_in, x, t)
         exact_bf16 = (x.astype(np.float64) @ wb.T).astype(np.float32)
