@@ -443,15 +443,46 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
     }
 }
 
-// Adds the K slices in order: y = p[0] + p[1] + ... (f32 or bf16 out).
-template <bool OUT_BF16>
+// Adds the K slices in order: y = p[0] + p[1] + ... (f32 or bf16 out). VEC outputs per thread (4 when n is a multiple of 4 and
+// the buffers are 16-byte aligned).
+template <bool OUT_BF16, int VEC>
 __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restrict__ p, size_t n, uint32_t slices, void* __restrict__ yv) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     if (i >= n) return;
-    float v = p[i];
-    for (uint32_t z = 1; z < slices; z++) v += p[(size_t)z * n + i];
-    if (OUT_BF16) reinterpret_cast<uint16_t*>(yv)[i] = f32_to_bf16_bits(v);
-    else reinterpret_cast<float*>(yv)[i] = v;
+    float v[VEC];
+    if (VEC == 4) {
+        const float4 a = *reinterpret_cast<const float4*>(p + i);
+        v[0] = a.x; v[1 % VEC] = a.y; v[2 % VEC] = a.z; v[3 % VEC] = a.w;
+        for (uint32_t z = 1; z < slices; z++) {
+            const float4 b = *reinterpret_cast<const float4*>(p + (size_t)z * n + i);
+            v[0] += b.x; v[1 % VEC] += b.y; v[2 % VEC] += b.z; v[3 % VEC] += b.w;
+        }
+        if (OUT_BF16) {
+            *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(yv) + i) =
+                make_uint2(f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1 % VEC]) << 16),
+                           f32_to_bf16_bits(v[2 % VEC]) | ((uint32_t)f32_to_bf16_bits(v[3 % VEC]) << 16));
+        } else {
+            *reinterpret_cast<float4*>(reinterpret_cast<float*>(yv) + i) = make_float4(v[0], v[1 % VEC], v[2 % VEC], v[3 % VEC]);
+        }
+    } else {
+        v[0] = p[i];
+        for (uint32_t z = 1; z < slices; z++) v[0] += p[(size_t)z * n + i];
+        if (OUT_BF16) reinterpret_cast<uint16_t*>(yv)[i] = f32_to_bf16_bits(v[0]);
+        else reinterpret_cast<float*>(yv)[i] = v[0];
+    }
+}
+
+static void run_gemm_reduce(const float* partial, size_t n, uint32_t slices, void* y, bool out_bf16, hipStream_t s) {
+    const bool wide = n % 4 == 0 && reinterpret_cast<uintptr_t>(partial) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+    if (wide) {
+        const unsigned grid = (unsigned)((n / 4 + 255) / 256);
+        if (out_bf16) gemm_reduce_kernel<true, 4><<<grid, 256, 0, s>>>(partial, n, slices, y);
+        else gemm_reduce_kernel<false, 4><<<grid, 256, 0, s>>>(partial, n, slices, y);
+    } else {
+        const unsigned grid = (unsigned)((n + 255) / 256);
+        if (out_bf16) gemm_reduce_kernel<true, 1><<<grid, 256, 0, s>>>(partial, n, slices, y);
+        else gemm_reduce_kernel<false, 1><<<grid, 256, 0, s>>>(partial, n, slices, y);
+    }
 }
 
 // K slices for a launch: enough workgroups to cover the CUs while each keeps at least 8 steps.
@@ -516,9 +547,7 @@ hipError_t run_gemm_bf16_nv(const WeightView& w, const void* apk, size_t t, size
     e = hipGetLastError();
     span_stop(s);
     if (e != hipSuccess || slices == 1) return e;
-    const size_t n = t * (size_t)w.n_out;
-    if (out_bf16) gemm_reduce_kernel<true><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
-    else gemm_reduce_kernel<false><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
+    run_gemm_reduce(partial, t * (size_t)w.n_out, slices, y, out_bf16, s);
     return hipGetLastError();
 }
 template <int FMT>
@@ -533,8 +562,7 @@ hipError_t run_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t 
 
 hipError_t launch_gemm_reduce(const float* partial, size_t n, uint32_t slices, void* y, bool out_bf16, hipStream_t s) {
     if (!n) return hipSuccess;
-    if (out_bf16) gemm_reduce_kernel<true><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
-    else gemm_reduce_kernel<false><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
+    run_gemm_reduce(partial, n, slices, y, out_bf16, s);
     return hipGetLastError();
 }
 
