@@ -271,16 +271,6 @@ __global__ __launch_bounds__(64 * F8_WAVES) void gemm_fp8_kernel(WeightView w, c
     }
 }
 
-template <bool OUT_BF16>
-__global__ __launch_bounds__(256) void gemm_fp8_reduce_kernel(const float* __restrict__ p, size_t n, uint32_t slices, void* __restrict__ yv) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    float v = p[i];
-    for (uint32_t z = 1; z < slices; z++) v += p[(size_t)z * n + i];
-    if (OUT_BF16) reinterpret_cast<uint16_t*>(yv)[i] = f32_to_bf16_bits(v);
-    else reinterpret_cast<float*>(yv)[i] = v;
-}
-
 uint32_t gemm_fp8_k_slices(const WeightView& w, size_t mtiles) {
     const uint32_t wgs = ((row_tiles(w.n_out) + F8_NT - 1) / F8_NT) * (uint32_t)((mtiles + F8_MT - 1) / F8_MT);
     const uint32_t kbs = (w.n_in + 127) / 128;
@@ -303,10 +293,7 @@ hipError_t launch_gemm_fp8(const WeightView& w, const void* apk, const float* sx
     hipError_t e = hipGetLastError();
     span_stop(s);
     if (e != hipSuccess || slices == 1) return e;
-    const size_t n = t * (size_t)w.n_out;
-    if (out_bf16) gemm_fp8_reduce_kernel<true><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
-    else gemm_fp8_reduce_kernel<false><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(partial, n, slices, y);
-    return hipGetLastError();
+    return launch_gemm_reduce(partial, t * (size_t)w.n_out, slices, y, out_bf16, s);  // (the slices in order, as gemm.hip's)
 }
 
 }  // namespace oxhip
