@@ -423,9 +423,22 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     if (i >= (size_t)t * h) return;
     uint32_t tok = i / h, c = i % h;
     float acc = add ? y[i] : 0.0f;
-    for (uint32_t j = 0; j < k; j++) {
-        const float w = route_w[(size_t)tok * k + j];
-        acc = acc + w * o[(size_t)row_of[(size_t)tok * k + j] * h + c];
+    // eight routes at a time: their row numbers, then their values, are all requested before the first is added (one after
+    // the other, every route costs two dependent round trips to memory)
+    for (uint32_t j0 = 0; j0 < k; j0 += 8) {
+        uint32_t row[8];
+        float w[8], v[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const uint32_t j = min(j0 + e, k - 1);
+            row[e] = (uint32_t)row_of[(size_t)tok * k + j];
+            w[e] = route_w[(size_t)tok * k + j];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = o[(size_t)row[e] * h + c];
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            if (j0 + e < k) acc = acc + w[e] * v[e];
     }
     y[i] = acc;
 }
