@@ -250,8 +250,9 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_q4m_kernel(WeightView w, const
 }
 
 // Wave tiles on offer: {row tiles, token tiles, phases}. The pick spreads the (row tile, token tile) pairs evenly
-// over the 1024 SIMDs at two waves each: time goes as the pairs the busiest SIMD works through; larger tiles win ties
-// (fewer loads). Four row tiles per wave measured 1.6 to 2.5 times slower than two and are not offered.
+// over the 1024 SIMDs at two waves each: time goes as the pairs the busiest SIMD works through; smaller tiles win ties
+// (2 x 2 runs four waves per SIMD: 147 us per M = 512 shape against 160 with 2 x 8 and 168 with 2 x 4). Four row tiles per wave
+// measured 1.6 to 2.5 times slower than two, one row tile 1.2 to 1.3 times, and are not offered.
 struct Tile {
     uint32_t rt, tt, ph;
 };
@@ -271,7 +272,7 @@ int pick_tile(uint32_t ntiles, uint32_t ttiles) {
         const Tile& c = TILES[i];
         const uint64_t waves = (uint64_t)((ntiles + c.rt - 1) / c.rt) * ((ttiles + c.tt - 1) / c.tt);
         const uint64_t cost = ((waves + 2047) / 2048) * c.rt * c.tt;
-        if (cost < best_cost) {
+        if (cost <= best_cost) {  // ties go to the smaller tile: four waves per SIMD hide the operand requests' latency better than fewer loads do
             best_cost = cost;
             best = i;
         }
