@@ -143,6 +143,37 @@ def test_gemm_bf16_gguf_reference_fixtures(be, oxref):
         assert row_err(y, oxref.gemm_quant(kind, raw, None, None, n_out, n_in, x, t)) < 2e-2, kind
 
 
+def test_gemm_bf16_random_shapes_match_oracle(be, oxref):
+    """Seeded draws of (format, rows, columns, tokens) over the token counts where the launch changes shape (64 / 65, 128 /
+    129, 256 / 257, 512 / 513: one or two token tiles per wave, one or more token blocks) and row counts around the 112-
+    and 128-row workgroups, bf16 and f32 inputs, f32 and bf16 outputs: bf16 matrix-core bound (2e-2) against the oracle."""
+    import torch
+    from oxinfer_amd import synth
+    rng = np.random.default_rng(20251)
+    names = list(GGUF_KINDS) + ["MLX"]
+    for it in range(21):
+        name = names[it % len(names)]
+        n_out = int(rng.choice([33, 112, 113, 128, 257, 600, 897]))
+        t = int(rng.choice([17, 64, 65, 128, 129, 256, 257, 400, 512, 513]))
+        if name == "MLX":
+            n_in = int(rng.choice([64, 512, 1088, 4160]))
+            wq, sc, bi = synth.mlx_q4(n_out, n_in, 100 + it)
+            w = be.upload_mlx_q4(wq, sc, bi, 64, n_out, n_in)
+            q, s16, off = oxref.from_mlx_q4(wq, sc, bi, n_out, n_in, 64)
+            x = synth.activations(t, n_in, 200 + it, bf16=True)
+            ref = oxref.gemm_quant(-1, q, s16, off, n_out, n_in, x, t)
+        else:
+            n_in = int(rng.choice([256, 768, 4352])) if name in ("Q4_K", "Q5_K", "Q6_K") else int(rng.choice([96, 544, 1120, 4096]))
+            raw = gguf_raw(name, n_out, n_in, 100 + it)
+            w = be.upload_gguf(GGUF_KINDS[name], raw, n_out, n_in)
+            x = synth.activations(t, n_in, 200 + it, bf16=True)
+            ref = oxref.gemm_quant(GGUF_KINDS[name], raw, None, None, n_out, n_in, x, t)
+        assert w is not None, be.last_error()
+        for xd, ob in ((torch.from_numpy(x).cuda().to(torch.bfloat16), False), (torch.from_numpy(x).cuda(), True)):
+            y = be.gemm(w, xd, out_bf16=ob).float().cpu().numpy()
+            assert np.isfinite(y).all() and row_err(y, ref) < 2e-2, (name, n_out, n_in, t, xd.dtype, ob)
+
+
 @pytest.mark.parametrize("n_out,n_in", [(40, 640), (130, 96)])
 def test_gemm_bf16_q8_matrix_matches_oracle(be, oxref, n_out, n_in):
     """QMatrix (int8 codes, f32 scale per 32; src/quant.rs:128-133) through the same kernel."""
