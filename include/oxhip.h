@@ -185,8 +185,11 @@ int oxhip_dev_decode_noalloc(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_
  * NULL) are recorded before / after the launch that holds the job; for jobs that share a launch the first start and the
  * last stop event take the shared launch's own start and end as the device saw them.
  * The device-pointer entry points keep their scratch (partial rows of K slices, packed GEMM activations) per calling
- * stream, created on a stream's first call: calls on one stream are ordered and share it, calls on different streams
- * may overlap one another and the host-pointer surface. */
+ * stream: calls on one stream are ordered and share it, calls on different streams may overlap one another and the
+ * host-pointer surface. A stream's scratch is allocated when a call first needs it (hipMalloc: such a call cannot run
+ * under stream capture and may wait for the device): 16 MiB of partial rows + 2 MiB of counters with the stream's first
+ * decode launch whose shape slices K across workgroups (cleared by a kernel on that stream), the GEMMs' packed
+ * activations with its first GEMM. It stays until oxhip_stream_release or oxhip_close. */
 typedef struct {
     const oxhip_weight* w;
     const oxhip_qact* xa; /* quantized weights */
@@ -197,6 +200,10 @@ typedef struct {
     void* ev_stop;
 } oxhip_decode_job;
 int oxhip_dev_decode_batch(oxhip_ctx* ctx, const oxhip_decode_job* jobs, size_t n_jobs, void* stream);
+/* Frees the scratch the device-pointer entry points hold for `stream` (after waiting for the stream's work); a later call
+ * on that stream allocates it again. For callers that create and destroy streams: the scratch of a destroyed stream is
+ * otherwise kept until oxhip_close. No counterpart in the reference (its backends serialize on one stream). */
+int oxhip_stream_release(oxhip_ctx* ctx, void* stream);
 /* HIP events for timing launches on a stream (Backend::stats-style measurement without a profiler). */
 void* oxhip_event_create(void);
 void oxhip_event_destroy(void* ev);
@@ -261,6 +268,13 @@ int oxhip_buf_read(oxhip_ctx* ctx, void* dst_host, const void* src, size_t bytes
  * parallel): r is within an ulp or two of the CPU's, the quantization of v is bit-exact. */
 int oxhip_dev_rmsnorm_quantize(oxhip_ctx* ctx, const float* x, const float* w_f32, const uint16_t* w_bf16, float eps, size_t t, size_t n,
                                float* out, const oxhip_qact* q, void* stream);
+/* Op::Norm with all its fields (src/gpu_decode.rs:53-66; the CUDA form, src/cuda_decode.cu:314-327): `rows` rows of n
+ * values, x_stride / out_stride floats apart (0 = n): x' = x * pre, v = (x' * r) * w with r = (mean(x'^2) + eps)^(-1/2),
+ * out = v or, with `add`, out += v; what `out` then holds is also quantized into `q` (optional; rows of q are dense).
+ * oxhip_dev_rmsnorm_quantize is this call with pre = 1, no add and dense rows. Pointers and strides that are multiples
+ * of 16 bytes take 16-byte accesses, any others (`View`s are float offsets into the arena) one float at a time. */
+int oxhip_dev_norm(oxhip_ctx* ctx, const float* x, float* out, const float* w_f32, const uint16_t* w_bf16, float pre, size_t n, size_t rows,
+                   size_t x_stride, size_t out_stride, float eps, int add, const oxhip_qact* q, void* stream);
 /* Op::Linear with its LinMode (src/gpu_decode.rs:37-50, :67-77): y [t, n_out] f32 on the device, t <= 16.
  *   STORE      y  = W x
  *   ADD        y += W x                        (residual)
@@ -283,7 +297,9 @@ int oxhip_dev_route(oxhip_ctx* ctx, const float* x, const float* router, const f
                     float* logits, uint32_t* sel, const float* expert_scale, void* stream);
 /* Op::Experts (src/gpu_decode.rs:318-337): the routed experts chosen in `sel` (as oxhip_dev_route writes it) over
  * x [t, h]: y += (add) or y = the weighted sum of down_e(act(gate_e x) * up_e x), in route order. The activation
- * (SiLU / GELU-tanh) is the layer's (oxhip_upload_moe). */
+ * (SiLU / GELU-tanh) is the layer's (oxhip_upload_moe). k <= 32. The expert ids in `sel` are read on the device and
+ * cannot be checked by this call: every id must be below the layer's n_experts (oxhip_dev_route and
+ * oxhip_dev_moe_routed write only such ids). */
 int oxhip_dev_experts(oxhip_ctx* ctx, oxhip_moe* m, const float* x, size_t t, const uint32_t* sel, size_t k, float* y, int add, void* stream);
 
 /* Op::Route's top-k and Op::Experts in one call, for plans that keep the router's logits on the device: `logits`

@@ -1253,9 +1253,46 @@ void oxref_route_top_k(const float* logits, size_t n, size_t k, uint32_t* idx, f
 // zero), so the result of the batched / grouped schedules equals running each (token, route) pair
 // on its own, which is what this does; the combine is an unfused y += w * o in route order.
 // ---------------------------------------------------------------------------------------------
-void oxref_moe_q4(const oxref_q4_ref* gate_up, const oxref_q4_ref* down, size_t ne, size_t group,
-                  size_t h, size_t inter, const float* x, size_t t, const uint32_t* route_idx,
-                  const float* route_w, size_t k, float* y, int decode_path) {
+// Act::apply (src/moe.rs:18-37) of n pairs in place: kind 0 SiLU (silu_mul), 1 GELU-tanh (gelu_mul, gelu_tanh
+// src/kernels.rs:2233-2239: both through fast_exp), 2 SiLU with DeepSeek V4's clamp `param` (gate min, up clamp, then
+// silu_mul).
+void oxref_act_apply(uint32_t kind, float param, float* g, const float* u, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        float x = g[i], b = u[i];
+        if (kind == 1) {
+            const float K2 = 2.0f * 0.7978846f;
+            float t = K2 * (x + 0.044715f * x * x * x);
+            g[i] = x / (1.0f + oxref_fast_exp(-t)) * b;
+            continue;
+        }
+        if (kind == 2) {
+            x = std::fmin(x, param);
+            b = std::fmin(std::fmax(b, -param), param);
+        }
+        g[i] = x / (1.0f + oxref_fast_exp(-x)) * b;
+    }
+}
+
+// Act::scalar (src/moe.rs:39-46), what the grouped prefill path applies: libm's exp for the SiLU kinds, gelu_tanh
+// (fast_exp) for GELU.
+float oxref_act_scalar(uint32_t kind, float param, float g, float u) {
+    if (kind == 1) {
+        const float K2 = 2.0f * 0.7978846f;
+        float t = K2 * (g + 0.044715f * g * g * g);
+        return g / (1.0f + oxref_fast_exp(-t)) * u;
+    }
+    if (kind == 2) {
+        g = std::fmin(g, param);
+        u = std::fmin(std::fmax(u, -param), param);
+    }
+    return g / (1.0f + std::exp(-g)) * u;
+}
+
+// `up` == nullptr: gate_up[e] is the fused [2 inter, h] matrix (gate rows, then up rows); else gate_up[e] is the gate
+// [inter, h] and up[e] the up projection [inter, h] (src/gpu.rs:206-216).
+void oxref_moe_q4_act(const oxref_q4_ref* gate_up, const oxref_q4_ref* up, const oxref_q4_ref* down, size_t ne, size_t group,
+                      size_t h, size_t inter, const float* x, size_t t, const uint32_t* route_idx,
+                      const float* route_w, size_t k, float* y, int decode_path, uint32_t act_kind, float act_param) {
     int threads = oxref_hw_threads();
     // expert -> (token, slot) pairs
     std::vector<std::vector<std::pair<size_t, size_t>>> by(ne);
@@ -1265,26 +1302,41 @@ void oxref_moe_q4(const oxref_q4_ref* gate_up, const oxref_q4_ref* down, size_t 
     pool(threads).run(ne, [&](size_t e) {
         size_t n = by[e].size();
         if (!n) return;
-        std::vector<float> xs(n * h), gu(n * 2 * inter), a(n * inter), o(n * h);
+        std::vector<float> xs(n * h), g(n * inter), u(n * inter), a(n * inter), o(n * h);
         for (size_t i = 0; i < n; i++) std::memcpy(&xs[i * h], x + by[e][i].first * h, h * 4);
-        if (decode_path) {
-            oxref_q4_decode(gate_up[e].q, gate_up[e].sc, gate_up[e].off, group, 2 * inter, h, xs.data(), n, gu.data(), nullptr);
-            // decode output is [n][2*inter]? No: y is [t][n_out], i.e. row-major per token.
+        // the gate and up products as [n][inter] each
+        auto split = [&](const std::vector<float>& gu) {
             for (size_t i = 0; i < n; i++) {
-                float* g = &gu[i * 2 * inter];
-                oxref_silu_mul(g, g + inter, inter);
-                std::memcpy(&a[i * inter], g, inter * 4);
+                std::memcpy(&g[i * inter], &gu[i * 2 * inter], inter * 4);
+                std::memcpy(&u[i * inter], &gu[i * 2 * inter + inter], inter * 4);
             }
+        };
+        if (decode_path) {
+            if (!up) {
+                std::vector<float> gu(n * 2 * inter);
+                oxref_q4_decode(gate_up[e].q, gate_up[e].sc, gate_up[e].off, group, 2 * inter, h, xs.data(), n, gu.data(), nullptr);
+                split(gu);
+            } else {
+                oxref_q4_decode(gate_up[e].q, gate_up[e].sc, gate_up[e].off, group, inter, h, xs.data(), n, g.data(), nullptr);
+                oxref_q4_decode(up[e].q, up[e].sc, up[e].off, group, inter, h, xs.data(), n, u.data(), nullptr);
+            }
+            oxref_act_apply(act_kind, act_param, g.data(), u.data(), n * inter);
+            a = g;
             oxref_q4_decode(down[e].q, down[e].sc, down[e].off, group, h, inter, a.data(), n, o.data(), nullptr);
         } else {
-            std::vector<float> wf(2 * inter * h);
-            oxref_dequant_rows_q4(gate_up[e].q, gate_up[e].sc, gate_up[e].off, group, h, 0, 2 * inter, wf.data());
-            oxref_gemm_f32(wf.data(), 2 * inter, h, xs.data(), n, gu.data(), 1);
-            for (size_t i = 0; i < n; i++)
-                for (size_t j = 0; j < inter; j++) {
-                    float g = gu[i * 2 * inter + j], u = gu[i * 2 * inter + inter + j];
-                    a[i * inter + j] = g / (1.0f + std::exp(-g)) * u;
-                }
+            const size_t gr = up ? inter : 2 * inter;
+            std::vector<float> wf(gr * h);
+            oxref_dequant_rows_q4(gate_up[e].q, gate_up[e].sc, gate_up[e].off, group, h, 0, gr, wf.data());
+            if (!up) {
+                std::vector<float> gu(n * 2 * inter);
+                oxref_gemm_f32(wf.data(), 2 * inter, h, xs.data(), n, gu.data(), 1);
+                split(gu);
+            } else {
+                oxref_gemm_f32(wf.data(), inter, h, xs.data(), n, g.data(), 1);
+                oxref_dequant_rows_q4(up[e].q, up[e].sc, up[e].off, group, h, 0, inter, wf.data());
+                oxref_gemm_f32(wf.data(), inter, h, xs.data(), n, u.data(), 1);
+            }
+            for (size_t i = 0; i < n * inter; i++) a[i] = oxref_act_scalar(act_kind, act_param, g[i], u[i]);
             wf.resize(h * inter);
             oxref_dequant_rows_q4(down[e].q, down[e].sc, down[e].off, group, inter, 0, h, wf.data());
             oxref_gemm_f32(wf.data(), h, inter, a.data(), n, o.data(), 1);
@@ -1298,6 +1350,12 @@ void oxref_moe_q4(const oxref_q4_ref* gate_up, const oxref_q4_ref* down, size_t 
             const float* o = &outs[(ti * k + j) * h];
             for (size_t i = 0; i < h; i++) y[ti * h + i] += w * o[i];
         }
+}
+
+void oxref_moe_q4(const oxref_q4_ref* gate_up, const oxref_q4_ref* down, size_t ne, size_t group,
+                  size_t h, size_t inter, const float* x, size_t t, const uint32_t* route_idx,
+                  const float* route_w, size_t k, float* y, int decode_path) {
+    oxref_moe_q4_act(gate_up, nullptr, down, ne, group, h, inter, x, t, route_idx, route_w, k, y, decode_path, 0, 0.0f);
 }
 
 // The decode-sized MoE pass as the x86 CPU schedules it, for the timed baseline (values as oxref_moe_q4's decode

@@ -16,6 +16,7 @@
  *   integer dot products ........ brute force; power-of-two scales make the f32 math exact
  *   decode / prefill / MoE ...... f64 definitions (src/ggml.rs:1712-1747, src/cuda.rs:2145-2179)
  *   route_top_k ................. equals full softmax -> top-k -> renormalize
+ *   act_apply / act_scalar ...... torch's silu, gelu(approximate="tanh") and clamp in f64 (to fast_exp's 3e-7)
  * Parity unpinned (only running the reference could fix these bit for bit; the parity contract
  * does not need them): the f32 summation order of the AVX2 Q4 kernel and of dot_bf16 inside
  * add_offsets, fast_exp's exact output bits, libm expf.
@@ -110,6 +111,16 @@ typedef struct {
 void oxref_moe_q4(const oxref_q4_ref* gate_up, const oxref_q4_ref* down, size_t ne, size_t group,
                   size_t h, size_t inter, const float* x, size_t t, const uint32_t* route_idx,
                   const float* route_w, size_t k, float* y, int decode_path);
+
+/* Act::apply (src/moe.rs:18-37) in place over n pairs, and Act::scalar (src/moe.rs:39-46). kind: 0 SiLU, 1 GELU-tanh,
+ * 2 SiLU with the clamp `param`. */
+void  oxref_act_apply(uint32_t kind, float param, float* g, const float* u, size_t n);
+float oxref_act_scalar(uint32_t kind, float param, float g, float u);
+/* oxref_moe_q4 with the layer's activation and, with `up` != NULL, split gate / up experts (gate_up[e] = the gate
+ * [inter, h], up[e] = [inter, h]; src/gpu.rs:206-216). */
+void oxref_moe_q4_act(const oxref_q4_ref* gate_up, const oxref_q4_ref* up, const oxref_q4_ref* down, size_t ne, size_t group,
+                      size_t h, size_t inter, const float* x, size_t t, const uint32_t* route_idx,
+                      const float* route_w, size_t k, float* y, int decode_path, uint32_t act_kind, float act_param);
 
 /* The decode-sized pass scheduled and vectorized as the x86 CPU does it (timed baseline). */
 void oxref_moe_q4_avx2(const oxref_q4_ref* gate_up, const oxref_q4_ref* down, size_t ne, size_t group,

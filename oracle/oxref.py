@@ -62,6 +62,9 @@ def _load():
         "oxref_silu_mul": (None, [vp, vp, sz]),
         "oxref_route_top_k": (None, [vp, sz, sz, vp, vp]),
         "oxref_moe_q4": (None, [vp, vp, sz, sz, sz, sz, vp, sz, vp, vp, sz, vp, C.c_int]),
+        "oxref_act_apply": (None, [C.c_uint32, C.c_float, vp, vp, sz]),
+        "oxref_act_scalar": (C.c_float, [C.c_uint32, C.c_float, C.c_float, C.c_float]),
+        "oxref_moe_q4_act": (None, [vp, vp, vp, sz, sz, sz, sz, vp, sz, vp, vp, sz, vp, C.c_int, C.c_uint32, C.c_float]),
         "oxref_moe_q4_avx2": (None, [vp, vp, sz, sz, sz, sz, vp, sz, vp, vp, sz, vp, C.c_int]),
         "oxref_hw_threads": (C.c_int, []),
     }
@@ -277,6 +280,19 @@ def silu_mul(a, b):
     return a
 
 
+def act_apply(kind, param, g, u):
+    """Act::apply (src/moe.rs:18-37): act(g) * u elementwise; kind 0 SiLU, 1 GELU-tanh, 2 SiLU with clamp `param`."""
+    g = np.array(g, np.float32, copy=True)
+    u = _c(u, np.float32)
+    lib.oxref_act_apply(kind, float(param), _p(g), _p(u), g.size)
+    return g
+
+
+def act_scalar(kind, param, g, u):
+    """Act::scalar (src/moe.rs:39-46) of one pair."""
+    return lib.oxref_act_scalar(kind, float(param), float(g), float(u))
+
+
 def route_top_k(logits, k):
     logits = _c(logits, np.float32)
     idx = np.empty(k, np.uint32)
@@ -289,9 +305,10 @@ class _Q4Ref(C.Structure):
     _fields_ = [("q", C.c_void_p), ("sc", C.c_void_p), ("off", C.c_void_p)]
 
 
-def moe_q4(gate_up, down, group, h, inter, x, t, route_idx, route_w, y, decode_path, avx2=False, threads=None):
+def moe_q4(gate_up, down, group, h, inter, x, t, route_idx, route_w, y, decode_path, avx2=False, threads=None, up=None, act=0, act_param=0.0):
     """gate_up / down: lists of (q, sc, off) numpy triples per expert. Adds into y ([t, h] f32) and returns it.
-    avx2: the decode path scheduled and vectorized as the x86 CPU runs it (the timed baseline)."""
+    avx2: the decode path scheduled and vectorized as the x86 CPU runs it (the timed baseline). up: split experts
+    (gate_up then holds the gates). act / act_param: the layer's MoeAct (0 SiLU, 1 GELU-tanh, 2 SiLU clamp)."""
     ne = len(gate_up)
     keep = []
 
@@ -304,6 +321,7 @@ def moe_q4(gate_up, down, group, h, inter, x, t, route_idx, route_w, y, decode_p
         return arr
 
     gu, dn = refs(gate_up), refs(down)
+    upr = refs(up) if up is not None else None
     x = _c(x, np.float32)
     route_idx, route_w = _c(route_idx, np.uint32), _c(route_w, np.float32)
     k = route_idx.size // t
@@ -312,5 +330,5 @@ def moe_q4(gate_up, down, group, h, inter, x, t, route_idx, route_w, y, decode_p
         assert decode_path
         lib.oxref_moe_q4_avx2(gu, dn, ne, group, h, inter, _p(x), t, _p(route_idx), _p(route_w), k, _p(y), threads or hw_threads())
         return y
-    lib.oxref_moe_q4(gu, dn, ne, group, h, inter, _p(x), t, _p(route_idx), _p(route_w), k, _p(y), int(decode_path))
+    lib.oxref_moe_q4_act(gu, upr, dn, ne, group, h, inter, _p(x), t, _p(route_idx), _p(route_w), k, _p(y), int(decode_path), act, float(act_param))
     return y

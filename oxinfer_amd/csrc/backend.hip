@@ -28,6 +28,16 @@ __global__ void fill_zero_kernel(uint32_t* p, size_t n) {
     if (i < n) p[i] = 0u;
 }
 
+namespace oxhip {
+// Clears n dwords with a kernel on `s` (not a memset: memset nodes captured into a graph have replayed wrongly, and a
+// memset on the null stream waits for the whole device).
+hipError_t launch_fill_zero(uint32_t* p, size_t n, hipStream_t s) {
+    if (!n) return hipSuccess;
+    fill_zero_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(p, n);
+    return hipGetLastError();
+}
+}  // namespace oxhip
+
 namespace {
 
 struct Planes {
@@ -486,7 +496,7 @@ static int decode_one(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa,
         v = view_of(*xa);
     }
     HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
-    StreamScratch* sc = scratch_for(c, static_cast<hipStream_t>(stream));
+    StreamScratch* sc = scratch_for(c, static_cast<hipStream_t>(stream), needs_slices(w));
     if (!sc) {
         set_error("decode: device memory short");
         return 0;
@@ -526,6 +536,7 @@ int oxhip_dev_decode_noalloc(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qa
         return 0;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
+    HIP_TRY(hipSetDevice(c->device), "hipSetDevice");  // `ptr` is this device's copy of the array
     DecodeScratch sc;
     sc.partial = static_cast<float*>(ptr);
     sc.counters = reinterpret_cast<uint32_t*>(static_cast<unsigned char*>(ptr) + NOALLOC_PARTIAL_FLOATS * 4);
@@ -534,8 +545,7 @@ int oxhip_dev_decode_noalloc(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qa
     if (need_c) {
         // the array keeps what the last call (of any caller on this GPU) left: the counters must start at zero. A small
         // kernel, not a memset: memset nodes captured into a graph have replayed wrongly.
-        fill_zero_kernel<<<(unsigned)((need_c + 255) / 256), 256, 0, s>>>(sc.counters, need_c);
-        HIP_TRY(hipGetLastError(), "decode_noalloc: counter clear launch");
+        HIP_TRY(launch_fill_zero(sc.counters, need_c, s), "decode_noalloc: counter clear launch");
     }
     HIP_TRY(launch_decode_mfma(w->v, view_of(*xa), t, y, sc, s), "decode_noalloc launch");
     return 1;
@@ -548,7 +558,9 @@ int oxhip_dev_decode_batch(oxhip_ctx* c, const oxhip_decode_job* jobs, size_t n_
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
-    StreamScratch* ssc = scratch_for(c, s);
+    bool any_slices = false;
+    for (size_t k = 0; k < n_jobs; k++) any_slices |= jobs[k].w && needs_slices(jobs[k].w);
+    StreamScratch* ssc = scratch_for(c, s, any_slices);
     if (!ssc) {
         set_error("decode_batch: device memory short");
         return 0;

@@ -81,9 +81,11 @@ namespace oxhip {
 
 // backend_gemm.hip: packs x into `ws` and runs the bf16-matrix-core GEMM (1 = done, 0 = declined with the error set)
 int gemm_bf16_run(DevBuf& ws, const oxhip_weight* w, const void* x, bool x_bf16, size_t t, void* y, bool y_bf16, hipStream_t s);
-// backend_graph.hip: the calling stream's scratch (created on the stream's first call; nullptr when memory is short)
-StreamScratch* scratch_for(oxhip_ctx* c, hipStream_t s);
+// backend_graph.hip: the calling stream's scratch (nullptr when memory is short). `slices`: the launch that follows may
+// slice K across workgroups, so the entry must hold the decode kernels' partial rows and counters (allocated on first need).
+StreamScratch* scratch_for(oxhip_ctx* c, hipStream_t s, bool slices);
 void free_stream_scratch(oxhip_ctx* c);
+bool needs_slices(const oxhip_weight* w);  // a decode launch of this weight alone slices K across workgroups
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 

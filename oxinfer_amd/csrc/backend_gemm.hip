@@ -111,7 +111,7 @@ int oxhip_dev_gemm_isums(oxhip_ctx* c, const oxhip_weight* w, const void* x, int
         return 0;
     }
     HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
-    StreamScratch* sc = scratch_for(c, static_cast<hipStream_t>(stream));
+    StreamScratch* sc = scratch_for(c, static_cast<hipStream_t>(stream), false);
     if (!sc) {
         set_error("gemm_isums: device memory short");
         return 0;
@@ -127,7 +127,7 @@ int oxhip_dev_gemm(oxhip_ctx* c, const oxhip_weight* w, const void* x, int x_dty
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
-    StreamScratch* sc = scratch_for(c, s);
+    StreamScratch* sc = scratch_for(c, s, false);
     if (!sc) {
         set_error("gemm: device memory short");
         return 0;

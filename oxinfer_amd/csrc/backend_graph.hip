@@ -10,41 +10,75 @@ using namespace oxhip;
 namespace oxhip {
 
 // The scratch of the device-pointer entry points, one set per stream: launches on one stream are ordered, so they may
-// share; launches on different streams may overlap and must not.
-StreamScratch* scratch_for(oxhip_ctx* c, hipStream_t s) {
+// share; launches on different streams may overlap and must not. A stream's entry holds no device memory until a call
+// needs some: the partial rows and arrival counters of the decode kernels (16 MiB + 2 MiB) come with the first launch on
+// that stream whose shape slices K across workgroups (`slices`), their counters cleared by a kernel on that same stream
+// (ordered before the launch that follows, and no wait for the rest of the device).
+StreamScratch* scratch_for(oxhip_ctx* c, hipStream_t s, bool slices) {
     std::lock_guard<std::mutex> g(c->smu);
+    StreamScratch* sc;
     auto it = c->per_stream.find(s);
-    if (it != c->per_stream.end()) return it->second;
-    auto* sc = new StreamScratch();
-    sc->dec.partial_floats = c->dec.partial_floats;
-    sc->dec.ncounters = c->dec.ncounters;
-    if (hipMalloc(reinterpret_cast<void**>(&sc->dec.partial), sc->dec.partial_floats * 4) != hipSuccess ||
-        hipMalloc(reinterpret_cast<void**>(&sc->dec.counters), sc->dec.ncounters * 4) != hipSuccess ||
-        hipMemset(sc->dec.counters, 0, sc->dec.ncounters * 4) != hipSuccess) {
-        if (sc->dec.partial) (void)hipFree(sc->dec.partial);
-        if (sc->dec.counters) (void)hipFree(sc->dec.counters);
-        delete sc;
-        return nullptr;
+    if (it != c->per_stream.end()) {
+        sc = it->second;
+    } else {
+        sc = new StreamScratch();
+        c->per_stream.emplace(s, sc);
     }
-    c->per_stream.emplace(s, sc);
+    if (slices && !sc->dec.partial) {
+        DecodeScratch d;
+        d.partial_floats = c->dec.partial_floats;
+        d.ncounters = c->dec.ncounters;
+        if (hipMalloc(reinterpret_cast<void**>(&d.partial), d.partial_floats * 4) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void**>(&d.counters), d.ncounters * 4) != hipSuccess ||
+            launch_fill_zero(d.counters, d.ncounters, s) != hipSuccess) {
+            if (d.partial) (void)hipFree(d.partial);
+            if (d.counters) (void)hipFree(d.counters);
+            return nullptr;
+        }
+        sc->dec = d;
+    }
     return sc;
+}
+
+static void release_scratch(StreamScratch* sc) {
+    if (sc->dec.partial) (void)hipFree(sc->dec.partial);
+    if (sc->dec.counters) (void)hipFree(sc->dec.counters);
+    sc->tmp.release();
+    sc->gemm_ws.release();
+    delete sc;
 }
 
 void free_stream_scratch(oxhip_ctx* c) {
     std::lock_guard<std::mutex> g(c->smu);
-    for (auto& kv : c->per_stream) {
-        (void)hipFree(kv.second->dec.partial);
-        (void)hipFree(kv.second->dec.counters);
-        kv.second->tmp.release();
-        kv.second->gemm_ws.release();
-        delete kv.second;
-    }
+    for (auto& kv : c->per_stream) release_scratch(kv.second);
     c->per_stream.clear();
+}
+
+bool needs_slices(const oxhip_weight* w) {
+    size_t p = 0, n = 0;
+    decode_scratch_need(w->v, &p, &n);
+    return p != 0;
 }
 
 }  // namespace oxhip
 
 extern "C" {
+
+int oxhip_stream_release(oxhip_ctx* c, void* stream) {
+    if (!c) {
+        set_error("stream_release: null context");
+        return 0;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
+    HIP_TRY(hipStreamSynchronize(s), "stream_release: the stream's work failed");  // its launches may still use the scratch
+    std::lock_guard<std::mutex> g(c->smu);
+    auto it = c->per_stream.find(s);
+    if (it == c->per_stream.end()) return 1;
+    release_scratch(it->second);
+    c->per_stream.erase(it);
+    return 1;
+}
 
 void* oxhip_buf_alloc(oxhip_ctx* c, size_t bytes) {
     if (!c || !bytes) {
@@ -100,6 +134,18 @@ int oxhip_dev_rmsnorm_quantize(oxhip_ctx* c, const float* x, const float* w_f32,
     return 1;
 }
 
+int oxhip_dev_norm(oxhip_ctx* c, const float* x, float* out, const float* w_f32, const uint16_t* w_bf16, float pre, size_t n, size_t rows,
+                   size_t x_stride, size_t out_stride, float eps, int add, const oxhip_qact* q, void* stream) {
+    if (!c || !x || (!out && !q) || n % 32 || !n || (w_f32 && w_bf16) || (q && (q->n_in != n || q->t < rows)) || (add && !out) ||
+        (x_stride && x_stride < n) || (out_stride && out_stride < n)) {
+        set_error("norm: bad arguments (n a multiple of 32, one kind of weights, strides of at least n floats, `add` needs `out`)");
+        return 0;
+    }
+    HIP_TRY(launch_rmsnorm_quantize(x, w_f32, w_bf16, eps, rows, n, out, q, static_cast<hipStream_t>(stream), pre, add != 0, x_stride, out_stride),
+            "norm launch");
+    return 1;
+}
+
 int oxhip_dev_glu(oxhip_ctx* c, const float* g, const float* u, size_t n, int gelu, float* y, void* stream) {
     if (!c || !g || !u || !y) {
         set_error("glu: null argument");
@@ -139,7 +185,7 @@ int oxhip_dev_linear(oxhip_ctx* c, const oxhip_weight* w, const oxhip_weight* w2
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
-    StreamScratch* sc = scratch_for(c, s);
+    StreamScratch* sc = scratch_for(c, s, needs_slices(w));
     if (!sc) {
         set_error("linear: device memory short");
         return 0;

@@ -19,6 +19,7 @@ struct oxhip_moe {
     DevBuf ws;                           // scratch of one pass
     size_t ws_pairs = 0, ws_t = 0;
     uint32_t mode = OXHIP_MOE_AUTO;      // oxhip_moe_set_mode
+    bool counters_dirty = false;         // a pass failed part-way: the arrival counters may not be back at zero
 };
 
 namespace {
@@ -86,8 +87,8 @@ struct RouteIn {
     const float* expert_scale = nullptr;
 };
 
-int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t* route_idx, const float* route_w, size_t k,
-            float* y, hipStream_t s, bool add = true, const RouteIn& rin = RouteIn{}) {
+int moe_pass(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t* route_idx, const float* route_w, size_t k,
+             float* y, hipStream_t s, bool add, const RouteIn& rin) {
     const size_t pairs = t * k, h = m->h, inter = m->inter;
     if (!pairs) return 1;
     uint32_t* ridx_out = const_cast<uint32_t*>(route_idx);
@@ -108,6 +109,12 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
         HIP_TRY(hipMemsetAsync(m->ws.p, 0, m->ws.cap, s), "moe scratch clear");
     }
     Scratch sc = carve(static_cast<uint8_t*>(m->ws.p), t, pairs, m->n_exp, h, inter);
+    if (m->counters_dirty) {
+        // an earlier pass ended in an error after its down launch may have started: the last workgroup of each row group
+        // puts its counter back to zero, which a failed launch may not have done
+        HIP_TRY(launch_fill_zero(sc.counters, (size_t)COMB_GROUPS * CTR_STRIDE, s), "moe counter clear launch");
+        m->counters_dirty = false;
+    }
     // Rows per chunk: one pass over an expert's weights serves a whole chunk, so chunks grow with the rows an expert
     // gets on average (8 rows per matrix-core instruction, up to 4 instructions per weight record).
     uint32_t max_rows = (uint32_t)(t < 8 ? t : 8);
@@ -229,6 +236,15 @@ int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t
     return 1;
 }
 
+// A pass that fails part-way (a launch error) may leave the down launch's arrival counters above zero; the next pass on
+// this layer clears them first.
+int moe_run(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t* route_idx, const float* route_w, size_t k,
+            float* y, hipStream_t s, bool add = true, const RouteIn& rin = RouteIn{}) {
+    const int rc = moe_pass(c, m, x, t, route_idx, route_w, k, y, s, add, rin);
+    if (!rc) m->counters_dirty = true;
+    return rc;
+}
+
 }  // namespace
 
 extern "C" {
@@ -333,12 +349,13 @@ int oxhip_dev_moe(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const ui
         set_error("moe: null argument");
         return 0;
     }
+    HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
     return moe_run(c, m, x, t, route_idx, route_w, k, y, static_cast<hipStream_t>(stream));
 }
 
 int oxhip_dev_experts(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_t* sel, size_t k, float* y, int add, void* stream) {
-    if (!c || !m || !x || !sel || !y || !k || !t) {
-        set_error("experts: bad arguments");
+    if (!c || !m || !x || !sel || !y || !k || !t || k > 32) {
+        set_error("experts: bad arguments (1 <= k <= 32)");
         return 0;
     }
     HIP_TRY(hipSetDevice(c->device), "hipSetDevice");

@@ -71,28 +71,43 @@ hipError_t launch_router_logits(const float* x, const float* router, const float
     return hipGetLastError();
 }
 
-// RMSNorm of one row per workgroup, then quantize_act of the normed row without a round trip through memory:
-//   r = (sum x^2 / n + eps)^(-1/2);  v = (x * r) * w  (or x * r);  v -> `out` (optional) and, per block of 32, the QAct.
+// RMSNorm of one row per workgroup (Op::Norm, src/gpu_decode.rs:53-66), then quantize_act of the row that was written,
+// without a round trip through memory:
+//   x' = x * pre;  r = (sum x'^2 / n + eps)^(-1/2);  v = (x' * r) * w  (or x' * r);  out = v, or out += v with `add`;
+//   what `out` then holds goes, per block of 32, to the QAct (optional).
 // The reference sums the squares one after the other in f32 (src/kernels.rs:2109), which no parallel machine can
 // repeat bit for bit in useful time: here the squares are exact in f64 and summed in f64 (a fixed order), the mean and
 // eps added in f32 as the reference does, and r is the correctly rounded power. The quantization of v is quantize_act's,
-// bit for bit (the same code on the same values).
+// bit for bit (the same code on the same values). VEC: rows of x, out and w start on 16-byte boundaries (float4 access);
+// otherwise every access is one float.
+template <bool VEC>
 __global__ __launch_bounds__(256) void rmsnorm_quantize_kernel(const float* __restrict__ x, const float* __restrict__ w_f32,
-                                                               const uint16_t* __restrict__ w_bf16, float eps, uint32_t n,
+                                                               const uint16_t* __restrict__ w_bf16, float eps, float pre, uint32_t add,
+                                                               uint32_t n, size_t x_stride, size_t out_stride,
                                                                float* __restrict__ out, int8_t* __restrict__ q, float* __restrict__ scales,
                                                                int32_t* __restrict__ sums, float* __restrict__ fsums,
                                                                float* __restrict__ hsums, int32_t* __restrict__ sums16) {
     __shared__ double part[4];
     __shared__ float r_s;
     const uint32_t tok = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const float* xr = x + (size_t)tok * n;
+    const float* xr = x + (size_t)tok * x_stride;
+    auto load4 = [&](const float* p, float* v) {
+        if constexpr (VEC) {
+            const float4 f = *reinterpret_cast<const float4*>(p);
+            v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+        } else {
+            v[0] = p[0]; v[1] = p[1]; v[2] = p[2]; v[3] = p[3];
+        }
+    };
     double ss = 0.0;
     for (uint32_t i = 4 * threadIdx.x; i < n; i += 1024) {  // n is a multiple of 32
-        const float4 v = *reinterpret_cast<const float4*>(xr + i);
-        ss += (double)v.x * v.x;
-        ss += (double)v.y * v.y;
-        ss += (double)v.z * v.z;
-        ss += (double)v.w * v.w;
+        float v[4];
+        load4(xr + i, v);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float p = v[j] * pre;
+            ss += (double)p * p;
+        }
     }
     for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off);
     if (lane == 0) part[wave] = ss;
@@ -109,11 +124,10 @@ __global__ __launch_bounds__(256) void rmsnorm_quantize_kernel(const float* __re
         float v[32];
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const float4 f = *reinterpret_cast<const float4*>(xr + 32 * b + 4 * i);
-            v[4 * i] = f.x * r;
-            v[4 * i + 1] = f.y * r;
-            v[4 * i + 2] = f.z * r;
-            v[4 * i + 3] = f.w * r;
+            float f[4];
+            load4(xr + 32 * b + 4 * i, f);
+#pragma unroll
+            for (int j = 0; j < 4; j++) v[4 * i + j] = (f[j] * pre) * r;
         }
         if (w_f32) {
 #pragma unroll
@@ -123,22 +137,46 @@ __global__ __launch_bounds__(256) void rmsnorm_quantize_kernel(const float* __re
             for (int i = 0; i < 32; i++) v[i] = v[i] * bf16_bits_to_f32(w_bf16[32 * b + i]);
         }
         const size_t gb = (size_t)tok * nblocks + b;
+        float* orow = out ? out + (size_t)tok * out_stride + 32 * b : nullptr;
+        if (out && add) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float f[4];
+                load4(orow + 4 * i, f);
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[4 * i + j] = f[j] + v[4 * i + j];
+            }
+        }
         if (out) {
 #pragma unroll
-            for (int i = 0; i < 8; i++)
-                *reinterpret_cast<float4*>(out + gb * 32 + 4 * i) = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+            for (int i = 0; i < 8; i++) {
+                if constexpr (VEC) {
+                    *reinterpret_cast<float4*>(orow + 4 * i) = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) orow[4 * i + j] = v[4 * i + j];
+                }
+            }
         }
         if (q) quantize_act_values(v, gb, q, scales, sums, fsums, hsums, sums16);
     }
 }
 
 hipError_t launch_rmsnorm_quantize(const float* x, const float* w_f32, const uint16_t* w_bf16, float eps, size_t t, size_t n, float* out,
-                                   const oxhip_qact* qa, hipStream_t s) {
+                                   const oxhip_qact* qa, hipStream_t s, float pre, bool add, size_t x_stride, size_t out_stride) {
     if (!t || !n) return hipSuccess;
     if (n % 32) return hipErrorInvalidValue;
-    rmsnorm_quantize_kernel<<<(unsigned)t, 256, 0, s>>>(x, w_f32, w_bf16, eps, (uint32_t)n, out, qa ? qa->q : nullptr, qa ? qa->scales : nullptr,
-                                                       qa ? qa->sums : nullptr, qa ? qa->fsums : nullptr, qa ? qa->hsums : nullptr,
-                                                       qa ? qa->sums16 : nullptr);
+    if (!x_stride) x_stride = n;
+    if (!out_stride) out_stride = n;
+    auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    const bool vec = al(x) && al(out) && al(w_f32) && x_stride % 4 == 0 && out_stride % 4 == 0;
+    auto go = [&](auto kern) {
+        kern<<<(unsigned)t, 256, 0, s>>>(x, w_f32, w_bf16, eps, pre, add ? 1u : 0u, (uint32_t)n, x_stride, out_stride, out, qa ? qa->q : nullptr,
+                                        qa ? qa->scales : nullptr, qa ? qa->sums : nullptr, qa ? qa->fsums : nullptr, qa ? qa->hsums : nullptr,
+                                        qa ? qa->sums16 : nullptr);
+    };
+    if (vec) go(rmsnorm_quantize_kernel<true>);
+    else go(rmsnorm_quantize_kernel<false>);
     return hipGetLastError();
 }
 

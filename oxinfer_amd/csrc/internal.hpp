@@ -225,8 +225,10 @@ hipError_t launch_moe_combine(const float* o, const int* row_of, const float* ro
 hipError_t launch_glu(const float* g, const float* u, size_t n, bool gelu, float* y, hipStream_t s);
 hipError_t launch_router_logits(const float* x, const float* router, const float* gate, size_t t, size_t n_exp, size_t h, float* logits,
                                 hipStream_t s);
+// x_stride / out_stride: floats between rows (0 = n); pre: x is scaled by it first; add: out += instead of out =
 hipError_t launch_rmsnorm_quantize(const float* x, const float* w_f32, const uint16_t* w_bf16, float eps, size_t t, size_t n, float* out,
-                                   const oxhip_qact* q, hipStream_t s);
+                                   const oxhip_qact* q, hipStream_t s, float pre = 1.0f, bool add = false, size_t x_stride = 0,
+                                   size_t out_stride = 0);
 // The bf16 form of the grouped expert matmuls for prefill passes (moe_bf16.hip): MLX 4-bit weights, chunks of <= 16 rows.
 bool moe_bf16_ok(const WeightView& w);
 size_t moe_bf16_frag_bytes(size_t max_chunks, size_t n_in);
@@ -235,6 +237,8 @@ hipError_t launch_moe_pack_bf16(const float* x, size_t n_in, const int* rowmap, 
 hipError_t launch_moe_act_pack_bf16(const float* g, const float* u, size_t stride, size_t inter, uint32_t kind, float param, const int4* chunks,
                                     const int* nchunks, uint32_t max_chunks, void* frag, hipStream_t s);
 hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max_chunks, const void* frag, float* out, hipStream_t s);
+
+hipError_t launch_fill_zero(uint32_t* p, size_t n, hipStream_t s);  // n dwords, by a kernel on `s`
 
 void set_error(const std::string& msg);
 

@@ -105,6 +105,8 @@ def load_library():
         "oxhip_buf_write": (C.c_int, [vp, vp, vp, sz, vp]),
         "oxhip_buf_read": (C.c_int, [vp, vp, vp, sz, vp]),
         "oxhip_dev_rmsnorm_quantize": (C.c_int, [vp, vp, vp, vp, C.c_float, sz, sz, vp, C.POINTER(QActC), vp]),
+        "oxhip_dev_norm": (C.c_int, [vp, vp, vp, vp, vp, C.c_float, sz, sz, sz, sz, C.c_float, C.c_int, C.POINTER(QActC), vp]),
+        "oxhip_stream_release": (C.c_int, [vp, vp]),
         "oxhip_dev_linear": (C.c_int, [vp, vp, vp, C.POINTER(QActC), vp, sz, vp, C.c_uint32, vp, vp]),
         "oxhip_dev_glu": (C.c_int, [vp, vp, vp, sz, C.c_int, vp, vp]),
         "oxhip_dev_route": (C.c_int, [vp, vp, vp, vp, sz, sz, sz, sz, vp, vp, vp, vp]),
@@ -402,6 +404,19 @@ class HipBackend:
         if not ok:
             raise RuntimeError(self.last_error())
         return out, q
+
+    def norm(self, x, n, rows, out=None, w=None, pre=1.0, x_stride=0, out_stride=0, eps=1e-6, add=False, want_q=False):
+        """Op::Norm with all its fields on device tensors (x, out: f32, any float offset into a larger buffer)."""
+        import torch
+        q = QAct(rows, n, x.device) if want_q else None
+        wf = w.data_ptr() if w is not None and w.dtype == torch.float32 else None
+        wb = w.data_ptr() if w is not None and w.dtype == torch.bfloat16 else None
+        ok = self.lib.oxhip_dev_norm(self.ctx, x.data_ptr(), out.data_ptr() if out is not None else None, wf, wb, pre, n, rows, x_stride,
+                                     out_stride, eps, int(add), C.byref(q.c) if want_q else None, self._stream())
+        return (bool(ok), q)
+
+    def stream_release(self, stream):
+        return bool(self.lib.oxhip_stream_release(self.ctx, C.c_void_p(stream)))
 
     def linear(self, w, y, xa=None, x=None, t=None, mode=LIN_STORE, w2=None, gate=None):
         """Op::Linear on device tensors; y [t, n_out] f32 is written or added to according to `mode`. False = declined."""

@@ -274,6 +274,34 @@ def fp8_activation_checks(y, ref, x, wf):
     assert rms(y - ref) <= E4M3_RMS * rms(ref), rms(y - ref) / rms(ref)
 
 
+FP8_RECIPE_BOUND = 2e-2  # the bound BASELINE's north_star states for fp8 matrix-core outputs
+
+
+def fp8_literal_recipe_status(y8, rows, ref, m):
+    """The status of the literal configs[4] recipe (activations quantized to e4m3 per 1 x 128, fp8 matrix cores) at the
+    config's own shape [7168, 18432] against the CPU's f32 product, by two measures, both printed:
+      * the reference's own CPU-vs-accelerator report (src/bin/membench.rs:151-152): the largest absolute difference over
+        the largest output magnitude of the whole product;
+      * the stricter measure of this file's other tests: per token, the largest difference of its sampled outputs over
+        that token's own largest output, the worst token of all.
+    Rounding every activation to e4m3 leaves each with a relative error of up to 2^-4 (rms 2.6 to 2.9 %); the errors of a
+    row's K products add up like the products themselves, so the error of an output stays near 2.6 % of the outputs' rms
+    whatever K is, and the largest of M x N of them lands at 2 to 3 % of the largest output. Measured at M = 1024: 0.0205
+    and 0.0269; at M = 32: below 0.02. The recipe therefore does NOT hold the stated 2e-2 at M = 1024 by either measure,
+    which is why it is an explicit variant (OXHIP_GEMM_FP8) and the bf16 matrix cores, which do hold it, are the default
+    for FP8 weights. What is asserted here is the bound it does keep (3e-2 / 4e-2); its arithmetic is pinned exactly
+    (1e-3) against its own f64 definition by the callers."""
+    mx = np.maximum(np.abs(y8).max(axis=1), 1e-30)
+    diff = np.abs(y8[:, rows] - ref)
+    per_token = float((diff.max(axis=1) / mx).max())
+    whole = float(diff.max() / np.abs(y8).max())
+    holds = "holds" if whole < FP8_RECIPE_BOUND else "does NOT hold"
+    print(f"fp8-activation GEMM [7168, 18432] M = {m}: max abs diff / max output {whole:.4f} ({holds} the stated {FP8_RECIPE_BOUND}); "
+          f"worst token by its own largest output {per_token:.4f}")
+    assert whole < 3e-2, whole
+    assert per_token < 4e-2, per_token
+
+
 @pytest.mark.parametrize("n_out,n_in", [(200, 512), (384, 2304), (100, 128), (130, 256), (64, 640), (257, 896)])  # 1 to 18 K-blocks: every phase of the kernel's three-deep pipeline
 def test_gemm_fp8_matches_oracle(be, oxref, n_out, n_in):
     import torch
@@ -358,6 +386,7 @@ def test_gemm_fp8_config_m1024_sampled_rows(be, oxref):
     y8 = be.gemm(w, xd, variant=2).cpu().numpy()
     assert row_err(y8[:, rows], fp8_emulation(x, data, scales, oxref, rows)) < 1e-3
     fp8_activation_checks(y8[:, rows], ref, x, wf)
+    fp8_literal_recipe_status(y8, rows, ref, m)
 
 
 def test_gemm_fp8_full_size_sampled_rows(be, oxref):
@@ -382,6 +411,7 @@ def test_gemm_fp8_full_size_sampled_rows(be, oxref):
     assert float((np.abs(y[:, rows] - ref).max(axis=1) / m).max()) < 2e-2
     assert row_err(y8[:, rows], fp8_emulation(x, data, scales, oxref, rows)) < 1e-3
     fp8_activation_checks(y8[:, rows], ref, x, wf)
+    fp8_literal_recipe_status(y8, rows, ref, 32)
     y1 = be.decode(w, x=torch.from_numpy(x[:1]).cuda()).cpu().numpy()
     assert float(np.abs(y1[0, rows] - ref[0]).max() / np.abs(y1).max()) < 1e-3
 
@@ -428,19 +458,27 @@ def test_gemm_i8_extremes_bit_exact(be, oxref):
     assert row_err(be.gemm(w, torch.from_numpy(x).cuda(), variant=1).cpu().numpy(), ref) < 1e-5
 
 
-def test_gemm_i8_full_size_sampled_rows(be, oxref):
+@pytest.mark.parametrize("n_out,n_in", [(4096, 14336), (14336, 4096)])
+def test_gemm_i8_full_size_sampled_rows(be, oxref, n_out, n_in):
+    """BASELINE configs[2] variant (b) at both of its shapes, M = 512: the int32 block sums of sampled rows equal the
+    CPU's bit for bit (all 512 tokens, every block of the row), outputs within 1e-3 of the oracle's restatement of
+    kernels_i8gemm and within the int8 bound of the exact product."""
     import torch
     from oxinfer_amd import synth
-    n_out, n_in, t = 4096, 14336, 512
+    t = 512
     wq, sc, bi = synth.mlx_q4(n_out, n_in, 21)
     w = be.upload_mlx_q4(wq, sc, bi, 64, n_out, n_in)
     assert w is not None, be.last_error()
     x = synth.activations(t, n_in, 22, bf16=True)
-    y = be.gemm(w, torch.from_numpy(x).cuda().to(torch.bfloat16), variant=1).cpu().numpy()
-    rows = np.r_[0:4, 2046:2050, n_out - 4:n_out, np.random.default_rng(1).integers(0, n_out, 12)]
+    xd = torch.from_numpy(x).cuda().to(torch.bfloat16)
+    y = be.gemm(w, xd, variant=1).cpu().numpy()
+    rows = np.r_[0:4, n_out // 2 - 2:n_out // 2 + 2, n_out - 4:n_out, np.random.default_rng(1).integers(0, n_out, 12)]
     q, s16, off = oxref.from_mlx_q4(wq[rows], sc[rows], bi[rows], len(rows), n_in, 64)
-    ref = oxref.i8gemm_q4(q, s16, off, 64, len(rows), n_in, x, t)
+    ref, isums = oxref.i8gemm_q4(q, s16, off, 64, len(rows), n_in, x, t, want_isums=True)
     m = np.maximum(np.abs(y).max(axis=1), 1e-30)
     assert float((np.abs(y[:, rows] - ref).max(axis=1) / m).max()) < 1e-3
     exact = oxref.gemm_quant(-1, q, s16, off, len(rows), n_in, x, t)
     assert float((np.abs(y[:, rows] - exact).max(axis=1) / m).max()) < 2e-2
+    got = be.gemm_isums(w, xd)  # [t, n_out, n_in / 32] on the device; only the sampled rows come back
+    got = got[:, torch.from_numpy(rows).cuda(), :].cpu().numpy()
+    assert np.array_equal(got, isums)

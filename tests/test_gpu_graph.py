@@ -172,6 +172,79 @@ def test_rmsnorm_quantize(be, oxref, n):
             assert np.array_equal(qb.q.cpu().numpy(), q) and np.array_equal(qb.scales.cpu().numpy().view(np.uint32), scales.view(np.uint32))
 
 
+def test_norm_with_all_fields(be, oxref):
+    """Op::Norm as the reference defines it (src/gpu_decode.rs:53-66, src/cuda_decode.cu:314-327): rows with strides
+    inside a larger buffer, the `pre` factor, `out +=`, and views that do not start on 16-byte boundaries. Against the f64
+    definition out (+)= ((x pre) r) w, r = (mean((x pre)^2) + eps)^(-1/2); the quantized row is quantize_act of what `out`
+    holds, bit for bit."""
+    import torch
+    rng = np.random.default_rng(9)
+    n, rows, eps = 256, 3, 1e-5
+    for x_off, o_off, xs, os_, pre, add in ((0, 0, 0, 0, 1.0, False), (4, 8, 320, 288, 0.5, True), (3, 1, 259, 261, 2.0, False), (1, 2, 256, 256, 1.5, True)):
+        xsf, osf = xs or n, os_ or n
+        xbuf = rng.normal(0, 2, x_off + rows * xsf + 7).astype(np.float32)
+        obuf = rng.normal(0, 1, o_off + rows * osf + 7).astype(np.float32)
+        w = rng.normal(1, 0.2, n + 1).astype(np.float32)
+        xd, od, wd = dev(xbuf), dev(obuf), dev(w)
+        w_view = wd[1:] if x_off % 4 else wd[:n]   # an unaligned weight view with the unaligned inputs
+        w_host = w[1:] if x_off % 4 else w[:n]
+        ok, qa = be.norm(xd[x_off:], n, rows, out=od[o_off:], w=w_view, pre=pre, x_stride=xs, out_stride=os_, eps=eps, add=add, want_q=True)
+        assert ok, be.last_error()
+        torch.cuda.synchronize()
+        got = od.cpu().numpy()
+        want = obuf.copy()
+        for r in range(rows):
+            xr = xbuf[x_off + r * xsf: x_off + r * xsf + n].astype(np.float64) * pre
+            v = xr / np.sqrt((xr * xr).mean() + eps) * w_host.astype(np.float64)
+            seg = slice(o_off + r * osf, o_off + r * osf + n)
+            want[seg] = (obuf[seg] + v if add else v).astype(np.float32)
+        assert np.abs(got - want).max() < 2e-6 * max(1.0, np.abs(want).max())
+        # nothing outside the rows was touched
+        mask = np.ones(obuf.size, bool)
+        for r in range(rows):
+            mask[o_off + r * osf: o_off + r * osf + n] = False
+        assert np.array_equal(got[mask], obuf[mask])
+        rows_out = np.stack([got[o_off + r * osf: o_off + r * osf + n] for r in range(rows)])
+        q, sc, sums, fs, hs = oxref.quantize_act(rows_out, rows, n)
+        assert np.array_equal(qa.q.cpu().numpy(), q) and np.array_equal(qa.scales.cpu().numpy().view(np.uint32), sc.view(np.uint32))
+        assert np.array_equal(qa.sums.cpu().numpy(), sums) and np.array_equal(qa.fsums.cpu().numpy().view(np.uint32), fs.view(np.uint32))
+    # `add` without an output, strides shorter than a row: declined
+    assert not be.norm(xd, n, 1, out=None, add=True, want_q=True)[0]
+    assert not be.norm(xd, n, 2, out=od, x_stride=n - 4)[0]
+
+
+def test_decode_on_two_streams_overlaps_and_keeps_the_bits(be, oxref):
+    """Calls on different streams keep separate scratch (partial rows and counters of K-sliced shapes), so they may
+    overlap: matmuls issued alternately on two streams give, bit for bit, the rows of the same calls issued one after the
+    other on one stream. A released stream's next call allocates its scratch again."""
+    import torch
+    n_out, n_in, t = 528, 14336, 8   # 14336 columns: K is sliced across workgroups, the slices meet through the scratch
+    raws = [oxref.random_blocks(8, n_out * n_in // 32, 60 + i)[0] for i in range(2)]
+    ws = [be.upload_gguf(8, r, n_out, n_in) for r in raws]
+    xs = [np.random.default_rng(70 + i).normal(0, 1, (t, n_in)).astype(np.float32) for i in range(2)]
+    xas = [be.quantize_act(dev(x)) for x in xs]
+    serial = [be.decode(ws[i], xa=xas[i], t=t).cpu().numpy() for i in range(2)]
+    for i in range(2):
+        assert row_err(serial[i], oxref.gguf_decode(8, raws[i], n_out, n_in, xs[i], t)) < 1e-3
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    ys = [[torch.empty((t, n_out), dtype=torch.float32, device="cuda") for _ in range(6)] for _ in range(2)]
+    for rep in range(6):
+        for i in range(2):
+            with torch.cuda.stream(streams[i]):
+                be.decode(ws[i], xa=xas[i], t=t, y=ys[i][rep])
+    torch.cuda.synchronize()
+    for i in range(2):
+        for rep in range(6):
+            assert np.array_equal(ys[i][rep].cpu().numpy().view(np.uint32), serial[i].view(np.uint32)), (i, rep)
+    assert be.stream_release(streams[0].cuda_stream)
+    with torch.cuda.stream(streams[0]):
+        again = be.decode(ws[0], xa=xas[0], t=t)
+    torch.cuda.synchronize()
+    assert np.array_equal(again.cpu().numpy().view(np.uint32), serial[0].view(np.uint32))
+    assert be.stream_release(streams[0].cuda_stream) and be.stream_release(streams[1].cuda_stream)
+
+
 @pytest.mark.parametrize("ne,h,k", [(128, 2048, 8), (6, 256, 3), (300, 130, 6)])
 def test_route(be, oxref, ne, h, k):
     """Op::Route (src/gpu_decode.rs:154-172): the router's logits (and the shared expert's gate logit behind them), then

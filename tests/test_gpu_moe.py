@@ -320,6 +320,80 @@ def test_moe_duplicate_routes_within_a_token(be, oxref, mlx_experts):
     assert row_err(y, ref) < 1e-3
 
 
+@pytest.mark.parametrize("act,param", [(1, 0.0), (2, 0.1)])   # MoeAct::GeluTanh, MoeAct::SiluClamp(0.1)
+@pytest.mark.parametrize("split", [False, True])               # fused [2 inter, h] experts / separate gate and up
+def test_moe_activation_kinds_and_split_experts(be, oxref, act, param, split):
+    """MoeAct::GeluTanh and SiluClamp(l), and experts uploaded as separate gate / up matrices (src/gpu.rs:35-54,
+    :206-216), at decode sizes (the integer kernels against Experts::forward_batched's semantics, 1e-3) and at a prefill
+    size (40 tokens: fused experts take the bf16 form against the grouped f32 path with Act::scalar, 1e-2; split experts
+    stay on the integer kernels: 1e-3 of the decode semantics, 5e-2 of the exact product on these short rows). The clamp limit lies inside
+    the products' range, so a missing clamp fails."""
+    from oxinfer_amd import synth
+    ne, h, inter, k = 6, 256, 128, 3
+    raw_g = [synth.mlx_q4(inter, h, 3100 + e) for e in range(ne)]
+    raw_u = [synth.mlx_q4(inter, h, 3200 + e) for e in range(ne)]
+    raw_d = [synth.mlx_q4(h, inter, 3300 + e) for e in range(ne)]
+    raw_gu = [tuple(np.concatenate([a, b]) for a, b in zip(raw_g[e], raw_u[e])) for e in range(ne)]
+    q_gu = [oxref.from_mlx_q4(*r, 2 * inter, h, 64) for r in raw_gu]
+    q_d = [oxref.from_mlx_q4(*r, h, inter, 64) for r in raw_d]
+    if split:
+        dev = be.upload_moe([be.desc_mlx_q4(*r, 64, inter, h) for r in raw_g], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_d], h, inter,
+                            up=[be.desc_mlx_q4(*r, 64, inter, h) for r in raw_u], act=act, act_param=param)
+    else:
+        dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_d], h, inter,
+                            act=act, act_param=param)
+    assert dev is not None, be.last_error()
+    for t in (1, 3, 8, 40):
+        x = synth.activations(t, h, 3400 + t)
+        _, idx, w = make_routes(oxref, t, ne, k, 3500 + t)
+        y0 = synth.activations(t, h, 3600 + t)
+        y = y0.copy()
+        assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
+        dec = oxref.moe_q4(q_gu, q_d, 64, h, inter, x, t, idx, w, y0, decode_path=True, act=act, act_param=param)
+        plain = oxref.moe_q4(q_gu, q_d, 64, h, inter, x, t, idx, w, y0, decode_path=True)
+        assert row_err(plain - y0, dec - y0) > 2e-2          # the activation kind matters on these inputs
+        if (t * k) // ne >= 6 and not split:
+            grouped = oxref.moe_q4(q_gu, q_d, 64, h, inter, x, t, idx, w, y0, decode_path=False, act=act, act_param=param)
+            assert row_err(y - y0, grouped - y0) < 1e-2, (t, row_err(y - y0, grouped - y0))
+        else:
+            assert row_err(y - y0, dec - y0) < 1e-3, (t, row_err(y - y0, dec - y0))
+            if t >= 8:
+                grouped = oxref.moe_q4(q_gu, q_d, 64, h, inter, x, t, idx, w, y0, decode_path=False, act=act, act_param=param)
+                # int8 activations against the exact product: the reference's bound for them is 3e-2 on its own shapes
+                # (src/ggml.rs:1904); these rows of 256 and 128 values average a little less
+                assert row_err(y - y0, grouped - y0) < 5e-2, t
+
+
+@pytest.mark.parametrize("act,param,split", [(1, 0.0, False), (2, 0.2, True)])
+def test_moe_activation_kinds_config_shapes(be, oxref, act, param, split):
+    """The same at the benchmark's expert shapes (h 2048, inter 768, top-8) over 16 experts: one token (decode) and 32
+    tokens (16 routed rows per expert: the prefill size)."""
+    from oxinfer_amd import synth
+    ne, h, inter, k = 16, 2048, 768, 8
+    raw_g = [synth.mlx_q4(inter, h, 4100 + e) for e in range(ne)]
+    raw_u = [synth.mlx_q4(inter, h, 4200 + e) for e in range(ne)]
+    raw_d = [synth.mlx_q4(h, inter, 4300 + e) for e in range(ne)]
+    raw_gu = [tuple(np.concatenate([a, b]) for a, b in zip(raw_g[e], raw_u[e])) for e in range(ne)]
+    q_gu = [oxref.from_mlx_q4(*r, 2 * inter, h, 64) for r in raw_gu]
+    q_d = [oxref.from_mlx_q4(*r, h, inter, 64) for r in raw_d]
+    if split:
+        dev = be.upload_moe([be.desc_mlx_q4(*r, 64, inter, h) for r in raw_g], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_d], h, inter,
+                            up=[be.desc_mlx_q4(*r, 64, inter, h) for r in raw_u], act=act, act_param=param)
+    else:
+        dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_d], h, inter,
+                            act=act, act_param=param)
+    assert dev is not None, be.last_error()
+    for t in (1, 32):
+        x = synth.activations(t, h, 4400 + t, bf16=True)
+        _, idx, w = make_routes(oxref, t, ne, k, 4500 + t)
+        y0 = np.zeros((t, h), np.float32)
+        y = y0.copy()
+        assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
+        prefill_form = t == 32 and not split
+        ref = oxref.moe_q4(q_gu, q_d, 64, h, inter, x, t, idx, w, y0, decode_path=not prefill_form, act=act, act_param=param)
+        assert row_err(y, ref) < (5e-3 if prefill_form else 1e-3), (t, row_err(y, ref))
+
+
 def test_moe_declines(be, oxref, mlx_experts):
     ne, h, inter, raw_gu, raw_dn, _, _ = mlx_experts
     dev = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)

@@ -263,3 +263,84 @@ def test_moe_against_the_f64_definition(oxref):
     assert row_err(fast - y0, dec - y0) < 1e-5
     one = oxref.moe_q4(gu, dn, 64, h, inter, x[:1], 1, idx[:1], w[:1], y0[:1], decode_path=True, avx2=True, threads=3)
     assert row_err(one, dec[:1] - y0[:1]) < 1e-5
+
+
+def test_gated_activations_match_the_library_definitions(oxref):
+    """Act::apply / Act::scalar (src/moe.rs:18-46): SiLU, GELU-tanh (gelu_pytorch_tanh, src/kernels.rs:2233-2239) and
+    DeepSeek V4's clamped SiLU against torch's silu, gelu(approximate="tanh") and clamp evaluated in f64: a dropped clamp,
+    a clamp on the wrong side, a wrong constant or gate and up swapped each fail one of these."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(3)
+    g = np.concatenate([rng.normal(0, 3, 4000), np.linspace(-30, 30, 301), [0.0, -0.0, 7.0, -7.0, 6.999, 7.001]]).astype(np.float32)
+    u = np.concatenate([rng.normal(0, 4, 4000), np.linspace(12, -12, 301), [1.0, -1.0, 9.0, -9.0, 7.0, -7.0]]).astype(np.float32)
+    g64, u64 = torch.from_numpy(g).double(), torch.from_numpy(u).double()
+    lim = 7.0
+    refs = {0: F.silu(g64) * u64, 1: F.gelu(g64, approximate="tanh") * u64,
+            2: F.silu(torch.clamp(g64, max=lim)) * torch.clamp(u64, -lim, lim)}
+    for kind, ref in refs.items():
+        ref = ref.numpy()
+        tol = 2e-6 * np.maximum(np.abs(ref), 1e-3)
+        got = oxref.act_apply(kind, lim, g, u)
+        assert (np.abs(got - ref) <= tol).all(), kind
+        sc = np.array([oxref.act_scalar(kind, lim, a, b) for a, b in zip(g[:500], u[:500])], np.float64)
+        assert (np.abs(sc - ref[:500]) <= tol[:500]).all(), kind
+    # kind 0 is silu_mul bit for bit (the MoE decode path's composition rests on it)
+    assert np.array_equal(oxref.act_apply(0, 0.0, g, u).view(np.uint32), oxref.silu_mul(g, u).view(np.uint32))
+    # the clamp really bites: an up value past the limit and a gate past it change the result
+    assert oxref.act_scalar(2, 1.0, 0.5, 5.0) == oxref.act_scalar(0, 0.0, 0.5, 1.0)
+    assert oxref.act_scalar(2, 1.0, 5.0, 0.5) == oxref.act_scalar(0, 0.0, 1.0, 0.5)
+    assert oxref.act_scalar(2, 1.0, -5.0, 0.5) == oxref.act_scalar(0, 0.0, -5.0, 0.5)  # the gate is clamped from above only
+
+
+@pytest.mark.parametrize("act,param", [(1, 0.0), (2, 0.1)])
+@pytest.mark.parametrize("split", [False, True])
+def test_moe_activation_kinds_and_split_experts_against_f64(oxref, act, param, split):
+    """MoeAct::GeluTanh / SiluClamp(l) and split gate / up experts (src/gpu.rs:35-54, :206-216) against the f64 definition
+    y[t] += sum_j w_j * Down_e(act(G_e x) * (U_e x)), brute force on tiny shapes; fused and split experts holding the
+    same rows give the same bits."""
+    import torch
+    import torch.nn.functional as F
+    from oxinfer_amd import synth
+    ne, h, inter, k, t = 5, 128, 64, 2, 9
+    g_ = [mlx_case(oxref, inter, h, 300 + e, False)[1] for e in range(ne)]
+    u_ = [mlx_case(oxref, inter, h, 400 + e, False)[1] for e in range(ne)]
+    dn = [mlx_case(oxref, h, inter, 500 + e, False)[1] for e in range(ne)]
+    fused = [tuple(np.concatenate([a, b]) for a, b in zip(g_[e], u_[e])) for e in range(ne)]
+    x = synth.activations(t, h, 11)
+    logits = synth.router_logits(t, ne, 12)
+    idx = np.zeros((t, k), np.uint32)
+    w = np.zeros((t, k), np.float32)
+    for i in range(t):
+        idx[i], w[i] = oxref.route_top_k(logits[i], k)
+    y0 = np.zeros((t, h), np.float32)
+
+    def act64(g, u):
+        g, u = torch.from_numpy(g), torch.from_numpy(u)
+        if act == 1:
+            return (F.gelu(g, approximate="tanh") * u).numpy()
+        return (F.silu(torch.clamp(g, max=param)) * torch.clamp(u, -param, param)).numpy()
+    ref = y0.astype(np.float64).copy()
+    clamped = 0
+    for i in range(t):
+        for j in range(k):
+            e = int(idx[i, j])
+            wg = oxref.dequant_rows_q4(*g_[e], 64, inter, h).astype(np.float64)
+            wu = oxref.dequant_rows_q4(*u_[e], 64, inter, h).astype(np.float64)
+            wd = oxref.dequant_rows_q4(*dn[e], 64, h, inter).astype(np.float64)
+            g, u = wg @ x[i].astype(np.float64), wu @ x[i].astype(np.float64)
+            clamped += int((np.abs(u) > param).sum() + (g > param).sum())
+            ref[i] += float(w[i, j]) * (wd @ act64(g, u))
+    if act == 2:
+        assert clamped > 50  # the limit is inside the data's range
+    kw = dict(up=u_, act=act, act_param=param) if split else dict(act=act, act_param=param)
+    first = g_ if split else fused
+    grouped = oxref.moe_q4(first, dn, 64, h, inter, x, t, idx, w, y0, decode_path=False, **kw)
+    assert row_err(grouped, ref) < 1e-4
+    dec = oxref.moe_q4(first, dn, 64, h, inter, x, t, idx, w, y0, decode_path=True, **kw)
+    assert row_err(dec, ref) < 3e-2
+    if split:
+        for path in (False, True):
+            a = oxref.moe_q4(g_, dn, 64, h, inter, x, t, idx, w, y0, decode_path=path, up=u_, act=act, act_param=param)
+            b = oxref.moe_q4(fused, dn, 64, h, inter, x, t, idx, w, y0, decode_path=path, act=act, act_param=param)
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), path

@@ -61,6 +61,26 @@ def test_no_alloc_decode_matches_decode_twice(be, oxref):
     del w1, w2, w3
 
 
+def test_no_alloc_call_leaves_device_memory_alone(be, oxref):
+    """The property the entry point exists for: once the weight and the buffers are there, a call allocates and frees
+    nothing on the device (free memory as the driver reports it is the same before and after), on a K-sliced shape and on
+    one whose K stays inside a workgroup."""
+    import torch
+    for kind, n_out, n_in, t in ((Q8_0, 528, 14336, 8), (Q4_K, 64, 1024, 2)):
+        raw, _ = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 4200)
+        w = be.upload_gguf(kind, raw, n_out, n_in)
+        xa = be.quantize_act(torch.ones((t, n_in), dtype=torch.float32, device="cuda"))
+        y = torch.empty((t, n_out), dtype=torch.float32, device="cuda")
+        assert be.decode_noalloc(w, xa, t=t, y=y) is not None, be.last_error()   # warm: the kernel's code object is loaded
+        torch.cuda.synchronize()
+        free0, _ = torch.cuda.mem_get_info()
+        for _ in range(3):
+            assert be.decode_noalloc(w, xa, t=t, y=y) is not None, be.last_error()
+        torch.cuda.synchronize()
+        free1, _ = torch.cuda.mem_get_info()
+        assert free1 == free0, (free0, free1)
+
+
 def test_no_alloc_rejects_what_the_scratch_cannot_hold(be):
     n_out, n_in = 16640, 32768  # 8 K slices x 8 x 16640 floats of partial rows > 4 MiB
     raw = np.zeros(n_out * (n_in // 256) * 144, np.uint8)
