@@ -41,7 +41,7 @@ enum {
 };
 
 /* GGUF type ids handled (src/ggml.rs:42-93). */
-enum { OXHIP_GGML_Q4_0 = 2, OXHIP_GGML_Q8_0 = 8, OXHIP_GGML_Q4_K = 12, OXHIP_GGML_Q5_K = 13, OXHIP_GGML_Q6_K = 14, OXHIP_GGML_MXFP4 = 39, OXHIP_GGML_F8E4M3 = 0x1000 };
+enum { OXHIP_GGML_Q4_0 = 2, OXHIP_GGML_Q8_0 = 8, OXHIP_GGML_Q4_K = 12, OXHIP_GGML_Q5_K = 13, OXHIP_GGML_Q6_K = 14, OXHIP_GGML_MXFP4 = 39, OXHIP_GGML_NVFP4 = 40, OXHIP_GGML_F8E4M3 = 0x1000 };
 
 typedef struct {
     uint32_t kind;            /* OXHIP_W_* */
@@ -51,7 +51,8 @@ typedef struct {
     const void* scales;
     const void* offsets;
     uint32_t group;           /* elements per offset (Q4) / per scale and bias (MLX) */
-    const float* block_scales;/* FP8: [ceil(n_out/bs_rows), ceil(n_in/bs_cols)] */
+    const float* block_scales;/* FP8: [ceil(n_out/bs_rows), ceil(n_in/bs_cols)]; NVFP4: the same, optional (its global scale:
+                                 one block spanning the matrix, src/model.rs:550-557), on top of the decoded values */
     uint32_t bs_rows, bs_cols;
 } oxhip_weight_desc;
 
@@ -111,8 +112,8 @@ size_t oxhip_weight_bytes(const oxhip_weight* w);
 /* Backend::matmul (src/gpu.rs:160; src/cuda.rs:1428-1493): all jobs share x [t, n_in] (host f32);
  * computes every job or none. Routing as matmul_quant_multi_at's (src/kernels.rs:1731-1879): up to 8 tokens the
  * Q8 / Q8_0 / Q4_K / Q5_K / Q6_K / MXFP4 / MLX 4-bit jobs share one launch of the int8 decode kernel (the CPU's decode semantics,
- * src/kernels.rs:1908-1928); more than 16 tokens over MLX 4-bit, Q8, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4 or FP8 (128-column blocks)
- * weights run the bf16 matrix-core GEMM; everything else runs the decode kernels over 16 tokens at a time. */
+ * src/kernels.rs:1908-1928); more than 16 tokens over MLX 4-bit, Q8, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4, NVFP4 or FP8 (128-column
+ * blocks) weights run the bf16 matrix-core GEMM; everything else runs the decode kernels over 16 tokens at a time. */
 int oxhip_matmul(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_job* jobs, size_t n_jobs);
 /* Backend::matvec_rows (src/gpu.rs:165): t in 1..=4. */
 int oxhip_matvec_rows(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_rows_job* jobs, size_t n_jobs);

@@ -235,6 +235,7 @@ size_t oxref_block_size(uint32_t kind) {
         case OXREF_F32: case OXREF_F16: case OXREF_BF16: case OXREF_F8E4M3: return 1;
         case OXREF_Q4_0: case OXREF_Q4_1: case OXREF_Q5_0: case OXREF_Q5_1: case OXREF_Q8_0: case OXREF_MXFP4: return 32;
         case OXREF_Q2_K: case OXREF_Q4_K: case OXREF_Q5_K: case OXREF_Q6_K: return QK_K;
+        case OXREF_NVFP4: return 64;
         default: return 0;
     }
 }
@@ -253,6 +254,7 @@ size_t oxref_type_size(uint32_t kind) {
         case OXREF_Q5_K: return 176;
         case OXREF_Q6_K: return 210;
         case OXREF_MXFP4: return 17;
+        case OXREF_NVFP4: return 36;
         default: return 0;
     }
 }
@@ -332,6 +334,15 @@ uint64_t oxref_fnv1a_f32(const float* v, size_t n) {
 // 2^(e - 128) (src/ggml.rs:466-475: the two smallest codes are subnormal f32 values).
 static const int8_t KVALUES_MXFP4[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
 static float e8m0_half(uint8_t e) { return e < 2 ? bits_f32(0x00200000u << e) : bits_f32(((uint32_t)e - 1) << 23); }
+// NVFP4: half the value of an unsigned E4M3 scale byte (src/ggml.rs:477-490): bits 3..6 the exponent (bias 7), bits 0..2
+// the mantissa, subnormals m 2^-9; 0 and 0x7f decode to 0; bit 7 is not looked at.
+float oxref_ue4m3_half(uint8_t x) {
+    if (x == 0 || x == 0x7F) return 0.0f;
+    int e = (x >> 3) & 0xF;
+    float m = (float)(x & 7);
+    float raw = e == 0 ? m * std::ldexp(1.0f, -9) : (1.0f + m / 8.0f) * std::ldexp(1.0f, e - 7);
+    return raw * 0.5f;
+}
 
 // ---------------------------------------------------------------------------------------------
 // dequantize_row (src/ggml.rs:630-793; MXFP4 :922-928)
@@ -370,6 +381,17 @@ void oxref_dequantize_row(uint32_t kind, const uint8_t* src, size_t n, float* ou
                 for (int j = 0; j < 16; j++) {
                     y[j] = d * (float)KVALUES_MXFP4[b[1 + j] & 0xF];
                     y[j + 16] = d * (float)KVALUES_MXFP4[b[1 + j] >> 4];
+                }
+                break;
+            }
+            case OXREF_NVFP4: {  // src/ggml.rs:936-947: four sub-blocks of 16, scale byte s, then 8 bytes: elements j (low) and j + 8 (high)
+                for (int sb = 0; sb < 4; sb++) {
+                    float d = oxref_ue4m3_half(b[sb]);
+                    const uint8_t* q = b + 4 + 8 * sb;
+                    for (int j = 0; j < 8; j++) {
+                        y[16 * sb + j] = d * (float)KVALUES_MXFP4[q[j] & 0xF];
+                        y[16 * sb + j + 8] = d * (float)KVALUES_MXFP4[q[j] >> 4];
+                    }
                 }
                 break;
             }
@@ -1123,6 +1145,19 @@ void oxref_gemm_f32(const float* w, size_t n_out, size_t n_in, const float* x, s
     });
 }
 
+// GgufMatrix::dequantize_rows for a block format that carries scales on top of what its kind decodes (NVFP4's global
+// scale; src/ggml.rs:420-432): dequantize_row, then every run of `bcols` columns times s[(r / brows) * ncb + c / bcols].
+void oxref_gguf_dequant_rows_scaled(uint32_t kind, const uint8_t* data, const float* scales, size_t n_in, size_t brows, size_t bcols,
+                                    size_t r0, size_t r1, float* out) {
+    size_t rb = oxref_row_bytes(kind, n_in), ncb = scales ? (n_in + bcols - 1) / bcols : 0;
+    for (size_t r = r0; r < r1; r++) {
+        float* o = out + (r - r0) * n_in;
+        oxref_dequantize_row(kind, data + r * rb, n_in, o);
+        if (!scales) continue;
+        for (size_t c = 0; c < n_in; c++) o[c] *= scales[(r / brows) * ncb + c / bcols];
+    }
+}
+
 void oxref_gemm_quant(int64_t kind, const void* data, const void* aux0, const void* aux1, size_t group,
                       size_t brows, size_t bcols, size_t n_out, size_t n_in, const float* x, size_t t,
                       float* y, int threads) {
@@ -1144,6 +1179,9 @@ void oxref_gemm_quant(int64_t kind, const void* data, const void* aux0, const vo
             else if (kind == OXREF_F8E4M3)
                 oxref_fp8_dequant_rows((const uint8_t*)data, (const float*)aux0, n_out, n_in, brows, bcols, r, r + rows,
                                        scratch.data());
+            else if (kind == OXREF_NVFP4)  // float-stored (is_float, src/ggml.rs:219-224), its global scale in aux0 (may be null)
+                oxref_gguf_dequant_rows_scaled((uint32_t)kind, (const uint8_t*)data, (const float*)aux0, n_in, brows, bcols, r, r + rows,
+                                               scratch.data());
             else
                 for (size_t i = 0; i < rows; i++)
                     oxref_dequantize_row((uint32_t)kind, (const uint8_t*)data + (r + i) * row_bytes, n_in,

@@ -11,6 +11,7 @@
  *                                 by gguf-py / ggml C, for every type restated here
  *   decode_i8 ................... invariant s*q+m == dequantize_row within 1e-6 (src/ggml.rs:1663-1681)
  *   e4m3 ........................ closed form + torch.float8_e4m3fn over all 256 bytes
+ *   NVFP4 ....................... every (scale byte, code) pair against torch.float8_e4m3fn and the E2M1 definition
  *   quantize_act ................ scalar definition (src/quant.rs:645-656), special cases
  *   from_mlx_q4 ................. invariant against mlx_dequant_row, exact where representable
  *   integer dot products ........ brute force; power-of-two scales make the f32 math exact
@@ -34,7 +35,7 @@ extern "C" {
 enum {
     OXREF_F32 = 0, OXREF_F16 = 1, OXREF_Q4_0 = 2, OXREF_Q4_1 = 3, OXREF_Q5_0 = 6, OXREF_Q5_1 = 7,
     OXREF_Q8_0 = 8, OXREF_Q2_K = 10, OXREF_Q3_K = 11, OXREF_Q4_K = 12, OXREF_Q5_K = 13,
-    OXREF_Q6_K = 14, OXREF_BF16 = 30, OXREF_MXFP4 = 39, OXREF_F8E4M3 = 0x1000
+    OXREF_Q6_K = 14, OXREF_BF16 = 30, OXREF_MXFP4 = 39, OXREF_NVFP4 = 40, OXREF_F8E4M3 = 0x1000
 };
 
 /* conversions (half crate 2.7.1 semantics: IEEE RNE) */
@@ -54,6 +55,11 @@ uint64_t oxref_fnv1a_f32(const float* v, size_t n);
 
 void oxref_dequantize_row(uint32_t kind, const uint8_t* src, size_t n, float* out);
 int  oxref_decode_i8(uint32_t kind, const uint8_t* blk, int8_t* q, float* s, float* m);
+
+/* NVFP4 (src/ggml.rs:79-83, :477-490, :936-947): half an unsigned E4M3 scale byte; rows with the matrix's scales on top. */
+float oxref_ue4m3_half(uint8_t x);
+void  oxref_gguf_dequant_rows_scaled(uint32_t kind, const uint8_t* data, const float* scales, size_t n_in, size_t brows, size_t bcols,
+                                     size_t r0, size_t r1, float* out);
 
 float oxref_e4m3_to_f32(uint8_t b);
 void  oxref_e4m3_scaled(const uint8_t* src, size_t n, float s, float* out);

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "liboxref.so")
 
 F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 = 0, 1, 2, 3, 6, 7, 8
-Q2_K, Q4_K, Q5_K, Q6_K, BF16, MXFP4, F8E4M3 = 10, 12, 13, 14, 30, 39, 0x1000
+Q2_K, Q4_K, Q5_K, Q6_K, BF16, MXFP4, NVFP4, F8E4M3 = 10, 12, 13, 14, 30, 39, 40, 0x1000
 NAMES = {F32: "F32", F16: "F16", Q4_0: "Q4_0", Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q8_0: "Q8_0",
          Q2_K: "Q2_K", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", BF16: "BF16", MXFP4: "MXFP4"}
 
@@ -43,6 +43,8 @@ def _load():
         "oxref_dequantize_row": (None, [C.c_uint32, vp, sz, vp]),
         "oxref_decode_i8": (C.c_int, [C.c_uint32, vp, vp, vp, vp]),
         "oxref_e4m3_to_f32": (C.c_float, [C.c_uint8]),
+        "oxref_ue4m3_half": (C.c_float, [C.c_uint8]),
+        "oxref_gguf_dequant_rows_scaled": (None, [C.c_uint32, vp, vp, sz, sz, sz, sz, sz, vp]),
         "oxref_e4m3_scaled": (None, [vp, sz, C.c_float, vp]),
         "oxref_fp8_dequant_rows": (None, [vp, vp, sz, sz, sz, sz, sz, sz, vp]),
         "oxref_quantize_act": (None, [vp, sz, sz, vp, vp, vp, vp, vp]),
@@ -160,6 +162,20 @@ def fp8_dequant_rows(data, scales, n_out, n_in, brows=128, bcols=128, r0=0, r1=N
     data, scales = _c(data, np.uint8), _c(scales, np.float32)
     out = np.empty((r1 - r0, n_in), np.float32)
     lib.oxref_fp8_dequant_rows(_p(data), _p(scales), n_out, n_in, brows, bcols, r0, r1, _p(out))
+    return out
+
+
+def ue4m3_half(b):
+    return lib.oxref_ue4m3_half(int(b))
+
+
+def gguf_dequant_rows_scaled(kind, data, scales, n_out, n_in, brows=None, bcols=None, r0=0, r1=None):
+    """GgufMatrix::dequantize_rows with block scales on top of the kind's own decoding (NVFP4's global scale)."""
+    r1 = n_out if r1 is None else r1
+    data = _c(data, np.uint8)
+    scales = None if scales is None else _c(scales, np.float32)
+    out = np.empty((r1 - r0, n_in), np.float32)
+    lib.oxref_gguf_dequant_rows_scaled(kind, _p(data), _p(scales), n_in, brows or n_out, bcols or n_in, r0, r1, _p(out))
     return out
 
 

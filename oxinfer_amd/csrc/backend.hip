@@ -365,6 +365,31 @@ static oxhip_weight* upload_weight(oxhip_ctx* c, const oxhip_weight_desc* d, boo
             }
             size_t raw_bytes;
             int np;
+            if (d->ggml_type == OXHIP_GGML_NVFP4) {
+                // ggml's blocks of 64 (36 B) with, optionally, the matrix's scales on top (compressed-tensors' global scale
+                // as a whole-matrix block, src/model.rs:550-557; any block geometry whose blocks are whole tiles)
+                if (n_in % 64) return fail("NVFP4 rows must be whole blocks of 64");
+                const bool scaled = d->block_scales != nullptr;
+                if (scaled && (!d->bs_rows || !d->bs_cols)) return fail("NVFP4 scales need their block geometry");
+                if (scaled && !((d->bs_rows % 16 == 0 || d->bs_rows >= n_out) && (d->bs_cols % 128 == 0 || d->bs_cols >= n_in)))
+                    return fail("NVFP4 scale blocks must be multiples of 16 rows x 128 columns (or span the matrix)");
+                w->v.fmt = FMT_NVFP4;
+                w->v.br = scaled ? d->bs_rows : 0;
+                w->v.bc = scaled ? d->bs_cols : 0;
+                const size_t ns = scaled ? ((n_out + d->bs_rows - 1) / d->bs_rows) * ((n_in + d->bs_cols - 1) / d->bs_cols) : 0;
+                pl.add(0, t4n_bytes((uint32_t)n_out, (uint32_t)n_in));
+                if (scaled) pl.add(1, ns * 4);
+                if (!alloc(pl, scaled ? 2 : 1)) return fail("device memory short");
+                if (scaled && hipMemcpyAsync(static_cast<uint8_t*>(w->base) + pl.off[1], d->block_scales, ns * 4, hipMemcpyHostToDevice, s) != hipSuccess)
+                    return fail("copy failed");
+                raw_bytes = n_out * (n_in / 64) * 36;
+                Temp raw;
+                if (!have_memory(raw_bytes) || !raw.put(d->data, raw_bytes, s)) return fail("device memory short");
+                if (launch_repack_gguf(w->v.fmt, static_cast<const uint8_t*>(raw.p), n_out, n_in, w->v, s) != hipSuccess)
+                    return fail("repack launch failed");
+                if (hipStreamSynchronize(s) != hipSuccess) return fail("repack failed");
+                break;
+            }
             if (d->ggml_type == OXHIP_GGML_Q8_0) {
                 if (n_in % 32) return fail("Q8_0 rows must be whole blocks of 32");
                 w->v.fmt = FMT_Q8_0;

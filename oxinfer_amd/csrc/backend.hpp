@@ -117,6 +117,7 @@ inline oxhip_qact carve_qact(void* base, size_t t, size_t n_in) {
     return a;
 }
 
-inline bool is_dense(const oxhip_weight* w) { return w->v.fmt == FMT_FP8 || w->v.fmt == FMT_BF16; }
+// float-stored matrices (is_float, src/ggml.rs:219-224): f32 activations at decode sizes
+inline bool is_dense(const oxhip_weight* w) { return w->v.fmt == FMT_FP8 || w->v.fmt == FMT_BF16 || w->v.fmt == FMT_NVFP4; }
 
 }  // namespace oxhip

@@ -16,6 +16,7 @@
 // nibble codes is folded through the per-16 integer sums of the activations, so no
 // per-element subtraction is needed.
 #include "internal.hpp"
+#include "layout.hpp"
 
 namespace oxhip {
 
@@ -202,6 +203,91 @@ __global__ __launch_bounds__(256) void decode_dense_kernel(WeightView w, const f
     }
 }
 
+// ---- NVFP4 (float-stored: f32 activations, src/ggml.rs:219-224) from its tile records --------------------------------
+// A workgroup of 8 waves owns a row tile and splits its K-steps; lane 16 kq + n of a wave owns row n's 32 weights of
+// the step that its 16 bytes hold (layout.hpp), dequantized as the reference does ((scale / 2) * doubled value, then the
+// matrix's scale) and multiplied with the f32 activations in f32. T tokens per pass.
+template <int T>
+__global__ __launch_bounds__(512) void decode_nvfp4_kernel(WeightView w, const float* __restrict__ x, float* __restrict__ y) {
+    __shared__ float red[8][T][16];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, kq = lane >> 4;
+    const uint32_t nsteps = t4m_steps(w.n_in), tile = blockIdx.x, row = tile * 16 + n;
+    const uint8_t* base = w.p0 + (size_t)tile * nsteps * T4N_REC;
+    const float* bs = reinterpret_cast<const float*>(w.p1);
+    const uint32_t ncb = w.br ? (w.n_in + w.bc - 1) / w.bc : 0;
+    float acc[T];
+#pragma unroll
+    for (int c = 0; c < T; c++) acc[c] = 0.0f;
+    for (uint32_t s = wave; s < nsteps; s += 8) {
+        const uint8_t* rec = base + (size_t)s * T4N_REC;
+        const uint4 cv = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+        const uint2 sv = *reinterpret_cast<const uint2*>(rec + 1024 + 8 * n);
+        const uint32_t cw[4] = {cv.x, cv.y, cv.z, cv.w};
+        const float g = w.br ? bs[(size_t)(min(row, w.n_out - 1) / w.br) * ncb + (128 * s) / w.bc] : 1.0f;
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            if (128 * s + 32 * b >= w.n_in) break;  // a row's last step may hold fewer than four groups of 32 (uniform)
+            const uint32_t sw = b < 2 ? sv.x : sv.y;
+            const float d[2] = {ue4m3_half(sw >> (16 * (b & 1))), ue4m3_half(sw >> (16 * (b & 1) + 8))};
+#pragma unroll
+            for (int h = 0; h < 2; h++) {  // the low nibbles: columns 32 b + 4 kq + j; the high ones: + 16
+                const uint32_t kv4 = mxfp4_values<0>((cw[b] >> (4 * h)) & 0x0F0F0F0Fu);
+                float wf[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    wf[j] = d[h] * (float)(int)(int8_t)((kv4 >> (8 * j)) & 0xFF);
+                    if (w.br) wf[j] *= g;
+                }
+                const size_t col = (size_t)128 * s + 32 * b + 16 * h + 4 * kq;
+#pragma unroll
+                for (int c = 0; c < T; c++) {
+                    const float4 xv = *reinterpret_cast<const float4*>(x + (size_t)c * w.n_in + col);
+                    acc[c] = __builtin_fmaf(wf[0], xv.x, acc[c]);
+                    acc[c] = __builtin_fmaf(wf[1], xv.y, acc[c]);
+                    acc[c] = __builtin_fmaf(wf[2], xv.z, acc[c]);
+                    acc[c] = __builtin_fmaf(wf[3], xv.w, acc[c]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < T; c++) {
+        float v = acc[c];
+        v += __shfl_xor(v, 16);
+        v += __shfl_xor(v, 32);
+        if (kq == 0) red[wave][c][n] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < 16 * T) {
+        const uint32_t c = threadIdx.x / 16, nn = threadIdx.x % 16;
+        float v = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; k++) v += red[k][c][nn];
+        if (tile * 16 + nn < w.n_out) y[(size_t)c * w.n_out + tile * 16 + nn] = v;
+    }
+}
+
+hipError_t launch_decode_nvfp4(const WeightView& w, const float* x, size_t t, float* y, hipStream_t s) {
+    if (w.fmt != FMT_NVFP4 || !x || reinterpret_cast<uintptr_t>(x) % 16) return hipErrorInvalidValue;  // (rows are multiples of 64 floats)
+    const unsigned grid = row_tiles(w.n_out);
+    size_t c0 = 0;
+    while (c0 < t) {
+        const size_t tc = t - c0 < 4 ? t - c0 : 4;
+        const float* xi = x + c0 * w.n_in;
+        float* yo = y + c0 * w.n_out;
+        switch (tc) {
+            case 1: decode_nvfp4_kernel<1><<<grid, 512, 0, s>>>(w, xi, yo); break;
+            case 2: decode_nvfp4_kernel<2><<<grid, 512, 0, s>>>(w, xi, yo); break;
+            case 3: decode_nvfp4_kernel<3><<<grid, 512, 0, s>>>(w, xi, yo); break;
+            default: decode_nvfp4_kernel<4><<<grid, 512, 0, s>>>(w, xi, yo); break;
+        }
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        c0 += tc;
+    }
+    return hipSuccess;
+}
+
 // ---- exact integer accumulators (parity checks): one thread per (token, row, unit) ---------------
 template <int FMT>
 __global__ __launch_bounds__(256) void isums_kernel(WeightView w, QActView xa, uint32_t t, int32_t* __restrict__ out) {
@@ -301,6 +387,7 @@ static hipError_t launch_decode_plain(const WeightView& w, const QActView& xa, c
                 return launch_skinny_fp8(w, x, false, true, t, y, false, sc.partial, s);
             return decode_dense_t<FMT_FP8, 4>(w, x, t, y, s);
         case FMT_BF16: return decode_dense_t<FMT_BF16, 4>(w, x, t, y, s);
+        case FMT_NVFP4: return launch_decode_nvfp4(w, x, t, y, s);
         default: return hipErrorInvalidValue;
     }
 }

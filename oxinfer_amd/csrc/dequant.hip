@@ -9,6 +9,7 @@
 //   Q5_K  the same with v = nibble + 16 * fifth bit       src/ggml.rs:750-773
 //   Q6_K  (d * sc) * q, q = 6-bit code - 32               src/ggml.rs:774-793
 //   MXFP4 2^(e - 128) * doubled E2M1 value               src/ggml.rs:922-928
+//   NVFP4 (ue4m3(scale) / 2) * doubled E2M1 value, then * the matrix's scale   src/ggml.rs:936-947, :420-432
 //   FP8   e4m3(byte) * block scale                        src/ggml.rs:282-293, :433-444
 //   MLX 4-bit -> Q4 + offsets                             src/quant.rs:518-563
 #include "internal.hpp"
@@ -83,6 +84,16 @@ __global__ __launch_bounds__(256) void dequantize_kernel(WeightView w, uint32_t 
             const uint32_t code = hi ? (byte >> 4) : (byte & 0xF);
             const int kv = (int)(int8_t)(mxfp4_values<0>(code) & 0xFF);
             v = e8m0_half(rec[1024 + 4 * nn + bi]) * (float)kv;
+            break;
+        }
+        case FMT_NVFP4: {
+            uint32_t tile = r >> 4, nn = r & 15, b = c >> 5, st = b >> 2, bi = b & 3, e = c & 31, hi = e >> 4, pp = e & 15, kq = pp >> 2;
+            const uint8_t* rec = w.p0 + ((size_t)tile * t4m_steps(n) + st) * T4N_REC;
+            uint8_t byte = rec[16 * (kq * 16 + nn) + 4 * bi + (pp & 3)];
+            const uint32_t code = hi ? (byte >> 4) : (byte & 0xF);
+            const int kv = (int)(int8_t)(mxfp4_values<0>(code) & 0xFF);
+            v = ue4m3_half(rec[1024 + 8 * nn + 2 * bi + hi]) * (float)kv;
+            if (w.br) v *= reinterpret_cast<const float*>(w.p1)[(r / w.br) * ((n + w.bc - 1) / w.bc) + c / w.bc];
             break;
         }
         case FMT_Q40: {  // (nib - 8) * d, no offset term (src/ggml.rs:675-683)
@@ -261,6 +272,35 @@ __global__ __launch_bounds__(256) void pack_t4x_kernel(const uint8_t* __restrict
     if (kq == 0) *reinterpret_cast<uint32_t*>(rec + 1024 + 4 * nn) = sc;
 }
 
+// ggml NVFP4 blocks (four scale bytes, then per sub-block of 16 eight bytes: elements j low, j + 8 high; src/ggml.rs:936-947)
+// -> T4N records; one thread per lane slot of a record.
+__global__ __launch_bounds__(256) void pack_t4n_kernel(const uint8_t* __restrict__ raw, uint32_t n_out, uint32_t n_in, uint8_t* __restrict__ dst) {
+    const uint32_t nsteps = t4m_steps(n_in), nb64 = n_in / 64;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x, total = (size_t)row_tiles(n_out) * nsteps * 64;
+    if (idx >= total) return;
+    const uint32_t l = idx & 63, nn = l & 15, kq = l >> 4;
+    const size_t ts = idx >> 6, tile = ts / nsteps, row = tile * 16 + nn;
+    const uint32_t st = (uint32_t)(ts % nsteps);
+    uint8_t* rec = dst + ts * T4N_REC;
+    uint32_t out[4] = {0, 0, 0, 0}, sc[2] = {0, 0};
+    for (uint32_t b = 0; b < 4; b++) {  // the step's 32-column group b: sub-blocks 2 (b & 1), 2 (b & 1) + 1 of block 2 st + b / 2
+        const uint32_t blk = 2 * st + (b >> 1);
+        if (row >= n_out || blk >= nb64) continue;
+        const uint8_t* src = raw + ((size_t)row * nb64 + blk) * 36;
+        const uint32_t s0 = 2 * (b & 1);
+        for (uint32_t j = 0; j < 4; j++) {
+            // element e of a sub-block: byte e % 8 of its eight, low nibble for e < 8
+            const uint32_t e = 4 * kq + j;
+            const uint32_t lo = (src[4 + 8 * s0 + (e & 7)] >> (4 * (e >> 3))) & 0xF;
+            const uint32_t hi = (src[4 + 8 * (s0 + 1) + (e & 7)] >> (4 * (e >> 3))) & 0xF;
+            out[b] |= (lo | (hi << 4)) << (8 * j);
+        }
+        sc[b >> 1] |= ((uint32_t)src[s0] | ((uint32_t)src[s0 + 1] << 8)) << (16 * (b & 1));
+    }
+    *reinterpret_cast<uint4*>(rec + 16 * l) = make_uint4(out[0], out[1], out[2], out[3]);
+    if (kq == 0) *reinterpret_cast<uint2*>(rec + 1024 + 8 * nn) = make_uint2(sc[0], sc[1]);
+}
+
 hipError_t launch_pack_q4m(const uint8_t* q, const uint16_t* sc, const uint16_t* off, size_t n_out, size_t n_in, uint8_t* dst,
                            hipStream_t s) {
     size_t total = (size_t)row_tiles((uint32_t)n_out) * t4m_steps((uint32_t)n_in) * 64;
@@ -380,6 +420,10 @@ hipError_t launch_repack_gguf(int fmt, const uint8_t* raw, size_t n_out, size_t 
         size_t total = (size_t)row_tiles((uint32_t)n_out) * t4m_steps((uint32_t)n_in) * 64;
         if (!total) return hipSuccess;
         pack_t4x_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
+    } else if (fmt == FMT_NVFP4) {
+        size_t total = (size_t)row_tiles((uint32_t)n_out) * t4m_steps((uint32_t)n_in) * 64;
+        if (!total) return hipSuccess;
+        pack_t4n_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(raw, (uint32_t)n_out, (uint32_t)n_in, p0);
     } else if (fmt == FMT_Q6_K) {
         size_t total = (size_t)row_tiles((uint32_t)n_out) * t6k_steps((uint32_t)n_in) * 64;
         if (!total) return hipSuccess;

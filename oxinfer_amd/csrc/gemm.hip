@@ -119,6 +119,8 @@ hipError_t launch_pack_a(const void* x, bool src_bf16, int mode, size_t t, size_
 
 namespace {
 
+// the formats in the T4M code geometry (NVFP4's records too: float-stored, so not one of the int8 decode formats)
+__host__ __device__ constexpr bool t4_geometry(int f) { return t4m_format(f) || f == FMT_NVFP4; }
 
 typedef uint32_t u32x4g __attribute__((ext_vector_type(4)));
 constexpr int WG_NT = 8;   // row tiles per workgroup (128 rows), or 7 where that fills more CUs (gemm_row_tiles)
@@ -191,8 +193,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
 #pragma unroll
     for (int i = 0; i < DT; i++) {
         const uint32_t tile = min(nt0 + DT * wave + i, ntiles - 1);
-        if (t4m_format(FMT)) {
-            wbase[i] = w.p0 + ((size_t)tile * all_steps + step0) * (FMT == FMT_MXFP4 ? T4X_REC : T4M_REC);
+        if (t4_geometry(FMT)) {
+            wbase[i] = w.p0 + ((size_t)tile * all_steps + step0) * (FMT == FMT_MXFP4 ? T4X_REC : T4M_REC);  // (T4N_REC == T4M_REC)
         } else if (q8_format(FMT)) {  // the tile's records; load_raw indexes them from the matrix's first step
             wbase[i] = w.p0 + (size_t)tile * t8_steps(w.n_in) * (FMT == FMT_Q8F ? T8F_REC : T8_REC);
         } else if (k45_format(FMT)) {
@@ -222,7 +224,17 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
     };
     auto load_raw_tile = [&](Raw* r, int i, uint32_t s) {  // the records of the wave's row tile i at step s
         if (NT % WAVES == 0 || DT * wave + i < NT) {  // (with NT = 7 the eighth wave has no tile)
-            if (t4m_format(FMT)) {
+            if (FMT == FMT_NVFP4) {  // the row's eight sub-block scale bytes, and the matrix's scale of this step's columns
+                const uint8_t* rec = wbase[i] + (size_t)s * T4N_REC;
+                r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
+                const uint2 sv = *reinterpret_cast<const uint2*>(rec + 1024 + 8 * n);
+                r[i].m[0] = sv.x;
+                r[i].m[1] = sv.y;
+                const uint32_t tile = min(nt0 + DT * wave + i, ntiles - 1);
+                r[i].m[2] = w.br ? __float_as_uint(reinterpret_cast<const float*>(w.p1)[(size_t)(min(tile * 16 + n, w.n_out - 1) / w.br) * ((w.n_in + w.bc - 1) / w.bc) +
+                                                                                    (128 * (step0 + s)) / w.bc])
+                                 : 0x3F800000u;
+            } else if (t4m_format(FMT)) {
                 const uint8_t* rec = wbase[i] + (size_t)s * (FMT == FMT_MXFP4 ? T4X_REC : T4M_REC);
                 r[i].c = *reinterpret_cast<const uint4*>(rec + 16 * lane);
                 r[i].m[0] = *reinterpret_cast<const uint32_t*>(rec + 1024 + 4 * n);
@@ -280,7 +292,21 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_bf16_kernel(WeightView w, con
     auto dequant_tile = [&](const Raw& r, int i, uint32_t buf, uint32_t s) {  // one of the wave's row tiles, 4 blocks
         if (NT % WAVES != 0 && DT * wave + i >= NT) return;
         uint4* dst = bfrag + ((size_t)(buf * 4) * NT + DT * wave + i) * 64 + lane;  // block b: + b * NT * 64
-        if (FMT == FMT_MXFP4) {  // the code's doubled value + 12 as an unsigned byte, times the block's power of two: exact in bf16
+        if (FMT == FMT_NVFP4) {  // as MXFP4 below with a scale per 16: the low nibbles' sub-block 2 b, the high nibbles' 2 b + 1
+            const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
+            const float g = __uint_as_float(r.m[2]);
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const uint32_t sw = r.m[b >> 1] >> (16 * (b & 1));
+                const float d0 = ue4m3_half(sw) * g, d1 = ue4m3_half(sw >> 8) * g;
+                const uint32_t lo = mxfp4_values<12>(cw[b] & 0x0F0F0F0Fu), hi = mxfp4_values<12>((cw[b] >> 4) & 0x0F0F0F0Fu);
+                const float c0 = -12.0f * d0, c1 = -12.0f * d1;
+                dst[b * NT * 64] = make_uint4(pack_bf16(__builtin_fmaf(byte_f32<0>(lo), d0, c0), __builtin_fmaf(byte_f32<1>(lo), d0, c0)),
+                                              pack_bf16(__builtin_fmaf(byte_f32<2>(lo), d0, c0), __builtin_fmaf(byte_f32<3>(lo), d0, c0)),
+                                              pack_bf16(__builtin_fmaf(byte_f32<0>(hi), d1, c1), __builtin_fmaf(byte_f32<1>(hi), d1, c1)),
+                                              pack_bf16(__builtin_fmaf(byte_f32<2>(hi), d1, c1), __builtin_fmaf(byte_f32<3>(hi), d1, c1)));
+            }
+        } else if (FMT == FMT_MXFP4) {  // the code's doubled value + 12 as an unsigned byte, times the block's power of two: exact in bf16
             const uint32_t cw[4] = {r.c.x, r.c.y, r.c.z, r.c.w};
 #pragma unroll
             for (int b = 0; b < 4; b++) {
@@ -570,12 +596,12 @@ hipError_t launch_gemm_reduce(const float* partial, size_t n, uint32_t slices, v
 // The formats the kernel dequantizes: tile-packed MLX 4-bit and Q4_0, Q8_0 / Q8, Q4_K, Q6_K, and FP8 rows of whole 128-column
 // steps with scale blocks of 16 k rows x 128 k columns.
 bool gemm_bf16_ok(const WeightView& w) {
-    if (t4m_format(w.fmt) || q8_format(w.fmt)) return true;
+    if (t4_geometry(w.fmt) || q8_format(w.fmt)) return true;
     if (k45_format(w.fmt) || w.fmt == FMT_Q6_K) return w.n_in % 256 == 0;
     return w.fmt == FMT_FP8 && w.br % 16 == 0 && w.bc % 128 == 0 && w.n_in % 128 == 0;
 }
 // pack_a's MODE for the format's fragments
-int gemm_bf16_pack_mode(const WeightView& w) { return t4m_format(w.fmt) ? 1 : w.fmt == FMT_FP8 ? 2 : w.fmt == FMT_Q6_K ? 3 : 0; }
+int gemm_bf16_pack_mode(const WeightView& w) { return t4_geometry(w.fmt) ? 1 : w.fmt == FMT_FP8 ? 2 : w.fmt == FMT_Q6_K ? 3 : 0; }
 
 hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size_t mtiles, void* y, bool out_bf16, float* partial,
                             hipStream_t s) {
@@ -584,6 +610,7 @@ hipError_t launch_gemm_bf16(const WeightView& w, const void* apk, size_t t, size
         case FMT_Q4M: return run_gemm_bf16<FMT_Q4M>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q40: return run_gemm_bf16<FMT_Q40>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_MXFP4: return run_gemm_bf16<FMT_MXFP4>(w, apk, t, mtiles, y, out_bf16, partial, s);
+        case FMT_NVFP4: return run_gemm_bf16<FMT_NVFP4>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q8_0: return run_gemm_bf16<FMT_Q8_0>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q8F: return run_gemm_bf16<FMT_Q8F>(w, apk, t, mtiles, y, out_bf16, partial, s);
         case FMT_Q4_K: return run_gemm_bf16<FMT_Q4_K>(w, apk, t, mtiles, y, out_bf16, partial, s);

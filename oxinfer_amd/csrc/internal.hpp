@@ -29,8 +29,10 @@ namespace oxhip {
 //   FP8   p0 q   [n_out][n_in]        e4m3 bytes (row-major, or tile-packed when group == 1: fp8_offset below);
 //         p1 bs f32 [ceil(n_out/br)][ceil(n_in/bc)]
 //   BF16  p0 q   [n_out][n_in]        bf16
+//   NVFP4 p0      T4N records (layout.hpp); p1 f32 scales on top of the decoded values [ceil(n_out/br)][ceil(n_in/bc)],
+//                 or none (br == 0). Float-stored like FP8: f32 activations at decode sizes.
 // ------------------------------------------------------------------------------------------------
-enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6, FMT_Q8F = 7, FMT_Q40 = 8, FMT_Q5_K = 9, FMT_MXFP4 = 10 };
+enum Fmt : int { FMT_Q4 = 0, FMT_Q8_0 = 1, FMT_Q4_K = 2, FMT_Q6_K = 3, FMT_FP8 = 4, FMT_BF16 = 5, FMT_Q4M = 6, FMT_Q8F = 7, FMT_Q40 = 8, FMT_Q5_K = 9, FMT_MXFP4 = 10, FMT_NVFP4 = 11 };
 // the formats of the matrix-core decode kernels (decode_mfma.hip); the two Q8 kinds carry no sums or offsets
 inline bool mfma_decode_format(int f) { return f == FMT_Q8_0 || f == FMT_Q8F || f == FMT_Q4_K || f == FMT_Q6_K || f == FMT_Q4M || f == FMT_Q40 || f == FMT_Q5_K || f == FMT_MXFP4; }
 // the two 4-bit formats in T4M records (MLX: a scale and an offset per 64; GGUF Q4_0: a scale per 32)
@@ -123,6 +125,20 @@ __host__ __device__ inline uint32_t fp8_second_chunk(const WeightView& w) { retu
 inline bool fp8_tileable(size_t n_in, uint32_t br, uint32_t bc) { return n_in % 128 == 0 && bc % 128 == 0 && br % 16 == 0; }
 hipError_t launch_pack_q8f(const int8_t* q, const float* scales, size_t n_out, size_t n_in, uint8_t* dst, hipStream_t s);
 hipError_t launch_pack_fp8(const uint8_t* raw, size_t n_out, size_t n_in, uint8_t* dst, hipStream_t s);
+// NVFP4: half the value of an unsigned E4M3 scale byte (src/ggml.rs:477-490: 0 and 0x7f decode to 0, bit 7 is ignored);
+// every value is exact in f32.
+__host__ __device__ inline float ue4m3_half(uint32_t x) {
+    x &= 0xFF;
+    if (x == 0 || x == 0x7F) return 0.0f;
+    const uint32_t e = (x >> 3) & 0xF, m = x & 7;
+    // (1 + m / 8) 2^(e - 7) / 2 = (1 + m / 8) 2^(e - 8): exponent field e - 8 + 127; subnormals m 2^-9 / 2 = m 2^-10
+    const uint32_t bits = e == 0 ? 0u : ((e + 119u) << 23) | (m << 20);
+    union { uint32_t u; float f; } v;
+    v.u = bits;
+    return e == 0 ? (float)m * (1.0f / 1024.0f) : v.f;
+}
+// decode.hip: NVFP4 weights at up to 16 tokens, f32 activations (float-stored, like FP8)
+hipError_t launch_decode_nvfp4(const WeightView& w, const float* x, size_t t, float* y, hipStream_t s);
 
 // Global scratch of the decode kernels that split K across workgroups: `partial` holds slices x 8 token rows of
 // n_out floats, `counters` (zero between launches) one entry per group of row tiles. Launches that share a scratch

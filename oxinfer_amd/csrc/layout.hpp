@@ -29,6 +29,10 @@
 //   where it has its offsets.
 //   MXFP4 (T4X) the T4M codes (byte j of a block: elements j and j + 16, as in the file) followed by the four E8M0 scale
 //               bytes of each row's blocks, record 1088 B
+//   NVFP4 (T4N) the T4M code geometry over ggml's blocks of 64 (sub-block s of 16: scale byte s, then 8 bytes whose byte j
+//               holds elements j and j + 8): byte j of a lane's dword b holds the step's elements 32 b + 4 kq + j (low
+//               nibble) and 32 b + 16 + 4 kq + j (high), followed by the eight unsigned-E4M3 scale bytes of each row's
+//               sub-blocks of 16 (sub-block 2 b + high), record 1152 B: 4.5 bit per weight, as in the file
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
@@ -42,6 +46,7 @@ constexpr uint32_t TK4_REC = 2368;
 constexpr uint32_t TK5_REC = TK4_REC + 512;
 constexpr uint32_t T4M_REC = 1152;
 constexpr uint32_t T4X_REC = 1088;
+constexpr uint32_t T4N_REC = 1152;
 // Q6_K, 16 rows x 128 columns (half a super-block), lane = 16 kq + n, code j of half h = row n, column 64 h + 16 kq + j:
 //   [0, 1024)    low nibbles, 16 bytes per lane: dword 2 h + j / 8, byte j % 4, low nibble if j % 8 < 4, else high
 //   [1024, 1536) the two high bits, 8 bytes per lane: dword h, bits 8 (j % 4) + 2 (j / 4)
@@ -61,6 +66,7 @@ __host__ __device__ inline size_t t8f_bytes(uint32_t n_out, uint32_t n_in) { ret
 __host__ __device__ inline size_t tk4_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * tk4_sbs(n_in) * TK4_REC; }
 __host__ __device__ inline size_t tk5_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * tk4_sbs(n_in) * TK5_REC; }
 __host__ __device__ inline size_t t4x_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t4m_steps(n_in) * T4X_REC; }
+__host__ __device__ inline size_t t4n_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t4m_steps(n_in) * T4N_REC; }
 __host__ __device__ inline size_t t4m_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t4m_steps(n_in) * T4M_REC; }
 
 __host__ __device__ inline size_t t6k_bytes(uint32_t n_out, uint32_t n_in) { return (size_t)row_tiles(n_out) * t6k_steps(n_in) * T6K_REC; }

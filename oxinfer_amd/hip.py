@@ -13,8 +13,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "liboxinfer_hip.so")
 
 W_BF16, W_Q8, W_Q4, W_GGUF, W_MLX_Q4 = 0, 1, 2, 3, 4
-GGML_Q4_0, GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_MXFP4, GGML_F8E4M3 = 2, 8, 12, 13, 14, 39, 0x1000
-GGML_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q4_K: (256, 144), GGML_Q5_K: (256, 176), GGML_Q6_K: (256, 210), GGML_MXFP4: (32, 17)}
+GGML_Q4_0, GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_MXFP4, GGML_NVFP4, GGML_F8E4M3 = 2, 8, 12, 13, 14, 39, 40, 0x1000
+GGML_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q4_K: (256, 144), GGML_Q5_K: (256, 176), GGML_Q6_K: (256, 210), GGML_MXFP4: (32, 17), GGML_NVFP4: (64, 36)}
 
 
 class WeightDesc(C.Structure):
@@ -298,6 +298,18 @@ class HipBackend:
         bs = np.ascontiguousarray(block_scales, np.float32)
         d = WeightDesc(kind=W_GGUF, ggml_type=GGML_F8E4M3, n_out=n_out, n_in=n_in, data=_np_ptr(data),
                        block_scales=_np_ptr(bs), bs_rows=block[0], bs_cols=block[1])
+        return self._upload(d, (data, bs))
+
+    def upload_nvfp4(self, data, n_out, n_in, scales=None, block=None):
+        """GgufMatrix of NVFP4 blocks (src/ggml.rs:79-83) with, optionally, the matrix's scales on top (`block` = rows x
+        columns per scale; default one scale for the matrix, as model::nvfp4_blocks builds it)."""
+        data = np.ascontiguousarray(data, np.uint8)
+        if data.size != n_out * (n_in // 64) * 36:
+            raise ValueError("NVFP4 byte count does not match the shape")
+        bs = None if scales is None else np.ascontiguousarray(np.atleast_1d(scales), np.float32)
+        br, bc = block or (n_out, n_in)
+        d = WeightDesc(kind=W_GGUF, ggml_type=GGML_NVFP4, n_out=n_out, n_in=n_in, data=_np_ptr(data), block_scales=_np_ptr(bs),
+                       bs_rows=br if bs is not None else 0, bs_cols=bc if bs is not None else 0)
         return self._upload(d, (data, bs))
 
     def upload_q8(self, q, scales, n_out, n_in):

@@ -100,6 +100,19 @@ def gguf_mxfp4(n_out, n_in, seed):
     return blk.reshape(-1)
 
 
+def gguf_nvfp4(n_out, n_in, seed):
+    """NVFP4 blocks of 64 in ggml's layout (36 B: four unsigned E4M3 scale bytes, one per 16 values, then 4 x 8 bytes of
+    E2M1 codes, uniform; src/ggml.rs:936-947), scales 2^-9 .. 2^-3 with random mantissas (a few zero), and a global f32
+    scale as compressed-tensors checkpoints carry it. Returns (bytes, global scale)."""
+    rng = np.random.default_rng(seed)
+    nb = n_out * n_in // 64
+    blk = rng.integers(0, 256, (nb, 36), dtype=np.uint8)
+    sc = (rng.integers(0, 7, (nb, 4)) << 3 | rng.integers(0, 8, (nb, 4))).astype(np.uint8)
+    sc[rng.random((nb, 4)) < 0.01] = 0
+    blk[:, :4] = sc
+    return blk.reshape(-1), np.float32(abs(rng.normal(0.0, 0.5)) + 0.25)
+
+
 def gguf_q6_k(n_out, n_in, seed):
     """Q6_K super-blocks (210 B): ql, qh uniform bits, int8 scales uniform, f16 d ~ +-|N(0, 0.005)|."""
     rng = np.random.default_rng(seed)

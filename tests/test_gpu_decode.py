@@ -328,6 +328,53 @@ def test_bf16_weights(be, oxref, n_out, n_in):
     assert be.upload_bf16(np.zeros((3, 12), np.uint16), 3, 12) is None  # rows must be whole 16-byte units
 
 
+@pytest.mark.parametrize("n_out,n_in,scaled", [(37, 192, "none"), (64, 1024, "global"), (48, 4160, "blocks"), (200, 14336, "global")])
+def test_nvfp4_upload_dequant_decode_gemm(be, oxref, n_out, n_in, scaled):
+    """NVFP4 (ggml's blocks of 64 with an unsigned E4M3 scale per 16, src/ggml.rs:79-83, :936-947), float-stored like FP8
+    (is_float, :219-224): dequantized rows bit-exact (with and without the matrix's scales on top, :420-432), decode at 1
+    to 16 tokens within 1e-3 of the CPU's f32 product of those rows, the bf16 matrix-core GEMM past 16 tokens within 2e-2,
+    and the host surface (Backend::matmul) routing both."""
+    import torch
+    from oxinfer_amd import synth
+    raw, g = synth.gguf_nvfp4(n_out, n_in, 9000 + n_in)
+    if scaled == "none":
+        scales, block = None, None
+    elif scaled == "global":
+        scales, block = np.array([g], np.float32), (n_out, n_in)
+    else:  # blocks of 16 rows x 128 columns, every scale different
+        block = (16, 128)
+        scales = np.abs(np.random.default_rng(5).normal(0.5, 0.2, (-(-n_out // 16), -(-n_in // 128)))).astype(np.float32) + 0.1
+    w = be.upload_nvfp4(raw, n_out, n_in, scales, block)
+    assert w is not None, be.last_error()
+    assert w.bytes <= (n_out + 15) // 16 * 16 * (n_in + 127) // 128 * 128 * 0.5625 + 256 + (0 if scales is None else scales.size * 4 + 256)
+    br, bc = block or (n_out, n_in)
+    want = oxref.gguf_dequant_rows_scaled(oxref.NVFP4, raw, scales, n_out, n_in, br, bc)
+    assert np.array_equal(be.dequantize(w).cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(be.dequantize(w, 5, 21).cpu().numpy().view(np.uint32), want[5:21].view(np.uint32))
+    for t in (1, 2, 3, 4, 7, 16):
+        x = lcg_input(t, n_in, 77 + t, oxref)
+        ref = oxref.gemm_quant(oxref.NVFP4, raw, scales, None, n_out, n_in, x, t, brows=br, bcols=bc)
+        y = be.decode(w, x=dev(x)).cpu().numpy()
+        assert row_err(y, ref) < TOL, (t, row_err(y, ref))
+        yh = np.full((t, n_out), np.nan, np.float32)
+        assert be.matmul(x, t, n_in, [(w, yh)]), be.last_error()
+        assert np.array_equal(yh.view(np.uint32), y.view(np.uint32))
+    for t in (17, 40, 130):
+        x = synth.activations(t, n_in, 88 + t)
+        ref = oxref.gemm_quant(oxref.NVFP4, raw, scales, None, n_out, n_in, x, t, brows=br, bcols=bc)
+        y = be.gemm(w, dev(x), variant=0).cpu().numpy()
+        assert row_err(y, ref) < 2e-2, (t, row_err(y, ref))
+        # both operands rounded to bf16, as the kernel rounds them: tight against that product
+        xb, wb = synth.bf16_round(x).astype(np.float64), synth.bf16_round(want).astype(np.float64)
+        assert row_err(y, (xb @ wb.T).astype(np.float32)) < 1e-3, t
+        yh = np.full((t, n_out), np.nan, np.float32)
+        assert be.matmul(x, t, n_in, [(w, yh)]), be.last_error()
+        assert row_err(yh, ref) < 2e-2
+    # rows that are not whole blocks of 64, and scale blocks that cut through a tile: declined at upload
+    assert be.lib.oxhip_upload(be.ctx, be.desc_gguf(40, raw[:36], 1, 32)[0]) is None and "64" in be.last_error()
+    assert be.upload_nvfp4(raw, n_out, n_in, np.ones(n_out * (-(-n_in // 64)), np.float32), (1, 64)) is None
+
+
 def test_host_matmul_matches_device_path_and_declines(be, oxref):
     from oxinfer_amd import synth
     n_in = 512

@@ -180,3 +180,48 @@ def test_type_geometry(oxref):
     assert oxref.row_bytes(12, 5120) == 20 * 144
     assert oxref.row_bytes(8, 4096) == 4352 and oxref.row_bytes(12, 4096) == 2304 and oxref.row_bytes(14, 4096) == 3360
     assert oxref.block_size(15) == 0  # Q8_K is not a weight format
+
+
+def test_nvfp4_against_the_format_definitions(oxref):
+    """NVFP4 (src/ggml.rs:79-83, :477-490, :936-947), which has no entry in the reference's hash table: every (scale byte,
+    code) pair against what the formats themselves define. The scale is an unsigned E4M3 value, halved (torch's
+    float8_e4m3fn decodes the byte's low seven bits; 0 and 0x7f give 0, the top bit is ignored); the codes are E2M1 values
+    (sign, two exponent bits, one mantissa bit: 0, 0.5, 1, 1.5, 2, 3, 4, 6), stored doubled. A block of 64 is four
+    sub-blocks of 16: scale byte s, then 8 bytes whose byte j holds elements j (low nibble) and j + 8 (high)."""
+    e4m3 = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+
+    def e2m1(code):
+        sign, e, m = -1.0 if code & 8 else 1.0, (code >> 1) & 3, code & 1
+        return sign * (m * 0.5 if e == 0 else (1 + m / 2) * 2.0 ** (e - 1))
+    for sc in range(256):
+        low7 = sc & 0x7F
+        want_scale = 0.0 if sc in (0, 0x7F) else (480.0 if sc == 0xFF else float(e4m3[low7])) * 0.5  # 0xff: e = 15, m = 7 read as a number, 1.875 * 2^8
+        assert oxref.ue4m3_half(sc) == want_scale, sc
+        # one block: sub-block 1 carries this scale, its 16 elements walk the 16 codes in an order that tells low from
+        # high nibbles and byte j from byte j + 1; the other sub-blocks carry other scales and codes
+        blk = np.zeros(36, np.uint8)
+        blk[0:4] = [0x38, sc, 0x30, 0x41]
+        codes = [(5 * i + 3) % 16 for i in range(16)]
+        for j in range(8):
+            blk[4 + 8 + j] = codes[j] | (codes[j + 8] << 4)
+            blk[4 + j] = 0x21
+            blk[4 + 16 + j] = 0x9C
+            blk[4 + 24 + j] = 0x5F
+        y = oxref.dequantize_row(oxref.NVFP4, blk, 64)
+        want = np.array([np.float32(want_scale) * np.float32(2 * e2m1(c) + 0.0) for c in codes], np.float32)  # (the table is integers: code 8 is +0)
+        assert np.array_equal(y[16:32].view(np.uint32), want.view(np.uint32)), sc
+        assert y[0] == np.float32(0.5) * np.float32(2 * e2m1(1)) and y[8] == np.float32(0.5) * np.float32(2 * e2m1(2))
+        assert y[32] == np.float32(0.25) * np.float32(2 * e2m1(0xC)) and y[40] == np.float32(0.25) * np.float32(2 * e2m1(9))
+    assert oxref.block_size(oxref.NVFP4) == 64 and oxref.type_size(oxref.NVFP4) == 36 and oxref.row_bytes(oxref.NVFP4, 128) == 72
+    # the matrix's scale on top of the decoded values: one more f32 multiply (src/ggml.rs:420-432), here per 2 x 64 block
+    from oxinfer_amd import synth
+    raw, _ = synth.gguf_nvfp4(4, 128, 3)
+    s = np.array([[2.0, 0.5], [3.0, 0.75]], np.float32)
+    got = oxref.gguf_dequant_rows_scaled(oxref.NVFP4, raw, s, 4, 128, 2, 64)
+    base = oxref.dequantize_rows(oxref.NVFP4, raw, 4, 128)
+    assert np.array_equal(got, base * np.repeat(np.repeat(s, 2, axis=0), 64, axis=1))
+    assert np.array_equal(oxref.gguf_dequant_rows_scaled(oxref.NVFP4, raw, None, 4, 128), base)
+    # the matmul is the f32 product of those rows (float-stored: the f32 path at every token count)
+    x = synth.activations(3, 128, 4)
+    y = oxref.gemm_quant(oxref.NVFP4, raw, s, None, 4, 128, x, 3, brows=2, bcols=64)
+    assert np.abs(y - x.astype(np.float64) @ got.astype(np.float64).T).max() < 1e-4 * np.abs(y).max()
