@@ -115,7 +115,8 @@ size_t oxhip_weight_bytes(const oxhip_weight* w);
  * src/kernels.rs:1908-1928); more than 16 tokens over MLX 4-bit, Q8, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4, NVFP4 or FP8 (128-column
  * blocks) weights run the bf16 matrix-core GEMM; everything else runs the decode kernels over 16 tokens at a time. */
 int oxhip_matmul(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_job* jobs, size_t n_jobs);
-/* Backend::matvec_rows (src/gpu.rs:165): t in 1..=4. */
+/* Backend::matvec_rows (src/gpu.rs:165): t in 1..=4. The jobs over the matrix-core formats share one launch, a gate / up
+ * job as a pair (see oxhip_dev_linear). */
 int oxhip_matvec_rows(oxhip_ctx* ctx, const float* x, size_t t, size_t n_in, oxhip_rows_job* jobs, size_t n_jobs);
 
 /* Backend::upload_moe (src/gpu.rs:206-216): expert e has gate_up[e] ([2*inter, h] fused, or [inter, h] when `up` is
@@ -284,7 +285,10 @@ int oxhip_dev_norm(oxhip_ctx* ctx, const float* x, float* out, const float* w_f3
  *   ADD_GATED  y += sigmoid(gate[token]) * W x (a gated shared expert; `gate` one f32 per token on the device)
  * Inputs as oxhip_dev_decode's: `xa` for quantized weights, f32 rows `x` for float-stored ones. The matrices of a
  * pair share shape and format (pairable, src/gpu_decode.rs:340-349). The store / add / gated modes are the decode
- * kernels' own output stage; a pair runs both products in one launch and the gate as a second one. */
+ * kernels' own output stage. A pair over the matrix-core formats (Q8, Q8_0, Q4_0, Q4_K, Q5_K, Q6_K, MXFP4, MLX 4-bit) is ONE
+ * launch: a workgroup streams the tiles of the same rows of both matrices and stores act(W x) * (W2 x) itself (the CUDA
+ * kernels' modes 2 and 3, src/cuda_decode.cu:131-167), bit-identical to the two products followed by oxhip_dev_glu; the
+ * other formats run the two products and the gate as launches of their own. */
 enum { OXHIP_LIN_STORE = 0, OXHIP_LIN_ADD = 1, OXHIP_LIN_SILU_PAIR = 2, OXHIP_LIN_GELU_PAIR = 3, OXHIP_LIN_ADD_GATED = 4 };
 int oxhip_dev_linear(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_weight* w2, const oxhip_qact* xa, const float* x, size_t t,
                      float* y, uint32_t mode, const float* gate, void* stream);

@@ -213,26 +213,24 @@ int oxhip_dev_linear(oxhip_ctx* c, const oxhip_weight* w, const oxhip_weight* w2
         HIP_TRY(launch_epilogue(tmp, t, n_out, y, epi, s), "linear epilogue launch");
         return 1;
     }
-    // y = act(W x) * (W2 x): both products in one shared launch where the kernel takes them, then the gate
+    // y = act(W x) * (W2 x). The matrix-core decode kernel pairs the two matrices' tiles of the same rows in one workgroup and
+    // applies the gate in its output stage: one launch, no intermediate rows (bit-identical to the two products and Op::Glu)
+    if (mfma_decode_format(w->v.fmt)) {
+        Epi pe;
+        pe.pair_p0 = w2->v.p0;
+        pe.pair_act = mode == OXHIP_LIN_GELU_PAIR ? 1u : 0u;
+        HIP_TRY(launch_decode_mfma(w->v, v, t, y, sc->dec, s, nullptr, nullptr, pe), "linear pair launch");
+        return 1;
+    }
+    // the other formats: both products into scratch, then the gate
     if (!sc->tmp.grow(2 * t * n_out * 4)) {
         set_error("linear: device memory short");
         return 0;
     }
     float* g = static_cast<float*>(sc->tmp.p);
     float* u = g + t * n_out;
-    if (t <= 8 && decode_batchable(w->v, t)) {
-        DecodeBatchItem items[2] = {{w->v, v, g, (uint32_t)t, Epi{}}, {w2->v, v, u, (uint32_t)t, Epi{}}};
-        hipError_t e = launch_decode_mfma_batch(items, 2, sc->dec, s);
-        if (e == hipErrorOutOfMemory) {
-            HIP_TRY(launch_decode(w->v, v, x, t, g, s, sc->dec), "linear launch");
-            HIP_TRY(launch_decode(w2->v, v, x, t, u, s, sc->dec), "linear launch");
-        } else {
-            HIP_TRY(e, "linear launch");
-        }
-    } else {
-        HIP_TRY(launch_decode(w->v, v, x, t, g, s, sc->dec), "linear launch");
-        HIP_TRY(launch_decode(w2->v, v, x, t, u, s, sc->dec), "linear launch");
-    }
+    HIP_TRY(launch_decode(w->v, v, x, t, g, s, sc->dec), "linear launch");
+    HIP_TRY(launch_decode(w2->v, v, x, t, u, s, sc->dec), "linear launch");
     HIP_TRY(launch_glu(g, u, t * n_out, mode == OXHIP_LIN_GELU_PAIR, y, s), "linear gate launch");
     return 1;
 }

@@ -448,16 +448,35 @@ int oxhip_matvec_rows(oxhip_ctx* c, const float* x, size_t t, size_t n_in, oxhip
     float* yd = static_cast<float*>(c->y.p);
     size_t off = 0;
     std::vector<size_t> at(n_jobs);
+    // The jobs the matrix-core decode kernel takes share ONE launch (they all read the same x): a plain job as it is, a
+    // gate / up job as a pair whose workgroups hold the tiles of the same rows of both matrices and store silu(W x) * (U x)
+    // themselves (src/cuda_decode.cu:131-167). The others launch one by one, a pair as two products and the gate.
+    std::vector<DecodeBatchItem> fused;
     for (size_t j = 0; j < n_jobs; j++) {
         const oxhip_rows_job& jb = jobs[j];
         const size_t n = t * jb.n_out;
         at[j] = off;
-        HIP_TRY(launch_decode(jb.w->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off, s, c->dec), "decode launch");
-        if (jb.up) {
-            HIP_TRY(launch_decode(jb.up->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off + n, s, c->dec), "decode launch");
-            HIP_TRY(launch_moe_act(yd + off, yd + off + n, jb.n_out, t, jb.n_out, OXHIP_ACT_SILU, 0.0f, yd + off, s), "act launch");
+        const bool pairable = !jb.up || (jb.up->v.fmt == jb.w->v.fmt && mfma_decode_format(jb.w->v.fmt));
+        if (pairable && !is_dense(jb.w) && decode_batchable(jb.w->v, t)) {
+            Epi e;
+            if (jb.up) e.pair_p0 = jb.up->v.p0;
+            fused.push_back(DecodeBatchItem{jb.w->v, view_of(xa), yd + off, (uint32_t)t, e});
+        } else {
+            HIP_TRY(launch_decode(jb.w->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off, s, c->dec), "decode launch");
+            if (jb.up) {
+                HIP_TRY(launch_decode(jb.up->v, view_of(xa), static_cast<const float*>(c->x.p), t, yd + off + n, s, c->dec), "decode launch");
+                HIP_TRY(launch_moe_act(yd + off, yd + off + n, jb.n_out, t, jb.n_out, OXHIP_ACT_SILU, 0.0f, yd + off, s), "act launch");
+            }
         }
         off += n * (jb.up ? 2 : 1);
+    }
+    if (!fused.empty()) {
+        hipError_t e = launch_decode_mfma_batch(fused.data(), fused.size(), c->dec, s);
+        if (e == hipErrorOutOfMemory) {  // the scratch does not hold these jobs' K slices together: one launch each
+            for (auto& it : fused) HIP_TRY(launch_decode_mfma(it.w, it.xa, t, it.y, c->dec, s, nullptr, nullptr, it.epi), "decode launch");
+        } else {
+            HIP_TRY(e, "decode batch launch");
+        }
     }
     std::vector<float> host(y_total);
     HIP_TRY(hipMemcpyAsync(host.data(), yd, y_total * 4, hipMemcpyDeviceToHost, s), "matvec_rows copy-out");

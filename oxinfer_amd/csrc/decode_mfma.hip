@@ -156,10 +156,14 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // known at run time costs some twenty instructions even when it is the same for the whole wave
     const uint32_t kwsh = (uint32_t)__builtin_ctz(kw), kssh = (uint32_t)__builtin_ctz(ksplit);
     const uint32_t r = wave >> kwsh, ks = wave & (kw - 1);
-    // (fused gate / up experts: the first rt / 2 tiles of the workgroup are gate tiles, the others the up tiles of the same rows)
+    // (fused gate / up experts: the first rt / 2 tiles of the workgroup are gate tiles, the others the up tiles of the same rows;
+    // a gate / up pair of two matrices likewise: the first rt / 2 waves' tiles come from `w`, the others' from epi.pair_p0)
     const bool glu = GROUPED && grp.glu_inter != 0;
+    const bool pair = !GROUPED && !DUMP && epi.pair_p0 != nullptr;
     const uint32_t ghalf = rt >> 1, gtiles = grp.glu_inter / 16;
-    const uint32_t tile = !glu ? bx * rt + r : r < ghalf ? bx * ghalf + r : gtiles + bx * ghalf + (r - ghalf);
+    const uint32_t tile = glu    ? (r < ghalf ? bx * ghalf + r : gtiles + bx * ghalf + (r - ghalf))
+                          : pair ? bx * ghalf + (r < ghalf ? r : r - ghalf)
+                                 : bx * rt + r;
     const uint32_t ntiles = glu && r < ghalf ? gtiles : row_tiles(w.n_out);
     // this workgroup's slice of K: steps [S0, S1), blocks [B0, B0 + nbl) (a multiple of 4 blocks)
     constexpr uint32_t BPS = q8_format(FMT) ? 2 : 4;  // blocks of 32 per step
@@ -212,7 +216,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     const uint32_t s0 = S0 + ks * per;
     const uint32_t s1 = tile < ntiles ? min(S1, s0 + per) : 0;  // a tile past the matrix streams nothing
     // (typed as global memory: a grouped launch reads w.p0 from the table of expert bases)
-    const gbytes base = as_global(w.p0) + (size_t)min(tile, ntiles - 1) * (FMT == FMT_Q8_0   ? (size_t)nsteps * T8_REC
+    const gbytes base = as_global(pair && r >= ghalf ? epi.pair_p0 : w.p0) + (size_t)min(tile, ntiles - 1) * (FMT == FMT_Q8_0   ? (size_t)nsteps * T8_REC
                                                                   : FMT == FMT_Q8F  ? (size_t)nsteps * T8F_REC
                                                                   : k45_format(FMT) ? (size_t)(nsteps / 2) * K45_REC
                                                                   : FMT == FMT_Q6_K ? (size_t)nsteps * T6K_REC
@@ -770,16 +774,33 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
         }
     }
     const bool combine = GROUPED && grp.comb_y != nullptr;
-    // the waves of a tile in order; with one slice that is the result, else this slice's partial rows
-    float* out = ksplit > 1 ? partial + (size_t)slice * t * w.n_out : y;
+    if (pair && ksplit == 1) {
+        // act(gate) * up of the workgroup's rt / 2 row tiles: each product summed over its waves in order, as a launch of its own would
+        for (uint32_t idx = threadIdx.x; idx < ghalf * TPAD * 16; idx += nthr) {
+            const uint32_t rr = idx / (TPAD * 16), tok = (idx / 16) % TPAD, nn = idx % 16;
+            const uint32_t row = (bx * ghalf + rr) * 16 + nn;
+            if (tok >= t || row >= w.n_out) continue;
+            float gs = 0.0f, us = 0.0f;
+            for (uint32_t k = 0; k < kw; k++) {
+                gs += red[(((size_t)rr * kw + k) * TPAD + tok) * 16 + nn];
+                us += red[(((size_t)(ghalf + rr) * kw + k) * TPAD + tok) * 16 + nn];
+            }
+            y[(size_t)tok * w.n_out + row] = gated_act(gs, us, epi.pair_act, 0.0f);
+        }
+        return;
+    }
+    // the waves of a tile in order; with one slice that is the result, else this slice's partial rows (a pair's partial rows are
+    // 2 n_out wide: the first matrix's, then the second's)
+    const uint32_t prow = pair ? 2 * w.n_out : w.n_out;
+    float* out = ksplit > 1 ? partial + (size_t)slice * t * prow : y;
     for (uint32_t idx = threadIdx.x; idx < rt * NG * TPAD * 16; idx += nthr) {
         const uint32_t rr = idx / (NG * TPAD * 16), g = (idx / (TPAD * 16)) % NG, tok = 8 * g + (idx / 16) % TPAD, nn = idx % 16;
-        const uint32_t row = (bx * rt + rr) * 16 + nn;
+        const uint32_t row = pair ? (bx * ghalf + (rr < ghalf ? rr : rr - ghalf)) * 16 + nn : (bx * rt + rr) * 16 + nn;
         if (tok >= t || row >= w.n_out || !y) continue;
         float sum = 0.0f;
         for (uint32_t k = 0; k < kw; k++) sum += red[((((size_t)rr * kw + k) * NG + g) * TPAD + (idx / 16) % TPAD) * 16 + nn];
         // partial rows go out as device-scope stores (written through to memory, where the other XCDs' L2s see them)
-        if (ksplit > 1 || combine) __hip_atomic_store(out + (size_t)tok * w.n_out + row, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (ksplit > 1 || combine) __hip_atomic_store(out + (size_t)tok * prow + (pair && rr >= ghalf ? w.n_out : 0u) + row, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         else emit(out + (size_t)tok * w.n_out + row, sum, tok);
     }
     if constexpr (GROUPED) {
@@ -834,21 +855,26 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     }
     __syncthreads();
     if (!is_last) return;
-    for (uint32_t idx = threadIdx.x; idx < rt * 16 * t; idx += nthr) {
-        const uint32_t tok = idx / (rt * 16), row = bx * rt * 16 + idx % (rt * 16);
-        if (row >= w.n_out) continue;
-        const float* p = partial + (size_t)tok * w.n_out + row;
-        // four slices per round trip (a loop of one load per slice waits for each in turn); still added in slice order
+    // four slices per round trip (a loop of one load per slice waits for each in turn); still added in slice order
+    auto slice_sum = [&](const float* p) {
         float sum = 0.0f;
         for (uint32_t z0 = 0; z0 < ksplit; z0 += 4) {
             float v[4];
 #pragma unroll
             for (uint32_t i = 0; i < 4; i++)
-                v[i] = __hip_atomic_load(p + (size_t)min(z0 + i, ksplit - 1) * t * w.n_out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                v[i] = __hip_atomic_load(p + (size_t)min(z0 + i, ksplit - 1) * t * prow, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
             for (uint32_t i = 0; i < 4; i++) sum = z0 + i == 0 ? v[i] : z0 + i < ksplit ? sum + v[i] : sum;
         }
-        emit(y + (size_t)tok * w.n_out + row, sum, tok);
+        return sum;
+    };
+    const uint32_t wrows = (pair ? ghalf : rt) * 16;  // output rows of the workgroup
+    for (uint32_t idx = threadIdx.x; idx < wrows * t; idx += nthr) {
+        const uint32_t tok = idx / wrows, row = bx * wrows + idx % wrows;
+        if (row >= w.n_out) continue;
+        const float* p = partial + (size_t)tok * prow + row;
+        if (pair) y[(size_t)tok * w.n_out + row] = gated_act(slice_sum(p), slice_sum(p + w.n_out), epi.pair_act, 0.0f);
+        else emit(y + (size_t)tok * w.n_out + row, slice_sum(p), tok);
     }
 }
 
@@ -1013,6 +1039,14 @@ Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices, int fmt) {
     return sh;
 }
 
+// A gate / up pair: a workgroup holds the tiles of the same rows of both matrices, so its tile count is even; kw and ks (the
+// order of a row's sum) stay what the weight's shape alone gives, which keeps each product's bits those of a launch of its own.
+Shape pair_shape(Shape sh) {
+    if (sh.rt % 2) sh.rt *= 2;  // (rt * kw <= 8 before: at most 16 waves)
+    return sh;
+}
+uint32_t pair_tiles(const Shape& sh, bool pair) { return pair ? pair_shape(sh).rt / 2 : sh.rt; }
+
 constexpr size_t LDS_MAX = 160 * 1024 - 256;  // dynamic LDS on offer (the kernel also holds a static word)
 
 // Dynamic LDS of a launch; `alds` comes back false when the operand-order activations do not fit (they are then read
@@ -1064,13 +1098,18 @@ template <int FMT, bool DUMP>
 hipError_t run(const WeightView& w, const QActView& xa, size_t t, float* y, int32_t* dump, const DecodeScratch& sc, hipStream_t s,
                hipEvent_t ev_start = nullptr, hipEvent_t ev_stop = nullptr, const Epi& epi0 = Epi{}) {
     const uint32_t ntiles = row_tiles(w.n_out), nsteps = steps_of<FMT>(w.n_in);
+    const bool pair = !DUMP && epi0.pair_p0 != nullptr;
     Shape sh = shape_for(ntiles, nsteps, true, FMT);
-    const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
-    // slices need scratch: 8 token rows per slice and a counter per row group
-    if (sh.ks > 1 && (!sc.partial || !sc.counters || sc.partial_floats < (size_t)sh.ks * 8 * w.n_out || sc.ncounters < (size_t)groups * CTR_STRIDE))
-        sh = shape_for(ntiles, nsteps, false, FMT);
+    // slices need scratch: 8 token rows per slice (of both matrices of a pair) and a counter per row group
+    auto scratch_ok = [&](const Shape& h) {
+        const uint32_t groups = (ntiles + pair_tiles(h, pair) - 1) / pair_tiles(h, pair);
+        return h.ks == 1 || (sc.partial && sc.counters && sc.partial_floats >= (size_t)h.ks * 8 * w.n_out * (pair ? 2 : 1) && sc.ncounters >= (size_t)groups * CTR_STRIDE);
+    };
+    if (!scratch_ok(sh)) sh = shape_for(ntiles, nsteps, false, FMT);
+    if (pair) sh = pair_shape(sh);
     const uint32_t nblk = w.n_in / 32;
-    dim3 grid((ntiles + sh.rt - 1) / sh.rt, sh.ks), block(64 * sh.rt * sh.kw);
+    const uint32_t per_wg = pair ? sh.rt / 2 : sh.rt;  // row tiles of the output per workgroup
+    dim3 grid((ntiles + per_wg - 1) / per_wg, sh.ks), block(64 * sh.rt * sh.kw);
     // timing events: one launch carries them itself; around several they are recorded on the stream
     const bool ride = t <= 8;
     if (!ride && ev_start) {
@@ -1179,14 +1218,15 @@ bool decode_batchable(const WeightView& w, size_t t) {
 
 // Scratch a launch of this weight alone takes when its shape slices K across workgroups (floats of partial rows,
 // arrival counters); both zero when K stays inside a workgroup.
-void decode_scratch_need(const WeightView& w, size_t* partial_floats, size_t* ncounters) {
+void decode_scratch_need(const WeightView& w, size_t* partial_floats, size_t* ncounters, bool pair) {
     *partial_floats = *ncounters = 0;
     if (!mfma_decode_format(w.fmt)) return;
     const uint32_t ntiles = row_tiles(w.n_out);
     const Shape sh = shape_for(ntiles, steps_rt(w), true, w.fmt);
     if (sh.ks <= 1) return;
-    *partial_floats = (size_t)sh.ks * 8 * w.n_out;
-    *ncounters = (size_t)((ntiles + sh.rt - 1) / sh.rt) * CTR_STRIDE;
+    const uint32_t per_wg = pair_tiles(sh, pair);
+    *partial_floats = (size_t)sh.ks * 8 * w.n_out * (pair ? 2 : 1);
+    *ncounters = (size_t)((ntiles + per_wg - 1) / per_wg) * CTR_STRIDE;
 }
 
 // Every item must be decode_batchable. Items go out in launches of up to BATCH_MAX jobs; jobs whose shape slices K
@@ -1237,15 +1277,18 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
         for (uint32_t j = 0; j < a.njobs; j++) {
             const DecodeBatchItem& it = items[i0 + order[j]];
             const uint32_t ntiles = row_tiles(it.w.n_out), nsteps = steps_rt(it.w);
-            const Shape sh = shape_for(ntiles, nsteps, true, it.w.fmt);
+            const bool pair = it.epi.pair_p0 != nullptr;
+            Shape sh = shape_for(ntiles, nsteps, true, it.w.fmt);
+            if (pair) sh = pair_shape(sh);
             bool alds;
             const size_t l = lds_bytes(it.w.fmt, false, nsteps, it.t <= 4 ? 4 : 8, sh, &alds);
             if (!alds || l > LDS_MAX || it.t < 1 || it.t > 8) return hipErrorInvalidValue;
-            const uint32_t groups = (ntiles + sh.rt - 1) / sh.rt;
+            const uint32_t per_wg = pair ? sh.rt / 2 : sh.rt;
+            const uint32_t groups = (ntiles + per_wg - 1) / per_wg;
             float* partial = nullptr;
             uint32_t* counters = nullptr;
             if (sh.ks > 1) {
-                const size_t need = (size_t)sh.ks * it.t * it.w.n_out;
+                const size_t need = (size_t)sh.ks * it.t * it.w.n_out * (pair ? 2 : 1);
                 if (!sc.partial || !sc.counters || pf + need > sc.partial_floats || nc + (size_t)groups * CTR_STRIDE > sc.ncounters) return hipErrorOutOfMemory;
                 partial = sc.partial + pf;
                 counters = sc.counters + nc;

@@ -69,6 +69,13 @@ enum : uint32_t { EPI_STORE = 0, EPI_ADD = 1, EPI_ADD_GATED = 2 };
 struct Epi {
     uint32_t mode = EPI_STORE;
     const float* gate = nullptr;  // EPI_ADD_GATED: one f32 per token
+    // A gate / up pair in one launch (LinMode::SiluPair / GeluPair, src/gpu_decode.rs:43-46; the CUDA kernels' modes 2 and
+    // 3, src/cuda_decode.cu:131-167): pair_p0 != nullptr is the second matrix's records (same shape and format as the
+    // first). A workgroup streams the tiles of the same rows of both matrices and stores act(W x) * (W2 x); each product's
+    // sum is formed exactly as a launch of its own forms it, so the result is gated_act of the two separate products, bit
+    // for bit. pair_act: 0 SiLU, 1 GELU-tanh. Stores only (mode EPI_STORE).
+    const uint8_t* pair_p0 = nullptr;
+    uint32_t pair_act = 0;
 };
 
 // A grouped launch (MoE): chunk c = {expert, first row, rows (<= 8), 0}; see decode_mfma.hip.
@@ -166,7 +173,7 @@ struct DecodeBatchItem {
     uint32_t t;
     Epi epi{};
 };
-void decode_scratch_need(const WeightView& w, size_t* partial_floats, size_t* ncounters);  // of a launch that slices K; else zeros
+void decode_scratch_need(const WeightView& w, size_t* partial_floats, size_t* ncounters, bool pair = false);  // of a launch that slices K; else zeros (a pair launch: twice the floats)
 bool decode_batchable(const WeightView& w, size_t t);  // the kernel takes it and its activations fit LDS
 // ev_start / ev_stop (optional): timing events around the launches.
 hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s, hipEvent_t ev_start = nullptr,

@@ -106,9 +106,13 @@ def test_linear_store_add_gated(be, oxref, kind, n_out, n_in):
     assert float(y.min()) == 7.0 and float(y.max()) == 7.0  # declined: nothing written
 
 
-@pytest.mark.parametrize("kind,n_out,n_in", [(Q4_K, 96, 512), (Q8_0, 40, 864), ("mlx", 80, 640), (Q4_K, 32, 14336), ("q4", 10, 512), ("bf16", 21, 520)])
+@pytest.mark.parametrize("kind,n_out,n_in", [(Q4_K, 96, 512), (Q8_0, 40, 864), ("mlx", 80, 640), (Q4_K, 32, 14336), ("q4", 10, 512), ("bf16", 21, 520),
+                                             (Q6_K, 48, 512), (Q4_K, 1000, 768), (Q8_0, 272, 14336), (Q4_0, 130, 1120), (Q6_K, 40, 14336)])
 def test_linear_pairs(be, oxref, kind, n_out, n_in):
-    """LinMode SiluPair / GeluPair: y = act(W x) * (W2 x) with silu_mul / gelu_mul (src/kernels.rs:2188-2198, :2234-2257)."""
+    """LinMode SiluPair / GeluPair: y = act(W x) * (W2 x) with silu_mul / gelu_mul (src/kernels.rs:2188-2198, :2234-2257). Over
+    the matrix-core formats the pair is one launch whose workgroups hold the same rows' tiles of both matrices (the CUDA
+    kernels' modes 2 and 3, src/cuda_decode.cu:131-167), with and without K slices, ragged last row groups, 1 to 13 tokens:
+    the rows must equal Op::Glu of the two products computed apart, bit for bit."""
     import torch
     from oxinfer_amd import hip, synth
     w, ref_w = weights(be, oxref, kind, n_out, n_in, 600)
@@ -132,6 +136,9 @@ def test_linear_pairs(be, oxref, kind, n_out, n_in):
         gd, ud = torch.empty((t, n_out), device="cuda"), torch.empty((t, n_out), device="cuda")
         assert be.linear(w, gd, t=t, **args) and be.linear(u, ud, t=t, **args)
         assert np.array_equal(be.glu(gd, ud, gelu=True).cpu().numpy().view(np.uint32), y.cpu().numpy().view(np.uint32))
+        ys = torch.full((t, n_out), float("nan"), device="cuda")
+        assert be.linear(w, ys, t=t, mode=hip.LIN_SILU_PAIR, w2=u, **args), be.last_error()
+        assert np.array_equal(be.glu(gd, ud, gelu=False).cpu().numpy().view(np.uint32), ys.cpu().numpy().view(np.uint32))
     if not dense:  # a second matrix of another storage format is not pairable: declined, nothing written
         other, _ = weights(be, oxref, Q8_0 if kind != Q8_0 else Q4_0, n_out, n_in, 602)
         y = torch.full((1, n_out), 7.0, device="cuda")

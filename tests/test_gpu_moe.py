@@ -421,3 +421,22 @@ def test_matvec_rows(be, oxref):
         ref = oxref.silu_mul(g, oxref.gguf_decode(Q4_K, uk, n_out, n_in, x, t))
         assert row_err(y1, ref) < 1e-3
     assert not be.matvec_rows(np.zeros((5, n_in), np.float32), 5, n_in, [(w, None, np.zeros((5, n_out), np.float32))])
+
+
+@pytest.mark.parametrize("kind,n_out,n_in", [(Q4_K, 1000, 768), (Q8_0, 272, 14336), (Q4_K, 48, 14336)])
+def test_matvec_rows_shares_a_launch_and_pairs_keep_the_bits(be, oxref, kind, n_out, n_in):
+    """Several RowsJobs of one call (plain and gate / up) share one launch; a gate / up job's rows are silu_mul of the two
+    products as separate plain jobs give them, bit for bit (K-sliced shapes and ragged row groups included)."""
+    from oxinfer_amd import synth
+    raws = [oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 70 + i)[0] for i in range(3)]
+    ws = [be.upload_gguf(kind, r, n_out, n_in) for r in raws]
+    for t in (1, 3, 4):
+        x = synth.activations(t, n_in, 80 + t)
+        ys = [np.zeros((t, n_out), np.float32) for _ in range(5)]
+        assert be.matvec_rows(x, t, n_in, [(ws[0], None, ys[0]), (ws[0], ws[1], ys[1]), (ws[2], None, ys[2]), (ws[1], None, ys[3]), (ws[2], ws[0], ys[4])]), be.last_error()
+        assert row_err(ys[0], oxref.gguf_decode(kind, raws[0], n_out, n_in, x, t)) < 1e-3
+        assert np.array_equal(ys[1].view(np.uint32), oxref.silu_mul(ys[0], ys[3]).view(np.uint32))
+        assert np.array_equal(ys[4].view(np.uint32), oxref.silu_mul(ys[2], ys[0]).view(np.uint32))
+        alone = np.zeros((t, n_out), np.float32)
+        assert be.matvec_rows(x, t, n_in, [(ws[2], None, alone)])
+        assert np.array_equal(alone.view(np.uint32), ys[2].view(np.uint32))
