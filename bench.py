@@ -406,8 +406,22 @@ def bench_moe(be, torch, synth, steps, warmup, pool_gb, t, experts, int8=False):
         be.moe_routed(devs[i % len(devs)], x, logits, k, y, sel=sel)
     wall, ms = timed_steps(torch, step, steps, warmup)
     ach = nbytes / (ms * 1e-3) / 1e9
+    replayed = None
+    if t == 1:
+        # the same pass recorded once per weight copy (oxhip_plan_*) and replayed: one host call submits its launches
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            plans = []
+            for d in devs:
+                be.moe_routed(d, x, logits, k, y, sel=sel)
+                plans.append(be.plan_record(lambda d=d: be.moe_routed(d, x, logits, k, y, sel=sel)))
+            pwall, pms = timed_steps(torch, lambda i: plans[i % len(plans)].replay(), steps, warmup)
+            side.synchronize()
+        replayed = {"what": "the same pass as a recorded plan (oxhip_plan_replay: one submission for its launches)", "launches": int(plans[0].launches),
+                    "ms_per_step": round(pwall / steps * 1e3, 5), "value": round(nbytes * steps / pwall / 1e9, 2), "avg_us_by_events": round(pms * 1e3, 2)}
+        del plans
     return dict(base_line(steps, warmup), value=round(nbytes * steps / wall / 1e9, 2), unit="GB/s", ms_per_step=round(wall / steps * 1e3, 5),
-                dtype="bf16" if prefill_form else "int8",
+                dtype="bf16" if prefill_form else "int8", **({"plan_replay": replayed} if replayed else {}),
                 config={"workload": f"configs[3]: MoE 128 experts top-8, h 2048, inter 768, MLX 4-bit g64, T = {t}",
                         "experts_touched": touched, "bytes_per_step": nbytes, "flops_per_step": flops,
                         "events": "around routing + the MoE call"},
@@ -604,7 +618,7 @@ def summary(line, cpu):
     for k in ("ceiling",):
         if k in r:
             e[k] = r[k]
-    for k in ("shared_launch_of_4", "steady_stream", "cache_resident", "tflops"):
+    for k in ("shared_launch_of_4", "steady_stream", "cache_resident", "tflops", "plan_replay"):
         if k in line:
             e[k] = line[k]
     e["cpu_baseline"] = cpu

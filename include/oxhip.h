@@ -316,6 +316,28 @@ int oxhip_dev_experts(oxhip_ctx* ctx, oxhip_moe* m, const float* x, size_t t, co
 int oxhip_dev_moe_routed(oxhip_ctx* ctx, oxhip_moe* m, const float* x, size_t t, const float* logits, size_t logit_stride, size_t k,
                          const float* expert_scale, uint32_t* sel, float* y, int add, void* stream);
 
+/* ---- a recorded chain of device-pointer ops, replayed as one submission ---------------------------------------------
+ * The matmul side of DecodePlan::step (src/gpu_decode.rs:572-587; CUDA's per-graph launch list, src/cuda_decode.rs:1044-1049):
+ * a token's ops (norm + quantize, linears, route, experts, ...) are issued once between oxhip_plan_begin and
+ * oxhip_plan_end on `stream` (a stream of the caller's, not the null stream), where they are recorded instead of run; every
+ * oxhip_plan_replay then submits the whole chain with one call. The recorded launches read and write the same device
+ * buffers every time (the plan's arena, oxhip_buf_alloc): a new token is new contents in those buffers. Results are those
+ * of the same calls issued one by one, bit for bit.
+ * Before recording, run the chain once on the same stream: scratch that grows on first use (K-slice rows of the stream, an
+ * MoE layer's pass buffers) must exist, since a recorded call can neither allocate nor wait; one that would have to makes
+ * oxhip_plan_end fail (0, nothing replayable). Calls with timing events (oxhip_dev_decode_batch's ev_start / ev_stop,
+ * oxhip_dev_gemm_timed) and the host-pointer surface cannot be recorded. While a plan records on a stream, no other
+ * thread may use that stream. A plan holds no buffers of its own: free the weights and buffers it names after the plan. */
+typedef struct oxhip_plan oxhip_plan;
+oxhip_plan* oxhip_plan_begin(oxhip_ctx* ctx, void* stream);
+int oxhip_plan_end(oxhip_plan* plan);
+/* Launches the plan holds (0 before oxhip_plan_end succeeded). */
+size_t oxhip_plan_launches(const oxhip_plan* plan);
+/* Submits the recorded chain on `stream` (NULL: the stream it was recorded on). */
+int oxhip_plan_replay(oxhip_plan* plan, void* stream);
+/* Also abandons a recording in progress. */
+void oxhip_plan_free(oxhip_plan* plan);
+
 /* The exact integer accumulators of the decode kernels, written by the kernels themselves: per
  * block of 32 ([t, n_out, n_in/32]) for Q4, Q8, Q8_0, Q4_K and Q5_K, per 16 ([t, n_out, n_in/16]) for Q6_K.
  * For parity checks (the CPU's per-16 sums add up to the per-32 ones exactly). */

@@ -9,7 +9,7 @@ CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "liboxinfer_hip.so")
 OBJ = os.path.join(HERE, "build")
 
-SOURCES = ["act.hip", "dequant.hip", "decode.hip", "decode_mfma.hip", "decode_fp8.hip", "moe.hip", "moe_bf16.hip", "gemm.hip", "gemm_fp8.hip", "gemm_i8.hip", "backend.hip", "backend_moe.hip", "backend_gemm.hip", "graph_ops.hip", "backend_graph.hip"]
+SOURCES = ["act.hip", "dequant.hip", "decode.hip", "decode_mfma.hip", "decode_fp8.hip", "moe.hip", "moe_bf16.hip", "gemm.hip", "gemm_fp8.hip", "gemm_i8.hip", "backend.hip", "backend_moe.hip", "backend_gemm.hip", "graph_ops.hip", "backend_graph.hip", "backend_plan.hip"]
 
 # -ffp-contract=off: multiply-adds fuse only where the source says fmaf (the bit-exact dequantizers
 # need the reference's unfused operations). Packed-FP32 instructions are switched off.

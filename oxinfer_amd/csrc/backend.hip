@@ -523,7 +523,8 @@ static int decode_one(oxhip_ctx* c, const oxhip_weight* w, const oxhip_qact* xa,
     HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
     StreamScratch* sc = scratch_for(c, static_cast<hipStream_t>(stream), needs_slices(w));
     if (!sc) {
-        set_error("decode: device memory short");
+        set_error(stream_recording(static_cast<hipStream_t>(stream)) ? "decode: the stream's K-slice scratch does not exist yet and a plan records on it (run the chain once before recording)"
+                                                                     : "decode: device memory short");
         return 0;
     }
     HIP_TRY(launch_decode(w->v, v, x, t, y, static_cast<hipStream_t>(stream), sc->dec, ev_start, ev_stop), "decode launch");
@@ -587,7 +588,8 @@ int oxhip_dev_decode_batch(oxhip_ctx* c, const oxhip_decode_job* jobs, size_t n_
     for (size_t k = 0; k < n_jobs; k++) any_slices |= jobs[k].w && needs_slices(jobs[k].w);
     StreamScratch* ssc = scratch_for(c, s, any_slices);
     if (!ssc) {
-        set_error("decode_batch: device memory short");
+        set_error(stream_recording(s) ? "decode_batch: the stream's K-slice scratch does not exist yet and a plan records on it (run the chain once before recording)"
+                                      : "decode_batch: device memory short");
         return 0;
     }
     // Runs of jobs that the matrix-core decode kernel takes share one launch; the others go out one by one.

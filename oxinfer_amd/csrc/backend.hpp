@@ -63,6 +63,8 @@ struct oxhip_weight {
     size_t bytes = 0;
 };
 
+#include <set>
+
 struct oxhip_ctx {
     int device = 0;
     std::string name;
@@ -73,6 +75,7 @@ struct oxhip_ctx {
     oxhip::DecodeScratch dec;  // partial rows and counters of the decode kernels that split K across workgroups (host surface, on `stream`)
     std::mutex smu;            // guards per_stream
     std::map<hipStream_t, oxhip::StreamScratch*> per_stream;  // the device-pointer entry points' scratch, by calling stream
+    std::set<hipStream_t> record_failed;  // streams whose plan recording met a call that had to allocate (guarded by smu)
     double ms_in = 0, ms_gpu = 0, ms_out = 0;
     size_t calls = 0;
 };
@@ -86,6 +89,23 @@ int gemm_bf16_run(DevBuf& ws, const oxhip_weight* w, const void* x, bool x_bf16,
 StreamScratch* scratch_for(oxhip_ctx* c, hipStream_t s, bool slices);
 void free_stream_scratch(oxhip_ctx* c);
 bool needs_slices(const oxhip_weight* w);  // a decode launch of this weight alone slices K across workgroups
+
+// True while `s` records a plan (stream capture): a call must then not allocate, free, wait or clear with a memset.
+inline bool stream_recording(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    return s && hipStreamIsCapturing(s, &st) == hipSuccess && st == hipStreamCaptureStatusActive;
+}
+// Called before a device-pointer entry point allocates on behalf of stream `s`: false (error set, the recording marked
+// failed so that oxhip_plan_end declines) while a plan records there.
+inline bool may_allocate(oxhip_ctx* c, hipStream_t s, const char* who) {
+    if (!stream_recording(s)) return true;
+    {
+        std::lock_guard<std::mutex> g(c->smu);
+        c->record_failed.insert(s);
+    }
+    set_error(std::string(who) + ": this call would have to allocate device memory while a plan records on its stream (run the chain once before recording)");
+    return false;
+}
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 

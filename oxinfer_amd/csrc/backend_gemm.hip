@@ -7,6 +7,21 @@ namespace oxhip {
 
 thread_local KernelSpan g_kernel_span;
 
+// The GEMMs' packed activations grow on first use (with a wait for the stream): not while a plan records on the stream.
+static bool grow_ws(DevBuf& ws, size_t bytes, hipStream_t s) {
+    if (ws.cap >= bytes) return true;
+    if (stream_recording(s)) {
+        set_error("gemm: this call would have to allocate device memory while a plan records on its stream (run the chain once before recording)");
+        return false;
+    }
+    (void)hipStreamSynchronize(s);  // an earlier GEMM may still read the old scratch
+    if (!ws.grow(bytes)) {
+        set_error("gemm: device memory short");
+        return false;
+    }
+    return true;
+}
+
 // Packs x and runs the bf16 GEMM; the packed activations live in `ws` (the calling stream's scratch: grown on first use).
 int gemm_bf16_run(DevBuf& ws, const oxhip_weight* w, const void* x, bool x_bf16, size_t t, void* y, bool y_bf16, hipStream_t s) {
     const bool fp8 = w->v.fmt == FMT_FP8;
@@ -16,13 +31,7 @@ int gemm_bf16_run(DevBuf& ws, const oxhip_weight* w, const void* x, bool x_bf16,
     }
     if (fp8 && skinny_fp8_ok(w->v, t)) {  // up to 32 tokens: bandwidth-bound, one pass over the weights
         const size_t need = skinny_fp8_pack_bytes(w->v, t, 1);
-        if (ws.cap < need) {
-            (void)hipStreamSynchronize(s);
-            if (!ws.grow(need)) {
-                set_error("gemm: device memory short");
-                return 0;
-            }
-        }
+        if (!grow_ws(ws, need, s)) return 0;
         span_start(s);  // (the skinny kernel and its packing launch count as one)
         HIP_TRY(launch_skinny_fp8(w->v, x, x_bf16, false, t, y, y_bf16, ws.p, s), "fp8 skinny launch");
         span_stop(s);
@@ -32,13 +41,7 @@ int gemm_bf16_run(DevBuf& ws, const oxhip_weight* w, const void* x, bool x_bf16,
     const size_t pack_bytes = align_up(mtiles * kblocks * 64 * 16, 256);
     const uint32_t slices = gemm_k_slices(w->v, mtiles);
     const size_t bytes = pack_bytes + (slices > 1 ? (size_t)slices * t * w->v.n_out * 4 : 0);
-    if (ws.cap < bytes) {
-        (void)hipStreamSynchronize(s);  // an earlier GEMM may still read the old scratch
-        if (!ws.grow(bytes)) {
-            set_error("gemm: device memory short");
-            return 0;
-        }
-    }
+    if (!grow_ws(ws, bytes, s)) return 0;
     HIP_TRY(launch_pack_a(x, x_bf16, gemm_bf16_pack_mode(w->v), t, w->v.n_in, mtiles, kblocks, ws.p, s), "gemm pack launch");
     float* partial = reinterpret_cast<float*>(static_cast<uint8_t*>(ws.p) + pack_bytes);
     HIP_TRY(launch_gemm_bf16(w->v, ws.p, t, mtiles, y, y_bf16, partial, s), "gemm launch");
@@ -55,13 +58,7 @@ int gemm_fp8_run(DevBuf& ws, const oxhip_weight* w, const void* x, bool x_bf16, 
     const size_t pack_bytes = align_up(mtiles * kblocks * 64 * 32, 256), sx_bytes = align_up(kblocks * mtiles * 16 * 4, 256);
     const uint32_t slices = gemm_fp8_k_slices(w->v, mtiles);
     const size_t bytes = pack_bytes + sx_bytes + (slices > 1 ? (size_t)slices * t * w->v.n_out * 4 : 0);
-    if (ws.cap < bytes) {
-        (void)hipStreamSynchronize(s);
-        if (!ws.grow(bytes)) {
-            set_error("gemm: device memory short");
-            return 0;
-        }
-    }
+    if (!grow_ws(ws, bytes, s)) return 0;
     uint8_t* base = static_cast<uint8_t*>(ws.p);
     float* sx = reinterpret_cast<float*>(base + pack_bytes);
     float* partial = reinterpret_cast<float*>(base + pack_bytes + sx_bytes);
@@ -85,13 +82,7 @@ int gemm_i8_run(DevBuf& ws, const oxhip_weight* w, const void* x, bool x_bf16, s
     const uint32_t slices = gemm_i8_k_slices(w->v, t);
     const bool direct = slices == 1 && !y_bf16 && y;
     const size_t bytes = frag_bytes + xs_bytes + fs_bytes + (direct ? 0 : (size_t)slices * t * w->v.n_out * 4);
-    if (ws.cap < bytes) {
-        (void)hipStreamSynchronize(s);
-        if (!ws.grow(bytes)) {
-            set_error("gemm: device memory short");
-            return 0;
-        }
-    }
+    if (!grow_ws(ws, bytes, s)) return 0;
     uint8_t* base = static_cast<uint8_t*>(ws.p);
     void *frag = base, *xs = base + frag_bytes, *fs = base + frag_bytes + xs_bytes;
     float* partial = reinterpret_cast<float*>(base + frag_bytes + xs_bytes + fs_bytes);
@@ -133,12 +124,18 @@ int oxhip_dev_gemm(oxhip_ctx* c, const oxhip_weight* w, const void* x, int x_dty
         return 0;
     }
     DevBuf& ws = sc->gemm_ws;
+    int rc = 0;
     switch (variant) {
-        case OXHIP_GEMM_BF16: return gemm_bf16_run(ws, w, x, x_dtype == OXHIP_BF16, t, y, y_dtype == OXHIP_BF16, s);
-        case OXHIP_GEMM_I8: return gemm_i8_run(ws, w, x, x_dtype == OXHIP_BF16, t, y, y_dtype == OXHIP_BF16, nullptr, s);
-        case OXHIP_GEMM_FP8: return gemm_fp8_run(ws, w, x, x_dtype == OXHIP_BF16, t, y, y_dtype == OXHIP_BF16, s);
+        case OXHIP_GEMM_BF16: rc = gemm_bf16_run(ws, w, x, x_dtype == OXHIP_BF16, t, y, y_dtype == OXHIP_BF16, s); break;
+        case OXHIP_GEMM_I8: rc = gemm_i8_run(ws, w, x, x_dtype == OXHIP_BF16, t, y, y_dtype == OXHIP_BF16, nullptr, s); break;
+        case OXHIP_GEMM_FP8: rc = gemm_fp8_run(ws, w, x, x_dtype == OXHIP_BF16, t, y, y_dtype == OXHIP_BF16, s); break;
         default: set_error("gemm: unknown variant"); return 0;
     }
+    if (!rc && stream_recording(s)) {  // a declined call leaves a hole in a recording: the plan must not be replayable
+        std::lock_guard<std::mutex> g(c->smu);
+        c->record_failed.insert(s);
+    }
+    return rc;
 }
 
 int oxhip_dev_gemm_timed(oxhip_ctx* c, const oxhip_weight* w, const void* x, int x_dtype, size_t t, void* y, int y_dtype, int variant,

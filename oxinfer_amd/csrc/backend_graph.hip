@@ -25,6 +25,10 @@ StreamScratch* scratch_for(oxhip_ctx* c, hipStream_t s, bool slices) {
         c->per_stream.emplace(s, sc);
     }
     if (slices && !sc->dec.partial) {
+        if (stream_recording(s)) {  // (smu is held: the failure is noted here, not through may_allocate)
+            c->record_failed.insert(s);
+            return nullptr;
+        }
         DecodeScratch d;
         d.partial_floats = c->dec.partial_floats;
         d.ncounters = c->dec.ncounters;
@@ -187,7 +191,8 @@ int oxhip_dev_linear(oxhip_ctx* c, const oxhip_weight* w, const oxhip_weight* w2
     HIP_TRY(hipSetDevice(c->device), "hipSetDevice");
     StreamScratch* sc = scratch_for(c, s, needs_slices(w));
     if (!sc) {
-        set_error("linear: device memory short");
+        set_error(stream_recording(s) ? "linear: the stream's K-slice scratch does not exist yet and a plan records on it (run the chain once before recording)"
+                                      : "linear: device memory short");
         return 0;
     }
     const size_t n_out = w->v.n_out;
@@ -204,6 +209,7 @@ int oxhip_dev_linear(oxhip_ctx* c, const oxhip_weight* w, const oxhip_weight* w2
             return 1;
         }
         // formats whose kernels only store: the product goes to scratch, the mode is a small kernel of its own
+        if (sc->tmp.cap < t * n_out * 4 && !may_allocate(c, s, "linear")) return 0;
         if (!sc->tmp.grow(t * n_out * 4)) {
             set_error("linear: device memory short");
             return 0;
@@ -223,6 +229,7 @@ int oxhip_dev_linear(oxhip_ctx* c, const oxhip_weight* w, const oxhip_weight* w2
         return 1;
     }
     // the other formats: both products into scratch, then the gate
+    if (sc->tmp.cap < 2 * t * n_out * 4 && !may_allocate(c, s, "linear")) return 0;
     if (!sc->tmp.grow(2 * t * n_out * 4)) {
         set_error("linear: device memory short");
         return 0;

@@ -95,6 +95,7 @@ int moe_pass(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_
     float* rw_out = const_cast<float*>(route_w);
     bool routed = rin.logits == nullptr;  // the routes are there (given, or already formed)
     if (pairs > m->ws_pairs || t > m->ws_t) {
+        if (!may_allocate(c, s, "moe")) return 0;
         (void)hipStreamSynchronize(s);  // an earlier pass may still read the old scratch
         const size_t np = pairs > m->ws_pairs ? pairs : m->ws_pairs, nt = t > m->ws_t ? t : m->ws_t;
         Scratch probe = carve(nullptr, nt, np, m->n_exp, h, inter);

@@ -112,6 +112,11 @@ def load_library():
         "oxhip_dev_route": (C.c_int, [vp, vp, vp, vp, sz, sz, sz, sz, vp, vp, vp, vp]),
         "oxhip_dev_experts": (C.c_int, [vp, vp, vp, sz, vp, sz, vp, C.c_int, vp]),
         "oxhip_dev_moe_routed": (C.c_int, [vp, vp, vp, sz, vp, sz, sz, vp, vp, vp, C.c_int, vp]),
+        "oxhip_plan_begin": (vp, [vp, vp]),
+        "oxhip_plan_end": (C.c_int, [vp]),
+        "oxhip_plan_launches": (sz, [vp]),
+        "oxhip_plan_replay": (C.c_int, [vp, vp]),
+        "oxhip_plan_free": (None, [vp]),
         "oxhip_event_create": (vp, []),
         "oxhip_event_destroy": (None, [vp]),
         "oxhip_event_elapsed_ms": (C.c_float, [vp, vp]),
@@ -166,6 +171,26 @@ class DeviceMoe:
     def __del__(self):
         if getattr(self, "handle", None) and self.be.ctx:
             load_library().oxhip_free_moe(self.be.ctx, self.handle)
+            self.handle = None
+
+
+class Plan:
+    """A recorded chain of device-pointer ops (oxhip_plan_*): the matmul side of `DecodePlan` (src/gpu_decode.rs:572-587)."""
+
+    def __init__(self, be, handle):
+        self.be, self.handle = be, handle
+
+    @property
+    def launches(self):
+        return load_library().oxhip_plan_launches(self.handle)
+
+    def replay(self, stream=None):
+        if not load_library().oxhip_plan_replay(self.handle, C.c_void_p(stream) if stream else None):
+            raise RuntimeError(self.be.last_error())
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            load_library().oxhip_plan_free(self.handle)
             self.handle = None
 
 
@@ -474,6 +499,23 @@ class HipBackend:
         if not ok:
             raise RuntimeError(self.last_error())
         return sel
+
+    def plan_record(self, chain):
+        """Records chain() (device-pointer calls on the current torch stream, which must not be the null stream) and
+        returns a Plan; raises when the recording fails. Run chain() once on that stream beforehand."""
+        h = self.lib.oxhip_plan_begin(self.ctx, self._stream())
+        if not h:
+            raise RuntimeError(self.last_error())
+        try:
+            chain()
+        except BaseException:
+            self.lib.oxhip_plan_free(h)
+            raise
+        if not self.lib.oxhip_plan_end(h):
+            msg = self.last_error()
+            self.lib.oxhip_plan_free(h)
+            raise RuntimeError(msg)
+        return Plan(self, h)
 
     def decode_jobs(self, jobs):
         """Builds a reusable job array for decode_batch: jobs = [(DeviceWeight, QAct | None, x | None, t, y, ev0, ev1)]."""

@@ -318,3 +318,126 @@ def test_layer_chain_stays_on_the_device(be, oxref, ne, h, inter, k):
         only = torch.full((t, h), float("nan"), device="cuda")
         assert be.experts(moe, normed, sel, only, add=False)
         assert row_err(only.cpu().numpy(), y2 - y1) < TOL
+
+
+@pytest.mark.parametrize("ne,h,inter,k,t", [(16, 2048, 768, 8, 1), (6, 256, 128, 3, 4)])
+def test_plan_replays_a_layer_bit_for_bit(be, oxref, ne, h, inter, k, t):
+    """A token's chain of ops recorded once and replayed (the matmul side of DecodePlan::step, src/gpu_decode.rs:572-587):
+    quantize -> gate / up pair linear -> quantize -> down linear (Add) -> RMSNorm + quantize -> Route -> Experts (add) ->
+    a K-sliced linear. Every replay, each on new contents of the same input buffer and with eager work and
+    synchronizations between the replays, must equal the same chain issued call by call, bit for bit; and that chain is
+    itself held to the oracle."""
+    import torch
+    from oxinfer_amd import hip, synth
+    ffn = 512
+    raw_gu = [synth.mlx_q4(2 * inter, h, 5100 + e) for e in range(ne)]
+    raw_dn = [synth.mlx_q4(h, inter, 5200 + e) for e in range(ne)]
+    q_gu = [oxref.from_mlx_q4(*r, 2 * inter, h, 64) for r in raw_gu]
+    q_dn = [oxref.from_mlx_q4(*r, h, inter, 64) for r in raw_dn]
+    moe = be.upload_moe([be.desc_mlx_q4(*r, 64, 2 * inter, h) for r in raw_gu], [be.desc_mlx_q4(*r, 64, h, inter) for r in raw_dn], h, inter)
+    assert moe is not None, be.last_error()
+    g_raw, u_raw, d_raw = synth.gguf_q4_k(ffn, h, 5300), synth.gguf_q4_k(ffn, h, 5301), synth.gguf_q8_0(h, ffn, 5302)
+    wg, wu, wd = be.upload_gguf(Q4_K, g_raw, ffn, h), be.upload_gguf(Q4_K, u_raw, ffn, h), be.upload_gguf(Q8_0, d_raw, h, ffn)
+    big_raw = synth.gguf_q8_0(272, 14336, 5303)                       # 14336 columns: its K slices meet through the stream's scratch
+    wbig = be.upload_gguf(Q8_0, big_raw, 272, 14336)
+    rng = np.random.default_rng(5400 + ne)
+    router = dev(rng.normal(0, 0.2, (ne, h)).astype(np.float32))
+    wn = dev((1.0 + 0.1 * rng.normal(size=h)).astype(np.float32))
+    # the plan's buffers: allocated once, named by every recorded launch
+    x_in = torch.zeros((t, h), device="cuda")
+    xbig = torch.zeros((t, 14336), device="cuda")
+    y = torch.zeros((t, h), device="cuda")
+    a = torch.zeros((t, ffn), device="cuda")
+    normed = torch.zeros((t, h), device="cuda")
+    ybig = torch.zeros((t, 272), device="cuda")
+    logits = torch.zeros((t, ne), device="cuda")
+    sel = torch.zeros((2, t, k), dtype=torch.int32, device="cuda")
+    qx, qa, qn, qbig = hip.QAct(t, h, "cuda"), hip.QAct(t, ffn, "cuda"), hip.QAct(t, h, "cuda"), hip.QAct(t, 14336, "cuda")
+    C = __import__("ctypes")
+
+    def chain():
+        be.quantize_act(x_in, out=qx)
+        assert be.linear(wg, a, xa=qx, t=t, mode=hip.LIN_SILU_PAIR, w2=wu), be.last_error()
+        be.quantize_act(a, out=qa)
+        assert be.linear(wd, y, xa=qa, t=t, mode=hip.LIN_ADD), be.last_error()
+        ok = be.lib.oxhip_dev_rmsnorm_quantize(be.ctx, y.data_ptr(), wn.data_ptr(), None, 1e-6, t, h, normed.data_ptr(), C.byref(qn.c), be._stream())
+        assert ok, be.last_error()
+        ok = be.lib.oxhip_dev_route(be.ctx, normed.data_ptr(), router.data_ptr(), None, t, ne, h, k, logits.data_ptr(), sel.data_ptr(), None, be._stream())
+        assert ok, be.last_error()
+        assert be.experts(moe, normed, sel, y, add=True), be.last_error()
+        be.quantize_act(xbig, out=qbig)
+        assert be.linear(wbig, ybig, xa=qbig, t=t), be.last_error()
+
+    stream = torch.cuda.Stream()
+    inputs = [(synth.activations(t, h, 5500 + i), synth.activations(t, h, 5600 + i), synth.activations(t, 14336, 5700 + i)) for i in range(4)]
+
+    def load(i):
+        x_in.copy_(dev(inputs[i][0]))
+        y.copy_(dev(inputs[i][1]))
+        xbig.copy_(dev(inputs[i][2]))
+
+    eager = []
+    with torch.cuda.stream(stream):
+        for i in range(4):   # call by call (the first pass also creates every scratch the chain needs)
+            load(i)
+            chain()
+            stream.synchronize()
+            eager.append((y.cpu().numpy().copy(), ybig.cpu().numpy().copy(), sel.cpu().numpy().copy(), a.cpu().numpy().copy()))
+        # the call-by-call chain against the oracle (input 0)
+        x0, r0, xb0 = inputs[0]
+        gate = oxref.gguf_decode(Q4_K, g_raw, ffn, h, x0, t)
+        act = oxref.silu_mul(gate, oxref.gguf_decode(Q4_K, u_raw, ffn, h, x0, t))
+        assert row_err(eager[0][3], act) < TOL
+        y1 = r0 + oxref.gguf_decode(Q8_0, d_raw, h, ffn, eager[0][3], t)
+        n1 = rmsnorm_ref(y1, wn.cpu().numpy(), 1e-6)
+        idx = eager[0][2][0].view(np.uint32)
+        wts = eager[0][2][1].view(np.float32)
+        y2 = oxref.moe_q4(q_gu, q_dn, 64, h, inter, n1, t, idx, wts, y1, decode_path=True)
+        assert row_err(eager[0][0], y2) < 2 * TOL, row_err(eager[0][0], y2)
+        assert row_err(eager[0][1], oxref.gguf_decode(Q8_0, big_raw, 272, 14336, xb0, t)) < TOL
+        plan = be.plan_record(chain)
+        assert plan.launches >= 9
+        for rnd in range(2):
+            for i in (2, 0, 3, 1):
+                load(i)
+                plan.replay()
+                stream.synchronize()
+                got = (y.cpu().numpy(), ybig.cpu().numpy(), sel.cpu().numpy(), a.cpu().numpy())
+                for g_, e_ in zip(got, eager[i]):
+                    assert np.array_equal(g_.view(np.uint32), e_.view(np.uint32)), (rnd, i)
+                # eager work of the program's own between the replays (another matmul through the same scratch)
+                be.quantize_act(xbig, out=qbig)
+                assert be.linear(wbig, ybig, xa=qbig, t=t)
+                torch.cuda.synchronize()
+        del plan
+
+
+def test_plan_recording_on_a_cold_stream_declines(be, oxref):
+    """Recording on a stream whose scratch does not exist yet: the call that would have to allocate declines, the
+    recording is refused as a whole (oxhip_plan_end returns 0, nothing is replayable) and the stream works again
+    afterwards; once the chain has run there, the same recording succeeds. The null stream is refused."""
+    import torch
+    assert not be.lib.oxhip_plan_begin(be.ctx, None)
+    raw, _ = oxref.random_blocks(8, 272 * 14336 // 32, 1)
+    w = be.upload_gguf(8, raw, 272, 14336)
+    x = torch.ones((1, 14336), device="cuda")
+    stream = torch.cuda.Stream()   # a fresh stream: its K-slice scratch does not exist yet
+    with torch.cuda.stream(stream):
+        qa = be.quantize_act(x)
+        y = torch.full((1, 272), 3.0, device="cuda")
+        stream.synchronize()
+        free0, _ = torch.cuda.mem_get_info()
+        with pytest.raises(RuntimeError, match="before recording"):
+            be.plan_record(lambda: be.linear(w, y, xa=qa, t=1))
+        stream.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free0 and float(y.min()) == 3.0   # nothing allocated, nothing run
+        assert be.linear(w, y, xa=qa, t=1), be.last_error()      # the same call outside a recording: allocates and runs
+        stream.synchronize()
+        want = y.cpu().numpy().copy()
+        assert row_err(want, oxref.gguf_decode(8, raw, 272, 14336, np.ones((1, 14336), np.float32), 1)) < TOL
+        plan = be.plan_record(lambda: be.linear(w, y, xa=qa, t=1))  # warmed now: recordable
+        assert plan.launches >= 1
+        y.zero_()
+        plan.replay()
+        stream.synchronize()
+        assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
