@@ -221,7 +221,7 @@ int oxhip_dev_linear(oxhip_ctx* c, const oxhip_weight* w, const oxhip_weight* w2
     }
     // y = act(W x) * (W2 x). The matrix-core decode kernel pairs the two matrices' tiles of the same rows in one workgroup and
     // applies the gate in its output stage: one launch, no intermediate rows (bit-identical to the two products and Op::Glu)
-    if (mfma_decode_format(w->v.fmt)) {
+    if (decode_pair_ok(w->v)) {
         Epi pe;
         pe.pair_p0 = w2->v.p0;
         pe.pair_act = mode == OXHIP_LIN_GELU_PAIR ? 1u : 0u;

@@ -457,7 +457,7 @@ int oxhip_matvec_rows(oxhip_ctx* c, const float* x, size_t t, size_t n_in, oxhip
         const oxhip_rows_job& jb = jobs[j];
         const size_t n = t * jb.n_out;
         at[j] = off;
-        const bool pairable = !jb.up || (jb.up->v.fmt == jb.w->v.fmt && mfma_decode_format(jb.w->v.fmt));
+        const bool pairable = !jb.up || (jb.up->v.fmt == jb.w->v.fmt && decode_pair_ok(jb.w->v));
         if (pairable && !is_dense(jb.w) && decode_batchable(jb.w->v, t)) {
             Epi e;
             if (jb.up) e.pair_p0 = jb.up->v.p0;

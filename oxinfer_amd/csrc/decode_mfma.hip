@@ -882,8 +882,9 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
 // Dynamic LDS is declared 16-byte aligned whatever static LDS a kernel also holds: the 8- and 16-byte LDS reads are split
 // into dwords (and the kernel runs two to three times longer) when the array starts at an odd dword.
 // (Grouped launches keep to 8 waves, which leaves them 256 registers for the accumulators of their token groups.)
+// (Q6_K: bounded at 8 waves like its shared-launch kernel, see decode_batch_kernel)
 template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS, int NG>
-__global__ __launch_bounds__(GROUPED ? 512 : 1024) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt,
+__global__ __launch_bounds__(GROUPED || FMT == FMT_Q6_K ? 512 : 1024) void decode_mfma_kernel(WeightView w, QActView xa, uint32_t t, uint32_t rt,
                                                                            uint32_t kw, float* __restrict__ y,
                                                                            int32_t* __restrict__ dump, GroupView grp, uint32_t ksplit,
                                                                            float* __restrict__ partial,
@@ -933,8 +934,10 @@ __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid,
 constexpr uint32_t fbit(int f) { return 1u << f; }
 constexpr uint32_t FSET_GGUF = fbit(FMT_Q8_0) | fbit(FMT_Q4_K), FSET_Q6K = fbit(FMT_Q6_K), FSET_MLX = fbit(FMT_Q4M),
                    FSET_ALL = FSET_GGUF | FSET_Q6K | FSET_MLX | fbit(FMT_Q8F) | fbit(FMT_Q5_K) | fbit(FMT_Q40) | fbit(FMT_MXFP4);
+// (Q6_K alone: its step needs a dozen registers more than the 128 that workgroups of 16 waves leave a wave, and spilled them
+// around its loop; its shapes never exceed 8 waves, so its kernel is bounded at 512 threads and keeps them in registers)
 template <uint32_t FSET>
-__global__ __launch_bounds__(1024) void decode_batch_kernel(BatchArgs a) {
+__global__ __launch_bounds__(FSET == (1u << FMT_Q6_K) ? 512 : 1024) void decode_batch_kernel(BatchArgs a) {
     extern __shared__ __align__(16) float lds_dyn[];
     uint32_t j = 0;
     while (j + 1 < a.njobs && blockIdx.x >= a.j[j + 1].wg0) j++;  // uniform
@@ -1042,7 +1045,7 @@ Shape shape_for(uint32_t ntiles, uint32_t nsteps, bool allow_slices, int fmt) {
 // A gate / up pair: a workgroup holds the tiles of the same rows of both matrices, so its tile count is even; kw and ks (the
 // order of a row's sum) stay what the weight's shape alone gives, which keeps each product's bits those of a launch of its own.
 Shape pair_shape(Shape sh) {
-    if (sh.rt % 2) sh.rt *= 2;  // (rt * kw <= 8 before: at most 16 waves)
+    if (sh.rt % 2) sh.rt = (sh.rt + 1) * sh.kw <= 8 ? sh.rt + 1 : sh.rt > 1 ? sh.rt - 1 : 2;  // (rt = 1 with kw = 8: 16 waves)
     return sh;
 }
 uint32_t pair_tiles(const Shape& sh, bool pair) { return pair ? pair_shape(sh).rt / 2 : sh.rt; }
@@ -1206,6 +1209,14 @@ uint32_t steps_rt(const WeightView& w) {
                                : steps_of<FMT_Q4M>(w.n_in);
 }
 }  // namespace
+
+// Whether a gate / up pair of this weight's shape and format runs as one launch (its workgroup of paired tiles fits the
+// kernel's bound: Q6_K's kernels take at most 8 waves).
+bool decode_pair_ok(const WeightView& w) {
+    if (!mfma_decode_format(w.fmt)) return false;
+    const Shape sh = pair_shape(shape_for(row_tiles(w.n_out), steps_rt(w), true, w.fmt));
+    return sh.rt * sh.kw <= (w.fmt == FMT_Q6_K ? 8u : 16u);
+}
 
 bool decode_batchable(const WeightView& w, size_t t) {
     if (!mfma_decode_format(w.fmt)) return false;

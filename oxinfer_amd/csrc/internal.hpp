@@ -174,6 +174,7 @@ struct DecodeBatchItem {
     Epi epi{};
 };
 void decode_scratch_need(const WeightView& w, size_t* partial_floats, size_t* ncounters, bool pair = false);  // of a launch that slices K; else zeros (a pair launch: twice the floats)
+bool decode_pair_ok(const WeightView& w);  // a gate / up pair of this shape and format runs as one launch (Epi::pair_p0)
 bool decode_batchable(const WeightView& w, size_t t);  // the kernel takes it and its activations fit LDS
 // ev_start / ev_stop (optional): timing events around the launches.
 hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s, hipEvent_t ev_start = nullptr,
