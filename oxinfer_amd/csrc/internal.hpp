@@ -255,11 +255,12 @@ hipError_t launch_rmsnorm_quantize(const float* x, const float* w_f32, const uin
                                    size_t out_stride = 0);
 // The bf16 form of the grouped expert matmuls for prefill passes (moe_bf16.hip): MLX 4-bit weights, chunks of <= 16 rows.
 bool moe_bf16_ok(const WeightView& w);
+bool moe_bf16_std_geometry(const WeightView& w);  // its fragments hold a block's columns as 8 kq + j (Q8_0, Q4_K), not as T4M records do
 size_t moe_bf16_frag_bytes(size_t max_chunks, size_t n_in);
 hipError_t launch_moe_pack_bf16(const float* x, size_t n_in, const int* rowmap, const int4* chunks, const int* nchunks, uint32_t max_chunks,
-                                void* frag, hipStream_t s);
+                                void* frag, hipStream_t s, bool std_geometry = false);
 hipError_t launch_moe_act_pack_bf16(const float* g, const float* u, size_t stride, size_t inter, uint32_t kind, float param, const int4* chunks,
-                                    const int* nchunks, uint32_t max_chunks, void* frag, hipStream_t s);
+                                    const int* nchunks, uint32_t max_chunks, void* frag, hipStream_t s, bool std_geometry = false);
 hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max_chunks, const void* frag, float* out, hipStream_t s);
 
 hipError_t launch_fill_zero(uint32_t* p, size_t n, hipStream_t s);  // n dwords, by a kernel on `s`

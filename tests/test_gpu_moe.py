@@ -166,20 +166,57 @@ def test_moe_batched_equals_one_at_a_time(be, oxref, mlx_experts):
         assert np.array_equal(y1[0].view(np.uint32), y[i].view(np.uint32)), i
 
 
+def moe_grouped_reference(oxref, kind, gate_up, down, h, inter, x, idx, w, y0):
+    """The grouped prefill path over GGUF experts (src/moe.rs:735-827): per (token, route) the f32 product of the
+    dequantized rows (matmul_quant_grouped, src/kernels.rs:195-279), Act::scalar (libm exp) between the two, combined in
+    route order."""
+    y = y0.copy()
+    t, k = idx.shape
+    for i in range(t):
+        for j in range(k):
+            e = int(idx[i, j])
+            gu = oxref.gemm_quant(kind, gate_up[e], None, None, 2 * inter, h, x[i:i + 1], 1, threads=1)[0]
+            g, u = gu[:inter], gu[inter:]
+            with np.errstate(over="ignore"):  # exp overflows to inf for very negative gates: the quotient is -0.0, as on the device
+                a = (g / (np.float32(1.0) + np.exp(-g, dtype=np.float32)) * u).astype(np.float32)
+            o = oxref.gemm_quant(kind, down[e], None, None, h, inter, a[None, :], 1, threads=1)[0]
+            y[i] = y[i] + w[i, j] * o
+    return y
+
+
 @pytest.mark.parametrize("kind", [Q4_0, Q8_0, Q4_K, MXFP4])
 def test_moe_gguf_experts(be, oxref, kind):
-    from oxinfer_amd import synth
+    """GGUF experts: decode-sized passes on the integer kernels against the decode semantics (1e-3). At prefill size (40
+    tokens, twenty routed rows per expert) they take the reference's grouped form on the bf16 matrix cores: within 2e-2 of
+    the grouped f32 path (src/moe.rs:735-827; 6e-3 when the activations are bf16 values already), and the integer kernels
+    (OXHIP_MOE_INT8) within 1e-3 of the decode semantics."""
+    from oxinfer_amd import hip, synth
     ne, h, inter, k = 4, 256, 256, 2
     gu = [oxref.random_blocks(kind, 2 * inter * h // oxref.block_size(kind), 10 + e)[0] for e in range(ne)]
     dn = [oxref.random_blocks(kind, h * inter // oxref.block_size(kind), 20 + e)[0] for e in range(ne)]
     dev = be.upload_moe([be.desc_gguf(kind, g, 2 * inter, h) for g in gu], [be.desc_gguf(kind, d, h, inter) for d in dn], h, inter)
     assert dev is not None, be.last_error()
-    for t in (1, 3, 11, 40):  # (40: twenty rows per expert, chunks of 32 rows on four accumulator sets)
+    for t in (1, 3, 11, 40):  # (40: twenty rows per expert)
         x = synth.activations(t, h, 30 + t)
         _, idx, w = make_routes(oxref, t, ne, k, 40 + t)
+        zero = np.zeros((t, h), np.float32)
+        ref = moe_reference(oxref, kind, gu, dn, h, inter, x, idx, w, zero)
         y = np.zeros((t, h), np.float32)
         assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
-        ref = moe_reference(oxref, kind, gu, dn, h, inter, x, idx, w, np.zeros((t, h), np.float32))
+        if t == 40:
+            grouped = moe_grouped_reference(oxref, kind, gu, dn, h, inter, x, idx, w, zero)
+            assert row_err(y, grouped) < 2e-2, (t, row_err(y, grouped))
+            assert row_err(y, ref) > 1e-5   # (not the integer kernels' rows: the bf16 form did run)
+            xb = synth.bf16_round(x)         # activations that are bf16 values already: only the intermediate is rounded
+            yb = np.zeros((t, h), np.float32)
+            assert be.moe(xb, t, h, inter, idx, w, k, dev, yb), be.last_error()
+            assert row_err(yb, moe_grouped_reference(oxref, kind, gu, dn, h, inter, xb, idx, w, zero)) < 6e-3
+            dev.set_mode(hip.MOE_INT8)
+            try:
+                y = np.zeros((t, h), np.float32)
+                assert be.moe(x, t, h, inter, idx, w, k, dev, y), be.last_error()
+            finally:
+                dev.set_mode(hip.MOE_AUTO)
         assert row_err(y, ref) < 1e-3, t
 
 
