@@ -37,21 +37,17 @@ ROW_BYTES = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
 FMT_NAME = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
 
 
-def profile_traffic(profile, kernel):
-    """HBM bytes per launch of `kernel` from the kept rocprofv3 summary `profiles/<profile>` (its table of scaled
-    FETCH_SIZE + WRITE_SIZE per dispatch); None when the summary or the row is missing."""
+def profile_traffic(profile):
+    """HBM bytes per launch of a roofline figure's kernel(s) from the kept rocprofv3 summary `profiles/<profile>`: its
+    "Roofline traffic:" line (FETCH_SIZE + WRITE_SIZE per dispatch, each scaled by what the counter reads for a plain
+    device copy of known size, summed over the launches the figure's time covers); None when the summary or the line
+    is missing."""
     try:
-        text = open(os.path.join(ROOT, "profiles", profile)).read()
+        text = open(os.path.join(ROOT, "profiles", profile or "-")).read()
     except OSError:
         return None
-    sect = text.split("## HBM traffic", 1)
-    if len(sect) < 2:
-        return None
-    for line in sect[1].splitlines():
-        m = re.match(r"\|\s*`" + re.escape(kernel) + r"(?:<[^`]*>)?`\s*\|.*\|\s*(\d+)\s*\|\s*$", line)
-        if m:
-            return int(m.group(1))
-    return None
+    m = re.search(r"^Roofline traffic: (\d+) bytes", text, re.M)
+    return int(m.group(1)) if m else None
 
 
 def weight_bytes(kind, n_out, n_in):
@@ -309,7 +305,7 @@ def bench_mlx_gemv(be, torch, synth, steps, warmup, pool_gb):
                 dtype="int8", config={"workload": "configs[0]: MLX 4-bit g64 GEMV 4096 -> 4096, T = 1", "bytes_per_step": nbytes,
                                       "events": "carried by the launch itself, on every fourth step"},
                 roofline={"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "decode_mfma_kernel<6, 1, ...>",
+                          "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": profile_traffic("decode_mfma_kernel_mlx_gemv.md"), "kernel": "decode_mfma_kernel<6, 1, ...>",
                           "bytes_per_launch": nbytes, "avg_launch_us": round(ms * 1e3, 2)})
     line["shared_launch_of_4"] = {"what": "a layer's four 4096 x 4096 matmuls (q, k, v, o) in one oxhip_dev_decode_batch launch, rotating copies (cold HBM)",
                                   "kernel": "decode_batch_kernel", "avg_launch_us": round(ms4 * 1e3, 2), "GBs": round(4 * nbytes / (ms4 * 1e-3) / 1e9, 1),
@@ -338,7 +334,8 @@ def bench_mlx_gemm(be, torch, synth, steps, warmup, variant_name):
     ach = flops / 2 / (ms * 1e-3) / 1e12
     peak = MFMA_PEAK[variant_name]
     roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s", "frac": round(ach / peak, 4),
-            "traffic": None, "kernel": "gemm_bf16_kernel<6, false, 2, 8, 7|8>" if variant == 0 else "gemm_i8_q4m_kernel",
+            "traffic": profile_traffic("gemm_bf16_kernel_mlx_prefill.md" if variant == 0 else "gemm_i8_q4m_kernel_mlx_prefill.md"),
+            "kernel": "gemm_bf16_kernel<6, false, 2, 8, 7|8>" if variant == 0 else "gemm_i8_q4m_kernel",
             "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3, 2), "call_us": round(step_ms * 1e3 / 2, 2)}
     if variant == 1:
         # one activation scale per token and block of 32: every int8 matrix instruction (16 x 16 x 32) is followed by a
@@ -370,7 +367,8 @@ def bench_gguf_gemm(be, torch, synth, steps, warmup, fmt):
                 config={"workload": f"GGUF {fmt.upper()} prefill GEMM, M = 512, 4096 -> 14336 and 14336 -> 4096 (bf16 matrix cores)",
                         "flops_per_step": flops, "events": GEMM_EVENTS},
                 roofline={"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_PEAK["bf16"], "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK["bf16"], 4),
-                          "traffic": None, "kernel": f"gemm_bf16_kernel<{ {'q8_0': 1, 'q4_k': 2, 'q6_k': 3}[fmt]}, false, 2, 8, 7|8>",
+                          "traffic": profile_traffic(f"gemm_bf16_kernel_gguf_{fmt}_prefill.md"),
+                          "kernel": f"gemm_bf16_kernel<{ {'q8_0': 1, 'q4_k': 2, 'q6_k': 3}[fmt]}, false, 2, 8, 7|8>",
                           "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3, 2), "call_us": round(step_ms * 1e3 / 2, 2)})
 
 
@@ -426,10 +424,15 @@ def bench_moe(be, torch, synth, steps, warmup, pool_gb, t, experts, int8=False):
                         "experts_touched": touched, "bytes_per_step": nbytes, "flops_per_step": flops,
                         "events": "around routing + the MoE call"},
                 roofline={"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+                          "frac": round(ach / HBM_PEAK_GBS, 4),
+                          "traffic": profile_traffic(f"moe_t{t}.md") if t in (1, 256) and not int8 else None,
                           "kernel": "moe_bf16_kernel<4> (grouped)" if prefill_form else "decode_mfma_kernel<6, *, false, true, true> (grouped)",
                           "bytes_per_launch": nbytes, "avg_launch_us": round(ms * 1e3, 2)},
                 tflops=round(flops / (ms * 1e-3) / 1e12, 2))
+
+
+FP8_PROFILE = {(1, 0): "fp8_m1_skinny_fp8_kernel.md", (32, 0): "fp8_m32_skinny_fp8_kernel.md",
+               (1024, 0): "fp8_m1024_gemm_bf16_kernel.md", (1024, 2): "fp8_m1024_gemm_fp8_kernel.md"}
 
 
 def fp8_weights(synth):
@@ -466,7 +469,8 @@ def bench_fp8(be, torch, synth, steps, warmup, pool_gb, m, variant_name, weights
                 config={"workload": f"configs[4]: FP8 E4M3 block-scaled GEMM [7168, 18432], M = {m}, variant {variant_name if m > 16 else 'decode'}",
                         "bytes_per_step": nbytes, "flops_per_step": flops, **({"events": GEMM_EVENTS} if call_ms is not None else {})},
                 roofline={"bound": "hbm" if hbm else "mfma", "achieved": round(ach, 1), "peak": peak, "unit": "GB/s" if hbm else "TFLOP/s",
-                          "frac": round(ach / peak, 4), "traffic": None, "kernel": kern, "avg_launch_us": round(ms * 1e3, 2),
+                          "frac": round(ach / peak, 4), "traffic": profile_traffic(FP8_PROFILE.get((m, variant))), "kernel": kern,
+                          "avg_launch_us": round(ms * 1e3, 2),
                           **({"call_us": round(call_ms * 1e3, 2)} if call_ms is not None else {})})
 
 
@@ -590,7 +594,7 @@ def bench_gguf_gemv(args, be, torch, synth, kinds, gens):
                              "frac_hbm": round(c["bytes"] / us / 1e3 / HBM_PEAK_GBS, 4)}
 
     q6k = kinds == [Q6_K]
-    traffic = profile_traffic("decode_batch_kernel_q6k_gemv.md" if q6k else "decode_batch_kernel_gguf_gemv.md", dom_symbol) if kinds in ([Q8_0, Q4_K], [Q6_K]) else None
+    traffic = profile_traffic("decode_batch_kernel_q6k_gemv.md" if q6k else "decode_batch_kernel_gguf_gemv.md") if kinds in ([Q8_0, Q4_K], [Q6_K]) else None
     out = dict(base_line(args.steps, args.warmup), value=round(value, 2), unit="GB/s", ms_per_step=round(elapsed / args.steps * 1e3, 5), dtype="int8",
                config={"workload": "configs[1]: GGUF GEMV batch 1 and 8, Llama-8B MLP shapes 4096->14336 and 14336->4096, "
                                    + " + ".join(FMT_NAME[k] for k in kinds),
@@ -614,7 +618,7 @@ def summary(line, cpu):
     r = line["roofline"]
     e = {"workload": line["config"]["workload"], "value": line["value"], "unit": line["unit"], "ms_per_step": line["ms_per_step"],
          "dtype": line["dtype"], "kernel": r["kernel"], "avg_us": r["avg_launch_us"], "bound": r["bound"],
-         "roofline_frac": r["frac"], "achieved": r["achieved"], "peak": r["peak"], "steps": line["steps"]}
+         "roofline_frac": r["frac"], "achieved": r["achieved"], "peak": r["peak"], "traffic": r["traffic"], "steps": line["steps"]}
     for k in ("ceiling",):
         if k in r:
             e[k] = r[k]

@@ -88,7 +88,7 @@ int gemm_bf16_run(DevBuf& ws, const oxhip_weight* w, const void* x, bool x_bf16,
 // slice K across workgroups, so the entry must hold the decode kernels' partial rows and counters (allocated on first need).
 StreamScratch* scratch_for(oxhip_ctx* c, hipStream_t s, bool slices);
 void free_stream_scratch(oxhip_ctx* c);
-bool needs_slices(const oxhip_weight* w);  // a decode launch of this weight alone slices K across workgroups
+bool needs_slices(const oxhip_weight* w);  // a decode launch of this weight alone uses the stream's decode scratch (K slices across workgroups, FP8's packed rows)
 
 // True while `s` records a plan (stream capture): a call must then not allocate, free, wait or clear with a memset.
 inline bool stream_recording(hipStream_t s) {

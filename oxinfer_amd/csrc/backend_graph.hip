@@ -59,6 +59,7 @@ void free_stream_scratch(oxhip_ctx* c) {
 }
 
 bool needs_slices(const oxhip_weight* w) {
+    if (w->v.fmt == FMT_FP8) return skinny_fp8_ok(w->v, 1);  // (its one-pass decode kernel keeps its packed rows in the same scratch)
     size_t p = 0, n = 0;
     decode_scratch_need(w->v, &p, &n);
     return p != 0;

@@ -929,15 +929,25 @@ __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid,
 }
 
 // FSET: the formats compiled in, one bit per Fmt. The compiler allocates registers over the whole kernel, so every
-// format in it costs the others (a seventh format made the common GGUF ones 15 % slower, and Q6_K beside Q8_0 and Q4_K
-// spilled registers inside its loop): a launch takes the smallest of the sets below that holds all its jobs' formats.
+// format in it costs the others (a seventh format made the common GGUF ones 15 % slower, Q6_K beside Q8_0 and Q4_K
+// spilled registers inside its loop, and one kernel of all formats spilled 480 registers): the formats are split into
+// the sets below, and a call whose jobs span several sets becomes one launch per set, back to back on the stream.
 constexpr uint32_t fbit(int f) { return 1u << f; }
 constexpr uint32_t FSET_GGUF = fbit(FMT_Q8_0) | fbit(FMT_Q4_K), FSET_Q6K = fbit(FMT_Q6_K), FSET_MLX = fbit(FMT_Q4M),
-                   FSET_ALL = FSET_GGUF | FSET_Q6K | FSET_MLX | fbit(FMT_Q8F) | fbit(FMT_Q5_K) | fbit(FMT_Q40) | fbit(FMT_MXFP4);
+                   FSET_Q5K = fbit(FMT_Q5_K), FSET_Q40 = fbit(FMT_Q40), FSET_MX4 = fbit(FMT_MXFP4), FSET_Q8F = fbit(FMT_Q8F);
+// The sets in launch order: more instruction work per byte first, so that the call's tail is made of the lightest jobs.
+constexpr uint32_t FSETS[] = {FSET_Q6K, FSET_Q5K, FSET_Q40, FSET_MX4, FSET_MLX, FSET_GGUF, FSET_Q8F};
+constexpr int NSETS = sizeof(FSETS) / sizeof(FSETS[0]);
+inline int set_of(int fmt) {
+    for (int i = 0; i < NSETS; i++)
+        if (FSETS[i] & fbit(fmt)) return i;
+    return -1;
+}
 // (Q6_K alone: its step needs a dozen registers more than the 128 that workgroups of 16 waves leave a wave, and spilled them
-// around its loop; its shapes never exceed 8 waves, so its kernel is bounded at 512 threads and keeps them in registers)
+// around its loop; its shapes never exceed 8 waves, so its kernel is bounded at 512 threads and keeps them in registers;
+// Q4_0's likewise, for nine registers)
 template <uint32_t FSET>
-__global__ __launch_bounds__(FSET == (1u << FMT_Q6_K) ? 512 : 1024) void decode_batch_kernel(BatchArgs a) {
+__global__ __launch_bounds__(FSET == (1u << FMT_Q6_K) || FSET == (1u << FMT_Q40) ? 512 : 1024) void decode_batch_kernel(BatchArgs a) {
     extern __shared__ __align__(16) float lds_dyn[];
     uint32_t j = 0;
     while (j + 1 < a.njobs && blockIdx.x >= a.j[j + 1].wg0) j++;  // uniform
@@ -1215,7 +1225,7 @@ uint32_t steps_rt(const WeightView& w) {
 bool decode_pair_ok(const WeightView& w) {
     if (!mfma_decode_format(w.fmt)) return false;
     const Shape sh = pair_shape(shape_for(row_tiles(w.n_out), steps_rt(w), true, w.fmt));
-    return sh.rt * sh.kw <= (w.fmt == FMT_Q6_K ? 8u : 16u);
+    return sh.rt * sh.kw <= (w.fmt == FMT_Q6_K || w.fmt == FMT_Q40 ? 8u : 16u);  // (their shared-launch kernels are bounded at 8 waves)
 }
 
 bool decode_batchable(const WeightView& w, size_t t) {
@@ -1251,7 +1261,8 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     const uint64_t bit = 1ull << (dev & 63);
     if (!(allowed[(dev >> 6) & 3].load(std::memory_order_acquire) & bit)) {
         for (const void* k : {reinterpret_cast<const void*>(decode_batch_kernel<FSET_GGUF>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_MLX>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_Q6K>),
-                              reinterpret_cast<const void*>(decode_batch_kernel<FSET_ALL>)}) {
+                              reinterpret_cast<const void*>(decode_batch_kernel<FSET_Q5K>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_Q40>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_MX4>),
+                              reinterpret_cast<const void*>(decode_batch_kernel<FSET_Q8F>)}) {
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
             if (e != hipSuccess) return e;
         }
@@ -1260,9 +1271,23 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     std::vector<BatchArgs> launches;
     std::vector<size_t> ldss;
     std::vector<uint32_t> threadss;
-    for (size_t i0 = 0; i0 < n; i0 += BATCH_MAX) {
+    // the jobs by format set (the caller's order within a set), then launches of up to BATCH_MAX jobs of one set
+    std::vector<const DecodeBatchItem*> sorted;
+    std::vector<std::pair<size_t, size_t>> runs;  // [first, count) into `sorted`
+    sorted.reserve(n);
+    for (int set = 0; set < NSETS; set++) {
+        const size_t first = sorted.size();
+        for (size_t i = 0; i < n; i++) {
+            const int so = set_of(items[i].w.fmt);
+            if (so < 0) return hipErrorInvalidValue;
+            if (so == set) sorted.push_back(&items[i]);
+        }
+        for (size_t i0 = first; i0 < sorted.size(); i0 += BATCH_MAX) runs.emplace_back(i0, std::min(sorted.size() - i0, (size_t)BATCH_MAX));
+    }
+    for (const auto& run : runs) {
+        const DecodeBatchItem* const* items_of = sorted.data() + run.first;
         BatchArgs a{};
-        a.njobs = (uint32_t)(n - i0 < (size_t)BATCH_MAX ? n - i0 : (size_t)BATCH_MAX);
+        a.njobs = (uint32_t)run.second;
         size_t lds = 0, pf = 0, nc = 0;  // scratch is shared by the jobs of one launch, reused by the next launch
         uint32_t wg = 0, threads = 64;
         // Block order within the launch. Workgroups start in block order, so the last jobs make the tail of the launch,
@@ -1276,17 +1301,17 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
                 return shape_for(row_tiles(w.n_out), steps_rt(w), true, w.fmt).ks > 1;
             };
             int last = 0;
-            for (uint32_t j = 0; j < a.njobs; j++) last = std::max(last, cls(items[i0 + j].w.fmt));
+            for (uint32_t j = 0; j < a.njobs; j++) last = std::max(last, cls(items_of[j]->w.fmt));
             uint32_t key[BATCH_MAX];
             for (uint32_t j = 0; j < a.njobs; j++) {
-                const WeightView& w = items[i0 + j].w;
+                const WeightView& w = items_of[j]->w;
                 key[j] = 2 * cls(w.fmt) + (cls(w.fmt) == last && !sliced(w) ? 1 : 0);
                 order[j] = j;
             }
             std::stable_sort(order, order + a.njobs, [&](uint32_t x, uint32_t y) { return key[x] < key[y]; });
         }
         for (uint32_t j = 0; j < a.njobs; j++) {
-            const DecodeBatchItem& it = items[i0 + order[j]];
+            const DecodeBatchItem& it = *items_of[order[j]];
             const uint32_t ntiles = row_tiles(it.w.n_out), nsteps = steps_rt(it.w);
             const bool pair = it.epi.pair_p0 != nullptr;
             Shape sh = shape_for(ntiles, nsteps, true, it.w.fmt);
@@ -1328,6 +1353,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
         if (!launches[i].nwg) continue;
         uint32_t fset = 0;
         for (uint32_t j = 0; j < launches[i].njobs; j++) fset |= fbit(launches[i].j[j].w.fmt);
+        if (threadss[i] > ((fset == FSET_Q6K || fset == FSET_Q40) ? 512u : 1024u)) return hipErrorInvalidValue;  // (the kernels' launch bounds)
         auto go = [&](auto kern) {
             if (ride) hipExtLaunchKernelGGL(kern, dim3(launches[i].nwg), dim3(threadss[i]), (uint32_t)ldss[i], s, ev_start, ev_stop, 0, launches[i]);
             else kern<<<launches[i].nwg, threadss[i], ldss[i], s>>>(launches[i]);
@@ -1335,7 +1361,11 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
         if (!(fset & ~FSET_GGUF)) go(decode_batch_kernel<FSET_GGUF>);
         else if (!(fset & ~FSET_MLX)) go(decode_batch_kernel<FSET_MLX>);
         else if (!(fset & ~FSET_Q6K)) go(decode_batch_kernel<FSET_Q6K>);
-        else go(decode_batch_kernel<FSET_ALL>);
+        else if (!(fset & ~FSET_Q5K)) go(decode_batch_kernel<FSET_Q5K>);
+        else if (!(fset & ~FSET_Q40)) go(decode_batch_kernel<FSET_Q40>);
+        else if (!(fset & ~FSET_MX4)) go(decode_batch_kernel<FSET_MX4>);
+        else if (!(fset & ~FSET_Q8F)) go(decode_batch_kernel<FSET_Q8F>);
+        else return hipErrorInvalidValue;
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

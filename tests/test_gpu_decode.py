@@ -281,6 +281,32 @@ def test_fp8_dequant_and_decode(be, oxref):
         assert row_err(y[:, 1:], ref[:, 1:]) < TOL
 
 
+def test_fp8_decode_on_a_fresh_stream_takes_the_one_pass_kernel(be, oxref):
+    """A stream's decode scratch comes into being on first need, and FP8's one-pass decode kernel keeps its packed rows
+    there: the first FP8 decode on a new stream must bring the scratch with it (device memory in use grows) and give the
+    rows of the host surface's product, which runs the same kernel over the context's scratch, bit for bit. Without the
+    scratch the call would fall back to the plain kernel: right within tolerance, three times slower, other bits."""
+    import torch
+    from oxinfer_amd import synth
+    n_out, n_in, t = 512, 2048, 1
+    data, scales = synth.fp8_e4m3(n_out, n_in, 91)
+    w = be.upload_fp8(data, scales, n_out, n_in)
+    x = synth.activations(t, n_in, 92, bf16=True)
+    host = np.empty((t, n_out), np.float32)
+    assert be.matmul(x, t, n_in, [(w, host)]), be.last_error()
+    assert row_err(host, oxref.gemm_quant(oxref.F8E4M3, data, scales, None, n_out, n_in, x, t)) < TOL
+    xd = dev(x)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    with torch.cuda.stream(side):
+        y = be.decode(w, x=xd)
+    side.synchronize()
+    assert torch.cuda.mem_get_info()[0] <= free0 - (8 << 20), "the stream's decode scratch was not allocated"
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), host.view(np.uint32))
+    assert be.stream_release(side.cuda_stream)
+
+
 def test_fp8_rows_scale_blocks(oxref, be):
     """Scale rows change every 128 weight rows; the row-1 dequant check above would miss a wrong row index."""
     from oxinfer_amd import synth
