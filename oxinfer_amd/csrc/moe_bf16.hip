@@ -66,24 +66,38 @@ __global__ __launch_bounds__(256) void moe_pack_bf16_kernel(const float* __restr
     out[(((size_t)c * nsteps + s) * 4 + b) * 64 + lane] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
 }
 
+// Which (run of row tiles gx, chunk c) a workgroup of the one-dimensional grid takes. Workgroups go to the 8 XCDs in turn
+// (linear id mod 8), and each XCD has an L2 of its own; an expert with more than 16 routed rows has several chunks, each
+// of which streams the expert's rows again. Items are numbered (gx, c) with c fastest, so that the chunks of one expert
+// are neighbours, and XCD k takes the k-th eighth of them in order: workgroups that read the same weights start
+// together on the same XCD, and all but the first find them in its L2 instead of asking HBM again. False: no item.
+__device__ __forceinline__ bool moe_bf16_item(uint32_t nx, uint32_t nch, uint32_t* gx, uint32_t* c) {
+    const uint32_t total = nx * nch, per = (total + 7) >> 3;
+    const uint32_t xcd = blockIdx.x & 7, q = blockIdx.x >> 3, v = xcd * per + q;
+    if (q >= per || v >= total) return false;
+    *gx = v / nch;
+    *c = v - *gx * nch;
+    return true;
+}
+
 // Workgroup: 8 waves = 8 / kw groups of RT row tiles x kw waves that split the K steps (wave v takes steps v, v + kw, ...)
-// and meet in LDS in wave order. grid x: runs of (8 / kw) RT row tiles; grid y: chunks {expert, first row, rows <= 16}.
+// and meet in LDS in wave order. A workgroup's item (moe_bf16_item): a run of (8 / kw) RT row tiles of a chunk {expert, first row, rows <= 16}.
 // The chunk's fragments (4 KiB per step) are staged into LDS once per workgroup: all eight waves multiply the same
 // rows (each wave asking memory for them costs more than the weights). out [gathered row][n_out] f32.
 template <int RT, int FMT>
 __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const uint8_t* const* __restrict__ bases, const int4* __restrict__ chunks,
-                                                          const int* __restrict__ nchunks, const uint4* __restrict__ afrag, uint32_t kw,
+                                                          const int* __restrict__ nchunks, const uint4* __restrict__ afrag, uint32_t kw, uint32_t nx,
                                                           float* __restrict__ out) {
     extern __shared__ __align__(16) float lds[];  // fragments [step][4][64] x 16 B; then the waves' sums [wave][RT][64][4]
-    const uint32_t c = blockIdx.y;
-    if (c >= (uint32_t)*nchunks) return;  // uniform over the workgroup
+    uint32_t gx, c;
+    if (!moe_bf16_item(nx, (uint32_t)*nchunks, &gx, &c)) return;  // uniform over the workgroup
     const int4 ch = chunks[c];
     const uint32_t first = (uint32_t)ch.y, rows = (uint32_t)ch.z;
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t n = lane & 15;
     const uint32_t nsteps = w.n_in / 128, ntiles = row_tiles(w.n_out);
     const uint32_t ng = 8 / kw, rg = wave / kw, kwave = wave % kw;
-    const uint32_t tile0 = (blockIdx.x * ng + rg) * RT;
+    const uint32_t tile0 = (gx * ng + rg) * RT;
     const gbytes base = as_global(bases[ch.x]);
     gbytes wp[RT];
     constexpr uint32_t REC = FMT == FMT_MXFP4 ? T4X_REC : T4M_REC;
@@ -218,7 +232,7 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
     // D[token 4 kq + i][row n]: thread (group, r, lane) adds the group's waves in order and stores its four tokens
     for (uint32_t idx = threadIdx.x; idx < ng * RT * 64; idx += blockDim.x) {
         const uint32_t l = idx & 63, r = (idx >> 6) % RT, g = (idx >> 6) / RT;
-        const uint32_t tile = (blockIdx.x * ng + g) * RT + r, row = tile * 16 + (l & 15);
+        const uint32_t tile = (gx * ng + g) * RT + r, row = tile * 16 + (l & 15);
         if (tile >= ntiles || row >= w.n_out) continue;
         f32x4 sum = *reinterpret_cast<const f32x4*>(red + (((size_t)(g * kw) * RT + r) * 64 + l) * 4);
         for (uint32_t k = 1; k < kw; k++) {
@@ -243,20 +257,20 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
 // Every product and sum is exact up to the f32 rounding of the matrix cores' accumulation.
 template <int RT, int FMT>
 __global__ __launch_bounds__(512, 4) void moe_bf16_std_kernel(WeightView w, const uint8_t* const* __restrict__ bases, const int4* __restrict__ chunks,
-                                                              const int* __restrict__ nchunks, const uint4* __restrict__ afrag, uint32_t kw,
+                                                              const int* __restrict__ nchunks, const uint4* __restrict__ afrag, uint32_t kw, uint32_t nx,
                                                               float* __restrict__ out) {
     static_assert(FMT == FMT_Q8_0 || FMT == FMT_Q4_K, "the formats whose records hold consecutive columns per lane");
     constexpr bool Q8 = FMT == FMT_Q8_0;
     extern __shared__ __align__(16) float lds[];  // fragments [step][4][64] x 16 B; then the waves' sums [wave][RT][64][4]
-    const uint32_t c = blockIdx.y;
-    if (c >= (uint32_t)*nchunks) return;  // uniform over the workgroup
+    uint32_t gx, c;
+    if (!moe_bf16_item(nx, (uint32_t)*nchunks, &gx, &c)) return;  // uniform over the workgroup
     const int4 ch = chunks[c];
     const uint32_t first = (uint32_t)ch.y, rows = (uint32_t)ch.z;
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t n = lane & 15, kq = lane >> 4;
     const uint32_t nsteps = w.n_in / 128, ntiles = row_tiles(w.n_out);
     const uint32_t ng = 8 / kw, rg = wave / kw, kwave = wave % kw;
-    const uint32_t tile0 = (blockIdx.x * ng + rg) * RT;
+    const uint32_t tile0 = (gx * ng + rg) * RT;
     const gbytes base = as_global(bases[ch.x]);
     gbytes wp[RT];
 #pragma unroll
@@ -374,7 +388,7 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_std_kernel(WeightView w, cons
     __syncthreads();
     for (uint32_t idx = threadIdx.x; idx < ng * RT * 64; idx += blockDim.x) {
         const uint32_t l = idx & 63, r = (idx >> 6) % RT, g = (idx >> 6) / RT;
-        const uint32_t tile = (blockIdx.x * ng + g) * RT + r, row = tile * 16 + (l & 15);
+        const uint32_t tile = (gx * ng + g) * RT + r, row = tile * 16 + (l & 15);
         if (tile >= ntiles || row >= w.n_out) continue;
         f32x4 sum = *reinterpret_cast<const f32x4*>(red + (((size_t)(g * kw) * RT + r) * 64 + l) * 4);
         for (uint32_t k = 1; k < kw; k++) {
@@ -440,11 +454,12 @@ hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max
 #endif
     const uint32_t ng = 8 / kw;
     const size_t red = (size_t)8 * rt * 64 * 16, fr = (size_t)nsteps * 4096, lds = fr > red ? fr : red;
-    const dim3 grid((ntiles + ng * rt - 1) / (ng * rt), max_chunks);
+    const uint32_t nx = (ntiles + ng * rt - 1) / (ng * rt);
+    const dim3 grid((nx * max_chunks + 7) / 8 * 8);  // every XCD's share of the items (moe_bf16_item), whatever the chunk count turns out to be
     hipError_t e = hipSuccess;
     auto go = [&](auto kern) {
         if (lds > 48 * 1024) e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e == hipSuccess) kern<<<grid, 512, lds, s>>>(w, g.bases, g.chunks, g.nchunks, static_cast<const uint4*>(frag), kw, out);
+        if (e == hipSuccess) kern<<<grid, 512, lds, s>>>(w, g.bases, g.chunks, g.nchunks, static_cast<const uint4*>(frag), kw, nx, out);
     };
     if (w.fmt == FMT_Q8_0) go(moe_bf16_std_kernel<2, FMT_Q8_0>);
     else if (w.fmt == FMT_Q4_K) rt == 2 ? go(moe_bf16_std_kernel<2, FMT_Q4_K>) : go(moe_bf16_std_kernel<4, FMT_Q4_K>);
