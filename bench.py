@@ -372,6 +372,28 @@ def bench_gguf_gemm(be, torch, synth, steps, warmup, fmt):
                           "flops_per_launch": flops / 2, "avg_launch_us": round(ms * 1e3, 2), "call_us": round(step_ms * 1e3 / 2, 2)})
 
 
+def bench_gguf_layer(be, torch, synth, steps, warmup, t, gens):
+    """Beyond BASELINE.json's configurations: the seven matmuls of one Llama-8B layer as a Q4_K_M file stores them
+    (Q4_K q, k, o, gate, up; Q6_K v, down) handed over as one oxhip_dev_decode_batch call: the library issues one launch
+    per format set, back to back. Weights rotate over copies larger than the Infinity Cache."""
+    spec = [(Q4_K, 4096, 4096), (Q4_K, 1024, 4096), (Q6_K, 1024, 4096), (Q4_K, 4096, 4096), (Q4_K, 14336, 4096), (Q4_K, 14336, 4096),
+            (Q6_K, 4096, 14336)]
+    nbytes = sum(algorithmic_bytes(k, n, kk, t) for k, n, kk in spec)
+    copies = max(2, int(np.ceil(0.6e9 / nbytes)))
+    ws = [[be.upload_gguf(k, gens[k](n, kk, 11 + j), n, kk) for j, (k, n, kk) in enumerate(spec)] for _ in range(copies)]
+    xa = {kk: be.quantize_act(torch.from_numpy(synth.activations(t, kk, 3)).cuda()) for kk in (4096, 14336)}
+    ys = [torch.empty((t, n), dtype=torch.float32, device="cuda") for _, n, _ in spec]
+    arrs = [be.decode_jobs([(ws[c][j], xa[spec[j][2]], None, t, ys[j], None, None) for j in range(len(spec))]) for c in range(copies)]
+    wall, ms = timed_steps(torch, lambda i: be.decode_batch(arrs[i % copies]), steps, warmup)
+    ach = nbytes / (ms * 1e-3) / 1e9
+    return dict(base_line(steps, warmup), value=round(nbytes * steps / wall / 1e9, 2), unit="GB/s", ms_per_step=round(wall / steps * 1e3, 5), dtype="int8",
+                config={"workload": f"a Q4_K_M layer's seven matmuls (Q4_K q, k, o, gate, up; Q6_K v, down; Llama-8B shapes) in one batch call, T = {t}",
+                        "bytes_per_step": nbytes, "events": "around the call (two launches: the Q6_K jobs, then the Q4_K jobs)"},
+                roofline={"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+                          "traffic": None, "kernel": "decode_batch_kernel<Q6_K> + decode_batch_kernel<Q8_0 | Q4_K>", "bytes_per_launch": nbytes,
+                          "avg_launch_us": round(ms * 1e3, 2)})
+
+
 def moe_experts(synth):
     ne, h, inter = 128, 2048, 768
     return ([synth.mlx_q4(2 * inter, h, 100 + e) for e in range(ne)], [synth.mlx_q4(h, inter, 300 + e) for e in range(ne)])
@@ -636,7 +658,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="all", choices=["all", "gguf_gemv", "gguf_gemv_q6k", "gguf_stream", "gguf_gemm", "mlx_gemv", "mlx_gemm", "moe", "fp8", "copy"],
+    ap.add_argument("--workload", default="all", choices=["all", "gguf_gemv", "gguf_gemv_q6k", "gguf_stream", "gguf_gemm", "gguf_layer", "mlx_gemv", "mlx_gemm", "moe", "fp8", "copy"],
                     help="all (default) = the headline configs[1] line with every other configuration in per_config; gguf_gemv = the headline alone; "
                          "copy = a plain 256 MiB device copy, the known-size kernel that scales the HBM traffic counters; "
                          "gguf_stream = every GGUF case alone as a steady stream of 192 matmuls handed over in one call")
@@ -684,6 +706,8 @@ def main():
             line["cpu_baseline"] = cpu_mlx_gemm()
     elif w == "gguf_gemm":
         line = bench_gguf_gemm(be, torch, synth, args.steps, args.warmup, args.format)
+    elif w == "gguf_layer":
+        line = bench_gguf_layer(be, torch, synth, args.steps, args.warmup, args.tokens or 1, gens)
     elif w == "moe":
         ex = moe_experts(synth)
         line = bench_moe(be, torch, synth, args.steps, args.warmup, args.pool_gb, args.tokens or 1, ex, args.moe_int8)
@@ -716,6 +740,8 @@ def main():
             for m in (1, 32, 1024):
                 per[f"configs[4] FP8 M={m}"] = summary(bench_fp8(be, torch, synth, ks, kw, args.pool_gb, m, "bf16", wts), cpu_fp8(m, *wts) if cpu else None)
             per["configs[4] FP8 M=1024 fp8 MFMA"] = summary(bench_fp8(be, torch, synth, ks, kw, args.pool_gb, 1024, "fp8", wts), per["configs[4] FP8 M=1024"]["cpu_baseline"])
+            for t in (1, 8):
+                per[f"beyond configs: Q4_K_M layer (Q4_K + Q6_K jobs in one call) T={t}"] = summary(bench_gguf_layer(be, torch, synth, ks, kw, t, gens), None)
             line["per_config"] = per
     print(json.dumps(line))
     be.close()

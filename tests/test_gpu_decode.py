@@ -512,11 +512,14 @@ def test_decode_batch_shares_a_launch_and_keeps_the_bits(be, oxref):
     cases = [(Q8_0, 208, 512, 1), (Q4_K, 96, 1024, 8), (Q8_0, 64, 2048, 3), (Q4_K, 176, 512, 2), ("mlx", 80, 640, 5),
              (Q6_K, 48, 512, 2), (Q4_K, 33, 256, 4), ("mlx", 128, 128, 8),
              (Q8_0, 48, 14336, 8), (Q4_K, 32, 14336, 1), (Q6_K, 16, 14336, 5),  # these three slice K across workgroups
-             (Q5_K, 72, 768, 7), (Q5_K, 40, 14336, 1), (MXFP4, 56, 1120, 6)]
+             (Q5_K, 72, 768, 7), (Q5_K, 40, 14336, 1), (MXFP4, 56, 1120, 6),
+             (Q4_0, 48, 1056, 8), (Q4_0, 24, 14336, 2), ("q8", 88, 608, 3), ("q8", 16, 14336, 8)]
     jobs, alone = [], []
     for i, (kind, n_out, n_in, t) in enumerate(cases):
         if kind == "mlx":
             w = be.upload_mlx_q4(*synth.mlx_q4(n_out, n_in, 70 + i), 64, n_out, n_in)
+        elif kind == "q8":
+            w = be.upload_q8(*synth.q8_matrix(n_out, n_in, 70 + i), n_out, n_in)
         else:
             raw, _ = oxref.random_blocks(kind, n_out * n_in // oxref.block_size(kind), 80 + i)
             w = be.upload_gguf(kind, raw, n_out, n_in)
@@ -525,7 +528,8 @@ def test_decode_batch_shares_a_launch_and_keeps_the_bits(be, oxref):
         alone.append(be.decode(w, xa=xa).cpu().numpy())
         y = torch.full((t, n_out), float("nan"), dtype=torch.float32, device="cuda")
         jobs.append((w, xa, None, t, y, None, None))
-    for order in (list(range(len(cases))), list(reversed(range(len(cases)))), [1, 3, 6], [4], [8, 0, 9, 10, 2], [11, 5, 12], [13, 4], [13]):
+    for order in (list(range(len(cases))), list(reversed(range(len(cases)))), [1, 3, 6], [4], [8, 0, 9, 10, 2], [11, 5, 12], [13, 4], [13],
+                  [14, 16, 15, 17], [15], [17, 0]):  # (every format set on its own and beside others)
         for i in order:
             jobs[i][4].fill_(float("nan"))
         be.decode_batch(be.decode_jobs([jobs[i] for i in order]))
