@@ -131,16 +131,27 @@ struct Step<FMT_Q6_K> {
 // {expert, first row, rows (<= 8 NG)}; the weights are expert's, activation row i of the chunk is row
 // rowmap[first + i] of xa (or first + i without a map), and its output is row first + i of y.
 // ALDS: the int8 activations are staged into LDS in operand order (the launcher checks that they fit).
-// `bx`, `by`: the workgroup's place in its launch unit (row group; K slice or chunk); `nthr` = 64 rt kw threads take
+// `bx`, `by`: the workgroup's place in its launch unit (row group; K slice or chunk); `nthr` threads take
 // part (a launch may hold more: those waves have left before the first barrier); `lds_all`: the dynamic LDS.
+// `kw` and `ksplit` say how a row's sum is associated: K is cut into ksplit slices of kw runs each, a run is summed
+// step by step, a slice's runs are added in order, and the slices in order. Who sums a run is a separate matter
+// (Mapping): in the plain mapping a wave has one run and a workgroup one slice (64 rt kw threads); a dense launch may
+// instead give a workgroup `fs` consecutive slices and a tile `kwp` waves, each of which then streams fs kw / kwp
+// consecutive runs in one go, leaving every run's sums apart. The bits are the same; the workgroups are fewer and fatter.
 // NG (grouped launches of 8 tokens per group): a chunk holds up to 8 NG rows; every weight record is used for NG
 // instructions, one per group of 8 tokens, before the next is touched.
-template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS, int NG = 1>
+struct Mapping {
+    uint32_t kwp = 0;  // waves per tile (0: kw, one run per wave)
+    uint32_t fs = 0;   // K slices per workgroup (0: one)
+};
+
+template <int FMT, int NT, bool DUMP, bool GROUPED, bool ALDS, int NG = 1, bool REMAP = false>
 __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t t, uint32_t rt, uint32_t kw, float* __restrict__ y,
                                             int32_t* __restrict__ dump, GroupView grp, uint32_t ksplit, float* __restrict__ partial,
                                             uint32_t* __restrict__ counters, uint32_t bx, uint32_t by, uint32_t nthr,
-                                            float* __restrict__ lds_all, Epi epi = Epi{}) {
+                                            float* __restrict__ lds_all, Epi epi = Epi{}, Mapping map = Mapping{}) {
     static_assert(NG == 1 || (GROUPED && ALDS && !DUMP && NT == 8), "token groups are for grouped launches");
+    static_assert(!REMAP || (!GROUPED && !DUMP && ALDS && NG == 1), "other mappings are for dense launches over staged activations");
     constexpr int TPAD = NT <= 4 ? 4 : 8;
     // the swizzled operand array pays at 8 tokens (where the staging stores are many); at fewer its address math costs more
     constexpr bool SWZ = NT >= 8;
@@ -155,7 +166,11 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // kw and the number of K slices are powers of two (the launchers see to it): shifts, where a division by a value only
     // known at run time costs some twenty instructions even when it is the same for the whole wave
     const uint32_t kwsh = (uint32_t)__builtin_ctz(kw), kssh = (uint32_t)__builtin_ctz(ksplit);
-    const uint32_t r = wave >> kwsh, ks = wave & (kw - 1);
+    // the mapping: kwp waves per tile and fs slices per workgroup (both powers of two); runs of a tile in the workgroup, runs
+    // per wave. Launchers only leave the plain mapping when every run has the same number of steps.
+    const uint32_t kwp = REMAP && map.kwp ? map.kwp : kw, fs = REMAP && map.fs ? map.fs : 1u;
+    const uint32_t runs = fs << kwsh, rpw = runs >> __builtin_ctz(kwp);
+    const uint32_t r = wave >> __builtin_ctz(kwp), kj = wave & (kwp - 1);
     // (fused gate / up experts: the first rt / 2 tiles of the workgroup are gate tiles, the others the up tiles of the same rows;
     // a gate / up pair of two matrices likewise: the first rt / 2 waves' tiles come from `w`, the others' from epi.pair_p0)
     const bool glu = GROUPED && grp.glu_inter != 0;
@@ -174,14 +189,14 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
                                               : t4m_steps(w.n_in);
     const uint32_t slice = GROUPED ? 0 : by;
     const uint32_t sl = (nsteps + ksplit - 1) >> kssh;
-    const uint32_t S0 = min(nsteps, slice * sl), S1 = min(nsteps, S0 + sl);
-    const uint32_t B0 = BPS * S0, nbl = BPS * sl, M0 = B0 / 2;
+    const uint32_t S0 = min(nsteps, slice * fs * sl), S1 = min(nsteps, S0 + fs * sl);  // (the workgroup's fs slices)
+    const uint32_t B0 = BPS * S0, nbl = BPS * fs * sl, M0 = B0 / 2;
     // LDS: [operand-order activations: 512 B per pair of blocks] [scales, sums] [partial sums]; with ALDS the
     // partial sums reuse the activations' space once every wave is done with them
     uint2* afr = reinterpret_cast<uint2*>(lds_all);  // [NG][nbl / 2][64]
     float* lds = lds_all + (ALDS ? (size_t)NG * (nbl / 2) * 128 : 0);
     const uint32_t nm = nbl * TPAD, as = NG * nm;  // scale entries of a token group; floats per array
-    float* red = ALDS ? lds_all : lds + (size_t)NARR * as;  // [rt * kw][NG][TPAD][16]
+    float* red = ALDS ? lds_all : lds + (size_t)NARR * as;  // [rt][runs][NG][TPAD][16]
     uint32_t row0 = 0;  // first activation / output row of this launch unit
     if (GROUPED) {
         if (grp.direct) {
@@ -212,9 +227,9 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // Q4_K: the bytes this lane takes from a step's {scales, mins} words (v_perm_b32: 0..3 = the scales, 4..7 = the mins)
     const uint32_t q4k_sel = d_half | ((2 + d_half) << 8) | (kq << 16) | ((4 + kq) << 24);
 
-    const uint32_t per = (S1 - S0 + kw - 1) >> kwsh;
-    const uint32_t s0 = S0 + ks * per;
-    const uint32_t s1 = tile < ntiles ? min(S1, s0 + per) : 0;  // a tile past the matrix streams nothing
+    const uint32_t per = fs == 1 && rpw == 1 ? (S1 - S0 + kw - 1) >> kwsh : sl >> kwsh;  // steps of a run
+    const uint32_t s0 = S0 + kj * rpw * per;
+    const uint32_t s1 = tile < ntiles ? min(S1, s0 + rpw * per) : 0;  // a tile past the matrix streams nothing
     // (typed as global memory: a grouped launch reads w.p0 from the table of expert bases)
     const gbytes base = as_global(pair && r >= ghalf ? epi.pair_p0 : w.p0) + (size_t)min(tile, ntiles - 1) * (FMT == FMT_Q8_0   ? (size_t)nsteps * T8_REC
                                                                   : FMT == FMT_Q8F  ? (size_t)nsteps * T8F_REC
@@ -642,6 +657,64 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // under a condition: the compiler counts the requests in flight to place its waits, and where a path may or may not
     // have issued one it waits for (nearly) all of them, which empties the ring at every step. So a generation that has
     // a successor refills every slot (past the wave's last step: with that step again, a hit), and the last one none.
+    // The end of a run: its sums as a wave of its own leaves them ...
+    auto close_run = [&]() {
+        if constexpr (FMT == FMT_Q6_K) {
+            // the four sub-blocks of a token meet across the lane groups; group 0 then holds tokens 0..3, group 1 tokens 4..7
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float a = acc6a[i], b = acc6b[i];
+                a += __shfl_xor(a, 16);
+                a += __shfl_xor(a, 32);
+                b += __shfl_xor(b, 16);
+                b += __shfl_xor(b, 32);
+                acc[0][i] = (kq & 1) ? b : a;
+            }
+        } else {
+            if constexpr (MINS) {
+#pragma unroll
+                for (int g = 0; g < NG; g++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc[g][i] += macc[g][i];
+            }
+            // the two block parities of a token meet across lane groups kq and kq ^ 2
+#pragma unroll
+            for (int g = 0; g < NG; g++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[g][i] += __shfl_xor(acc[g][i], 32);
+        }
+    };
+    // ... go to the run's place among its tile's partial sums ...
+    auto store_run = [&](uint32_t run) {
+        if (kq < 2) {
+#pragma unroll
+            for (int g = 0; g < NG; g++)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (d_tok0 + i < (uint32_t)TPAD) red[((((size_t)r * runs + run) * NG + g) * TPAD + d_tok0 + i) * 16 + n] = acc[g][i];
+        }
+    };
+    // A wave with further runs (up to MAXRUNS in all) keeps the closed run's sums in registers (the partial sums' place in
+    // LDS still holds the activations) and starts the next run from zero. `left`: steps to the end of the run in hand.
+    constexpr int MAXRUNS = 4;
+    float held[REMAP ? MAXRUNS - 1 : 1][4] = {};
+    uint32_t nrun = 0, left = per;  // runs closed so far
+    auto step_done = [&]() {
+        if constexpr (REMAP) {
+            if (rpw > 1 && --left == 0 && nrun + 1 < rpw) {  // uniform over the wave
+                close_run();
+#pragma unroll
+                for (int h = 0; h < MAXRUNS - 1; h++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) held[h][i] = nrun == (uint32_t)h ? acc[0][i] : held[h][i];
+                nrun++;
+                left = per;
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[0][i] = acc6a[i] = acc6b[i] = 0.0f;
+                macc[0] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        }
+    };
     uint32_t sb = s0;
     for (; sb + PF < s1; sb += PF) {
 #pragma unroll
@@ -655,6 +728,7 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             scales_of(scur, p % 4, sw);
             compute_step(ring[p], sw, sb + p);
             load_step(ring[p], min(sb + PF + p, slast));
+            step_done();
         }
     }
 #pragma unroll
@@ -667,40 +741,23 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
             uint32_t sw[NM];
             scales_of(scur, p % 4, sw);
             compute_step(ring[p], sw, sb + p);
+            step_done();
         }
     }
-    if constexpr (FMT == FMT_Q6_K) {
-        // the four sub-blocks of a token meet across the lane groups; group 0 then holds tokens 0..3, group 1 tokens 4..7
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            float a = acc6a[i], b = acc6b[i];
-            a += __shfl_xor(a, 16);
-            a += __shfl_xor(a, 32);
-            b += __shfl_xor(b, 16);
-            b += __shfl_xor(b, 32);
-            acc[0][i] = (kq & 1) ? b : a;
-        }
-    } else {
-        if constexpr (MINS) {
-#pragma unroll
-            for (int g = 0; g < NG; g++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) acc[g][i] += macc[g][i];
-        }
-        // the two block parities of a token meet across lane groups kq and kq ^ 2
-#pragma unroll
-        for (int g = 0; g < NG; g++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) acc[g][i] += __shfl_xor(acc[g][i], 32);
-    }
+    close_run();
     if (ALDS) __syncthreads();  // the partial sums overwrite the staged activations
-    if (kq < 2) {
+    if constexpr (REMAP) {
+        if (rpw > 1 && kq < 2) {  // the runs closed on the way
 #pragma unroll
-        for (int g = 0; g < NG; g++)
+            for (int h = 0; h < MAXRUNS - 1; h++)
+                if ((uint32_t)h < rpw - 1) {
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                if (d_tok0 + i < (uint32_t)TPAD) red[(((size_t)wave * NG + g) * TPAD + d_tok0 + i) * 16 + n] = acc[g][i];
+                    for (int i = 0; i < 4; i++)
+                        if (d_tok0 + i < (uint32_t)TPAD) red[(((size_t)r * runs + kj * rpw + h) * TPAD + d_tok0 + i) * 16 + n] = held[h][i];
+                }
+        }
     }
+    store_run(kj * rpw + rpw - 1);
     __syncthreads();
     // how a finished sum goes out (uniform branches)
     auto emit = [&](float* dst, float v, uint32_t tok) {
@@ -795,16 +852,18 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // the waves of a tile in order; with one slice that is the result, else this slice's partial rows (a pair's partial rows are
     // 2 n_out wide: the first matrix's, then the second's)
     const uint32_t prow = pair ? 2 * w.n_out : w.n_out;
-    float* out = ksplit > 1 ? partial + (size_t)slice * t * prow : y;
-    for (uint32_t idx = threadIdx.x; idx < rt * NG * TPAD * 16; idx += nthr) {
-        const uint32_t rr = idx / (NG * TPAD * 16), g = (idx / (TPAD * 16)) % NG, tok = 8 * g + (idx / 16) % TPAD, nn = idx % 16;
-        const uint32_t row = pair ? (bx * ghalf + (rr < ghalf ? rr : rr - ghalf)) * 16 + nn : (bx * rt + rr) * 16 + nn;
-        if (tok >= t || row >= w.n_out || !y) continue;
-        float sum = 0.0f;
-        for (uint32_t k = 0; k < kw; k++) sum += red[((((size_t)rr * kw + k) * NG + g) * TPAD + (idx / 16) % TPAD) * 16 + nn];
-        // partial rows go out as device-scope stores (written through to memory, where the other XCDs' L2s see them)
-        if (ksplit > 1 || combine) __hip_atomic_store(out + (size_t)tok * prow + (pair && rr >= ghalf ? w.n_out : 0u) + row, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        else emit(out + (size_t)tok * w.n_out + row, sum, tok);
+    for (uint32_t zl = 0; zl < fs; zl++) {  // the workgroup's slices, each with a partial row of its own
+        float* out = ksplit > 1 ? partial + (size_t)(slice * fs + zl) * t * prow : y;
+        for (uint32_t idx = threadIdx.x; idx < rt * NG * TPAD * 16; idx += nthr) {
+            const uint32_t rr = idx / (NG * TPAD * 16), g = (idx / (TPAD * 16)) % NG, tok = 8 * g + (idx / 16) % TPAD, nn = idx % 16;
+            const uint32_t row = pair ? (bx * ghalf + (rr < ghalf ? rr : rr - ghalf)) * 16 + nn : (bx * rt + rr) * 16 + nn;
+            if (tok >= t || row >= w.n_out || !y) continue;
+            float sum = 0.0f;
+            for (uint32_t k = 0; k < kw; k++) sum += red[((((size_t)rr * runs + (zl << kwsh) + k) * NG + g) * TPAD + (idx / 16) % TPAD) * 16 + nn];
+            // partial rows go out as device-scope stores (written through to memory, where the other XCDs' L2s see them)
+            if (ksplit > 1 || combine) __hip_atomic_store(out + (size_t)tok * prow + (pair && rr >= ghalf ? w.n_out : 0u) + row, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else emit(out + (size_t)tok * w.n_out + row, sum, tok);
+        }
     }
     if constexpr (GROUPED) {
         if (!combine) return;
@@ -853,8 +912,9 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     __syncthreads();
     if (threadIdx.x == 0) {
         const uint32_t seen = __hip_atomic_fetch_add(&counters[(size_t)bx * CTR_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = seen == ksplit - 1;
-        if (seen == ksplit - 1) __hip_atomic_store(&counters[(size_t)bx * CTR_STRIDE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t arrivals = ksplit >> __builtin_ctz(fs);  // workgroups of this row group
+        is_last = seen == arrivals - 1;
+        if (seen == arrivals - 1) __hip_atomic_store(&counters[(size_t)bx * CTR_STRIDE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!is_last) return;
@@ -911,6 +971,7 @@ struct BatchJob {
     float* partial;      // this job's share of the scratch (K slices across workgroups)
     uint32_t* counters;
     uint32_t t, rt, kw, ks, wg0;
+    Mapping map;  // (ks / fs slices across workgroups, 64 rt kwp threads)
     Epi epi;
 };
 struct BatchArgs {
@@ -918,17 +979,18 @@ struct BatchArgs {
     BatchJob j[BATCH_MAX];
 };
 
-template <int FMT>
+template <int FMT, bool FAT>
 __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid, float* lds) {
-    const uint32_t nthr = 64 * jb.rt * jb.kw;
+    const uint32_t nthr = 64 * jb.rt * jb.map.kwp;
     if (threadIdx.x >= nthr) return;  // whole waves (nthr is a multiple of 64), before any barrier
     const GroupView none{};
-    const uint32_t bx = bid >> __builtin_ctz(jb.ks), by = bid & (jb.ks - 1);  // the slices of a row group are neighbours in launch order (ks: a power of two)
-    if (jb.t == 1) decode_body<FMT, 1, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi);
-    else if (jb.t == 2 && !t4m_format(FMT)) decode_body<FMT, 2, false, false, true>(  // (MLX at 2 tokens: the 4-token body, which fits the registers)
-        jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi);
-    else if (jb.t <= 4) decode_body<FMT, 4, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi);
-    else decode_body<FMT, 8, false, false, true>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi);
+    const uint32_t ksp = jb.ks >> __builtin_ctz(jb.map.fs);  // slices across workgroups
+    const uint32_t bx = bid >> __builtin_ctz(ksp), by = bid & (ksp - 1);  // the slices of a row group are neighbours in launch order (a power of two)
+    if (jb.t == 1) decode_body<FMT, 1, false, false, true, 1, FAT>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi, jb.map);
+    else if (jb.t == 2 && !t4m_format(FMT)) decode_body<FMT, 2, false, false, true, 1, FAT>(  // (MLX at 2 tokens: the 4-token body, which fits the registers)
+        jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi, jb.map);
+    else if (jb.t <= 4) decode_body<FMT, 4, false, false, true, 1, FAT>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi, jb.map);
+    else decode_body<FMT, 8, false, false, true, 1, FAT>(jb.w, jb.xa, jb.t, jb.rt, jb.kw, jb.y, nullptr, none, jb.ks, jb.partial, jb.counters, bx, by, nthr, lds, jb.epi, jb.map);
 }
 
 // FSET: the formats compiled in, one bit per Fmt. The compiler allocates registers over the whole kernel, so every
@@ -949,7 +1011,8 @@ inline int set_of(int fmt) {
 // (Q6_K alone: its step needs a dozen registers more than the 128 that workgroups of 16 waves leave a wave, and spilled them
 // around its loop; its shapes never exceed 8 waves, so its kernel is bounded at 512 threads and keeps them in registers;
 // Q4_0's likewise, for nine registers)
-template <uint32_t FSET>
+// FAT: the launch's jobs use the fat mapping (see place_job); the plain kernels do without its bookkeeping.
+template <uint32_t FSET, bool FAT>
 __global__ __launch_bounds__(FSET == (1u << FMT_Q6_K) || FSET == (1u << FMT_Q40) ? 512 : 1024) void decode_batch_kernel(BatchArgs a) {
     extern __shared__ __align__(16) float lds_dyn[];
     uint32_t j = 0;
@@ -957,14 +1020,14 @@ __global__ __launch_bounds__(FSET == (1u << FMT_Q6_K) || FSET == (1u << FMT_Q40)
     const BatchJob& jb = a.j[j];
     const uint32_t bx = blockIdx.x - jb.wg0;
     switch (jb.w.fmt) {
-        case FMT_Q8_0: if constexpr (FSET & fbit(FMT_Q8_0)) batch_dispatch<FMT_Q8_0>(jb, bx, lds_dyn); break;
-        case FMT_Q8F: if constexpr (FSET & fbit(FMT_Q8F)) batch_dispatch<FMT_Q8F>(jb, bx, lds_dyn); break;
-        case FMT_Q4_K: if constexpr (FSET & fbit(FMT_Q4_K)) batch_dispatch<FMT_Q4_K>(jb, bx, lds_dyn); break;
-        case FMT_Q5_K: if constexpr (FSET & fbit(FMT_Q5_K)) batch_dispatch<FMT_Q5_K>(jb, bx, lds_dyn); break;
-        case FMT_Q6_K: if constexpr (FSET & fbit(FMT_Q6_K)) batch_dispatch<FMT_Q6_K>(jb, bx, lds_dyn); break;
-        case FMT_Q4M: if constexpr (FSET & fbit(FMT_Q4M)) batch_dispatch<FMT_Q4M>(jb, bx, lds_dyn); break;
-        case FMT_Q40: if constexpr (FSET & fbit(FMT_Q40)) batch_dispatch<FMT_Q40>(jb, bx, lds_dyn); break;
-        case FMT_MXFP4: if constexpr (FSET & fbit(FMT_MXFP4)) batch_dispatch<FMT_MXFP4>(jb, bx, lds_dyn); break;
+        case FMT_Q8_0: if constexpr (FSET & fbit(FMT_Q8_0)) batch_dispatch<FMT_Q8_0, FAT>(jb, bx, lds_dyn); break;
+        case FMT_Q8F: if constexpr (FSET & fbit(FMT_Q8F)) batch_dispatch<FMT_Q8F, FAT>(jb, bx, lds_dyn); break;
+        case FMT_Q4_K: if constexpr (FSET & fbit(FMT_Q4_K)) batch_dispatch<FMT_Q4_K, FAT>(jb, bx, lds_dyn); break;
+        case FMT_Q5_K: if constexpr (FSET & fbit(FMT_Q5_K)) batch_dispatch<FMT_Q5_K, FAT>(jb, bx, lds_dyn); break;
+        case FMT_Q6_K: if constexpr (FSET & fbit(FMT_Q6_K)) batch_dispatch<FMT_Q6_K, FAT>(jb, bx, lds_dyn); break;
+        case FMT_Q4M: if constexpr (FSET & fbit(FMT_Q4M)) batch_dispatch<FMT_Q4M, FAT>(jb, bx, lds_dyn); break;
+        case FMT_Q40: if constexpr (FSET & fbit(FMT_Q40)) batch_dispatch<FMT_Q40, FAT>(jb, bx, lds_dyn); break;
+        case FMT_MXFP4: if constexpr (FSET & fbit(FMT_MXFP4)) batch_dispatch<FMT_MXFP4, FAT>(jb, bx, lds_dyn); break;
         default: break;
     }
 }
@@ -1067,11 +1130,13 @@ constexpr size_t LDS_MAX = 160 * 1024 - 256;  // dynamic LDS on offer (the kerne
 
 // Dynamic LDS of a launch; `alds` comes back false when the operand-order activations do not fit (they are then read
 // from L2 per record).
-size_t lds_bytes(int fmt, bool dump, uint32_t nsteps, int tpad, const Shape& sh, bool* alds, uint32_t ng = 1) {
+// `map`: the workgroup's fs slices (see decode_body); zeros for the plain mapping.
+size_t lds_bytes(int fmt, bool dump, uint32_t nsteps, int tpad, const Shape& sh, bool* alds, uint32_t ng = 1, Mapping map = Mapping{}) {
     const uint32_t bps = q8_format(fmt) ? 2 : 4;
-    const uint32_t nbl = bps * ((nsteps + sh.ks - 1) / sh.ks);  // blocks of a slice
+    const uint32_t fs = map.fs ? map.fs : 1;
+    const uint32_t nbl = bps * fs * ((nsteps + sh.ks - 1) / sh.ks);  // blocks of the workgroup's slices
     const uint32_t narr = q8_format(fmt) || fmt == FMT_Q40 || fmt == FMT_MXFP4 ? 1 : fmt == FMT_Q6_K ? (dump ? 4 : 3) : 2;  // metadata arrays
-    const size_t meta = (size_t)narr * ng * nbl * tpad * 4, red = (size_t)sh.rt * sh.kw * ng * tpad * 16 * 4;
+    const size_t meta = (size_t)narr * ng * nbl * tpad * 4, red = (size_t)sh.rt * fs * sh.kw * ng * tpad * 16 * 4;
     const size_t act = (size_t)ng * (nbl / 2) * 512;
     const size_t with = act + meta > red ? act + meta : red;  // the partial sums reuse the activations' space
     *alds = with <= LDS_MAX;
@@ -1256,6 +1321,57 @@ void decode_scratch_need(const WeightView& w, size_t* partial_floats, size_t* nc
 // Every item must be decode_batchable. Items go out in launches of up to BATCH_MAX jobs; jobs whose shape slices K
 // across workgroups take their partial rows and counters from `sc` (hipErrorOutOfMemory when it is too small:
 // nothing has been launched then and the caller launches the jobs one by one).
+// A job's workgroups in a shared launch: row tiles per workgroup and the mapping of runs to waves (decode_body).
+struct Placed {
+    uint32_t rt;
+    Mapping map;
+    uint32_t wgs;
+    size_t lds;
+};
+// Plain: the shape's own workgroups, as a launch of the job alone has them.
+// Fat (for launches with work for every CU several times over): a workgroup takes as many of the shape's slices as
+// keep two workgroups' staging within a CU's LDS, a wave streams about FAT_STEPS steps, and the workgroup has
+// eight waves' worth of tiles. Fewer, fatter workgroups stage less, start and finish less often and keep longer
+// streams: the shared launch of eight GGUF matmuls runs 5 % faster with them, every row's bits unchanged. A launch of a
+// job alone needs the many small workgroups to cover the chip, which is why the shape keeps describing those.
+constexpr uint32_t FAT_STEPS = 32;
+Placed place_job(const DecodeBatchItem& it, bool fat, uint32_t fat_steps) {
+    const uint32_t ntiles = row_tiles(it.w.n_out), nsteps = steps_rt(it.w);
+    const bool pair = it.epi.pair_p0 != nullptr;
+    Shape sh = shape_for(ntiles, nsteps, true, it.w.fmt);
+    if (pair) sh = pair_shape(sh);
+    const int tpad = it.t <= 4 ? 4 : 8;
+    Placed pl{sh.rt, Mapping{sh.kw, 1}, 0, 0};
+    bool alds = false;
+    if (fat && nsteps % (sh.ks * sh.kw) == 0) {  // (every run has the same number of steps)
+        const uint32_t sl = nsteps / sh.ks;
+        uint32_t fs = sh.ks;
+        Shape probe = sh;
+        probe.rt = 8;
+        while (fs > 1 && lds_bytes(it.w.fmt, false, nsteps, tpad, probe, &alds, 1, Mapping{1, fs}) > 80 * 1024) fs /= 2;
+        uint32_t kwp = 1;
+        while (kwp * 2 <= fs * sh.kw && kwp * 2 <= 8 && (fs * sl / (kwp * 2) >= fat_steps || fs * sh.kw / kwp > 4)) kwp *= 2;  // (a wave holds four runs at most)
+        if (pair && kwp == 8) kwp = 4;  // (a pair's workgroup holds an even number of tiles)
+        uint32_t rt = 8 / kwp;
+        const uint32_t cap = pair ? 2 * ntiles : ntiles;
+        while (rt > 1 && rt / 2 >= cap) rt /= 2;
+        probe.rt = rt;
+        const size_t l = lds_bytes(it.w.fmt, false, nsteps, tpad, probe, &alds, 1, Mapping{kwp, fs});
+        if (alds && l <= LDS_MAX && (!pair || rt % 2 == 0)) {
+            pl.rt = rt;
+            pl.map = Mapping{kwp, fs};
+            pl.lds = l;
+        }
+    }
+    if (!pl.lds) {
+        pl.lds = lds_bytes(it.w.fmt, false, nsteps, tpad, sh, &alds);
+        if (!alds) pl.lds = LDS_MAX + 1;  // (refused by the caller)
+    }
+    const uint32_t per_wg = pair ? pl.rt / 2 : pl.rt;
+    pl.wgs = (ntiles + per_wg - 1) / per_wg * (sh.ks / pl.map.fs);
+    return pl;
+}
+
 hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, const DecodeScratch& sc, hipStream_t s, hipEvent_t ev_start,
                                     hipEvent_t ev_stop) {
     static std::atomic<uint64_t> allowed[4];  // whole LDS allowed, one bit per device
@@ -1263,9 +1379,10 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     (void)hipGetDevice(&dev);
     const uint64_t bit = 1ull << (dev & 63);
     if (!(allowed[(dev >> 6) & 3].load(std::memory_order_acquire) & bit)) {
-        for (const void* k : {reinterpret_cast<const void*>(decode_batch_kernel<FSET_GGUF>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_MLX>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_Q6K>),
-                              reinterpret_cast<const void*>(decode_batch_kernel<FSET_Q5K>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_Q40>), reinterpret_cast<const void*>(decode_batch_kernel<FSET_MX4>),
-                              reinterpret_cast<const void*>(decode_batch_kernel<FSET_Q8F>)}) {
+#define OXHIP_BATCH_KERNELS(F) reinterpret_cast<const void*>(decode_batch_kernel<F, false>), reinterpret_cast<const void*>(decode_batch_kernel<F, true>)
+        for (const void* k : {OXHIP_BATCH_KERNELS(FSET_GGUF), OXHIP_BATCH_KERNELS(FSET_MLX), OXHIP_BATCH_KERNELS(FSET_Q6K), OXHIP_BATCH_KERNELS(FSET_Q5K),
+                              OXHIP_BATCH_KERNELS(FSET_Q40), OXHIP_BATCH_KERNELS(FSET_MX4), OXHIP_BATCH_KERNELS(FSET_Q8F)}) {
+#undef OXHIP_BATCH_KERNELS
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
             if (e != hipSuccess) return e;
         }
@@ -1274,6 +1391,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     std::vector<BatchArgs> launches;
     std::vector<size_t> ldss;
     std::vector<uint32_t> threadss;
+    std::vector<bool> fats;
     // the jobs by format set (the caller's order within a set), then launches of up to BATCH_MAX jobs of one set
     std::vector<const DecodeBatchItem*> sorted;
     std::vector<std::pair<size_t, size_t>> runs;  // [first, count) into `sorted`
@@ -1313,15 +1431,30 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
             }
             std::stable_sort(order, order + a.njobs, [&](uint32_t x, uint32_t y) { return key[x] < key[y]; });
         }
+        // fat workgroups when they still cover the chip several times over
+        uint32_t fat_steps = FAT_STEPS, fat_min = 3 * NCU;
+#ifdef OXHIP_TUNING  // tuning builds only: "steps a wave streams, least number of workgroups" in OXHIP_FAT
+        if (const char* e = getenv("OXHIP_FAT")) {
+            unsigned x = 0, y = 0;
+            if (sscanf(e, "%u,%u", &x, &y) == 2 && x >= 1) {
+                fat_steps = x;
+                fat_min = y;
+            }
+        }
+#endif
+        uint64_t fat_wgs = 0;
+        for (uint32_t j = 0; j < a.njobs; j++) fat_wgs += place_job(*items_of[j], true, fat_steps).wgs;
+        const bool fat = fat_wgs >= fat_min;
         for (uint32_t j = 0; j < a.njobs; j++) {
             const DecodeBatchItem& it = *items_of[order[j]];
             const uint32_t ntiles = row_tiles(it.w.n_out), nsteps = steps_rt(it.w);
             const bool pair = it.epi.pair_p0 != nullptr;
             Shape sh = shape_for(ntiles, nsteps, true, it.w.fmt);
             if (pair) sh = pair_shape(sh);
-            bool alds;
-            const size_t l = lds_bytes(it.w.fmt, false, nsteps, it.t <= 4 ? 4 : 8, sh, &alds);
-            if (!alds || l > LDS_MAX || it.t < 1 || it.t > 8) return hipErrorInvalidValue;
+            const Placed pl = place_job(it, fat, fat_steps);
+            const size_t l = pl.lds;
+            if (l > LDS_MAX || it.t < 1 || it.t > 8) return hipErrorInvalidValue;
+            sh.rt = pl.rt;
             const uint32_t per_wg = pair ? sh.rt / 2 : sh.rt;
             const uint32_t groups = (ntiles + per_wg - 1) / per_wg;
             float* partial = nullptr;
@@ -1335,12 +1468,13 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
                 nc += (size_t)groups * CTR_STRIDE;
             }
             lds = l > lds ? l : lds;
-            threads = 64 * sh.rt * sh.kw > threads ? 64 * sh.rt * sh.kw : threads;
-            a.j[j] = BatchJob{it.w, it.xa, it.y, partial, counters, it.t, sh.rt, sh.kw, sh.ks, wg, it.epi};
-            wg += groups * sh.ks;
+            threads = 64 * sh.rt * pl.map.kwp > threads ? 64 * sh.rt * pl.map.kwp : threads;
+            a.j[j] = BatchJob{it.w, it.xa, it.y, partial, counters, it.t, sh.rt, sh.kw, sh.ks, wg, pl.map, it.epi};
+            wg += groups * (sh.ks / pl.map.fs);
         }
         a.nwg = wg;
         launches.push_back(a);
+        fats.push_back(fat);
         ldss.push_back(lds);
         threadss.push_back(threads);
     }
@@ -1361,13 +1495,16 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
             if (ride) hipExtLaunchKernelGGL(kern, dim3(launches[i].nwg), dim3(threadss[i]), (uint32_t)ldss[i], s, ev_start, ev_stop, 0, launches[i]);
             else kern<<<launches[i].nwg, threadss[i], ldss[i], s>>>(launches[i]);
         };
-        if (!(fset & ~FSET_GGUF)) go(decode_batch_kernel<FSET_GGUF>);
-        else if (!(fset & ~FSET_MLX)) go(decode_batch_kernel<FSET_MLX>);
-        else if (!(fset & ~FSET_Q6K)) go(decode_batch_kernel<FSET_Q6K>);
-        else if (!(fset & ~FSET_Q5K)) go(decode_batch_kernel<FSET_Q5K>);
-        else if (!(fset & ~FSET_Q40)) go(decode_batch_kernel<FSET_Q40>);
-        else if (!(fset & ~FSET_MX4)) go(decode_batch_kernel<FSET_MX4>);
-        else if (!(fset & ~FSET_Q8F)) go(decode_batch_kernel<FSET_Q8F>);
+        const bool fat = fats[i];
+#define OXHIP_GO(F) (fat ? go(decode_batch_kernel<F, true>) : go(decode_batch_kernel<F, false>))
+        if (!(fset & ~FSET_GGUF)) OXHIP_GO(FSET_GGUF);
+        else if (!(fset & ~FSET_MLX)) OXHIP_GO(FSET_MLX);
+        else if (!(fset & ~FSET_Q6K)) OXHIP_GO(FSET_Q6K);
+        else if (!(fset & ~FSET_Q5K)) OXHIP_GO(FSET_Q5K);
+        else if (!(fset & ~FSET_Q40)) OXHIP_GO(FSET_Q40);
+        else if (!(fset & ~FSET_MX4)) OXHIP_GO(FSET_MX4);
+        else if (!(fset & ~FSET_Q8F)) OXHIP_GO(FSET_Q8F);
+#undef OXHIP_GO
         else return hipErrorInvalidValue;
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
