@@ -12,6 +12,7 @@
 // a small buffer that stays in L2. Rows are bit-identical whatever the batch (one fixed order per (token, row)).
 #include "internal.hpp"
 
+#include <cstdlib>
 #include <type_traits>
 
 namespace oxhip {
@@ -278,7 +279,10 @@ hipError_t launch_skinny_fp8(const WeightView& w, const void* x, bool x_bf16, bo
     float* partial = reinterpret_cast<float*>(static_cast<uint8_t*>(pack) + frag_bytes(w, t, (int)planes));
     uint32_t slices = 1;
     auto go = [&](auto kern, uint32_t rt, uint32_t ntt) {
-        uint32_t kw = 8;
+        uint32_t kw = 4;  // (four waves of 36 steps stream [7168, 18432] 5 % faster than eight of 18; two: 45 % slower)
+#ifdef OXHIP_TUNING  // tuning builds only: waves per workgroup in OXHIP_FP8_KW
+        if (const char* e = getenv("OXHIP_FP8_KW")) kw = (uint32_t)atoi(e);
+#endif
         while (kw > 1 && nsteps / (kw * slices) < 4) kw /= 2;
         const size_t lds = (size_t)kw * rt * ntt * 64 * 16;
         if (lds > 48 * 1024) {
