@@ -539,6 +539,43 @@ def test_decode_batch_shares_a_launch_and_keeps_the_bits(be, oxref):
             assert np.array_equal(got.view(np.uint32), alone[i].view(np.uint32)), (order, i, cases[i])
 
 
+def test_decode_batch_of_full_size_jobs_keeps_the_bits(be, oxref):
+    """A shared launch with work for every CU several times over maps runs to waves the fat way (a workgroup takes
+    several K slices, a wave several runs): the benchmark's eight matmuls (Q8_0 and Q4_K, 4096 -> 14336 and 14336 -> 4096,
+    1 and 8 tokens) and four Q6_K ones as one batch give every job the rows of its own launch bit for bit, and a sample
+    of those rows is the CPU's within 1e-3."""
+    import torch
+    from oxinfer_amd import synth
+    gens = {Q8_0: synth.gguf_q8_0, Q4_K: synth.gguf_q4_k, Q6_K: synth.gguf_q6_k}
+    shapes = [(14336, 4096), (4096, 14336)]
+    raws = {(kind, n): gens[kind](n, k, 40 + kind + i) for kind in gens for i, (n, k) in enumerate(shapes)}
+    ws = {(kind, n): be.upload_gguf(kind, raws[(kind, n)], n, k) for kind in gens for n, k in shapes}
+    jobs, alone, meta = [], [], []
+    for kind in (Q8_0, Q4_K, Q6_K):
+        for n, k in shapes:
+            for t in (1, 8):
+                xs = synth.activations(t, k, 50 + t)
+                xa = be.quantize_act(torch.from_numpy(xs).cuda())
+                alone.append(be.decode(ws[(kind, n)], xa=xa).cpu().numpy())
+                jobs.append((ws[(kind, n)], xa, None, t, torch.full((t, n), float("nan"), dtype=torch.float32, device="cuda"), None, None))
+                meta.append((kind, n, k, t, xs))
+    for order in (list(range(8)), list(range(12)), [11, 3, 8, 0, 9, 5, 10, 6, 1, 7, 2, 4]):
+        for i in order:
+            jobs[i][4].fill_(float("nan"))
+        be.decode_batch(be.decode_jobs([jobs[i] for i in order]))
+        torch.cuda.synchronize()
+        for i in order:
+            assert np.array_equal(jobs[i][4].cpu().numpy().view(np.uint32), alone[i].view(np.uint32)), (order, i, meta[i][:4])
+    rng = np.random.default_rng(5)
+    for i in (1, 3, 5, 7, 9, 11):  # the eight-token jobs: 24 sampled rows each against the CPU's decode
+        kind, n, k, t, xs = meta[i]
+        rows = np.sort(rng.choice(n, 24, replace=False))
+        rb = oxref.row_bytes(kind, k)
+        sub = np.ascontiguousarray(np.asarray(raws[(kind, n)], np.uint8).reshape(n, rb)[rows])
+        want = oxref.gguf_decode(kind, sub, len(rows), k, xs, t)
+        assert row_err(alone[i][:, rows], want) < TOL, meta[i][:4]
+
+
 def test_decode_batch_events(be, oxref):
     """Timing events of oxhip_dev_decode_batch: a lone job's launch and a shared launch carry them themselves, jobs of
     other kernels and split runs get them recorded around; either way the interval is positive and the rows unchanged."""

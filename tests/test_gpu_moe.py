@@ -477,3 +477,42 @@ def test_matvec_rows_shares_a_launch_and_pairs_keep_the_bits(be, oxref, kind, n_
         alone = np.zeros((t, n_out), np.float32)
         assert be.matvec_rows(x, t, n_in, [(ws[2], None, alone)])
         assert np.array_equal(alone.view(np.uint32), ys[2].view(np.uint32))
+
+
+def test_matvec_rows_of_full_size_pairs_keep_the_bits(be, oxref):
+    """A call large enough for the shared launch's fat mapping (several K slices per workgroup, several runs per wave), with
+    gate / up pairs in it: Llama-8B MLP shapes in Q8_0 and Q4_K, plain and paired. Every plain job gives the rows of a
+    call of its own, every pair silu_mul of its two plain products, bit for bit."""
+    from oxinfer_amd import synth
+    gens = {8: synth.gguf_q8_0, 12: synth.gguf_q4_k}
+    up_shape, down_shape = (14336, 4096), (4096, 14336)
+    ws = {(kind, i): be.upload_gguf(kind, gens[kind](*up_shape, 20 + kind + i), *up_shape) for kind in gens for i in range(2)}
+    for t in (1, 4):
+        x = synth.activations(t, up_shape[1], 30 + t)
+        names = [(kind, i) for kind in gens for i in range(2)]
+        plain = {nm: np.zeros((t, up_shape[0]), np.float32) for nm in names}
+        for nm in names:  # each alone
+            assert be.matvec_rows(x, t, up_shape[1], [(ws[nm], None, plain[nm])]), be.last_error()
+        together = {nm: np.zeros((t, up_shape[0]), np.float32) for nm in names}
+        pairs = {kind: np.zeros((t, up_shape[0]), np.float32) for kind in gens}
+        jobs = [(ws[nm], None, together[nm]) for nm in names] + [(ws[(kind, 0)], ws[(kind, 1)], pairs[kind]) for kind in gens]
+        assert be.matvec_rows(x, t, up_shape[1], jobs), be.last_error()
+        for nm in names:
+            assert np.array_equal(together[nm].view(np.uint32), plain[nm].view(np.uint32)), (t, nm)
+        for kind in gens:
+            want = oxref.silu_mul(plain[(kind, 0)], plain[(kind, 1)])
+            assert np.array_equal(pairs[kind].view(np.uint32), want.view(np.uint32)), (t, kind)
+    # the long-K shape (K sliced across workgroups), paired
+    wd = {(kind, i): be.upload_gguf(kind, gens[kind](*down_shape, 60 + kind + i), *down_shape) for kind in gens for i in range(2)}
+    t = 2
+    x = synth.activations(t, down_shape[1], 77)
+    plain = {nm: np.zeros((t, down_shape[0]), np.float32) for nm in wd}
+    for nm in wd:
+        assert be.matvec_rows(x, t, down_shape[1], [(wd[nm], None, plain[nm])]), be.last_error()
+    pairs = {kind: [np.zeros((t, down_shape[0]), np.float32) for _ in range(4)] for kind in gens}
+    jobs = [(wd[(kind, 0)], wd[(kind, 1)], y) for kind in gens for y in pairs[kind]] + [(wd[nm], None, np.zeros((t, down_shape[0]), np.float32)) for nm in wd]
+    assert be.matvec_rows(x, t, down_shape[1], jobs), be.last_error()
+    for kind in gens:
+        want = oxref.silu_mul(plain[(kind, 0)], plain[(kind, 1)])
+        for y in pairs[kind]:
+            assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), kind
