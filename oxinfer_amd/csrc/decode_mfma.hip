@@ -279,6 +279,9 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     // kq asks for the words of step `first + kq` (row n of it), and at step first + q every lane takes them from lane
     // 16 q + n. Q8_0: {d of the two blocks}; Q4_K: {four sub-block scales, four mins, (d, dmin)}: this step's four
     // sub-blocks are 4 (s & 1) .. + 3 of the super-block; MLX: {d of the two groups, offsets of the two groups}.
+    // (The scale words are ordinary loads, not read-once ones like the codes: a record is not a whole number of cache lines,
+    // so its scales share a line with the next record's first codes, and a line that came in as read-once is gone again
+    // before its other half is asked for: Q6_K's launch fetched 7.5 % more than its records hold, one line per record.)
     constexpr int NM = FMT == FMT_Q8_0 || FMT == FMT_MXFP4 ? 1 : (k45_format(FMT) || FMT == FMT_Q6_K) ? 3 : 2;  // (Q8F: the two f32 scales)
     uint32_t slast = max(s1, 1u) - 1;
     // (Q6_K: with the clamp's bound opaque the compiler keeps 111 registers instead of 141 and a fourth wave per SIMD fits: the
@@ -287,26 +290,26 @@ __device__ __forceinline__ void decode_body(WeightView w, QActView xa, uint32_t 
     auto load_scales = [&](uint32_t* m, uint32_t first) {
         const uint32_t s = min(first + kq, slast);
         if constexpr (FMT == FMT_Q8F) {
-            m[0] = gload_once<uint32_t>(base + (size_t)s * T8F_REC + 1024 + 8 * n);
-            m[1] = gload_once<uint32_t>(base + (size_t)s * T8F_REC + 1028 + 8 * n);
+            m[0] = gload<uint32_t>(base + (size_t)s * T8F_REC + 1024 + 8 * n);
+            m[1] = gload<uint32_t>(base + (size_t)s * T8F_REC + 1028 + 8 * n);
         } else if constexpr (FMT == FMT_Q8_0) {
-            m[0] = gload_once<uint32_t>(base + (size_t)s * T8_REC + 1024 + 4 * n);
+            m[0] = gload<uint32_t>(base + (size_t)s * T8_REC + 1024 + 4 * n);
         } else if constexpr (k45_format(FMT)) {
             const gbytes rec = base + (size_t)(s >> 1) * K45_REC;
-            m[0] = gload_once<uint32_t>(rec + 2048 + 16 * n + 4 * (s & 1));
-            m[1] = gload_once<uint32_t>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
-            m[2] = gload_once<uint32_t>(rec + 2304 + 4 * n);
+            m[0] = gload<uint32_t>(rec + 2048 + 16 * n + 4 * (s & 1));
+            m[1] = gload<uint32_t>(rec + 2048 + 16 * n + 8 + 4 * (s & 1));
+            m[2] = gload<uint32_t>(rec + 2304 + 4 * n);
         } else if constexpr (FMT == FMT_Q6_K) {  // {scales of sub-blocks 0..3, of 4..7, d}
             const gbytes rec = base + (size_t)s * T6K_REC;
-            m[0] = gload_once<uint32_t>(rec + 1536 + 8 * n);
-            m[1] = gload_once<uint32_t>(rec + 1540 + 8 * n);
-            m[2] = gload_once<uint16_t>(rec + 1664 + 2 * n);
+            m[0] = gload<uint32_t>(rec + 1536 + 8 * n);
+            m[1] = gload<uint32_t>(rec + 1540 + 8 * n);
+            m[2] = gload<uint16_t>(rec + 1664 + 2 * n);
         } else if constexpr (FMT == FMT_MXFP4) {  // the four scale bytes of row n's blocks
-            m[0] = gload_once<uint32_t>(base + (size_t)s * T4X_REC + 1024 + 4 * n);
+            m[0] = gload<uint32_t>(base + (size_t)s * T4X_REC + 1024 + 4 * n);
         } else {
             const gbytes rec = base + (size_t)s * T4M_REC;
-            m[0] = gload_once<uint32_t>(rec + 1024 + 4 * n);
-            m[1] = gload_once<uint32_t>(rec + 1088 + 4 * n);
+            m[0] = gload<uint32_t>(rec + 1024 + 4 * n);
+            m[1] = gload<uint32_t>(rec + 1088 + 4 * n);
         }
     };
     const int take0 = (int)(4 * n);  // byte index of lane n for the lane-to-lane read; + 64 q: lane 16 q + n
