@@ -162,10 +162,17 @@ int moe_pass(oxhip_ctx* c, oxhip_moe* m, const float* x, size_t t, const uint32_
         HIP_TRY(launch_moe_plan(route_idx, pairs, k, m->n_exp, max_rows, sc.row_of, sc.src, sc.chunks, sc.nchunks, s), "moe plan launch");
         HIP_TRY(launch_moe_pack_bf16(x, h, sc.src, sc.chunks, sc.nchunks, grid_chunks, sc.fx, s, moe_bf16_std_geometry(m->gate_up[0]->v)), "moe pack launch");
         g.bases = m->bases_gu;
-        HIP_TRY(launch_moe_bf16(m->gate_up[0]->v, g, grid_chunks, sc.fx, sc.gu, s), "moe gate launch");
-        HIP_TRY(launch_moe_act_pack_bf16(sc.gu, sc.gu + inter, 2 * inter, inter, m->act_kind, m->act_param, sc.chunks, sc.nchunks, grid_chunks, sc.fa, s,
-                                         moe_bf16_std_geometry(m->down[0]->v)),
-                "moe act launch");
+        if (moe_bf16_glu_ok(m->gate_up[0]->v, inter, grid_chunks)) {
+            // the gate / up launch pairs gate and up tiles per workgroup, applies the activation and writes the down projection's fragments
+            HIP_TRY(launch_moe_bf16(m->gate_up[0]->v, g, grid_chunks, sc.fx, nullptr, s, inter, m->act_kind, m->act_param, moe_bf16_std_geometry(m->down[0]->v),
+                                    sc.fa),
+                    "moe gate launch");
+        } else {
+            HIP_TRY(launch_moe_bf16(m->gate_up[0]->v, g, grid_chunks, sc.fx, sc.gu, s), "moe gate launch");
+            HIP_TRY(launch_moe_act_pack_bf16(sc.gu, sc.gu + inter, 2 * inter, inter, m->act_kind, m->act_param, sc.chunks, sc.nchunks, grid_chunks, sc.fa, s,
+                                             moe_bf16_std_geometry(m->down[0]->v)),
+                    "moe act launch");
+        }
         g.bases = m->bases_dn;
         HIP_TRY(launch_moe_bf16(m->down[0]->v, g, grid_chunks, sc.fa, sc.o, s), "moe down launch");
     } else {

@@ -261,7 +261,9 @@ hipError_t launch_moe_pack_bf16(const float* x, size_t n_in, const int* rowmap, 
                                 void* frag, hipStream_t s, bool std_geometry = false);
 hipError_t launch_moe_act_pack_bf16(const float* g, const float* u, size_t stride, size_t inter, uint32_t kind, float param, const int4* chunks,
                                     const int* nchunks, uint32_t max_chunks, void* frag, hipStream_t s, bool std_geometry = false);
-hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max_chunks, const void* frag, float* out, hipStream_t s);
+bool moe_bf16_glu_ok(const WeightView& w, size_t inter, uint32_t max_chunks);  // the gate / up launch can apply the activation and write the down projection's fragments
+hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max_chunks, const void* frag, float* out, hipStream_t s,
+                           size_t glu_inter = 0, uint32_t act_kind = 0, float act_param = 0.0f, bool std_out = false, void* out_frag = nullptr);
 
 hipError_t launch_fill_zero(uint32_t* p, size_t n, hipStream_t s);  // n dwords, by a kernel on `s`
 

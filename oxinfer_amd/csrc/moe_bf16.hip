@@ -66,6 +66,40 @@ __global__ __launch_bounds__(256) void moe_pack_bf16_kernel(const float* __restr
     out[(((size_t)c * nsteps + s) * 4 + b) * 64 + lane] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
 }
 
+// Fused gate / up experts with the activation in the output stage: the workgroup's waves 0..3 take RT tiles each of the gate
+// rows [64 RT gx, 64 RT (gx + 1)), waves 4..7 the up tiles of the same rows, and instead of the products the workgroup writes
+// act(gate) * up of its rows as the down projection's fragments (what moe_pack_bf16_kernel<ACT> makes of the stored
+// products, value for value: the same f32 sums go through the same gated_act_scalar and the same rounding).
+struct MoeGlu {
+    uint32_t inter = 0;      // 0: plain products to `out`
+    uint32_t kind = 0;
+    float param = 0.0f;
+    uint32_t std_out = 0;    // the down projection's records hold consecutive columns per lane (Q8_0, Q4_K)
+    uint4* frag = nullptr;   // [chunk][inter / 128][4][64] x 16 B
+};
+template <int RT>
+__device__ __forceinline__ void moe_glu_store(const float* red, const MoeGlu& glu, uint32_t gx, uint32_t c, uint32_t rows) {
+    constexpr uint32_t STEPS = 64 * RT / 128 ? 64 * RT / 128 : 1;  // steps of 128 columns the workgroup's rows make
+    static_assert(64 * RT % 128 == 0, "whole steps per workgroup");
+    for (uint32_t idx = threadIdx.x; idx < STEPS * 256; idx += blockDim.x) {
+        const uint32_t l = idx & 63, b = (idx >> 6) & 3, sl = idx >> 8, n = l & 15, kq = l >> 4;
+        uint32_t pk[4] = {0, 0, 0, 0};
+        if (n < rows) {
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const uint32_t col = 128 * sl + 32 * b + (glu.std_out ? 8 * kq + j : 4 * kq + (j & 3) + 16 * (j >> 2));
+                const uint32_t t = col >> 4, wv = t / RT, r = t % RT;
+                const size_t at = (((size_t)wv * RT + r) * 64 + 16 * (n >> 2) + (col & 15)) * 4 + (n & 3);
+                v[j] = gated_act_scalar(red[at], red[at + (size_t)4 * RT * 64 * 4], glu.kind, glu.param);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) pk[j] = (uint32_t)f32_to_bf16_bits(v[2 * j]) | ((uint32_t)f32_to_bf16_bits(v[2 * j + 1]) << 16);
+        }
+        glu.frag[(((size_t)c * (glu.inter / 128) + gx * STEPS + sl) * 4 + b) * 64 + l] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+    }
+}
+
 // Which (run of row tiles gx, chunk c) a workgroup of the one-dimensional grid takes. Workgroups go to the 8 XCDs in turn
 // (linear id mod 8), and each XCD has an L2 of its own; an expert with more than 16 routed rows has several chunks, each
 // of which streams the expert's rows again. Items are numbered (gx, c) with c fastest, so that the chunks of one expert
@@ -86,7 +120,7 @@ __device__ __forceinline__ bool moe_bf16_item(uint32_t nx, uint32_t nch, uint32_
 // rows (each wave asking memory for them costs more than the weights). out [gathered row][n_out] f32.
 template <int RT, int FMT>
 __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const uint8_t* const* __restrict__ bases, const int4* __restrict__ chunks,
-                                                          const int* __restrict__ nchunks, const uint4* __restrict__ afrag, uint32_t kw, uint32_t nx,
+                                                          const int* __restrict__ nchunks, const uint4* __restrict__ afrag, uint32_t kw, uint32_t nx, MoeGlu glu,
                                                           float* __restrict__ out) {
     extern __shared__ __align__(16) float lds[];  // fragments [step][4][64] x 16 B; then the waves' sums [wave][RT][64][4]
     uint32_t gx, c;
@@ -97,7 +131,8 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
     const uint32_t n = lane & 15;
     const uint32_t nsteps = w.n_in / 128, ntiles = row_tiles(w.n_out);
     const uint32_t ng = 8 / kw, rg = wave / kw, kwave = wave % kw;
-    const uint32_t tile0 = (gx * ng + rg) * RT;
+    // (with the activation fused: waves 0..3 the gate tiles of the workgroup's rows, waves 4..7 the up tiles; kw = 1)
+    const uint32_t tile0 = glu.inter ? (rg < 4 ? (gx * 4 + rg) * RT : glu.inter / 16 + (gx * 4 + rg - 4) * RT) : (gx * ng + rg) * RT;
     const gbytes base = as_global(bases[ch.x]);
     gbytes wp[RT];
     constexpr uint32_t REC = FMT == FMT_MXFP4 ? T4X_REC : T4M_REC;
@@ -229,6 +264,10 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
 #pragma unroll
     for (int r = 0; r < RT; r++) *reinterpret_cast<f32x4*>(red + (((size_t)wave * RT + r) * 64 + lane) * 4) = acc[r];
     __syncthreads();
+    if (glu.inter) {  // uniform over the launch
+        moe_glu_store<RT>(red, glu, gx, c, rows);
+        return;
+    }
     // D[token 4 kq + i][row n]: thread (group, r, lane) adds the group's waves in order and stores its four tokens
     for (uint32_t idx = threadIdx.x; idx < ng * RT * 64; idx += blockDim.x) {
         const uint32_t l = idx & 63, r = (idx >> 6) % RT, g = (idx >> 6) / RT;
@@ -257,7 +296,7 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_kernel(WeightView w, const ui
 // Every product and sum is exact up to the f32 rounding of the matrix cores' accumulation.
 template <int RT, int FMT>
 __global__ __launch_bounds__(512, 4) void moe_bf16_std_kernel(WeightView w, const uint8_t* const* __restrict__ bases, const int4* __restrict__ chunks,
-                                                              const int* __restrict__ nchunks, const uint4* __restrict__ afrag, uint32_t kw, uint32_t nx,
+                                                              const int* __restrict__ nchunks, const uint4* __restrict__ afrag, uint32_t kw, uint32_t nx, MoeGlu glu,
                                                               float* __restrict__ out) {
     static_assert(FMT == FMT_Q8_0 || FMT == FMT_Q4_K, "the formats whose records hold consecutive columns per lane");
     constexpr bool Q8 = FMT == FMT_Q8_0;
@@ -270,7 +309,8 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_std_kernel(WeightView w, cons
     const uint32_t n = lane & 15, kq = lane >> 4;
     const uint32_t nsteps = w.n_in / 128, ntiles = row_tiles(w.n_out);
     const uint32_t ng = 8 / kw, rg = wave / kw, kwave = wave % kw;
-    const uint32_t tile0 = (gx * ng + rg) * RT;
+    // (with the activation fused: waves 0..3 the gate tiles of the workgroup's rows, waves 4..7 the up tiles; kw = 1)
+    const uint32_t tile0 = glu.inter ? (rg < 4 ? (gx * 4 + rg) * RT : glu.inter / 16 + (gx * 4 + rg - 4) * RT) : (gx * ng + rg) * RT;
     const gbytes base = as_global(bases[ch.x]);
     gbytes wp[RT];
 #pragma unroll
@@ -386,6 +426,10 @@ __global__ __launch_bounds__(512, 4) void moe_bf16_std_kernel(WeightView w, cons
 #pragma unroll
     for (int r = 0; r < RT; r++) *reinterpret_cast<f32x4*>(red + (((size_t)wave * RT + r) * 64 + lane) * 4) = acc[r];
     __syncthreads();
+    if (glu.inter) {  // uniform over the launch
+        moe_glu_store<RT>(red, glu, gx, c, rows);
+        return;
+    }
     for (uint32_t idx = threadIdx.x; idx < ng * RT * 64; idx += blockDim.x) {
         const uint32_t l = idx & 63, r = (idx >> 6) % RT, g = (idx >> 6) / RT;
         const uint32_t tile = (gx * ng + g) * RT + r, row = tile * 16 + (l & 15);
@@ -436,13 +480,30 @@ hipError_t launch_moe_act_pack_bf16(const float* g, const float* u, size_t strid
     return hipGetLastError();
 }
 
-hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max_chunks, const void* frag, float* out, hipStream_t s) {
+// Whether the gate / up launch over fused experts `w` ([2 inter, h]) can apply the activation itself and write the down
+// projection's fragments (launch_moe_bf16 with glu_inter): whole workgroups of gate rows, and the plain one-wave-per-row shape.
+bool moe_bf16_glu_ok(const WeightView& w, size_t inter, uint32_t max_chunks) {
+    if (!moe_bf16_ok(w) || w.n_out != 2 * inter || inter % 128) return false;
+    const uint32_t rt = w.fmt == FMT_Q8_0 ? 2 : 4, nsteps = w.n_in / 128, ntiles = row_tiles(w.n_out);
+    if (inter % (64 * rt)) return false;
+    return !(nsteps / 2 >= 4 && (uint64_t)((ntiles + 8 * rt - 1) / (8 * rt)) * max_chunks < 512);  // (the launcher would split K over waves)
+}
+
+// glu_inter != 0 (moe_bf16_glu_ok): `out_frag` receives the fragments of act(gate) * up for a down projection whose records
+// are in `std_out` geometry or not; else `out` receives the products' rows.
+hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max_chunks, const void* frag, float* out, hipStream_t s,
+                           size_t glu_inter, uint32_t act_kind, float act_param, bool std_out, void* out_frag) {
     if (!moe_bf16_ok(w)) return hipErrorInvalidValue;
     if (!max_chunks) return hipSuccess;
     const uint32_t nsteps = w.n_in / 128, ntiles = row_tiles(w.n_out);
     // a wave streams a whole row of records (kw = 1) unless that leaves fewer workgroups than two per CU
     uint32_t rt = w.fmt == FMT_Q8_0 ? 2 : 4, kw = 1;  // (Q8_0: a step is two records per row tile)
     while (kw < 4 && nsteps / (2 * kw) >= 4 && (uint64_t)((ntiles + (8 / kw) * rt - 1) / ((8 / kw) * rt)) * max_chunks < 512) kw *= 2;
+    MoeGlu glu{};
+    if (glu_inter) {
+        if (!moe_bf16_glu_ok(w, glu_inter, max_chunks) || kw != 1 || !out_frag) return hipErrorInvalidValue;
+        glu = MoeGlu{(uint32_t)glu_inter, act_kind, act_param, std_out ? 1u : 0u, static_cast<uint4*>(out_frag)};
+    }
 #ifdef OXHIP_TUNING  // tuning builds only: "rt,kw" in OXHIP_MOE_BF16
     if (const char* e = getenv("OXHIP_MOE_BF16")) {
         unsigned a = 0, b = 0;
@@ -454,12 +515,12 @@ hipError_t launch_moe_bf16(const WeightView& w, const GroupView& g, uint32_t max
 #endif
     const uint32_t ng = 8 / kw;
     const size_t red = (size_t)8 * rt * 64 * 16, fr = (size_t)nsteps * 4096, lds = fr > red ? fr : red;
-    const uint32_t nx = (ntiles + ng * rt - 1) / (ng * rt);
+    const uint32_t nx = glu_inter ? (uint32_t)(glu_inter / (64 * rt)) : (ntiles + ng * rt - 1) / (ng * rt);
     const dim3 grid((nx * max_chunks + 7) / 8 * 8);  // every XCD's share of the items (moe_bf16_item), whatever the chunk count turns out to be
     hipError_t e = hipSuccess;
     auto go = [&](auto kern) {
         if (lds > 48 * 1024) e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e == hipSuccess) kern<<<grid, 512, lds, s>>>(w, g.bases, g.chunks, g.nchunks, static_cast<const uint4*>(frag), kw, nx, out);
+        if (e == hipSuccess) kern<<<grid, 512, lds, s>>>(w, g.bases, g.chunks, g.nchunks, static_cast<const uint4*>(frag), kw, nx, glu, out);
     };
     if (w.fmt == FMT_Q8_0) go(moe_bf16_std_kernel<2, FMT_Q8_0>);
     else if (w.fmt == FMT_Q4_K) rt == 2 ? go(moe_bf16_std_kernel<2, FMT_Q4_K>) : go(moe_bf16_std_kernel<4, FMT_Q4_K>);
