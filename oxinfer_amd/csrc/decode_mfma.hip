@@ -1332,13 +1332,14 @@ struct Placed {
     size_t lds;
 };
 // Plain: the shape's own workgroups, as a launch of the job alone has them.
-// Fat (for launches with work for every CU several times over): a workgroup takes as many of the shape's slices as
+// Fat (for launches that still fill seven eighths of the chip's two places per CU that way): a workgroup takes as many of the shape's slices as
 // keep two workgroups' staging within a CU's LDS, a wave streams about FAT_STEPS steps, and the workgroup has
 // eight waves' worth of tiles. Fewer, fatter workgroups stage less, start and finish less often and keep longer
 // streams: the shared launch of eight GGUF matmuls runs 5 % faster with them, every row's bits unchanged. A launch of a
 // job alone needs the many small workgroups to cover the chip, which is why the shape keeps describing those.
-constexpr uint32_t FAT_STEPS = 32;
+constexpr uint32_t FAT_STEPS = 32, FAT_STEPS_Q6K = 24;  // (Q6_K's records are 1.7 KiB, the others' 1 to 1.2 KiB)
 Placed place_job(const DecodeBatchItem& it, bool fat, uint32_t fat_steps) {
+    if (it.w.fmt == FMT_Q6_K && fat_steps == FAT_STEPS) fat_steps = FAT_STEPS_Q6K;
     const uint32_t ntiles = row_tiles(it.w.n_out), nsteps = steps_rt(it.w);
     const bool pair = it.epi.pair_p0 != nullptr;
     Shape sh = shape_for(ntiles, nsteps, true, it.w.fmt);
@@ -1434,8 +1435,9 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
             }
             std::stable_sort(order, order + a.njobs, [&](uint32_t x, uint32_t y) { return key[x] < key[y]; });
         }
-        // fat workgroups when they still cover the chip several times over
-        uint32_t fat_steps = FAT_STEPS, fat_min = 3 * NCU;
+        // fat workgroups when they still fill most of the chip
+        // (measured: 1056 and 480 fat workgroups beat the plain mapping by 4 to 5 %, 512 are even, 296 lose 40 %)
+        uint32_t fat_steps = FAT_STEPS, fat_min = 7 * NCU / 4;
 #ifdef OXHIP_TUNING  // tuning builds only: "steps a wave streams, least number of workgroups" in OXHIP_FAT
         if (const char* e = getenv("OXHIP_FAT")) {
             unsigned x = 0, y = 0;
