@@ -1367,6 +1367,29 @@ Placed place_job(const DecodeBatchItem& it, bool fat, uint32_t fat_steps) {
             pl.lds = l;
         }
     }
+#ifdef OXHIP_TUNING  // tuning builds only: "tiles:steps:tokens=rt,kwp,fs;..." in OXHIP_MAP overrides a job's mapping (tokens: 4 or 8 = its padding)
+    if (const char* e = getenv("OXHIP_MAP")) {
+        for (const char* p = e; fat && p && *p;) {
+            unsigned nt = 0, ns = 0, tp = 0, a = 0, b = 0, c = 0;
+            if (sscanf(p, "%u:%u:%u=%u,%u,%u", &nt, &ns, &tp, &a, &b, &c) == 6 && nt == ntiles && ns == nsteps && (int)tp == tpad && a >= 1 && b >= 1 && c >= 1 &&
+                a * b <= 8 && sh.ks % c == 0 && (c * sh.kw) % b == 0 && c * sh.kw / b <= 4 && nsteps % (sh.ks * sh.kw) == 0 && (!pair || a % 2 == 0)) {
+                Shape probe = sh;
+                probe.rt = a;
+                const size_t l = lds_bytes(it.w.fmt, false, nsteps, tpad, probe, &alds, 1, Mapping{b, c});
+                if (alds && l <= LDS_MAX) {
+                    pl.rt = a;
+                    pl.map = Mapping{b, c};
+                    pl.lds = l;
+                }
+            }
+            p = strchr(p, ';');
+            if (p) p++;
+        }
+        if (getenv("OXHIP_MAP_PRINT"))
+            fprintf(stderr, "job fmt %d tiles %u steps %u tpad %d: shape (%u,%u,%u) -> rt %u kwp %u fs %u lds %zu\n", it.w.fmt, ntiles, nsteps, tpad, sh.rt, sh.kw, sh.ks, pl.rt,
+                    pl.map.kwp, pl.map.fs, pl.lds);
+    }
+#endif
     if (!pl.lds) {
         pl.lds = lds_bytes(it.w.fmt, false, nsteps, tpad, sh, &alds);
         if (!alds) pl.lds = LDS_MAX + 1;  // (refused by the caller)
