@@ -997,26 +997,26 @@ __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid,
 }
 
 // FSET: the formats compiled in, one bit per Fmt. The compiler allocates registers over the whole kernel, so every
-// format in it costs the others (a seventh format made the common GGUF ones 15 % slower, Q6_K beside Q8_0 and Q4_K
-// spilled registers inside its loop, and one kernel of all formats spilled 480 registers): the formats are split into
+// format in it costs the others (a seventh format made the common GGUF ones 15 % slower, and one kernel of all formats
+// spilled 480 registers): the formats are split into
 // the sets below, and a call whose jobs span several sets becomes one launch per set, back to back on the stream.
 constexpr uint32_t fbit(int f) { return 1u << f; }
-constexpr uint32_t FSET_GGUF = fbit(FMT_Q8_0) | fbit(FMT_Q4_K), FSET_Q6K = fbit(FMT_Q6_K), FSET_MLX = fbit(FMT_Q4M),
+constexpr uint32_t FSET_GGUF = fbit(FMT_Q8_0) | fbit(FMT_Q4_K) | fbit(FMT_Q6_K), FSET_MLX = fbit(FMT_Q4M),
                    FSET_Q5K = fbit(FMT_Q5_K), FSET_Q40 = fbit(FMT_Q40), FSET_MX4 = fbit(FMT_MXFP4), FSET_Q8F = fbit(FMT_Q8F);
 // The sets in launch order: more instruction work per byte first, so that the call's tail is made of the lightest jobs.
-constexpr uint32_t FSETS[] = {FSET_Q6K, FSET_Q5K, FSET_Q40, FSET_MX4, FSET_MLX, FSET_GGUF, FSET_Q8F};
+constexpr uint32_t FSETS[] = {FSET_Q5K, FSET_Q40, FSET_MX4, FSET_MLX, FSET_GGUF, FSET_Q8F};
 constexpr int NSETS = sizeof(FSETS) / sizeof(FSETS[0]);
 inline int set_of(int fmt) {
     for (int i = 0; i < NSETS; i++)
         if (FSETS[i] & fbit(fmt)) return i;
     return -1;
 }
-// (Q6_K alone: its step needs a dozen registers more than the 128 that workgroups of 16 waves leave a wave, and spilled them
-// around its loop; its shapes never exceed 8 waves, so its kernel is bounded at 512 threads and keeps them in registers;
-// Q4_0's likewise, for nine registers)
+// (Q6_K shares the kernel of Q8_0 and Q4_K since its step keeps 111 registers: a Q4_K_M file's layers mix the three, and their
+// matmuls go out in one launch. Q4_0's kernel is bounded at 512 threads, which saves it nine spilled registers; its shapes
+// never exceed 8 waves.)
 // FAT: the launch's jobs use the fat mapping (see place_job); the plain kernels do without its bookkeeping.
 template <uint32_t FSET, bool FAT>
-__global__ __launch_bounds__(FSET == (1u << FMT_Q6_K) || FSET == (1u << FMT_Q40) ? 512 : 1024) void decode_batch_kernel(BatchArgs a) {
+__global__ __launch_bounds__(FSET == (1u << FMT_Q40) ? 512 : 1024) void decode_batch_kernel(BatchArgs a) {
     extern __shared__ __align__(16) float lds_dyn[];
     uint32_t j = 0;
     while (j + 1 < a.njobs && blockIdx.x >= a.j[j + 1].wg0) j++;  // uniform
@@ -1407,7 +1407,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     const uint64_t bit = 1ull << (dev & 63);
     if (!(allowed[(dev >> 6) & 3].load(std::memory_order_acquire) & bit)) {
 #define OXHIP_BATCH_KERNELS(F) reinterpret_cast<const void*>(decode_batch_kernel<F, false>), reinterpret_cast<const void*>(decode_batch_kernel<F, true>)
-        for (const void* k : {OXHIP_BATCH_KERNELS(FSET_GGUF), OXHIP_BATCH_KERNELS(FSET_MLX), OXHIP_BATCH_KERNELS(FSET_Q6K), OXHIP_BATCH_KERNELS(FSET_Q5K),
+        for (const void* k : {OXHIP_BATCH_KERNELS(FSET_GGUF), OXHIP_BATCH_KERNELS(FSET_MLX), OXHIP_BATCH_KERNELS(FSET_Q5K),
                               OXHIP_BATCH_KERNELS(FSET_Q40), OXHIP_BATCH_KERNELS(FSET_MX4), OXHIP_BATCH_KERNELS(FSET_Q8F)}) {
 #undef OXHIP_BATCH_KERNELS
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
@@ -1518,7 +1518,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
         if (!launches[i].nwg) continue;
         uint32_t fset = 0;
         for (uint32_t j = 0; j < launches[i].njobs; j++) fset |= fbit(launches[i].j[j].w.fmt);
-        if (threadss[i] > ((fset == FSET_Q6K || fset == FSET_Q40) ? 512u : 1024u)) return hipErrorInvalidValue;  // (the kernels' launch bounds)
+        if (threadss[i] > (fset == FSET_Q40 ? 512u : 1024u)) return hipErrorInvalidValue;  // (the kernels' launch bounds)
         auto go = [&](auto kern) {
             if (ride) hipExtLaunchKernelGGL(kern, dim3(launches[i].nwg), dim3(threadss[i]), (uint32_t)ldss[i], s, ev_start, ev_stop, 0, launches[i]);
             else kern<<<launches[i].nwg, threadss[i], ldss[i], s>>>(launches[i]);
@@ -1527,7 +1527,6 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
 #define OXHIP_GO(F) (fat ? go(decode_batch_kernel<F, true>) : go(decode_batch_kernel<F, false>))
         if (!(fset & ~FSET_GGUF)) OXHIP_GO(FSET_GGUF);
         else if (!(fset & ~FSET_MLX)) OXHIP_GO(FSET_MLX);
-        else if (!(fset & ~FSET_Q6K)) OXHIP_GO(FSET_Q6K);
         else if (!(fset & ~FSET_Q5K)) OXHIP_GO(FSET_Q5K);
         else if (!(fset & ~FSET_Q40)) OXHIP_GO(FSET_Q40);
         else if (!(fset & ~FSET_MX4)) OXHIP_GO(FSET_MX4);
