@@ -182,7 +182,7 @@ int oxhip_dev_decode_noalloc(oxhip_ctx* ctx, const oxhip_weight* w, const oxhip_
 /* Several independent decode matmuls in one call (a decode step issues many small matmuls; what
  * matmul_quant_batch does for the CPU, src/kernels.rs:1937-1994). The jobs must not depend on one another: runs of
  * consecutive jobs of at most 8 tokens over Q8 / Q8_0 / Q4_K / Q5_K / Q6_K / Q4_0 / MXFP4 / MLX 4-bit weights share launches: one per
- * kernel among them (Q8_0, Q4_K and Q6_K share one, each other format has its own), up to 16 jobs each; their latency chains
+ * kernel among them (Q8_0, Q4_K and Q6_K share one, Q5_K takes Q4_K and Q6_K jobs into its own, each other format has its own), up to 16 jobs each; their latency chains
  * overlap, and every job's rows are bit-identical to a launch of its own. The others launch one by one, in order, on
  * `stream` (inside a shared launch the library orders the jobs itself). ev_start / ev_stop (from oxhip_event_create, or
  * NULL) are recorded before / after the launch that holds the job; for jobs that share a launch the first start and the

@@ -1002,13 +1002,21 @@ __device__ __forceinline__ void batch_dispatch(const BatchJob& jb, uint32_t bid,
 // the sets below, and a call whose jobs span several sets becomes one launch per set, back to back on the stream.
 constexpr uint32_t fbit(int f) { return 1u << f; }
 constexpr uint32_t FSET_GGUF = fbit(FMT_Q8_0) | fbit(FMT_Q4_K) | fbit(FMT_Q6_K), FSET_MLX = fbit(FMT_Q4M),
-                   FSET_Q5K = fbit(FMT_Q5_K), FSET_Q40 = fbit(FMT_Q40), FSET_MX4 = fbit(FMT_MXFP4), FSET_Q8F = fbit(FMT_Q8F);
+                   FSET_K5 = fbit(FMT_Q5_K) | fbit(FMT_Q4_K) | fbit(FMT_Q6_K), FSET_Q40 = fbit(FMT_Q40), FSET_MX4 = fbit(FMT_MXFP4), FSET_Q8F = fbit(FMT_Q8F);
 // The sets in launch order: more instruction work per byte first, so that the call's tail is made of the lightest jobs.
-constexpr uint32_t FSETS[] = {FSET_Q5K, FSET_Q40, FSET_MX4, FSET_MLX, FSET_GGUF, FSET_Q8F};
+constexpr uint32_t FSETS[] = {FSET_K5, FSET_Q40, FSET_MX4, FSET_MLX, FSET_GGUF, FSET_Q8F};
 constexpr int NSETS = sizeof(FSETS) / sizeof(FSETS[0]);
-inline int set_of(int fmt) {
-    for (int i = 0; i < NSETS; i++)
-        if (FSETS[i] & fbit(fmt)) return i;
+// The set a job of format `fmt` goes out with, given the formats present in the call (`mask`). Q4_K and Q6_K are in two sets:
+// with Q8_0 (the formats a Q4_K_M file mixes) and with Q5_K (a Q5_K_M file's), whose step needs a few registers more; they
+// take the second only when the call has Q5_K jobs, so that its layers' matmuls share one launch too.
+inline int set_of(int fmt, uint32_t mask) {
+    const uint32_t both = fbit(FMT_Q4_K) | fbit(FMT_Q6_K);
+    for (int i = 0; i < NSETS; i++) {
+        if (!(FSETS[i] & fbit(fmt))) continue;
+        if ((fbit(fmt) & both) && FSETS[i] == FSET_K5 && !(mask & fbit(FMT_Q5_K))) continue;
+        if ((fbit(fmt) & both) && FSETS[i] == FSET_GGUF && (mask & fbit(FMT_Q5_K))) continue;
+        return i;
+    }
     return -1;
 }
 // (Q6_K shares the kernel of Q8_0 and Q4_K since its step keeps 111 registers: a Q4_K_M file's layers mix the three, and their
@@ -1407,7 +1415,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     const uint64_t bit = 1ull << (dev & 63);
     if (!(allowed[(dev >> 6) & 3].load(std::memory_order_acquire) & bit)) {
 #define OXHIP_BATCH_KERNELS(F) reinterpret_cast<const void*>(decode_batch_kernel<F, false>), reinterpret_cast<const void*>(decode_batch_kernel<F, true>)
-        for (const void* k : {OXHIP_BATCH_KERNELS(FSET_GGUF), OXHIP_BATCH_KERNELS(FSET_MLX), OXHIP_BATCH_KERNELS(FSET_Q5K),
+        for (const void* k : {OXHIP_BATCH_KERNELS(FSET_GGUF), OXHIP_BATCH_KERNELS(FSET_MLX), OXHIP_BATCH_KERNELS(FSET_K5),
                               OXHIP_BATCH_KERNELS(FSET_Q40), OXHIP_BATCH_KERNELS(FSET_MX4), OXHIP_BATCH_KERNELS(FSET_Q8F)}) {
 #undef OXHIP_BATCH_KERNELS
             hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
@@ -1423,10 +1431,12 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
     std::vector<const DecodeBatchItem*> sorted;
     std::vector<std::pair<size_t, size_t>> runs;  // [first, count) into `sorted`
     sorted.reserve(n);
+    uint32_t call_mask = 0;
+    for (size_t i = 0; i < n; i++) call_mask |= fbit(items[i].w.fmt);
     for (int set = 0; set < NSETS; set++) {
         const size_t first = sorted.size();
         for (size_t i = 0; i < n; i++) {
-            const int so = set_of(items[i].w.fmt);
+            const int so = set_of(items[i].w.fmt, call_mask);
             if (so < 0) return hipErrorInvalidValue;
             if (so == set) sorted.push_back(&items[i]);
         }
@@ -1527,7 +1537,7 @@ hipError_t launch_decode_mfma_batch(const DecodeBatchItem* items, size_t n, cons
 #define OXHIP_GO(F) (fat ? go(decode_batch_kernel<F, true>) : go(decode_batch_kernel<F, false>))
         if (!(fset & ~FSET_GGUF)) OXHIP_GO(FSET_GGUF);
         else if (!(fset & ~FSET_MLX)) OXHIP_GO(FSET_MLX);
-        else if (!(fset & ~FSET_Q5K)) OXHIP_GO(FSET_Q5K);
+        else if (!(fset & ~FSET_K5)) OXHIP_GO(FSET_K5);
         else if (!(fset & ~FSET_Q40)) OXHIP_GO(FSET_Q40);
         else if (!(fset & ~FSET_MX4)) OXHIP_GO(FSET_MX4);
         else if (!(fset & ~FSET_Q8F)) OXHIP_GO(FSET_Q8F);
