@@ -390,7 +390,8 @@ def bench_gguf_layer(be, torch, synth, steps, warmup, t, gens):
                 config={"workload": f"a Q4_K_M layer's seven matmuls (Q4_K q, k, o, gate, up; Q6_K v, down; Llama-8B shapes) in one batch call, T = {t}",
                         "bytes_per_step": nbytes, "events": "around the call (one launch)"},
                 roofline={"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
-                          "traffic": None, "kernel": "decode_batch_kernel<Q8_0 | Q4_K | Q6_K>", "bytes_per_launch": nbytes,
+                          "traffic": profile_traffic("decode_batch_kernel_q4_k_m_layer.md") if t == 1 else None,
+                          "kernel": "decode_batch_kernel<Q8_0 | Q4_K | Q6_K>", "bytes_per_launch": nbytes,
                           "avg_launch_us": round(ms * 1e3, 2)})
 
 
