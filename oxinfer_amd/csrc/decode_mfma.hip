@@ -26,7 +26,9 @@
 // per tile; the waves' partial sums meet in LDS in a fixed order. With more than one slice each workgroup leaves
 // its partial rows in global scratch and the last one to arrive (a counter per row group) adds the slices in slice
 // order: the association of a row's sum depends on the weight's shape only, never on arrival order, and there is
-// no second launch. A workgroup stages only its slice of the activations.
+// no second launch. A workgroup stages only its slice of the activations. (That is the plain mapping of a launch of one
+// matmul; a shared launch with enough work gives a workgroup several slices and a wave several waves' shares, each summed
+// apart as before: see decode_body's Mapping and place_job.)
 #include <algorithm>
 #include <atomic>
 #include <cstdio>
